@@ -1,0 +1,119 @@
+/*
+ * gdn_hip.h — C ABI of libgdn_hip.so: the gated delta-rule sequence mixer for gfx950.
+ *
+ * The reference reaches this path through a Python import seam, not an FFI:
+ *   from fla.ops.gated_delta_rule import chunk_gated_delta_rule, fused_recurrent_gated_delta_rule
+ *   (lm_engine/modeling_utils/sequence_mixer_blocks/gated_deltanet/module.py:24-25)
+ * and calls both with keywords q, k, v, g, beta, scale, initial_state, output_final_state,
+ * cu_seqlens, use_qk_l2norm_in_kernel (module.py:197-222).  The entry points below are what a
+ * binding for those two functions needs; every pointer is a DEVICE pointer owned by the
+ * caller.  Except for the per-device kernel attribute set-up done on first use, the library
+ * holds no state, never allocates, frees or synchronises, and launches asynchronously on the
+ * stream it is given (current device of the calling thread).
+ *
+ * Return value of every int-returning entry point: 0 on success, a negative gdn_status on
+ * rejected arguments, a positive hipError_t if a launch failed.
+ */
+#ifndef GDN_HIP_H
+#define GDN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GDN_ABI_VERSION 1
+
+typedef enum gdn_dtype { GDN_BF16 = 0, GDN_F32 = 1 } gdn_dtype;
+
+typedef enum gdn_status {
+    GDN_OK = 0,
+    GDN_ERR_NULL = -1,        /* a required pointer is NULL */
+    GDN_ERR_SHAPE = -2,       /* B, T, H, K, V, N inconsistent or non-positive */
+    GDN_ERR_UNSUPPORTED = -3, /* head dims / dtype / chunk size this build has no kernel for */
+    GDN_ERR_ALIGN = -4,       /* pointer or stride not aligned as the kernels require */
+    GDN_ERR_WORKSPACE = -5,   /* workspace missing or smaller than gdn_workspace_bytes() */
+    GDN_ERR_VARLEN = -6       /* cu_seqlens given with B != 1 */
+} gdn_status;
+
+enum {
+    GDN_FLAG_L2NORM = 1,        /* normalise q and k rows in-kernel: x / sqrt(sum x^2 + 1e-6) */
+    GDN_FLAG_STATE_INPLACE = 2, /* decode: ht == h0 is allowed and expected */
+};
+
+/*
+ * One call = one forward of the operator over all sequences and heads.
+ *
+ *   q, k   [B, T, H, K]   element strides q_stride_{b,t,h}, last dim contiguous
+ *   v, o   [B, T, H, V]   element strides v_/o_stride_{b,t,h}, last dim contiguous
+ *   g      [B, T, H] fp32 contiguous, log-decay (<= 0), or NULL for the ungated rule
+ *   beta   [B, T, H] contiguous in beta_dtype, or NULL for beta == 1
+ *   h0     [N, H, K, V] fp32 contiguous or NULL (zero state)
+ *   ht     [N, H, K, V] fp32 contiguous or NULL (final state not written)
+ *   cu_seqlens  int32 [N + 1] with a leading 0 (packed sequences, then B must be 1), or NULL
+ *               (then N must equal B)
+ *
+ * Replaces the argument list of both fla calls at gated_deltanet/module.py:198-222.
+ */
+typedef struct gdn_args {
+    const void *q;
+    const void *k;
+    const void *v;
+    const void *beta;
+    const float *g;
+    const float *h0;
+    float *ht;
+    void *o;
+    const int32_t *cu_seqlens;
+    void *workspace;
+    uint64_t workspace_bytes;
+
+    int64_t q_stride_b, q_stride_t, q_stride_h;
+    int64_t k_stride_b, k_stride_t, k_stride_h;
+    int64_t v_stride_b, v_stride_t, v_stride_h;
+    int64_t o_stride_b, o_stride_t, o_stride_h;
+
+    int32_t B, T, H, K, V, N;
+    int32_t chunk;      /* chunk length of the chunked forward; this build supports 64 (0 = default) */
+    int32_t dtype;      /* gdn_dtype of q, k, v, o */
+    int32_t beta_dtype; /* gdn_dtype of beta */
+    int32_t flags;      /* GDN_FLAG_* */
+    float scale;        /* multiplies q (after optional normalisation) */
+    int32_t reserved;
+} gdn_args;
+
+/* Version of this header the library was built from; a binding checks it equals GDN_ABI_VERSION. */
+int gdn_abi_version(void);
+
+/* Human-readable text for a value returned by the functions below (gdn_status or hipError_t). */
+const char *gdn_strerror(int status);
+
+/*
+ * Bytes of device scratch gdn_chunk_fwd needs for these shapes (only the shape fields of
+ * `args` are read).  The caller allocates it and passes it in args->workspace.  Returns 0
+ * for unsupported shapes (gdn_chunk_fwd then reports why).
+ */
+uint64_t gdn_workspace_bytes(const gdn_args *args);
+
+/*
+ * Chunked forward over full sequences (bf16 q/k/v/o, fp32 state, chunk 64):
+ * replaces fla.ops.gated_delta_rule.chunk_gated_delta_rule as called at
+ * gated_deltanet/module.py:197-209.  `stream` is a hipStream_t.
+ */
+int gdn_chunk_fwd(const gdn_args *args, void *stream);
+
+/*
+ * Token-by-token recurrence with the state tile held in registers; T may be any length and
+ * q/k/v may be bf16 or fp32.  With T == 1 this is the decode step: one read and one write
+ * of the fp32 state, in place when GDN_FLAG_STATE_INPLACE is set and ht == h0.
+ * Replaces fla.ops.gated_delta_rule.fused_recurrent_gated_delta_rule as called at
+ * gated_deltanet/module.py:210-222.  `stream` is a hipStream_t.
+ */
+int gdn_recurrent_fwd(const gdn_args *args, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GDN_HIP_H */

@@ -1,0 +1,19 @@
+"""MI355X-native gated delta-rule sequence mixer: the operator lm-engine's GatedDeltaNet layer
+calls, as hand-written gfx950 HIP kernels behind a C-ABI library."""
+
+from .fla_shim import install_as_fla, uninstall_fla_shim
+from .kernels import Kernel, enable_all_kernels, enable_kernels, is_kernel_allowed
+from .ops import chunk_gated_delta_rule, fused_recurrent_gated_delta_rule, gated_delta_rule
+
+
+__all__ = [
+    "Kernel",
+    "chunk_gated_delta_rule",
+    "enable_all_kernels",
+    "enable_kernels",
+    "fused_recurrent_gated_delta_rule",
+    "gated_delta_rule",
+    "install_as_fla",
+    "is_kernel_allowed",
+    "uninstall_fla_shim",
+]

@@ -1,0 +1,99 @@
+"""ctypes binding of libgdn_hip.so (the C ABI declared in include/gdn_hip.h).
+
+The library is loaded lazily and the load fails loudly: there is no CPU or PyTorch fallback
+behind the HIP path.  Build it with ``python -m lm_engine_amd.build``.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+
+
+GDN_ABI_VERSION = 1
+
+GDN_BF16 = 0
+GDN_F32 = 1
+
+GDN_FLAG_L2NORM = 1
+GDN_FLAG_STATE_INPLACE = 2
+
+LIBRARY_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libgdn_hip.so")
+
+EXPORTED_SYMBOLS = (
+    "gdn_abi_version",
+    "gdn_strerror",
+    "gdn_workspace_bytes",
+    "gdn_chunk_fwd",
+    "gdn_recurrent_fwd",
+)
+
+
+class GdnArgs(ctypes.Structure):
+    """Mirror of ``struct gdn_args``; field order and types must match include/gdn_hip.h."""
+
+    _fields_ = (
+        [(name, ctypes.c_void_p) for name in ("q", "k", "v", "beta", "g", "h0", "ht", "o", "cu_seqlens", "workspace")]
+        + [("workspace_bytes", ctypes.c_uint64)]
+        + [
+            (f"{t}_stride_{d}", ctypes.c_int64)
+            for t in ("q", "k", "v", "o")
+            for d in ("b", "t", "h")
+        ]
+        + [(name, ctypes.c_int32) for name in ("B", "T", "H", "K", "V", "N", "chunk", "dtype", "beta_dtype", "flags")]
+        + [("scale", ctypes.c_float), ("reserved", ctypes.c_int32)]
+    )
+
+
+class GdnLibraryError(RuntimeError):
+    pass
+
+
+_lib = None
+
+
+def load_library() -> ctypes.CDLL:
+    """Loads libgdn_hip.so once, checks its ABI version and declares the prototypes."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIBRARY_PATH):
+        raise GdnLibraryError(
+            f"{LIBRARY_PATH} is missing: the gated delta-rule HIP library has not been built "
+            "(run `python -m lm_engine_amd.build`); there is no fallback path."
+        )
+    lib = ctypes.CDLL(LIBRARY_PATH)
+    for symbol in EXPORTED_SYMBOLS:
+        if not hasattr(lib, symbol):
+            raise GdnLibraryError(f"{LIBRARY_PATH} does not export {symbol}")
+
+    lib.gdn_abi_version.argtypes = []
+    lib.gdn_abi_version.restype = ctypes.c_int
+    lib.gdn_strerror.argtypes = [ctypes.c_int]
+    lib.gdn_strerror.restype = ctypes.c_char_p
+    lib.gdn_workspace_bytes.argtypes = [ctypes.POINTER(GdnArgs)]
+    lib.gdn_workspace_bytes.restype = ctypes.c_uint64
+    lib.gdn_chunk_fwd.argtypes = [ctypes.POINTER(GdnArgs), ctypes.c_void_p]
+    lib.gdn_chunk_fwd.restype = ctypes.c_int
+    lib.gdn_recurrent_fwd.argtypes = [ctypes.POINTER(GdnArgs), ctypes.c_void_p]
+    lib.gdn_recurrent_fwd.restype = ctypes.c_int
+
+    version = lib.gdn_abi_version()
+    if version != GDN_ABI_VERSION:
+        raise GdnLibraryError(f"libgdn_hip.so has ABI version {version}, this binding expects {GDN_ABI_VERSION}")
+    _lib = lib
+    return lib
+
+
+def strerror(status: int) -> str:
+    return load_library().gdn_strerror(status).decode()
+
+
+def check_status(status: int, what: str) -> None:
+    """Negative codes are rejected arguments (ValueError), positive ones HIP errors (RuntimeError)."""
+    if status == 0:
+        return
+    message = f"{what}: {strerror(status)} (status {status})"
+    if status < 0:
+        raise ValueError(message)
+    raise RuntimeError(message)

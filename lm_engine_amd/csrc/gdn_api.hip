@@ -1,0 +1,89 @@
+// C ABI of libgdn_hip.so (declared in include/gdn_hip.h): argument validation and dispatch.
+// Everything that can fault a kernel (shapes, strides, alignment, workspace size) is checked
+// here on the host before any launch.
+
+#include <hip/hip_runtime.h>
+
+#include "gdn_hip.h"
+#include "gdn_launch.h"
+
+namespace {
+
+inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+int validate_common(const gdn_args* a) {
+    if (a == nullptr) return GDN_ERR_NULL;
+    if (!a->q || !a->k || !a->v || !a->o) return GDN_ERR_NULL;
+    if (a->B <= 0 || a->T <= 0 || a->H <= 0 || a->K <= 0 || a->V <= 0 || a->N <= 0) return GDN_ERR_SHAPE;
+    if (a->cu_seqlens != nullptr) {
+        if (a->B != 1) return GDN_ERR_VARLEN;
+    } else if (a->N != a->B) {
+        return GDN_ERR_SHAPE;
+    }
+    if (a->H > 65535 || a->N > 65535) return GDN_ERR_UNSUPPORTED;
+    if (a->dtype != GDN_BF16 && a->dtype != GDN_F32) return GDN_ERR_UNSUPPORTED;
+    if (a->beta && a->beta_dtype != GDN_BF16 && a->beta_dtype != GDN_F32) return GDN_ERR_UNSUPPORTED;
+    if (a->K != 64 && a->K != 128 && a->K != 256) return GDN_ERR_UNSUPPORTED;
+    if (a->V % 32 != 0) return GDN_ERR_UNSUPPORTED;
+
+    // rows are read and written with 16-byte accesses
+    const int64_t elems16 = (a->dtype == GDN_BF16) ? 8 : 4;
+    const int64_t strides[] = {a->q_stride_b, a->q_stride_t, a->q_stride_h, a->k_stride_b, a->k_stride_t,
+                               a->k_stride_h, a->v_stride_b, a->v_stride_t, a->v_stride_h, a->o_stride_b,
+                               a->o_stride_t, a->o_stride_h};
+    for (int64_t s : strides)
+        if (s < 0 || s % elems16 != 0) return GDN_ERR_ALIGN;
+    if (a->q_stride_h < a->K || a->k_stride_h < a->K || a->v_stride_h < a->V || a->o_stride_h < a->V)
+        return GDN_ERR_SHAPE;
+    if (!aligned(a->q, 16) || !aligned(a->k, 16) || !aligned(a->v, 16) || !aligned(a->o, 16)) return GDN_ERR_ALIGN;
+    if ((a->h0 && !aligned(a->h0, 16)) || (a->ht && !aligned(a->ht, 16))) return GDN_ERR_ALIGN;
+    if (a->g && !aligned(a->g, 4)) return GDN_ERR_ALIGN;
+    if (a->cu_seqlens && !aligned(a->cu_seqlens, 4)) return GDN_ERR_ALIGN;
+    if (a->h0 && a->ht && a->h0 == a->ht && !(a->flags & GDN_FLAG_STATE_INPLACE)) return GDN_ERR_SHAPE;
+    return GDN_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int gdn_abi_version(void) { return GDN_ABI_VERSION; }
+
+const char* gdn_strerror(int status) {
+    switch (status) {
+        case GDN_OK: return "success";
+        case GDN_ERR_NULL: return "a required pointer is NULL";
+        case GDN_ERR_SHAPE: return "inconsistent or non-positive shape";
+        case GDN_ERR_UNSUPPORTED:
+            return "unsupported configuration (need K in {64,128,256}, V % 32 == 0, bf16/fp32; chunked forward: "
+                   "bf16, chunk 64)";
+        case GDN_ERR_ALIGN: return "pointer or stride not 16-byte aligned";
+        case GDN_ERR_WORKSPACE: return "workspace missing or too small";
+        case GDN_ERR_VARLEN: return "cu_seqlens requires B == 1";
+        default: break;
+    }
+    if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));
+    return "unknown gdn status";
+}
+
+uint64_t gdn_workspace_bytes(const gdn_args* a) {
+    if (a == nullptr || !gdn::chunk_shape_supported(*a)) return 0;
+    return gdn::chunk_workspace_bytes(*a);
+}
+
+int gdn_recurrent_fwd(const gdn_args* a, void* stream) {
+    const int rc = validate_common(a);
+    if (rc != GDN_OK) return rc;
+    return gdn::launch_recurrent(*a, static_cast<hipStream_t>(stream));
+}
+
+int gdn_chunk_fwd(const gdn_args* a, void* stream) {
+    const int rc = validate_common(a);
+    if (rc != GDN_OK) return rc;
+    if (!gdn::chunk_shape_supported(*a)) return GDN_ERR_UNSUPPORTED;
+    const uint64_t need = gdn::chunk_workspace_bytes(*a);
+    if (a->workspace == nullptr || a->workspace_bytes < need || !aligned(a->workspace, 256)) return GDN_ERR_WORKSPACE;
+    return gdn::launch_chunk_fwd(*a, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

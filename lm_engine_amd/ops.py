@@ -1,0 +1,249 @@
+"""The gated delta-rule operator behind the signature the reference layer calls.
+
+The reference's ``GatedDeltaNet.forward`` makes exactly two calls on this path
+(lm_engine/modeling_utils/sequence_mixer_blocks/gated_deltanet/module.py:197-222), both with
+the keywords ``q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens,
+use_qk_l2norm_in_kernel`` and both returning ``(o, final_state)``:
+
+* ``chunk_gated_delta_rule``            for sequences longer than 64 tokens (training, prefill)
+* ``fused_recurrent_gated_delta_rule``  otherwise, in particular the one-token decode step
+
+Both are provided here with the same names, argument meaning and return convention, on top
+of the HIP library (``libgdn_hip.so``, C ABI in include/gdn_hip.h).  PyTorch only owns the
+device memory and the stream; there is no eager or CPU fallback: without the library every
+call raises.
+
+    q, k            [B, T, H, K]   bf16 (or fp32), last dim contiguous
+    v               [B, T, H, V]
+    g               [B, T, H]      fp32 log-decay (<= 0); None = ungated
+    beta            [B, T, H]      None = 1
+    initial_state   [N, H, K, V]   fp32; N = B, or number of packed sequences
+    cu_seqlens      [N + 1]        int32 with leading 0 (then B must be 1)
+    returns  o [B, T, H, V] in v.dtype, final_state [N, H, K, V] fp32 or None
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import _lib
+from .kernels import Kernel, is_kernel_allowed
+
+
+RECURRENT_MAX_TOKENS = 64  # the reference's mode switch, gated_deltanet/module.py:193
+
+_SUPPORTED_K = (64, 128, 256)
+
+
+def _dtype_code(dtype: torch.dtype, what: str) -> int:
+    if dtype == torch.bfloat16:
+        return _lib.GDN_BF16
+    if dtype == torch.float32:
+        return _lib.GDN_F32
+    raise ValueError(f"{what} must be bfloat16 or float32, got {dtype}")
+
+
+def _require_hip_path() -> None:
+    if not is_kernel_allowed(Kernel.gated_delta_rule):
+        raise RuntimeError(
+            "Kernel.gated_delta_rule is disabled and this package ships no other implementation of the "
+            "gated delta rule; enable it (it is on by default) with lm_engine_amd.kernels.enable_kernels"
+        )
+
+
+def _last_dim_contiguous(x: torch.Tensor) -> torch.Tensor:
+    return x if x.stride(-1) == 1 else x.contiguous()
+
+
+def _check_inputs(q, k, v, g, beta, initial_state, cu_seqlens):
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise ValueError("q, k, v must be [B, T, H, D] tensors")
+    B, T, H, K = q.shape
+    V = v.size(-1)
+    if k.shape != q.shape:
+        raise ValueError(f"k {tuple(k.shape)} must have the shape of q {tuple(q.shape)}")
+    if v.shape[:3] != q.shape[:3]:
+        raise ValueError(f"v {tuple(v.shape)} must share [B, T, H] with q {tuple(q.shape)}")
+    if not q.is_cuda:
+        raise ValueError("the gated delta rule runs on the GPU only; inputs must be device tensors")
+    for name, x in (("k", k), ("v", v), ("g", g), ("beta", beta), ("initial_state", initial_state),
+                    ("cu_seqlens", cu_seqlens)):  # fmt: skip
+        if x is not None and x.device != q.device:
+            raise ValueError(f"{name} is on {x.device}, q is on {q.device}")
+    if k.dtype != q.dtype or v.dtype != q.dtype:
+        raise ValueError(f"q, k, v must share a dtype, got {q.dtype}, {k.dtype}, {v.dtype}")
+    if K not in _SUPPORTED_K:
+        raise ValueError(f"head dim K={K} is not supported (supported: {_SUPPORTED_K})")
+    if V % 32 != 0:
+        raise ValueError(f"value head dim V={V} must be a multiple of 32")
+    for name, x in (("g", g), ("beta", beta)):
+        if x is not None and tuple(x.shape) != (B, T, H):
+            raise ValueError(f"{name} must be [B, T, H] = {(B, T, H)}, got {tuple(x.shape)}")
+    if cu_seqlens is not None:
+        if B != 1:
+            raise ValueError(f"with cu_seqlens the batch dim must be 1 (tokens packed along T), got B={B}")
+        if cu_seqlens.dim() != 1 or cu_seqlens.numel() < 2:
+            raise ValueError("cu_seqlens must be a 1-D tensor [N + 1]")
+        N = cu_seqlens.numel() - 1
+    else:
+        N = B
+    if initial_state is not None:
+        if tuple(initial_state.shape) != (N, H, K, V):
+            raise ValueError(f"initial_state must be [N, H, K, V] = {(N, H, K, V)}, got {tuple(initial_state.shape)}")
+        if initial_state.dtype != torch.float32:
+            raise ValueError(f"initial_state must be float32, got {initial_state.dtype}")
+    return B, T, H, K, V, N
+
+
+def _fill_args(q, k, v, g, beta, h0, ht, o, cu_seqlens, scale, l2norm, inplace, dims) -> _lib.GdnArgs:
+    B, T, H, K, V, N = dims
+    a = _lib.GdnArgs()
+    a.q, a.k, a.v, a.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr()
+    a.beta = None if beta is None else beta.data_ptr()
+    a.g = None if g is None else g.data_ptr()
+    a.h0 = None if h0 is None else h0.data_ptr()
+    a.ht = None if ht is None else ht.data_ptr()
+    a.cu_seqlens = None if cu_seqlens is None else cu_seqlens.data_ptr()
+    a.workspace, a.workspace_bytes = None, 0
+    for name, x in (("q", q), ("k", k), ("v", v), ("o", o)):
+        setattr(a, f"{name}_stride_b", x.stride(0))
+        setattr(a, f"{name}_stride_t", x.stride(1))
+        setattr(a, f"{name}_stride_h", x.stride(2))
+    a.B, a.T, a.H, a.K, a.V, a.N = B, T, H, K, V, N
+    a.chunk = 64
+    a.dtype = _dtype_code(q.dtype, "q, k, v")
+    a.beta_dtype = _lib.GDN_F32 if beta is None else _dtype_code(beta.dtype, "beta")
+    a.flags = (_lib.GDN_FLAG_L2NORM if l2norm else 0) | (_lib.GDN_FLAG_STATE_INPLACE if inplace else 0)
+    a.scale = float(K**-0.5 if scale is None else scale)
+    return a
+
+
+def _run(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm, inplace_state):
+    _require_hip_path()
+    lib = _lib.load_library()
+    dims = _check_inputs(q, k, v, g, beta, initial_state, cu_seqlens)
+    B, T, H, K, V, N = dims
+
+    q, k, v = _last_dim_contiguous(q), _last_dim_contiguous(k), _last_dim_contiguous(v)
+    if g is not None:
+        g = g.to(torch.float32).contiguous()
+    if beta is not None:
+        beta = beta.contiguous() if beta.dtype in (torch.bfloat16, torch.float32) else beta.float().contiguous()
+    if cu_seqlens is not None:
+        cu_seqlens = cu_seqlens.to(torch.int32).contiguous()
+    h0 = None if initial_state is None else initial_state.contiguous()
+
+    o = torch.empty(B, T, H, V, dtype=v.dtype, device=v.device)
+    ht = None
+    if output_final_state:
+        if inplace_state:
+            if h0 is None or h0.data_ptr() != initial_state.data_ptr():
+                raise ValueError("inplace_state needs a contiguous initial_state to update")
+            ht = h0
+        else:
+            ht = torch.empty(N, H, K, V, dtype=torch.float32, device=v.device)
+
+    args = _fill_args(q, k, v, g, beta, h0, ht, o, cu_seqlens, scale, l2norm, inplace_state and ht is not None, dims)
+    stream = ctypes.c_void_p(torch.cuda.current_stream(q.device).cuda_stream)
+
+    with torch.cuda.device(q.device):
+        if mode == "chunk":
+            nbytes = lib.gdn_workspace_bytes(ctypes.byref(args))
+            workspace = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=q.device)
+            args.workspace, args.workspace_bytes = workspace.data_ptr(), workspace.numel()
+            _lib.check_status(lib.gdn_chunk_fwd(ctypes.byref(args), stream), "gdn_chunk_fwd")
+        else:
+            _lib.check_status(lib.gdn_recurrent_fwd(ctypes.byref(args), stream), "gdn_recurrent_fwd")
+    return o, ht
+
+
+class _ForwardOnly(torch.autograd.Function):
+    """The operator has no backward yet; differentiating through it must fail, not pass silently."""
+
+    @staticmethod
+    def forward(ctx, mode, scale, output_final_state, l2norm, inplace_state, q, k, v, g, beta, initial_state,
+                cu_seqlens):  # fmt: skip
+        o, ht = _run(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm,
+                     inplace_state)  # fmt: skip
+        return o, ht
+
+    @staticmethod
+    def backward(ctx, *grads):
+        raise NotImplementedError("the HIP gated delta rule is forward-only; its backward is not implemented")
+
+
+def _dispatch(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm, inplace_state):
+    tensors = (q, k, v, g, beta, initial_state)
+    if torch.is_grad_enabled() and any(x is not None and x.requires_grad for x in tensors):
+        return _ForwardOnly.apply(mode, scale, output_final_state, l2norm, inplace_state, q, k, v, g, beta,
+                                  initial_state, cu_seqlens)  # fmt: skip
+    return _run(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm, inplace_state)
+
+
+def chunk_gated_delta_rule(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    g: torch.Tensor | None = None,
+    beta: torch.Tensor | None = None,
+    scale: float | None = None,
+    initial_state: torch.Tensor | None = None,
+    output_final_state: bool = False,
+    cu_seqlens: torch.Tensor | None = None,
+    head_first: bool = False,
+    use_qk_l2norm_in_kernel: bool = False,
+) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """Chunked (chunk = 64) forward; drop-in for the call at gated_deltanet/module.py:197-209.
+
+    bf16 inputs run the MFMA chunk kernels.  fp32 inputs are computed exactly, token by token,
+    by the recurrent kernel (the chunk kernels round their matrix operands to bf16)."""
+    if head_first:
+        raise ValueError("head_first layouts are not supported; pass [B, T, H, D] tensors")
+    mode = "chunk" if q.dtype == torch.bfloat16 else "recurrent"
+    return _dispatch(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens,
+                     use_qk_l2norm_in_kernel, False)  # fmt: skip
+
+
+def fused_recurrent_gated_delta_rule(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    g: torch.Tensor | None = None,
+    beta: torch.Tensor | None = None,
+    scale: float | None = None,
+    initial_state: torch.Tensor | None = None,
+    output_final_state: bool = False,
+    cu_seqlens: torch.Tensor | None = None,
+    use_qk_l2norm_in_kernel: bool = False,
+    inplace_state: bool = False,
+) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """Token-by-token forward; drop-in for the call at gated_deltanet/module.py:210-222.
+
+    With ``inplace_state=True`` (and ``output_final_state=True``) the final state overwrites
+    ``initial_state`` and that same tensor is returned: one read and one write of the state per
+    decode step instead of a fresh allocation.  The reference's cache replaces its tensor with
+    whatever is returned (lm_engine/generation_cache/constant.py:17-23), so both modes fit it."""
+    return _dispatch("recurrent", q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens,
+                     use_qk_l2norm_in_kernel, inplace_state)  # fmt: skip
+
+
+def gated_delta_rule(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    beta: torch.Tensor | None,
+    g: torch.Tensor | None,
+    initial_state: torch.Tensor | None = None,
+    cu_seqlens: torch.Tensor | None = None,
+    scale: float | None = None,
+    use_qk_l2norm_in_kernel: bool = False,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """``(q, k, v, beta, g, initial_state, cu_seqlens) -> (o, final_state)``.
+
+    Picks the kernel the way the reference layer does (gated_deltanet/module.py:193): token
+    dimension <= 64 runs the recurrent kernel, anything longer the chunked forward."""
+    fn = fused_recurrent_gated_delta_rule if q.size(1) <= RECURRENT_MAX_TOKENS else chunk_gated_delta_rule
+    return fn(q=q, k=k, v=v, g=g, beta=beta, scale=scale, initial_state=initial_state, output_final_state=True,
+              cu_seqlens=cu_seqlens, use_qk_l2norm_in_kernel=use_qk_l2norm_in_kernel)  # fmt: skip

@@ -1,0 +1,165 @@
+"""Host-side checks that need no GPU: the C-ABI library loads, exports what include/gdn_hip.h
+declares, agrees with the ctypes mirror of the argument struct, and rejects bad arguments
+before anything is launched."""
+
+import ctypes
+import os
+import re
+import subprocess
+import sys
+import tempfile
+
+import pytest
+import torch
+
+import lm_engine_amd
+from lm_engine_amd import _lib
+from lm_engine_amd.kernels import Kernel, enable_kernels, is_kernel_allowed
+
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "gdn_hip.h")
+
+
+def _declared_functions() -> list[str]:
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return re.findall(r"\b(gdn_[a-z_]+)\s*\(", text)
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load_library()
+    declared = set(_declared_functions())
+    assert declared == set(_lib.EXPORTED_SYMBOLS), declared
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.gdn_abi_version() == _lib.GDN_ABI_VERSION
+
+
+def test_struct_layout_matches_the_header():
+    source = r"""
+    #include <stdio.h>
+    #include <stddef.h>
+    #include "gdn_hip.h"
+    int main(void) {
+        printf("%zu %zu %zu %zu %zu %zu %zu\n", sizeof(gdn_args), offsetof(gdn_args, workspace_bytes),
+               offsetof(gdn_args, q_stride_b), offsetof(gdn_args, o_stride_h), offsetof(gdn_args, B),
+               offsetof(gdn_args, flags), offsetof(gdn_args, scale));
+        return 0;
+    }
+    """
+    with tempfile.TemporaryDirectory() as tmp:
+        src, exe = os.path.join(tmp, "layout.c"), os.path.join(tmp, "layout")
+        open(src, "w").write(source)
+        subprocess.run(["gcc", f"-I{os.path.dirname(HEADER)}", src, "-o", exe], check=True)
+        values = [int(x) for x in subprocess.run([exe], check=True, capture_output=True, text=True).stdout.split()]
+    A = _lib.GdnArgs
+    assert values == [ctypes.sizeof(A), A.workspace_bytes.offset, A.q_stride_b.offset, A.o_stride_h.offset,
+                      A.B.offset, A.flags.offset, A.scale.offset]  # fmt: skip
+
+
+def _args(**over):
+    a = _lib.GdnArgs()
+    fake = 0x1000  # never dereferenced: validation fails before any launch
+    a.q = a.k = a.v = a.o = fake
+    a.B, a.T, a.H, a.K, a.V, a.N = 1, 8, 2, 64, 64, 1
+    a.q_stride_h = a.k_stride_h = 64
+    a.v_stride_h = a.o_stride_h = 64
+    a.q_stride_t = a.k_stride_t = a.v_stride_t = a.o_stride_t = 128
+    a.q_stride_b = a.k_stride_b = a.v_stride_b = a.o_stride_b = 1024
+    a.dtype, a.beta_dtype, a.scale = _lib.GDN_BF16, _lib.GDN_BF16, 0.125
+    for name, value in over.items():
+        setattr(a, name, value)
+    return a
+
+
+@pytest.mark.parametrize(
+    "over, status",
+    [
+        (dict(q=None), -1),
+        (dict(T=0), -2),
+        (dict(N=3), -2),
+        (dict(K=48), -3),
+        (dict(V=40), -3),
+        (dict(dtype=7), -3),
+        (dict(q_stride_t=129), -4),
+        (dict(v=0x1004), -4),
+        (dict(cu_seqlens=0x2000, B=2, N=2), -6),
+        (dict(q_stride_h=32), -2),
+    ],
+)
+def test_bad_arguments_are_rejected_before_launch(over, status):
+    lib = _lib.load_library()
+    a = _args(**over)
+    assert lib.gdn_recurrent_fwd(ctypes.byref(a), None) == status
+    assert lib.gdn_chunk_fwd(ctypes.byref(a), None) == status
+    assert _lib.strerror(status) != "unknown gdn status"
+
+
+def test_chunk_fwd_needs_a_workspace():
+    lib = _lib.load_library()
+    a = _args(T=128, K=128, V=128, q_stride_h=128, k_stride_h=128, v_stride_h=128, o_stride_h=128,
+              q_stride_t=256, k_stride_t=256, v_stride_t=256, o_stride_t=256, q_stride_b=256 * 128,
+              k_stride_b=256 * 128, v_stride_b=256 * 128, o_stride_b=256 * 128)  # fmt: skip
+    need = lib.gdn_workspace_bytes(ctypes.byref(a))
+    assert need > 0
+    assert lib.gdn_chunk_fwd(ctypes.byref(a), None) == -5
+    a.workspace, a.workspace_bytes = 0x10000, need - 1
+    assert lib.gdn_chunk_fwd(ctypes.byref(a), None) == -5
+    a.dtype = _lib.GDN_F32  # fp32 inputs have no chunk kernel
+    assert lib.gdn_workspace_bytes(ctypes.byref(a)) == 0
+    assert lib.gdn_chunk_fwd(ctypes.byref(a), None) == -3
+
+
+def test_python_wrapper_validates_and_never_falls_back():
+    q = torch.zeros(1, 8, 2, 64, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="GPU only"):
+        lm_engine_amd.fused_recurrent_gated_delta_rule(q=q, k=q, v=q)
+    with pytest.raises(ValueError, match="shape of q"):
+        lm_engine_amd.chunk_gated_delta_rule(q=q, k=q[:, :4], v=q)
+    with pytest.raises(ValueError, match="head_first"):
+        lm_engine_amd.chunk_gated_delta_rule(q=q, k=q, v=q, head_first=True)
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIBRARY_PATH", "/nonexistent/libgdn_hip.so")
+    with pytest.raises(_lib.GdnLibraryError, match="no fallback"):
+        _lib.load_library()
+
+
+def test_kernel_flag_registry_follows_the_reference_convention():
+    assert is_kernel_allowed(Kernel.gated_delta_rule)
+    with enable_kernels([], reset=True):
+        assert not is_kernel_allowed(Kernel.gated_delta_rule)
+        q = torch.zeros(1, 8, 2, 64, dtype=torch.bfloat16)
+        with pytest.raises(RuntimeError, match="no other implementation"):
+            lm_engine_amd.fused_recurrent_gated_delta_rule(q=q, k=q, v=q)
+        with enable_kernels([Kernel.gated_delta_rule]):
+            assert is_kernel_allowed(Kernel.gated_delta_rule)
+        assert not is_kernel_allowed(Kernel.gated_delta_rule)
+    assert is_kernel_allowed(Kernel.gated_delta_rule)
+
+
+def test_kernel_flag_env_variable():
+    code = "from lm_engine_amd.kernels import Kernel, is_kernel_allowed; print(is_kernel_allowed(Kernel.gated_delta_rule))"
+    run = lambda env: subprocess.run([sys.executable, "-c", code], env={**os.environ, **env}, cwd=ROOT,
+                                     capture_output=True, text=True, check=True).stdout.strip()  # noqa: E731  # fmt: skip
+    assert run({"ENABLE_KERNELS": "rmsnorm"}) == "False"
+    assert run({"ENABLE_KERNELS": "rmsnorm, gated_delta_rule"}) == "True"
+    assert run({"ENABLE_ALL_KERNELS": "1"}) == "True"
+
+
+def test_fla_shim_resolves_the_reference_imports():
+    from lm_engine_amd import install_as_fla, uninstall_fla_shim
+
+    install_as_fla()
+    try:
+        from fla.ops.gated_delta_rule import chunk_gated_delta_rule, fused_recurrent_gated_delta_rule
+        import fla  # noqa: F401  (the reference's availability probe, lm_engine/utils/packages.py:56-61)
+
+        assert chunk_gated_delta_rule is lm_engine_amd.chunk_gated_delta_rule
+        assert fused_recurrent_gated_delta_rule is lm_engine_amd.fused_recurrent_gated_delta_rule
+    finally:
+        uninstall_fla_shim()
+    assert "fla" not in sys.modules
