@@ -1,0 +1,249 @@
+"""Benchmark of the gated delta-rule path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 1|2|4] [--no-cpu-baseline] [--no-decode]
+
+A "step" is one chunked forward (``chunk_gated_delta_rule``) over one batch of synthetic input of
+the benchmark configuration (default: configuration 1, B=4, T=4096, H=16, K=V=128, bf16, chunk 64),
+inputs already resident in HBM.  Prints ONE JSON line:
+
+  value        tokens/s of the whole step (B*T / wall time per step, all kernels, workspace
+               allocation through the caching allocator included)
+  roofline     the dominant kernel of the step against the bf16 dense MFMA peak: algorithmic
+               FLOPs of the contractions that kernel performs / its HIP-event duration
+  decode       the decode step (configuration 3: 256 sequences x 32 heads, fp32 state 512 MiB
+               updated in place) against the HBM peak, state buffers rotated so the state
+               cannot live in the 256 MB Infinity Cache
+  cpu_baseline the naive token-by-token torch restatement of the operator (oracle/), timed on
+               this host's cores on a bounded prefix of the same workload
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", type=int, default=1, choices=(1, 2, 4))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-decode", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target duration of the CPU baseline sample")
+    return ap.parse_args()
+
+
+def bench_chunk(w, steps, warmup):
+    import torch
+
+    import lm_engine_amd
+    from lm_engine_amd.ops import chunk_forward_kernel_times
+    from lm_engine_amd.workloads import chunk_fwd_bytes_per_token_head, chunk_fwd_flops_per_token_head, make_inputs
+
+    inp = make_inputs(w, device="cuda")
+    call = lambda: lm_engine_amd.chunk_gated_delta_rule(**inp, output_final_state=True)  # noqa: E731
+
+    for _ in range(warmup):
+        call()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        call()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / steps * 1e3
+
+    # per-kernel durations: HIP events recorded on the launch stream around every kernel of the step
+    sums: dict[str, float] = {}
+    for _ in range(steps):
+        for name, ms in chunk_forward_kernel_times(**inp, output_final_state=True).items():
+            sums[name] = sums.get(name, 0.0) + ms
+    kernel_ms = {name: total / steps for name, total in sums.items()}
+
+    tokens = w.B * w.T
+    token_heads = tokens * w.H
+    flops = chunk_fwd_flops_per_token_head(w.K, w.V)
+    n_seq = w.B if inp["cu_seqlens"] is None else inp["cu_seqlens"].numel() - 1
+    state_bytes = n_seq * w.H * w.K * w.V * 4 * (2 if inp["initial_state"] is not None else 1)
+    algo_bytes = token_heads * chunk_fwd_bytes_per_token_head(w.K, w.V) + state_bytes
+
+    per_kernel = {}
+    for name, part in (("chunk_prepare", "prepare"), ("chunk_scan", "scan")):
+        tflops = token_heads * flops[part] / (kernel_ms[name] * 1e-3) / 1e12
+        per_kernel[name] = {"ms": round(kernel_ms[name], 4), "algorithmic_flop_per_token_head": flops[part],
+                            "tflops": round(tflops, 1), "mfma_frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4)}  # fmt: skip
+    dominant = max(per_kernel, key=lambda name: per_kernel[name]["ms"])
+    whole_tflops = token_heads * flops["dense"] / (ms_per_step * 1e-3) / 1e12
+
+    result = {
+        "metric": "GDN chunk-fwd tokens/s",
+        "value": round(tokens / (ms_per_step * 1e-3), 1),
+        "unit": "tokens/s",
+        "ms_per_step": round(ms_per_step, 4),
+        "dtype": "bf16",
+        "config": {"workload": w.name, "B": w.B, "T": w.T, "H": w.H, "K": w.K, "V": w.V, "chunk": 64,
+                   "sequences": n_seq, "initial_state": inp["initial_state"] is not None},  # fmt: skip
+        "roofline": {
+            "kernel": dominant,
+            "bound": "mfma",
+            "achieved": per_kernel[dominant]["tflops"],
+            "peak": MFMA_BF16_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": per_kernel[dominant]["mfma_frac"],
+            "traffic": None,
+        },
+        "step": {
+            "tflops_dense": round(whole_tflops, 1),
+            "mfma_frac_dense": round(whole_tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+            "tflops_strict": round(token_heads * flops["strict"] / (ms_per_step * 1e-3) / 1e12, 1),
+            "algorithmic_gbs": round(algo_bytes / (ms_per_step * 1e-3) / 1e9, 1),
+            "hbm_frac": round(algo_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "kernels": per_kernel,
+        },
+    }
+    return result, inp
+
+
+def bench_decode(steps, warmup):
+    import torch
+
+    import lm_engine_amd
+    from lm_engine_amd.workloads import decode_bytes_per_seq_head, get_workload, make_inputs
+
+    w = get_workload(3)
+    inp = make_inputs(w, device="cuda")
+    states = [inp["initial_state"].clone() for _ in range(3)]  # 3 x 512 MiB > Infinity Cache
+
+    def call(i):
+        args = dict(inp, initial_state=states[i % len(states)])
+        return lm_engine_amd.fused_recurrent_gated_delta_rule(**args, output_final_state=True, inplace_state=True)
+
+    for i in range(warmup):
+        call(i)
+    torch.cuda.synchronize()
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i, (start, stop) in enumerate(events):
+        start.record()
+        call(i)
+        stop.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) / steps * 1e3
+    kernel_ms = sum(start.elapsed_time(stop) for start, stop in events) / steps
+    nbytes = decode_bytes_per_seq_head(w.K, w.V) * w.B * w.H
+    gbs = nbytes / (kernel_ms * 1e-3) / 1e9
+    return {
+        "workload": w.name,
+        "sequences": w.B, "H": w.H, "K": w.K, "V": w.V,
+        "ms_per_step": round(wall_ms, 4),
+        "kernel_ms": round(kernel_ms, 4),
+        "seq_tokens_per_s": round(w.B / (wall_ms * 1e-3), 1),
+        "roofline": {"kernel": "recurrent_kernel", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+    }  # fmt: skip
+
+
+def cpu_baseline(w, inp_gpu, target_seconds):
+    """Naive recurrent torch restatement on this host's cores, on a bounded prefix of the workload:
+    the first sequence, all heads, as many tokens as fit the time budget (the cost is exactly
+    linear in the token count)."""
+    import torch
+
+    from oracle import recurrent_gated_delta_rule_ref
+    from oracle.c_oracle import recurrent_gated_delta_rule_c
+
+    cores = torch.get_num_threads()
+    first = 0 if inp_gpu["cu_seqlens"] is None else None
+    cpu = {n: (x.cpu() if isinstance(x, torch.Tensor) else x) for n, x in inp_gpu.items()}
+    seq_len = w.T if first is not None else int(cpu["cu_seqlens"][1])
+
+    def prefix(tokens):
+        sub = {n: cpu[n][:1, :tokens] for n in ("q", "k", "v", "g", "beta") if cpu[n] is not None}
+        h0 = cpu["initial_state"]
+        return dict(sub, initial_state=None if h0 is None else h0[:1], scale=cpu["scale"])
+
+    probe = min(64, seq_len)
+    t0 = time.perf_counter()
+    recurrent_gated_delta_rule_ref(**prefix(probe), output_final_state=True)
+    per_token = (time.perf_counter() - t0) / probe
+    tokens = max(probe, min(seq_len, int(target_seconds / per_token)))
+    t0 = time.perf_counter()
+    recurrent_gated_delta_rule_ref(**prefix(tokens), output_final_state=True)
+    seconds = time.perf_counter() - t0
+
+    t0 = time.perf_counter()
+    recurrent_gated_delta_rule_c(**prefix(seq_len), output_final_state=True, f64_state=False)
+    c_seconds = time.perf_counter() - t0
+
+    return {
+        "value": round(tokens / seconds, 1),
+        "unit": "tokens/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"first sequence of {w.name}, first {tokens} of {seq_len} tokens, all {w.H} heads, fp32, "
+                  f"torch token loop ({seconds:.1f} s)",
+        "c_port_tokens_per_s": round(seq_len / c_seconds, 1),
+        "c_port_sample": f"same sequence, all {seq_len} tokens, C restatement with OpenMP over heads ({c_seconds:.2f} s)",
+    }  # fmt: skip
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this build has no multi-GPU path (got --gpus {args.gpus}). "
+              "The operator shards over sequences and heads without any exchange; run one process per GPU.",
+              file=sys.stderr)  # fmt: skip
+        sys.exit(2)
+
+    import torch
+
+    from lm_engine_amd.workloads import get_workload
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU: the gated delta rule has no CPU path", file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.set_device(0)
+
+    w = get_workload(args.workload)
+    result, inp = bench_chunk(w, args.steps, args.warmup)
+    decode = None if args.no_decode else bench_decode(args.steps, args.warmup)
+    baseline = None if args.no_cpu_baseline else cpu_baseline(w, inp, args.cpu_seconds)
+
+    line = {
+        "metric": result["metric"],
+        "value": result["value"],
+        "unit": result["unit"],
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": result["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": result["dtype"],
+        "data": "synthetic",
+        "config": result["config"],
+        "roofline": result["roofline"],
+        "cpu_baseline": baseline,
+        "step": result["step"],
+        "decode": decode,
+        "device": torch.cuda.get_device_name(0),
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

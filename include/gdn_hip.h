@@ -7,9 +7,9 @@
  * and calls both with keywords q, k, v, g, beta, scale, initial_state, output_final_state,
  * cu_seqlens, use_qk_l2norm_in_kernel (module.py:197-222).  The entry points below are what a
  * binding for those two functions needs; every pointer is a DEVICE pointer owned by the
- * caller.  Except for the per-device kernel attribute set-up done on first use, the library
- * holds no state, never allocates, frees or synchronises, and launches asynchronously on the
- * stream it is given (current device of the calling thread).
+ * caller.  The library holds no state, never allocates, frees or synchronises (the measurement
+ * aid gdn_chunk_fwd_profile excepted), and launches asynchronously on the stream it is given
+ * (current device of the calling thread).
  *
  * Return value of every int-returning entry point: 0 on success, a negative gdn_status on
  * rejected arguments, a positive hipError_t if a launch failed.
@@ -112,6 +112,16 @@ int gdn_chunk_fwd(const gdn_args *args, void *stream);
  * gated_deltanet/module.py:210-222.  `stream` is a hipStream_t.
  */
 int gdn_recurrent_fwd(const gdn_args *args, void *stream);
+
+/*
+ * Measurement aid, no counterpart in the reference: runs exactly what gdn_chunk_fwd runs, with a
+ * HIP event recorded on `stream` before and after every kernel, waits for the last one and
+ * returns each kernel's duration in milliseconds in kernel_ms[GDN_CHUNK_KERNELS], in launch
+ * order: [0] chunk offsets of packed sequences (0 when cu_seqlens is NULL), [1] prepare, [2] scan.
+ * Unlike every other entry point it creates events and blocks the calling thread.
+ */
+#define GDN_CHUNK_KERNELS 3
+int gdn_chunk_fwd_profile(const gdn_args *args, void *stream, float *kernel_ms);
 
 #ifdef __cplusplus
 }

@@ -26,7 +26,11 @@ EXPORTED_SYMBOLS = (
     "gdn_workspace_bytes",
     "gdn_chunk_fwd",
     "gdn_recurrent_fwd",
+    "gdn_chunk_fwd_profile",
 )
+
+GDN_CHUNK_KERNELS = 3
+CHUNK_KERNEL_NAMES = ("chunk_offsets", "chunk_prepare", "chunk_scan")
 
 
 class GdnArgs(ctypes.Structure):
@@ -77,6 +81,8 @@ def load_library() -> ctypes.CDLL:
     lib.gdn_chunk_fwd.restype = ctypes.c_int
     lib.gdn_recurrent_fwd.argtypes = [ctypes.POINTER(GdnArgs), ctypes.c_void_p]
     lib.gdn_recurrent_fwd.restype = ctypes.c_int
+    lib.gdn_chunk_fwd_profile.argtypes = [ctypes.POINTER(GdnArgs), ctypes.c_void_p, ctypes.POINTER(ctypes.c_float)]
+    lib.gdn_chunk_fwd_profile.restype = ctypes.c_int
 
     version = lib.gdn_abi_version()
     if version != GDN_ABI_VERSION:

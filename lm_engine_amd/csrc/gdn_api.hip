@@ -77,13 +77,41 @@ int gdn_recurrent_fwd(const gdn_args* a, void* stream) {
     return gdn::launch_recurrent(*a, static_cast<hipStream_t>(stream));
 }
 
-int gdn_chunk_fwd(const gdn_args* a, void* stream) {
+static int validate_chunk(const gdn_args* a) {
     const int rc = validate_common(a);
     if (rc != GDN_OK) return rc;
     if (!gdn::chunk_shape_supported(*a)) return GDN_ERR_UNSUPPORTED;
     const uint64_t need = gdn::chunk_workspace_bytes(*a);
     if (a->workspace == nullptr || a->workspace_bytes < need || !aligned(a->workspace, 256)) return GDN_ERR_WORKSPACE;
+    return GDN_OK;
+}
+
+int gdn_chunk_fwd(const gdn_args* a, void* stream) {
+    const int rc = validate_chunk(a);
+    if (rc != GDN_OK) return rc;
     return gdn::launch_chunk_fwd(*a, static_cast<hipStream_t>(stream));
+}
+
+int gdn_chunk_fwd_profile(const gdn_args* a, void* stream, float* kernel_ms) {
+    if (kernel_ms == nullptr) return GDN_ERR_NULL;
+    int rc = validate_chunk(a);
+    if (rc != GDN_OK) return rc;
+    hipEvent_t events[GDN_CHUNK_KERNELS + 1];
+    int created = 0;
+    for (; created <= GDN_CHUNK_KERNELS; created++)
+        if (hipError_t e = hipEventCreate(&events[created]); e != hipSuccess) {
+            rc = (int)e;
+            break;
+        }
+    if (rc == GDN_OK) rc = gdn::launch_chunk_fwd(*a, static_cast<hipStream_t>(stream), events);
+    if (rc == GDN_OK) rc = (int)hipEventSynchronize(events[GDN_CHUNK_KERNELS]);
+    for (int i = 0; rc == GDN_OK && i < GDN_CHUNK_KERNELS; i++) {
+        kernel_ms[i] = 0.f;
+        if (i == 0 && a->cu_seqlens == nullptr) continue;
+        rc = (int)hipEventElapsedTime(&kernel_ms[i], events[i], events[i + 1]);
+    }
+    for (int i = 0; i < created; i++) (void)hipEventDestroy(events[i]);
+    return rc;
 }
 
 }  // extern "C"

@@ -159,6 +159,35 @@ def _run(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_se
     return o, ht
 
 
+def chunk_forward_kernel_times(
+    q, k, v, g=None, beta=None, scale=None, initial_state=None, output_final_state=False, cu_seqlens=None,
+    use_qk_l2norm_in_kernel=False,
+) -> dict[str, float]:  # fmt: skip
+    """Runs the chunked forward once through ``gdn_chunk_fwd_profile`` and returns the duration of
+    each of its kernels in milliseconds, measured with HIP events on the launch stream.  Same
+    arguments as ``chunk_gated_delta_rule``; blocks until the kernels have finished."""
+    _require_hip_path()
+    lib = _lib.load_library()
+    dims = _check_inputs(q, k, v, g, beta, initial_state, cu_seqlens)
+    B, T, H, K, V, N = dims
+    q, k, v = _last_dim_contiguous(q), _last_dim_contiguous(k), _last_dim_contiguous(v)
+    g = None if g is None else g.to(torch.float32).contiguous()
+    beta = None if beta is None else beta.contiguous()
+    cu_seqlens = None if cu_seqlens is None else cu_seqlens.to(torch.int32).contiguous()
+    h0 = None if initial_state is None else initial_state.contiguous()
+    o = torch.empty(B, T, H, V, dtype=v.dtype, device=v.device)
+    ht = torch.empty(N, H, K, V, dtype=torch.float32, device=v.device) if output_final_state else None
+    args = _fill_args(q, k, v, g, beta, h0, ht, o, cu_seqlens, scale, use_qk_l2norm_in_kernel, False, dims)
+    times = (ctypes.c_float * _lib.GDN_CHUNK_KERNELS)()
+    with torch.cuda.device(q.device):
+        workspace = torch.empty(max(int(lib.gdn_workspace_bytes(ctypes.byref(args))), 256), dtype=torch.uint8,
+                                device=q.device)  # fmt: skip
+        args.workspace, args.workspace_bytes = workspace.data_ptr(), workspace.numel()
+        stream = ctypes.c_void_p(torch.cuda.current_stream(q.device).cuda_stream)
+        _lib.check_status(lib.gdn_chunk_fwd_profile(ctypes.byref(args), stream, times), "gdn_chunk_fwd_profile")
+    return dict(zip(_lib.CHUNK_KERNEL_NAMES, (float(x) for x in times)))
+
+
 class _ForwardOnly(torch.autograd.Function):
     """The operator has no backward yet; differentiating through it must fail, not pass silently."""
 
