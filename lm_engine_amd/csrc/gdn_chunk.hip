@@ -40,59 +40,10 @@
 
 #include <type_traits>
 
-#include "gdn_common.h"
+#include "gdn_chunk_common.h"
 #include "gdn_launch.h"
 
 namespace gdn {
-
-constexpr int C = 64;  // chunk length
-constexpr int PREP_THREADS = 256;
-constexpr int FRAG_BYTES = WAVE * 16;  // one MFMA operand fragment: 8 bf16 per lane
-
-struct ChunkParams {
-    const bf16_t* q;
-    const bf16_t* k;
-    const bf16_t* v;
-    const void* beta;
-    const float* g;
-    const float* h0;
-    float* ht;
-    bf16_t* o;
-    const int32_t* cu_seqlens;
-    int32_t* chunk_off;  // [N + 1] prefix of chunks per sequence (packed input only)
-    uint8_t* rec;        // workspace records, [H][TC]
-    int64_t q_stride_b, q_stride_t, q_stride_h;
-    int64_t k_stride_b, k_stride_t, k_stride_h;
-    int64_t v_stride_b, v_stride_t, v_stride_h;
-    int64_t o_stride_b, o_stride_t, o_stride_h;
-    int B, T, H, V, N;
-    int NT;  // chunks per sequence (fixed-length input)
-    int TC;  // chunk slots per head
-    int beta_dtype;
-    int l2norm;
-    float scale;
-    uint32_t rec_bytes, off_qs, off_kt, off_p, off_u, off_eg;
-    int scan_groups;  // workgroups per (sequence, head) in the scan kernel
-};
-
-struct RecordLayout {
-    uint32_t off_wn, off_qs, off_kt, off_p, off_u, off_eg, bytes;
-};
-
-// Record of one (head, chunk): Wn (-W), Qs, Kt, P as A-operand fragments, U as accumulator
-// fragments, e^{gamma_C}.
-static RecordLayout record_layout(int K, int V) {
-    RecordLayout r;
-    const uint32_t kfrag = (uint32_t)(C / 16) * (K / 32) * FRAG_BYTES;  // [C x K] or [K x C] bf16
-    r.off_wn = 0;
-    r.off_qs = kfrag;
-    r.off_kt = 2 * kfrag;
-    r.off_p = 3 * kfrag;
-    r.off_u = r.off_p + (C / 16) * (C / 32) * FRAG_BYTES;
-    r.off_eg = r.off_u + (uint32_t)C * V * 2;
-    r.bytes = (r.off_eg + 4 + 255u) & ~255u;
-    return r;
-}
 
 static int chunk_slots(const gdn_args& a) {
     const int nt = (a.T + C - 1) / C;
@@ -143,56 +94,6 @@ __global__ __launch_bounds__(256) void chunk_offsets_kernel(const int32_t* __res
         off[n] = run;
         run += (cu[n + 1] - cu[n] + C - 1) / C;
     }
-}
-
-// Where chunk slot `slot` of the grid lives: sequence, first token, valid length (0 = unused slot).
-struct ChunkCoord {
-    int n;
-    int64_t b, t0;
-    int len;
-};
-
-__device__ __forceinline__ ChunkCoord locate_chunk(const ChunkParams& p, int slot) {
-    ChunkCoord cc;
-    if (p.cu_seqlens == nullptr) {
-        cc.n = slot / p.NT;
-        const int c = slot - cc.n * p.NT;
-        cc.b = cc.n;
-        cc.t0 = (int64_t)c * C;
-        cc.len = min(C, p.T - c * C);
-        return cc;
-    }
-    cc.b = 0;
-    if (slot >= p.chunk_off[p.N]) {
-        cc.n = 0, cc.t0 = 0, cc.len = 0;
-        return cc;
-    }
-    int lo = 0, hi = p.N;  // largest n with chunk_off[n] <= slot
-    while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (p.chunk_off[mid] <= slot) lo = mid;
-        else hi = mid;
-    }
-    cc.n = lo;
-    const int c = slot - p.chunk_off[lo];
-    cc.t0 = (int64_t)p.cu_seqlens[lo] + (int64_t)c * C;
-    cc.len = min(C, p.cu_seqlens[lo + 1] - (int)cc.t0);
-    return cc;
-}
-
-__device__ __forceinline__ f32x4 mfma_bf16(bf16x8 a, bf16x8 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
-}
-
-__device__ __forceinline__ f32x4 mfma_f32(float a, float b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
-}
-
-__device__ __forceinline__ bf16x8 pack8(f32x4 lo, f32x4 hi) {
-    bf16x8 r;
-    r[0] = (bf16_t)lo[0], r[1] = (bf16_t)lo[1], r[2] = (bf16_t)lo[2], r[3] = (bf16_t)lo[3];
-    r[4] = (bf16_t)hi[0], r[5] = (bf16_t)hi[1], r[6] = (bf16_t)hi[2], r[7] = (bf16_t)hi[3];
-    return r;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -652,309 +553,43 @@ __global__ __launch_bounds__(NW* WAVE) void chunk_scan_kernel(const ChunkParams 
 }
 
 // ------------------------------------------------------------------------------------------
-// scan, LDS-staged and wave-specialised: the same arithmetic as chunk_scan_kernel.
-//
-// A workgroup is NL loader waves + NW compute waves working on one (sequence, head).  Everything
-// a chunk needs from its record (the A-operand fragments W, Q~, K~^T, P, the U tiles of this
-// workgroup's columns and e^{gamma_C}) goes through a double buffer in LDS: during iteration c
-// the loaders move record c + 1 global -> registers -> LDS (plain 16 B loads; the global->LDS DMA
-// path measured ~16 B/clk per CU here, four times slower) and issue the loads of record c + 2,
-// while the compute waves run the 56 MFMAs of chunk c out of the other half.  One workgroup
-// barrier per chunk, placed where a compute wave has pulled the last operand of the chunk into
-// registers, hands the halves over; the first reads of chunk c + 1 then run under the last MFMA
-// phase of chunk c.  The compute waves issue no vector-memory loads in
-// the loop, so the copy's issue stalls stay out of the MFMA waves.  Each compute wave owns 16
-// columns of the state.  O is accumulated transposed (operands of its MFMAs swapped) so that a
-// lane ends up with 4 consecutive columns of one token: 4 stores of 8 B per chunk instead of 16
-// of 2 B.
-// ------------------------------------------------------------------------------------------
-template <int K, int NW>
-__global__ __launch_bounds__((NW + 2) * WAVE) void chunk_scan_lds_kernel(const ChunkParams p) {
-    constexpr int NL = 2;  // loader waves
-    constexpr int KT = K / 16;
-    constexpr int KS = K / 32;
-    constexpr int KFRAG = (C / 16) * KS * FRAG_BYTES;                     // bytes of W, Qs or Kt fragments
-    constexpr int SHARED_BYTES = 3 * KFRAG + (C / 16) * 2 * FRAG_BYTES;  // W, Qs, Kt, P: contiguous in the record
-    constexpr int SHARED_FRAGS = SHARED_BYTES / FRAG_BYTES;
-    constexpr int U_FRAGS = 2 * NW;  // U tiles of this workgroup's columns: contiguous in the record
-    constexpr int STAGE_FRAGS = SHARED_FRAGS + U_FRAGS;
-    constexpr int STAGE_BYTES = STAGE_FRAGS * FRAG_BYTES + 16;  // + e^{gamma_C}
-    constexpr int NLOAD = STAGE_FRAGS / NL;                     // fragments moved by each loader wave
-    static_assert(2 * STAGE_BYTES <= 160 * 1024, "double buffer exceeds LDS");
-    static_assert(STAGE_FRAGS % NL == 0 && SHARED_FRAGS % NL == 0, "fragments must divide over the loader waves");
-
-    __shared__ __attribute__((aligned(16))) uint8_t stage[2][STAGE_BYTES];
-
-    const int lane = threadIdx.x % WAVE;
-    const int wave = threadIdx.x / WAVE;
-    const int l16 = lane % 16;
-    const int lq = lane / 16;
-
-    const int id = blockIdx.x;
-    const int xcd = id % 8, rest = id / 8;
-    const int vgroup = rest % p.scan_groups;
-    const int chain = (rest / p.scan_groups) * 8 + xcd;
-    if (chain >= p.N * p.H) return;  // whole workgroup
-    const int n = chain / p.H, h = chain % p.H;
-
-    int slot_begin, slot_end;
-    int64_t b, seq_t0, seq_len;
-    if (p.cu_seqlens == nullptr) {
-        slot_begin = n * p.NT, slot_end = slot_begin + p.NT;
-        b = n, seq_t0 = 0, seq_len = p.T;
-    } else {
-        slot_begin = p.chunk_off[n], slot_end = p.chunk_off[n + 1];
-        b = 0, seq_t0 = p.cu_seqlens[n], seq_len = p.cu_seqlens[n + 1] - seq_t0;
-    }
-    const int nchunks = slot_end - slot_begin;
-    const uint8_t* rec = p.rec + ((int64_t)h * p.TC + slot_begin) * p.rec_bytes;
-
-    if (wave >= NW) {
-        // ------------------------------ loader ------------------------------
-        // fragment f of the stage: f < SHARED_FRAGS comes from the head of the record, the rest
-        // from this workgroup's slice of the U block
-        const int lw = wave - NW;
-        const int64_t u_shift = (int64_t)p.off_u + (int64_t)vgroup * U_FRAGS * FRAG_BYTES - SHARED_BYTES;
-        // two register buffers: while one record is written to LDS, two younger ones are in flight
-        bf16x8 buf0[NLOAD], buf1[NLOAD];
-        float eg0 = 0.f, eg1 = 0.f;
-        auto src_of = [&](int c, int i) {
-            const int f = lw * NLOAD + i;
-            return rec + (int64_t)c * p.rec_bytes + (int64_t)f * FRAG_BYTES + (f >= SHARED_FRAGS ? u_shift : 0) + lane * 16;
-        };
-        auto load = [&](bf16x8(&buf)[NLOAD], float& eg, int c) {
-#pragma unroll
-            for (int i = 0; i < NLOAD; i++) buf[i] = *reinterpret_cast<const bf16x8*>(src_of(c, i));
-            if (lw == 0) eg = *reinterpret_cast<const float*>(rec + (int64_t)c * p.rec_bytes + p.off_eg);
-        };
-        auto store = [&](const bf16x8(&buf)[NLOAD], float eg, int c) {
-            uint8_t* dst = stage[c & 1];
-            bf16x8* d = reinterpret_cast<bf16x8*>(dst) + (lw * NLOAD) * WAVE + lane;
-#pragma unroll
-            for (int i = 0; i < NLOAD; i++) d[i * WAVE] = buf[i];
-            if (lw == 0 && lane == 0) *reinterpret_cast<float*>(dst + STAGE_FRAGS * FRAG_BYTES) = eg;
-        };
-        // write record c to LDS and refill each register with record c2 right behind its write,
-        // so the LDS-write and the vector-memory queues fill together
-        auto store_and_reload = [&](bf16x8(&buf)[NLOAD], float& eg, int c, int c2, auto reload_tag) {
-            constexpr bool reload = decltype(reload_tag)::value;
-            uint8_t* dst = stage[c & 1];
-            bf16x8* d = reinterpret_cast<bf16x8*>(dst) + (lw * NLOAD) * WAVE + lane;
-            if (lw == 0 && lane == 0) *reinterpret_cast<float*>(dst + STAGE_FRAGS * FRAG_BYTES) = eg;
-#pragma unroll
-            for (int i = 0; i < NLOAD; i++) {
-                d[i * WAVE] = buf[i];
-                if constexpr (reload) buf[i] = *reinterpret_cast<const bf16x8*>(src_of(c2, i));
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            if constexpr (reload) {
-                if (lw == 0) eg = *reinterpret_cast<const float*>(rec + (int64_t)c2 * p.rec_bytes + p.off_eg);
-            }
-        };
-        // records 0 (-> LDS now), 1 and 2 (in flight); even records use buf0, odd ones buf1
-        if (nchunks > 0) {
-            load(buf0, eg0, 0);
-            if (nchunks > 1) load(buf1, eg1, 1);
-            store(buf0, eg0, 0);
-            if (nchunks > 2) load(buf0, eg0, 2);
-        }
-        __syncthreads();  // stage[0] holds record 0
-        // barrier of iteration c: the compute waves have read all of stage[c & 1] into registers and
-        // record c + 1 is in stage[(c + 1) & 1].  Before it: write record c + 1 (its half was released
-        // by the barrier of iteration c - 1) and refill the freed registers with record c + 3.
-        constexpr std::true_type yes{};
-        constexpr std::false_type no{};
-        int c = 0;
-        for (; c + 4 < nchunks; c += 2) {  // steady state: straight-line code, both reloads exist
-            store_and_reload(buf1, eg1, c + 1, c + 3, yes);
-            __syncthreads();
-            store_and_reload(buf0, eg0, c + 2, c + 4, yes);
-            __syncthreads();
-        }
-        for (; c < nchunks; c += 2) {  // the last (at most four) chunks
-            if (c + 1 < nchunks) {
-                if (c + 3 < nchunks) store_and_reload(buf1, eg1, c + 1, c + 3, yes);
-                else store_and_reload(buf1, eg1, c + 1, 0, no);
-            }
-            __syncthreads();
-            if (c + 1 < nchunks) {
-                if (c + 2 < nchunks) store_and_reload(buf0, eg0, c + 2, 0, no);
-                __syncthreads();
-            }
-        }
-        return;
-    }
-
-    // ------------------------------ compute ------------------------------
-    const int tn = vgroup * NW + wave;  // host guarantees V / 16 is a multiple of NW
-    f32x4 S[KT];
-    const int64_t st_off = ((int64_t)n * p.H + h) * K * p.V + (int64_t)(4 * lq) * p.V + 16 * tn + l16;
-    if (p.h0 != nullptr) {
-#pragma unroll
-        for (int t = 0; t < KT; t++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) S[t][e] = p.h0[st_off + (int64_t)(16 * t + e) * p.V];
-    } else {
-#pragma unroll
-        for (int t = 0; t < KT; t++) S[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-    }
-    // O^T tile ti: lane holds token 16 ti + l16, columns 16 tn + 4 lq + 0..3
-    bf16_t* const og = p.o + b * p.o_stride_b + (seq_t0 + l16) * p.o_stride_t + (int64_t)h * p.o_stride_h + 16 * tn +
-                       4 * lq;
-
-    // Operands of the first MFMA phase of a chunk (W, Q~, U, e^{gamma_C}).  LDS reads are issued
-    // one at a time between the MFMAs of the previous phase: a wave64 16 B read occupies the LDS
-    // return path for ~20 cycles, about what one MFMA takes, so the two streams hide each other.
-    constexpr int HEAD_READS = 2 + 8 * KS;  // U (2), W (4 KS), Q~ (4 KS)
-    constexpr int TAIL_READS = 2 * KT + 8;  // K~^T (2 KT), P (8)
-    constexpr int PHASE_A = 8 * KS;         // MFMAs of V~ = U - W S0 and O^T = S0^T Q~^T
-    constexpr int PHASE_B = 2 * (KT + 4);   // MFMAs of the state update and O^T += V~^T P^T
-    bf16x8 wr[4 * KS], qr[4 * KS], kr[KT * 2], pr[8], u01 = {}, u23 = {};
-    float egc = 0.f;
-    auto read_head = [&](const uint8_t* st, int r) {
-        if (r < 2) {
-            const bf16x8* uf = reinterpret_cast<const bf16x8*>(st + SHARED_BYTES) + (wave * WAVE + lane) * 2;
-            if (r == 0) u01 = uf[0];
-            else u23 = uf[1];
-        } else if (r < 2 + 4 * KS) {
-            wr[r - 2] = reinterpret_cast<const bf16x8*>(st)[(r - 2) * WAVE + lane];
-        } else {
-            qr[r - 2 - 4 * KS] = reinterpret_cast<const bf16x8*>(st + KFRAG)[(r - 2 - 4 * KS) * WAVE + lane];
-        }
-    };
-    auto read_tail = [&](const uint8_t* st, int r) {
-        if (r < 2 * KT) kr[r] = reinterpret_cast<const bf16x8*>(st + 2 * KFRAG)[r * WAVE + lane];
-        else pr[r - 2 * KT] = reinterpret_cast<const bf16x8*>(st + 3 * KFRAG)[(r - 2 * KT) * WAVE + lane];
-    };
-
-    __syncthreads();  // stage[0] holds record 0
-    if (nchunks > 0) {
-        egc = *reinterpret_cast<const float*>(stage[0] + STAGE_FRAGS * FRAG_BYTES);
-#pragma unroll
-        for (int r = 0; r < HEAD_READS; r++) read_head(stage[0], r);
-    }
-
-    auto iteration = [&](int c, auto more_tag) {
-        constexpr bool more = decltype(more_tag)::value;
-        const uint8_t* st = stage[c & 1];
-        const uint8_t* st_next = stage[(c + 1) & 1];
-
-        bf16x8 sb[KS];
-#pragma unroll
-        for (int s = 0; s < KS; s++) sb[s] = pack8(S[2 * s], S[2 * s + 1]);
-        f32x4 accv[4], acco[4];
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            accv[0][e] = (float)u01[e], accv[1][e] = (float)u01[4 + e];
-            accv[2][e] = (float)u23[e], accv[3][e] = (float)u23[4 + e];
-        }
-#pragma unroll
-        for (int ti = 0; ti < 4; ti++) acco[ti] = f32x4{0.f, 0.f, 0.f, 0.f};
-        const float eg_cur = egc;
-        __builtin_amdgcn_sched_barrier(0);
-
-        // phase A: V~ = U - W S0, then O^T = S0^T Q~^T; consecutive MFMAs go to different
-        // accumulators; the reads of K~^T and P ride along
-#pragma unroll
-        for (int i = 0; i < PHASE_A; i++) {
-            const int j = i % (4 * KS), s = j / 4, ti = j % 4;
-            if (i < 4 * KS) accv[ti] = mfma_bf16(wr[ti * KS + s], sb[s], accv[ti]);
-            else acco[ti] = mfma_bf16(sb[s], qr[ti * KS + s], acco[ti]);
-#pragma unroll
-            for (int r = i * TAIL_READS / PHASE_A; r < (i + 1) * TAIL_READS / PHASE_A; r++) read_tail(st, r);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-
-        bf16x8 vb[2];
-        vb[0] = pack8(accv[0], accv[1]);
-        vb[1] = pack8(accv[2], accv[3]);
-#pragma unroll
-        for (int t = 0; t < KT; t++) S[t] = S[t] * eg_cur;
-        __builtin_amdgcn_sched_barrier(0);
-
-        // every operand of this chunk is in registers: release this LDS half, take the next one
-        __syncthreads();
-        if constexpr (more) egc = *reinterpret_cast<const float*>(st_next + STAGE_FRAGS * FRAG_BYTES);
-        __builtin_amdgcn_sched_barrier(0);
-
-        // phase B: S = e^{gamma_C} S + K~^T V~ and O^T += V~^T P^T; the head reads of chunk c + 1 ride along
-#pragma unroll
-        for (int i = 0; i < PHASE_B; i++) {
-            const int s = i / (KT + 4), j = i % (KT + 4);
-            if (j < KT) S[j] = mfma_bf16(kr[j * 2 + s], vb[s], S[j]);
-            else acco[j - KT] = mfma_bf16(vb[s], pr[(j - KT) * 2 + s], acco[j - KT]);
-            if constexpr (more) {
-#pragma unroll
-                for (int r = i * HEAD_READS / PHASE_B; r < (i + 1) * HEAD_READS / PHASE_B; r++) read_head(st_next, r);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-
-        const int64_t tok0 = (int64_t)c * C;
-        const int valid = (int)min((int64_t)C, seq_len - tok0);
-#pragma unroll
-        for (int ti = 0; ti < 4; ti++) {
-            bf16x4 r;
-            r[0] = (bf16_t)acco[ti][0], r[1] = (bf16_t)acco[ti][1], r[2] = (bf16_t)acco[ti][2], r[3] = (bf16_t)acco[ti][3];
-            if (16 * ti + l16 < valid) *reinterpret_cast<bf16x4*>(og + (tok0 + 16 * ti) * p.o_stride_t) = r;
-        }
-    };
-    for (int c = 0; c + 1 < nchunks; c++) iteration(c, std::true_type{});
-    if (nchunks > 0) iteration(nchunks - 1, std::false_type{});
-
-    if (p.ht != nullptr) {
-#pragma unroll
-        for (int t = 0; t < KT; t++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) p.ht[st_off + (int64_t)(16 * t + e) * p.V] = S[t][e];
-    }
-}
-
-// ------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------
-template <int K>
-static int launch_chunk_k(ChunkParams& p, hipStream_t stream, hipEvent_t* events) {
-    auto mark = [&](int i) {
-        if (events != nullptr) (void)hipEventRecord(events[i], stream);
-    };
-    mark(0);
-    if (p.cu_seqlens != nullptr) {
-        hipLaunchKernelGGL(chunk_offsets_kernel, dim3(1), dim3(256), 0, stream, p.cu_seqlens, p.chunk_off, p.N);
-        if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
+int launch_chunk32(ChunkParams& p, int K, hipStream_t stream, hipEvent_t* events, int num_cus);  // gdn_chunk32.hip
+
+static int compute_units() {
+    static int cached[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev] = n;
     }
-    mark(1);
+    return cached[dev];
+}
+
+// K = 256: 16x16x32 kernels of this file (one workgroup per chunk in prepare, 16-column waves in the scan)
+static int launch_chunk_256(ChunkParams& p, hipStream_t stream, hipEvent_t* events) {
+    constexpr int K = 256;
     hipLaunchKernelGGL((chunk_prepare_kernel<K>), dim3(p.TC, p.H), dim3(PREP_THREADS), 0, stream, p);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
-    mark(2);
+    if (events != nullptr) (void)hipEventRecord(events[2], stream);
 
     // waves per workgroup: as many as keep at least ~one workgroup per CU
     const int64_t chains = (int64_t)p.N * p.H;
     const int vtiles = p.V / 16;
     const int64_t waves = chains * vtiles;
     int nw = 1;
-    if constexpr (K > 128) {
-        if (waves >= 4 * 256 && vtiles % 4 == 0) nw = 4;
-        else if (waves >= 2 * 256 && vtiles % 2 == 0) nw = 2;
-    } else {
-        // the LDS-staged kernel runs one wave per SIMD (it needs the whole register file): at most
-        // two compute waves next to the two loader waves
-        if (waves >= 2 * 256 && vtiles % 2 == 0) nw = 2;
-    }
+    if (waves >= 4 * 256 && vtiles % 4 == 0) nw = 4;
+    else if (waves >= 2 * 256 && vtiles % 2 == 0) nw = 2;
     p.scan_groups = (vtiles + nw - 1) / nw;
     const int64_t chains8 = (chains + 7) / 8 * 8;
     const dim3 grid((unsigned)(chains8 * p.scan_groups));
-    if constexpr (K <= 128) {  // the double-buffered record fits LDS
-        if (nw == 2) hipLaunchKernelGGL((chunk_scan_lds_kernel<K, 2>), grid, dim3(4 * WAVE), 0, stream, p);
-        else hipLaunchKernelGGL((chunk_scan_lds_kernel<K, 1>), grid, dim3(3 * WAVE), 0, stream, p);
-    } else {
-        if (nw == 4) hipLaunchKernelGGL((chunk_scan_kernel<K, 4>), grid, dim3(4 * WAVE), 0, stream, p);
-        else if (nw == 2) hipLaunchKernelGGL((chunk_scan_kernel<K, 2>), grid, dim3(2 * WAVE), 0, stream, p);
-        else hipLaunchKernelGGL((chunk_scan_kernel<K, 1>), grid, dim3(WAVE), 0, stream, p);
-    }
-    const hipError_t e = hipGetLastError();
-    mark(3);
-    return (int)e;
+    if (nw == 4) hipLaunchKernelGGL((chunk_scan_kernel<K, 4>), grid, dim3(4 * WAVE), 0, stream, p);
+    else if (nw == 2) hipLaunchKernelGGL((chunk_scan_kernel<K, 2>), grid, dim3(2 * WAVE), 0, stream, p);
+    else hipLaunchKernelGGL((chunk_scan_kernel<K, 1>), grid, dim3(WAVE), 0, stream, p);
+    return (int)hipGetLastError();
 }
 
 int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events) {
@@ -984,12 +619,19 @@ int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events) 
     p.rec_bytes = r.bytes, p.off_qs = r.off_qs, p.off_kt = r.off_kt, p.off_p = r.off_p, p.off_u = r.off_u;
     p.off_eg = r.off_eg;
     p.scan_groups = 1;
-    switch (a.K) {
-        case 64: return launch_chunk_k<64>(p, stream, events);
-        case 128: return launch_chunk_k<128>(p, stream, events);
-        case 256: return launch_chunk_k<256>(p, stream, events);
-        default: return GDN_ERR_UNSUPPORTED;
+
+    auto mark = [&](int i) {
+        if (events != nullptr) (void)hipEventRecord(events[i], stream);
+    };
+    mark(0);
+    if (p.cu_seqlens != nullptr) {
+        hipLaunchKernelGGL(chunk_offsets_kernel, dim3(1), dim3(256), 0, stream, p.cu_seqlens, p.chunk_off, p.N);
+        if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
     }
+    mark(1);
+    const int rc = (a.K == 256) ? launch_chunk_256(p, stream, events) : launch_chunk32(p, a.K, stream, events, compute_units());
+    mark(3);
+    return rc;
 }
 
 }  // namespace gdn

@@ -1,0 +1,733 @@
+// Chunked forward of the gated delta rule, K <= 128: kernels built on v_mfma_f32_32x32x16_bf16
+// (the only bf16 MFMA shape that reaches the full matrix-core rate on gfx950; 16x16x32 measured
+// ~0.8x of it).
+//
+// Same mathematics and the same two-kernel split as gdn_chunk.hip (prepare: everything that
+// does not depend on the state, written as MFMA operand fragments to a workspace record per
+// (head, chunk); scan: the serial pass over the chunks of a sequence with the state held in
+// MFMA accumulators).  What differs:
+//
+//   * a wave of the scan owns a K x 32 slice of the state; operand fragments are laid out for
+//     the 32x32x16 shape;
+//   * the scan has no LDS and no barrier: every wave streams its fragments global -> registers
+//     with a rolling prefetch (the registers of fragment i are reloaded from the next record
+//     right after the MFMA that consumed them), one vector load between two MFMAs;
+//   * prepare is persistent: a workgroup walks over (chunk, head) items and loads q, k, v of
+//     the next item into registers while it computes the current one;
+//   * the triangular inverse runs its block products on bf16 MFMA with operands split into
+//     hi + lo halves (error ~2^-16, far below the final bf16 rounding of T), and transposed
+//     operands come from ds_read_tr16_b64 instead of 2-byte gathers.
+//
+// 32x32x16 layouts (wave64, l = lane, h = l / 32):
+//   A[i = l%32][k = 8 h + 0..7]    B[k = 8 h + 0..7][j = l%32]
+//   D[i = 8 (r/4) + 4 h + r%4][j = l%32]   for accumulator register r = 0..15
+//
+// Permuted reduction order: a D tile reused as B (or A) operand gives, for the 16-row slab s of
+// the tile (s = 0, 1), registers 8 s .. 8 s + 7, i.e. rows 16 s + 4 h + 0..3 and 16 s + 8 + 4 h + 0..3.
+// The matching fragment of a row-major matrix Y holds Y[m][16 s' + 4 h + 0..3], Y[m][16 s' + 8 + 4 h + 0..3]
+// for the global slab index s' (16 reduction entries per slab).
+//
+// Record (same sizes and offsets as the 16x16 variant):
+//   W~  = -W       [T_tok 2][slab K/16]  A fragments, rows = tokens, reduction = key dim
+//   Q~             [T_tok 2][slab K/16]  B fragments of O^T = S^T Q~^T (same register layout)
+//   K~^T           [T_d K/32][slab 4]    A fragments, rows = key dim, reduction = tokens
+//   P              [T_i 2][slab 4]       B fragments of O^T += V~^T P^T
+//   U              [T_n V/32][lane][T_tok 2][16]  accumulator layout
+//   e^{gamma_C}
+
+#include <type_traits>
+
+#include "gdn_chunk_common.h"
+#include "gdn_launch.h"
+
+namespace gdn {
+
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+
+__device__ __forceinline__ bf16x8 pack8_16(const f32x16& d, int s, float sign) {
+    bf16x8 r;
+#pragma unroll
+    for (int e = 0; e < 8; e++) r[e] = (bf16_t)(sign * d[8 * s + e]);
+    return r;
+}
+
+// 4 consecutive rows x 16 consecutive columns of a row-major bf16 LDS matrix, transposed on the
+// way in: lane i of each 16-lane group receives M[row0 + 0..3][col0 + i].
+__device__ __forceinline__ bf16x4 lds_read_tr4x16(const bf16_t* m, int ld, int row0, int col0, int l16) {
+    const bf16_t* p = m + (row0 + l16 / 4) * ld + col0 + 4 * (l16 % 4);
+    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p);
+    return __builtin_bit_cast(bf16x4, v);
+}
+
+__device__ __forceinline__ void split_hi_lo(float x, bf16_t& hi, bf16_t& lo) {
+    hi = (bf16_t)x;
+    lo = (bf16_t)(x - (float)hi);
+}
+
+// ------------------------------------------------------------------------------------------
+// prepare
+// ------------------------------------------------------------------------------------------
+template <int K>
+__global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const ChunkParams p) {
+    constexpr int LDK = K + 8;  // bf16 elements per LDS row of K / Q
+    constexpr int VP = 128;     // columns of V staged per pass
+    constexpr int LDV = VP + 8;
+    constexpr int LDA = C + 4;  // fp32 elements per LDS row of A / T
+    constexpr int LDT = 36;     // fp32 elements per row of the 32 x 32 transposed blocks
+    constexpr int LDM = 20;     // fp32 elements per row of a 16 x 16 scratch block
+    constexpr int KS16 = K / 16;
+    constexpr int KD = K / 32;  // 32-row tiles of the key dim
+    constexpr int CPR = K / 8;  // 16 B pieces per row of K / Q
+    constexpr int RPP = PREP_THREADS / CPR;  // rows per pass of the K / Q copy
+    constexpr int NPASS = C / RPP;
+    constexpr int QT_BYTES = (C * LDK * 2 > C * LDA * 4) ? C * LDK * 2 : C * LDA * 4;
+    constexpr int AV_BYTES = (C * LDV * 2 > C * LDA * 4) ? C * LDV * 2 : C * LDA * 4;
+
+    __shared__ __attribute__((aligned(16))) bf16_t sK[C * LDK];
+    __shared__ __attribute__((aligned(16))) uint8_t sQT[QT_BYTES];  // Q (bf16), then T (fp32)
+    __shared__ __attribute__((aligned(16))) uint8_t sAV[AV_BYTES];  // A (fp32), then V (bf16)
+    __shared__ __attribute__((aligned(16))) float sTtA[32 * LDT];   // transpose of the top-left 32 x 32 of T
+    __shared__ __attribute__((aligned(16))) float sTt2[16 * LDM];   // transpose of diagonal block 2 of T
+    __shared__ __attribute__((aligned(16))) float sMt[2 * 16 * LDM + 32 * LDT];  // transposed products
+    __shared__ __attribute__((aligned(16))) float s_gam[C], s_beta[C], s_ssk[C], s_ssq[C];
+    __shared__ __attribute__((aligned(16))) float s_rk[C], s_rq[C], s_cw[C], s_ks[C], s_qs[C];
+    bf16_t* const sQ = reinterpret_cast<bf16_t*>(sQT);
+    float* const sT = reinterpret_cast<float*>(sQT);
+    float* const sA = reinterpret_cast<float*>(sAV);
+    bf16_t* const sV = reinterpret_cast<bf16_t*>(sAV);
+    float* const sMtB = sMt + 2 * 16 * LDM;
+
+    const int tid = threadIdx.x;
+    const int wave = tid / WAVE;
+    const int64_t items = (int64_t)p.TC * p.H;
+
+    // ---- register prefetch of one item's inputs ----
+    bf16x8 kx[NPASS], qx[NPASS], vx[C * (VP / 8) / PREP_THREADS];
+    float gx = 0.f;
+    uint32_t bx_raw = 0;  // beta of the prefetched item, converted where it is used (a conversion here would wait for every load)
+    ChunkCoord ncc;  // coordinates of the prefetched item
+    int nh = 0;
+    auto locate = [&](int64_t w) {
+        nh = (int)(w % p.H);
+        ncc = locate_chunk(p, (int)(w / p.H));
+    };
+    // Loads are written as (workgroup-uniform base pointer) + (32-bit per-lane element offset) so that the
+    // compiler keeps one offset register per stream instead of a 64-bit address per load.
+    const uint32_t kq_piece = tid % CPR, kq_row0 = tid / CPR;
+    const uint32_t k_lane_off = kq_row0 * (uint32_t)p.k_stride_t + kq_piece * 8;
+    const uint32_t q_lane_off = kq_row0 * (uint32_t)p.q_stride_t + kq_piece * 8;
+    const uint32_t v_piece = tid % (VP / 8), v_row0 = tid / (VP / 8);
+    const uint32_t v_lane_off = v_row0 * (uint32_t)p.v_stride_t + v_piece * 8;
+    const int lane0 = tid % WAVE;
+    auto prefetch_kq = [&]() {
+        const bf16_t* kg = p.k + ncc.b * p.k_stride_b + ncc.t0 * p.k_stride_t + (int64_t)nh * p.k_stride_h;
+        const bf16_t* qg = p.q + ncc.b * p.q_stride_b + ncc.t0 * p.q_stride_t + (int64_t)nh * p.q_stride_h;
+#pragma unroll
+        for (int it = 0; it < NPASS; it++) {
+            const int row = kq_row0 + it * RPP;
+            kx[it] = bf16x8{};
+            qx[it] = bf16x8{};
+            if (row < ncc.len) {
+                kx[it] = *reinterpret_cast<const bf16x8*>(kg + (int64_t)(it * RPP) * p.k_stride_t + k_lane_off);
+                qx[it] = *reinterpret_cast<const bf16x8*>(qg + (int64_t)(it * RPP) * p.q_stride_t + q_lane_off);
+            }
+        }
+        if (wave == 0) {
+            gx = 0.f, bx_raw = 0u;
+            if (lane0 < ncc.len) {
+                const int64_t sbase = (ncc.b * p.T + ncc.t0) * p.H + nh;
+                const uint32_t soff = (uint32_t)lane0 * (uint32_t)p.H;
+                if (p.g != nullptr) gx = (p.g + sbase)[soff];
+                if (p.beta == nullptr) bx_raw = 0x3f800000u;  // 1.0f
+                else if (p.beta_dtype == GDN_BF16) bx_raw = (uint32_t)(reinterpret_cast<const uint16_t*>(p.beta) + sbase)[soff] << 16;
+                else bx_raw = (reinterpret_cast<const uint32_t*>(p.beta) + sbase)[soff];
+            }
+        }
+    };
+    auto prefetch_v = [&]() {  // first pass of V (columns 0 .. min(V, VP))
+        const bf16_t* vg = p.v + ncc.b * p.v_stride_b + ncc.t0 * p.v_stride_t + (int64_t)nh * p.v_stride_h;
+#pragma unroll
+        for (int it = 0; it < C * (VP / 8) / PREP_THREADS; it++) {
+            const int row = v_row0 + it * (PREP_THREADS / (VP / 8));
+            vx[it] = bf16x8{};
+            if (row < ncc.len && (int)v_piece * 8 < p.V)
+                vx[it] = *reinterpret_cast<const bf16x8*>(vg + (int64_t)(it * (PREP_THREADS / (VP / 8))) * p.v_stride_t + v_lane_off);
+        }
+    };
+
+    int64_t w = blockIdx.x;
+    if (w >= items) return;
+    locate(w);
+    prefetch_kq();
+    prefetch_v();
+
+    for (; w < items; w += gridDim.x) {
+        // Lane coordinates are re-derived in every iteration from a value the optimiser cannot see
+        // through: hoisted out of this loop, the many lane-dependent addresses and masks below would
+        // stay live across all phases and spill.
+        int lane = tid % WAVE;
+        asm volatile("" : "+v"(lane));
+        const int l16 = lane % 16, lq = lane / 16;  // 16 x 16 MFMA coordinates
+        const int l32 = lane % 32, lh = lane / 32;  // 32 x 32 MFMA coordinates
+        const int g16 = l32 / 16;                   // which 16-lane group of the 32-row operand
+        const ChunkCoord cc = ncc;
+        const int h = nh;
+        const int len = cc.len;  // <= 0 for an unused slot of a packed batch: nothing to do
+        uint8_t* const rec = p.rec + ((int64_t)h * p.TC + (w / p.H)) * p.rec_bytes;
+        const bool has_next = w + gridDim.x < items;
+
+        // ---- registers -> LDS (K, Q), row sums of squares, gamma = cumsum(g), beta ----
+        if (len > 0) {
+            const int piece = tid % CPR;
+#pragma unroll
+            for (int it = 0; it < NPASS; it++) {
+                const int row = tid / CPR + it * RPP;
+                *reinterpret_cast<bf16x8*>(&sK[row * LDK + piece * 8]) = kx[it];
+                *reinterpret_cast<bf16x8*>(&sQ[row * LDK + piece * 8]) = qx[it];
+                float a = 0.f, b = 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    a += (float)kx[it][e] * (float)kx[it][e];
+                    b += (float)qx[it][e] * (float)qx[it][e];
+                }
+#pragma unroll
+                for (int off = 1; off < CPR; off <<= 1) {
+                    a += __shfl_xor(a, off, WAVE);
+                    b += __shfl_xor(b, off, WAVE);
+                }
+                if (piece == 0) s_ssk[row] = a, s_ssq[row] = b;
+            }
+            if (wave == 0) {
+                float gv = gx;
+#pragma unroll
+                for (int off = 1; off < WAVE; off <<= 1) {
+                    const float up = __shfl_up(gv, off, WAVE);
+                    if (lane >= off) gv += up;
+                }
+                s_gam[lane] = gv;
+                s_beta[lane] = __builtin_bit_cast(float, bx_raw);
+            }
+        }
+        // the q, k registers are free: start on the next item
+        if (has_next) {
+            locate(w + gridDim.x);
+            prefetch_kq();
+        }
+        if (len <= 0) {  // uniform over the workgroup
+            if (has_next) prefetch_v();
+            continue;
+        }
+        __syncthreads();  // #1
+
+        if (tid < C) {
+            const float gam = s_gam[tid], gl = s_gam[C - 1];
+            const float rk = p.l2norm ? rsqrtf(s_ssk[tid] + L2NORM_EPS) : 1.f;
+            const float rq = p.l2norm ? rsqrtf(s_ssq[tid] + L2NORM_EPS) : 1.f;
+            s_rk[tid] = rk;
+            s_rq[tid] = rq;
+            s_cw[tid] = s_beta[tid] * __expf(gam) * rk;  // column scale of T for W
+            s_ks[tid] = __expf(gl - gam) * rk;           // row scale of K~
+            s_qs[tid] = __expf(gam) * p.scale * rq;      // row scale of Q~
+            if (tid == 0) *reinterpret_cast<float*>(rec + p.off_eg) = __expf(gl);
+        }
+        __syncthreads();  // #2
+
+        // ---- A = strict-lower(beta_i e^{gamma_i - gamma_j} k^_i . k^_j) -> sA;  P -> record ----
+        {
+            // 32 x 32 tile jobs: G(Ti, Tj) = K_Ti K_Tj^T (rows i, column j), Pt(Tj, Ti) = K_Tj Q_Ti^T (rows j, column i)
+            auto tile_job = [&](bool is_p, int trow, int tcol) {
+                f32x16 acc;
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[r] = 0.f;
+                const bf16_t* bsrc = is_p ? sQ : sK;
+#pragma unroll
+                for (int s = 0; s < KS16; s++) {
+                    const bf16x8 a = *reinterpret_cast<const bf16x8*>(&sK[(32 * trow + l32) * LDK + 16 * s + 8 * lh]);
+                    const bf16x8 b = *reinterpret_cast<const bf16x8*>(&bsrc[(32 * tcol + l32) * LDK + 16 * s + 8 * lh]);
+                    acc = mfma32_bf16(a, b, acc);
+                    if (s % 2 == 1) __builtin_amdgcn_sched_barrier(0);  // keeps the operand reads from piling up in registers
+                }
+                if (!is_p) {
+                    const int j = 32 * tcol + l32;
+                    const float gj = s_gam[j], rkj = s_rk[j];
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int i = 32 * trow + 8 * (r / 4) + 4 * lh + r % 4;
+                        const float val = s_beta[i] * s_rk[i] * rkj * __expf(s_gam[i] - gj) * acc[r];
+                        sA[i * LDA + j] = (i > j) ? val : 0.f;
+                    }
+                } else {
+                    const int i = 32 * tcol + l32;
+                    const float gi = s_gam[i], qi = p.scale * s_rq[i];
+                    f32x16 pv;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int j = 32 * trow + 8 * (r / 4) + 4 * lh + r % 4;
+                        const float val = qi * s_rk[j] * __expf(gi - s_gam[j]) * acc[r];
+                        pv[r] = (i >= j) ? val : 0.f;
+                    }
+                    bf16x8* pf = reinterpret_cast<bf16x8*>(rec + p.off_p);
+                    pf[(tcol * 4 + 2 * trow + 0) * WAVE + lane] = pack8_16(pv, 0, 1.f);
+                    pf[(tcol * 4 + 2 * trow + 1) * WAVE + lane] = pack8_16(pv, 1, 1.f);
+                }
+            };
+            // Q~ fragments (T_tok, slab): Q~[tok][16 s + 4 h + e], Q~[tok][16 s + 8 + 4 h + e]; made here, by the
+            // two waves with a single tile job, because the region of Q is overwritten by T after the next barrier
+            auto q_frags = [&](int first) {
+                bf16x8* qf = reinterpret_cast<bf16x8*>(rec + p.off_qs);
+                for (int f = first; f < 2 * KS16; f += 2) {
+                    const int tt = f / KS16, s = f % KS16;
+                    const int i = 32 * tt + l32;
+                    const float sc = s_qs[i];
+                    const bf16x4 a = *reinterpret_cast<const bf16x4*>(&sQ[i * LDK + 16 * s + 4 * lh]);
+                    const bf16x4 b = *reinterpret_cast<const bf16x4*>(&sQ[i * LDK + 16 * s + 8 + 4 * lh]);
+                    bf16x8 r;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        r[e] = (bf16_t)((float)a[e] * sc);
+                        r[4 + e] = (bf16_t)((float)b[e] * sc);
+                    }
+                    qf[f * WAVE + lane] = r;
+                }
+            };
+            if (wave == 0) {
+                tile_job(false, 1, 0);
+                tile_job(false, 0, 0);
+            } else if (wave == 1) {
+                tile_job(true, 0, 1);
+                tile_job(true, 0, 0);
+            } else if (wave == 2) {
+                tile_job(false, 1, 1);
+                // P[i < 32][j >= 32] = 0
+                bf16x8* pf = reinterpret_cast<bf16x8*>(rec + p.off_p);
+                pf[2 * WAVE + lane] = bf16x8{};
+                pf[3 * WAVE + lane] = bf16x8{};
+                q_frags(0);
+            } else {
+                tile_job(true, 1, 1);
+                q_frags(1);
+            }
+        }
+        __syncthreads();  // #3: A complete, Q consumed (its region becomes T)
+
+        // ---- wave 0: inverses of the four 16 x 16 diagonal blocks; waves 1-3: K~^T fragments ----
+        if (wave == 0) {
+            const int blk = lq, j = l16;  // lane owns column j of block `blk`
+            const float* a = &sA[(16 * blk) * LDA + 16 * blk];
+            float x[16];
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                f32x4 row[4];
+#pragma unroll
+                for (int c4 = 0; c4 < (i + 3) / 4; c4++) row[c4] = *reinterpret_cast<const f32x4*>(&a[i * LDA + 4 * c4]);
+                float part[4] = {(i == j) ? 1.f : 0.f, 0.f, 0.f, 0.f};  // four independent partial sums
+#pragma unroll
+                for (int kk = 0; kk < i; kk++) part[kk % 4] -= row[kk / 4][kk % 4] * x[kk];
+                x[i] = (part[0] + part[1]) + (part[2] + part[3]);
+            }
+#pragma unroll
+            for (int i = 0; i < 16; i++) sT[(16 * blk + i) * LDA + 16 * blk + j] = x[i];
+            // transposes used as B operands below; zero blocks above the diagonal where a product reads them
+            if (blk < 2) {
+#pragma unroll
+                for (int c4 = 0; c4 < 4; c4++)
+                    *reinterpret_cast<f32x4*>(&sTtA[(16 * blk + j) * LDT + 16 * blk + 4 * c4]) =
+                        f32x4{x[4 * c4], x[4 * c4 + 1], x[4 * c4 + 2], x[4 * c4 + 3]};
+                if (blk == 1) {
+#pragma unroll
+                    for (int c4 = 0; c4 < 4; c4++)
+                        *reinterpret_cast<f32x4*>(&sTtA[(16 + j) * LDT + 4 * c4]) = f32x4{0.f, 0.f, 0.f, 0.f};
+                }
+            } else if (blk == 2) {
+#pragma unroll
+                for (int c4 = 0; c4 < 4; c4++)
+                    *reinterpret_cast<f32x4*>(&sTt2[j * LDM + 4 * c4]) = f32x4{x[4 * c4], x[4 * c4 + 1], x[4 * c4 + 2], x[4 * c4 + 3]};
+#pragma unroll
+                for (int i = 0; i < 16; i++) sT[(32 + i) * LDA + 48 + j] = 0.f;  // T block (2, 3)
+            }
+        } else {
+            // K~^T fragments (T_d, token slab): K~[16 s + 4 h + e][d], K~[16 s + 8 + 4 h + e][d]
+            bf16x8* kf = reinterpret_cast<bf16x8*>(rec + p.off_kt);
+            for (int f = wave - 1; f < KD * 4; f += 3) {
+                const int td = f / 4, s = f % 4;
+                const int ja = 16 * s + 4 * lh, jb = ja + 8;
+                const bf16x4 a = lds_read_tr4x16(sK, LDK, ja, 32 * td + 16 * g16, l16);
+                const bf16x4 b = lds_read_tr4x16(sK, LDK, jb, 32 * td + 16 * g16, l16);
+                const f32x4 sa = *reinterpret_cast<const f32x4*>(&s_ks[ja]);
+                const f32x4 sb = *reinterpret_cast<const f32x4*>(&s_ks[jb]);
+                bf16x8 r;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    r[e] = (bf16_t)((float)a[e] * sa[e]);
+                    r[4 + e] = (bf16_t)((float)b[e] * sb[e]);
+                }
+                kf[f * WAVE + lane] = r;
+            }
+        }
+        __syncthreads();  // #4: diagonal blocks of T
+
+        // 16 x 16 x 16 product on one 16x16x32 MFMA pair with hi/lo split operands.
+        // x = rows of X (8 consecutive reduction entries k' = 8 (lq % 2) + e of row l16),
+        // y = rows of Y^T (same entries of column l16 of Y).  Returns X Y.
+        auto mm16 = [&](const float* xrow, const float* ytrow) -> f32x4 {
+            const f32x4 x0 = *reinterpret_cast<const f32x4*>(xrow), x1 = *reinterpret_cast<const f32x4*>(xrow + 4);
+            const f32x4 y0 = *reinterpret_cast<const f32x4*>(ytrow), y1 = *reinterpret_cast<const f32x4*>(ytrow + 4);
+            bf16x8 a1, b1, a2, b2;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                bf16_t xh, xl, yh, yl;
+                split_hi_lo(e < 4 ? x0[e] : x1[e - 4], xh, xl);
+                split_hi_lo(e < 4 ? y0[e] : y1[e - 4], yh, yl);
+                a1[e] = lq < 2 ? xh : xl;  // [X_hi | X_lo]
+                b1[e] = yh;                // [Y_hi ; Y_hi]
+                a2[e] = lq < 2 ? xh : (bf16_t)0.f;  // [X_hi | 0]
+                b2[e] = lq < 2 ? yl : (bf16_t)0.f;  // [Y_lo ; 0]
+            }
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+            acc = mfma_bf16(a1, b1, acc);
+            acc = mfma_bf16(a2, b2, acc);
+            return acc;
+        };
+        // 16 x 16 output tile of a product with 32 reduction entries (k = 8 lq + e), hi/lo split: 3 MFMAs
+        auto mm16x32 = [&](const float* xrow, const float* ytrow) -> f32x4 {
+            const f32x4 x0 = *reinterpret_cast<const f32x4*>(xrow), x1 = *reinterpret_cast<const f32x4*>(xrow + 4);
+            const f32x4 y0 = *reinterpret_cast<const f32x4*>(ytrow), y1 = *reinterpret_cast<const f32x4*>(ytrow + 4);
+            bf16x8 xh, xl, yh, yl;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                bf16_t a, b, c, d;
+                split_hi_lo(e < 4 ? x0[e] : x1[e - 4], a, b);
+                split_hi_lo(e < 4 ? y0[e] : y1[e - 4], c, d);
+                xh[e] = a, xl[e] = b, yh[e] = c, yl[e] = d;
+            }
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+            acc = mfma_bf16(xh, yh, acc);
+            acc = mfma_bf16(xl, yh, acc);
+            acc = mfma_bf16(xh, yl, acc);
+            return acc;
+        };
+
+        // ---- level A: T_10 = -T_11 (A_10 T_00) on wave 0, T_32 = -T_33 (A_32 T_22) on wave 1 ----
+        if (wave < 2) {
+            const int bi = 2 * wave + 1, bj = 2 * wave;
+            const int kk = 8 * (lq % 2);
+            float* const mt = &sMt[wave * 16 * LDM];
+            const float* ttrow = (wave == 0) ? &sTtA[l16 * LDT + kk] : &sTt2[l16 * LDM + kk];  // (T_bj,bj)^T row l16
+            const f32x4 m = mm16(&sA[(16 * bi + l16) * LDA + 16 * bj + kk], ttrow);
+            *reinterpret_cast<f32x4*>(&mt[l16 * LDM + 4 * lq]) = m;  // M^T[n][4 lq + e]
+            const f32x4 t = mm16(&sT[(16 * bi + l16) * LDA + 16 * bi + kk], &mt[l16 * LDM + kk]);
+#pragma unroll
+            for (int e = 0; e < 4; e++) sT[(16 * bi + 4 * lq + e) * LDA + 16 * bj + l16] = -t[e];
+            if (wave == 0) *reinterpret_cast<f32x4*>(&sTtA[l16 * LDT + 16 + 4 * lq]) = -t;  // (T_10)^T
+        }
+        __syncthreads();  // #5
+
+        // ---- level B: T_BA = -T_BB (A_BA T_AA) with 32 x 32 blocks; one 16 x 16 output tile per wave ----
+        {
+            const int ta = wave / 2, tb = wave % 2;
+            const f32x4 m = mm16x32(&sA[(32 + 16 * ta + l16) * LDA + 8 * lq], &sTtA[(16 * tb + l16) * LDT + 8 * lq]);
+            *reinterpret_cast<f32x4*>(&sMtB[(16 * tb + l16) * LDT + 16 * ta + 4 * lq]) = m;
+            __syncthreads();  // #6
+            const f32x4 t = mm16x32(&sT[(32 + 16 * ta + l16) * LDA + 32 + 8 * lq], &sMtB[(16 * tb + l16) * LDT + 8 * lq]);
+#pragma unroll
+            for (int e = 0; e < 4; e++) sT[(32 + 16 * ta + 4 * lq + e) * LDA + 16 * tb + l16] = -t[e];
+        }
+        // A is dead: its region takes the first pass of V, whose registers then go for the next item
+        {
+            const int piece = tid % (VP / 8);
+#pragma unroll
+            for (int it = 0; it < C * (VP / 8) / PREP_THREADS; it++) {
+                const int row = tid / (VP / 8) + it * (PREP_THREADS / (VP / 8));
+                *reinterpret_cast<bf16x8*>(&sV[row * LDV + piece * 8]) = vx[it];
+            }
+            if (has_next) prefetch_v();
+        }
+        __syncthreads();  // #7: T and V complete
+
+        // T fragment for 32-row tile tt and 16-wide slab s (natural order j = 16 s + 8 h + e), columns scaled
+        auto t_frag = [&](int tt, int s, const float* colscale) -> bf16x8 {
+            const int i = 32 * tt + l32;
+            const int j0 = 16 * s + 8 * lh;
+            const f32x4 t0 = *reinterpret_cast<const f32x4*>(&sT[i * LDA + j0]);
+            const f32x4 t1 = *reinterpret_cast<const f32x4*>(&sT[i * LDA + j0 + 4]);
+            const f32x4 c0 = *reinterpret_cast<const f32x4*>(&colscale[j0]);
+            const f32x4 c1 = *reinterpret_cast<const f32x4*>(&colscale[j0 + 4]);
+            bf16x8 r;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int ja = j0 + e, jb = j0 + 4 + e;
+                r[e] = (bf16_t)(ja < i ? t0[e] * c0[e] : (ja == i ? c0[e] : 0.f));
+                r[4 + e] = (bf16_t)(jb < i ? t1[e] * c1[e] : (jb == i ? c1[e] : 0.f));
+            }
+            return r;
+        };
+        // transposed operand: 8 consecutive tokens j = 16 s + 8 h + e of column 32 tile + l32 of a row-major matrix
+        auto tr_frag = [&](const bf16_t* m, int ld, int s, int tile) -> bf16x8 {
+            const bf16x4 a = lds_read_tr4x16(m, ld, 16 * s + 8 * lh, 32 * tile + 16 * g16, l16);
+            const bf16x4 b = lds_read_tr4x16(m, ld, 16 * s + 8 * lh + 4, 32 * tile + 16 * g16, l16);
+            bf16x8 r;
+#pragma unroll
+            for (int e = 0; e < 4; e++) r[e] = a[e], r[4 + e] = b[e];
+            return r;
+        };
+
+        // ---- W^T = K^T (T diag(cw))^T, tile (T_d, T_tok): D[d][tok]; emitted negated ----
+        if (wave < KD) {
+            const int td = wave;
+            f32x16 acc[2];
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[0][r] = 0.f, acc[1][r] = 0.f;
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+                const bf16x8 kt = tr_frag(sK, LDK, s, td);
+                if (s < 2) acc[0] = mfma32_bf16(kt, t_frag(0, s, s_cw), acc[0]);  // tokens < 32 only see j < 32
+                acc[1] = mfma32_bf16(kt, t_frag(1, s, s_cw), acc[1]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            bf16x8* wf = reinterpret_cast<bf16x8*>(rec);
+#pragma unroll
+            for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+                for (int s = 0; s < 2; s++) wf[(tt * KS16 + 2 * td + s) * WAVE + lane] = pack8_16(acc[tt], s, -1.f);
+        }
+
+        // ---- U = (T diag(beta)) V, tile (T_tok, T_n): D[tok][n]; emitted in accumulator layout ----
+        {
+            bf16x8 ta0[2], ta1[4];
+#pragma unroll
+            for (int s = 0; s < 2; s++) ta0[s] = t_frag(0, s, s_beta);
+#pragma unroll
+            for (int s = 0; s < 4; s++) ta1[s] = t_frag(1, s, s_beta);
+            for (int v0 = 0; v0 < p.V; v0 += VP) {
+                const int vcols = min(VP, p.V - v0);
+                if (v0 > 0) {  // later passes of a wide V are staged here, without prefetch
+                    __syncthreads();
+                    const bf16_t* vg = p.v + cc.b * p.v_stride_b + cc.t0 * p.v_stride_t + (int64_t)h * p.v_stride_h;
+                    const int cpr = vcols / 8;
+                    for (int idx = tid; idx < C * cpr; idx += PREP_THREADS) {
+                        const int row = idx / cpr, piece = idx % cpr;
+                        bf16x8 x = {};
+                        if (row < len) x = *reinterpret_cast<const bf16x8*>(vg + row * p.v_stride_t + v0 + piece * 8);
+                        *reinterpret_cast<bf16x8*>(&sV[row * LDV + piece * 8]) = x;
+                    }
+                    __syncthreads();
+                }
+                for (int tl = wave; tl < vcols / 32; tl += 4) {
+                    f32x16 acc[2];
+#pragma unroll
+                    for (int r = 0; r < 16; r++) acc[0][r] = 0.f, acc[1][r] = 0.f;
+#pragma unroll
+                    for (int s = 0; s < 4; s++) {
+                        const bf16x8 vb = tr_frag(sV, LDV, s, tl);
+                        if (s < 2) acc[0] = mfma32_bf16(ta0[s], vb, acc[0]);
+                        acc[1] = mfma32_bf16(ta1[s], vb, acc[1]);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                    const int tn = v0 / 32 + tl;
+                    bf16x8* uf = reinterpret_cast<bf16x8*>(rec + p.off_u) + ((int64_t)tn * WAVE + lane) * 4;
+                    uf[0] = pack8_16(acc[0], 0, 1.f);
+                    uf[1] = pack8_16(acc[0], 1, 1.f);
+                    uf[2] = pack8_16(acc[1], 0, 1.f);
+                    uf[3] = pack8_16(acc[1], 1, 1.f);
+                }
+            }
+        }
+        __syncthreads();  // #8: LDS is reused by the next item
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// scan
+// ------------------------------------------------------------------------------------------
+template <int K>
+__global__ __launch_bounds__(WAVE) void chunk_scan32_kernel(const ChunkParams p) {
+    constexpr int KD = K / 32;    // 32-row tiles of the state
+    constexpr int KS16 = K / 16;  // 16-wide slabs over the key dim
+    constexpr int NW_ = 2 * KS16, NQ_ = 2 * KS16, NK_ = KD * 4, NP_ = 8;  // fragments per record
+
+    const int lane = threadIdx.x;
+    const int l32 = lane % 32, lh = lane / 32;
+
+    // workgroup (= one wave) -> (sequence-head chain, 32-column slice); the slices of a chain stay on
+    // one XCD (id % 8) so that its records are fetched into a single L2
+    const int id = blockIdx.x;
+    const int xcd = id % 8, rest = id / 8;
+    const int tn = rest % p.scan_groups;
+    const int chain = (rest / p.scan_groups) * 8 + xcd;
+    if (chain >= p.N * p.H) return;
+    const int n = chain / p.H, h = chain % p.H;
+
+    int slot_begin, slot_end;
+    int64_t b, seq_t0, seq_len;
+    if (p.cu_seqlens == nullptr) {
+        slot_begin = n * p.NT, slot_end = slot_begin + p.NT;
+        b = n, seq_t0 = 0, seq_len = p.T;
+    } else {
+        slot_begin = p.chunk_off[n], slot_end = p.chunk_off[n + 1];
+        b = 0, seq_t0 = p.cu_seqlens[n], seq_len = p.cu_seqlens[n + 1] - seq_t0;
+    }
+    const int nchunks = slot_end - slot_begin;
+
+    // state tile td, register r: row 32 td + 8 (r/4) + 4 h + r%4, column 32 tn + l32
+    f32x16 S[KD];
+    const int64_t st_off = ((int64_t)n * p.H + h) * K * p.V + (int64_t)(4 * lh) * p.V + 32 * tn + l32;
+#pragma unroll
+    for (int td = 0; td < KD; td++)
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+            S[td][r] = (p.h0 != nullptr) ? p.h0[st_off + (int64_t)(32 * td + 8 * (r / 4) + r % 4) * p.V] : 0.f;
+
+    // O^T tile tt, register r: token 32 tt + l32, column 32 tn + 8 (r/4) + 4 h + r%4
+    bf16_t* const og = p.o + b * p.o_stride_b + (seq_t0 + l32) * p.o_stride_t + (int64_t)h * p.o_stride_h + 32 * tn + 4 * lh;
+    const uint8_t* rec = p.rec + ((int64_t)h * p.TC + slot_begin) * p.rec_bytes;
+
+    bf16x8 wr[NW_], qr[NQ_], kr[NK_], pr[NP_], ur[4];
+    float egc = 0.f;
+    auto frag_ptr = [&](const uint8_t* r, uint32_t off, int f) {
+        return reinterpret_cast<const bf16x8*>(r + off) + f * WAVE + lane;
+    };
+    if (nchunks > 0) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) ur[i] = *(reinterpret_cast<const bf16x8*>(rec + p.off_u) + ((int64_t)tn * WAVE + lane) * 4 + i);
+        egc = *reinterpret_cast<const float*>(rec + p.off_eg);
+#pragma unroll
+        for (int i = 0; i < NW_; i++) wr[i] = *frag_ptr(rec, 0, i);
+#pragma unroll
+        for (int i = 0; i < NQ_; i++) qr[i] = *frag_ptr(rec, p.off_qs, i);
+#pragma unroll
+        for (int i = 0; i < NK_; i++) kr[i] = *frag_ptr(rec, p.off_kt, i);
+#pragma unroll
+        for (int i = 0; i < NP_; i++) pr[i] = *frag_ptr(rec, p.off_p, i);
+    }
+
+    auto iteration = [&](int c, auto more_tag) {
+        constexpr bool more = decltype(more_tag)::value;
+        const uint8_t* nxt = rec + p.rec_bytes;  // only dereferenced when `more`
+
+        // state as bf16 operand, one fragment per 16-row slab
+        bf16x8 sb[KS16];
+#pragma unroll
+        for (int s = 0; s < KS16; s++) sb[s] = pack8_16(S[s / 2], s % 2, 1.f);
+        f32x16 accv[2], acco[2];
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                accv[tt][r] = (float)ur[2 * tt + r / 8][r % 8];
+                acco[tt][r] = 0.f;
+            }
+        const float eg_cur = egc;
+        if constexpr (more) {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                ur[i] = *(reinterpret_cast<const bf16x8*>(nxt + p.off_u) + ((int64_t)tn * WAVE + lane) * 4 + i);
+            egc = *reinterpret_cast<const float*>(nxt + p.off_eg);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+
+        // V~ = U - W S0: accv[tt] += W~(tt, s) sb[s]; each fragment register is refilled from the next
+        // record right behind the MFMA that consumed it
+#pragma unroll
+        for (int s = 0; s < KS16; s++)
+#pragma unroll
+            for (int tt = 0; tt < 2; tt++) {
+                const int f = tt * KS16 + s;
+                accv[tt] = mfma32_bf16(wr[f], sb[s], accv[tt]);
+                if constexpr (more) wr[f] = *frag_ptr(nxt, 0, f);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        // O^T = S0^T Q~^T
+#pragma unroll
+        for (int s = 0; s < KS16; s++)
+#pragma unroll
+            for (int tt = 0; tt < 2; tt++) {
+                const int f = tt * KS16 + s;
+                acco[tt] = mfma32_bf16(sb[s], qr[f], acco[tt]);
+                if constexpr (more) qr[f] = *frag_ptr(nxt, p.off_qs, f);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+
+        // V~ as operand, one fragment per 16-token slab; decay of the state
+        bf16x8 vb[4];
+#pragma unroll
+        for (int s = 0; s < 4; s++) vb[s] = pack8_16(accv[s / 2], s % 2, 1.f);
+#pragma unroll
+        for (int td = 0; td < KD; td++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) S[td][r] *= eg_cur;
+        __builtin_amdgcn_sched_barrier(0);
+
+        // S = e^{gamma_C} S + K~^T V~
+#pragma unroll
+        for (int s = 0; s < 4; s++)
+#pragma unroll
+            for (int td = 0; td < KD; td++) {
+                const int f = td * 4 + s;
+                S[td] = mfma32_bf16(kr[f], vb[s], S[td]);
+                if constexpr (more) kr[f] = *frag_ptr(nxt, p.off_kt, f);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        // O^T += V~^T P^T (P[i < 32][j >= 32] = 0: those two products are skipped)
+#pragma unroll
+        for (int s = 0; s < 4; s++)
+#pragma unroll
+            for (int tt = 0; tt < 2; tt++) {
+                const int f = tt * 4 + s;
+                if (tt == 1 || s < 2) acco[tt] = mfma32_bf16(vb[s], pr[f], acco[tt]);
+                if constexpr (more) {
+                    if (tt == 1 || s < 2) pr[f] = *frag_ptr(nxt, p.off_p, f);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+
+        const int64_t tok0 = (int64_t)c * C;
+        const int valid = (int)min((int64_t)C, seq_len - tok0);
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++)
+            if (32 * tt + l32 < valid) {
+#pragma unroll
+                for (int q4 = 0; q4 < 4; q4++) {
+                    bf16x4 r;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) r[e] = (bf16_t)acco[tt][4 * q4 + e];
+                    *reinterpret_cast<bf16x4*>(og + (tok0 + 32 * tt) * p.o_stride_t + 8 * q4) = r;
+                }
+            }
+        rec += p.rec_bytes;
+    };
+    for (int c = 0; c + 1 < nchunks; c++) iteration(c, std::true_type{});
+    if (nchunks > 0) iteration(nchunks - 1, std::false_type{});
+
+    if (p.ht != nullptr) {
+#pragma unroll
+        for (int td = 0; td < KD; td++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) p.ht[st_off + (int64_t)(32 * td + 8 * (r / 4) + r % 4) * p.V] = S[td][r];
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// launch
+// ------------------------------------------------------------------------------------------
+template <int K>
+static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int num_cus) {
+    const int64_t items = (int64_t)p.TC * p.H;
+    const int grid_prep = (int)(items < 2 * (int64_t)num_cus ? items : 2 * (int64_t)num_cus);  // two workgroups per CU
+    hipLaunchKernelGGL((chunk_prepare32_kernel<K>), dim3(grid_prep), dim3(PREP_THREADS), 0, stream, p);
+    if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
+    if (events != nullptr) (void)hipEventRecord(events[2], stream);
+
+    const int64_t chains = (int64_t)p.N * p.H;
+    p.scan_groups = p.V / 32;
+    const int64_t chains8 = (chains + 7) / 8 * 8;
+    hipLaunchKernelGGL((chunk_scan32_kernel<K>), dim3((unsigned)(chains8 * p.scan_groups)), dim3(WAVE), 0, stream, p);
+    return (int)hipGetLastError();
+}
+
+int launch_chunk32(ChunkParams& p, int K, hipStream_t stream, hipEvent_t* events, int num_cus) {
+    if (K == 64) return launch32<64>(p, stream, events, num_cus);
+    if (K == 128) return launch32<128>(p, stream, events, num_cus);
+    return GDN_ERR_UNSUPPORTED;
+}
+
+}  // namespace gdn

@@ -1,0 +1,115 @@
+// Types and device helpers shared by the chunked-forward kernels of the gated delta rule.
+#pragma once
+
+#include "gdn_common.h"
+
+namespace gdn {
+
+constexpr int C = 64;  // chunk length
+constexpr int PREP_THREADS = 256;
+constexpr int FRAG_BYTES = WAVE * 16;  // one MFMA operand fragment: 8 bf16 per lane
+
+struct ChunkParams {
+    const bf16_t* q;
+    const bf16_t* k;
+    const bf16_t* v;
+    const void* beta;
+    const float* g;
+    const float* h0;
+    float* ht;
+    bf16_t* o;
+    const int32_t* cu_seqlens;
+    int32_t* chunk_off;  // [N + 1] prefix of chunks per sequence (packed input only)
+    uint8_t* rec;        // workspace records, [H][TC]
+    int64_t q_stride_b, q_stride_t, q_stride_h;
+    int64_t k_stride_b, k_stride_t, k_stride_h;
+    int64_t v_stride_b, v_stride_t, v_stride_h;
+    int64_t o_stride_b, o_stride_t, o_stride_h;
+    int B, T, H, V, N;
+    int NT;  // chunks per sequence (fixed-length input)
+    int TC;  // chunk slots per head
+    int beta_dtype;
+    int l2norm;
+    float scale;
+    uint32_t rec_bytes, off_qs, off_kt, off_p, off_u, off_eg;
+    int scan_groups;  // workgroups per (sequence, head) in the scan kernel
+};
+
+struct RecordLayout {
+    uint32_t off_wn, off_qs, off_kt, off_p, off_u, off_eg, bytes;
+};
+
+// Record of one (head, chunk): Wn (-W), Qs, Kt, P as A-operand fragments, U as accumulator
+// fragments, e^{gamma_C}.
+inline RecordLayout record_layout(int K, int V) {
+    RecordLayout r;
+    const uint32_t kfrag = (uint32_t)(C / 16) * (K / 32) * FRAG_BYTES;  // [C x K] or [K x C] bf16
+    r.off_wn = 0;
+    r.off_qs = kfrag;
+    r.off_kt = 2 * kfrag;
+    r.off_p = 3 * kfrag;
+    r.off_u = r.off_p + (C / 16) * (C / 32) * FRAG_BYTES;
+    r.off_eg = r.off_u + (uint32_t)C * V * 2;
+    r.bytes = (r.off_eg + 4 + 255u) & ~255u;
+    return r;
+}
+
+// Where chunk slot `slot` of the grid lives: sequence, first token, valid length (0 = unused slot).
+struct ChunkCoord {
+    int n;
+    int64_t b, t0;
+    int len;
+};
+
+__device__ __forceinline__ ChunkCoord locate_chunk(const ChunkParams& p, int slot) {
+    ChunkCoord cc;
+    if (p.cu_seqlens == nullptr) {
+        cc.n = slot / p.NT;
+        const int c = slot - cc.n * p.NT;
+        cc.b = cc.n;
+        cc.t0 = (int64_t)c * C;
+        cc.len = min(C, p.T - c * C);
+        return cc;
+    }
+    cc.b = 0;
+    if (slot >= p.chunk_off[p.N]) {
+        cc.n = 0, cc.t0 = 0, cc.len = 0;
+        return cc;
+    }
+    int lo = 0, hi = p.N;  // largest n with chunk_off[n] <= slot
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (p.chunk_off[mid] <= slot) lo = mid;
+        else hi = mid;
+    }
+    cc.n = lo;
+    const int c = slot - p.chunk_off[lo];
+    cc.t0 = (int64_t)p.cu_seqlens[lo] + (int64_t)c * C;
+    cc.len = min(C, p.cu_seqlens[lo + 1] - (int)cc.t0);
+    return cc;
+}
+
+__device__ __forceinline__ f32x4 mfma_bf16(bf16x8 a, bf16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ f32x4 mfma_f32(float a, float b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ bf16x8 pack8(f32x4 lo, f32x4 hi) {
+    bf16x8 r;
+    r[0] = (bf16_t)lo[0], r[1] = (bf16_t)lo[1], r[2] = (bf16_t)lo[2], r[3] = (bf16_t)lo[3];
+    r[4] = (bf16_t)hi[0], r[5] = (bf16_t)hi[1], r[6] = (bf16_t)hi[2], r[7] = (bf16_t)hi[3];
+    return r;
+}
+
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+// v_mfma_f32_32x32x16_bf16:  A[i = l%32][k = 8 (l/32) + 0..7]   B[k = 8 (l/32) + 0..7][j = l%32]
+//                            D[i = 8 (r/4) + 4 (l/32) + r%4][j = l%32],  r = 0..15 the register index
+__device__ __forceinline__ f32x16 mfma32_bf16(bf16x8 a, bf16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+}  // namespace gdn
