@@ -43,6 +43,8 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target duration of the CPU baseline sample")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy, the known-size kernel the HBM counters are scaled by")
     return ap.parse_args()
 
 
@@ -157,35 +159,57 @@ def bench_decode(steps, warmup):
 
 
 def cpu_baseline(w, inp_gpu, target_seconds):
-    """Naive recurrent torch restatement on this host's cores, on a bounded prefix of the workload:
-    the first sequence, all heads, as many tokens as fit the time budget (the cost is exactly
-    linear in the token count)."""
+    """Naive recurrent torch restatement on this host's cores, on a bounded sample of the workload:
+    whole sequences in order (all heads) until the time budget is used, or a prefix of the first
+    sequence if even that does not fit (the cost is exactly linear in the token count)."""
     import torch
 
     from oracle import recurrent_gated_delta_rule_ref
     from oracle.c_oracle import recurrent_gated_delta_rule_c
 
     cores = torch.get_num_threads()
-    first = 0 if inp_gpu["cu_seqlens"] is None else None
     cpu = {n: (x.cpu() if isinstance(x, torch.Tensor) else x) for n, x in inp_gpu.items()}
-    seq_len = w.T if first is not None else int(cpu["cu_seqlens"][1])
+    packed = cpu["cu_seqlens"] is not None
+    bounds = [int(x) for x in cpu["cu_seqlens"]] if packed else None
+    n_seq = len(bounds) - 1 if packed else w.B
 
-    def prefix(tokens):
-        sub = {n: cpu[n][:1, :tokens] for n in ("q", "k", "v", "g", "beta") if cpu[n] is not None}
+    def sequence(i, tokens=None):
+        if packed:
+            t0, t1 = bounds[i], bounds[i + 1] if tokens is None else bounds[i] + tokens
+            sub = {n: cpu[n][:, t0:t1] for n in ("q", "k", "v", "g", "beta") if cpu[n] is not None}
+        else:
+            t1 = w.T if tokens is None else tokens
+            sub = {n: cpu[n][i : i + 1, :t1] for n in ("q", "k", "v", "g", "beta") if cpu[n] is not None}
         h0 = cpu["initial_state"]
-        return dict(sub, initial_state=None if h0 is None else h0[:1], scale=cpu["scale"])
+        return dict(sub, initial_state=None if h0 is None else h0[i : i + 1], scale=cpu["scale"])
 
-    probe = min(64, seq_len)
+    first_len = (bounds[1] - bounds[0]) if packed else w.T
+    probe = min(64, first_len)
     t0 = time.perf_counter()
-    recurrent_gated_delta_rule_ref(**prefix(probe), output_final_state=True)
+    recurrent_gated_delta_rule_ref(**sequence(0, probe), output_final_state=True)
     per_token = (time.perf_counter() - t0) / probe
-    tokens = max(probe, min(seq_len, int(target_seconds / per_token)))
-    t0 = time.perf_counter()
-    recurrent_gated_delta_rule_ref(**prefix(tokens), output_final_state=True)
-    seconds = time.perf_counter() - t0
 
+    tokens, seconds, what = 0, 0.0, ""
+    if per_token * first_len > target_seconds:
+        tokens = max(probe, int(target_seconds / per_token))
+        t0 = time.perf_counter()
+        recurrent_gated_delta_rule_ref(**sequence(0, tokens), output_final_state=True)
+        seconds = time.perf_counter() - t0
+        what = f"first {tokens} of {first_len} tokens of the first sequence"
+    else:
+        done = 0
+        while done < n_seq and seconds < target_seconds:
+            inp = sequence(done)
+            t0 = time.perf_counter()
+            recurrent_gated_delta_rule_ref(**inp, output_final_state=True)
+            seconds += time.perf_counter() - t0
+            tokens += inp["q"].size(1)
+            done += 1
+        what = f"{done} of {n_seq} whole sequences ({tokens} tokens)"
+
+    full = sequence(0)
     t0 = time.perf_counter()
-    recurrent_gated_delta_rule_c(**prefix(seq_len), output_final_state=True, f64_state=False)
+    recurrent_gated_delta_rule_c(**full, output_final_state=True, f64_state=False)
     c_seconds = time.perf_counter() - t0
 
     return {
@@ -193,11 +217,22 @@ def cpu_baseline(w, inp_gpu, target_seconds):
         "unit": "tokens/s",
         "cores": cores,
         "kind": "port",
-        "sample": f"first sequence of {w.name}, first {tokens} of {seq_len} tokens, all {w.H} heads, fp32, "
-                  f"torch token loop ({seconds:.1f} s)",
-        "c_port_tokens_per_s": round(seq_len / c_seconds, 1),
-        "c_port_sample": f"same sequence, all {seq_len} tokens, C restatement with OpenMP over heads ({c_seconds:.2f} s)",
-    }  # fmt: skip
+        "sample": f"{w.name}: {what}, all {w.H} heads, fp32 torch token loop, {seconds:.1f} s",
+        "c_port_tokens_per_s": round(first_len / c_seconds, 1),
+        "c_port_sample": f"first sequence ({first_len} tokens), C restatement with OpenMP over heads, {c_seconds:.2f} s",
+    }
+
+
+def calibrate_copy():
+    """A plain device-to-device copy of 1 GiB: the kernel of known traffic (1 GiB read, 1 GiB written)
+    against which FETCH_SIZE / WRITE_SIZE readings of the other kernels are scaled."""
+    import torch
+
+    src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").fill_(1)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
 
 
 def main():
@@ -221,6 +256,8 @@ def main():
     result, inp = bench_chunk(w, args.steps, args.warmup)
     decode = None if args.no_decode else bench_decode(args.steps, args.warmup)
     baseline = None if args.no_cpu_baseline else cpu_baseline(w, inp, args.cpu_seconds)
+    if args.calibrate_copy:
+        calibrate_copy()
 
     line = {
         "metric": result["metric"],

@@ -104,7 +104,7 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
     // ---- register prefetch of one item's inputs ----
     bf16x8 kx[NPASS], qx[NPASS], vx[C * (VP / 8) / PREP_THREADS];
     float gx = 0.f;
-    uint32_t bx_raw = 0;  // beta of the prefetched item, converted where it is used (a conversion here would wait for every load)
+    uint32_t bx_raw = 0;  // beta of the prefetched item, raw bits: any arithmetic on it here would wait for every load in flight
     ChunkCoord ncc;  // coordinates of the prefetched item
     int nh = 0;
     auto locate = [&](int64_t w) {
@@ -139,7 +139,7 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
                 const uint32_t soff = (uint32_t)lane0 * (uint32_t)p.H;
                 if (p.g != nullptr) gx = (p.g + sbase)[soff];
                 if (p.beta == nullptr) bx_raw = 0x3f800000u;  // 1.0f
-                else if (p.beta_dtype == GDN_BF16) bx_raw = (uint32_t)(reinterpret_cast<const uint16_t*>(p.beta) + sbase)[soff] << 16;
+                else if (p.beta_dtype == GDN_BF16) bx_raw = (reinterpret_cast<const uint16_t*>(p.beta) + sbase)[soff];  // shifted at use
                 else bx_raw = (reinterpret_cast<const uint32_t*>(p.beta) + sbase)[soff];
             }
         }
@@ -205,7 +205,7 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
                     if (lane >= off) gv += up;
                 }
                 s_gam[lane] = gv;
-                s_beta[lane] = __builtin_bit_cast(float, bx_raw);
+                s_beta[lane] = __builtin_bit_cast(float, (p.beta != nullptr && p.beta_dtype == GDN_BF16) ? bx_raw << 16 : bx_raw);
             }
         }
         // the q, k registers are free: start on the next item
