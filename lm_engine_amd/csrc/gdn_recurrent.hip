@@ -7,7 +7,8 @@
 //
 //     r  = beta (v - e^g S^T k)        S' = e^g S + k r^T        o = e^g S^T q + (k . q) r
 //
-// i.e. one read and one write of the state for T == 1 (the decode step).  The two
+// i.e. one read and one write of the state for T == 1 (the decode step); both are streaming
+// (non-temporal) accesses, since a state far larger than the caches is touched exactly once per step.  The two
 // K-reductions (S^T k, S^T q) are done in registers, then across the row groups of a wave
 // with shuffles and across the four waves through LDS.
 //
@@ -77,7 +78,7 @@ __global__ __launch_bounds__(REC_THREADS) void recurrent_kernel(const RecurrentP
     f32x4 S[RPT];
     if (p.h0 != nullptr) {
 #pragma unroll
-        for (int i = 0; i < RPT; i++) S[i] = *reinterpret_cast<const f32x4*>(p.h0 + state_off + (int64_t)i * p.V);
+        for (int i = 0; i < RPT; i++) S[i] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p.h0 + state_off + (int64_t)i * p.V));
     } else {
 #pragma unroll
         for (int i = 0; i < RPT; i++) S[i] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -125,12 +126,11 @@ __global__ __launch_bounds__(REC_THREADS) void recurrent_kernel(const RecurrentP
 
         // ---- partial S^T k and S^T q over this thread's rows ----
         f32x4 pk = {0.f, 0.f, 0.f, 0.f}, pq = {0.f, 0.f, 0.f, 0.f};
-        float kr[RPT];
 #pragma unroll
         for (int i = 0; i < RPT; i++) {
-            kr[i] = s_k[rg * RPT + i];
+            const float kr = s_k[rg * RPT + i];
             const float qr = s_q[rg * RPT + i];
-            pk += S[i] * kr[i];
+            pk += S[i] * kr;
             pq += S[i] * qr;
         }
         const float kq = s_kq[0];
@@ -158,13 +158,13 @@ __global__ __launch_bounds__(REC_THREADS) void recurrent_kernel(const RecurrentP
         // ---- rank-1 update and output ----
         const f32x4 r = (vt - sk * eg) * beta;
 #pragma unroll
-        for (int i = 0; i < RPT; i++) S[i] = S[i] * eg + r * kr[i];
+        for (int i = 0; i < RPT; i++) S[i] = S[i] * eg + r * s_k[rg * RPT + i];  // k^ re-read: keeps 16 registers free
         if (rg == 0) store4<T>(op + t * p.o_stride_t, sq * eg + r * kq);
     }
 
     if (p.ht != nullptr) {
 #pragma unroll
-        for (int i = 0; i < RPT; i++) *reinterpret_cast<f32x4*>(p.ht + state_off + (int64_t)i * p.V) = S[i];
+        for (int i = 0; i < RPT; i++) __builtin_nontemporal_store(S[i], reinterpret_cast<f32x4*>(p.ht + state_off + (int64_t)i * p.V));
     }
 }
 
