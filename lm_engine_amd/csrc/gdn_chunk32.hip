@@ -9,9 +9,8 @@
 //
 //   * a wave of the scan owns a K x 32 slice of the state; operand fragments are laid out for
 //     the 32x32x16 shape;
-//   * the scan has no LDS and no barrier: every wave streams its fragments global -> registers
-//     with a rolling prefetch (the registers of fragment i are reloaded from the next record
-//     right after the MFMA that consumed them), one vector load between two MFMAs;
+//   * the scan shares each record between the compute waves of a workgroup through a double buffer
+//     in LDS filled by dedicated loader waves;
 //   * prepare is persistent: a workgroup walks over (chunk, head) items and loads q, k, v of
 //     the next item into registers while it computes the current one;
 //   * the triangular inverse runs its block products on bf16 MFMA with operands split into
@@ -538,9 +537,251 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
 
 // ------------------------------------------------------------------------------------------
 // scan
+//
+// A workgroup works on one (sequence, head): NW compute waves, each owning a K x 32 slice of the
+// fp32 state as MFMA accumulators, and NL = 4 loader waves.  Everything a chunk needs from its
+// record (the operand fragments W~, Q~, K~^T, P, the U tiles of this workgroup's columns and
+// e^{gamma_C}) goes through a double buffer in LDS: during chunk c the loaders move record c + 1
+// global -> registers -> LDS and already have record c + 2 (and c + 3) in flight in a second
+// register buffer, while the compute waves run the 54 MFMAs of chunk c out of the other half,
+// reading each fragment from LDS a few MFMAs before it is used.  One workgroup barrier per chunk
+// hands the halves over.  Sharing the record between the compute waves is what makes the scan
+// cheap per column: a wave that streams its own copy of the record spends its time issuing loads
+// (measured: one wave per CU loading 58 KB per chunk directly needs ~4600 cycles per chunk).
+// O is accumulated transposed (operands swapped) so that a lane ends up with 4 consecutive
+// columns of one token (8-byte stores).
 // ------------------------------------------------------------------------------------------
+constexpr int SCAN_LOADERS = 4;
+
+template <int K, int NW>
+__global__ __launch_bounds__((NW + SCAN_LOADERS) * WAVE) void chunk_scan32_kernel(const ChunkParams p) {
+    constexpr int NL = SCAN_LOADERS;
+    constexpr int KD = K / 32;    // 32-row tiles of the state
+    constexpr int KS16 = K / 16;  // 16-wide slabs over the key dim
+    constexpr int NWF = 2 * KS16, NQF = 2 * KS16, NKF = KD * 4, NPF = 8;  // fragments of W~, Q~, K~^T, P
+    constexpr int SHARED_FRAGS = NWF + NQF + NKF + NPF;  // contiguous at the head of the record
+    constexpr int SHARED_BYTES = SHARED_FRAGS * FRAG_BYTES;
+    constexpr int U_FRAGS = 4 * NW;  // U tiles of this workgroup's columns: contiguous in the record
+    constexpr int STAGE_FRAGS = SHARED_FRAGS + U_FRAGS;
+    constexpr int STAGE_BYTES = STAGE_FRAGS * FRAG_BYTES + 16;  // + e^{gamma_C}
+    constexpr int NLOAD = STAGE_FRAGS / NL;                     // fragments moved by each loader wave
+    static_assert(2 * STAGE_BYTES <= 160 * 1024, "double buffer exceeds LDS");
+    static_assert(STAGE_FRAGS % NL == 0, "fragments must divide over the loader waves");
+
+    __shared__ __attribute__((aligned(16))) uint8_t stage[2][STAGE_BYTES];
+
+    const int lane = threadIdx.x % WAVE;
+    const int wave = threadIdx.x / WAVE;
+    const int l32 = lane % 32, lh = lane / 32;
+
+    // workgroup -> (sequence-head chain, column group); the groups of a chain stay on one XCD (id % 8)
+    // so that its records are fetched into a single L2
+    const int id = blockIdx.x;
+    const int xcd = id % 8, rest = id / 8;
+    const int vgroup = rest % p.scan_groups;
+    const int chain = (rest / p.scan_groups) * 8 + xcd;
+    if (chain >= p.N * p.H) return;  // whole workgroup
+    const int n = chain / p.H, h = chain % p.H;
+
+    int slot_begin, slot_end;
+    int64_t b, seq_t0, seq_len;
+    if (p.cu_seqlens == nullptr) {
+        slot_begin = n * p.NT, slot_end = slot_begin + p.NT;
+        b = n, seq_t0 = 0, seq_len = p.T;
+    } else {
+        slot_begin = p.chunk_off[n], slot_end = p.chunk_off[n + 1];
+        b = 0, seq_t0 = p.cu_seqlens[n], seq_len = p.cu_seqlens[n + 1] - seq_t0;
+    }
+    const int nchunks = slot_end - slot_begin;
+    const uint8_t* rec = p.rec + ((int64_t)h * p.TC + slot_begin) * p.rec_bytes;
+
+    if (wave >= NW) {
+        // ------------------------------ loader ------------------------------
+        // fragment f of the stage: f < SHARED_FRAGS comes from the head of the record, the rest from
+        // this workgroup's slice of the U block
+        const int lw = wave - NW;
+        const int64_t u_shift = (int64_t)p.off_u + (int64_t)vgroup * U_FRAGS * FRAG_BYTES - SHARED_BYTES;
+        // two register buffers: while one record is written to LDS, younger ones are in flight
+        bf16x8 buf0[NLOAD], buf1[NLOAD];
+        float eg0 = 0.f, eg1 = 0.f;
+        auto src_of = [&](int c, int i) {
+            const int f = lw * NLOAD + i;
+            return rec + (int64_t)c * p.rec_bytes + (int64_t)f * FRAG_BYTES + (f >= SHARED_FRAGS ? u_shift : 0) + lane * 16;
+        };
+        auto load = [&](bf16x8(&buf)[NLOAD], float& eg, int c) {
+#pragma unroll
+            for (int i = 0; i < NLOAD; i++) buf[i] = *reinterpret_cast<const bf16x8*>(src_of(c, i));
+            if (lw == 0) eg = *reinterpret_cast<const float*>(rec + (int64_t)c * p.rec_bytes + p.off_eg);
+        };
+        // write record c to LDS and refill each register with record c2 right behind its write, so the
+        // LDS-write and the vector-memory queues fill together
+        auto store_and_reload = [&](bf16x8(&buf)[NLOAD], float& eg, int c, int c2, auto reload_tag) {
+            constexpr bool reload = decltype(reload_tag)::value;
+            uint8_t* dst = stage[c & 1];
+            bf16x8* d = reinterpret_cast<bf16x8*>(dst) + (lw * NLOAD) * WAVE + lane;
+            if (lw == 0 && lane == 0) *reinterpret_cast<float*>(dst + STAGE_FRAGS * FRAG_BYTES) = eg;
+#pragma unroll
+            for (int i = 0; i < NLOAD; i++) {
+                d[i * WAVE] = buf[i];
+                if constexpr (reload) buf[i] = *reinterpret_cast<const bf16x8*>(src_of(c2, i));
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if constexpr (reload) {
+                if (lw == 0) eg = *reinterpret_cast<const float*>(rec + (int64_t)c2 * p.rec_bytes + p.off_eg);
+            }
+        };
+        constexpr std::true_type yes{};
+        constexpr std::false_type no{};
+        // records 0 (-> LDS now), 1 and 2 (in flight); even records use buf0, odd ones buf1
+        if (nchunks > 0) {
+            load(buf0, eg0, 0);
+            if (nchunks > 1) load(buf1, eg1, 1);
+            if (nchunks > 2) store_and_reload(buf0, eg0, 0, 2, yes);
+            else store_and_reload(buf0, eg0, 0, 0, no);
+        }
+        __syncthreads();  // stage[0] holds record 0
+        // Barrier of iteration c: the compute waves are done with stage[c & 1] and record c + 1 is in the
+        // other half.  Before it: write record c + 1 (its half was released by the barrier of iteration
+        // c - 1) and refill the freed registers with record c + 3.
+        int c = 0;
+        for (; c + 4 < nchunks; c += 2) {  // steady state: straight-line code, both reloads exist
+            store_and_reload(buf1, eg1, c + 1, c + 3, yes);
+            __syncthreads();
+            store_and_reload(buf0, eg0, c + 2, c + 4, yes);
+            __syncthreads();
+        }
+        for (; c < nchunks; c += 2) {  // the last (at most four) chunks
+            if (c + 1 < nchunks) {
+                if (c + 3 < nchunks) store_and_reload(buf1, eg1, c + 1, c + 3, yes);
+                else store_and_reload(buf1, eg1, c + 1, 0, no);
+            }
+            __syncthreads();
+            if (c + 1 < nchunks) {
+                if (c + 2 < nchunks) store_and_reload(buf0, eg0, c + 2, 0, no);
+                __syncthreads();
+            }
+        }
+        return;
+    }
+
+    // ------------------------------ compute ------------------------------
+    const int tn = vgroup * NW + wave;  // 32-column tile of V owned by this wave
+    const bool active = 32 * tn < p.V;  // a last, partial column group has idle waves (they only keep the barriers)
+    // state tile td, register r: row 32 td + 8 (r/4) + 4 h + r%4, column 32 tn + l32
+    f32x16 S[KD];
+    const int64_t st_off = ((int64_t)n * p.H + h) * K * p.V + (int64_t)(4 * lh) * p.V + 32 * tn + l32;
+#pragma unroll
+    for (int td = 0; td < KD; td++)
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+            S[td][r] = (active && p.h0 != nullptr) ? p.h0[st_off + (int64_t)(32 * td + 8 * (r / 4) + r % 4) * p.V] : 0.f;
+    // O^T tile tt, register r: token 32 tt + l32, column 32 tn + 8 (r/4) + 4 h + r%4
+    bf16_t* const og = p.o + b * p.o_stride_b + (seq_t0 + l32) * p.o_stride_t + (int64_t)h * p.o_stride_h + 32 * tn + 4 * lh;
+
+    // MFMA schedule of one chunk: W~ (NWF) | Q~ (NQF) | K~^T (NKF) | P (6: the two zero fragments are skipped)
+    constexpr int NOPS = NWF + NQF + NKF + 6;
+    constexpr int LOOKAHEAD = 6;  // LDS reads are issued this many MFMAs ahead of their use
+    auto lds_frag = [&](const uint8_t* st, int op) -> bf16x8 {
+        int f = op;
+        if (op >= NWF + NQF + NKF) {  // P fragments (tt, s) with tt == 1 or s < 2: indices 0, 1, 4, 5, 6, 7
+            const int j = op - (NWF + NQF + NKF);
+            f = NWF + NQF + NKF + (j < 2 ? j : j + 2);
+        }
+        return reinterpret_cast<const bf16x8*>(st)[f * WAVE + lane];
+    };
+
+    __syncthreads();  // stage[0] holds record 0
+
+    for (int c = 0; c < nchunks; c++) {
+        const uint8_t* st = stage[c & 1];
+        if (active) {
+            const bf16x8* uf = reinterpret_cast<const bf16x8*>(st + SHARED_BYTES) + (wave * WAVE + lane) * 4;
+            bf16x8 ur[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) ur[i] = uf[i];
+            const float egc = *reinterpret_cast<const float*>(st + STAGE_FRAGS * FRAG_BYTES);
+            bf16x8 fr[NOPS];
+#pragma unroll
+            for (int op = 0; op < LOOKAHEAD; op++) fr[op] = lds_frag(st, op);
+
+            // state as bf16 operand, one fragment per 16-row slab
+            bf16x8 sb[KS16];
+#pragma unroll
+            for (int s = 0; s < KS16; s++) sb[s] = pack8_16(S[s / 2], s % 2, 1.f);
+            f32x16 accv[2], acco[2];
+#pragma unroll
+            for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    accv[tt][r] = (float)ur[2 * tt + r / 8][r % 8];
+                    acco[tt][r] = 0.f;
+                }
+            bf16x8 vb[4];
+            __builtin_amdgcn_sched_barrier(0);
+
+#pragma unroll
+            for (int op = 0; op < NOPS; op++) {
+                if (op + LOOKAHEAD < NOPS) fr[op + LOOKAHEAD] = lds_frag(st, op + LOOKAHEAD);
+                if (op == NWF + NQF) {
+                    // V~ complete: as operand, one fragment per 16-token slab; decay of the state
+#pragma unroll
+                    for (int s = 0; s < 4; s++) vb[s] = pack8_16(accv[s / 2], s % 2, 1.f);
+#pragma unroll
+                    for (int td = 0; td < KD; td++)
+#pragma unroll
+                        for (int r = 0; r < 16; r++) S[td][r] *= egc;
+                }
+                if (op < NWF) {  // V~ = U + W~ S0, fragment (tt, s) = op
+                    const int s = op % KS16, tt = op / KS16;
+                    accv[tt] = mfma32_bf16(fr[op], sb[s], accv[tt]);
+                } else if (op < NWF + NQF) {  // O^T = S0^T Q~^T
+                    const int j = op - NWF, s = j % KS16, tt = j / KS16;
+                    acco[tt] = mfma32_bf16(sb[s], fr[op], acco[tt]);
+                } else if (op < NWF + NQF + NKF) {  // S = e^{gamma_C} S + K~^T V~, fragment (td, s)
+                    const int j = op - NWF - NQF, s = j % 4, td = j / 4;
+                    S[td] = mfma32_bf16(fr[op], vb[s], S[td]);
+                } else {  // O^T += V~^T P^T; P[i < 32][j >= 32] = 0 is skipped
+                    const int j = op - NWF - NQF - NKF;
+                    const int tt = j < 2 ? 0 : 1, s = j < 2 ? j : j - 2;
+                    acco[tt] = mfma32_bf16(vb[s], fr[op], acco[tt]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+
+            __syncthreads();  // done with this half of the buffer; the next record is in the other one
+
+            const int64_t tok0 = (int64_t)c * C;
+            const int valid = (int)min((int64_t)C, seq_len - tok0);
+#pragma unroll
+            for (int tt = 0; tt < 2; tt++)
+                if (32 * tt + l32 < valid) {
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; q4++) {
+                        bf16x4 r;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) r[e] = (bf16_t)acco[tt][4 * q4 + e];
+                        *reinterpret_cast<bf16x4*>(og + (tok0 + 32 * tt) * p.o_stride_t + 8 * q4) = r;
+                    }
+                }
+        } else {
+            __syncthreads();
+        }
+    }
+
+    if (active && p.ht != nullptr) {
+#pragma unroll
+        for (int td = 0; td < KD; td++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) p.ht[st_off + (int64_t)(32 * td + 8 * (r / 4) + r % 4) * p.V] = S[td][r];
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// launch
+// ------------------------------------------------------------------------------------------
+// ---- scan, variant without LDS: one wave per (chain, 32-column slice) reads its fragments straight from the records ----
 template <int K>
-__global__ __launch_bounds__(WAVE) void chunk_scan32_kernel(const ChunkParams p) {
+__global__ __launch_bounds__(WAVE) void chunk_scan32_direct_kernel(const ChunkParams p) {
     constexpr int KD = K / 32;    // 32-row tiles of the state
     constexpr int KS16 = K / 16;  // 16-wide slabs over the key dim
     constexpr int NW_ = 2 * KS16, NQ_ = 2 * KS16, NK_ = KD * 4, NP_ = 8;  // fragments per record
@@ -718,9 +959,22 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     if (events != nullptr) (void)hipEventRecord(events[2], stream);
 
     const int64_t chains = (int64_t)p.N * p.H;
-    p.scan_groups = p.V / 32;
     const int64_t chains8 = (chains + 7) / 8 * 8;
-    hipLaunchKernelGGL((chunk_scan32_kernel<K>), dim3((unsigned)(chains8 * p.scan_groups)), dim3(WAVE), 0, stream, p);
+    const int vtiles = p.V / 32;
+    if (chains * vtiles <= (int64_t)num_cus) {
+        // no more slices than CUs: one independent wave per 32-column slice, each on a CU of its own
+        p.scan_groups = vtiles;
+        hipLaunchKernelGGL((chunk_scan32_direct_kernel<K>), dim3((unsigned)(chains8 * vtiles)), dim3(WAVE), 0, stream, p);
+        return (int)hipGetLastError();
+    }
+    // many chains: the slices of a chain share each record through LDS; compute waves per workgroup = the
+    // widest group of 32-column tiles that divides V's tiles (up to 4)
+    const int nw = (vtiles % 4 == 0) ? 4 : (vtiles % 2 == 0) ? 2 : 1;
+    p.scan_groups = vtiles / nw;
+    const dim3 grid((unsigned)(chains8 * p.scan_groups));
+    if (nw == 4) hipLaunchKernelGGL((chunk_scan32_kernel<K, 4>), grid, dim3((4 + SCAN_LOADERS) * WAVE), 0, stream, p);
+    else if (nw == 2) hipLaunchKernelGGL((chunk_scan32_kernel<K, 2>), grid, dim3((2 + SCAN_LOADERS) * WAVE), 0, stream, p);
+    else hipLaunchKernelGGL((chunk_scan32_kernel<K, 1>), grid, dim3((1 + SCAN_LOADERS) * WAVE), 0, stream, p);
     return (int)hipGetLastError();
 }
 
