@@ -31,7 +31,7 @@
 //   Q~             [T_tok 2][slab K/16]  B fragments of O^T = S^T Q~^T (same register layout)
 //   K~^T           [T_d K/32][slab 4]    A fragments, rows = key dim, reduction = tokens
 //   P              [T_i 2][slab 4]       B fragments of O^T += V~^T P^T
-//   U              [T_n V/32][lane][T_tok 2][16]  accumulator layout
+//   U              [T_n V/32][lane][T_tok 2][16]  accumulator layout, lane l32 = column slice_col(l32) of the tile
 //   e^{gamma_C}
 
 #include <type_traits>
@@ -52,11 +52,20 @@ __device__ __forceinline__ bf16x8 pack8_16(const f32x16& d, int s, float sign) {
 
 // 4 consecutive rows x 16 consecutive columns of a row-major bf16 LDS matrix, transposed on the
 // way in: lane i of each 16-lane group receives M[row0 + 0..3][col0 + i].
+// With SWAP, the two middle groups of 4 columns change places: lane i receives column col0 + sigma(i),
+// sigma(4 q + b) = 4 swap(q) + b, swap(1) = 2, swap(2) = 1 (the column order of the scan's state slices).
+template <bool SWAP = false>
 __device__ __forceinline__ bf16x4 lds_read_tr4x16(const bf16_t* m, int ld, int row0, int col0, int l16) {
-    const bf16_t* p = m + (row0 + l16 / 4) * ld + col0 + 4 * (l16 % 4);
+    const int q = l16 % 4;
+    const int piece = SWAP ? ((q & 1) << 1 | (q >> 1)) : q;
+    const bf16_t* p = m + (row0 + l16 / 4) * ld + col0 + 4 * piece;
     const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p);
     return __builtin_bit_cast(bf16x4, v);
 }
+
+// Column of a 32-column state slice held by lane l32 (the order lds_read_tr4x16<true> produces): with it,
+// register pair (2 m, 2 m + 1) of a transposed accumulator tile covers 8 consecutive columns per lane.
+__device__ __forceinline__ int slice_col(int l32) { return (l32 & 0x13) | ((l32 & 4) << 1) | ((l32 & 8) >> 1); }
 
 __device__ __forceinline__ void split_hi_lo(float x, bf16_t& hi, bf16_t& lo) {
     hi = (bf16_t)x;
@@ -461,9 +470,10 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
             return r;
         };
         // transposed operand: 8 consecutive tokens j = 16 s + 8 h + e of column 32 tile + l32 of a row-major matrix
-        auto tr_frag = [&](const bf16_t* m, int ld, int s, int tile) -> bf16x8 {
-            const bf16x4 a = lds_read_tr4x16(m, ld, 16 * s + 8 * lh, 32 * tile + 16 * g16, l16);
-            const bf16x4 b = lds_read_tr4x16(m, ld, 16 * s + 8 * lh + 4, 32 * tile + 16 * g16, l16);
+        auto tr_frag = [&](const bf16_t* m, int ld, int s, int tile, auto swap_tag) -> bf16x8 {
+            constexpr bool SW = decltype(swap_tag)::value;
+            const bf16x4 a = lds_read_tr4x16<SW>(m, ld, 16 * s + 8 * lh, 32 * tile + 16 * g16, l16);
+            const bf16x4 b = lds_read_tr4x16<SW>(m, ld, 16 * s + 8 * lh + 4, 32 * tile + 16 * g16, l16);
             bf16x8 r;
 #pragma unroll
             for (int e = 0; e < 4; e++) r[e] = a[e], r[4 + e] = b[e];
@@ -478,7 +488,7 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
             for (int r = 0; r < 16; r++) acc[0][r] = 0.f, acc[1][r] = 0.f;
 #pragma unroll
             for (int s = 0; s < 4; s++) {
-                const bf16x8 kt = tr_frag(sK, LDK, s, td);
+                const bf16x8 kt = tr_frag(sK, LDK, s, td, std::false_type{});
                 if (s < 2) acc[0] = mfma32_bf16(kt, t_frag(0, s, s_cw), acc[0]);  // tokens < 32 only see j < 32
                 acc[1] = mfma32_bf16(kt, t_frag(1, s, s_cw), acc[1]);
                 __builtin_amdgcn_sched_barrier(0);
@@ -517,7 +527,7 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
                     for (int r = 0; r < 16; r++) acc[0][r] = 0.f, acc[1][r] = 0.f;
 #pragma unroll
                     for (int s = 0; s < 4; s++) {
-                        const bf16x8 vb = tr_frag(sV, LDV, s, tl);
+                        const bf16x8 vb = tr_frag(sV, LDV, s, tl, std::true_type{});  // columns in the scan's slice order
                         if (s < 2) acc[0] = mfma32_bf16(ta0[s], vb, acc[0]);
                         acc[1] = mfma32_bf16(ta1[s], vb, acc[1]);
                         __builtin_amdgcn_sched_barrier(0);
@@ -667,16 +677,21 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS) * WAVE) void chunk_scan32_kerne
     // ------------------------------ compute ------------------------------
     const int tn = vgroup * NW + wave;  // 32-column tile of V owned by this wave
     const bool active = 32 * tn < p.V;  // a last, partial column group has idle waves (they only keep the barriers)
-    // state tile td, register r: row 32 td + 8 (r/4) + 4 h + r%4, column 32 tn + l32
+    // state tile td, register r: row 32 td + 8 (r/4) + 4 h + r%4, column 32 tn + slice_col(l32)
     f32x16 S[KD];
-    const int64_t st_off = ((int64_t)n * p.H + h) * K * p.V + (int64_t)(4 * lh) * p.V + 32 * tn + l32;
+    const int64_t st_off = ((int64_t)n * p.H + h) * K * p.V + (int64_t)(4 * lh) * p.V + 32 * tn + slice_col(l32);
 #pragma unroll
     for (int td = 0; td < KD; td++)
 #pragma unroll
-        for (int r = 0; r < 16; r++)
-            S[td][r] = (active && p.h0 != nullptr) ? p.h0[st_off + (int64_t)(32 * td + 8 * (r / 4) + r % 4) * p.V] : 0.f;
-    // O^T tile tt, register r: token 32 tt + l32, column 32 tn + 8 (r/4) + 4 h + r%4
-    bf16_t* const og = p.o + b * p.o_stride_b + (seq_t0 + l32) * p.o_stride_t + (int64_t)h * p.o_stride_h + 32 * tn + 4 * lh;
+        for (int r = 0; r < 16; r++) S[td][r] = 0.f;
+    if (active && p.h0 != nullptr) {
+#pragma unroll
+        for (int td = 0; td < KD; td++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) S[td][r] = p.h0[st_off + (int64_t)(32 * td + 8 * (r / 4) + r % 4) * p.V];
+    }
+    // O^T tile tt, register r: token 32 tt + l32, column 32 tn + 16 (r/8) + 8 h + r%8 (slice_col order)
+    bf16_t* const og = p.o + b * p.o_stride_b + (seq_t0 + l32) * p.o_stride_t + (int64_t)h * p.o_stride_h + 32 * tn + 8 * lh;
 
     // MFMA schedule of one chunk: W~ (NWF) | Q~ (NQF) | K~^T (NKF) | P (6: the two zero fragments are skipped)
     constexpr int NOPS = NWF + NQF + NKF + 6;
@@ -756,12 +771,8 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS) * WAVE) void chunk_scan32_kerne
             for (int tt = 0; tt < 2; tt++)
                 if (32 * tt + l32 < valid) {
 #pragma unroll
-                    for (int q4 = 0; q4 < 4; q4++) {
-                        bf16x4 r;
-#pragma unroll
-                        for (int e = 0; e < 4; e++) r[e] = (bf16_t)acco[tt][4 * q4 + e];
-                        *reinterpret_cast<bf16x4*>(og + (tok0 + 32 * tt) * p.o_stride_t + 8 * q4) = r;
-                    }
+                    for (int half = 0; half < 2; half++)  // registers 8 half .. 8 half + 7: columns 16 half + 8 h + 0..7
+                        *reinterpret_cast<bf16x8*>(og + (tok0 + 32 * tt) * p.o_stride_t + 16 * half) = pack8_16(acco[tt], half, 1.f);
                 }
         } else {
             __syncthreads();
@@ -809,17 +820,17 @@ __global__ __launch_bounds__(WAVE) void chunk_scan32_direct_kernel(const ChunkPa
     }
     const int nchunks = slot_end - slot_begin;
 
-    // state tile td, register r: row 32 td + 8 (r/4) + 4 h + r%4, column 32 tn + l32
+    // state tile td, register r: row 32 td + 8 (r/4) + 4 h + r%4, column 32 tn + slice_col(l32)
     f32x16 S[KD];
-    const int64_t st_off = ((int64_t)n * p.H + h) * K * p.V + (int64_t)(4 * lh) * p.V + 32 * tn + l32;
+    const int64_t st_off = ((int64_t)n * p.H + h) * K * p.V + (int64_t)(4 * lh) * p.V + 32 * tn + slice_col(l32);
 #pragma unroll
     for (int td = 0; td < KD; td++)
 #pragma unroll
         for (int r = 0; r < 16; r++)
             S[td][r] = (p.h0 != nullptr) ? p.h0[st_off + (int64_t)(32 * td + 8 * (r / 4) + r % 4) * p.V] : 0.f;
 
-    // O^T tile tt, register r: token 32 tt + l32, column 32 tn + 8 (r/4) + 4 h + r%4
-    bf16_t* const og = p.o + b * p.o_stride_b + (seq_t0 + l32) * p.o_stride_t + (int64_t)h * p.o_stride_h + 32 * tn + 4 * lh;
+    // O^T tile tt, register r: token 32 tt + l32, column 32 tn + 16 (r/8) + 8 h + r%8 (slice_col order)
+    bf16_t* const og = p.o + b * p.o_stride_b + (seq_t0 + l32) * p.o_stride_t + (int64_t)h * p.o_stride_h + 32 * tn + 8 * lh;
     const uint8_t* rec = p.rec + ((int64_t)h * p.TC + slot_begin) * p.rec_bytes;
 
     bf16x8 wr[NW_], qr[NQ_], kr[NK_], pr[NP_], ur[4];
@@ -927,12 +938,8 @@ __global__ __launch_bounds__(WAVE) void chunk_scan32_direct_kernel(const ChunkPa
         for (int tt = 0; tt < 2; tt++)
             if (32 * tt + l32 < valid) {
 #pragma unroll
-                for (int q4 = 0; q4 < 4; q4++) {
-                    bf16x4 r;
-#pragma unroll
-                    for (int e = 0; e < 4; e++) r[e] = (bf16_t)acco[tt][4 * q4 + e];
-                    *reinterpret_cast<bf16x4*>(og + (tok0 + 32 * tt) * p.o_stride_t + 8 * q4) = r;
-                }
+                for (int half = 0; half < 2; half++)  // registers 8 half .. 8 half + 7: columns 16 half + 8 h + 0..7
+                    *reinterpret_cast<bf16x8*>(og + (tok0 + 32 * tt) * p.o_stride_t + 16 * half) = pack8_16(acco[tt], half, 1.f);
             }
         rec += p.rec_bytes;
     };
