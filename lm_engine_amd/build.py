@@ -33,6 +33,9 @@ HIPCC_FLAGS = (
     "-Wno-unused-function",
     # packed fp32 VALU forms are switched off for every kernel of this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the scan kernels are one fully unrolled schedule per chunk; the default size limit for "#pragma unroll"
+    # would leave their register arrays dynamically indexed, i.e. in scratch memory
+    "-mllvm", "-pragma-unroll-threshold=200000",
 )  # fmt: skip
 
 

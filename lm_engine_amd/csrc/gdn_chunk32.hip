@@ -9,8 +9,8 @@
 //
 //   * a wave of the scan owns a K x 32 slice of the state; operand fragments are laid out for
 //     the 32x32x16 shape;
-//   * the scan shares each record between the compute waves of a workgroup through a double buffer
-//     in LDS filled by dedicated loader waves;
+//   * the scan stages each record in an LDS double buffer filled by dedicated loader waves, hands its
+//     output to a dedicated store wave, and keeps its compute waves free of memory instructions;
 //   * prepare is persistent: a workgroup walks over (chunk, head) items and loads q, k, v of
 //     the next item into registers while it computes the current one;
 //   * the triangular inverse runs its block products on bf16 MFMA with operands split into
@@ -192,18 +192,20 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
                 const int row = tid / CPR + it * RPP;
                 *reinterpret_cast<bf16x8*>(&sK[row * LDK + piece * 8]) = kx[it];
                 *reinterpret_cast<bf16x8*>(&sQ[row * LDK + piece * 8]) = qx[it];
-                float a = 0.f, b = 0.f;
+                if (p.l2norm) {  // row sums of squares (uniform branch)
+                    float a = 0.f, b = 0.f;
 #pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    a += (float)kx[it][e] * (float)kx[it][e];
-                    b += (float)qx[it][e] * (float)qx[it][e];
-                }
+                    for (int e = 0; e < 8; e++) {
+                        a += (float)kx[it][e] * (float)kx[it][e];
+                        b += (float)qx[it][e] * (float)qx[it][e];
+                    }
 #pragma unroll
-                for (int off = 1; off < CPR; off <<= 1) {
-                    a += __shfl_xor(a, off, WAVE);
-                    b += __shfl_xor(b, off, WAVE);
+                    for (int off = 1; off < CPR; off <<= 1) {
+                        a += __shfl_xor(a, off, WAVE);
+                        b += __shfl_xor(b, off, WAVE);
+                    }
+                    if (piece == 0) s_ssk[row] = a, s_ssq[row] = b;
                 }
-                if (piece == 0) s_ssk[row] = a, s_ssq[row] = b;
             }
             if (wave == 0) {
                 float gv = gx;
@@ -548,24 +550,41 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
 // ------------------------------------------------------------------------------------------
 // scan
 //
-// A workgroup works on one (sequence, head): NW compute waves, each owning a K x 32 slice of the
-// fp32 state as MFMA accumulators, and NL = 4 loader waves.  Everything a chunk needs from its
-// record (the operand fragments W~, Q~, K~^T, P, the U tiles of this workgroup's columns and
-// e^{gamma_C}) goes through a double buffer in LDS: during chunk c the loaders move record c + 1
-// global -> registers -> LDS and already have record c + 2 (and c + 3) in flight in a second
-// register buffer, while the compute waves run the 54 MFMAs of chunk c out of the other half,
-// reading each fragment from LDS a few MFMAs before it is used.  One workgroup barrier per chunk
-// hands the halves over.  Sharing the record between the compute waves is what makes the scan
-// cheap per column: a wave that streams its own copy of the record spends its time issuing loads
-// (measured: one wave per CU loading 58 KB per chunk directly needs ~4600 cycles per chunk).
-// O is accumulated transposed (operands swapped) so that a lane ends up with 4 consecutive
-// columns of one token (8-byte stores).
+// A workgroup works on one (sequence, head) chain and NW of its 32-column slices: NW compute
+// waves, each owning a K x 32 slice of the fp32 state as MFMA accumulators, 4 loader waves and
+// (NW < 4) one output wave.
+//
+// Everything a chunk needs from its record (the operand fragments W~, Q~, K~^T, P, the U tiles
+// of this workgroup's columns and e^{gamma_C}) goes through a double buffer in LDS: during chunk
+// c the loaders move record c + 1 global -> registers -> LDS and already have records c + 2 and
+// c + 3 in flight in a second register buffer.  One workgroup barrier per chunk hands the halves
+// over.  The memory instructions are kept out of the compute waves on purpose: a wave that
+// issues a load or a store while the CU's vector-memory queue is full stalls until there is
+// room, and with one compute wave per SIMD that stall is a stall of the matrix pipe.  (Measured:
+// one wave per CU that streams its own 58 KB per chunk needs ~4600 cycles per chunk, and the 4
+// output stores per chunk cost a compute wave 340 - 980 cycles.)
+//
+// A compute wave runs the 54 MFMAs of a chunk (K = 128) as one unrolled schedule
+//     V~ = U + W~ S0 | O^T = S0^T Q~^T | S = e^{gamma_C} S0 + K~^T V~ | O^T += V~^T P^T
+// reading each fragment from LDS a few MFMAs before its use.  All other per-chunk work - decay of
+// the state, bf16 repacking of V~ and of the new state, conversion of the next chunk's U, the
+// hand-over of the output tile - is cut into pieces placed between MFMAs that do not depend on
+// them.  O is accumulated transposed (operands swapped) and the slice's columns are held in
+// slice_col order, so a lane ends up with 8 consecutive columns of one token (16 bytes).
+//
+// The slices of a chain sit in workgroups on one XCD and read the same records at the same time,
+// so the records come out of HBM once per chain (measured L2 hit rate 71 %, fetch = the record
+// bytes).  What bounds the kernel when every CU has a workgroup is the rate at which a CU gets
+// lines that were not in its L2 yet when asked for (~15 - 20 B/clk per CU, whatever the number of
+// waves asking); touching the lines ahead of time from a helper wave did not change that.
 // ------------------------------------------------------------------------------------------
 constexpr int SCAN_LOADERS = 4;
 
 template <int K, int NW>
-__global__ __launch_bounds__((NW + SCAN_LOADERS) * WAVE) void chunk_scan32_kernel(const ChunkParams p) {
+__global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void chunk_scan32_kernel(const ChunkParams p) {
     constexpr int NL = SCAN_LOADERS;
+    // a separate wave writes the output (see below); with four compute waves the LDS has no room for its staging
+    constexpr bool OS = NW < 4;
     constexpr int KD = K / 32;    // 32-row tiles of the state
     constexpr int KS16 = K / 16;  // 16-wide slabs over the key dim
     constexpr int NWF = 2 * KS16, NQF = 2 * KS16, NKF = KD * 4, NPF = 8;  // fragments of W~, Q~, K~^T, P
@@ -579,6 +598,7 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS) * WAVE) void chunk_scan32_kerne
     static_assert(STAGE_FRAGS % NL == 0, "fragments must divide over the loader waves");
 
     __shared__ __attribute__((aligned(16))) uint8_t stage[2][STAGE_BYTES];
+    __shared__ __attribute__((aligned(16))) uint8_t ostage[OS ? NW * 2 * C * 64 : 16];
 
     const int lane = threadIdx.x % WAVE;
     const int wave = threadIdx.x / WAVE;
@@ -605,6 +625,42 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS) * WAVE) void chunk_scan32_kerne
     const int nchunks = slot_end - slot_begin;
     const uint8_t* rec = p.rec + ((int64_t)h * p.TC + slot_begin) * p.rec_bytes;
 
+    // output staging: [compute wave][chunk parity][64 tokens][64 bytes], the four 16-byte pieces of a row
+    // XOR-swizzled with (row / 4) % 4 so that both sides access it without bank conflicts
+    auto ostage_at = [&](int w, int parity, int row, int piece) -> uint8_t* {
+        return ostage + ((w * 2 + parity) * C + row) * 64 + ((piece ^ ((row >> 2) & 3)) << 4);
+    };
+    if (OS && wave == NW + NL) {
+        // ------------------------------ output store ------------------------------
+        // The compute waves leave the bf16 output tile of chunk c in LDS while they work on chunk c + 1; this
+        // wave writes it out after the next barrier.  A store that waits for queue space then stalls here and
+        // not in the wave that feeds the matrix pipe.
+        const int row0 = lane / 4, piece = lane % 4;
+        bf16_t* og = p.o + b * p.o_stride_b + (seq_t0 + row0) * p.o_stride_t + (int64_t)h * p.o_stride_h +
+                     32 * (vgroup * NW) + 8 * piece;
+        auto flush = [&](int c) {  // output of chunk c
+            const int valid = (int)min((int64_t)C, seq_len - (int64_t)c * C);
+#pragma unroll
+            for (int w = 0; w < NW; w++) {
+                bf16x8 rows[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    rows[i] = *reinterpret_cast<const bf16x8*>(ostage_at(w, c & 1, row0 + 16 * i, piece));
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    if (row0 + 16 * i < valid)
+                        *reinterpret_cast<bf16x8*>(og + ((int64_t)c * C + 16 * i) * p.o_stride_t + 32 * w) = rows[i];
+            }
+        };
+        __syncthreads();
+        for (int c = 0; c < nchunks; c++) {
+            __syncthreads();
+            if (c > 0) flush(c - 1);
+        }
+        __syncthreads();
+        if (nchunks > 0) flush(nchunks - 1);
+        return;
+    }
     if (wave >= NW) {
         // ------------------------------ loader ------------------------------
         // fragment f of the stage: f < SHARED_FRAGS comes from the head of the record, the rest from
@@ -671,12 +727,12 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS) * WAVE) void chunk_scan32_kerne
                 __syncthreads();
             }
         }
+        if (OS) __syncthreads();  // the hand-over of the last output tile
         return;
     }
 
     // ------------------------------ compute ------------------------------
-    const int tn = vgroup * NW + wave;  // 32-column tile of V owned by this wave
-    const bool active = 32 * tn < p.V;  // a last, partial column group has idle waves (they only keep the barriers)
+    const int tn = vgroup * NW + wave;  // 32-column tile of V owned by this wave (the launcher makes NW divide V / 32)
     // state tile td, register r: row 32 td + 8 (r/4) + 4 h + r%4, column 32 tn + slice_col(l32)
     f32x16 S[KD];
     const int64_t st_off = ((int64_t)n * p.H + h) * K * p.V + (int64_t)(4 * lh) * p.V + 32 * tn + slice_col(l32);
@@ -684,267 +740,156 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS) * WAVE) void chunk_scan32_kerne
     for (int td = 0; td < KD; td++)
 #pragma unroll
         for (int r = 0; r < 16; r++) S[td][r] = 0.f;
-    if (active && p.h0 != nullptr) {
+    if (p.h0 != nullptr) {
 #pragma unroll
         for (int td = 0; td < KD; td++)
 #pragma unroll
             for (int r = 0; r < 16; r++) S[td][r] = p.h0[st_off + (int64_t)(32 * td + 8 * (r / 4) + r % 4) * p.V];
     }
     // O^T tile tt, register r: token 32 tt + l32, column 32 tn + 16 (r/8) + 8 h + r%8 (slice_col order)
-    bf16_t* const og = p.o + b * p.o_stride_b + (seq_t0 + l32) * p.o_stride_t + (int64_t)h * p.o_stride_h + 32 * tn + 8 * lh;
+    bf16_t* og = p.o + b * p.o_stride_b + (seq_t0 + l32) * p.o_stride_t + (int64_t)h * p.o_stride_h + 32 * tn + 8 * lh;
+    const int64_t og_step = (int64_t)C * p.o_stride_t;
 
-    // MFMA schedule of one chunk: W~ (NWF) | Q~ (NQF) | K~^T (NKF) | P (6: the two zero fragments are skipped)
+    // MFMA schedule of one chunk: W~ (NWF) | Q~ (NQF) | K~^T (NKF) | P (6: the two zero fragments are skipped).
+    // Everything else a chunk needs (decay of the state, bf16 repacking of V~ and of the new state, conversion
+    // of the next U, conversion and store of the previous chunk's output) is cut into pieces that sit between
+    // MFMAs whose operands do not depend on them, so the matrix pipe stays fed by this one wave.
     constexpr int NOPS = NWF + NQF + NKF + 6;
-    constexpr int LOOKAHEAD = 6;  // LDS reads are issued this many MFMAs ahead of their use
+    constexpr int LA = 6;  // LDS reads are issued this many MFMAs ahead of their use
+    constexpr int OP_Q = NWF, OP_K = NWF + NQF, OP_P = NWF + NQF + NKF, OP_BAR = NOPS - LA;
+    static_assert(OP_BAR >= OP_K, "the barrier must come after the reads of the W~ and Q~ fragments");
     auto lds_frag = [&](const uint8_t* st, int op) -> bf16x8 {
         int f = op;
-        if (op >= NWF + NQF + NKF) {  // P fragments (tt, s) with tt == 1 or s < 2: indices 0, 1, 4, 5, 6, 7
-            const int j = op - (NWF + NQF + NKF);
-            f = NWF + NQF + NKF + (j < 2 ? j : j + 2);
+        if (op >= OP_P) {  // P fragments (tt, s) with tt == 1 or s < 2: indices 0, 1, 4, 5, 6, 7
+            const int j = op - OP_P;
+            f = OP_P + (j < 2 ? j : j + 2);
         }
         return reinterpret_cast<const bf16x8*>(st)[f * WAVE + lane];
     };
+    auto lds_u = [&](const uint8_t* st, int i) -> bf16x8 {
+        return reinterpret_cast<const bf16x8*>(st + SHARED_BYTES)[(wave * WAVE + lane) * 4 + i];
+    };
+    auto lds_eg = [&](const uint8_t* st) -> float { return *reinterpret_cast<const float*>(st + STAGE_FRAGS * FRAG_BYTES); };
+
+    f32x16 accv[2], acco[2];
+    bf16x8 sb[KS16], vb[4], ur[4], fnext[LA];
+    float egc;
+#pragma unroll
+    for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acco[tt][r] = 0.f;
 
     __syncthreads();  // stage[0] holds record 0
 
+    // what the tail of a chunk does for the next one, for chunk 0
+#pragma unroll
+    for (int i = 0; i < 4; i++) ur[i] = lds_u(stage[0], i);
+    egc = lds_eg(stage[0]);
+#pragma unroll
+    for (int i = 0; i < LA; i++) fnext[i] = lds_frag(stage[0], i);
+#pragma unroll
+    for (int s = 0; s < KS16; s++) sb[s] = pack8_16(S[s / 2], s % 2, 1.f);
+#pragma unroll
+    for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) accv[tt][r] = (float)ur[2 * tt + r / 8][r % 8];
+
+    int valid_prev = 0;  // tokens of the previous chunk, whose output is still in acco
     for (int c = 0; c < nchunks; c++) {
         const uint8_t* st = stage[c & 1];
-        if (active) {
-            const bf16x8* uf = reinterpret_cast<const bf16x8*>(st + SHARED_BYTES) + (wave * WAVE + lane) * 4;
-            bf16x8 ur[4];
+        const uint8_t* stn = stage[(c + 1) & 1];
+        const int valid = (int)min((int64_t)C, seq_len - (int64_t)c * C);
+        bf16x8 fr[NOPS];
 #pragma unroll
-            for (int i = 0; i < 4; i++) ur[i] = uf[i];
-            const float egc = *reinterpret_cast<const float*>(st + STAGE_FRAGS * FRAG_BYTES);
-            bf16x8 fr[NOPS];
-#pragma unroll
-            for (int op = 0; op < LOOKAHEAD; op++) fr[op] = lds_frag(st, op);
-
-            // state as bf16 operand, one fragment per 16-row slab
-            bf16x8 sb[KS16];
-#pragma unroll
-            for (int s = 0; s < KS16; s++) sb[s] = pack8_16(S[s / 2], s % 2, 1.f);
-            f32x16 accv[2], acco[2];
-#pragma unroll
-            for (int tt = 0; tt < 2; tt++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    accv[tt][r] = (float)ur[2 * tt + r / 8][r % 8];
-                    acco[tt][r] = 0.f;
-                }
-            bf16x8 vb[4];
-            __builtin_amdgcn_sched_barrier(0);
+        for (int i = 0; i < LA; i++) fr[i] = fnext[i];
+        __builtin_amdgcn_sched_barrier(0);
 
 #pragma unroll
-            for (int op = 0; op < NOPS; op++) {
-                if (op + LOOKAHEAD < NOPS) fr[op + LOOKAHEAD] = lds_frag(st, op + LOOKAHEAD);
-                if (op == NWF + NQF) {
-                    // V~ complete: as operand, one fragment per 16-token slab; decay of the state
+        for (int op = 0; op < NOPS; op++) {
+            // ---- operand reads: this record until the barrier, the next one after it ----
+            if (op + LA < NOPS) fr[op + LA] = lds_frag(st, op + LA);
+            if (op == OP_BAR) {
+                __syncthreads();  // this wave is done with record c; record c + 1 is in the other half
 #pragma unroll
-                    for (int s = 0; s < 4; s++) vb[s] = pack8_16(accv[s / 2], s % 2, 1.f);
-#pragma unroll
-                    for (int td = 0; td < KD; td++)
-#pragma unroll
-                        for (int r = 0; r < 16; r++) S[td][r] *= egc;
+                for (int i = 0; i < 4; i++) ur[i] = lds_u(stn, i);
+                egc = lds_eg(stn);
+            }
+            if (op >= OP_BAR) fnext[op - OP_BAR] = lds_frag(stn, op - OP_BAR);
+
+            // ---- side work ----
+            if (op >= 1 && op <= 4) {  // output of the previous chunk: tile (op-1)/2, registers 8 half .. 8 half + 7
+                const int tt = (op - 1) / 2, half = (op - 1) % 2;
+                if (OS) {
+                    if (c > 0)
+                        *reinterpret_cast<bf16x8*>(ostage_at(wave, (c - 1) & 1, 32 * tt + l32, 2 * half + lh)) =
+                            pack8_16(acco[tt], half, 1.f);
+                } else if (32 * tt + l32 < valid_prev) {
+                    *reinterpret_cast<bf16x8*>(og - og_step + (int64_t)(32 * tt) * p.o_stride_t + 16 * half) =
+                        pack8_16(acco[tt], half, 1.f);
                 }
-                if (op < NWF) {  // V~ = U + W~ S0, fragment (tt, s) = op
-                    const int s = op % KS16, tt = op / KS16;
-                    accv[tt] = mfma32_bf16(fr[op], sb[s], accv[tt]);
-                } else if (op < NWF + NQF) {  // O^T = S0^T Q~^T
-                    const int j = op - NWF, s = j % KS16, tt = j / KS16;
+            }
+            if (op < NWF) {  // decay of the state (its bf16 copy for this chunk is already in sb)
+                constexpr int PER = (KD * 16) / NWF;
+#pragma unroll
+                for (int i = 0; i < PER; i++) S[(op * PER + i) / 16][(op * PER + i) % 16] *= egc;
+            }
+            if (op == KS16 + 2) vb[0] = pack8_16(accv[0], 0, 1.f);  // V~ rows 0..31 are complete after op KS16 - 1
+            if (op == KS16 + 3) vb[1] = pack8_16(accv[0], 1, 1.f);
+            if (op == OP_Q + 2) vb[2] = pack8_16(accv[1], 0, 1.f);  // rows 32..63 after op NWF - 1
+            if (op == OP_Q + 3) vb[3] = pack8_16(accv[1], 1, 1.f);
+            if (op >= OP_K + 5) {  // new state tile td is complete after K~^T op 4 td + 3: its two slabs as operands
+                const int j = op - OP_K - 5;
+                if (j % 4 < 2 && j / 4 < KD) sb[2 * (j / 4) + j % 4] = pack8_16(S[j / 4], j % 4, 1.f);
+            }
+            if (op >= NOPS - 4) {  // U of the next chunk -> fp32 accumulators (V~ of this chunk lives on in vb)
+                const int q = op - (NOPS - 4);
+#pragma unroll
+                for (int i = 0; i < 8; i++) accv[q / 2][8 * (q % 2) + i] = (float)ur[q][i];
+            }
+
+            // ---- the MFMA ----
+            if (op < OP_Q) {  // V~ = U + W~ S0, fragment (tt, s) = op
+                const int s = op % KS16, tt = op / KS16;
+                accv[tt] = mfma32_bf16(fr[op], sb[s], accv[tt]);
+            } else if (op < OP_K) {  // O^T = S0^T Q~^T
+                const int j = op - OP_Q, s = j % KS16, tt = j / KS16;
+                if (s == 0) {
+                    f32x16 zero;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) zero[r] = 0.f;
+                    acco[tt] = mfma32_bf16(sb[s], fr[op], zero);
+                } else {
                     acco[tt] = mfma32_bf16(sb[s], fr[op], acco[tt]);
-                } else if (op < NWF + NQF + NKF) {  // S = e^{gamma_C} S + K~^T V~, fragment (td, s)
-                    const int j = op - NWF - NQF, s = j % 4, td = j / 4;
-                    S[td] = mfma32_bf16(fr[op], vb[s], S[td]);
-                } else {  // O^T += V~^T P^T; P[i < 32][j >= 32] = 0 is skipped
-                    const int j = op - NWF - NQF - NKF;
-                    const int tt = j < 2 ? 0 : 1, s = j < 2 ? j : j - 2;
-                    acco[tt] = mfma32_bf16(vb[s], fr[op], acco[tt]);
                 }
-                __builtin_amdgcn_sched_barrier(0);
+            } else if (op < OP_P) {  // S = e^{gamma_C} S + K~^T V~, fragment (td, s)
+                const int j = op - OP_K, s = j % 4, td = j / 4;
+                S[td] = mfma32_bf16(fr[op], vb[s], S[td]);
+            } else {  // O^T += V~^T P^T; P[i < 32][j >= 32] = 0 is skipped
+                const int j = op - OP_P;
+                const int tt = j < 2 ? 0 : 1, s = j < 2 ? j : j - 2;
+                acco[tt] = mfma32_bf16(vb[s], fr[op], acco[tt]);
             }
-
-            __syncthreads();  // done with this half of the buffer; the next record is in the other one
-
-            const int64_t tok0 = (int64_t)c * C;
-            const int valid = (int)min((int64_t)C, seq_len - tok0);
-#pragma unroll
-            for (int tt = 0; tt < 2; tt++)
-                if (32 * tt + l32 < valid) {
-#pragma unroll
-                    for (int half = 0; half < 2; half++)  // registers 8 half .. 8 half + 7: columns 16 half + 8 h + 0..7
-                        *reinterpret_cast<bf16x8*>(og + (tok0 + 32 * tt) * p.o_stride_t + 16 * half) = pack8_16(acco[tt], half, 1.f);
-                }
-        } else {
-            __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
         }
+        valid_prev = valid;
+        og += og_step;
     }
 
-    if (active && p.ht != nullptr) {
+    // output of the last chunk
 #pragma unroll
-        for (int td = 0; td < KD; td++)
+    for (int tt = 0; tt < 2; tt++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) p.ht[st_off + (int64_t)(32 * td + 8 * (r / 4) + r % 4) * p.V] = S[td][r];
-    }
-}
-
-// ------------------------------------------------------------------------------------------
-// launch
-// ------------------------------------------------------------------------------------------
-// ---- scan, variant without LDS: one wave per (chain, 32-column slice) reads its fragments straight from the records ----
-template <int K>
-__global__ __launch_bounds__(WAVE) void chunk_scan32_direct_kernel(const ChunkParams p) {
-    constexpr int KD = K / 32;    // 32-row tiles of the state
-    constexpr int KS16 = K / 16;  // 16-wide slabs over the key dim
-    constexpr int NW_ = 2 * KS16, NQ_ = 2 * KS16, NK_ = KD * 4, NP_ = 8;  // fragments per record
-
-    const int lane = threadIdx.x;
-    const int l32 = lane % 32, lh = lane / 32;
-
-    // workgroup (= one wave) -> (sequence-head chain, 32-column slice); the slices of a chain stay on
-    // one XCD (id % 8) so that its records are fetched into a single L2
-    const int id = blockIdx.x;
-    const int xcd = id % 8, rest = id / 8;
-    const int tn = rest % p.scan_groups;
-    const int chain = (rest / p.scan_groups) * 8 + xcd;
-    if (chain >= p.N * p.H) return;
-    const int n = chain / p.H, h = chain % p.H;
-
-    int slot_begin, slot_end;
-    int64_t b, seq_t0, seq_len;
-    if (p.cu_seqlens == nullptr) {
-        slot_begin = n * p.NT, slot_end = slot_begin + p.NT;
-        b = n, seq_t0 = 0, seq_len = p.T;
-    } else {
-        slot_begin = p.chunk_off[n], slot_end = p.chunk_off[n + 1];
-        b = 0, seq_t0 = p.cu_seqlens[n], seq_len = p.cu_seqlens[n + 1] - seq_t0;
-    }
-    const int nchunks = slot_end - slot_begin;
-
-    // state tile td, register r: row 32 td + 8 (r/4) + 4 h + r%4, column 32 tn + slice_col(l32)
-    f32x16 S[KD];
-    const int64_t st_off = ((int64_t)n * p.H + h) * K * p.V + (int64_t)(4 * lh) * p.V + 32 * tn + slice_col(l32);
-#pragma unroll
-    for (int td = 0; td < KD; td++)
-#pragma unroll
-        for (int r = 0; r < 16; r++)
-            S[td][r] = (p.h0 != nullptr) ? p.h0[st_off + (int64_t)(32 * td + 8 * (r / 4) + r % 4) * p.V] : 0.f;
-
-    // O^T tile tt, register r: token 32 tt + l32, column 32 tn + 16 (r/8) + 8 h + r%8 (slice_col order)
-    bf16_t* const og = p.o + b * p.o_stride_b + (seq_t0 + l32) * p.o_stride_t + (int64_t)h * p.o_stride_h + 32 * tn + 8 * lh;
-    const uint8_t* rec = p.rec + ((int64_t)h * p.TC + slot_begin) * p.rec_bytes;
-
-    bf16x8 wr[NW_], qr[NQ_], kr[NK_], pr[NP_], ur[4];
-    float egc = 0.f;
-    auto frag_ptr = [&](const uint8_t* r, uint32_t off, int f) {
-        return reinterpret_cast<const bf16x8*>(r + off) + f * WAVE + lane;
-    };
-    if (nchunks > 0) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) ur[i] = *(reinterpret_cast<const bf16x8*>(rec + p.off_u) + ((int64_t)tn * WAVE + lane) * 4 + i);
-        egc = *reinterpret_cast<const float*>(rec + p.off_eg);
-#pragma unroll
-        for (int i = 0; i < NW_; i++) wr[i] = *frag_ptr(rec, 0, i);
-#pragma unroll
-        for (int i = 0; i < NQ_; i++) qr[i] = *frag_ptr(rec, p.off_qs, i);
-#pragma unroll
-        for (int i = 0; i < NK_; i++) kr[i] = *frag_ptr(rec, p.off_kt, i);
-#pragma unroll
-        for (int i = 0; i < NP_; i++) pr[i] = *frag_ptr(rec, p.off_p, i);
-    }
-
-    auto iteration = [&](int c, auto more_tag) {
-        constexpr bool more = decltype(more_tag)::value;
-        const uint8_t* nxt = rec + p.rec_bytes;  // only dereferenced when `more`
-
-        // state as bf16 operand, one fragment per 16-row slab
-        bf16x8 sb[KS16];
-#pragma unroll
-        for (int s = 0; s < KS16; s++) sb[s] = pack8_16(S[s / 2], s % 2, 1.f);
-        f32x16 accv[2], acco[2];
-#pragma unroll
-        for (int tt = 0; tt < 2; tt++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                accv[tt][r] = (float)ur[2 * tt + r / 8][r % 8];
-                acco[tt][r] = 0.f;
+        for (int half = 0; half < 2; half++) {
+            if (OS) {
+                if (nchunks > 0)
+                    *reinterpret_cast<bf16x8*>(ostage_at(wave, (nchunks - 1) & 1, 32 * tt + l32, 2 * half + lh)) =
+                        pack8_16(acco[tt], half, 1.f);
+            } else if (32 * tt + l32 < valid_prev) {
+                *reinterpret_cast<bf16x8*>(og - og_step + (int64_t)(32 * tt) * p.o_stride_t + 16 * half) =
+                    pack8_16(acco[tt], half, 1.f);
             }
-        const float eg_cur = egc;
-        if constexpr (more) {
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                ur[i] = *(reinterpret_cast<const bf16x8*>(nxt + p.off_u) + ((int64_t)tn * WAVE + lane) * 4 + i);
-            egc = *reinterpret_cast<const float*>(nxt + p.off_eg);
         }
-        __builtin_amdgcn_sched_barrier(0);
-
-        // V~ = U - W S0: accv[tt] += W~(tt, s) sb[s]; each fragment register is refilled from the next
-        // record right behind the MFMA that consumed it
-#pragma unroll
-        for (int s = 0; s < KS16; s++)
-#pragma unroll
-            for (int tt = 0; tt < 2; tt++) {
-                const int f = tt * KS16 + s;
-                accv[tt] = mfma32_bf16(wr[f], sb[s], accv[tt]);
-                if constexpr (more) wr[f] = *frag_ptr(nxt, 0, f);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        // O^T = S0^T Q~^T
-#pragma unroll
-        for (int s = 0; s < KS16; s++)
-#pragma unroll
-            for (int tt = 0; tt < 2; tt++) {
-                const int f = tt * KS16 + s;
-                acco[tt] = mfma32_bf16(sb[s], qr[f], acco[tt]);
-                if constexpr (more) qr[f] = *frag_ptr(nxt, p.off_qs, f);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-
-        // V~ as operand, one fragment per 16-token slab; decay of the state
-        bf16x8 vb[4];
-#pragma unroll
-        for (int s = 0; s < 4; s++) vb[s] = pack8_16(accv[s / 2], s % 2, 1.f);
-#pragma unroll
-        for (int td = 0; td < KD; td++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) S[td][r] *= eg_cur;
-        __builtin_amdgcn_sched_barrier(0);
-
-        // S = e^{gamma_C} S + K~^T V~
-#pragma unroll
-        for (int s = 0; s < 4; s++)
-#pragma unroll
-            for (int td = 0; td < KD; td++) {
-                const int f = td * 4 + s;
-                S[td] = mfma32_bf16(kr[f], vb[s], S[td]);
-                if constexpr (more) kr[f] = *frag_ptr(nxt, p.off_kt, f);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        // O^T += V~^T P^T (P[i < 32][j >= 32] = 0: those two products are skipped)
-#pragma unroll
-        for (int s = 0; s < 4; s++)
-#pragma unroll
-            for (int tt = 0; tt < 2; tt++) {
-                const int f = tt * 4 + s;
-                if (tt == 1 || s < 2) acco[tt] = mfma32_bf16(vb[s], pr[f], acco[tt]);
-                if constexpr (more) {
-                    if (tt == 1 || s < 2) pr[f] = *frag_ptr(nxt, p.off_p, f);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-
-        const int64_t tok0 = (int64_t)c * C;
-        const int valid = (int)min((int64_t)C, seq_len - tok0);
-#pragma unroll
-        for (int tt = 0; tt < 2; tt++)
-            if (32 * tt + l32 < valid) {
-#pragma unroll
-                for (int half = 0; half < 2; half++)  // registers 8 half .. 8 half + 7: columns 16 half + 8 h + 0..7
-                    *reinterpret_cast<bf16x8*>(og + (tok0 + 32 * tt) * p.o_stride_t + 16 * half) = pack8_16(acco[tt], half, 1.f);
-            }
-        rec += p.rec_bytes;
-    };
-    for (int c = 0; c + 1 < nchunks; c++) iteration(c, std::true_type{});
-    if (nchunks > 0) iteration(nchunks - 1, std::false_type{});
+    if (OS) __syncthreads();
 
     if (p.ht != nullptr) {
 #pragma unroll
@@ -965,23 +910,19 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
     if (events != nullptr) (void)hipEventRecord(events[2], stream);
 
+    // Compute waves (32-column slices) per scan workgroup: one while that gives no more workgroups than CUs, so
+    // that every slice has a CU's load bandwidth to itself; otherwise 2 or 4 slices of a chain share the
+    // records through one workgroup's LDS (they must divide the V / 32 tiles).
     const int64_t chains = (int64_t)p.N * p.H;
     const int64_t chains8 = (chains + 7) / 8 * 8;
     const int vtiles = p.V / 32;
-    if (chains * vtiles <= (int64_t)num_cus) {
-        // no more slices than CUs: one independent wave per 32-column slice, each on a CU of its own
-        p.scan_groups = vtiles;
-        hipLaunchKernelGGL((chunk_scan32_direct_kernel<K>), dim3((unsigned)(chains8 * vtiles)), dim3(WAVE), 0, stream, p);
-        return (int)hipGetLastError();
-    }
-    // many chains: the slices of a chain share each record through LDS; compute waves per workgroup = the
-    // widest group of 32-column tiles that divides V's tiles (up to 4)
-    const int nw = (vtiles % 4 == 0) ? 4 : (vtiles % 2 == 0) ? 2 : 1;
+    int nw = 1;
+    while (nw < 4 && vtiles % (2 * nw) == 0 && chains * (vtiles / nw) > (int64_t)num_cus) nw *= 2;
     p.scan_groups = vtiles / nw;
     const dim3 grid((unsigned)(chains8 * p.scan_groups));
     if (nw == 4) hipLaunchKernelGGL((chunk_scan32_kernel<K, 4>), grid, dim3((4 + SCAN_LOADERS) * WAVE), 0, stream, p);
-    else if (nw == 2) hipLaunchKernelGGL((chunk_scan32_kernel<K, 2>), grid, dim3((2 + SCAN_LOADERS) * WAVE), 0, stream, p);
-    else hipLaunchKernelGGL((chunk_scan32_kernel<K, 1>), grid, dim3((1 + SCAN_LOADERS) * WAVE), 0, stream, p);
+    else if (nw == 2) hipLaunchKernelGGL((chunk_scan32_kernel<K, 2>), grid, dim3((2 + SCAN_LOADERS + 1) * WAVE), 0, stream, p);
+    else hipLaunchKernelGGL((chunk_scan32_kernel<K, 1>), grid, dim3((1 + SCAN_LOADERS + 1) * WAVE), 0, stream, p);
     return (int)hipGetLastError();
 }
 
