@@ -33,6 +33,22 @@ if ROOT not in sys.path:
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 
+# HBM bytes per launch, (workload, kernel) -> bytes.  Not measurable from inside this process: these are
+# rocprofv3 --pmc readings of FETCH_SIZE and WRITE_SIZE (KiB per dispatch) for this very command, each scaled
+# by what the same counter reads for a plain 1 GiB copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the counter
+# summaries are kept under profiles/.  Workloads that were not profiled report null.
+_KIB = 1024
+MEASURED_HBM_TRAFFIC_BYTES = {
+    ("cfg1_chunk_fwd_bf16", "chunk_prepare"): (2.0 * 104712.5 + 295041.7) * _KIB,
+    ("cfg1_chunk_fwd_bf16", "chunk_scan"): (2.0 * 147853.4 + 69632.6) * _KIB,
+    ("cfg3_decode_bf16", "recurrent_kernel"): (2.0 * 265449.7 + 526881.4) * _KIB,
+}
+
+
+def measured_traffic(workload: str, kernel: str):
+    value = MEASURED_HBM_TRAFFIC_BYTES.get((workload, kernel))
+    return None if value is None else int(value)
+
 
 def parse_args():
     ap = argparse.ArgumentParser()
@@ -105,7 +121,7 @@ def bench_chunk(w, steps, warmup):
             "peak": MFMA_BF16_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": per_kernel[dominant]["mfma_frac"],
-            "traffic": None,
+            "traffic": measured_traffic(w.name, dominant),
         },
         "step": {
             "tflops_dense": round(whole_tflops, 1),
@@ -154,7 +170,8 @@ def bench_decode(steps, warmup):
         "kernel_ms": round(kernel_ms, 4),
         "seq_tokens_per_s": round(w.B / (wall_ms * 1e-3), 1),
         "roofline": {"kernel": "recurrent_kernel", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": measured_traffic("cfg3_decode_bf16", "recurrent_kernel")},
     }  # fmt: skip
 
 
