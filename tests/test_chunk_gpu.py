@@ -44,6 +44,23 @@ def test_head_dims(K, V):
     _check(random_inputs(B=1, T=200, H=2, K=K, V=V, dtype=BF16, seed=60 + K + V), f"K={K} V={V}")
 
 
+@pytest.mark.parametrize(
+    "B, T, H, K, V, slices_per_workgroup",
+    [
+        (9, 130, 16, 128, 128, 2),   # 144 chains x 4 slices: more slices than CUs -> two per workgroup
+        (20, 130, 16, 128, 128, 4),  # 320 chains x 4 slices -> four per workgroup
+        (12, 130, 8, 128, 256, 4),   # 96 chains x 8 slices -> four per workgroup, two groups per chain
+        (17, 130, 16, 64, 64, 2),    # 272 chains x 2 slices -> two per workgroup (all of V)
+        (30, 130, 16, 128, 96, 1),   # 3 tiles of V: only one slice per workgroup divides them
+    ],
+)
+def test_many_chains_share_records_in_a_workgroup(B, T, H, K, V, slices_per_workgroup):
+    # the scan puts 1, 2 or 4 column slices of a chain into one workgroup depending on how many slices
+    # there are against the number of CUs (256 on MI355X); ragged length so the last chunk is partial
+    inp = random_inputs(B=B, T=T, H=H, K=K, V=V, dtype=BF16, seed=400 + B + V)
+    _check(inp, f"B={B} H={H} K={K} V={V}: {slices_per_workgroup} slice(s) per workgroup")
+
+
 def test_short_sequence_single_partial_chunk():
     _check(random_inputs(B=3, T=17, H=2, K=128, V=128, dtype=BF16, seed=70), "T=17")
 
