@@ -13,6 +13,7 @@ inputs already resident in HBM.  Prints ONE JSON line:
   decode       the decode step (configuration 3: 256 sequences x 32 heads, fp32 state 512 MiB
                updated in place) against the HBM peak, state buffers rotated so the state
                cannot live in the 256 MB Infinity Cache
+  conv         the depthwise causal convolution in front of the operator, same batch, against the HBM peak
   cpu_baseline the naive token-by-token torch restatement of the operator (oracle/), timed on
                this host's cores on a bounded prefix of the same workload
 """
@@ -57,7 +58,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", type=int, default=1, choices=(1, 2, 4))
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-decode", action="store_true")
+    ap.add_argument("--no-decode", action="store_true", help="skip the decode and convolution legs")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target duration of the CPU baseline sample")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, the known-size kernel the HBM counters are scaled by")
@@ -175,6 +176,41 @@ def bench_decode(steps, warmup):
     }  # fmt: skip
 
 
+def bench_conv(w, steps, warmup):
+    """The depthwise causal convolution (kernel size 4, bias, SiLU) over the fused q | k | v projection of
+    the same workload: [B, T, H (2K + V)] bf16 in, same shape out, carried state written.  HBM-bound:
+    algorithmic bytes = one read of x + one write of y."""
+    import torch
+
+    import lm_engine_amd
+
+    C = w.H * (2 * w.K + w.V)
+    gen = torch.Generator("cpu").manual_seed(4321)
+    x = torch.randn(w.B, w.T, C, generator=gen).to(torch.bfloat16).cuda()
+    weight = (0.5 * torch.randn(C, 1, 4, generator=gen)).to(torch.bfloat16).cuda()
+    bias = (0.1 * torch.randn(C, generator=gen)).to(torch.bfloat16).cuda()
+    call = lambda: lm_engine_amd.depthwise_causal_convolution(x, weight, bias, None, None, True, "silu")  # noqa: E731
+    for _ in range(warmup):
+        call()
+    torch.cuda.synchronize()
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for start, stop in events:
+        start.record()
+        call()
+        stop.record()
+    torch.cuda.synchronize()
+    kernel_ms = sum(start.elapsed_time(stop) for start, stop in events) / steps
+    nbytes = 2 * x.numel() * x.element_size()
+    gbs = nbytes / (kernel_ms * 1e-3) / 1e9
+    return {
+        "workload": f"conv1d_k4_silu_bf16 B={w.B} S={w.T} C={C}",
+        "kernel_ms": round(kernel_ms, 4),
+        "tokens_per_s": round(w.B * w.T / (kernel_ms * 1e-3), 1),
+        "roofline": {"kernel": "causal_conv1d_kernel", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+    }  # fmt: skip
+
+
 def cpu_baseline(w, inp_gpu, target_seconds):
     """Naive recurrent torch restatement on this host's cores, on a bounded sample of the workload:
     whole sequences in order (all heads) until the time budget is used, or a prefix of the first
@@ -272,6 +308,7 @@ def main():
     w = get_workload(args.workload)
     result, inp = bench_chunk(w, args.steps, args.warmup)
     decode = None if args.no_decode else bench_decode(args.steps, args.warmup)
+    conv = None if args.no_decode else bench_conv(w, args.steps, args.warmup)
     baseline = None if args.no_cpu_baseline else cpu_baseline(w, inp, args.cpu_seconds)
     if args.calibrate_copy:
         calibrate_copy()
@@ -294,6 +331,7 @@ def main():
         "cpu_baseline": baseline,
         "step": result["step"],
         "decode": decode,
+        "conv": conv,
         "device": torch.cuda.get_device_name(0),
     }
     print(json.dumps(line))

@@ -123,6 +123,48 @@ int gdn_recurrent_fwd(const gdn_args *args, void *stream);
 #define GDN_CHUNK_KERNELS 3
 int gdn_chunk_fwd_profile(const gdn_args *args, void *stream, float *kernel_ms);
 
+/*
+ * Depthwise causal convolution over the token axis, the step right before the operator in the layer
+ * (q, k, v are slices of its output): replaces DepthwiseCausalConvolution.forward,
+ * lm_engine/modeling_utils/depthwise_causal_convolution.py:103-241, in all three of its modes
+ * (fresh prefill :157-197, one-token update :199-231, multi-token continuation :232-246), i.e. the
+ * causal_conv1d_fn / causal_conv1d_update calls and their torch restatements there.
+ *
+ *   y[b, s, c] = act(bias[c] + sum_j weight[c, j] * xx[b, s - (kernel_size - 1) + j, c]) * mask[b, s]
+ *   xx = input_state (positions -(kernel_size-1) .. -1, zeros when NULL) followed by x * mask
+ *   final_state[b, c, :] = the last kernel_size - 1 positions of xx        (:53-64)
+ *
+ *   x, y          [B, S, C]  element strides *_stride_b, *_stride_s, channels contiguous; y must not overlap x
+ *   weight        [C, kernel_size] contiguous in w_dtype (nn.Conv1d's [C, 1, kernel_size])
+ *   bias          [C] in w_dtype, or NULL
+ *   input_state   [B, C, kernel_size - 1] contiguous in dtype, or NULL
+ *   mask          [B, S] contiguous in dtype, or NULL  (the reference's 0/1 padding mask, :28-37)
+ *   final_state   [B, C, kernel_size - 1] contiguous in dtype, or NULL (not written)
+ *
+ * kernel_size 2..4, C a multiple of 8 (bf16) or 4 (fp32), rows, weight and bias 16-byte aligned;
+ * w_dtype equals dtype or is fp32.
+ */
+typedef enum gdn_activation { GDN_ACT_NONE = 0, GDN_ACT_SILU = 1 } gdn_activation;
+
+typedef struct gdn_conv_args {
+    const void *x;
+    const void *weight;
+    const void *bias;
+    const void *input_state;
+    const void *mask;
+    void *y;
+    void *final_state;
+    int64_t x_stride_b, x_stride_s;
+    int64_t y_stride_b, y_stride_s;
+    int32_t B, S, C, kernel_size;
+    int32_t dtype;      /* gdn_dtype of x, y, input_state, final_state, mask */
+    int32_t w_dtype;    /* gdn_dtype of weight and bias */
+    int32_t activation; /* gdn_activation */
+    int32_t reserved;
+} gdn_conv_args;
+
+int gdn_causal_conv1d_fwd(const gdn_conv_args *args, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,6 +1,7 @@
 """MI355X-native gated delta-rule sequence mixer: the operator lm-engine's GatedDeltaNet layer
 calls, as hand-written gfx950 HIP kernels behind a C-ABI library."""
 
+from .conv import depthwise_causal_convolution
 from .fla_shim import install_as_fla, uninstall_fla_shim
 from .kernels import Kernel, enable_all_kernels, enable_kernels, is_kernel_allowed
 from .ops import chunk_gated_delta_rule, fused_recurrent_gated_delta_rule, gated_delta_rule
@@ -9,6 +10,7 @@ from .ops import chunk_gated_delta_rule, fused_recurrent_gated_delta_rule, gated
 __all__ = [
     "Kernel",
     "chunk_gated_delta_rule",
+    "depthwise_causal_convolution",
     "enable_all_kernels",
     "enable_kernels",
     "fused_recurrent_gated_delta_rule",

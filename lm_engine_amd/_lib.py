@@ -18,6 +18,9 @@ GDN_F32 = 1
 GDN_FLAG_L2NORM = 1
 GDN_FLAG_STATE_INPLACE = 2
 
+GDN_ACT_NONE = 0
+GDN_ACT_SILU = 1
+
 LIBRARY_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libgdn_hip.so")
 
 EXPORTED_SYMBOLS = (
@@ -27,6 +30,7 @@ EXPORTED_SYMBOLS = (
     "gdn_chunk_fwd",
     "gdn_recurrent_fwd",
     "gdn_chunk_fwd_profile",
+    "gdn_causal_conv1d_fwd",
 )
 
 GDN_CHUNK_KERNELS = 3
@@ -46,6 +50,16 @@ class GdnArgs(ctypes.Structure):
         ]
         + [(name, ctypes.c_int32) for name in ("B", "T", "H", "K", "V", "N", "chunk", "dtype", "beta_dtype", "flags")]
         + [("scale", ctypes.c_float), ("reserved", ctypes.c_int32)]
+    )
+
+
+class GdnConvArgs(ctypes.Structure):
+    """Mirror of ``struct gdn_conv_args``."""
+
+    _fields_ = (
+        [(name, ctypes.c_void_p) for name in ("x", "weight", "bias", "input_state", "mask", "y", "final_state")]
+        + [(name, ctypes.c_int64) for name in ("x_stride_b", "x_stride_s", "y_stride_b", "y_stride_s")]
+        + [(name, ctypes.c_int32) for name in ("B", "S", "C", "kernel_size", "dtype", "w_dtype", "activation", "reserved")]
     )
 
 
@@ -83,6 +97,8 @@ def load_library() -> ctypes.CDLL:
     lib.gdn_recurrent_fwd.restype = ctypes.c_int
     lib.gdn_chunk_fwd_profile.argtypes = [ctypes.POINTER(GdnArgs), ctypes.c_void_p, ctypes.POINTER(ctypes.c_float)]
     lib.gdn_chunk_fwd_profile.restype = ctypes.c_int
+    lib.gdn_causal_conv1d_fwd.argtypes = [ctypes.POINTER(GdnConvArgs), ctypes.c_void_p]
+    lib.gdn_causal_conv1d_fwd.restype = ctypes.c_int
 
     version = lib.gdn_abi_version()
     if version != GDN_ABI_VERSION:

@@ -1,0 +1,111 @@
+"""Depthwise causal convolution with its carried state, the step in front of the gated delta rule.
+
+Functional form of the reference's ``DepthwiseCausalConvolution.forward``
+(lm_engine/modeling_utils/depthwise_causal_convolution.py:103-241): same arguments, same three
+modes (fresh prefill, one-token update, multi-token continuation), same return ``(y, final_state)``.
+It runs one HIP kernel (``gdn_causal_conv1d_fwd`` of libgdn_hip.so); there is no torch fallback.
+
+    x             [B, S, C]          bf16 or fp32, channels contiguous
+    weight        [C, 1, ks] or [C, ks]   nn.Conv1d's depthwise weight, ks in 2..4
+    bias          [C] or None
+    input_state   [B, C, ks - 1] or None   the last ks - 1 inputs of the previous call
+    attention_mask [B, S] or None    0/1 padding mask; applied to x and to y as the reference does
+                                     (only when B > 1 and S > 1, depthwise_causal_convolution.py:28-37)
+    returns  y [B, S, C], final_state [B, C, ks - 1] (None unless output_state)
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import _lib
+from .kernels import Kernel, is_kernel_allowed
+
+
+_IN_KERNEL_ACTIVATIONS = {None: _lib.GDN_ACT_NONE, "silu": _lib.GDN_ACT_SILU, "swish": _lib.GDN_ACT_SILU}
+
+
+def _dtype_code(dtype: torch.dtype, what: str) -> int:
+    if dtype == torch.bfloat16:
+        return _lib.GDN_BF16
+    if dtype == torch.float32:
+        return _lib.GDN_F32
+    raise ValueError(f"{what} must be bfloat16 or float32, got {dtype}")
+
+
+def depthwise_causal_convolution(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    bias: torch.Tensor | None = None,
+    input_state: torch.Tensor | None = None,
+    attention_mask: torch.Tensor | None = None,
+    output_state: bool = False,
+    activation: str | None = "silu",
+) -> tuple[torch.Tensor, torch.Tensor | None]:
+    if not is_kernel_allowed(Kernel.gated_delta_rule):
+        raise RuntimeError("Kernel.gated_delta_rule is disabled and this package ships no other implementation")
+    if activation not in _IN_KERNEL_ACTIVATIONS:
+        # the reference applies any other activation after the kernel (depthwise_causal_convolution.py:172-173)
+        raise ValueError(f"activation {activation!r} is not fused; pass activation=None and apply it to the result")
+    if x.dim() != 3:
+        raise ValueError("x must be [B, S, C]")
+    if not x.is_cuda:
+        raise ValueError("the convolution runs on the GPU only; x must be a device tensor")
+    B, S, C = x.shape
+    if weight.dim() == 3:
+        if weight.size(1) != 1:
+            raise ValueError("weight must be depthwise: [C, 1, kernel_size]")
+        weight = weight.squeeze(1)
+    if weight.dim() != 2 or weight.size(0) != C:
+        raise ValueError(f"weight must be [C, kernel_size] with C = {C}, got {tuple(weight.shape)}")
+    ks = weight.size(1)
+    if not 2 <= ks <= 4:
+        raise ValueError(f"kernel_size {ks} is not supported (2..4)")
+    if bias is not None and tuple(bias.shape) != (C,):
+        raise ValueError(f"bias must be [C] = {(C,)}, got {tuple(bias.shape)}")
+    if bias is not None and bias.dtype != weight.dtype:
+        raise ValueError("weight and bias must share a dtype")
+    if input_state is not None:
+        if tuple(input_state.shape) != (B, C, ks - 1):
+            raise ValueError(f"input_state must be [B, C, kernel_size - 1] = {(B, C, ks - 1)}, got {tuple(input_state.shape)}")
+        input_state = input_state.to(x.dtype).contiguous()
+    for name, t in (("weight", weight), ("bias", bias), ("input_state", input_state), ("attention_mask", attention_mask)):
+        if t is not None and t.device != x.device:
+            raise ValueError(f"{name} is on {t.device}, x is on {x.device}")
+
+    mask = None
+    if attention_mask is not None and attention_mask.shape[1] > 1 and attention_mask.shape[0] > 1:
+        if tuple(attention_mask.shape) != (B, S):
+            raise ValueError(f"attention_mask must be [B, S] = {(B, S)}, got {tuple(attention_mask.shape)}")
+        mask = attention_mask.to(x.dtype).contiguous()
+
+    if x.stride(-1) != 1:
+        x = x.contiguous()
+    if x.dtype == torch.float32 and weight.dtype != torch.float32:  # the kernel wants weights as wide as the data
+        weight = weight.float()
+        bias = None if bias is None else bias.float()
+    weight = weight.contiguous()
+    bias = None if bias is None else bias.contiguous()
+    y = torch.empty(B, S, C, dtype=x.dtype, device=x.device)
+    final_state = torch.empty(B, C, ks - 1, dtype=x.dtype, device=x.device) if output_state else None
+
+    a = _lib.GdnConvArgs()
+    a.x, a.weight, a.y = x.data_ptr(), weight.data_ptr(), y.data_ptr()
+    a.bias = None if bias is None else bias.data_ptr()
+    a.input_state = None if input_state is None else input_state.data_ptr()
+    a.mask = None if mask is None else mask.data_ptr()
+    a.final_state = None if final_state is None else final_state.data_ptr()
+    a.x_stride_b, a.x_stride_s = x.stride(0), x.stride(1)
+    a.y_stride_b, a.y_stride_s = y.stride(0), y.stride(1)
+    a.B, a.S, a.C, a.kernel_size = B, S, C, ks
+    a.dtype = _dtype_code(x.dtype, "x")
+    a.w_dtype = _dtype_code(weight.dtype, "weight")
+    a.activation = _IN_KERNEL_ACTIVATIONS[activation]
+
+    lib = _lib.load_library()
+    with torch.cuda.device(x.device):
+        stream = ctypes.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)
+        _lib.check_status(lib.gdn_causal_conv1d_fwd(ctypes.byref(a), stream), "gdn_causal_conv1d_fwd")
+    return y, final_state

@@ -24,7 +24,7 @@ HEADER = os.path.join(ROOT, "include", "gdn_hip.h")
 def _declared_functions() -> list[str]:
     text = open(HEADER).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return re.findall(r"\b(gdn_[a-z_]+)\s*\(", text)
+    return re.findall(r"\b(gdn_[a-z0-9_]+)\s*\(", text)
 
 
 def test_library_exports_every_declared_symbol():
@@ -45,6 +45,8 @@ def test_struct_layout_matches_the_header():
         printf("%zu %zu %zu %zu %zu %zu %zu\n", sizeof(gdn_args), offsetof(gdn_args, workspace_bytes),
                offsetof(gdn_args, q_stride_b), offsetof(gdn_args, o_stride_h), offsetof(gdn_args, B),
                offsetof(gdn_args, flags), offsetof(gdn_args, scale));
+        printf("%zu %zu %zu %zu %zu\n", sizeof(gdn_conv_args), offsetof(gdn_conv_args, final_state),
+               offsetof(gdn_conv_args, x_stride_b), offsetof(gdn_conv_args, B), offsetof(gdn_conv_args, activation));
         return 0;
     }
     """
@@ -54,8 +56,40 @@ def test_struct_layout_matches_the_header():
         subprocess.run(["gcc", f"-I{os.path.dirname(HEADER)}", src, "-o", exe], check=True)
         values = [int(x) for x in subprocess.run([exe], check=True, capture_output=True, text=True).stdout.split()]
     A = _lib.GdnArgs
+    Cv = _lib.GdnConvArgs
     assert values == [ctypes.sizeof(A), A.workspace_bytes.offset, A.q_stride_b.offset, A.o_stride_h.offset,
-                      A.B.offset, A.flags.offset, A.scale.offset]  # fmt: skip
+                      A.B.offset, A.flags.offset, A.scale.offset,
+                      ctypes.sizeof(Cv), Cv.final_state.offset, Cv.x_stride_b.offset, Cv.B.offset,
+                      Cv.activation.offset]  # fmt: skip
+
+
+def test_convolution_rejects_bad_arguments_before_any_launch():
+    lib = _lib.load_library()
+
+    def conv_args(**over):
+        a = _lib.GdnConvArgs()
+        a.x, a.y, a.weight = 0x1000, 0x2000, 0x3000  # never dereferenced
+        a.B, a.S, a.C, a.kernel_size = 2, 8, 16, 4
+        a.x_stride_s = a.y_stride_s = 16
+        a.x_stride_b = a.y_stride_b = 128
+        a.dtype, a.w_dtype, a.activation = _lib.GDN_BF16, _lib.GDN_BF16, _lib.GDN_ACT_SILU
+        for name, value in over.items():
+            setattr(a, name, value)
+        return a
+
+    for over, status in [
+        (dict(x=None), -1),
+        (dict(S=0), -2),
+        (dict(kernel_size=5), -3),
+        (dict(kernel_size=1), -3),
+        (dict(C=12), -3),
+        (dict(activation=7), -3),
+        (dict(x_stride_s=20), -4),
+        (dict(x=0x1008), -4),
+        (dict(y=0x1000), -2),
+        (dict(x_stride_s=8), -2),
+    ]:
+        assert lib.gdn_causal_conv1d_fwd(ctypes.byref(conv_args(**over)), None) == status, over
 
 
 def _args(**over):
