@@ -7,7 +7,7 @@
 //
 // A thread owns 16 bytes of channels (8 bf16 / 4 fp32) and walks TOKENS consecutive tokens with
 // the kernel_size - 1 previous rows in registers, so inside a block every row of x is read once;
-// neighbouring token blocks re-read kernel_size - 1 rows of halo (3 / 32 extra, served by L2).
+// neighbouring token blocks re-read kernel_size - 1 rows of halo (3 / 16 extra, served by L2).
 // Lanes cover consecutive channel vectors: every load and store of a wave is one contiguous row
 // segment.
 
@@ -16,7 +16,7 @@
 namespace gdn {
 
 constexpr int CONV_THREADS = 256;
-constexpr int CONV_TOKENS = 32;  // tokens per thread
+constexpr int CONV_TOKENS = 16;  // tokens per thread (measured: 16 beats 32, 64, 128; more workgroups in flight)
 
 struct ConvParams {
     const void* x;
