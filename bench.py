@@ -14,6 +14,7 @@ inputs already resident in HBM.  Prints ONE JSON line:
                updated in place) against the HBM peak, state buffers rotated so the state
                cannot live in the 256 MB Infinity Cache
   conv         the depthwise causal convolution in front of the operator, same batch, against the HBM peak
+  epilogue     rmsnorm(o * silu(gate)) behind the operator, same batch, against the HBM peak
   cpu_baseline the naive token-by-token torch restatement of the operator (oracle/), timed on
                this host's cores on a bounded prefix of the same workload
 """
@@ -58,7 +59,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", type=int, default=1, choices=(1, 2, 4))
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-decode", action="store_true", help="skip the decode and convolution legs")
+    ap.add_argument("--no-decode", action="store_true", help="skip the decode, convolution and epilogue legs")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target duration of the CPU baseline sample")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, the known-size kernel the HBM counters are scaled by")
@@ -211,6 +212,39 @@ def bench_conv(w, steps, warmup):
     }  # fmt: skip
 
 
+def bench_epilogue(w, steps, warmup):
+    """rmsnorm(o * silu(gate)) * weight over the operator's output of the same workload, gate read as a
+    slice of a wider projection.  HBM-bound: algorithmic bytes = o and gate in, y out."""
+    import torch
+
+    import lm_engine_amd
+
+    gen = torch.Generator("cpu").manual_seed(987)
+    o = torch.randn(w.B, w.T, w.H, w.V, generator=gen).to(torch.bfloat16).cuda()
+    proj = torch.randn(w.B, w.T, 2 * w.H + w.H * w.V, generator=gen).to(torch.bfloat16).cuda()
+    gate = proj[..., 2 * w.H:]
+    weight = torch.ones(w.V, dtype=torch.bfloat16, device="cuda")
+    call = lambda: lm_engine_amd.gated_rmsnorm(o, gate, weight, 1e-5)  # noqa: E731
+    for _ in range(warmup):
+        call()
+    torch.cuda.synchronize()
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for start, stop in events:
+        start.record()
+        call()
+        stop.record()
+    torch.cuda.synchronize()
+    kernel_ms = sum(start.elapsed_time(stop) for start, stop in events) / steps
+    nbytes = 3 * o.numel() * o.element_size()
+    gbs = nbytes / (kernel_ms * 1e-3) / 1e9
+    return {
+        "workload": f"gated_rmsnorm_bf16 B={w.B} T={w.T} H={w.H} V={w.V}",
+        "kernel_ms": round(kernel_ms, 4),
+        "roofline": {"kernel": "gated_rmsnorm_kernel", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+    }  # fmt: skip
+
+
 def cpu_baseline(w, inp_gpu, target_seconds):
     """Naive recurrent torch restatement on this host's cores, on a bounded sample of the workload:
     whole sequences in order (all heads) until the time budget is used, or a prefix of the first
@@ -309,6 +343,7 @@ def main():
     result, inp = bench_chunk(w, args.steps, args.warmup)
     decode = None if args.no_decode else bench_decode(args.steps, args.warmup)
     conv = None if args.no_decode else bench_conv(w, args.steps, args.warmup)
+    epilogue = None if args.no_decode else bench_epilogue(w, args.steps, args.warmup)
     baseline = None if args.no_cpu_baseline else cpu_baseline(w, inp, args.cpu_seconds)
     if args.calibrate_copy:
         calibrate_copy()
@@ -332,6 +367,7 @@ def main():
         "step": result["step"],
         "decode": decode,
         "conv": conv,
+        "epilogue": epilogue,
         "device": torch.cuda.get_device_name(0),
     }
     print(json.dumps(line))

@@ -165,6 +165,57 @@ typedef struct gdn_conv_args {
 
 int gdn_causal_conv1d_fwd(const gdn_conv_args *args, void *stream);
 
+/*
+ * The operator's scalar inputs from the layer's projections, one pass:
+ *   g    = -exp(A_log[h]) * softplus(a + dt_bias[h])     fp32   SoftplusDecayGate.forward with
+ *          final_exponential=False, lm_engine/modeling_utils/softplus_decay_gate/module.py:69-96
+ *   beta = beta_scale * sigmoid(b)                       dtype  gated_deltanet/module.py:179-181
+ *          (beta_scale 2 when allow_neg_eigval, else 1)
+ * a, b: [tokens, H] with element strides a_stride / b_stride between tokens (slices of one projection);
+ * A_log, dt_bias: [H] fp32; g: [tokens, H] fp32 contiguous; beta: [tokens, H] contiguous in dtype.
+ */
+typedef struct gdn_gate_args {
+    const void *a;
+    const void *b;
+    const float *A_log;
+    const float *dt_bias;
+    float *g;
+    void *beta;
+    int64_t a_stride, b_stride;
+    int64_t tokens;
+    int32_t H;
+    int32_t dtype; /* gdn_dtype of a, b, beta */
+    float beta_scale;
+    int32_t reserved;
+} gdn_gate_args;
+
+int gdn_gates_fwd(const gdn_gate_args *args, void *stream);
+
+/*
+ * What the layer does to the operator's output before the output projection, one pass:
+ *   y = rmsnorm(o * silu(gate)) * weight   over the V columns of every (token, head)
+ * gated_deltanet/module.py:238-242 (`o = o * silu(g)`, `o = self.o_norm(o)`), RMSNorm of
+ * lm_engine/modeling_utils/normalization.py:69-124: x / sqrt(mean(x^2) + eps) * weight.
+ * o, y: [tokens, H, V] with element strides *_stride_t between tokens; gate: same shape with
+ * gate_stride_t (a slice of a projection), or NULL (no gating); weight: [V] in w_dtype or NULL.
+ * V a multiple of 8, at most 512; 16-byte aligned rows.
+ */
+typedef struct gdn_norm_args {
+    const void *o;
+    const void *gate;
+    const void *weight;
+    void *y;
+    int64_t o_stride_t, gate_stride_t, y_stride_t;
+    int64_t tokens;
+    int32_t H, V;
+    int32_t dtype;   /* gdn_dtype of o, gate, y */
+    int32_t w_dtype; /* gdn_dtype of weight */
+    float eps;
+    int32_t reserved;
+} gdn_norm_args;
+
+int gdn_gated_rmsnorm_fwd(const gdn_norm_args *args, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

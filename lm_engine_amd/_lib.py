@@ -31,6 +31,8 @@ EXPORTED_SYMBOLS = (
     "gdn_recurrent_fwd",
     "gdn_chunk_fwd_profile",
     "gdn_causal_conv1d_fwd",
+    "gdn_gates_fwd",
+    "gdn_gated_rmsnorm_fwd",
 )
 
 GDN_CHUNK_KERNELS = 3
@@ -60,6 +62,27 @@ class GdnConvArgs(ctypes.Structure):
         [(name, ctypes.c_void_p) for name in ("x", "weight", "bias", "input_state", "mask", "y", "final_state")]
         + [(name, ctypes.c_int64) for name in ("x_stride_b", "x_stride_s", "y_stride_b", "y_stride_s")]
         + [(name, ctypes.c_int32) for name in ("B", "S", "C", "kernel_size", "dtype", "w_dtype", "activation", "reserved")]
+    )
+
+
+class GdnGateArgs(ctypes.Structure):
+    """Mirror of ``struct gdn_gate_args``."""
+
+    _fields_ = (
+        [(name, ctypes.c_void_p) for name in ("a", "b", "A_log", "dt_bias", "g", "beta")]
+        + [(name, ctypes.c_int64) for name in ("a_stride", "b_stride", "tokens")]
+        + [("H", ctypes.c_int32), ("dtype", ctypes.c_int32), ("beta_scale", ctypes.c_float), ("reserved", ctypes.c_int32)]
+    )
+
+
+class GdnNormArgs(ctypes.Structure):
+    """Mirror of ``struct gdn_norm_args``."""
+
+    _fields_ = (
+        [(name, ctypes.c_void_p) for name in ("o", "gate", "weight", "y")]
+        + [(name, ctypes.c_int64) for name in ("o_stride_t", "gate_stride_t", "y_stride_t", "tokens")]
+        + [(name, ctypes.c_int32) for name in ("H", "V", "dtype", "w_dtype")]
+        + [("eps", ctypes.c_float), ("reserved", ctypes.c_int32)]
     )
 
 
@@ -99,6 +122,10 @@ def load_library() -> ctypes.CDLL:
     lib.gdn_chunk_fwd_profile.restype = ctypes.c_int
     lib.gdn_causal_conv1d_fwd.argtypes = [ctypes.POINTER(GdnConvArgs), ctypes.c_void_p]
     lib.gdn_causal_conv1d_fwd.restype = ctypes.c_int
+    lib.gdn_gates_fwd.argtypes = [ctypes.POINTER(GdnGateArgs), ctypes.c_void_p]
+    lib.gdn_gates_fwd.restype = ctypes.c_int
+    lib.gdn_gated_rmsnorm_fwd.argtypes = [ctypes.POINTER(GdnNormArgs), ctypes.c_void_p]
+    lib.gdn_gated_rmsnorm_fwd.restype = ctypes.c_int
 
     version = lib.gdn_abi_version()
     if version != GDN_ABI_VERSION:

@@ -63,6 +63,28 @@ def test_struct_layout_matches_the_header():
                       Cv.activation.offset]  # fmt: skip
 
 
+def test_layer_ops_reject_bad_arguments_before_any_launch():
+    lib = _lib.load_library()
+    g = _lib.GdnGateArgs()
+    g.a = g.b = g.A_log = g.dt_bias = g.g = g.beta = 0x1000
+    g.tokens, g.H, g.a_stride, g.b_stride, g.dtype, g.beta_scale = 4, 8, 8, 8, _lib.GDN_BF16, 1.0
+    for over, status in [(dict(a=None), -1), (dict(tokens=0), -2), (dict(a_stride=4), -2), (dict(dtype=5), -3)]:
+        a = _lib.GdnGateArgs.from_buffer_copy(g)
+        for name, value in over.items():
+            setattr(a, name, value)
+        assert lib.gdn_gates_fwd(ctypes.byref(a), None) == status, over
+    n = _lib.GdnNormArgs()
+    n.o, n.y = 0x1000, 0x2000
+    n.tokens, n.H, n.V, n.dtype, n.w_dtype, n.eps = 4, 2, 64, _lib.GDN_BF16, _lib.GDN_F32, 1e-6
+    n.o_stride_t = n.y_stride_t = 128
+    for over, status in [(dict(o=None), -1), (dict(V=0), -2), (dict(V=20), -3), (dict(V=1024), -3), (dict(o_stride_t=64), -2),
+                         (dict(o=0x1002), -4), (dict(gate=0x3008, gate_stride_t=128), -4), (dict(o_stride_t=132), -4)]:  # fmt: skip
+        a = _lib.GdnNormArgs.from_buffer_copy(n)
+        for name, value in over.items():
+            setattr(a, name, value)
+        assert lib.gdn_gated_rmsnorm_fwd(ctypes.byref(a), None) == status, over
+
+
 def test_convolution_rejects_bad_arguments_before_any_launch():
     lib = _lib.load_library()
 
