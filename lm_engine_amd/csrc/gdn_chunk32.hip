@@ -666,12 +666,17 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
         // fragment f of the stage: f < SHARED_FRAGS comes from the head of the record, the rest from
         // this workgroup's slice of the U block
         const int lw = wave - NW;
+        // This wave moves fragments lw * NLOAD .. + NLOAD - 1 of the stage, starting `rot` into the block: the
+        // workgroups of a chain (one per column group) then ask for different lines at any one time, and a
+        // line's memory latency is paid by one of them instead of being waited out by all.
+        const int rot = (vgroup * ((NLOAD + 3) / 4)) % NLOAD;
+        auto frag_of = [&](int i) { return lw * NLOAD + (i + rot < NLOAD ? i + rot : i + rot - NLOAD); };
         const int64_t u_shift = (int64_t)p.off_u + (int64_t)vgroup * U_FRAGS * FRAG_BYTES - SHARED_BYTES;
         // two register buffers: while one record is written to LDS, younger ones are in flight
         bf16x8 buf0[NLOAD], buf1[NLOAD];
         float eg0 = 0.f, eg1 = 0.f;
         auto src_of = [&](int c, int i) {
-            const int f = lw * NLOAD + i;
+            const int f = frag_of(i);
             return rec + (int64_t)c * p.rec_bytes + (int64_t)f * FRAG_BYTES + (f >= SHARED_FRAGS ? u_shift : 0) + lane * 16;
         };
         auto load = [&](bf16x8(&buf)[NLOAD], float& eg, int c) {
@@ -684,11 +689,11 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
         auto store_and_reload = [&](bf16x8(&buf)[NLOAD], float& eg, int c, int c2, auto reload_tag) {
             constexpr bool reload = decltype(reload_tag)::value;
             uint8_t* dst = stage[c & 1];
-            bf16x8* d = reinterpret_cast<bf16x8*>(dst) + (lw * NLOAD) * WAVE + lane;
+            bf16x8* d = reinterpret_cast<bf16x8*>(dst) + lane;
             if (lw == 0 && lane == 0) *reinterpret_cast<float*>(dst + STAGE_FRAGS * FRAG_BYTES) = eg;
 #pragma unroll
             for (int i = 0; i < NLOAD; i++) {
-                d[i * WAVE] = buf[i];
+                d[frag_of(i) * WAVE] = buf[i];
                 if constexpr (reload) buf[i] = *reinterpret_cast<const bf16x8*>(src_of(c2, i));
                 __builtin_amdgcn_sched_barrier(0);
             }
