@@ -338,6 +338,10 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
 #pragma unroll
             for (int i = 0; i < 16; i++) sT[(16 * blk + i) * LDA + 16 * blk + j] = x[i];
             // transposes used as B operands below; zero blocks above the diagonal where a product reads them
+            if (blk == 0) {
+#pragma unroll
+                for (int i = 0; i < 16; i++) sT[i * LDA + 16 + j] = 0.f;  // T block (0, 1)
+            }
             if (blk < 2) {
 #pragma unroll
                 for (int c4 = 0; c4 < 4; c4++)
@@ -464,10 +468,9 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
             const f32x4 c1 = *reinterpret_cast<const f32x4*>(&colscale[j0 + 4]);
             bf16x8 r;
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const int ja = j0 + e, jb = j0 + 4 + e;
-                r[e] = (bf16_t)(ja < i ? t0[e] * c0[e] : (ja == i ? c0[e] : 0.f));
-                r[4 + e] = (bf16_t)(jb < i ? t1[e] * c1[e] : (jb == i ? c1[e] : 0.f));
+            for (int e = 0; e < 4; e++) {  // sT holds the whole of T here: unit diagonal, zeros above it
+                r[e] = (bf16_t)(t0[e] * c0[e]);
+                r[4 + e] = (bf16_t)(t1[e] * c1[e]);
             }
             return r;
         };
