@@ -104,6 +104,16 @@ def test_varlen_packed_sequences_match_and_equal_separate_runs():
         assert torch.equal(ht[n : n + 1], h_n)
 
 
+@pytest.mark.parametrize("K, V", [(128, 128), (64, 64), (256, 128)])
+def test_varlen_with_an_empty_sequence(K, V):
+    # a sequence of length 0 has no chunk: its final state is its initial state, and its neighbours are untouched
+    lengths = [70, 0, 129, 0]
+    inp = random_inputs(B=1, T=sum(lengths), H=2, K=K, V=V, dtype=BF16, seed=77, N=len(lengths))
+    cu = torch.tensor([0] + lengths).cumsum(0).to(torch.int32)
+    o, ht = _check(dict(inp, cu_seqlens=cu), f"varlen with empty sequences K={K} V={V}")
+    assert torch.equal(ht[1].cpu(), inp["initial_state"][1]) and torch.equal(ht[3].cpu(), inp["initial_state"][3])
+
+
 def test_strided_views_of_a_fused_projection():
     B, T, H, K, V = 2, 150, 2, 128, 128
     gen = torch.Generator().manual_seed(76)

@@ -70,6 +70,13 @@ def test_varlen_packed_sequences():
     _check(inp, torch.bfloat16)
 
 
+def test_varlen_with_empty_sequences():
+    lengths = [0, 9, 0, 30, 0]
+    inp = random_inputs(B=1, T=sum(lengths), H=2, K=64, V=64, dtype=torch.bfloat16, seed=44, N=len(lengths))
+    inp["cu_seqlens"] = torch.tensor([0] + lengths).cumsum(0).to(torch.int32)
+    _check(inp, torch.bfloat16)
+
+
 def test_strided_views_of_a_fused_projection():
     # q, k, v as the reference layer produces them: slices of one [B, T, 2 H K + H V] projection
     B, T, H, K, V = 2, 5, 2, 64, 128
