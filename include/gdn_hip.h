@@ -41,6 +41,7 @@ typedef enum gdn_status {
 enum {
     GDN_FLAG_L2NORM = 1,        /* normalise q and k rows in-kernel: x / sqrt(sum x^2 + 1e-6) */
     GDN_FLAG_STATE_INPLACE = 2, /* decode: ht == h0 is allowed and expected */
+    GDN_FLAG_LEFT_PADDED = 4,   /* cu_seqlens describes a left-padded batch, see gdn_args */
 };
 
 /*
@@ -53,7 +54,11 @@ enum {
  *   h0     [N, H, K, V] fp32 contiguous or NULL (zero state)
  *   ht     [N, H, K, V] fp32 contiguous or NULL (final state not written)
  *   cu_seqlens  int32 [N + 1] with a leading 0 (packed sequences, then B must be 1), or NULL
- *               (then N must equal B)
+ *               (then N must equal B).  With GDN_FLAG_LEFT_PADDED the batch stays [B, T, ...], N must
+ *               equal B, and cu_seqlens holds the prefix sums of the valid lengths: sequence b is the
+ *               last cu_seqlens[b+1] - cu_seqlens[b] tokens of row b (what the reference gets from
+ *               compute_cu_seqlens_and_max_seqlen_from_attention_mask, sequence_packing.py:18-22, and
+ *               then packs and unpacks around the operator, :25-93); o is written at valid tokens only.
  *
  * Replaces the argument list of both fla calls at gated_deltanet/module.py:198-222.
  */

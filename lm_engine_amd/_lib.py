@@ -17,6 +17,7 @@ GDN_F32 = 1
 
 GDN_FLAG_L2NORM = 1
 GDN_FLAG_STATE_INPLACE = 2
+GDN_FLAG_LEFT_PADDED = 4
 
 GDN_ACT_NONE = 0
 GDN_ACT_SILU = 1

@@ -15,11 +15,12 @@ int validate_common(const gdn_args* a) {
     if (a == nullptr) return GDN_ERR_NULL;
     if (!a->q || !a->k || !a->v || !a->o) return GDN_ERR_NULL;
     if (a->B <= 0 || a->T <= 0 || a->H <= 0 || a->K <= 0 || a->V <= 0 || a->N <= 0) return GDN_ERR_SHAPE;
-    if (a->cu_seqlens != nullptr) {
+    if (a->cu_seqlens != nullptr && !(a->flags & GDN_FLAG_LEFT_PADDED)) {
         if (a->B != 1) return GDN_ERR_VARLEN;
     } else if (a->N != a->B) {
         return GDN_ERR_SHAPE;
     }
+    if ((a->flags & GDN_FLAG_LEFT_PADDED) && a->cu_seqlens == nullptr) return GDN_ERR_NULL;
     if (a->H > 65535 || a->N > 65535) return GDN_ERR_UNSUPPORTED;
     if (a->dtype != GDN_BF16 && a->dtype != GDN_F32) return GDN_ERR_UNSUPPORTED;
     if (a->beta && a->beta_dtype != GDN_BF16 && a->beta_dtype != GDN_F32) return GDN_ERR_UNSUPPORTED;
@@ -59,7 +60,7 @@ const char* gdn_strerror(int status) {
                    "bf16, chunk 64)";
         case GDN_ERR_ALIGN: return "pointer or stride not 16-byte aligned";
         case GDN_ERR_WORKSPACE: return "workspace missing or too small";
-        case GDN_ERR_VARLEN: return "cu_seqlens requires B == 1";
+        case GDN_ERR_VARLEN: return "cu_seqlens requires B == 1 (packed) or GDN_FLAG_LEFT_PADDED";
         default: break;
     }
     if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));
@@ -107,7 +108,7 @@ int gdn_chunk_fwd_profile(const gdn_args* a, void* stream, float* kernel_ms) {
     if (rc == GDN_OK) rc = (int)hipEventSynchronize(events[GDN_CHUNK_KERNELS]);
     for (int i = 0; rc == GDN_OK && i < GDN_CHUNK_KERNELS; i++) {
         kernel_ms[i] = 0.f;
-        if (i == 0 && a->cu_seqlens == nullptr) continue;
+        if (i == 0 && (a->cu_seqlens == nullptr || (a->flags & GDN_FLAG_LEFT_PADDED))) continue;
         rc = (int)hipEventElapsedTime(&kernel_ms[i], events[i], events[i + 1]);
     }
     for (int i = 0; i < created; i++) (void)hipEventDestroy(events[i]);

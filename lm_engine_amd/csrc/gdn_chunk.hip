@@ -47,7 +47,8 @@ namespace gdn {
 
 static int chunk_slots(const gdn_args& a) {
     const int nt = (a.T + C - 1) / C;
-    return a.cu_seqlens ? a.T / C + a.N : a.B * nt;
+    const bool packed = a.cu_seqlens != nullptr && !(a.flags & GDN_FLAG_LEFT_PADDED);
+    return packed ? a.T / C + a.N : a.B * nt;
 }
 
 static uint64_t chunk_off_bytes(const gdn_args& a) { return (((uint64_t)a.N + 1) * 4 + 255u) & ~(uint64_t)255u; }
@@ -458,8 +459,9 @@ __global__ __launch_bounds__(NW* WAVE) void chunk_scan_kernel(const ChunkParams 
     int slot_begin, slot_end;
     int64_t b, seq_t0, seq_len;
     if (p.cu_seqlens == nullptr) {
-        slot_begin = n * p.NT, slot_end = slot_begin + p.NT;
-        b = n, seq_t0 = 0, seq_len = p.T;
+        seq_len = p.pad_lens == nullptr ? p.T : min(max(p.pad_lens[n + 1] - p.pad_lens[n], 0), p.T);  // the last seq_len tokens of row n
+        slot_begin = n * p.NT, slot_end = slot_begin + (int)((seq_len + C - 1) / C);
+        b = n, seq_t0 = p.T - seq_len;
     } else {
         slot_begin = p.chunk_off[n], slot_end = p.chunk_off[n + 1];
         b = 0, seq_t0 = p.cu_seqlens[n], seq_len = p.cu_seqlens[n + 1] - seq_t0;
@@ -603,7 +605,9 @@ int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events) 
     p.h0 = a.h0;
     p.ht = a.ht;
     p.o = static_cast<bf16_t*>(a.o);
-    p.cu_seqlens = a.cu_seqlens;
+    const bool left_padded = (a.flags & GDN_FLAG_LEFT_PADDED) != 0;
+    p.cu_seqlens = left_padded ? nullptr : a.cu_seqlens;
+    p.pad_lens = left_padded ? a.cu_seqlens : nullptr;
     p.chunk_off = static_cast<int32_t*>(a.workspace);
     p.rec = static_cast<uint8_t*>(a.workspace) + chunk_off_bytes(a);
     p.q_stride_b = a.q_stride_b, p.q_stride_t = a.q_stride_t, p.q_stride_h = a.q_stride_h;

@@ -619,8 +619,9 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
     int slot_begin, slot_end;
     int64_t b, seq_t0, seq_len;
     if (p.cu_seqlens == nullptr) {
-        slot_begin = n * p.NT, slot_end = slot_begin + p.NT;
-        b = n, seq_t0 = 0, seq_len = p.T;
+        seq_len = p.pad_lens == nullptr ? p.T : min(max(p.pad_lens[n + 1] - p.pad_lens[n], 0), p.T);  // the last seq_len tokens of row n
+        slot_begin = n * p.NT, slot_end = slot_begin + (int)((seq_len + C - 1) / C);
+        b = n, seq_t0 = p.T - seq_len;
     } else {
         slot_begin = p.chunk_off[n], slot_end = p.chunk_off[n + 1];
         b = 0, seq_t0 = p.cu_seqlens[n], seq_len = p.cu_seqlens[n + 1] - seq_t0;

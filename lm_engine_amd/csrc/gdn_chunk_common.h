@@ -18,7 +18,8 @@ struct ChunkParams {
     const float* h0;
     float* ht;
     bf16_t* o;
-    const int32_t* cu_seqlens;
+    const int32_t* cu_seqlens;  // packed sequences (B == 1), else NULL
+    const int32_t* pad_lens;    // left-padded batch: prefix sums of the valid lengths, else NULL
     int32_t* chunk_off;  // [N + 1] prefix of chunks per sequence (packed input only)
     uint8_t* rec;        // workspace records, [H][TC]
     int64_t q_stride_b, q_stride_t, q_stride_h;
@@ -67,8 +68,10 @@ __device__ __forceinline__ ChunkCoord locate_chunk(const ChunkParams& p, int slo
         cc.n = slot / p.NT;
         const int c = slot - cc.n * p.NT;
         cc.b = cc.n;
-        cc.t0 = (int64_t)c * C;
-        cc.len = min(C, p.T - c * C);
+        // the last `len` tokens of the row (clamped: a malformed prefix must not send a load out of the row)
+        const int len = p.pad_lens == nullptr ? p.T : min(max(p.pad_lens[cc.n + 1] - p.pad_lens[cc.n], 0), p.T);
+        cc.t0 = (int64_t)(p.T - len) + (int64_t)c * C;
+        cc.len = min(C, len - c * C);
         return cc;
     }
     cc.b = 0;

@@ -33,6 +33,7 @@ struct RecurrentParams {
     float* ht;
     void* o;
     const int32_t* cu_seqlens;
+    const int32_t* pad_lens;  // left-padded batch: prefix sums of the valid lengths
     int64_t q_stride_b, q_stride_t, q_stride_h;
     int64_t k_stride_b, k_stride_t, k_stride_h;
     int64_t v_stride_b, v_stride_t, v_stride_h;
@@ -67,6 +68,7 @@ __global__ __launch_bounds__(REC_THREADS) void recurrent_kernel(const RecurrentP
     const int n = blockIdx.z;
 
     int64_t b = n, t_begin = 0, t_end = p.T;
+    if (p.pad_lens != nullptr) t_begin = p.T - min(max(p.pad_lens[n + 1] - p.pad_lens[n], 0), p.T);  // the last tokens of row n
     if (p.cu_seqlens != nullptr) {
         b = 0;
         t_begin = p.cu_seqlens[n];
@@ -207,7 +209,8 @@ int launch_recurrent(const gdn_args& a, hipStream_t stream) {
     p.h0 = a.h0;
     p.ht = a.ht;
     p.o = a.o;
-    p.cu_seqlens = a.cu_seqlens;
+    p.cu_seqlens = (a.flags & GDN_FLAG_LEFT_PADDED) ? nullptr : a.cu_seqlens;
+    p.pad_lens = (a.flags & GDN_FLAG_LEFT_PADDED) ? a.cu_seqlens : nullptr;
     p.q_stride_b = a.q_stride_b, p.q_stride_t = a.q_stride_t, p.q_stride_h = a.q_stride_h;
     p.k_stride_b = a.k_stride_b, p.k_stride_t = a.k_stride_t, p.k_stride_h = a.k_stride_h;
     p.v_stride_b = a.v_stride_b, p.v_stride_t = a.v_stride_t, p.v_stride_h = a.v_stride_h;

@@ -57,7 +57,7 @@ def _last_dim_contiguous(x: torch.Tensor) -> torch.Tensor:
     return x if x.stride(-1) == 1 else x.contiguous()
 
 
-def _check_inputs(q, k, v, g, beta, initial_state, cu_seqlens):
+def _check_inputs(q, k, v, g, beta, initial_state, cu_seqlens, left_padded=False):
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
         raise ValueError("q, k, v must be [B, T, H, D] tensors")
     B, T, H, K = q.shape
@@ -81,7 +81,11 @@ def _check_inputs(q, k, v, g, beta, initial_state, cu_seqlens):
     for name, x in (("g", g), ("beta", beta)):
         if x is not None and tuple(x.shape) != (B, T, H):
             raise ValueError(f"{name} must be [B, T, H] = {(B, T, H)}, got {tuple(x.shape)}")
-    if cu_seqlens is not None:
+    if left_padded:
+        if cu_seqlens is None or cu_seqlens.dim() != 1 or cu_seqlens.numel() != B + 1:
+            raise ValueError(f"left_padded needs cu_seqlens [B + 1] = [{B + 1}]: the prefix sums of the valid lengths")
+        N = B
+    elif cu_seqlens is not None:
         if B != 1:
             raise ValueError(f"with cu_seqlens the batch dim must be 1 (tokens packed along T), got B={B}")
         if cu_seqlens.dim() != 1 or cu_seqlens.numel() < 2:
@@ -97,7 +101,7 @@ def _check_inputs(q, k, v, g, beta, initial_state, cu_seqlens):
     return B, T, H, K, V, N
 
 
-def _fill_args(q, k, v, g, beta, h0, ht, o, cu_seqlens, scale, l2norm, inplace, dims) -> _lib.GdnArgs:
+def _fill_args(q, k, v, g, beta, h0, ht, o, cu_seqlens, scale, l2norm, inplace, dims, left_padded=False) -> _lib.GdnArgs:
     B, T, H, K, V, N = dims
     a = _lib.GdnArgs()
     a.q, a.k, a.v, a.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr()
@@ -115,15 +119,17 @@ def _fill_args(q, k, v, g, beta, h0, ht, o, cu_seqlens, scale, l2norm, inplace, 
     a.chunk = 64
     a.dtype = _dtype_code(q.dtype, "q, k, v")
     a.beta_dtype = _lib.GDN_F32 if beta is None else _dtype_code(beta.dtype, "beta")
-    a.flags = (_lib.GDN_FLAG_L2NORM if l2norm else 0) | (_lib.GDN_FLAG_STATE_INPLACE if inplace else 0)
+    a.flags = ((_lib.GDN_FLAG_L2NORM if l2norm else 0) | (_lib.GDN_FLAG_STATE_INPLACE if inplace else 0)
+               | (_lib.GDN_FLAG_LEFT_PADDED if left_padded else 0))  # fmt: skip
     a.scale = float(K**-0.5 if scale is None else scale)
     return a
 
 
-def _run(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm, inplace_state):
+def _run(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm, inplace_state,
+         left_padded=False):
     _require_hip_path()
     lib = _lib.load_library()
-    dims = _check_inputs(q, k, v, g, beta, initial_state, cu_seqlens)
+    dims = _check_inputs(q, k, v, g, beta, initial_state, cu_seqlens, left_padded)
     B, T, H, K, V, N = dims
 
     q, k, v = _last_dim_contiguous(q), _last_dim_contiguous(k), _last_dim_contiguous(v)
@@ -135,7 +141,8 @@ def _run(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_se
         cu_seqlens = cu_seqlens.to(torch.int32).contiguous()
     h0 = None if initial_state is None else initial_state.contiguous()
 
-    o = torch.empty(B, T, H, V, dtype=v.dtype, device=v.device)
+    # padding positions of a left-padded batch are not written by the kernels: they read as zeros
+    o = (torch.zeros if left_padded else torch.empty)(B, T, H, V, dtype=v.dtype, device=v.device)
     ht = None
     if output_final_state:
         if inplace_state:
@@ -145,7 +152,8 @@ def _run(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_se
         else:
             ht = torch.empty(N, H, K, V, dtype=torch.float32, device=v.device)
 
-    args = _fill_args(q, k, v, g, beta, h0, ht, o, cu_seqlens, scale, l2norm, inplace_state and ht is not None, dims)
+    args = _fill_args(q, k, v, g, beta, h0, ht, o, cu_seqlens, scale, l2norm, inplace_state and ht is not None, dims,
+                      left_padded)  # fmt: skip
     stream = ctypes.c_void_p(torch.cuda.current_stream(q.device).cuda_stream)
 
     with torch.cuda.device(q.device):
@@ -192,10 +200,10 @@ class _ForwardOnly(torch.autograd.Function):
     """The operator has no backward yet; differentiating through it must fail, not pass silently."""
 
     @staticmethod
-    def forward(ctx, mode, scale, output_final_state, l2norm, inplace_state, q, k, v, g, beta, initial_state,
-                cu_seqlens):  # fmt: skip
+    def forward(ctx, mode, scale, output_final_state, l2norm, inplace_state, left_padded, q, k, v, g, beta,
+                initial_state, cu_seqlens):  # fmt: skip
         o, ht = _run(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm,
-                     inplace_state)  # fmt: skip
+                     inplace_state, left_padded)  # fmt: skip
         return o, ht
 
     @staticmethod
@@ -203,12 +211,14 @@ class _ForwardOnly(torch.autograd.Function):
         raise NotImplementedError("the HIP gated delta rule is forward-only; its backward is not implemented")
 
 
-def _dispatch(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm, inplace_state):
+def _dispatch(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm, inplace_state,
+              left_padded=False):
     tensors = (q, k, v, g, beta, initial_state)
     if torch.is_grad_enabled() and any(x is not None and x.requires_grad for x in tensors):
-        return _ForwardOnly.apply(mode, scale, output_final_state, l2norm, inplace_state, q, k, v, g, beta,
-                                  initial_state, cu_seqlens)  # fmt: skip
-    return _run(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm, inplace_state)
+        return _ForwardOnly.apply(mode, scale, output_final_state, l2norm, inplace_state, left_padded, q, k, v, g,
+                                  beta, initial_state, cu_seqlens)  # fmt: skip
+    return _run(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm, inplace_state,
+                left_padded)  # fmt: skip
 
 
 def chunk_gated_delta_rule(
@@ -223,16 +233,23 @@ def chunk_gated_delta_rule(
     cu_seqlens: torch.Tensor | None = None,
     head_first: bool = False,
     use_qk_l2norm_in_kernel: bool = False,
+    left_padded: bool = False,
 ) -> tuple[torch.Tensor, torch.Tensor | None]:
     """Chunked (chunk = 64) forward; drop-in for the call at gated_deltanet/module.py:197-209.
 
     bf16 inputs run the MFMA chunk kernels.  fp32 inputs are computed exactly, token by token,
-    by the recurrent kernel (the chunk kernels round their matrix operands to bf16)."""
+    by the recurrent kernel (the chunk kernels round their matrix operands to bf16).
+
+    ``left_padded=True`` (not an fla argument) keeps a padded batch ``[B, T, ...]`` as it is: ``cu_seqlens``
+    ``[B + 1]`` then holds the prefix sums of the valid lengths and sequence b is the last
+    ``cu_seqlens[b+1] - cu_seqlens[b]`` tokens of row b - what the reference derives from its attention mask
+    (sequence_packing.py:18-22) before it packs and unpacks around the operator (:25-93).  The kernels skip
+    the padding; ``o`` is zero there, as after the reference's unpack."""
     if head_first:
         raise ValueError("head_first layouts are not supported; pass [B, T, H, D] tensors")
     mode = "chunk" if q.dtype == torch.bfloat16 else "recurrent"
     return _dispatch(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens,
-                     use_qk_l2norm_in_kernel, False)  # fmt: skip
+                     use_qk_l2norm_in_kernel, False, left_padded)  # fmt: skip
 
 
 def fused_recurrent_gated_delta_rule(
@@ -247,15 +264,17 @@ def fused_recurrent_gated_delta_rule(
     cu_seqlens: torch.Tensor | None = None,
     use_qk_l2norm_in_kernel: bool = False,
     inplace_state: bool = False,
+    left_padded: bool = False,
 ) -> tuple[torch.Tensor, torch.Tensor | None]:
     """Token-by-token forward; drop-in for the call at gated_deltanet/module.py:210-222.
 
     With ``inplace_state=True`` (and ``output_final_state=True``) the final state overwrites
     ``initial_state`` and that same tensor is returned: one read and one write of the state per
     decode step instead of a fresh allocation.  The reference's cache replaces its tensor with
-    whatever is returned (lm_engine/generation_cache/constant.py:17-23), so both modes fit it."""
+    whatever is returned (lm_engine/generation_cache/constant.py:17-23), so both modes fit it.
+    ``left_padded``: as in ``chunk_gated_delta_rule``."""
     return _dispatch("recurrent", q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens,
-                     use_qk_l2norm_in_kernel, inplace_state)  # fmt: skip
+                     use_qk_l2norm_in_kernel, inplace_state, left_padded)  # fmt: skip
 
 
 def gated_delta_rule(

@@ -114,6 +114,33 @@ def test_varlen_with_an_empty_sequence(K, V):
     assert torch.equal(ht[1].cpu(), inp["initial_state"][1]) and torch.equal(ht[3].cpu(), inp["initial_state"][3])
 
 
+@pytest.mark.parametrize("K, V", [(128, 128), (256, 128)])
+def test_left_padded_batch_equals_separate_runs(K, V):
+    # [B, T] batch whose rows are padded on the left; cu_seqlens = prefix sums of the valid lengths
+    B, T, H = 4, 200, 2
+    lengths = [200, 37, 0, 129]
+    inp = random_inputs(B=B, T=T, H=H, K=K, V=V, dtype=BF16, seed=78)
+    gpu = _to_gpu(inp)
+    cu = torch.tensor([0] + lengths).cumsum(0).to(torch.int32).cuda()
+    print(f"case: chunk left-padded lengths {lengths} K={K} V={V}", flush=True)
+    o, ht = lm_engine_amd.chunk_gated_delta_rule(**gpu, cu_seqlens=cu, output_final_state=True, left_padded=True)
+    for b, n in enumerate(lengths):
+        assert torch.all(o[b, : T - n] == 0), f"row {b}: padding must read as zeros"
+        if n == 0:
+            assert torch.equal(ht[b], gpu["initial_state"][b])
+            continue
+        one = {name: x[b : b + 1, T - n :] for name, x in gpu.items() if name != "initial_state"}
+        fn = lm_engine_amd.chunk_gated_delta_rule if n > 64 else lm_engine_amd.fused_recurrent_gated_delta_rule
+        o_b, h_b = lm_engine_amd.chunk_gated_delta_rule(**one, initial_state=gpu["initial_state"][b : b + 1], output_final_state=True)
+        assert torch.equal(o[b : b + 1, T - n :], o_b), f"row {b}: padded-batch and separate outputs differ"
+        assert torch.equal(ht[b : b + 1], h_b)
+        # and against the oracle on the valid tokens
+        cpu = {name: x[b : b + 1, T - n :] for name, x in inp.items() if name != "initial_state"}
+        o_ref, h_ref = recurrent_gated_delta_rule_c(**cpu, initial_state=inp["initial_state"][b : b + 1], output_final_state=True)
+        assert_parity(o_b.float(), o_ref, BF16, "o")
+        assert_parity(h_b, h_ref, BF16, "final_state")
+
+
 def test_strided_views_of_a_fused_projection():
     B, T, H, K, V = 2, 150, 2, 128, 128
     gen = torch.Generator().manual_seed(76)

@@ -141,6 +141,8 @@ def _args(**over):
         (dict(q_stride_t=129), -4),
         (dict(v=0x1004), -4),
         (dict(cu_seqlens=0x2000, B=2, N=2), -6),
+        (dict(flags=_lib.GDN_FLAG_LEFT_PADDED), -1),  # left-padded needs the prefix sums
+        (dict(flags=_lib.GDN_FLAG_LEFT_PADDED, cu_seqlens=0x2000, B=2, N=3), -2),  # one sequence per row
         (dict(q_stride_h=32), -2),
     ],
 )

@@ -77,6 +77,24 @@ def test_varlen_with_empty_sequences():
     _check(inp, torch.bfloat16)
 
 
+def test_left_padded_batch_equals_separate_runs():
+    B, T, H = 3, 20, 2
+    lengths = [20, 0, 7]
+    inp = random_inputs(B=B, T=T, H=H, K=64, V=64, dtype=torch.bfloat16, seed=45)
+    gpu = {n: x.cuda() for n, x in inp.items()}
+    cu = torch.tensor([0] + lengths).cumsum(0).to(torch.int32).cuda()
+    o, ht = lm_engine_amd.fused_recurrent_gated_delta_rule(**gpu, cu_seqlens=cu, output_final_state=True, left_padded=True)
+    for b, n in enumerate(lengths):
+        assert torch.all(o[b, : T - n] == 0)
+        if n == 0:
+            assert torch.equal(ht[b], gpu["initial_state"][b])
+            continue
+        one = {name: x[b : b + 1, T - n :] for name, x in gpu.items() if name != "initial_state"}
+        o_b, h_b = lm_engine_amd.fused_recurrent_gated_delta_rule(**one, initial_state=gpu["initial_state"][b : b + 1],
+                                                                  output_final_state=True)  # fmt: skip
+        assert torch.equal(o[b : b + 1, T - n :], o_b) and torch.equal(ht[b : b + 1], h_b)
+
+
 def test_strided_views_of_a_fused_projection():
     # q, k, v as the reference layer produces them: slices of one [B, T, 2 H K + H V] projection
     B, T, H, K, V = 2, 5, 2, 64, 128
