@@ -44,6 +44,8 @@ MEASURED_HBM_TRAFFIC_BYTES = {
     ("cfg1_chunk_fwd_bf16", "chunk_prepare"): (2.0 * 104712.5 + 295041.7) * _KIB,
     ("cfg1_chunk_fwd_bf16", "chunk_scan"): (2.0 * 147853.4 + 69632.6) * _KIB,
     ("cfg3_decode_bf16", "recurrent_kernel"): (2.0 * 265449.7 + 526881.4) * _KIB,
+    ("cfg1_chunk_fwd_bf16", "causal_conv1d_kernel"): (2.0 * 117467.1 + 196752.0) * _KIB,
+    ("cfg1_chunk_fwd_bf16", "gated_rmsnorm_kernel"): (2.0 * 66081.4 + 65536.0) * _KIB,
 }
 
 
@@ -208,7 +210,8 @@ def bench_conv(w, steps, warmup):
         "kernel_ms": round(kernel_ms, 4),
         "tokens_per_s": round(w.B * w.T / (kernel_ms * 1e-3), 1),
         "roofline": {"kernel": "causal_conv1d_kernel", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": measured_traffic(w.name, "causal_conv1d_kernel")},
     }  # fmt: skip
 
 
@@ -241,7 +244,8 @@ def bench_epilogue(w, steps, warmup):
         "workload": f"gated_rmsnorm_bf16 B={w.B} T={w.T} H={w.H} V={w.V}",
         "kernel_ms": round(kernel_ms, 4),
         "roofline": {"kernel": "gated_rmsnorm_kernel", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": measured_traffic(w.name, "gated_rmsnorm_kernel")},
     }  # fmt: skip
 
 
