@@ -7,9 +7,9 @@
 //
 // A thread owns 16 bytes of channels (8 bf16 / 4 fp32) and walks TOKENS consecutive tokens with
 // the kernel_size - 1 previous rows in registers, so inside a block every row of x is read once;
-// neighbouring token blocks re-read kernel_size - 1 rows of halo (3 / 16 extra, served by L2).
-// Lanes cover consecutive channel vectors: every load and store of a wave is one contiguous row
-// segment.
+// neighbouring token blocks re-read kernel_size - 1 rows of halo.  Lanes cover consecutive channel
+// vectors: every load and store of a wave is one contiguous row segment; the four waves of a
+// workgroup take consecutive token blocks of the same channels.
 
 #include "gdn_common.h"
 
@@ -63,10 +63,13 @@ __global__ __launch_bounds__(CONV_THREADS) void causal_conv1d_kernel(const ConvP
     constexpr int VEC = ConvVec<T>::N;
     typedef typename ConvVec<T>::type vec_t;
 
-    const int c0 = (blockIdx.x * CONV_THREADS + threadIdx.x) * VEC;
+    // a workgroup covers 64 channel vectors x (4 waves x CONV_TOKENS tokens): the halo rows of a wave are the
+    // last rows of the wave before it, read on the same CU at about the same time
+    const int c0 = (blockIdx.x * WAVE + threadIdx.x % WAVE) * VEC;
     if (c0 >= p.C) return;
     const int b = blockIdx.z;
-    const int s_begin = blockIdx.y * CONV_TOKENS;
+    const int s_begin = (blockIdx.y * (CONV_THREADS / WAVE) + threadIdx.x / WAVE) * CONV_TOKENS;
+    if (s_begin >= p.S) return;
     const int s_end = min(s_begin + CONV_TOKENS, p.S);
 
     const T* xb = reinterpret_cast<const T*>(p.x) + (int64_t)b * p.x_stride_b + c0;
@@ -143,7 +146,8 @@ static void launch_conv_ks(const ConvParams& p, bool silu, dim3 grid, hipStream_
 template <typename T, typename WT>
 static int launch_conv(const ConvParams& p, int kernel_size, bool silu, hipStream_t stream) {
     const int vecs = p.C / ConvVec<T>::N;
-    const dim3 grid((vecs + CONV_THREADS - 1) / CONV_THREADS, (p.S + CONV_TOKENS - 1) / CONV_TOKENS, p.B);
+    constexpr int SPAN = (CONV_THREADS / WAVE) * CONV_TOKENS;  // tokens per workgroup
+    const dim3 grid((vecs + WAVE - 1) / WAVE, (p.S + SPAN - 1) / SPAN, p.B);
     if (kernel_size == 2) launch_conv_ks<T, WT, 2>(p, silu, grid, stream);
     else if (kernel_size == 3) launch_conv_ks<T, WT, 3>(p, silu, grid, stream);
     else launch_conv_ks<T, WT, 4>(p, silu, grid, stream);
@@ -164,7 +168,7 @@ extern "C" int gdn_causal_conv1d_fwd(const gdn_conv_args* a, void* stream) {
     if (a->w_dtype != GDN_BF16 && a->w_dtype != GDN_F32) return GDN_ERR_UNSUPPORTED;
     if (a->dtype == GDN_F32 && a->w_dtype != GDN_F32) return GDN_ERR_UNSUPPORTED;  // weights as wide as the data
     if (a->activation != GDN_ACT_NONE && a->activation != GDN_ACT_SILU) return GDN_ERR_UNSUPPORTED;
-    if (a->B > 65535 || (a->S + gdn::CONV_TOKENS - 1) / gdn::CONV_TOKENS > 65535) return GDN_ERR_UNSUPPORTED;
+    if (a->B > 65535 || a->S / (gdn::CONV_TOKENS * (gdn::CONV_THREADS / gdn::WAVE)) >= 65535) return GDN_ERR_UNSUPPORTED;
     const int64_t vec = (a->dtype == GDN_BF16) ? 8 : 4;
     if (a->C % vec != 0) return GDN_ERR_UNSUPPORTED;
     const int64_t strides[] = {a->x_stride_b, a->x_stride_s, a->y_stride_b, a->y_stride_s};
