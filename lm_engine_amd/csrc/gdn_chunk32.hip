@@ -31,7 +31,8 @@
 //   Q~             [T_tok 2][slab K/16]  B fragments of O^T = S^T Q~^T (same register layout)
 //   K~^T           [T_d K/32][slab 4]    A fragments, rows = key dim, reduction = tokens
 //   P              [T_i 2][slab 4]       B fragments of O^T += V~^T P^T
-//   U              [T_n V/32][lane][T_tok 2][16]  accumulator layout, lane l32 = column slice_col(l32) of the tile
+//   U              [T_n V/32][T_tok 2][half 2][lane][8]  accumulator layout (registers 8 half .. 8 half + 7 of token
+//                  tile T_tok), lane l32 = column slice_col(l32) of the tile
 //   e^{gamma_C}
 
 #include <type_traits>
@@ -538,11 +539,12 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
                         __builtin_amdgcn_sched_barrier(0);
                     }
                     const int tn = v0 / 32 + tl;
-                    bf16x8* uf = reinterpret_cast<bf16x8*>(rec + p.off_u) + ((int64_t)tn * WAVE + lane) * 4;
-                    uf[0] = pack8_16(acc[0], 0, 1.f);
-                    uf[1] = pack8_16(acc[0], 1, 1.f);
-                    uf[2] = pack8_16(acc[1], 0, 1.f);
-                    uf[3] = pack8_16(acc[1], 1, 1.f);
+                    // four fragments of 1 KiB per tile, each one contiguous store of the wave (whole cache lines)
+                    bf16x8* uf = reinterpret_cast<bf16x8*>(rec + p.off_u) + (int64_t)tn * 4 * WAVE + lane;
+                    uf[0 * WAVE] = pack8_16(acc[0], 0, 1.f);
+                    uf[1 * WAVE] = pack8_16(acc[0], 1, 1.f);
+                    uf[2 * WAVE] = pack8_16(acc[1], 0, 1.f);
+                    uf[3 * WAVE] = pack8_16(acc[1], 1, 1.f);
                 }
             }
         }
@@ -776,7 +778,7 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
         return reinterpret_cast<const bf16x8*>(st)[f * WAVE + lane];
     };
     auto lds_u = [&](const uint8_t* st, int i) -> bf16x8 {
-        return reinterpret_cast<const bf16x8*>(st + SHARED_BYTES)[(wave * WAVE + lane) * 4 + i];
+        return reinterpret_cast<const bf16x8*>(st + SHARED_BYTES)[(wave * 4 + i) * WAVE + lane];
     };
     auto lds_eg = [&](const uint8_t* st) -> float { return *reinterpret_cast<const float*>(st + STAGE_FRAGS * FRAG_BYTES); };
 
