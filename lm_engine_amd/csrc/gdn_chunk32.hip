@@ -21,19 +21,24 @@
 //   A[i = l%32][k = 8 h + 0..7]    B[k = 8 h + 0..7][j = l%32]
 //   D[i = 8 (r/4) + 4 h + r%4][j = l%32]   for accumulator register r = 0..15
 //
-// Permuted reduction order: a D tile reused as B (or A) operand gives, for the 16-row slab s of
-// the tile (s = 0, 1), registers 8 s .. 8 s + 7, i.e. rows 16 s + 4 h + 0..3 and 16 s + 8 + 4 h + 0..3.
-// The matching fragment of a row-major matrix Y holds Y[m][16 s' + 4 h + 0..3], Y[m][16 s' + 8 + 4 h + 0..3]
-// for the global slab index s' (16 reduction entries per slab).
+// Reduction order: a D tile reused as B (or A) operand gives, for the 16-row slab s of the tile
+// (s = 0, 1), registers 8 s .. 8 s + 7, i.e. MFMA rows 16 s + 4 h + 0..3 and 16 s + 8 + 4 h + 0..3.
+// The state keeps its rows (key dim) and its columns in the order slice_col (bits 2 and 3 of the
+// index within a 32-block swapped): MFMA row i of a state tile is key column slice_col(i), so the 8
+// entries a lane half contributes per slab are the 8 consecutive key columns 16 s + 8 h + 0..7.
+// Prepare reads K through the transposing LDS load in that order at no cost, and the scan can use
+// q straight from its row-major rows.  (The token index of V~, where it is the reduction index of
+// K~^T V~ and P V~, keeps the MFMA order; K~^T and P fragments are built to match.)
 //
-// Record (same sizes and offsets as the 16x16 variant):
+// Record:
 //   W~  = -W       [T_tok 2][slab K/16]  A fragments, rows = tokens, reduction = key dim
-//   Q~             [T_tok 2][slab K/16]  B fragments of O^T = S^T Q~^T (same register layout)
 //   K~^T           [T_d K/32][slab 4]    A fragments, rows = key dim, reduction = tokens
-//   P              [T_i 2][slab 4]       B fragments of O^T += V~^T P^T
+//   P              6 fragments           B fragments of O^T += V~^T P^T: (query tile 0; key slabs 0, 1),
+//                                        (query tile 1; key slabs 0..3); P[i < 32][j >= 32] = 0 is not stored
 //   U              [T_n V/32][T_tok 2][half 2][lane][8]  accumulator layout (registers 8 half .. 8 half + 7 of token
 //                  tile T_tok), lane l32 = column slice_col(l32) of the tile
-//   e^{gamma_C}
+//   64 fp32 row scales of q (e^{gamma} scale / |q|), e^{gamma_C}
+// q itself is not copied: the scan reads its rows from the caller's tensor.
 
 #include <type_traits>
 
@@ -239,6 +244,7 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
             s_cw[tid] = s_beta[tid] * __expf(gam) * rk;  // column scale of T for W
             s_ks[tid] = __expf(gl - gam) * rk;           // row scale of K~
             s_qs[tid] = __expf(gam) * p.scale * rq;      // row scale of Q~
+            reinterpret_cast<float*>(rec + p.off_qs)[tid] = s_qs[tid];
             if (tid == 0) *reinterpret_cast<float*>(rec + p.off_eg) = __expf(gl);
         }
         __syncthreads();  // #2
@@ -277,28 +283,11 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
                         const float val = qi * s_rk[j] * __expf(gi - s_gam[j]) * acc[r];
                         pv[r] = (i >= j) ? val : 0.f;
                     }
+                    // fragments (tcol, 2 trow + s); the all-zero pair (tcol 0, trow 1) has no place in the record
                     bf16x8* pf = reinterpret_cast<bf16x8*>(rec + p.off_p);
-                    pf[(tcol * 4 + 2 * trow + 0) * WAVE + lane] = pack8_16(pv, 0, 1.f);
-                    pf[(tcol * 4 + 2 * trow + 1) * WAVE + lane] = pack8_16(pv, 1, 1.f);
-                }
-            };
-            // Q~ fragments (T_tok, slab): Q~[tok][16 s + 4 h + e], Q~[tok][16 s + 8 + 4 h + e]; made here, by the
-            // two waves with a single tile job, because the region of Q is overwritten by T after the next barrier
-            auto q_frags = [&](int first) {
-                bf16x8* qf = reinterpret_cast<bf16x8*>(rec + p.off_qs);
-                for (int f = first; f < 2 * KS16; f += 2) {
-                    const int tt = f / KS16, s = f % KS16;
-                    const int i = 32 * tt + l32;
-                    const float sc = s_qs[i];
-                    const bf16x4 a = *reinterpret_cast<const bf16x4*>(&sQ[i * LDK + 16 * s + 4 * lh]);
-                    const bf16x4 b = *reinterpret_cast<const bf16x4*>(&sQ[i * LDK + 16 * s + 8 + 4 * lh]);
-                    bf16x8 r;
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        r[e] = (bf16_t)((float)a[e] * sc);
-                        r[4 + e] = (bf16_t)((float)b[e] * sc);
-                    }
-                    qf[f * WAVE + lane] = r;
+                    const int first = tcol == 0 ? 0 : 2 + 2 * trow;
+                    pf[(first + 0) * WAVE + lane] = pack8_16(pv, 0, 1.f);
+                    pf[(first + 1) * WAVE + lane] = pack8_16(pv, 1, 1.f);
                 }
             };
             if (wave == 0) {
@@ -309,14 +298,8 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
                 tile_job(true, 0, 0);
             } else if (wave == 2) {
                 tile_job(false, 1, 1);
-                // P[i < 32][j >= 32] = 0
-                bf16x8* pf = reinterpret_cast<bf16x8*>(rec + p.off_p);
-                pf[2 * WAVE + lane] = bf16x8{};
-                pf[3 * WAVE + lane] = bf16x8{};
-                q_frags(0);
             } else {
-                tile_job(true, 1, 1);
-                q_frags(1);
+                tile_job(true, 1, 1);  // P[i < 32][j >= 32] = 0 is not stored
             }
         }
         __syncthreads();  // #3: A complete, Q consumed (its region becomes T)
@@ -366,8 +349,8 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
             for (int f = wave - 1; f < KD * 4; f += 3) {
                 const int td = f / 4, s = f % 4;
                 const int ja = 16 * s + 4 * lh, jb = ja + 8;
-                const bf16x4 a = lds_read_tr4x16(sK, LDK, ja, 32 * td + 16 * g16, l16);
-                const bf16x4 b = lds_read_tr4x16(sK, LDK, jb, 32 * td + 16 * g16, l16);
+                const bf16x4 a = lds_read_tr4x16<true>(sK, LDK, ja, 32 * td + 16 * g16, l16);  // state-row order
+                const bf16x4 b = lds_read_tr4x16<true>(sK, LDK, jb, 32 * td + 16 * g16, l16);
                 const f32x4 sa = *reinterpret_cast<const f32x4*>(&s_ks[ja]);
                 const f32x4 sb = *reinterpret_cast<const f32x4*>(&s_ks[jb]);
                 bf16x8 r;
@@ -494,7 +477,7 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
             for (int r = 0; r < 16; r++) acc[0][r] = 0.f, acc[1][r] = 0.f;
 #pragma unroll
             for (int s = 0; s < 4; s++) {
-                const bf16x8 kt = tr_frag(sK, LDK, s, td, std::false_type{});
+                const bf16x8 kt = tr_frag(sK, LDK, s, td, std::true_type{});  // key columns in state-row order
                 if (s < 2) acc[0] = mfma32_bf16(kt, t_frag(0, s, s_cw), acc[0]);  // tokens < 32 only see j < 32
                 acc[1] = mfma32_bf16(kt, t_frag(1, s, s_cw), acc[1]);
                 __builtin_amdgcn_sched_barrier(0);
@@ -559,8 +542,9 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
 // waves, each owning a K x 32 slice of the fp32 state as MFMA accumulators, 4 loader waves and
 // (NW < 4) one output wave.
 //
-// Everything a chunk needs from its record (the operand fragments W~, Q~, K~^T, P, the U tiles
-// of this workgroup's columns and e^{gamma_C}) goes through a double buffer in LDS: during chunk
+// Everything a chunk needs (the operand fragments W~, K~^T, P of its record, the U tiles of this
+// workgroup's columns, the chunk's rows of q from the caller's tensor, q's row scales and
+// e^{gamma_C}) goes through a double buffer in LDS: during chunk
 // c the loaders move record c + 1 global -> registers -> LDS and already have records c + 2 and
 // c + 3 in flight in a second register buffer.  One workgroup barrier per chunk hands the halves
 // over.  The memory instructions are kept out of the compute waves on purpose: a wave that
@@ -570,7 +554,7 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
 // output stores per chunk cost a compute wave 340 - 980 cycles.)
 //
 // A compute wave runs the 54 MFMAs of a chunk (K = 128) as one unrolled schedule
-//     V~ = U + W~ S0 | O^T = S0^T Q~^T | S = e^{gamma_C} S0 + K~^T V~ | O^T += V~^T P^T
+//     V~ = U + W~ S0 | O^T = diag(q scales) (q S0)^T | S = e^{gamma_C} S0 + K~^T V~ | O^T += V~^T P^T
 // reading each fragment from LDS a few MFMAs before its use.  All other per-chunk work - decay of
 // the state, bf16 repacking of V~ and of the new state, conversion of the next chunk's U, the
 // hand-over of the output tile - is cut into pieces placed between MFMAs that do not depend on
@@ -592,15 +576,25 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
     constexpr bool OS = NW < 4;
     constexpr int KD = K / 32;    // 32-row tiles of the state
     constexpr int KS16 = K / 16;  // 16-wide slabs over the key dim
-    constexpr int NWF = 2 * KS16, NQF = 2 * KS16, NKF = KD * 4, NPF = 8;  // fragments of W~, Q~, K~^T, P
-    constexpr int SHARED_FRAGS = NWF + NQF + NKF + NPF;  // contiguous at the head of the record
+    constexpr int NWF = 2 * KS16, NQF = 2 * KS16, NKF = KD * 4, NPF = 6;  // fragments of W~, (rows of q), K~^T, P
+    // One half of the stage: [W~ | K~^T | P] (contiguous at the head of the record) | U tiles of this workgroup's
+    // columns (contiguous in the record) | the chunk's 64 rows of q, row-major, copied from the caller's tensor |
+    // 64 row scales of q | e^{gamma_C}
+    constexpr int SHARED_FRAGS = NWF + NKF + NPF;
     constexpr int SHARED_BYTES = SHARED_FRAGS * FRAG_BYTES;
-    constexpr int U_FRAGS = 4 * NW;  // U tiles of this workgroup's columns: contiguous in the record
+    constexpr int U_FRAGS = 4 * NW;
     constexpr int STAGE_FRAGS = SHARED_FRAGS + U_FRAGS;
-    constexpr int STAGE_BYTES = STAGE_FRAGS * FRAG_BYTES + 16;  // + e^{gamma_C}
-    constexpr int NLOAD = STAGE_FRAGS / NL;                     // fragments moved by each loader wave
-    static_assert(2 * STAGE_BYTES <= 160 * 1024, "double buffer exceeds LDS");
-    static_assert(STAGE_FRAGS % NL == 0, "fragments must divide over the loader waves");
+    constexpr int QLD = 2 * K + 16;             // bytes per staged row of q (16 bytes of padding against bank conflicts)
+    constexpr int Q_UNITS = C * 2 * K / FRAG_BYTES;  // 1 KiB pieces of the q rows: 512 / K whole rows each
+    constexpr int Q_OFF = STAGE_FRAGS * FRAG_BYTES;
+    constexpr int QS_OFF = Q_OFF + C * QLD;
+    constexpr int EG_OFF = QS_OFF + C * 4;
+    constexpr int STAGE_BYTES = EG_OFF + 16;
+    constexpr int NF = (STAGE_FRAGS + NL - 1) / NL;  // fragment slots per loader wave
+    constexpr int NQ = Q_UNITS / NL;                 // q-row slots per loader wave
+    constexpr int NLOAD = NF + NQ;                   // 1 KiB moves per loader wave and record
+    static_assert(Q_UNITS % NL == 0, "the pieces of q must divide over the loader waves");
+    static_assert(2 * STAGE_BYTES + (OS ? NW * 2 * C * 64 : 16) <= 160 * 1024, "stage exceeds LDS");
 
     __shared__ __attribute__((aligned(16))) uint8_t stage[2][STAGE_BYTES];
     __shared__ __attribute__((aligned(16))) uint8_t ostage[OS ? NW * 2 * C * 64 : 16];
@@ -671,50 +665,74 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
         // ------------------------------ loader ------------------------------
         // fragment f of the stage: f < SHARED_FRAGS comes from the head of the record, the rest from
         // this workgroup's slice of the U block
-        const int lw = wave - NW;
-        // This wave moves fragments lw * NLOAD .. + NLOAD - 1 of the stage, starting `rot` into the block: the
-        // workgroups of a chain (one per column group) then ask for different lines at any one time, and a
-        // line's memory latency is paid by one of them instead of being waited out by all.
-        const int rot = (vgroup * ((NLOAD + 3) / 4)) % NLOAD;
-        auto frag_of = [&](int i) { return lw * NLOAD + (i + rot < NLOAD ? i + rot : i + rot - NLOAD); };
+        const int lw = __builtin_amdgcn_readfirstlane(wave - NW);  // wave-uniform: unit numbers and bases stay scalar
+        // Slots 0 .. NF - 1 of this wave move fragments lw * NF + (rotated slot), slots NF .. NLOAD - 1 move 1 KiB
+        // pieces of the q rows; a surplus fragment slot repeats the last fragment.  Which kind a slot is, is known
+        // at compile time, so there is no branch in these loops (a branch makes the compiler wait for every load
+        // in flight).  The rotation by column group lets the workgroups of a chain ask for different lines at
+        // any one time: a line's memory latency is then paid by one of them instead of being waited out by all.
+        const int rot_f = (vgroup * ((NF + 3) / 4)) % NF;
+        const int rot_q = vgroup % NQ;
+        auto frag_of = [&](int i) {  // i < NF
+            const int f = lw * NF + (i + rot_f < NF ? i + rot_f : i + rot_f - NF);
+            return f < STAGE_FRAGS ? f : STAGE_FRAGS - 1;
+        };
+        auto qunit_of = [&](int i) { return lw * NQ + (i + rot_q < NQ ? i + rot_q : i + rot_q - NQ); };  // i < NQ
         const int64_t u_shift = (int64_t)p.off_u + (int64_t)vgroup * U_FRAGS * FRAG_BYTES - SHARED_BYTES;
+        // rows of q: lane -> (row within the unit, 16-byte piece)
+        constexpr int Q_ROWS = C / Q_UNITS, Q_PIECES = WAVE / Q_ROWS;
+        const int q_row = lane / Q_PIECES, q_piece = lane % Q_PIECES;
+        const bf16_t* const qg = p.q + b * p.q_stride_b + seq_t0 * p.q_stride_t + (int64_t)h * p.q_stride_h + q_piece * 8;
         // two register buffers: while one record is written to LDS, younger ones are in flight
         bf16x8 buf0[NLOAD], buf1[NLOAD];
+        float sc0 = 0.f, sc1 = 0.f;  // q's row scale of token `lane`
         float eg0 = 0.f, eg1 = 0.f;
-        auto src_of = [&](int c, int i) {
-            const int f = frag_of(i);
-            return rec + (int64_t)c * p.rec_bytes + (int64_t)f * FRAG_BYTES + (f >= SHARED_FRAGS ? u_shift : 0) + lane * 16;
+        auto src_of = [&](int c, int i) -> const uint8_t* {
+            if (i < NF) {
+                const int f = frag_of(i);
+                return rec + ((int64_t)c * p.rec_bytes + (int64_t)f * FRAG_BYTES + (f >= SHARED_FRAGS ? u_shift : 0)) + lane * 16;
+            }
+            // a row past the end of the sequence (tail chunk) is read from the last token instead: never used
+            const int tok = min(c * C + qunit_of(i - NF) * Q_ROWS + q_row, (int)seq_len - 1);
+            return reinterpret_cast<const uint8_t*>(qg + (int64_t)tok * p.q_stride_t);
         };
-        auto load = [&](bf16x8(&buf)[NLOAD], float& eg, int c) {
+        auto dst_of = [&](uint8_t* st, int i) -> uint8_t* {
+            if (i < NF) return st + frag_of(i) * FRAG_BYTES + lane * 16;
+            return st + Q_OFF + (qunit_of(i - NF) * Q_ROWS + q_row) * QLD + q_piece * 16;
+        };
+        // every loader wave carries the 64 row scales of q and e^{gamma_C} (identical values, identical LDS writes)
+        auto load_scalars = [&](float& sc, float& eg, int c) {
+            sc = reinterpret_cast<const float*>(rec + (int64_t)c * p.rec_bytes + p.off_qs)[lane];
+            eg = *reinterpret_cast<const float*>(rec + (int64_t)c * p.rec_bytes + p.off_eg);
+        };
+        auto load = [&](bf16x8(&buf)[NLOAD], float& sc, float& eg, int c) {
 #pragma unroll
             for (int i = 0; i < NLOAD; i++) buf[i] = *reinterpret_cast<const bf16x8*>(src_of(c, i));
-            if (lw == 0) eg = *reinterpret_cast<const float*>(rec + (int64_t)c * p.rec_bytes + p.off_eg);
+            load_scalars(sc, eg, c);
         };
         // write record c to LDS and refill each register with record c2 right behind its write, so the
         // LDS-write and the vector-memory queues fill together
-        auto store_and_reload = [&](bf16x8(&buf)[NLOAD], float& eg, int c, int c2, auto reload_tag) {
+        auto store_and_reload = [&](bf16x8(&buf)[NLOAD], float& sc, float& eg, int c, int c2, auto reload_tag) {
             constexpr bool reload = decltype(reload_tag)::value;
             uint8_t* dst = stage[c & 1];
-            bf16x8* d = reinterpret_cast<bf16x8*>(dst) + lane;
-            if (lw == 0 && lane == 0) *reinterpret_cast<float*>(dst + STAGE_FRAGS * FRAG_BYTES) = eg;
+            reinterpret_cast<float*>(dst + QS_OFF)[lane] = sc;
+            if (lane == 0) *reinterpret_cast<float*>(dst + EG_OFF) = eg;
 #pragma unroll
             for (int i = 0; i < NLOAD; i++) {
-                d[frag_of(i) * WAVE] = buf[i];
+                *reinterpret_cast<bf16x8*>(dst_of(dst, i)) = buf[i];
                 if constexpr (reload) buf[i] = *reinterpret_cast<const bf16x8*>(src_of(c2, i));
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if constexpr (reload) {
-                if (lw == 0) eg = *reinterpret_cast<const float*>(rec + (int64_t)c2 * p.rec_bytes + p.off_eg);
-            }
+            if constexpr (reload) load_scalars(sc, eg, c2);
         };
         constexpr std::true_type yes{};
         constexpr std::false_type no{};
         // records 0 (-> LDS now), 1 and 2 (in flight); even records use buf0, odd ones buf1
         if (nchunks > 0) {
-            load(buf0, eg0, 0);
-            if (nchunks > 1) load(buf1, eg1, 1);
-            if (nchunks > 2) store_and_reload(buf0, eg0, 0, 2, yes);
-            else store_and_reload(buf0, eg0, 0, 0, no);
+            load(buf0, sc0, eg0, 0);
+            if (nchunks > 1) load(buf1, sc1, eg1, 1);
+            if (nchunks > 2) store_and_reload(buf0, sc0, eg0, 0, 2, yes);
+            else store_and_reload(buf0, sc0, eg0, 0, 0, no);
         }
         __syncthreads();  // stage[0] holds record 0
         // Barrier of iteration c: the compute waves are done with stage[c & 1] and record c + 1 is in the
@@ -722,19 +740,19 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
         // c - 1) and refill the freed registers with record c + 3.
         int c = 0;
         for (; c + 4 < nchunks; c += 2) {  // steady state: straight-line code, both reloads exist
-            store_and_reload(buf1, eg1, c + 1, c + 3, yes);
+            store_and_reload(buf1, sc1, eg1, c + 1, c + 3, yes);
             __syncthreads();
-            store_and_reload(buf0, eg0, c + 2, c + 4, yes);
+            store_and_reload(buf0, sc0, eg0, c + 2, c + 4, yes);
             __syncthreads();
         }
         for (; c < nchunks; c += 2) {  // the last (at most four) chunks
             if (c + 1 < nchunks) {
-                if (c + 3 < nchunks) store_and_reload(buf1, eg1, c + 1, c + 3, yes);
-                else store_and_reload(buf1, eg1, c + 1, 0, no);
+                if (c + 3 < nchunks) store_and_reload(buf1, sc1, eg1, c + 1, c + 3, yes);
+                else store_and_reload(buf1, sc1, eg1, c + 1, 0, no);
             }
             __syncthreads();
             if (c + 1 < nchunks) {
-                if (c + 2 < nchunks) store_and_reload(buf0, eg0, c + 2, 0, no);
+                if (c + 2 < nchunks) store_and_reload(buf0, sc0, eg0, c + 2, 0, no);
                 __syncthreads();
             }
         }
@@ -744,9 +762,13 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
 
     // ------------------------------ compute ------------------------------
     const int tn = vgroup * NW + wave;  // 32-column tile of V owned by this wave (the launcher makes NW divide V / 32)
-    // state tile td, register r: row 32 td + 8 (r/4) + 4 h + r%4, column 32 tn + slice_col(l32)
+    // State tile td, register r: MFMA row i = 8 (r/4) + 4 h + r%4 holds state row 32 td + slice_col(i)
+    // = 32 td + 16 (r/8) + 8 h + 4 ((r/4) % 2) + r%4, column 32 tn + slice_col(l32).  With the rows of a 16-block
+    // in that order, the 8 reduction entries a lane half feeds per 16-row slab are 8 consecutive key columns:
+    // q is used straight from its row-major rows.
     f32x16 S[KD];
-    const int64_t st_off = ((int64_t)n * p.H + h) * K * p.V + (int64_t)(4 * lh) * p.V + 32 * tn + slice_col(l32);
+    const int64_t st_off = ((int64_t)n * p.H + h) * K * p.V + (int64_t)(8 * lh) * p.V + 32 * tn + slice_col(l32);
+    auto st_row = [](int td, int r) { return 32 * td + 16 * (r / 8) + 4 * ((r / 4) % 2) + r % 4; };
 #pragma unroll
     for (int td = 0; td < KD; td++)
 #pragma unroll
@@ -755,36 +777,37 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
 #pragma unroll
         for (int td = 0; td < KD; td++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) S[td][r] = p.h0[st_off + (int64_t)(32 * td + 8 * (r / 4) + r % 4) * p.V];
+            for (int r = 0; r < 16; r++) S[td][r] = p.h0[st_off + (int64_t)st_row(td, r) * p.V];
     }
     // O^T tile tt, register r: token 32 tt + l32, column 32 tn + 16 (r/8) + 8 h + r%8 (slice_col order)
     bf16_t* og = p.o + b * p.o_stride_b + (seq_t0 + l32) * p.o_stride_t + (int64_t)h * p.o_stride_h + 32 * tn + 8 * lh;
     const int64_t og_step = (int64_t)C * p.o_stride_t;
 
-    // MFMA schedule of one chunk: W~ (NWF) | Q~ (NQF) | K~^T (NKF) | P (6: the two zero fragments are skipped).
-    // Everything else a chunk needs (decay of the state, bf16 repacking of V~ and of the new state, conversion
-    // of the next U, conversion and store of the previous chunk's output) is cut into pieces that sit between
-    // MFMAs whose operands do not depend on them, so the matrix pipe stays fed by this one wave.
-    constexpr int NOPS = NWF + NQF + NKF + 6;
+    // MFMA schedule of one chunk: W~ (NWF) | q (NQF) | K~^T (NKF) | P (6).
+    // Everything else a chunk needs (decay of the state, bf16 repacking of V~ and of the new state, the row
+    // scale of q S0, conversion of the next U, hand-over of the previous chunk's output) is cut into pieces
+    // that sit between MFMAs whose operands do not depend on them, so the matrix pipe stays fed by this one wave.
+    constexpr int NOPS = NWF + NQF + NKF + NPF;
     constexpr int LA = 6;  // LDS reads are issued this many MFMAs ahead of their use
     constexpr int OP_Q = NWF, OP_K = NWF + NQF, OP_P = NWF + NQF + NKF, OP_BAR = NOPS - LA;
-    static_assert(OP_BAR >= OP_K, "the barrier must come after the reads of the W~ and Q~ fragments");
+    static_assert(OP_BAR >= OP_K, "the barrier must come after the reads of the W~ fragments and of q");
     auto lds_frag = [&](const uint8_t* st, int op) -> bf16x8 {
-        int f = op;
-        if (op >= OP_P) {  // P fragments (tt, s) with tt == 1 or s < 2: indices 0, 1, 4, 5, 6, 7
-            const int j = op - OP_P;
-            f = OP_P + (j < 2 ? j : j + 2);
+        if (op >= OP_Q && op < OP_K) {  // q, token tile tt, 16-column slab s: 8 consecutive columns per lane half
+            const int j = op - OP_Q, s = j % KS16, tt = j / KS16;
+            return *reinterpret_cast<const bf16x8*>(st + Q_OFF + (32 * tt + l32) * QLD + (16 * s + 8 * lh) * 2);
         }
+        const int f = op < OP_Q ? op : op - NQF;  // W~ | K~^T | P are contiguous in the stage
         return reinterpret_cast<const bf16x8*>(st)[f * WAVE + lane];
     };
     auto lds_u = [&](const uint8_t* st, int i) -> bf16x8 {
         return reinterpret_cast<const bf16x8*>(st + SHARED_BYTES)[(wave * 4 + i) * WAVE + lane];
     };
-    auto lds_eg = [&](const uint8_t* st) -> float { return *reinterpret_cast<const float*>(st + STAGE_FRAGS * FRAG_BYTES); };
+    auto lds_eg = [&](const uint8_t* st) -> float { return *reinterpret_cast<const float*>(st + EG_OFF); };
+    auto lds_qs = [&](const uint8_t* st, int tt) -> float { return reinterpret_cast<const float*>(st + QS_OFF)[32 * tt + l32]; };
 
     f32x16 accv[2], acco[2];
     bf16x8 sb[KS16], vb[4], ur[4], fnext[LA];
-    float egc;
+    float egc, qsc[2];  // e^{gamma_C} and this lane's two row scales of q (tokens l32 and 32 + l32)
 #pragma unroll
     for (int tt = 0; tt < 2; tt++)
 #pragma unroll
@@ -796,6 +819,7 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
 #pragma unroll
     for (int i = 0; i < 4; i++) ur[i] = lds_u(stage[0], i);
     egc = lds_eg(stage[0]);
+    qsc[0] = lds_qs(stage[0], 0), qsc[1] = lds_qs(stage[0], 1);
 #pragma unroll
     for (int i = 0; i < LA; i++) fnext[i] = lds_frag(stage[0], i);
 #pragma unroll
@@ -824,6 +848,7 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
 #pragma unroll
                 for (int i = 0; i < 4; i++) ur[i] = lds_u(stn, i);
                 egc = lds_eg(stn);
+                qsc[0] = lds_qs(stn, 0), qsc[1] = lds_qs(stn, 1);  // this chunk's scales were applied before OP_P
             }
             if (op >= OP_BAR) fnext[op - OP_BAR] = lds_frag(stn, op - OP_BAR);
 
@@ -852,6 +877,17 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
                 const int j = op - OP_K - 5;
                 if (j % 4 < 2 && j / 4 < KD) sb[2 * (j / 4) + j % 4] = pack8_16(S[j / 4], j % 4, 1.f);
             }
+            // O^T = (q S0)^T so far: its columns (tokens) take the row scale of q before the P terms are added
+            if (op >= OP_Q + KS16 + 2 && op < OP_Q + KS16 + 6) {
+                const int q4 = op - (OP_Q + KS16 + 2);
+#pragma unroll
+                for (int i = 0; i < 4; i++) acco[0][4 * q4 + i] *= qsc[0];
+            }
+            if (op >= OP_K + 2 && op < OP_K + 6) {
+                const int q4 = op - (OP_K + 2);
+#pragma unroll
+                for (int i = 0; i < 4; i++) acco[1][4 * q4 + i] *= qsc[1];
+            }
             if (op >= NOPS - 4) {  // U of the next chunk -> fp32 accumulators (V~ of this chunk lives on in vb)
                 const int q = op - (NOPS - 4);
 #pragma unroll
@@ -862,7 +898,7 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
             if (op < OP_Q) {  // V~ = U + W~ S0, fragment (tt, s) = op
                 const int s = op % KS16, tt = op / KS16;
                 accv[tt] = mfma32_bf16(fr[op], sb[s], accv[tt]);
-            } else if (op < OP_K) {  // O^T = S0^T Q~^T
+            } else if (op < OP_K) {  // O^T = (q S0)^T, scaled per token further down
                 const int j = op - OP_Q, s = j % KS16, tt = j / KS16;
                 if (s == 0) {
                     f32x16 zero;
@@ -906,7 +942,7 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
 #pragma unroll
         for (int td = 0; td < KD; td++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) p.ht[st_off + (int64_t)(32 * td + 8 * (r / 4) + r % 4) * p.V] = S[td][r];
+            for (int r = 0; r < 16; r++) p.ht[st_off + (int64_t)st_row(td, r) * p.V] = S[td][r];
     }
 }
 

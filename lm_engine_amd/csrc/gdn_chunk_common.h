@@ -40,17 +40,28 @@ struct RecordLayout {
     uint32_t off_wn, off_qs, off_kt, off_p, off_u, off_eg, bytes;
 };
 
-// Record of one (head, chunk): Wn (-W), Qs, Kt, P as A-operand fragments, U as accumulator
-// fragments, e^{gamma_C}.
+// Record of one (head, chunk).
+//   K = 256 (16x16x32 kernels): Wn (-W), Qs, Kt, P (8 fragments) as operand fragments, U as accumulator
+//   fragments, e^{gamma_C}.
+//   K <= 128 (32x32x16 kernels): Wn, Kt, the 6 non-zero fragments of P, U, then at off_qs the 64 fp32 row
+//   scales of q (e^{gamma} scale / |q|) and e^{gamma_C}; q itself is read from the caller's tensor by the scan.
 inline RecordLayout record_layout(int K, int V) {
     RecordLayout r;
     const uint32_t kfrag = (uint32_t)(C / 16) * (K / 32) * FRAG_BYTES;  // [C x K] or [K x C] bf16
     r.off_wn = 0;
-    r.off_qs = kfrag;
-    r.off_kt = 2 * kfrag;
-    r.off_p = 3 * kfrag;
-    r.off_u = r.off_p + (C / 16) * (C / 32) * FRAG_BYTES;
-    r.off_eg = r.off_u + (uint32_t)C * V * 2;
+    if (K > 128) {
+        r.off_qs = kfrag;
+        r.off_kt = 2 * kfrag;
+        r.off_p = 3 * kfrag;
+        r.off_u = r.off_p + (C / 16) * (C / 32) * FRAG_BYTES;
+        r.off_eg = r.off_u + (uint32_t)C * V * 2;
+    } else {
+        r.off_kt = kfrag;
+        r.off_p = 2 * kfrag;
+        r.off_u = r.off_p + 6 * FRAG_BYTES;
+        r.off_qs = r.off_u + (uint32_t)C * V * 2;
+        r.off_eg = r.off_qs + C * 4;
+    }
     r.bytes = (r.off_eg + 4 + 255u) & ~255u;
     return r;
 }
