@@ -245,6 +245,7 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
             s_ks[tid] = __expf(gl - gam) * rk;           // row scale of K~
             s_qs[tid] = __expf(gam) * p.scale * rq;      // row scale of Q~
             reinterpret_cast<float*>(rec + p.off_qs)[tid] = s_qs[tid];
+            reinterpret_cast<float*>(rec + p.off_ks)[tid] = s_ks[tid];
             if (tid == 0) *reinterpret_cast<float*>(rec + p.off_eg) = __expf(gl);
         }
         __syncthreads();  // #2
@@ -304,7 +305,7 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
         }
         __syncthreads();  // #3: A complete, Q consumed (its region becomes T)
 
-        // ---- wave 0: inverses of the four 16 x 16 diagonal blocks; waves 1-3: K~^T fragments ----
+        // ---- wave 0: inverses of the four 16 x 16 diagonal blocks ----
         if (wave == 0) {
             const int blk = lq, j = l16;  // lane owns column j of block `blk`
             const float* a = &sA[(16 * blk) * LDA + 16 * blk];
@@ -342,24 +343,6 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
                     *reinterpret_cast<f32x4*>(&sTt2[j * LDM + 4 * c4]) = f32x4{x[4 * c4], x[4 * c4 + 1], x[4 * c4 + 2], x[4 * c4 + 3]};
 #pragma unroll
                 for (int i = 0; i < 16; i++) sT[(32 + i) * LDA + 48 + j] = 0.f;  // T block (2, 3)
-            }
-        } else {
-            // K~^T fragments (T_d, token slab): K~[16 s + 4 h + e][d], K~[16 s + 8 + 4 h + e][d]
-            bf16x8* kf = reinterpret_cast<bf16x8*>(rec + p.off_kt);
-            for (int f = wave - 1; f < KD * 4; f += 3) {
-                const int td = f / 4, s = f % 4;
-                const int ja = 16 * s + 4 * lh, jb = ja + 8;
-                const bf16x4 a = lds_read_tr4x16<true>(sK, LDK, ja, 32 * td + 16 * g16, l16);  // state-row order
-                const bf16x4 b = lds_read_tr4x16<true>(sK, LDK, jb, 32 * td + 16 * g16, l16);
-                const f32x4 sa = *reinterpret_cast<const f32x4*>(&s_ks[ja]);
-                const f32x4 sb = *reinterpret_cast<const f32x4*>(&s_ks[jb]);
-                bf16x8 r;
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    r[e] = (bf16_t)((float)a[e] * sa[e]);
-                    r[4 + e] = (bf16_t)((float)b[e] * sb[e]);
-                }
-                kf[f * WAVE + lane] = r;
             }
         }
         __syncthreads();  // #4: diagonal blocks of T
@@ -576,24 +559,26 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
     constexpr bool OS = NW < 4;
     constexpr int KD = K / 32;    // 32-row tiles of the state
     constexpr int KS16 = K / 16;  // 16-wide slabs over the key dim
-    constexpr int NWF = 2 * KS16, NQF = 2 * KS16, NKF = KD * 4, NPF = 6;  // fragments of W~, (rows of q), K~^T, P
-    // One half of the stage: [W~ | K~^T | P] (contiguous at the head of the record) | U tiles of this workgroup's
-    // columns (contiguous in the record) | the chunk's 64 rows of q, row-major, copied from the caller's tensor |
-    // 64 row scales of q | e^{gamma_C}
-    constexpr int SHARED_FRAGS = NWF + NKF + NPF;
+    constexpr int NWF = 2 * KS16, NQF = 2 * KS16, NKF = KD * 4, NPF = 6;  // MFMAs on W~, on q, on k^T, on P
+    // One half of the stage: [W~ | P] (contiguous at the head of the record) | U tiles of this workgroup's columns
+    // (contiguous in the record) | the chunk's 64 rows of q, then of k, row-major, copied from the caller's
+    // tensors | 64 row scales of q | 64 row scales of k | e^{gamma_C}
+    constexpr int SHARED_FRAGS = NWF + NPF;
     constexpr int SHARED_BYTES = SHARED_FRAGS * FRAG_BYTES;
     constexpr int U_FRAGS = 4 * NW;
     constexpr int STAGE_FRAGS = SHARED_FRAGS + U_FRAGS;
-    constexpr int QLD = 2 * K + 16;             // bytes per staged row of q (16 bytes of padding against bank conflicts)
-    constexpr int Q_UNITS = C * 2 * K / FRAG_BYTES;  // 1 KiB pieces of the q rows: 512 / K whole rows each
+    constexpr int QLD = 2 * K + 16;                  // bytes per staged row of q / k (16 bytes of padding against bank conflicts)
+    constexpr int Q_UNITS = C * 2 * K / FRAG_BYTES;  // 1 KiB pieces of the q rows: 512 / K whole rows each; as many for k
     constexpr int Q_OFF = STAGE_FRAGS * FRAG_BYTES;
-    constexpr int QS_OFF = Q_OFF + C * QLD;
-    constexpr int EG_OFF = QS_OFF + C * 4;
+    constexpr int K_OFF = Q_OFF + C * QLD;
+    constexpr int QS_OFF = K_OFF + C * QLD;
+    constexpr int KS_OFF = QS_OFF + C * 4;
+    constexpr int EG_OFF = KS_OFF + C * 4;
     constexpr int STAGE_BYTES = EG_OFF + 16;
     constexpr int NF = (STAGE_FRAGS + NL - 1) / NL;  // fragment slots per loader wave
-    constexpr int NQ = Q_UNITS / NL;                 // q-row slots per loader wave
+    constexpr int NQ = 2 * Q_UNITS / NL;             // q / k row slots per loader wave
     constexpr int NLOAD = NF + NQ;                   // 1 KiB moves per loader wave and record
-    static_assert(Q_UNITS % NL == 0, "the pieces of q must divide over the loader waves");
+    static_assert((2 * Q_UNITS) % NL == 0, "the pieces of q and k must divide over the loader waves");
     static_assert(2 * STAGE_BYTES + (OS ? NW * 2 * C * 64 : 16) <= 160 * 1024, "stage exceeds LDS");
 
     __shared__ __attribute__((aligned(16))) uint8_t stage[2][STAGE_BYTES];
@@ -683,39 +668,47 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
         constexpr int Q_ROWS = C / Q_UNITS, Q_PIECES = WAVE / Q_ROWS;
         const int q_row = lane / Q_PIECES, q_piece = lane % Q_PIECES;
         const bf16_t* const qg = p.q + b * p.q_stride_b + seq_t0 * p.q_stride_t + (int64_t)h * p.q_stride_h + q_piece * 8;
+        const bf16_t* const kg = p.k + b * p.k_stride_b + seq_t0 * p.k_stride_t + (int64_t)h * p.k_stride_h + q_piece * 8;
         // two register buffers: while one record is written to LDS, younger ones are in flight
         bf16x8 buf0[NLOAD], buf1[NLOAD];
-        float sc0 = 0.f, sc1 = 0.f;  // q's row scale of token `lane`
+        float sc0 = 0.f, sc1 = 0.f;  // lanes 0..63: row scale of q of token `lane`
+        float kc0 = 0.f, kc1 = 0.f;  // the same for k
         float eg0 = 0.f, eg1 = 0.f;
         auto src_of = [&](int c, int i) -> const uint8_t* {
             if (i < NF) {
                 const int f = frag_of(i);
                 return rec + ((int64_t)c * p.rec_bytes + (int64_t)f * FRAG_BYTES + (f >= SHARED_FRAGS ? u_shift : 0)) + lane * 16;
             }
-            // a row past the end of the sequence (tail chunk) is read from the last token instead: never used
-            const int tok = min(c * C + qunit_of(i - NF) * Q_ROWS + q_row, (int)seq_len - 1);
-            return reinterpret_cast<const uint8_t*>(qg + (int64_t)tok * p.q_stride_t);
+            // units 0 .. Q_UNITS - 1 are rows of q, the rest rows of k (wave-uniform choice); a row past the end of
+            // the sequence (tail chunk) is read from the last token instead: never used
+            const int u = qunit_of(i - NF);
+            const bool is_k = u >= Q_UNITS;
+            const int tok = min(c * C + (is_k ? u - Q_UNITS : u) * Q_ROWS + q_row, (int)seq_len - 1);
+            return reinterpret_cast<const uint8_t*>((is_k ? kg : qg) + (int64_t)tok * (is_k ? p.k_stride_t : p.q_stride_t));
         };
         auto dst_of = [&](uint8_t* st, int i) -> uint8_t* {
             if (i < NF) return st + frag_of(i) * FRAG_BYTES + lane * 16;
-            return st + Q_OFF + (qunit_of(i - NF) * Q_ROWS + q_row) * QLD + q_piece * 16;
+            return st + Q_OFF + (qunit_of(i - NF) * Q_ROWS + q_row) * QLD + q_piece * 16;  // the k rows follow the q rows
         };
-        // every loader wave carries the 64 row scales of q and e^{gamma_C} (identical values, identical LDS writes)
-        auto load_scalars = [&](float& sc, float& eg, int c) {
-            sc = reinterpret_cast<const float*>(rec + (int64_t)c * p.rec_bytes + p.off_qs)[lane];
-            eg = *reinterpret_cast<const float*>(rec + (int64_t)c * p.rec_bytes + p.off_eg);
+        // every loader wave carries the row scales of q and k and e^{gamma_C} (identical values, identical LDS writes)
+        auto load_scalars = [&](float& sc, float& kc, float& eg, int c) {
+            const uint8_t* r = rec + (int64_t)c * p.rec_bytes;
+            sc = reinterpret_cast<const float*>(r + p.off_qs)[lane];
+            kc = reinterpret_cast<const float*>(r + p.off_ks)[lane];
+            eg = *reinterpret_cast<const float*>(r + p.off_eg);
         };
-        auto load = [&](bf16x8(&buf)[NLOAD], float& sc, float& eg, int c) {
+        auto load = [&](bf16x8(&buf)[NLOAD], float& sc, float& kc, float& eg, int c) {
 #pragma unroll
             for (int i = 0; i < NLOAD; i++) buf[i] = *reinterpret_cast<const bf16x8*>(src_of(c, i));
-            load_scalars(sc, eg, c);
+            load_scalars(sc, kc, eg, c);
         };
         // write record c to LDS and refill each register with record c2 right behind its write, so the
         // LDS-write and the vector-memory queues fill together
-        auto store_and_reload = [&](bf16x8(&buf)[NLOAD], float& sc, float& eg, int c, int c2, auto reload_tag) {
+        auto store_and_reload = [&](bf16x8(&buf)[NLOAD], float& sc, float& kc, float& eg, int c, int c2, auto reload_tag) {
             constexpr bool reload = decltype(reload_tag)::value;
             uint8_t* dst = stage[c & 1];
             reinterpret_cast<float*>(dst + QS_OFF)[lane] = sc;
+            reinterpret_cast<float*>(dst + KS_OFF)[lane] = kc;
             if (lane == 0) *reinterpret_cast<float*>(dst + EG_OFF) = eg;
 #pragma unroll
             for (int i = 0; i < NLOAD; i++) {
@@ -723,16 +716,16 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
                 if constexpr (reload) buf[i] = *reinterpret_cast<const bf16x8*>(src_of(c2, i));
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if constexpr (reload) load_scalars(sc, eg, c2);
+            if constexpr (reload) load_scalars(sc, kc, eg, c2);
         };
         constexpr std::true_type yes{};
         constexpr std::false_type no{};
         // records 0 (-> LDS now), 1 and 2 (in flight); even records use buf0, odd ones buf1
         if (nchunks > 0) {
-            load(buf0, sc0, eg0, 0);
-            if (nchunks > 1) load(buf1, sc1, eg1, 1);
-            if (nchunks > 2) store_and_reload(buf0, sc0, eg0, 0, 2, yes);
-            else store_and_reload(buf0, sc0, eg0, 0, 0, no);
+            load(buf0, sc0, kc0, eg0, 0);
+            if (nchunks > 1) load(buf1, sc1, kc1, eg1, 1);
+            if (nchunks > 2) store_and_reload(buf0, sc0, kc0, eg0, 0, 2, yes);
+            else store_and_reload(buf0, sc0, kc0, eg0, 0, 0, no);
         }
         __syncthreads();  // stage[0] holds record 0
         // Barrier of iteration c: the compute waves are done with stage[c & 1] and record c + 1 is in the
@@ -740,19 +733,19 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
         // c - 1) and refill the freed registers with record c + 3.
         int c = 0;
         for (; c + 4 < nchunks; c += 2) {  // steady state: straight-line code, both reloads exist
-            store_and_reload(buf1, sc1, eg1, c + 1, c + 3, yes);
+            store_and_reload(buf1, sc1, kc1, eg1, c + 1, c + 3, yes);
             __syncthreads();
-            store_and_reload(buf0, sc0, eg0, c + 2, c + 4, yes);
+            store_and_reload(buf0, sc0, kc0, eg0, c + 2, c + 4, yes);
             __syncthreads();
         }
         for (; c < nchunks; c += 2) {  // the last (at most four) chunks
             if (c + 1 < nchunks) {
-                if (c + 3 < nchunks) store_and_reload(buf1, sc1, eg1, c + 1, c + 3, yes);
-                else store_and_reload(buf1, sc1, eg1, c + 1, 0, no);
+                if (c + 3 < nchunks) store_and_reload(buf1, sc1, kc1, eg1, c + 1, c + 3, yes);
+                else store_and_reload(buf1, sc1, kc1, eg1, c + 1, 0, no);
             }
             __syncthreads();
             if (c + 1 < nchunks) {
-                if (c + 2 < nchunks) store_and_reload(buf0, sc0, eg0, c + 2, 0, no);
+                if (c + 2 < nchunks) store_and_reload(buf0, sc0, kc0, eg0, c + 2, 0, no);
                 __syncthreads();
             }
         }
@@ -791,12 +784,25 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
     constexpr int LA = 6;  // LDS reads are issued this many MFMAs ahead of their use
     constexpr int OP_Q = NWF, OP_K = NWF + NQF, OP_P = NWF + NQF + NKF, OP_BAR = NOPS - LA;
     static_assert(OP_BAR >= OP_K, "the barrier must come after the reads of the W~ fragments and of q");
+    const int l16 = lane % 16, g16 = l32 / 16;
     auto lds_frag = [&](const uint8_t* st, int op) -> bf16x8 {
         if (op >= OP_Q && op < OP_K) {  // q, token tile tt, 16-column slab s: 8 consecutive columns per lane half
             const int j = op - OP_Q, s = j % KS16, tt = j / KS16;
             return *reinterpret_cast<const bf16x8*>(st + Q_OFF + (32 * tt + l32) * QLD + (16 * s + 8 * lh) * 2);
         }
-        const int f = op < OP_Q ? op : op - NQF;  // W~ | K~^T | P are contiguous in the stage
+        if (op >= OP_K && op < OP_P) {
+            // k^T, key tile td (rows in state order), token slab s: tokens 16 s + 4 h + 0..3 and 16 s + 8 + 4 h + 0..3
+            // of key column 32 td + slice_col(l32), through the transposing LDS load
+            const int j = op - OP_K, s = j % 4, td = j / 4;
+            const bf16_t* km = reinterpret_cast<const bf16_t*>(st + K_OFF);
+            const bf16x4 a = lds_read_tr4x16<true>(km, QLD / 2, 16 * s + 4 * lh, 32 * td + 16 * g16, l16);
+            const bf16x4 b = lds_read_tr4x16<true>(km, QLD / 2, 16 * s + 8 + 4 * lh, 32 * td + 16 * g16, l16);
+            bf16x8 r;
+#pragma unroll
+            for (int e = 0; e < 4; e++) r[e] = a[e], r[4 + e] = b[e];
+            return r;
+        }
+        const int f = op < OP_Q ? op : op - NQF - NKF;  // W~ | P are contiguous in the stage
         return reinterpret_cast<const bf16x8*>(st)[f * WAVE + lane];
     };
     auto lds_u = [&](const uint8_t* st, int i) -> bf16x8 {
@@ -806,7 +812,7 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
     auto lds_qs = [&](const uint8_t* st, int tt) -> float { return reinterpret_cast<const float*>(st + QS_OFF)[32 * tt + l32]; };
 
     f32x16 accv[2], acco[2];
-    bf16x8 sb[KS16], vb[4], ur[4], fnext[LA];
+    bf16x8 sb[KS16], vb[4], vbs[4], ur[4], fnext[LA];  // vbs: V~ with its rows scaled like K~'s, for the state update
     float egc, qsc[2];  // e^{gamma_C} and this lane's two row scales of q (tokens l32 and 32 + l32)
 #pragma unroll
     for (int tt = 0; tt < 2; tt++)
@@ -869,10 +875,24 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
 #pragma unroll
                 for (int i = 0; i < PER; i++) S[(op * PER + i) / 16][(op * PER + i) % 16] *= egc;
             }
-            if (op == KS16 + 2) vb[0] = pack8_16(accv[0], 0, 1.f);  // V~ rows 0..31 are complete after op KS16 - 1
-            if (op == KS16 + 3) vb[1] = pack8_16(accv[0], 1, 1.f);
-            if (op == OP_Q + 2) vb[2] = pack8_16(accv[1], 0, 1.f);  // rows 32..63 after op NWF - 1
-            if (op == OP_Q + 3) vb[3] = pack8_16(accv[1], 1, 1.f);
+            // V~ rows 0..31 are complete after op KS16 - 1, rows 32..63 after op NWF - 1: as operands, plain for
+            // P V~ and with each row (token) scaled by e^{gamma_C - gamma} / |k| for k^T V~
+            auto pack_rows = [&](int tt, int half) {
+                vb[2 * tt + half] = pack8_16(accv[tt], half, 1.f);
+                const f32x4 s0 = *reinterpret_cast<const f32x4*>(st + KS_OFF + (32 * tt + 16 * half + 4 * lh) * 4);
+                const f32x4 s1 = *reinterpret_cast<const f32x4*>(st + KS_OFF + (32 * tt + 16 * half + 8 + 4 * lh) * 4);
+                bf16x8 r;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    r[e] = (bf16_t)(accv[tt][8 * half + e] * s0[e]);
+                    r[4 + e] = (bf16_t)(accv[tt][8 * half + 4 + e] * s1[e]);
+                }
+                vbs[2 * tt + half] = r;
+            };
+            if (op == KS16 + 2) pack_rows(0, 0);
+            if (op == KS16 + 3) pack_rows(0, 1);
+            if (op == OP_Q + 2) pack_rows(1, 0);
+            if (op == OP_Q + 3) pack_rows(1, 1);
             if (op >= OP_K + 5) {  // new state tile td is complete after K~^T op 4 td + 3: its two slabs as operands
                 const int j = op - OP_K - 5;
                 if (j % 4 < 2 && j / 4 < KD) sb[2 * (j / 4) + j % 4] = pack8_16(S[j / 4], j % 4, 1.f);
@@ -908,9 +928,9 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
                 } else {
                     acco[tt] = mfma32_bf16(sb[s], fr[op], acco[tt]);
                 }
-            } else if (op < OP_P) {  // S = e^{gamma_C} S + K~^T V~, fragment (td, s)
+            } else if (op < OP_P) {  // S = e^{gamma_C} S + k^T (row-scaled V~), fragment (td, s)
                 const int j = op - OP_K, s = j % 4, td = j / 4;
-                S[td] = mfma32_bf16(fr[op], vb[s], S[td]);
+                S[td] = mfma32_bf16(fr[op], vbs[s], S[td]);
             } else {  // O^T += V~^T P^T; P[i < 32][j >= 32] = 0 is skipped
                 const int j = op - OP_P;
                 const int tt = j < 2 ? 0 : 1, s = j < 2 ? j : j - 2;
