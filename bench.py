@@ -41,10 +41,10 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # summaries are kept under profiles/.  Workloads that were not profiled report null.
 _KIB = 1024
 MEASURED_HBM_TRAFFIC_BYTES = {
-    ("cfg1_chunk_fwd_bf16", "chunk_prepare"): (2.0 * 104712.5 + 295041.7) * _KIB,
-    ("cfg1_chunk_fwd_bf16", "chunk_scan"): (2.0 * 147853.4 + 69632.6) * _KIB,
+    ("cfg1_chunk_fwd_bf16", "chunk_prepare"): (2.0 * 104650.2 + 157824.0) * _KIB,
+    ("cfg1_chunk_fwd_bf16", "chunk_scan"): (2.0 * 144834.1 + 69682.2) * _KIB,
     ("cfg3_decode_bf16", "recurrent_kernel"): (2.0 * 265449.7 + 526881.4) * _KIB,
-    ("cfg1_chunk_fwd_bf16", "causal_conv1d_kernel"): (2.0 * 117467.1 + 196752.0) * _KIB,
+    ("cfg1_chunk_fwd_bf16", "causal_conv1d_kernel"): (2.0 * 116926.8 + 196752.0) * _KIB,
     ("cfg1_chunk_fwd_bf16", "gated_rmsnorm_kernel"): (2.0 * 66081.4 + 65536.0) * _KIB,
 }
 

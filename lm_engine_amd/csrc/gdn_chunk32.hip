@@ -27,18 +27,19 @@
 // index within a 32-block swapped): MFMA row i of a state tile is key column slice_col(i), so the 8
 // entries a lane half contributes per slab are the 8 consecutive key columns 16 s + 8 h + 0..7.
 // Prepare reads K through the transposing LDS load in that order at no cost, and the scan can use
-// q straight from its row-major rows.  (The token index of V~, where it is the reduction index of
-// K~^T V~ and P V~, keeps the MFMA order; K~^T and P fragments are built to match.)
+// q and k straight from their row-major rows.  (The token index of V~, where it is the reduction
+// index of K^T V~ and P V~, keeps the MFMA order; the scan's transposing LDS reads of k and the P
+// fragments are built to match.)
 //
 // Record:
 //   W~  = -W       [T_tok 2][slab K/16]  A fragments, rows = tokens, reduction = key dim
-//   K~^T           [T_d K/32][slab 4]    A fragments, rows = key dim, reduction = tokens
 //   P              6 fragments           B fragments of O^T += V~^T P^T: (query tile 0; key slabs 0, 1),
 //                                        (query tile 1; key slabs 0..3); P[i < 32][j >= 32] = 0 is not stored
 //   U              [T_n V/32][T_tok 2][half 2][lane][8]  accumulator layout (registers 8 half .. 8 half + 7 of token
 //                  tile T_tok), lane l32 = column slice_col(l32) of the tile
-//   64 fp32 row scales of q (e^{gamma} scale / |q|), e^{gamma_C}
-// q itself is not copied: the scan reads its rows from the caller's tensor.
+//   64 fp32 row scales of q (e^{gamma} scale / |q|), 64 of k (e^{gamma_C - gamma} / |k|), e^{gamma_C}
+// q and k themselves are not copied: the scan reads their rows from the caller's tensors, applies
+// q's scales to the rows of the output tile and k's to the rows of V~ before the state update.
 
 #include <type_traits>
 
