@@ -114,17 +114,24 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
 
     const int tid = threadIdx.x;
     const int wave = tid / WAVE;
-    const int64_t items = (int64_t)p.TC * p.H;
+    // Work items: (chunk slot, head), the slots rounded up to a multiple of 8.  Workgroup i runs on XCD i % 8 and
+    // takes items i, i + grid, ... with the grid a multiple of 8, so w % 8 names the XCD.  That digit goes into
+    // the slot number and the heads rotate with the rest: every XCD works on all heads.  The rows of one head
+    // lie a whole token row (a multiple of 2 KiB) apart, so they fall on few channels of an XCD's L2; an XCD
+    // that only ever sees one or two heads would send all its q, k, v traffic there.
+    const int64_t items = (int64_t)((p.TC + 7) / 8) * 8 * p.H;
 
     // ---- register prefetch of one item's inputs ----
     bf16x8 kx[NPASS], qx[NPASS], vx[C * (VP / 8) / PREP_THREADS];
     float gx = 0.f;
     uint32_t bx_raw = 0;  // beta of the prefetched item, raw bits: any arithmetic on it here would wait for every load in flight
     ChunkCoord ncc;  // coordinates of the prefetched item
-    int nh = 0;
+    int nh = 0, nslot = 0;
     auto locate = [&](int64_t w) {
-        nh = (int)(w % p.H);
-        ncc = locate_chunk(p, (int)(w / p.H));
+        const int64_t j = w / 8;
+        nh = (int)(j % p.H);
+        nslot = (int)(j / p.H) * 8 + (int)(w % 8);
+        ncc = locate_chunk(p, nslot);
     };
     // Loads are written as (workgroup-uniform base pointer) + (32-bit per-lane element offset) so that the
     // compiler keeps one offset register per stream instead of a 64-bit address per load.
@@ -187,8 +194,8 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
         const int g16 = l32 / 16;                   // which 16-lane group of the 32-row operand
         const ChunkCoord cc = ncc;
         const int h = nh;
-        const int len = cc.len;  // <= 0 for an unused slot of a packed batch: nothing to do
-        uint8_t* const rec = p.rec + ((int64_t)h * p.TC + (w / p.H)) * p.rec_bytes;
+        const int len = cc.len;  // <= 0 for an unused slot (packed batch, rounded-up grid): nothing to do
+        uint8_t* const rec = p.rec + ((int64_t)h * p.TC + nslot) * p.rec_bytes;
         const bool has_next = w + gridDim.x < items;
 
         // ---- registers -> LDS (K, Q), row sums of squares, gamma = cumsum(g), beta ----
@@ -553,8 +560,126 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
 // ------------------------------------------------------------------------------------------
 constexpr int SCAN_LOADERS = 4;
 
+// Waves of a scan workgroup.  The hardware deals the waves of a workgroup round over the four SIMDs (wave w runs on
+// SIMD w % 4), and a wave that shares a SIMD with a compute wave takes instruction-issue slots from it (measured:
+// the loader on the compute wave's SIMD ran twice as long as the other three, and the compute wave waited for it).
+// So with fewer than four compute waves the waves that land on their SIMDs get the light jobs:
+//   NW = 1:  0 compute | 1 2 3 loaders | 4 output store | 5 loader
+//   NW = 2:  0 1 compute | 2 3 loaders | 4 output store | 5 exits at once | 6 7 loaders
+//   NW = 4:  0..3 compute | 4..7 loaders (each compute wave shares with one loader; no output wave)
+__host__ __device__ constexpr int scan_waves(int nw) { return nw == 1 ? 6 : 8; }
+
+// compile-time loop: f(std::integral_constant<int, I>{}) for I = B .. E - 1
+template <int B, int E, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (B < E) {
+        f(std::integral_constant<int, B>{});
+        static_for<B + 1, E>(f);
+    }
+}
+
+// keeps the computation of x at this point of the program
+__device__ __forceinline__ void pin_regs(bf16x8& x) {
+    typedef __attribute__((ext_vector_type(4))) int i32x4;
+    i32x4 t = __builtin_bit_cast(i32x4, x);
+    asm volatile("" : "+v"(t));
+    x = __builtin_bit_cast(bf16x8, t);
+}
+
+// Order of the MFMAs of one chunk in the scan's compute wave, and where its side work goes.
+//
+// MFMAs ("ops"): O^T = S0^T q^T (NQF) | V~ = U + W~ S0 (NWF) | S += k^T V~' (NKF) | O^T += V~^T P^T (6).  The
+// third group runs token slabs 0, 1 of every key tile before slabs 2, 3, so that the second token tile of V~,
+// finished last, is needed late.
+//
+// Everything else (conversion of U, decay of the state, bf16 repacking of V~ and of the new state, the row scales,
+// hand-over of the output) is cut into pieces of four to six vector instructions.  A piece has a window: the first
+// op at which its inputs exist (an MFMA result is taken two ops after the MFMA was issued) and the op that needs
+// its result.  A lone wave issues an instruction every four to five cycles and an MFMA occupies the matrix pipe
+// for 33, so more than about six instructions between two MFMAs idle the pipe: the pieces are spread one per op,
+// earliest deadline first, as far as their windows allow.
+template <int K>
+struct ScanScheduleRules {
+    static constexpr int KD = K / 32, KS16 = K / 16;
+    static constexpr int NQF = 2 * KS16, NWF = 2 * KS16, NKF = 4 * KD, NPF = 6;
+    static constexpr int NOPS = NQF + NWF + NKF + NPF;
+    static constexpr int LA = 6;
+    static constexpr int OP_W = NQF, OP_K = NQF + NWF, OP_P = OP_K + NKF, OP_BAR = NOPS - LA;
+    static constexpr int KS_AHEAD = 2;  // the row scales of k are read this many ops before their piece
+    static_assert(OP_BAR >= OP_P, "q's scales, the decay and k's scales of this chunk are used before the barrier");
+
+    // op j of the third group -> key tile, token slab
+    static constexpr int k_tile(int j) { return (j % (2 * KD)) / 2; }
+    static constexpr int k_slab(int j) { return 2 * (j / (2 * KD)) + j % 2; }
+
+    // pieces: U conversion (4 elements) | output hand-over (half a tile) | q row scale (4 registers) | decay
+    // (4 registers) | scaled V~ (half a fragment) | plain V~ (a fragment) | new state (a fragment)
+    static constexpr int N_UC = 8, N_OUT = 4, N_AS = 8, N_DEC = 4 * KD, N_VS = 8, N_VB = 4, N_SB = 2 * KD;
+    static constexpr int P_UC = 0, P_OUT = P_UC + N_UC, P_AS = P_OUT + N_OUT, P_DEC = P_AS + N_AS, P_VS = P_DEC + N_DEC,
+                         P_VB = P_VS + N_VS, P_SB = P_VB + N_VB, NPIECES = P_SB + N_SB;
+
+    struct Window {
+        int first, end;  // the piece runs before the MFMA of an op in [first, end)
+    };
+    static constexpr Window window(int pc) {
+        if (pc < P_OUT) return {0, OP_W + KS16 * ((pc - P_UC) / 4)};  // accv[tt] is free since the last chunk's packs
+        if (pc < P_AS) {  // tile 0: this chunk's, after its two P ops; tile 1: the previous chunk's, before q overwrites it
+            return (pc - P_OUT) / 2 == 0 ? Window{OP_P + 3, NOPS} : Window{1, KS16};
+        }
+        if (pc < P_DEC) {
+            const int tt = (pc - P_AS) / 4;
+            const int end = OP_P + 2 * tt;
+            return {KS16 * (tt + 1) + 1, end < OP_BAR ? end : OP_BAR};
+        }
+        if (pc < P_VS) return {0, OP_K + 2 * ((pc - P_DEC) / 4)};
+        if (pc < P_VB) {
+            const int x = (pc - P_VS) / 2;
+            return {OP_W + KS16 * (x / 2 + 1) + 1, x < 2 ? OP_K + x : OP_K + NKF / 2 + (x - 2)};
+        }
+        if (pc < P_SB) return {OP_W + KS16 * ((pc - P_VB) / 2 + 1) + 1, OP_P};
+        return {OP_K + NKF / 2 + 2 * ((pc - P_SB) / 2) + 3, NOPS};
+    }
+
+    struct Table {
+        int op[NPIECES];
+        bool ok;
+    };
+    static constexpr Table make() {
+        Table t{};
+        bool done[NPIECES] = {};
+        int left = NPIECES;
+        t.ok = true;
+        for (int op = 0; op < NOPS; op++) {
+            const int quota = (left + (NOPS - op) - 1) / (NOPS - op);
+            for (int n = 0;; n++) {
+                int best = -1;
+                for (int pc = 0; pc < NPIECES; pc++)
+                    if (!done[pc] && window(pc).first <= op && (best < 0 || window(pc).end < window(best).end)) best = pc;
+                if (best < 0) break;
+                if (n >= quota && window(best).end > op + 1) break;
+                if (window(best).end <= op) t.ok = false;  // window missed
+                t.op[best] = op, done[best] = true, left--;
+            }
+        }
+        if (left != 0) t.ok = false;
+        // a scale register (ring of four) is refilled only after the piece four places earlier has used it
+        for (int i = 4; i < N_VS; i++)
+            if (t.op[P_VS + i] - KS_AHEAD <= t.op[P_VS + i - 4]) t.ok = false;
+        for (int i = 0; i < N_VS; i++)
+            if (t.op[P_VS + i] - KS_AHEAD < 0) t.ok = false;
+        return t;
+    }
+};
+
+template <int K>
+struct ScanSchedule : ScanScheduleRules<K> {
+    static constexpr typename ScanScheduleRules<K>::Table TABLE = ScanScheduleRules<K>::make();
+    static_assert(TABLE.ok, "no placement of the side work satisfies the windows");
+    static constexpr int op_of(int pc) { return TABLE.op[pc]; }
+};
+
 template <int K, int NW>
-__global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void chunk_scan32_kernel(const ChunkParams p) {
+__global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(const ChunkParams p) {
     constexpr int NL = SCAN_LOADERS;
     // a separate wave writes the output (see below); with four compute waves the LDS has no room for its staging
     constexpr bool OS = NW < 4;
@@ -594,8 +719,11 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
     const int id = blockIdx.x;
     const int xcd = id % 8, rest = id / 8;
     const int vgroup = rest % p.scan_groups;
-    const int chain = (rest / p.scan_groups) * 8 + xcd;
-    if (chain >= p.N * p.H) return;  // whole workgroup
+    // XCD x takes the chains x * per_xcd .. : consecutive chains are different heads, whose rows of q, k and o
+    // fall on different channels of the XCD's L2 (the rows of one head lie a multiple of 2 KiB apart)
+    const int per_xcd = (p.N * p.H + 7) / 8;
+    const int chain = xcd * per_xcd + rest / p.scan_groups;
+    if (rest / p.scan_groups >= per_xcd || chain >= p.N * p.H) return;  // whole workgroup
     const int n = chain / p.H, h = chain % p.H;
 
     int slot_begin, slot_end;
@@ -616,7 +744,11 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
     auto ostage_at = [&](int w, int parity, int row, int piece) -> uint8_t* {
         return ostage + ((w * 2 + parity) * C + row) * 64 + ((piece ^ ((row >> 2) & 3)) << 4);
     };
-    if (OS && wave == NW + NL) {
+    // role of this wave (see scan_waves)
+    const bool is_store = OS && wave == 4;
+    const bool is_loader = NW == 4 ? wave >= 4 : NW == 2 ? (wave == 2 || wave == 3 || wave >= 6) : (wave >= 1 && wave != 4);
+    if (NW == 2 && wave == 5) return;
+    if (is_store) {
         // ------------------------------ output store ------------------------------
         // The compute waves leave the bf16 output tile of chunk c in LDS while they work on chunk c + 1; this
         // wave writes it out after the next barrier.  A store that waits for queue space then stalls here and
@@ -647,11 +779,12 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
         if (nchunks > 0) flush(nchunks - 1);
         return;
     }
-    if (wave >= NW) {
+    if (is_loader) {
         // ------------------------------ loader ------------------------------
         // fragment f of the stage: f < SHARED_FRAGS comes from the head of the record, the rest from
         // this workgroup's slice of the U block
-        const int lw = __builtin_amdgcn_readfirstlane(wave - NW);  // wave-uniform: unit numbers and bases stay scalar
+        // loader number 0..3, wave-uniform: unit numbers and bases stay scalar
+        const int lw = __builtin_amdgcn_readfirstlane(NW == 4 ? wave - 4 : NW == 2 ? (wave < 4 ? wave - 2 : wave - 4) : (wave < 4 ? wave - 1 : 3));
         // Slots 0 .. NF - 1 of this wave move fragments lw * NF + (rotated slot), slots NF .. NLOAD - 1 move 1 KiB
         // pieces of the q rows; a surplus fragment slot repeats the last fragment.  Which kind a slot is, is known
         // at compile time, so there is no branch in these loops (a branch makes the compiler wait for every load
@@ -777,24 +910,21 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
     bf16_t* og = p.o + b * p.o_stride_b + (seq_t0 + l32) * p.o_stride_t + (int64_t)h * p.o_stride_h + 32 * tn + 8 * lh;
     const int64_t og_step = (int64_t)C * p.o_stride_t;
 
-    // MFMA schedule of one chunk: W~ (NWF) | q (NQF) | K~^T (NKF) | P (6).
-    // Everything else a chunk needs (decay of the state, bf16 repacking of V~ and of the new state, the row
-    // scale of q S0, conversion of the next U, hand-over of the previous chunk's output) is cut into pieces
-    // that sit between MFMAs whose operands do not depend on them, so the matrix pipe stays fed by this one wave.
-    constexpr int NOPS = NWF + NQF + NKF + NPF;
-    constexpr int LA = 6;  // LDS reads are issued this many MFMAs ahead of their use
-    constexpr int OP_Q = NWF, OP_K = NWF + NQF, OP_P = NWF + NQF + NKF, OP_BAR = NOPS - LA;
-    static_assert(OP_BAR >= OP_K, "the barrier must come after the reads of the W~ fragments and of q");
+    // MFMA schedule of one chunk: q (NQF) | W~ (NWF) | k^T (NKF) | P (6); the side work sits between the MFMAs
+    // at the ops ScanSchedule<K> assigns.
+    typedef ScanSchedule<K> SCH;
+    constexpr int NOPS = SCH::NOPS, OP_W = SCH::OP_W, OP_K = SCH::OP_K, OP_P = SCH::OP_P, OP_BAR = SCH::OP_BAR;
+    constexpr int LA = SCH::LA;  // LDS reads are issued this many MFMAs ahead of their use
     const int l16 = lane % 16, g16 = l32 / 16;
-    auto lds_frag = [&](const uint8_t* st, int op) -> bf16x8 {
-        if (op >= OP_Q && op < OP_K) {  // q, token tile tt, 16-column slab s: 8 consecutive columns per lane half
-            const int j = op - OP_Q, s = j % KS16, tt = j / KS16;
+    auto lds_frag = [&](const uint8_t* st, auto opc) -> bf16x8 {
+        constexpr int op = decltype(opc)::value;
+        if constexpr (op < OP_W) {  // q, token tile tt, 16-column slab s: 8 consecutive columns per lane half
+            constexpr int s = op % KS16, tt = op / KS16;
             return *reinterpret_cast<const bf16x8*>(st + Q_OFF + (32 * tt + l32) * QLD + (16 * s + 8 * lh) * 2);
-        }
-        if (op >= OP_K && op < OP_P) {
+        } else if constexpr (op >= OP_K && op < OP_P) {
             // k^T, key tile td (rows in state order), token slab s: tokens 16 s + 4 h + 0..3 and 16 s + 8 + 4 h + 0..3
             // of key column 32 td + slice_col(l32), through the transposing LDS load
-            const int j = op - OP_K, s = j % 4, td = j / 4;
+            constexpr int s = SCH::k_slab(op - OP_K), td = SCH::k_tile(op - OP_K);
             const bf16_t* km = reinterpret_cast<const bf16_t*>(st + K_OFF);
             const bf16x4 a = lds_read_tr4x16<true>(km, QLD / 2, 16 * s + 4 * lh, 32 * td + 16 * g16, l16);
             const bf16x4 b = lds_read_tr4x16<true>(km, QLD / 2, 16 * s + 8 + 4 * lh, 32 * td + 16 * g16, l16);
@@ -802,9 +932,10 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
 #pragma unroll
             for (int e = 0; e < 4; e++) r[e] = a[e], r[4 + e] = b[e];
             return r;
+        } else {
+            constexpr int f = op < OP_K ? op - OP_W : NWF + (op - OP_P);  // W~ | P are contiguous in the stage
+            return reinterpret_cast<const bf16x8*>(st)[f * WAVE + lane];
         }
-        const int f = op < OP_Q ? op : op - NQF - NKF;  // W~ | P are contiguous in the stage
-        return reinterpret_cast<const bf16x8*>(st)[f * WAVE + lane];
     };
     auto lds_u = [&](const uint8_t* st, int i) -> bf16x8 {
         return reinterpret_cast<const bf16x8*>(st + SHARED_BYTES)[(wave * 4 + i) * WAVE + lane];
@@ -814,11 +945,8 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
 
     f32x16 accv[2], acco[2];
     bf16x8 sb[KS16], vb[4], vbs[4], ur[4], fnext[LA];  // vbs: V~ with its rows scaled like K~'s, for the state update
+    f32x4 ksr[4];                                      // row scales of k on their way to the pieces that use them
     float egc, qsc[2];  // e^{gamma_C} and this lane's two row scales of q (tokens l32 and 32 + l32)
-#pragma unroll
-    for (int tt = 0; tt < 2; tt++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) acco[tt][r] = 0.f;
 
     __syncthreads();  // stage[0] holds record 0
 
@@ -827,16 +955,11 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
     for (int i = 0; i < 4; i++) ur[i] = lds_u(stage[0], i);
     egc = lds_eg(stage[0]);
     qsc[0] = lds_qs(stage[0], 0), qsc[1] = lds_qs(stage[0], 1);
-#pragma unroll
-    for (int i = 0; i < LA; i++) fnext[i] = lds_frag(stage[0], i);
+    static_for<0, LA>([&](auto i) { fnext[decltype(i)::value] = lds_frag(stage[0], i); });
 #pragma unroll
     for (int s = 0; s < KS16; s++) sb[s] = pack8_16(S[s / 2], s % 2, 1.f);
-#pragma unroll
-    for (int tt = 0; tt < 2; tt++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) accv[tt][r] = (float)ur[2 * tt + r / 8][r % 8];
 
-    int valid_prev = 0;  // tokens of the previous chunk, whose output is still in acco
+    int valid_prev = 0;  // tokens of the previous chunk, the second half of whose output is still in acco[1]
     for (int c = 0; c < nchunks; c++) {
         const uint8_t* st = stage[c & 1];
         const uint8_t* stn = stage[(c + 1) & 1];
@@ -846,82 +969,89 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
         for (int i = 0; i < LA; i++) fr[i] = fnext[i];
         __builtin_amdgcn_sched_barrier(0);
 
+        // one piece of side work (pc: index into ScanSchedule's piece list)
+        auto run_piece = [&](auto pcc) {
+            constexpr int pc = decltype(pcc)::value;
+            if constexpr (pc >= SCH::P_UC && pc < SCH::P_UC + SCH::N_UC) {
+                // U of this chunk -> fp32 accumulators: 4 elements of ur[q]
+                constexpr int i = pc - SCH::P_UC, q = i / 2, hh = i % 2;
 #pragma unroll
-        for (int op = 0; op < NOPS; op++) {
+                for (int e = 0; e < 4; e++) accv[q / 2][8 * (q % 2) + 4 * hh + e] = (float)ur[q][4 * hh + e];
+            } else if constexpr (pc >= SCH::P_OUT && pc < SCH::P_OUT + SCH::N_OUT) {
+                // output tile tt, registers 8 half .. 8 half + 7: tile 0 belongs to this chunk (its P terms are
+                // complete), tile 1 to the previous one
+                constexpr int i = pc - SCH::P_OUT, tt = i / 2, half = i % 2;
+                if constexpr (tt == 0) {
+                    if (OS) {
+                        *reinterpret_cast<bf16x8*>(ostage_at(wave, c & 1, l32, 2 * half + lh)) = pack8_16(acco[0], half, 1.f);
+                    } else if (l32 < valid) {
+                        *reinterpret_cast<bf16x8*>(og + 16 * half) = pack8_16(acco[0], half, 1.f);
+                    }
+                } else {
+                    if (OS) {
+                        if (c > 0)
+                            *reinterpret_cast<bf16x8*>(ostage_at(wave, (c - 1) & 1, 32 + l32, 2 * half + lh)) =
+                                pack8_16(acco[1], half, 1.f);
+                    } else if (32 + l32 < valid_prev) {
+                        *reinterpret_cast<bf16x8*>(og - og_step + (int64_t)32 * p.o_stride_t + 16 * half) =
+                            pack8_16(acco[1], half, 1.f);
+                    }
+                }
+            } else if constexpr (pc >= SCH::P_AS && pc < SCH::P_AS + SCH::N_AS) {
+                // O^T = (q S0)^T so far: its columns (tokens) take the row scale of q before the P terms are added
+                constexpr int i = pc - SCH::P_AS, tt = i / 4, q4 = i % 4;
+#pragma unroll
+                for (int e = 0; e < 4; e++) acco[tt][4 * q4 + e] *= qsc[tt];
+            } else if constexpr (pc >= SCH::P_DEC && pc < SCH::P_DEC + SCH::N_DEC) {
+                // decay of the state (its bf16 copy for this chunk is already in sb)
+                constexpr int i = pc - SCH::P_DEC, td = i / 4, q4 = i % 4;
+#pragma unroll
+                for (int e = 0; e < 4; e++) S[td][4 * q4 + e] *= egc;
+            } else if constexpr (pc >= SCH::P_VS && pc < SCH::P_VS + SCH::N_VS) {
+                // V~ as operand of k^T V~: each row (token) scaled by e^{gamma_C - gamma} / |k|; half a fragment
+                constexpr int i = pc - SCH::P_VS, x = i / 2, sub = i % 2, tt = x / 2, half = x % 2;
+#pragma unroll
+                for (int e = 0; e < 4; e++) vbs[x][4 * sub + e] = (bf16_t)(accv[tt][8 * half + 4 * sub + e] * ksr[i % 4][e]);
+            } else if constexpr (pc >= SCH::P_VB && pc < SCH::P_VB + SCH::N_VB) {
+                constexpr int i = pc - SCH::P_VB;  // V~ as operand of P V~
+                vb[i] = pack8_16(accv[i / 2], i % 2, 1.f);
+            } else {
+                // the new state tile as operand of the next chunk; pinned here, or the compiler moves all of them
+                // behind the last MFMA of the loop
+                constexpr int i = pc - SCH::P_SB;
+                sb[i] = pack8_16(S[i / 2], i % 2, 1.f);
+                pin_regs(sb[i]);
+            }
+        };
+
+        static_for<0, NOPS>([&](auto opc) {
+            constexpr int op = decltype(opc)::value;
             // ---- operand reads: this record until the barrier, the next one after it ----
-            if (op + LA < NOPS) fr[op + LA] = lds_frag(st, op + LA);
-            if (op == OP_BAR) {
+            if constexpr (op + LA < NOPS) fr[op + LA] = lds_frag(st, std::integral_constant<int, (op + LA < NOPS ? op + LA : 0)>{});
+            if constexpr (op == OP_BAR) {
                 __syncthreads();  // this wave is done with record c; record c + 1 is in the other half
 #pragma unroll
                 for (int i = 0; i < 4; i++) ur[i] = lds_u(stn, i);
                 egc = lds_eg(stn);
-                qsc[0] = lds_qs(stn, 0), qsc[1] = lds_qs(stn, 1);  // this chunk's scales were applied before OP_P
+                qsc[0] = lds_qs(stn, 0), qsc[1] = lds_qs(stn, 1);  // this chunk's scales were applied before the barrier
             }
-            if (op >= OP_BAR) fnext[op - OP_BAR] = lds_frag(stn, op - OP_BAR);
+            if constexpr (op >= OP_BAR) fnext[op >= OP_BAR ? op - OP_BAR : 0] = lds_frag(stn, std::integral_constant<int, (op >= OP_BAR ? op - OP_BAR : 0)>{});
+            // the row scales of k, two ops ahead of the piece that uses them
+            static_for<0, SCH::N_VS>([&](auto ic) {
+                constexpr int i = decltype(ic)::value, x = i / 2, sub = i % 2;
+                if constexpr (SCH::op_of(SCH::P_VS + i) - SCH::KS_AHEAD == op)
+                    ksr[i % 4] = *reinterpret_cast<const f32x4*>(st + KS_OFF + (16 * x + 8 * sub + 4 * lh) * 4);
+            });
 
             // ---- side work ----
-            if (op >= 1 && op <= 4) {  // output of the previous chunk: tile (op-1)/2, registers 8 half .. 8 half + 7
-                const int tt = (op - 1) / 2, half = (op - 1) % 2;
-                if (OS) {
-                    if (c > 0)
-                        *reinterpret_cast<bf16x8*>(ostage_at(wave, (c - 1) & 1, 32 * tt + l32, 2 * half + lh)) =
-                            pack8_16(acco[tt], half, 1.f);
-                } else if (32 * tt + l32 < valid_prev) {
-                    *reinterpret_cast<bf16x8*>(og - og_step + (int64_t)(32 * tt) * p.o_stride_t + 16 * half) =
-                        pack8_16(acco[tt], half, 1.f);
-                }
-            }
-            if (op < NWF) {  // decay of the state (its bf16 copy for this chunk is already in sb)
-                constexpr int PER = (KD * 16) / NWF;
-#pragma unroll
-                for (int i = 0; i < PER; i++) S[(op * PER + i) / 16][(op * PER + i) % 16] *= egc;
-            }
-            // V~ rows 0..31 are complete after op KS16 - 1, rows 32..63 after op NWF - 1: as operands, plain for
-            // P V~ and with each row (token) scaled by e^{gamma_C - gamma} / |k| for k^T V~
-            auto pack_rows = [&](int tt, int half) {
-                vb[2 * tt + half] = pack8_16(accv[tt], half, 1.f);
-                const f32x4 s0 = *reinterpret_cast<const f32x4*>(st + KS_OFF + (32 * tt + 16 * half + 4 * lh) * 4);
-                const f32x4 s1 = *reinterpret_cast<const f32x4*>(st + KS_OFF + (32 * tt + 16 * half + 8 + 4 * lh) * 4);
-                bf16x8 r;
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    r[e] = (bf16_t)(accv[tt][8 * half + e] * s0[e]);
-                    r[4 + e] = (bf16_t)(accv[tt][8 * half + 4 + e] * s1[e]);
-                }
-                vbs[2 * tt + half] = r;
-            };
-            if (op == KS16 + 2) pack_rows(0, 0);
-            if (op == KS16 + 3) pack_rows(0, 1);
-            if (op == OP_Q + 2) pack_rows(1, 0);
-            if (op == OP_Q + 3) pack_rows(1, 1);
-            if (op >= OP_K + 5) {  // new state tile td is complete after K~^T op 4 td + 3: its two slabs as operands
-                const int j = op - OP_K - 5;
-                if (j % 4 < 2 && j / 4 < KD) sb[2 * (j / 4) + j % 4] = pack8_16(S[j / 4], j % 4, 1.f);
-            }
-            // O^T = (q S0)^T so far: its columns (tokens) take the row scale of q before the P terms are added
-            if (op >= OP_Q + KS16 + 2 && op < OP_Q + KS16 + 6) {
-                const int q4 = op - (OP_Q + KS16 + 2);
-#pragma unroll
-                for (int i = 0; i < 4; i++) acco[0][4 * q4 + i] *= qsc[0];
-            }
-            if (op >= OP_K + 2 && op < OP_K + 6) {
-                const int q4 = op - (OP_K + 2);
-#pragma unroll
-                for (int i = 0; i < 4; i++) acco[1][4 * q4 + i] *= qsc[1];
-            }
-            if (op >= NOPS - 4) {  // U of the next chunk -> fp32 accumulators (V~ of this chunk lives on in vb)
-                const int q = op - (NOPS - 4);
-#pragma unroll
-                for (int i = 0; i < 8; i++) accv[q / 2][8 * (q % 2) + i] = (float)ur[q][i];
-            }
+            static_for<0, SCH::NPIECES>([&](auto pcc) {
+                if constexpr (SCH::op_of(decltype(pcc)::value) == op) run_piece(pcc);
+            });
 
             // ---- the MFMA ----
-            if (op < OP_Q) {  // V~ = U + W~ S0, fragment (tt, s) = op
-                const int s = op % KS16, tt = op / KS16;
-                accv[tt] = mfma32_bf16(fr[op], sb[s], accv[tt]);
-            } else if (op < OP_K) {  // O^T = (q S0)^T, scaled per token further down
-                const int j = op - OP_Q, s = j % KS16, tt = j / KS16;
-                if (s == 0) {
+            if constexpr (op < OP_W) {  // O^T = (q S0)^T, scaled per token by a later piece
+                constexpr int s = op % KS16, tt = op / KS16;
+                if constexpr (s == 0) {
                     f32x16 zero;
 #pragma unroll
                     for (int r = 0; r < 16; r++) zero[r] = 0.f;
@@ -929,34 +1059,33 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
                 } else {
                     acco[tt] = mfma32_bf16(sb[s], fr[op], acco[tt]);
                 }
-            } else if (op < OP_P) {  // S = e^{gamma_C} S + k^T (row-scaled V~), fragment (td, s)
-                const int j = op - OP_K, s = j % 4, td = j / 4;
+            } else if constexpr (op < OP_K) {  // V~ = U + W~ S0, fragment (tt, s)
+                constexpr int j = op - OP_W, s = j % KS16, tt = j / KS16;
+                accv[tt] = mfma32_bf16(fr[op], sb[s], accv[tt]);
+            } else if constexpr (op < OP_P) {  // S = e^{gamma_C} S + k^T (row-scaled V~), fragment (td, s)
+                constexpr int s = SCH::k_slab(op - OP_K), td = SCH::k_tile(op - OP_K);
                 S[td] = mfma32_bf16(fr[op], vbs[s], S[td]);
             } else {  // O^T += V~^T P^T; P[i < 32][j >= 32] = 0 is skipped
-                const int j = op - OP_P;
-                const int tt = j < 2 ? 0 : 1, s = j < 2 ? j : j - 2;
+                constexpr int j = op - OP_P;
+                constexpr int tt = j < 2 ? 0 : 1, s = j < 2 ? j : j - 2;
                 acco[tt] = mfma32_bf16(vb[s], fr[op], acco[tt]);
             }
             __builtin_amdgcn_sched_barrier(0);
-        }
+        });
         valid_prev = valid;
         og += og_step;
     }
 
-    // output of the last chunk
+    // the second half of the output of the last chunk
 #pragma unroll
-    for (int tt = 0; tt < 2; tt++)
-#pragma unroll
-        for (int half = 0; half < 2; half++) {
-            if (OS) {
-                if (nchunks > 0)
-                    *reinterpret_cast<bf16x8*>(ostage_at(wave, (nchunks - 1) & 1, 32 * tt + l32, 2 * half + lh)) =
-                        pack8_16(acco[tt], half, 1.f);
-            } else if (32 * tt + l32 < valid_prev) {
-                *reinterpret_cast<bf16x8*>(og - og_step + (int64_t)(32 * tt) * p.o_stride_t + 16 * half) =
-                    pack8_16(acco[tt], half, 1.f);
-            }
+    for (int half = 0; half < 2; half++) {
+        if (OS) {
+            if (nchunks > 0)
+                *reinterpret_cast<bf16x8*>(ostage_at(wave, (nchunks - 1) & 1, 32 + l32, 2 * half + lh)) = pack8_16(acco[1], half, 1.f);
+        } else if (32 + l32 < valid_prev) {
+            *reinterpret_cast<bf16x8*>(og - og_step + (int64_t)32 * p.o_stride_t + 16 * half) = pack8_16(acco[1], half, 1.f);
         }
+    }
     if (OS) __syncthreads();
 
     if (p.ht != nullptr) {
@@ -972,8 +1101,9 @@ __global__ __launch_bounds__((NW + SCAN_LOADERS + (NW < 4 ? 1 : 0)) * WAVE) void
 // ------------------------------------------------------------------------------------------
 template <int K>
 static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int num_cus) {
-    const int64_t items = (int64_t)p.TC * p.H;
-    const int grid_prep = (int)(items < 2 * (int64_t)num_cus ? items : 2 * (int64_t)num_cus);  // two workgroups per CU
+    const int64_t items = (int64_t)((p.TC + 7) / 8) * 8 * p.H;  // a multiple of 8, see the kernel
+    const int64_t cap = (int64_t)(2 * num_cus + 7) / 8 * 8;      // two workgroups per CU
+    const int grid_prep = (int)(items < cap ? items : cap);
     hipLaunchKernelGGL((chunk_prepare32_kernel<K>), dim3(grid_prep), dim3(PREP_THREADS), 0, stream, p);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
     if (events != nullptr) (void)hipEventRecord(events[2], stream);
@@ -988,9 +1118,9 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     while (nw < 4 && vtiles % (2 * nw) == 0 && chains * (vtiles / nw) > (int64_t)num_cus) nw *= 2;
     p.scan_groups = vtiles / nw;
     const dim3 grid((unsigned)(chains8 * p.scan_groups));
-    if (nw == 4) hipLaunchKernelGGL((chunk_scan32_kernel<K, 4>), grid, dim3((4 + SCAN_LOADERS) * WAVE), 0, stream, p);
-    else if (nw == 2) hipLaunchKernelGGL((chunk_scan32_kernel<K, 2>), grid, dim3((2 + SCAN_LOADERS + 1) * WAVE), 0, stream, p);
-    else hipLaunchKernelGGL((chunk_scan32_kernel<K, 1>), grid, dim3((1 + SCAN_LOADERS + 1) * WAVE), 0, stream, p);
+    if (nw == 4) hipLaunchKernelGGL((chunk_scan32_kernel<K, 4>), grid, dim3(scan_waves(4) * WAVE), 0, stream, p);
+    else if (nw == 2) hipLaunchKernelGGL((chunk_scan32_kernel<K, 2>), grid, dim3(scan_waves(2) * WAVE), 0, stream, p);
+    else hipLaunchKernelGGL((chunk_scan32_kernel<K, 1>), grid, dim3(scan_waves(1) * WAVE), 0, stream, p);
     return (int)hipGetLastError();
 }
 

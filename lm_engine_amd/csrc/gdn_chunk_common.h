@@ -78,6 +78,10 @@ struct ChunkCoord {
 
 __device__ __forceinline__ ChunkCoord locate_chunk(const ChunkParams& p, int slot) {
     ChunkCoord cc;
+    if (slot >= p.TC) {  // past the last slot (the item grid of prepare is rounded up): nothing there
+        cc.n = 0, cc.b = 0, cc.t0 = 0, cc.len = 0;
+        return cc;
+    }
     if (p.cu_seqlens == nullptr) {
         cc.n = slot / p.NT;
         const int c = slot - cc.n * p.NT;
