@@ -620,7 +620,7 @@ int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events) 
     p.beta_dtype = a.beta_dtype;
     p.l2norm = (a.flags & GDN_FLAG_L2NORM) ? 1 : 0;
     p.scale = a.scale;
-    p.rec_bytes = r.bytes, p.off_qs = r.off_qs, p.off_kt = r.off_kt, p.off_ks = r.off_ks, p.off_p = r.off_p, p.off_u = r.off_u;
+    p.rec_bytes = r.bytes, p.off_qs = r.off_qs, p.off_kt = r.off_kt, p.off_ks = r.off_ks, p.off_cs = r.off_cs, p.off_p = r.off_p, p.off_u = r.off_u;
     p.off_eg = r.off_eg;
     p.scan_groups = 1;
 

@@ -85,8 +85,6 @@ __device__ __forceinline__ void split_hi_lo(float x, bf16_t& hi, bf16_t& lo) {
 template <int K>
 __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const ChunkParams p) {
     constexpr int LDK = K + 8;  // bf16 elements per LDS row of K / Q
-    constexpr int VP = 128;     // columns of V staged per pass
-    constexpr int LDV = VP + 8;
     constexpr int LDA = C + 4;  // fp32 elements per LDS row of A / T
     constexpr int LDT = 36;     // fp32 elements per row of the 32 x 32 transposed blocks
     constexpr int LDM = 20;     // fp32 elements per row of a 16 x 16 scratch block
@@ -96,20 +94,17 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
     constexpr int RPP = PREP_THREADS / CPR;  // rows per pass of the K / Q copy
     constexpr int NPASS = C / RPP;
     constexpr int QT_BYTES = (C * LDK * 2 > C * LDA * 4) ? C * LDK * 2 : C * LDA * 4;
-    constexpr int AV_BYTES = (C * LDV * 2 > C * LDA * 4) ? C * LDV * 2 : C * LDA * 4;
 
     __shared__ __attribute__((aligned(16))) bf16_t sK[C * LDK];
     __shared__ __attribute__((aligned(16))) uint8_t sQT[QT_BYTES];  // Q (bf16), then T (fp32)
-    __shared__ __attribute__((aligned(16))) uint8_t sAV[AV_BYTES];  // A (fp32), then V (bf16)
+    __shared__ __attribute__((aligned(16))) float sA[C * LDA];
     __shared__ __attribute__((aligned(16))) float sTtA[32 * LDT];   // transpose of the top-left 32 x 32 of T
     __shared__ __attribute__((aligned(16))) float sTt2[16 * LDM];   // transpose of diagonal block 2 of T
     __shared__ __attribute__((aligned(16))) float sMt[2 * 16 * LDM + 32 * LDT];  // transposed products
     __shared__ __attribute__((aligned(16))) float s_gam[C], s_beta[C], s_ssk[C], s_ssq[C];
-    __shared__ __attribute__((aligned(16))) float s_rk[C], s_rq[C], s_cw[C], s_ks[C], s_qs[C];
+    __shared__ __attribute__((aligned(16))) float s_rk[C], s_rq[C];
     bf16_t* const sQ = reinterpret_cast<bf16_t*>(sQT);
     float* const sT = reinterpret_cast<float*>(sQT);
-    float* const sA = reinterpret_cast<float*>(sAV);
-    bf16_t* const sV = reinterpret_cast<bf16_t*>(sAV);
     float* const sMtB = sMt + 2 * 16 * LDM;
 
     const int tid = threadIdx.x;
@@ -122,7 +117,7 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
     const int64_t items = (int64_t)((p.TC + 7) / 8) * 8 * p.H;
 
     // ---- register prefetch of one item's inputs ----
-    bf16x8 kx[NPASS], qx[NPASS], vx[C * (VP / 8) / PREP_THREADS];
+    bf16x8 kx[NPASS], qx[NPASS];
     float gx = 0.f;
     uint32_t bx_raw = 0;  // beta of the prefetched item, raw bits: any arithmetic on it here would wait for every load in flight
     ChunkCoord ncc;  // coordinates of the prefetched item
@@ -138,8 +133,6 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
     const uint32_t kq_piece = tid % CPR, kq_row0 = tid / CPR;
     const uint32_t k_lane_off = kq_row0 * (uint32_t)p.k_stride_t + kq_piece * 8;
     const uint32_t q_lane_off = kq_row0 * (uint32_t)p.q_stride_t + kq_piece * 8;
-    const uint32_t v_piece = tid % (VP / 8), v_row0 = tid / (VP / 8);
-    const uint32_t v_lane_off = v_row0 * (uint32_t)p.v_stride_t + v_piece * 8;
     const int lane0 = tid % WAVE;
     auto prefetch_kq = [&]() {
         const bf16_t* kg = p.k + ncc.b * p.k_stride_b + ncc.t0 * p.k_stride_t + (int64_t)nh * p.k_stride_h;
@@ -166,22 +159,10 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
             }
         }
     };
-    auto prefetch_v = [&]() {  // first pass of V (columns 0 .. min(V, VP))
-        const bf16_t* vg = p.v + ncc.b * p.v_stride_b + ncc.t0 * p.v_stride_t + (int64_t)nh * p.v_stride_h;
-#pragma unroll
-        for (int it = 0; it < C * (VP / 8) / PREP_THREADS; it++) {
-            const int row = v_row0 + it * (PREP_THREADS / (VP / 8));
-            vx[it] = bf16x8{};
-            if (row < ncc.len && (int)v_piece * 8 < p.V)
-                vx[it] = *reinterpret_cast<const bf16x8*>(vg + (int64_t)(it * (PREP_THREADS / (VP / 8))) * p.v_stride_t + v_lane_off);
-        }
-    };
-
     int64_t w = blockIdx.x;
     if (w >= items) return;
     locate(w);
     prefetch_kq();
-    prefetch_v();
 
     for (; w < items; w += gridDim.x) {
         // Lane coordinates are re-derived in every iteration from a value the optimiser cannot see
@@ -237,10 +218,7 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
             locate(w + gridDim.x);
             prefetch_kq();
         }
-        if (len <= 0) {  // uniform over the workgroup
-            if (has_next) prefetch_v();
-            continue;
-        }
+        if (len <= 0) continue;  // uniform over the workgroup
         __syncthreads();  // #1
 
         if (tid < C) {
@@ -249,11 +227,12 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
             const float rq = p.l2norm ? rsqrtf(s_ssq[tid] + L2NORM_EPS) : 1.f;
             s_rk[tid] = rk;
             s_rq[tid] = rq;
-            s_cw[tid] = s_beta[tid] * __expf(gam) * rk;  // column scale of T for W
-            s_ks[tid] = __expf(gl - gam) * rk;           // row scale of K~
-            s_qs[tid] = __expf(gam) * p.scale * rq;      // row scale of Q~
-            reinterpret_cast<float*>(rec + p.off_qs)[tid] = s_qs[tid];
-            reinterpret_cast<float*>(rec + p.off_ks)[tid] = s_ks[tid];
+            // row scales the scan applies: to q S0, to the rows of V~ in the state update, to k S0 (none for
+            // the rows past the end of a short chunk: the scan reads some other token's k and v there)
+            const bool valid = tid < len;
+            reinterpret_cast<float*>(rec + p.off_qs)[tid] = __expf(gam) * p.scale * rq;
+            reinterpret_cast<float*>(rec + p.off_ks)[tid] = valid ? __expf(gl - gam) * rk : 0.f;
+            reinterpret_cast<float*>(rec + p.off_cs)[tid] = valid ? __expf(gam) * rk : 0.f;
             if (tid == 0) *reinterpret_cast<float*>(rec + p.off_eg) = __expf(gl);
         }
         __syncthreads();  // #2
@@ -421,106 +400,25 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
 #pragma unroll
             for (int e = 0; e < 4; e++) sT[(32 + 16 * ta + 4 * lq + e) * LDA + 16 * tb + l16] = -t[e];
         }
-        // A is dead: its region takes the first pass of V, whose registers then go for the next item
-        {
-            const int piece = tid % (VP / 8);
-#pragma unroll
-            for (int it = 0; it < C * (VP / 8) / PREP_THREADS; it++) {
-                const int row = tid / (VP / 8) + it * (PREP_THREADS / (VP / 8));
-                *reinterpret_cast<bf16x8*>(&sV[row * LDV + piece * 8]) = vx[it];
-            }
-            if (has_next) prefetch_v();
-        }
-        __syncthreads();  // #7: T and V complete
+        __syncthreads();  // #7: T complete
 
-        // T fragment for 32-row tile tt and 16-wide slab s (natural order j = 16 s + 8 h + e), columns scaled
-        auto t_frag = [&](int tt, int s, const float* colscale) -> bf16x8 {
-            const int i = 32 * tt + l32;
-            const int j0 = 16 * s + 8 * lh;
+        // ---- T diag(beta) as A operands of V~ = T' X: tiles (0, 0), (1, 0), (1, 1), two 16-token slabs each ----
+        // The reduction index (token j of X) runs in the order in which an accumulator tile of the scan hands its
+        // rows over as a B operand: lane half h supplies tokens 16 s + 4 h + 0..3 and 16 s + 8 + 4 h + 0..3.
+        for (int f = wave; f < 6; f += 4) {
+            const int ti = f < 2 ? 0 : 1, tj = f < 4 ? 0 : 1, sl = f % 2;
+            const int i = 32 * ti + l32, j0 = 32 * tj + 16 * sl + 4 * lh;
             const f32x4 t0 = *reinterpret_cast<const f32x4*>(&sT[i * LDA + j0]);
-            const f32x4 t1 = *reinterpret_cast<const f32x4*>(&sT[i * LDA + j0 + 4]);
-            const f32x4 c0 = *reinterpret_cast<const f32x4*>(&colscale[j0]);
-            const f32x4 c1 = *reinterpret_cast<const f32x4*>(&colscale[j0 + 4]);
+            const f32x4 t1 = *reinterpret_cast<const f32x4*>(&sT[i * LDA + j0 + 8]);
+            const f32x4 c0 = *reinterpret_cast<const f32x4*>(&s_beta[j0]);
+            const f32x4 c1 = *reinterpret_cast<const f32x4*>(&s_beta[j0 + 8]);
             bf16x8 r;
 #pragma unroll
             for (int e = 0; e < 4; e++) {  // sT holds the whole of T here: unit diagonal, zeros above it
                 r[e] = (bf16_t)(t0[e] * c0[e]);
                 r[4 + e] = (bf16_t)(t1[e] * c1[e]);
             }
-            return r;
-        };
-        // transposed operand: 8 consecutive tokens j = 16 s + 8 h + e of column 32 tile + l32 of a row-major matrix
-        auto tr_frag = [&](const bf16_t* m, int ld, int s, int tile, auto swap_tag) -> bf16x8 {
-            constexpr bool SW = decltype(swap_tag)::value;
-            const bf16x4 a = lds_read_tr4x16<SW>(m, ld, 16 * s + 8 * lh, 32 * tile + 16 * g16, l16);
-            const bf16x4 b = lds_read_tr4x16<SW>(m, ld, 16 * s + 8 * lh + 4, 32 * tile + 16 * g16, l16);
-            bf16x8 r;
-#pragma unroll
-            for (int e = 0; e < 4; e++) r[e] = a[e], r[4 + e] = b[e];
-            return r;
-        };
-
-        // ---- W^T = K^T (T diag(cw))^T, tile (T_d, T_tok): D[d][tok]; emitted negated ----
-        if (wave < KD) {
-            const int td = wave;
-            f32x16 acc[2];
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[0][r] = 0.f, acc[1][r] = 0.f;
-#pragma unroll
-            for (int s = 0; s < 4; s++) {
-                const bf16x8 kt = tr_frag(sK, LDK, s, td, std::true_type{});  // key columns in state-row order
-                if (s < 2) acc[0] = mfma32_bf16(kt, t_frag(0, s, s_cw), acc[0]);  // tokens < 32 only see j < 32
-                acc[1] = mfma32_bf16(kt, t_frag(1, s, s_cw), acc[1]);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            bf16x8* wf = reinterpret_cast<bf16x8*>(rec);
-#pragma unroll
-            for (int tt = 0; tt < 2; tt++)
-#pragma unroll
-                for (int s = 0; s < 2; s++) wf[(tt * KS16 + 2 * td + s) * WAVE + lane] = pack8_16(acc[tt], s, -1.f);
-        }
-
-        // ---- U = (T diag(beta)) V, tile (T_tok, T_n): D[tok][n]; emitted in accumulator layout ----
-        {
-            bf16x8 ta0[2], ta1[4];
-#pragma unroll
-            for (int s = 0; s < 2; s++) ta0[s] = t_frag(0, s, s_beta);
-#pragma unroll
-            for (int s = 0; s < 4; s++) ta1[s] = t_frag(1, s, s_beta);
-            for (int v0 = 0; v0 < p.V; v0 += VP) {
-                const int vcols = min(VP, p.V - v0);
-                if (v0 > 0) {  // later passes of a wide V are staged here, without prefetch
-                    __syncthreads();
-                    const bf16_t* vg = p.v + cc.b * p.v_stride_b + cc.t0 * p.v_stride_t + (int64_t)h * p.v_stride_h;
-                    const int cpr = vcols / 8;
-                    for (int idx = tid; idx < C * cpr; idx += PREP_THREADS) {
-                        const int row = idx / cpr, piece = idx % cpr;
-                        bf16x8 x = {};
-                        if (row < len) x = *reinterpret_cast<const bf16x8*>(vg + row * p.v_stride_t + v0 + piece * 8);
-                        *reinterpret_cast<bf16x8*>(&sV[row * LDV + piece * 8]) = x;
-                    }
-                    __syncthreads();
-                }
-                for (int tl = wave; tl < vcols / 32; tl += 4) {
-                    f32x16 acc[2];
-#pragma unroll
-                    for (int r = 0; r < 16; r++) acc[0][r] = 0.f, acc[1][r] = 0.f;
-#pragma unroll
-                    for (int s = 0; s < 4; s++) {
-                        const bf16x8 vb = tr_frag(sV, LDV, s, tl, std::true_type{});  // columns in the scan's slice order
-                        if (s < 2) acc[0] = mfma32_bf16(ta0[s], vb, acc[0]);
-                        acc[1] = mfma32_bf16(ta1[s], vb, acc[1]);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                    const int tn = v0 / 32 + tl;
-                    // four fragments of 1 KiB per tile, each one contiguous store of the wave (whole cache lines)
-                    bf16x8* uf = reinterpret_cast<bf16x8*>(rec + p.off_u) + (int64_t)tn * 4 * WAVE + lane;
-                    uf[0 * WAVE] = pack8_16(acc[0], 0, 1.f);
-                    uf[1 * WAVE] = pack8_16(acc[0], 1, 1.f);
-                    uf[2 * WAVE] = pack8_16(acc[1], 0, 1.f);
-                    uf[3 * WAVE] = pack8_16(acc[1], 1, 1.f);
-                }
-            }
+            reinterpret_cast<bf16x8*>(rec)[f * WAVE + lane] = r;
         }
         __syncthreads();  // #8: LDS is reused by the next item
     }
@@ -533,30 +431,28 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
 // waves, each owning a K x 32 slice of the fp32 state as MFMA accumulators, 4 loader waves and
 // (NW < 4) one output wave.
 //
-// Everything a chunk needs (the operand fragments W~, K~^T, P of its record, the U tiles of this
-// workgroup's columns, the chunk's rows of q from the caller's tensor, q's row scales and
-// e^{gamma_C}) goes through a double buffer in LDS: during chunk
-// c the loaders move record c + 1 global -> registers -> LDS and already have records c + 2 and
-// c + 3 in flight in a second register buffer.  One workgroup barrier per chunk hands the halves
-// over.  The memory instructions are kept out of the compute waves on purpose: a wave that
-// issues a load or a store while the CU's vector-memory queue is full stalls until there is
-// room, and with one compute wave per SIMD that stall is a stall of the matrix pipe.  (Measured:
-// one wave per CU that streams its own 58 KB per chunk needs ~4600 cycles per chunk, and the 4
-// output stores per chunk cost a compute wave 340 - 980 cycles.)
+// Per chunk, with S0 the state at its start (gamma, beta, T = (I + A)^-1 and P as in prepare):
+//     X   = V - diag(cs) K S0            cs = e^{gamma} / |k|
+//     V~  = T diag(beta) X               (the WY form U - W S0 with T pulled out: the record needs no W, no U)
+//     O   = diag(qs) Q S0 + P V~         qs = e^{gamma} scale / |q|
+//     S   = e^{gamma_C} S0 + K^T diag(ks) V~      ks = e^{gamma_C - gamma} / |k|
+// Everything a chunk needs - the 12 operand fragments T diag(beta) | P of its record, the chunk's rows of q and k
+// and this workgroup's columns of v straight from the caller's tensors, three vectors of row scales and
+// e^{gamma_C} - goes through a double buffer in LDS: during chunk c the loaders move the data of chunk c + 1
+// global -> registers -> LDS and already have chunks c + 2 and c + 3 in flight in a second register buffer.
+// One workgroup barrier per chunk hands the halves over.  The memory instructions are kept out of the compute
+// waves on purpose: a wave that issues a load or a store while the CU's vector-memory queue is full stalls
+// until there is room, and with one compute wave per SIMD that stall is a stall of the matrix pipe.
 //
-// A compute wave runs the 54 MFMAs of a chunk (K = 128) as one unrolled schedule
-//     V~ = U + W~ S0 | O^T = diag(q scales) (q S0)^T | S = e^{gamma_C} S0 + K~^T V~ | O^T += V~^T P^T
-// reading each fragment from LDS a few MFMAs before its use.  All other per-chunk work - decay of
-// the state, bf16 repacking of V~ and of the new state, conversion of the next chunk's U, the
-// hand-over of the output tile - is cut into pieces placed between MFMAs that do not depend on
-// them.  O is accumulated transposed (operands swapped) and the slice's columns are held in
-// slice_col order, so a lane ends up with 8 consecutive columns of one token (16 bytes).
+// A compute wave runs the 60 MFMAs of a chunk (K = 128) as one unrolled schedule, reading each fragment from
+// LDS a few MFMAs before its use; all other per-chunk work is cut into pieces placed between MFMAs that do not
+// depend on them (ScanSchedule).  O is accumulated transposed (operands swapped) and the slice's columns are
+// held in slice_col order, so a lane ends up with 8 consecutive columns of one token (16 bytes).
 //
-// The slices of a chain sit in workgroups on one XCD and read the same records at the same time,
-// so the records come out of HBM once per chain (measured L2 hit rate 71 %, fetch = the record
-// bytes).  What bounds the kernel when every CU has a workgroup is the rate at which a CU gets
-// lines that were not in its L2 yet when asked for (~15 - 20 B/clk per CU, whatever the number of
-// waves asking); touching the lines ahead of time from a helper wave did not change that.
+// The slices of a chain sit in workgroups on one XCD and read the same lines at the same time, so those come
+// out of HBM once per chain.  What bounds the kernel when every CU has a workgroup is the rate at which a CU
+// gets lines that were not in its L2 yet when asked for (~15 - 20 B/clk per CU, whatever the number of waves
+// asking).
 // ------------------------------------------------------------------------------------------
 constexpr int SCAN_LOADERS = 4;
 
@@ -588,55 +484,62 @@ __device__ __forceinline__ void pin_regs(bf16x8& x) {
 
 // Order of the MFMAs of one chunk in the scan's compute wave, and where its side work goes.
 //
-// MFMAs ("ops"): O^T = S0^T q^T (NQF) | V~ = U + W~ S0 (NWF) | S += k^T V~' (NKF) | O^T += V~^T P^T (6).  The
-// third group runs token slabs 0, 1 of every key tile before slabs 2, 3, so that the second token tile of V~,
+// MFMAs ("ops"):  K S0 (NSF) | O^T = S0^T q^T (NQF) | V~ = T' X (6) | S += k^T V~' (NKF) | O^T += V~^T P^T (6).
+// The fourth group runs token slabs 0, 1 of every key tile before slabs 2, 3, so that the second token tile of V~,
 // finished last, is needed late.
 //
-// Everything else (conversion of U, decay of the state, bf16 repacking of V~ and of the new state, the row scales,
-// hand-over of the output) is cut into pieces of four to six vector instructions.  A piece has a window: the first
-// op at which its inputs exist (an MFMA result is taken two ops after the MFMA was issued) and the op that needs
-// its result.  A lone wave issues an instruction every four to five cycles and an MFMA occupies the matrix pipe
-// for 33, so more than about six instructions between two MFMAs idle the pipe: the pieces are spread one per op,
-// earliest deadline first, as far as their windows allow.
+// Everything else (X = V - diag(cs) K S0 and its bf16 copy, decay of the state, bf16 repacking of V~ and of the new
+// state, the row scales, hand-over of the output) is cut into pieces of four to twelve vector instructions.  A piece
+// has a window: the first op at which its inputs exist (an MFMA result is taken two ops after the MFMA was issued)
+// and the op that needs its result.  A lone wave issues an instruction every four to five cycles and an MFMA
+// occupies the matrix pipe for 33, so more than about six instructions between two MFMAs idle the pipe: the pieces
+// are spread one per op, earliest deadline first, as far as their windows allow.
 template <int K>
 struct ScanScheduleRules {
     static constexpr int KD = K / 32, KS16 = K / 16;
-    static constexpr int NQF = 2 * KS16, NWF = 2 * KS16, NKF = 4 * KD, NPF = 6;
-    static constexpr int NOPS = NQF + NWF + NKF + NPF;
+    static constexpr int NSF = 2 * KS16, NQF = 2 * KS16, NTF = 6, NKF = 4 * KD, NPF = 6;
+    static constexpr int NOPS = NSF + NQF + NTF + NKF + NPF;
     static constexpr int LA = 6;
-    static constexpr int OP_W = NQF, OP_K = NQF + NWF, OP_P = OP_K + NKF, OP_BAR = NOPS - LA;
-    static constexpr int KS_AHEAD = 2;  // the row scales of k are read this many ops before their piece
-    static_assert(OP_BAR >= OP_P, "q's scales, the decay and k's scales of this chunk are used before the barrier");
+    static constexpr int OP_Q = NSF, OP_T = OP_Q + NQF, OP_K = OP_T + NTF, OP_P = OP_K + NKF, OP_BAR = NOPS - LA;
+    static constexpr int AHEAD = 2;  // scales and rows of v are read this many ops before their piece
+    static_assert(OP_BAR >= OP_P, "the scales and v of this chunk are used before the barrier");
 
-    // op j of the third group -> key tile, token slab
+    // op j of the fourth group -> key tile, token slab
     static constexpr int k_tile(int j) { return (j % (2 * KD)) / 2; }
     static constexpr int k_slab(int j) { return 2 * (j / (2 * KD)) + j % 2; }
+    // op j of the third group -> token tile of V~, slab of X (fragment j of the record)
+    static constexpr int t_tile(int j) { return j < 2 ? 0 : 1; }
+    static constexpr int t_slab(int j) { return j < 2 ? j : j - 2; }
 
-    // pieces: U conversion (4 elements) | output hand-over (half a tile) | q row scale (4 registers) | decay
-    // (4 registers) | scaled V~ (half a fragment) | plain V~ (a fragment) | new state (a fragment)
-    static constexpr int N_UC = 8, N_OUT = 4, N_AS = 8, N_DEC = 4 * KD, N_VS = 8, N_VB = 4, N_SB = 2 * KD;
-    static constexpr int P_UC = 0, P_OUT = P_UC + N_UC, P_AS = P_OUT + N_OUT, P_DEC = P_AS + N_AS, P_VS = P_DEC + N_DEC,
+    // pieces: X (4 registers; every second one also packs half a tile of X) | output hand-over (half a tile) | q row
+    // scale (4 registers) | decay (4 registers) | scaled V~ (half a fragment) | plain V~ (a fragment) | new state
+    // (a fragment)
+    static constexpr int N_XC = 8, N_OUT = 4, N_AS = 8, N_DEC = 4 * KD, N_VS = 8, N_VB = 4, N_SB = 2 * KD;
+    static constexpr int P_XC = 0, P_OUT = P_XC + N_XC, P_AS = P_OUT + N_OUT, P_DEC = P_AS + N_AS, P_VS = P_DEC + N_DEC,
                          P_VB = P_VS + N_VS, P_SB = P_VB + N_VB, NPIECES = P_SB + N_SB;
 
     struct Window {
         int first, end;  // the piece runs before the MFMA of an op in [first, end)
     };
     static constexpr Window window(int pc) {
-        if (pc < P_OUT) return {0, OP_W + KS16 * ((pc - P_UC) / 4)};  // accv[tt] is free since the last chunk's packs
+        if (pc < P_OUT) {  // K S0 of tile tt is complete after op KS16 (tt + 1) - 1; T' X overwrites tile 1 at its third op
+            const int tt = (pc - P_XC) / 4;
+            return {KS16 * (tt + 1) + 1, OP_T + 2 * tt};
+        }
         if (pc < P_AS) {  // tile 0: this chunk's, after its two P ops; tile 1: the previous chunk's, before q overwrites it
-            return (pc - P_OUT) / 2 == 0 ? Window{OP_P + 3, NOPS} : Window{1, KS16};
+            return (pc - P_OUT) / 2 == 0 ? Window{OP_P + 3, NOPS} : Window{1, OP_Q + KS16};
         }
         if (pc < P_DEC) {
             const int tt = (pc - P_AS) / 4;
             const int end = OP_P + 2 * tt;
-            return {KS16 * (tt + 1) + 1, end < OP_BAR ? end : OP_BAR};
+            return {OP_Q + KS16 * (tt + 1) + 1, end < OP_BAR ? end : OP_BAR};
         }
         if (pc < P_VS) return {0, OP_K + 2 * ((pc - P_DEC) / 4)};
-        if (pc < P_VB) {
+        if (pc < P_VB) {  // V~ tile 0 is complete after the second op of T' X, tile 1 after the sixth
             const int x = (pc - P_VS) / 2;
-            return {OP_W + KS16 * (x / 2 + 1) + 1, x < 2 ? OP_K + x : OP_K + NKF / 2 + (x - 2)};
+            return {OP_T + (x / 2 == 0 ? 2 : 6) + 1, x < 2 ? OP_K + x : OP_K + NKF / 2 + (x - 2)};
         }
-        if (pc < P_SB) return {OP_W + KS16 * ((pc - P_VB) / 2 + 1) + 1, OP_P};
+        if (pc < P_SB) return {OP_T + ((pc - P_VB) / 2 == 0 ? 2 : 6) + 1, OP_P};
         return {OP_K + NKF / 2 + 2 * ((pc - P_SB) / 2) + 3, NOPS};
     }
 
@@ -662,11 +565,16 @@ struct ScanScheduleRules {
             }
         }
         if (left != 0) t.ok = false;
-        // a scale register (ring of four) is refilled only after the piece four places earlier has used it
+        // the X pieces of a tile run in order (the odd ones pack what the even ones left)
+        for (int i = 1; i < N_XC; i++)
+            if (i % 4 != 0 && t.op[P_XC + i] < t.op[P_XC + i - 1]) t.ok = false;
+        // a ring register (rings of four) is refilled only after the piece four places earlier has used it
         for (int i = 4; i < N_VS; i++)
-            if (t.op[P_VS + i] - KS_AHEAD <= t.op[P_VS + i - 4]) t.ok = false;
+            if (t.op[P_VS + i] - AHEAD <= t.op[P_VS + i - 4]) t.ok = false;
+        for (int i = 4; i < N_XC; i++)
+            if (t.op[P_XC + i] - AHEAD <= t.op[P_XC + i - 4]) t.ok = false;
         for (int i = 0; i < N_VS; i++)
-            if (t.op[P_VS + i] - KS_AHEAD < 0) t.ok = false;
+            if (t.op[P_VS + i] - AHEAD < 0) t.ok = false;
         return t;
     }
 };
@@ -685,26 +593,29 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
     constexpr bool OS = NW < 4;
     constexpr int KD = K / 32;    // 32-row tiles of the state
     constexpr int KS16 = K / 16;  // 16-wide slabs over the key dim
-    constexpr int NWF = 2 * KS16, NQF = 2 * KS16, NKF = KD * 4, NPF = 6;  // MFMAs on W~, on q, on k^T, on P
-    // One half of the stage: [W~ | P] (contiguous at the head of the record) | U tiles of this workgroup's columns
-    // (contiguous in the record) | the chunk's 64 rows of q, then of k, row-major, copied from the caller's
-    // tensors | 64 row scales of q | 64 row scales of k | e^{gamma_C}
-    constexpr int SHARED_FRAGS = NWF + NPF;
+    // One half of the stage: [T diag(beta) 6 | P 6] (the head of the record) | the chunk's 64 rows of this
+    // workgroup's columns of v | of q | of k, row-major, copied from the caller's tensors | 64 row scales of q |
+    // of k for the state update | of k S0 | e^{gamma_C}
+    constexpr int SHARED_FRAGS = 12;
     constexpr int SHARED_BYTES = SHARED_FRAGS * FRAG_BYTES;
-    constexpr int U_FRAGS = 4 * NW;
-    constexpr int STAGE_FRAGS = SHARED_FRAGS + U_FRAGS;
+    constexpr int VROW = 64 * NW;                    // bytes per row of v held by this workgroup (32 columns per compute wave)
+    constexpr int VLD = VROW + 16;                   // bytes per staged row of v
+    constexpr int V_UNITS = C * VROW / FRAG_BYTES;   // 1 KiB pieces of the v rows: 1024 / VROW whole rows each
     constexpr int QLD = 2 * K + 16;                  // bytes per staged row of q / k (16 bytes of padding against bank conflicts)
     constexpr int Q_UNITS = C * 2 * K / FRAG_BYTES;  // 1 KiB pieces of the q rows: 512 / K whole rows each; as many for k
-    constexpr int Q_OFF = STAGE_FRAGS * FRAG_BYTES;
+    constexpr int V_OFF = SHARED_BYTES;
+    constexpr int Q_OFF = V_OFF + C * VLD;
     constexpr int K_OFF = Q_OFF + C * QLD;
     constexpr int QS_OFF = K_OFF + C * QLD;
     constexpr int KS_OFF = QS_OFF + C * 4;
-    constexpr int EG_OFF = KS_OFF + C * 4;
+    constexpr int CS_OFF = KS_OFF + C * 4;
+    constexpr int EG_OFF = CS_OFF + C * 4;
     constexpr int STAGE_BYTES = EG_OFF + 16;
-    constexpr int NF = (STAGE_FRAGS + NL - 1) / NL;  // fragment slots per loader wave
-    constexpr int NQ = 2 * Q_UNITS / NL;             // q / k row slots per loader wave
-    constexpr int NLOAD = NF + NQ;                   // 1 KiB moves per loader wave and record
-    static_assert((2 * Q_UNITS) % NL == 0, "the pieces of q and k must divide over the loader waves");
+    constexpr int NF = SHARED_FRAGS / NL;  // fragment slots per loader wave
+    constexpr int NV = V_UNITS / NL;       // v row slots per loader wave
+    constexpr int NQ = 2 * Q_UNITS / NL;   // q / k row slots per loader wave
+    constexpr int NLOAD = NF + NV + NQ;    // 1 KiB moves per loader wave and chunk
+    static_assert(SHARED_FRAGS % NL == 0 && V_UNITS % NL == 0 && (2 * Q_UNITS) % NL == 0, "the pieces must divide over the loader waves");
     static_assert(2 * STAGE_BYTES + (OS ? NW * 2 * C * 64 : 16) <= 160 * 1024, "stage exceeds LDS");
 
     __shared__ __attribute__((aligned(16))) uint8_t stage[2][STAGE_BYTES];
@@ -715,12 +626,11 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
     const int l32 = lane % 32, lh = lane / 32;
 
     // workgroup -> (sequence-head chain, column group); the groups of a chain stay on one XCD (id % 8)
-    // so that its records are fetched into a single L2
+    // so that the lines they share are fetched into a single L2
     const int id = blockIdx.x;
     const int xcd = id % 8, rest = id / 8;
     const int vgroup = rest % p.scan_groups;
-    // XCD x takes the chains x * per_xcd .. : consecutive chains are different heads, whose rows of q, k and o
-    // fall on different channels of the XCD's L2 (the rows of one head lie a multiple of 2 KiB apart)
+    // XCD x takes the chains x * per_xcd .. : consecutive chains are different heads
     const int per_xcd = (p.N * p.H + 7) / 8;
     const int chain = xcd * per_xcd + rest / p.scan_groups;
     if (rest / p.scan_groups >= per_xcd || chain >= p.N * p.H) return;  // whole workgroup
@@ -781,105 +691,109 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
     }
     if (is_loader) {
         // ------------------------------ loader ------------------------------
-        // fragment f of the stage: f < SHARED_FRAGS comes from the head of the record, the rest from
-        // this workgroup's slice of the U block
         // loader number 0..3, wave-uniform: unit numbers and bases stay scalar
         const int lw = __builtin_amdgcn_readfirstlane(NW == 4 ? wave - 4 : NW == 2 ? (wave < 4 ? wave - 2 : wave - 4) : (wave < 4 ? wave - 1 : 3));
-        // Slots 0 .. NF - 1 of this wave move fragments lw * NF + (rotated slot), slots NF .. NLOAD - 1 move 1 KiB
-        // pieces of the q rows; a surplus fragment slot repeats the last fragment.  Which kind a slot is, is known
-        // at compile time, so there is no branch in these loops (a branch makes the compiler wait for every load
-        // in flight).  The rotation by column group lets the workgroups of a chain ask for different lines at
-        // any one time: a line's memory latency is then paid by one of them instead of being waited out by all.
-        const int rot_f = (vgroup * ((NF + 3) / 4)) % NF;
+        // Slots 0 .. NF - 1 of this wave move record fragments lw * NF + (rotated slot), the next NV slots 1 KiB
+        // pieces of the v rows, the last NQ slots pieces of the q and k rows.  Which kind a slot is, is known at
+        // compile time, so there is no branch in these loops (a branch makes the compiler wait for every load in
+        // flight).  The rotation by column group lets the workgroups of a chain ask for different lines at any
+        // one time: a line's memory latency is then paid by one of them instead of being waited out by all.
+        const int rot_f = vgroup % NF;
         const int rot_q = vgroup % NQ;
-        auto frag_of = [&](int i) {  // i < NF
-            const int f = lw * NF + (i + rot_f < NF ? i + rot_f : i + rot_f - NF);
-            return f < STAGE_FRAGS ? f : STAGE_FRAGS - 1;
-        };
+        auto frag_of = [&](int i) { return lw * NF + (i + rot_f < NF ? i + rot_f : i + rot_f - NF); };   // i < NF
+        auto vunit_of = [&](int i) { return lw * NV + i; };                                              // i < NV
         auto qunit_of = [&](int i) { return lw * NQ + (i + rot_q < NQ ? i + rot_q : i + rot_q - NQ); };  // i < NQ
-        const int64_t u_shift = (int64_t)p.off_u + (int64_t)vgroup * U_FRAGS * FRAG_BYTES - SHARED_BYTES;
-        // rows of q: lane -> (row within the unit, 16-byte piece)
+        // rows of q, k: lane -> (row within the unit, 16-byte piece); likewise for v
         constexpr int Q_ROWS = C / Q_UNITS, Q_PIECES = WAVE / Q_ROWS;
+        constexpr int V_ROWS = C / V_UNITS, V_PIECES = WAVE / V_ROWS;
         const int q_row = lane / Q_PIECES, q_piece = lane % Q_PIECES;
+        const int v_row = lane / V_PIECES, v_piece = lane % V_PIECES;
         const bf16_t* const qg = p.q + b * p.q_stride_b + seq_t0 * p.q_stride_t + (int64_t)h * p.q_stride_h + q_piece * 8;
         const bf16_t* const kg = p.k + b * p.k_stride_b + seq_t0 * p.k_stride_t + (int64_t)h * p.k_stride_h + q_piece * 8;
-        // two register buffers: while one record is written to LDS, younger ones are in flight
+        const bf16_t* const vg = p.v + b * p.v_stride_b + seq_t0 * p.v_stride_t + (int64_t)h * p.v_stride_h + 32 * (vgroup * NW) + v_piece * 8;
+        // two register buffers: while one chunk is written to LDS, younger ones are in flight
         bf16x8 buf0[NLOAD], buf1[NLOAD];
-        float sc0 = 0.f, sc1 = 0.f;  // lanes 0..63: row scale of q of token `lane`
-        float kc0 = 0.f, kc1 = 0.f;  // the same for k
-        float eg0 = 0.f, eg1 = 0.f;
+        // lanes 0..63: row scales of token `lane` (of q, of k for the state update, of k S0), and e^{gamma_C}
+        struct Scalars {
+            float qs, ks, cs, eg;
+        };
+        Scalars sc0 = {0.f, 0.f, 0.f, 0.f}, sc1 = {0.f, 0.f, 0.f, 0.f};
         auto src_of = [&](int c, int i) -> const uint8_t* {
-            if (i < NF) {
-                const int f = frag_of(i);
-                return rec + ((int64_t)c * p.rec_bytes + (int64_t)f * FRAG_BYTES + (f >= SHARED_FRAGS ? u_shift : 0)) + lane * 16;
+            if (i < NF) return rec + ((int64_t)c * p.rec_bytes + (int64_t)frag_of(i) * FRAG_BYTES) + lane * 16;
+            // a row past the end of the sequence (tail chunk) is read from the last token instead: never used
+            if (i < NF + NV) {
+                const int tok = min(c * C + vunit_of(i - NF) * V_ROWS + v_row, (int)seq_len - 1);
+                return reinterpret_cast<const uint8_t*>(vg + (int64_t)tok * p.v_stride_t);
             }
-            // units 0 .. Q_UNITS - 1 are rows of q, the rest rows of k (wave-uniform choice); a row past the end of
-            // the sequence (tail chunk) is read from the last token instead: never used
-            const int u = qunit_of(i - NF);
+            // units 0 .. Q_UNITS - 1 are rows of q, the rest rows of k (wave-uniform choice)
+            const int u = qunit_of(i - NF - NV);
             const bool is_k = u >= Q_UNITS;
             const int tok = min(c * C + (is_k ? u - Q_UNITS : u) * Q_ROWS + q_row, (int)seq_len - 1);
             return reinterpret_cast<const uint8_t*>((is_k ? kg : qg) + (int64_t)tok * (is_k ? p.k_stride_t : p.q_stride_t));
         };
         auto dst_of = [&](uint8_t* st, int i) -> uint8_t* {
             if (i < NF) return st + frag_of(i) * FRAG_BYTES + lane * 16;
-            return st + Q_OFF + (qunit_of(i - NF) * Q_ROWS + q_row) * QLD + q_piece * 16;  // the k rows follow the q rows
+            if (i < NF + NV) return st + V_OFF + (vunit_of(i - NF) * V_ROWS + v_row) * VLD + v_piece * 16;
+            return st + Q_OFF + (qunit_of(i - NF - NV) * Q_ROWS + q_row) * QLD + q_piece * 16;  // the k rows follow the q rows
         };
-        // every loader wave carries the row scales of q and k and e^{gamma_C} (identical values, identical LDS writes)
-        auto load_scalars = [&](float& sc, float& kc, float& eg, int c) {
+        // every loader wave carries the scales (identical values, identical LDS writes)
+        auto load_scalars = [&](Scalars& sc, int c) {
             const uint8_t* r = rec + (int64_t)c * p.rec_bytes;
-            sc = reinterpret_cast<const float*>(r + p.off_qs)[lane];
-            kc = reinterpret_cast<const float*>(r + p.off_ks)[lane];
-            eg = *reinterpret_cast<const float*>(r + p.off_eg);
+            sc.qs = reinterpret_cast<const float*>(r + p.off_qs)[lane];
+            sc.ks = reinterpret_cast<const float*>(r + p.off_ks)[lane];
+            sc.cs = reinterpret_cast<const float*>(r + p.off_cs)[lane];
+            sc.eg = *reinterpret_cast<const float*>(r + p.off_eg);
         };
-        auto load = [&](bf16x8(&buf)[NLOAD], float& sc, float& kc, float& eg, int c) {
+        auto load = [&](bf16x8(&buf)[NLOAD], Scalars& sc, int c) {
 #pragma unroll
             for (int i = 0; i < NLOAD; i++) buf[i] = *reinterpret_cast<const bf16x8*>(src_of(c, i));
-            load_scalars(sc, kc, eg, c);
+            load_scalars(sc, c);
         };
-        // write record c to LDS and refill each register with record c2 right behind its write, so the
+        // write chunk c to LDS and refill each register with chunk c2 right behind its write, so the
         // LDS-write and the vector-memory queues fill together
-        auto store_and_reload = [&](bf16x8(&buf)[NLOAD], float& sc, float& kc, float& eg, int c, int c2, auto reload_tag) {
+        auto store_and_reload = [&](bf16x8(&buf)[NLOAD], Scalars& sc, int c, int c2, auto reload_tag) {
             constexpr bool reload = decltype(reload_tag)::value;
             uint8_t* dst = stage[c & 1];
-            reinterpret_cast<float*>(dst + QS_OFF)[lane] = sc;
-            reinterpret_cast<float*>(dst + KS_OFF)[lane] = kc;
-            if (lane == 0) *reinterpret_cast<float*>(dst + EG_OFF) = eg;
+            reinterpret_cast<float*>(dst + QS_OFF)[lane] = sc.qs;
+            reinterpret_cast<float*>(dst + KS_OFF)[lane] = sc.ks;
+            reinterpret_cast<float*>(dst + CS_OFF)[lane] = sc.cs;
+            if (lane == 0) *reinterpret_cast<float*>(dst + EG_OFF) = sc.eg;
 #pragma unroll
             for (int i = 0; i < NLOAD; i++) {
                 *reinterpret_cast<bf16x8*>(dst_of(dst, i)) = buf[i];
                 if constexpr (reload) buf[i] = *reinterpret_cast<const bf16x8*>(src_of(c2, i));
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if constexpr (reload) load_scalars(sc, kc, eg, c2);
+            if constexpr (reload) load_scalars(sc, c2);
         };
         constexpr std::true_type yes{};
         constexpr std::false_type no{};
-        // records 0 (-> LDS now), 1 and 2 (in flight); even records use buf0, odd ones buf1
+        // chunks 0 (-> LDS now), 1 and 2 (in flight); even chunks use buf0, odd ones buf1
         if (nchunks > 0) {
-            load(buf0, sc0, kc0, eg0, 0);
-            if (nchunks > 1) load(buf1, sc1, kc1, eg1, 1);
-            if (nchunks > 2) store_and_reload(buf0, sc0, kc0, eg0, 0, 2, yes);
-            else store_and_reload(buf0, sc0, kc0, eg0, 0, 0, no);
+            load(buf0, sc0, 0);
+            if (nchunks > 1) load(buf1, sc1, 1);
+            if (nchunks > 2) store_and_reload(buf0, sc0, 0, 2, yes);
+            else store_and_reload(buf0, sc0, 0, 0, no);
         }
-        __syncthreads();  // stage[0] holds record 0
-        // Barrier of iteration c: the compute waves are done with stage[c & 1] and record c + 1 is in the
-        // other half.  Before it: write record c + 1 (its half was released by the barrier of iteration
-        // c - 1) and refill the freed registers with record c + 3.
+        __syncthreads();  // stage[0] holds chunk 0
+        // Barrier of iteration c: the compute waves are done with stage[c & 1] and chunk c + 1 is in the
+        // other half.  Before it: write chunk c + 1 (its half was released by the barrier of iteration
+        // c - 1) and refill the freed registers with chunk c + 3.
         int c = 0;
         for (; c + 4 < nchunks; c += 2) {  // steady state: straight-line code, both reloads exist
-            store_and_reload(buf1, sc1, kc1, eg1, c + 1, c + 3, yes);
+            store_and_reload(buf1, sc1, c + 1, c + 3, yes);
             __syncthreads();
-            store_and_reload(buf0, sc0, kc0, eg0, c + 2, c + 4, yes);
+            store_and_reload(buf0, sc0, c + 2, c + 4, yes);
             __syncthreads();
         }
         for (; c < nchunks; c += 2) {  // the last (at most four) chunks
             if (c + 1 < nchunks) {
-                if (c + 3 < nchunks) store_and_reload(buf1, sc1, kc1, eg1, c + 1, c + 3, yes);
-                else store_and_reload(buf1, sc1, kc1, eg1, c + 1, 0, no);
+                if (c + 3 < nchunks) store_and_reload(buf1, sc1, c + 1, c + 3, yes);
+                else store_and_reload(buf1, sc1, c + 1, 0, no);
             }
             __syncthreads();
             if (c + 1 < nchunks) {
-                if (c + 2 < nchunks) store_and_reload(buf0, sc0, kc0, eg0, c + 2, 0, no);
+                if (c + 2 < nchunks) store_and_reload(buf0, sc0, c + 2, 0, no);
                 __syncthreads();
             }
         }
@@ -892,7 +806,7 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
     // State tile td, register r: MFMA row i = 8 (r/4) + 4 h + r%4 holds state row 32 td + slice_col(i)
     // = 32 td + 16 (r/8) + 8 h + 4 ((r/4) % 2) + r%4, column 32 tn + slice_col(l32).  With the rows of a 16-block
     // in that order, the 8 reduction entries a lane half feeds per 16-row slab are 8 consecutive key columns:
-    // q is used straight from its row-major rows.
+    // q and k are used straight from their row-major rows.
     f32x16 S[KD];
     const int64_t st_off = ((int64_t)n * p.H + h) * K * p.V + (int64_t)(8 * lh) * p.V + 32 * tn + slice_col(l32);
     auto st_row = [](int td, int r) { return 32 * td + 16 * (r / 8) + 4 * ((r / 4) % 2) + r % 4; };
@@ -910,17 +824,19 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
     bf16_t* og = p.o + b * p.o_stride_b + (seq_t0 + l32) * p.o_stride_t + (int64_t)h * p.o_stride_h + 32 * tn + 8 * lh;
     const int64_t og_step = (int64_t)C * p.o_stride_t;
 
-    // MFMA schedule of one chunk: q (NQF) | W~ (NWF) | k^T (NKF) | P (6); the side work sits between the MFMAs
-    // at the ops ScanSchedule<K> assigns.
+    // MFMA schedule of one chunk: K S0 | q | T' X | k^T | P; the side work sits between the MFMAs at the ops
+    // ScanSchedule<K> assigns.
     typedef ScanSchedule<K> SCH;
-    constexpr int NOPS = SCH::NOPS, OP_W = SCH::OP_W, OP_K = SCH::OP_K, OP_P = SCH::OP_P, OP_BAR = SCH::OP_BAR;
+    constexpr int NOPS = SCH::NOPS, OP_Q = SCH::OP_Q, OP_T = SCH::OP_T, OP_K = SCH::OP_K, OP_P = SCH::OP_P, OP_BAR = SCH::OP_BAR;
     constexpr int LA = SCH::LA;  // LDS reads are issued this many MFMAs ahead of their use
     const int l16 = lane % 16, g16 = l32 / 16;
     auto lds_frag = [&](const uint8_t* st, auto opc) -> bf16x8 {
         constexpr int op = decltype(opc)::value;
-        if constexpr (op < OP_W) {  // q, token tile tt, 16-column slab s: 8 consecutive columns per lane half
-            constexpr int s = op % KS16, tt = op / KS16;
-            return *reinterpret_cast<const bf16x8*>(st + Q_OFF + (32 * tt + l32) * QLD + (16 * s + 8 * lh) * 2);
+        if constexpr (op < OP_T) {
+            // rows of k (A operand of K S0) or of q (B operand of S0^T q^T): token tile tt, 16-column slab s,
+            // 8 consecutive key columns per lane half
+            constexpr int j = op < OP_Q ? op : op - OP_Q, s = j % KS16, tt = j / KS16;
+            return *reinterpret_cast<const bf16x8*>(st + (op < OP_Q ? K_OFF : Q_OFF) + (32 * tt + l32) * QLD + (16 * s + 8 * lh) * 2);
         } else if constexpr (op >= OP_K && op < OP_P) {
             // k^T, key tile td (rows in state order), token slab s: tokens 16 s + 4 h + 0..3 and 16 s + 8 + 4 h + 0..3
             // of key column 32 td + slice_col(l32), through the transposing LDS load
@@ -933,26 +849,22 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
             for (int e = 0; e < 4; e++) r[e] = a[e], r[4 + e] = b[e];
             return r;
         } else {
-            constexpr int f = op < OP_K ? op - OP_W : NWF + (op - OP_P);  // W~ | P are contiguous in the stage
+            constexpr int f = op < OP_K ? op - OP_T : 6 + (op - OP_P);  // T' | P are contiguous in the stage
             return reinterpret_cast<const bf16x8*>(st)[f * WAVE + lane];
         }
-    };
-    auto lds_u = [&](const uint8_t* st, int i) -> bf16x8 {
-        return reinterpret_cast<const bf16x8*>(st + SHARED_BYTES)[(wave * 4 + i) * WAVE + lane];
     };
     auto lds_eg = [&](const uint8_t* st) -> float { return *reinterpret_cast<const float*>(st + EG_OFF); };
     auto lds_qs = [&](const uint8_t* st, int tt) -> float { return reinterpret_cast<const float*>(st + QS_OFF)[32 * tt + l32]; };
 
     f32x16 accv[2], acco[2];
-    bf16x8 sb[KS16], vb[4], vbs[4], ur[4], fnext[LA];  // vbs: V~ with its rows scaled like K~'s, for the state update
-    f32x4 ksr[4];                                      // row scales of k on their way to the pieces that use them
+    bf16x8 sb[KS16], xb[4], vb[4], vbs[4], fnext[LA];  // xb: X, vb: V~, vbs: V~ with its rows scaled for the state update
+    f32x4 ksr[4], csr[4];                              // row scales on their way to the pieces that use them
+    bf16x4 xvr[4];                                     // and rows of v
     float egc, qsc[2];  // e^{gamma_C} and this lane's two row scales of q (tokens l32 and 32 + l32)
 
-    __syncthreads();  // stage[0] holds record 0
+    __syncthreads();  // stage[0] holds chunk 0
 
     // what the tail of a chunk does for the next one, for chunk 0
-#pragma unroll
-    for (int i = 0; i < 4; i++) ur[i] = lds_u(stage[0], i);
     egc = lds_eg(stage[0]);
     qsc[0] = lds_qs(stage[0], 0), qsc[1] = lds_qs(stage[0], 1);
     static_for<0, LA>([&](auto i) { fnext[decltype(i)::value] = lds_frag(stage[0], i); });
@@ -972,11 +884,13 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
         // one piece of side work (pc: index into ScanSchedule's piece list)
         auto run_piece = [&](auto pcc) {
             constexpr int pc = decltype(pcc)::value;
-            if constexpr (pc >= SCH::P_UC && pc < SCH::P_UC + SCH::N_UC) {
-                // U of this chunk -> fp32 accumulators: 4 elements of ur[q]
-                constexpr int i = pc - SCH::P_UC, q = i / 2, hh = i % 2;
+            if constexpr (pc >= SCH::P_XC && pc < SCH::P_XC + SCH::N_XC) {
+                // X = V - diag(cs) (K S0), registers 4 q4 .. 4 q4 + 3 of tile tt: tokens 32 tt + 8 q4 + 4 h + 0..3 of
+                // this lane's column; the second piece of a half tile also packs it as an operand of T' X
+                constexpr int i = pc - SCH::P_XC, tt = i / 4, q4 = i % 4;
 #pragma unroll
-                for (int e = 0; e < 4; e++) accv[q / 2][8 * (q % 2) + 4 * hh + e] = (float)ur[q][4 * hh + e];
+                for (int e = 0; e < 4; e++) accv[tt][4 * q4 + e] = (float)xvr[i % 4][e] - csr[i % 4][e] * accv[tt][4 * q4 + e];
+                if constexpr (q4 % 2 == 1) xb[2 * tt + q4 / 2] = pack8_16(accv[tt], q4 / 2, 1.f);
             } else if constexpr (pc >= SCH::P_OUT && pc < SCH::P_OUT + SCH::N_OUT) {
                 // output tile tt, registers 8 half .. 8 half + 7: tile 0 belongs to this chunk (its P terms are
                 // complete), tile 1 to the previous one
@@ -1026,21 +940,26 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
 
         static_for<0, NOPS>([&](auto opc) {
             constexpr int op = decltype(opc)::value;
-            // ---- operand reads: this record until the barrier, the next one after it ----
+            // ---- operand reads: this chunk until the barrier, the next one after it ----
             if constexpr (op + LA < NOPS) fr[op + LA] = lds_frag(st, std::integral_constant<int, (op + LA < NOPS ? op + LA : 0)>{});
             if constexpr (op == OP_BAR) {
-                __syncthreads();  // this wave is done with record c; record c + 1 is in the other half
-#pragma unroll
-                for (int i = 0; i < 4; i++) ur[i] = lds_u(stn, i);
+                __syncthreads();  // this wave is done with chunk c's half; chunk c + 1 is in the other one
                 egc = lds_eg(stn);
                 qsc[0] = lds_qs(stn, 0), qsc[1] = lds_qs(stn, 1);  // this chunk's scales were applied before the barrier
             }
             if constexpr (op >= OP_BAR) fnext[op >= OP_BAR ? op - OP_BAR : 0] = lds_frag(stn, std::integral_constant<int, (op >= OP_BAR ? op - OP_BAR : 0)>{});
-            // the row scales of k, two ops ahead of the piece that uses them
+            // row scales and rows of v, a few ops ahead of the piece that uses them
             static_for<0, SCH::N_VS>([&](auto ic) {
                 constexpr int i = decltype(ic)::value, x = i / 2, sub = i % 2;
-                if constexpr (SCH::op_of(SCH::P_VS + i) - SCH::KS_AHEAD == op)
+                if constexpr (SCH::op_of(SCH::P_VS + i) - SCH::AHEAD == op)
                     ksr[i % 4] = *reinterpret_cast<const f32x4*>(st + KS_OFF + (16 * x + 8 * sub + 4 * lh) * 4);
+            });
+            static_for<0, SCH::N_XC>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                if constexpr (SCH::op_of(SCH::P_XC + i) - SCH::AHEAD == op) {
+                    csr[i % 4] = *reinterpret_cast<const f32x4*>(st + CS_OFF + (8 * i + 4 * lh) * 4);
+                    xvr[i % 4] = lds_read_tr4x16<true>(reinterpret_cast<const bf16_t*>(st + V_OFF), VLD / 2, 8 * i + 4 * lh, 32 * wave + 16 * g16, l16);
+                }
             });
 
             // ---- side work ----
@@ -1049,8 +968,18 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
             });
 
             // ---- the MFMA ----
-            if constexpr (op < OP_W) {  // O^T = (q S0)^T, scaled per token by a later piece
+            if constexpr (op < OP_Q) {  // K S0, fragment (tt, s): rows = tokens
                 constexpr int s = op % KS16, tt = op / KS16;
+                if constexpr (s == 0) {
+                    f32x16 zero;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) zero[r] = 0.f;
+                    accv[tt] = mfma32_bf16(fr[op], sb[s], zero);
+                } else {
+                    accv[tt] = mfma32_bf16(fr[op], sb[s], accv[tt]);
+                }
+            } else if constexpr (op < OP_T) {  // O^T = (q S0)^T, scaled per token by a later piece
+                constexpr int j = op - OP_Q, s = j % KS16, tt = j / KS16;
                 if constexpr (s == 0) {
                     f32x16 zero;
 #pragma unroll
@@ -1059,9 +988,16 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
                 } else {
                     acco[tt] = mfma32_bf16(sb[s], fr[op], acco[tt]);
                 }
-            } else if constexpr (op < OP_K) {  // V~ = U + W~ S0, fragment (tt, s)
-                constexpr int j = op - OP_W, s = j % KS16, tt = j / KS16;
-                accv[tt] = mfma32_bf16(fr[op], sb[s], accv[tt]);
+            } else if constexpr (op < OP_K) {  // V~ = T' X: tile 0 from X tile 0, tile 1 from both
+                constexpr int j = op - OP_T, tt = SCH::t_tile(j), s = SCH::t_slab(j);
+                if constexpr (s == 0) {
+                    f32x16 zero;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) zero[r] = 0.f;
+                    accv[tt] = mfma32_bf16(fr[op], xb[s], zero);
+                } else {
+                    accv[tt] = mfma32_bf16(fr[op], xb[s], accv[tt]);
+                }
             } else if constexpr (op < OP_P) {  // S = e^{gamma_C} S + k^T (row-scaled V~), fragment (td, s)
                 constexpr int s = SCH::k_slab(op - OP_K), td = SCH::k_tile(op - OP_K);
                 S[td] = mfma32_bf16(fr[op], vbs[s], S[td]);
