@@ -83,7 +83,7 @@ __device__ __forceinline__ void split_hi_lo(float x, bf16_t& hi, bf16_t& lo) {
 // prepare
 // ------------------------------------------------------------------------------------------
 template <int K>
-__global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const ChunkParams p) {
+__global__ __launch_bounds__(PREP_THREADS, 3) void chunk_prepare32_kernel(const ChunkParams p) {
     constexpr int LDK = K + 8;  // bf16 elements per LDS row of K / Q
     constexpr int LDA = C + 4;  // fp32 elements per LDS row of A / T
     constexpr int LDT = 36;     // fp32 elements per row of the 32 x 32 transposed blocks
@@ -95,16 +95,20 @@ __global__ __launch_bounds__(PREP_THREADS, 2) void chunk_prepare32_kernel(const 
     constexpr int NPASS = C / RPP;
     constexpr int QT_BYTES = (C * LDK * 2 > C * LDA * 4) ? C * LDK * 2 : C * LDA * 4;
 
-    __shared__ __attribute__((aligned(16))) bf16_t sK[C * LDK];
+    // K is dead once A and P are formed; the scratch blocks of the inverse take its place
+    constexpr int SCRATCH_FLOATS = 32 * LDT + 16 * LDM + 2 * 16 * LDM + 32 * LDT;
+    constexpr int KM_BYTES = (C * LDK * 2 > SCRATCH_FLOATS * 4) ? C * LDK * 2 : SCRATCH_FLOATS * 4;
+    __shared__ __attribute__((aligned(16))) uint8_t sKM[KM_BYTES];
     __shared__ __attribute__((aligned(16))) uint8_t sQT[QT_BYTES];  // Q (bf16), then T (fp32)
     __shared__ __attribute__((aligned(16))) float sA[C * LDA];
-    __shared__ __attribute__((aligned(16))) float sTtA[32 * LDT];   // transpose of the top-left 32 x 32 of T
-    __shared__ __attribute__((aligned(16))) float sTt2[16 * LDM];   // transpose of diagonal block 2 of T
-    __shared__ __attribute__((aligned(16))) float sMt[2 * 16 * LDM + 32 * LDT];  // transposed products
     __shared__ __attribute__((aligned(16))) float s_gam[C], s_beta[C], s_ssk[C], s_ssq[C];
     __shared__ __attribute__((aligned(16))) float s_rk[C], s_rq[C];
     bf16_t* const sQ = reinterpret_cast<bf16_t*>(sQT);
     float* const sT = reinterpret_cast<float*>(sQT);
+    bf16_t* const sK = reinterpret_cast<bf16_t*>(sKM);
+    float* const sTtA = reinterpret_cast<float*>(sKM);  // transpose of the top-left 32 x 32 of T
+    float* const sTt2 = sTtA + 32 * LDT;                // transpose of diagonal block 2 of T
+    float* const sMt = sTt2 + 16 * LDM;                 // transposed products
     float* const sMtB = sMt + 2 * 16 * LDM;
 
     const int tid = threadIdx.x;
@@ -1038,7 +1042,7 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
 template <int K>
 static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int num_cus) {
     const int64_t items = (int64_t)((p.TC + 7) / 8) * 8 * p.H;  // a multiple of 8, see the kernel
-    const int64_t cap = (int64_t)(2 * num_cus + 7) / 8 * 8;      // two workgroups per CU
+    const int64_t cap = (int64_t)(3 * num_cus + 7) / 8 * 8;      // three workgroups per CU (LDS and registers allow it)
     const int grid_prep = (int)(items < cap ? items : cap);
     hipLaunchKernelGGL((chunk_prepare32_kernel<K>), dim3(grid_prep), dim3(PREP_THREADS), 0, stream, p);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
