@@ -590,7 +590,9 @@ struct ScanSchedule : ScanScheduleRules<K> {
     static constexpr int op_of(int pc) { return TABLE.op[pc]; }
 };
 
-template <int K, int NW>
+// NT: the loaders use non-temporal loads.  Right when no other workgroup reads the same lines (one workgroup per
+// chain; measured 7 % faster at 1024 chains), wrong when column groups share them through the L2 (8 % slower).
+template <int K, int NW, bool NT = false>
 __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(const ChunkParams p) {
     constexpr int NL = SCAN_LOADERS;
     // a separate wave writes the output (see below); with four compute waves the LDS has no room for its staging
@@ -748,9 +750,13 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
             sc.cs = reinterpret_cast<const float*>(r + p.off_cs)[lane];
             sc.eg = *reinterpret_cast<const float*>(r + p.off_eg);
         };
+        auto fetch = [&](const uint8_t* src) -> bf16x8 {
+            if constexpr (NT) return __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(src));
+            else return *reinterpret_cast<const bf16x8*>(src);
+        };
         auto load = [&](bf16x8(&buf)[NLOAD], Scalars& sc, int c) {
 #pragma unroll
-            for (int i = 0; i < NLOAD; i++) buf[i] = *reinterpret_cast<const bf16x8*>(src_of(c, i));
+            for (int i = 0; i < NLOAD; i++) buf[i] = fetch(src_of(c, i));
             load_scalars(sc, c);
         };
         // write chunk c to LDS and refill each register with chunk c2 right behind its write, so the
@@ -765,7 +771,7 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
 #pragma unroll
             for (int i = 0; i < NLOAD; i++) {
                 *reinterpret_cast<bf16x8*>(dst_of(dst, i)) = buf[i];
-                if constexpr (reload) buf[i] = *reinterpret_cast<const bf16x8*>(src_of(c2, i));
+                if constexpr (reload) buf[i] = fetch(src_of(c2, i));
                 __builtin_amdgcn_sched_barrier(0);
             }
             if constexpr (reload) load_scalars(sc, c2);
@@ -1058,7 +1064,8 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     while (nw < 4 && vtiles % (2 * nw) == 0 && chains * (vtiles / nw) > (int64_t)num_cus) nw *= 2;
     p.scan_groups = vtiles / nw;
     const dim3 grid((unsigned)(chains8 * p.scan_groups));
-    if (nw == 4) hipLaunchKernelGGL((chunk_scan32_kernel<K, 4>), grid, dim3(scan_waves(4) * WAVE), 0, stream, p);
+    if (nw == 4 && p.scan_groups == 1) hipLaunchKernelGGL((chunk_scan32_kernel<K, 4, true>), grid, dim3(scan_waves(4) * WAVE), 0, stream, p);
+    else if (nw == 4) hipLaunchKernelGGL((chunk_scan32_kernel<K, 4>), grid, dim3(scan_waves(4) * WAVE), 0, stream, p);
     else if (nw == 2) hipLaunchKernelGGL((chunk_scan32_kernel<K, 2>), grid, dim3(scan_waves(2) * WAVE), 0, stream, p);
     else hipLaunchKernelGGL((chunk_scan32_kernel<K, 1>), grid, dim3(scan_waves(1) * WAVE), 0, stream, p);
     return (int)hipGetLastError();
