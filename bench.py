@@ -41,8 +41,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # summaries are kept under profiles/.  Workloads that were not profiled report null.
 _KIB = 1024
 MEASURED_HBM_TRAFFIC_BYTES = {
-    ("cfg1_chunk_fwd_bf16", "chunk_prepare"): (2.0 * 104650.2 + 157824.0) * _KIB,
-    ("cfg1_chunk_fwd_bf16", "chunk_scan"): (2.0 * 144834.1 + 69682.2) * _KIB,
+    ("cfg1_chunk_fwd_bf16", "chunk_prepare"): (2.0 * 66468.2 + 52352.0) * _KIB,
+    ("cfg1_chunk_fwd_bf16", "chunk_scan"): (2.0 * 124827.2 + 69632.0) * _KIB,
     ("cfg3_decode_bf16", "recurrent_kernel"): (2.0 * 265449.7 + 526881.4) * _KIB,
     ("cfg1_chunk_fwd_bf16", "causal_conv1d_kernel"): (2.0 * 116926.8 + 196752.0) * _KIB,
     ("cfg1_chunk_fwd_bf16", "gated_rmsnorm_kernel"): (2.0 * 66081.4 + 65536.0) * _KIB,
@@ -131,6 +131,7 @@ def bench_chunk(w, steps, warmup):
             "tflops_dense": round(whole_tflops, 1),
             "mfma_frac_dense": round(whole_tflops / MFMA_BF16_PEAK_TFLOPS, 4),
             "tflops_strict": round(token_heads * flops["strict"] / (ms_per_step * 1e-3) / 1e12, 1),
+            "tflops_wy_count": round(token_heads * flops["wy"] / (ms_per_step * 1e-3) / 1e12, 1),
             "algorithmic_gbs": round(algo_bytes / (ms_per_step * 1e-3) / 1e9, 1),
             "hbm_frac": round(algo_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
             "kernels": per_kernel,

@@ -119,14 +119,18 @@ CHUNK = 64
 
 
 def chunk_fwd_flops_per_token_head(K: int, V: int, C: int = CHUNK) -> dict:
-    """Dense count of the eight contractions of the chunked forward, per token and head:
-    K K^T, T (beta e^gamma K), T (beta V), Q K^T  -> "prepare" = 2 C (3K + V)
-    W S, Q S, K~^T V~, P V~                        -> "scan"    = 2 (3 K V + C V)
-    Triangular solve and all elementwise work are excluded; padding is never counted."""
-    prepare = 2 * C * (3 * K + V)
-    scan = 2 * (3 * K * V + C * V)
-    strict = 2 * ((C // 2) * (3 * K + 2 * V) + 3 * K * V)
-    return {"prepare": prepare, "scan": scan, "dense": prepare + scan, "strict": strict}
+    """Dense count of the contractions of the chunked forward as the kernels run it, per token and head:
+    K K^T, Q K^T                                   -> "prepare" = 2 C (2K)
+    K S0, Q S0, K^T V~ (K x V each), T' X, P V~    -> "scan"    = 2 (3 K V + 2 C V)
+    with V~ = T diag(beta) (V - diag(cs) K S0): the product T (beta e^gamma K) of the WY form (2 C K) is never
+    formed.  "wy" is the count of the WY form's eight contractions, 2 (C (3K + 2V) + 3 K V), for comparison with
+    figures quoted on that count.  Triangular solve and all elementwise work are excluded; padding is never
+    counted.  "strict" halves the products with a triangular factor."""
+    prepare = 2 * C * (2 * K)
+    scan = 2 * (3 * K * V + 2 * C * V)
+    strict = 2 * ((C // 2) * (2 * K + 2 * V) + 3 * K * V)
+    wy = 2 * (C * (3 * K + 2 * V) + 3 * K * V)
+    return {"prepare": prepare, "scan": scan, "dense": prepare + scan, "strict": strict, "wy": wy}
 
 
 def chunk_fwd_bytes_per_token_head(K: int, V: int, in_bytes: int = 2) -> int:
