@@ -2,16 +2,18 @@
 // (the only bf16 MFMA shape that reaches the full matrix-core rate on gfx950; 16x16x32 measured
 // ~0.8x of it).
 //
-// Same mathematics and the same two-kernel split as gdn_chunk.hip (prepare: everything that
-// does not depend on the state, written as MFMA operand fragments to a workspace record per
-// (head, chunk); scan: the serial pass over the chunks of a sequence with the state held in
-// MFMA accumulators).  What differs:
+// Two kernels as in gdn_chunk.hip (prepare: what does not depend on the state, written as MFMA
+// operand fragments to a workspace record per (head, chunk); scan: the serial pass over the chunks
+// of a sequence with the state held in MFMA accumulators), but with the WY form's T pulled out:
+//     V~ = U - W S0 = T diag(beta) (V - diag(cs) K S0),      cs = e^{gamma} / |k|
+// so the record holds T diag(beta) and P only, prepare never touches V, and the scan works from the
+// caller's q, k and v.  Further:
 //
 //   * a wave of the scan owns a K x 32 slice of the state; operand fragments are laid out for
 //     the 32x32x16 shape;
-//   * the scan stages each record in an LDS double buffer filled by dedicated loader waves, hands its
-//     output to a dedicated store wave, and keeps its compute waves free of memory instructions;
-//   * prepare is persistent: a workgroup walks over (chunk, head) items and loads q, k, v of
+//   * the scan stages everything a chunk needs in an LDS double buffer filled by dedicated loader waves,
+//     hands its output to a dedicated store wave, and keeps its compute waves free of memory instructions;
+//   * prepare is persistent: a workgroup walks over (chunk, head) items and loads q, k of
 //     the next item into registers while it computes the current one;
 //   * the triangular inverse runs its block products on bf16 MFMA with operands split into
 //     hi + lo halves (error ~2^-16, far below the final bf16 rounding of T), and transposed
@@ -26,20 +28,17 @@
 // The state keeps its rows (key dim) and its columns in the order slice_col (bits 2 and 3 of the
 // index within a 32-block swapped): MFMA row i of a state tile is key column slice_col(i), so the 8
 // entries a lane half contributes per slab are the 8 consecutive key columns 16 s + 8 h + 0..7.
-// Prepare reads K through the transposing LDS load in that order at no cost, and the scan can use
-// q and k straight from their row-major rows.  (The token index of V~, where it is the reduction
-// index of K^T V~ and P V~, keeps the MFMA order; the scan's transposing LDS reads of k and the P
-// fragments are built to match.)
+// So the scan uses q and k straight from their row-major rows.  (The token index, where it is the
+// reduction index - of T' X, K^T V~ and P V~ - keeps the MFMA order; the T' and P fragments and the scan's
+// transposing LDS reads of k are built to match.)
 //
 // Record:
-//   W~  = -W       [T_tok 2][slab K/16]  A fragments, rows = tokens, reduction = key dim
-//   P              6 fragments           B fragments of O^T += V~^T P^T: (query tile 0; key slabs 0, 1),
+//   T' = T diag(beta)   6 fragments      A fragments of V~ = T' X, rows = tokens: (token tile 0; X slabs 0, 1),
+//                                        (token tile 1; X slabs 0..3); the zero quarter above the diagonal is not stored
+//   P                   6 fragments      B fragments of O^T += V~^T P^T: (query tile 0; key slabs 0, 1),
 //                                        (query tile 1; key slabs 0..3); P[i < 32][j >= 32] = 0 is not stored
-//   U              [T_n V/32][T_tok 2][half 2][lane][8]  accumulator layout (registers 8 half .. 8 half + 7 of token
-//                  tile T_tok), lane l32 = column slice_col(l32) of the tile
-//   64 fp32 row scales of q (e^{gamma} scale / |q|), 64 of k (e^{gamma_C - gamma} / |k|), e^{gamma_C}
-// q and k themselves are not copied: the scan reads their rows from the caller's tensors, applies
-// q's scales to the rows of the output tile and k's to the rows of V~ before the state update.
+//   64 fp32 row scales of q (e^{gamma} scale / |q|), 64 of k for the state update (e^{gamma_C - gamma} / |k|),
+//   64 of k for K S0 (e^{gamma} / |k|), e^{gamma_C}
 
 #include <type_traits>
 
