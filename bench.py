@@ -44,7 +44,7 @@ MEASURED_HBM_TRAFFIC_BYTES = {
     ("cfg1_chunk_fwd_bf16", "chunk_prepare"): (2.0 * 66468.2 + 52352.0) * _KIB,
     ("cfg1_chunk_fwd_bf16", "chunk_scan"): (2.0 * 124827.2 + 69632.0) * _KIB,
     ("cfg3_decode_bf16", "recurrent_kernel"): (2.0 * 265449.7 + 526881.4) * _KIB,
-    ("cfg1_chunk_fwd_bf16", "causal_conv1d_kernel"): (2.0 * 116926.8 + 196752.0) * _KIB,
+    ("cfg1_chunk_fwd_bf16", "causal_conv1d_kernel"): (2.0 * 103205.2 + 196752.0) * _KIB,
     ("cfg1_chunk_fwd_bf16", "gated_rmsnorm_kernel"): (2.0 * 66081.4 + 65536.0) * _KIB,
 }
 

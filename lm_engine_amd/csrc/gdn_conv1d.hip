@@ -7,7 +7,8 @@
 //
 // A thread owns 16 bytes of channels (8 bf16 / 4 fp32) and walks TOKENS consecutive tokens with
 // the kernel_size - 1 previous rows in registers, so inside a block every row of x is read once;
-// neighbouring token blocks re-read kernel_size - 1 rows of halo.  Lanes cover consecutive channel
+// neighbouring token blocks share kernel_size - 1 rows of halo and are walked in opposite directions, so
+// that both read them at the same moment.  Lanes cover consecutive channel
 // vectors: every load and store of a wave is one contiguous row segment; the four waves of a
 // workgroup take consecutive token blocks of the same channels.
 
@@ -89,26 +90,19 @@ __global__ __launch_bounds__(CONV_THREADS) void causal_conv1d_kernel(const ConvP
         for (int e = 0; e < VEC; e++) row[e] = (float)v[e] * m;
     };
 
-    // the kernel_size - 1 rows before this block: masked inputs, the carried state, or zeros
-    float hist[KS - 1][VEC];
-#pragma unroll
-    for (int j = 0; j < KS - 1; j++) {
-        const int s = s_begin - (KS - 1) + j;
+    // row s of the (masked) input for s >= 0, the carried state or zeros for the kernel_size - 1 rows before the sequence
+    auto load_any = [&](int s, float (&row)[VEC]) {
         if (s >= 0) {
-            load_row(s, hist[j]);
+            load_row(s, row);
         } else {
 #pragma unroll
             for (int e = 0; e < VEC; e++)
-                hist[j][e] = p.input_state == nullptr
-                                 ? 0.f
-                                 : (float)reinterpret_cast<const T*>(p.input_state)[((int64_t)b * p.C + c0 + e) * (KS - 1) + (KS - 1) + s];
+                row[e] = p.input_state == nullptr
+                             ? 0.f
+                             : (float)reinterpret_cast<const T*>(p.input_state)[((int64_t)b * p.C + c0 + e) * (KS - 1) + (KS - 1) + s];
         }
-    }
-
-#pragma unroll 8
-    for (int s = s_begin; s < s_end; s++) {
-        float cur[VEC];
-        load_row(s, cur);
+    };
+    auto emit = [&](int s, const float (&cur)[VEC], const float (&hist)[KS - 1][VEC]) {  // hist[j] = row s - (KS - 1) + j
         const float m = mb == nullptr ? 1.f : (float)mb[s];
         vec_t out;
 #pragma unroll
@@ -120,20 +114,66 @@ __global__ __launch_bounds__(CONV_THREADS) void causal_conv1d_kernel(const ConvP
             out[e] = (T)(acc * m);
         }
         *reinterpret_cast<vec_t*>(yb + (int64_t)s * p.y_stride_s) = out;
-#pragma unroll
-        for (int e = 0; e < VEC; e++) {
-#pragma unroll
-            for (int j = 0; j + 1 < KS - 1; j++) hist[j][e] = hist[j + 1][e];
-            hist[KS - 2][e] = cur[e];
-        }
-    }
+    };
 
-    if (p.final_state != nullptr && s_end == p.S) {
-        T* fs = reinterpret_cast<T*>(p.final_state) + ((int64_t)b * p.C + c0) * (KS - 1);
+    // Token blocks are walked in alternating directions: an even block from its last token down, an odd one
+    // from its first token up.  The kernel_size - 1 rows two neighbouring blocks have in common are then read
+    // by both at the same moment - at the start of both walks or at the end of both - and come out of the
+    // cache; walked the same way, the second reader comes a whole walk later and fetches them from memory
+    // again (measured: 19 % more bytes fetched than the input holds, 5 % this way; the kernel time did not
+    // change, it streams at the rate of a plain copy either way).
+    const bool downward = ((s_begin / CONV_TOKENS) & 1) == 0;
+    float hist[KS - 1][VEC];
+    if (!downward) {
 #pragma unroll
-        for (int e = 0; e < VEC; e++)
+        for (int j = 0; j < KS - 1; j++) load_any(s_begin - (KS - 1) + j, hist[j]);
+#pragma unroll 8
+        for (int s = s_begin; s < s_end; s++) {
+            float cur[VEC];
+            load_row(s, cur);
+            emit(s, cur, hist);
 #pragma unroll
-            for (int j = 0; j < KS - 1; j++) fs[e * (KS - 1) + j] = (T)hist[j][e];
+            for (int e = 0; e < VEC; e++) {
+#pragma unroll
+                for (int j = 0; j + 1 < KS - 1; j++) hist[j][e] = hist[j + 1][e];
+                hist[KS - 2][e] = cur[e];
+            }
+        }
+        if (p.final_state != nullptr && s_end == p.S) {
+            T* fs = reinterpret_cast<T*>(p.final_state) + ((int64_t)b * p.C + c0) * (KS - 1);
+#pragma unroll
+            for (int e = 0; e < VEC; e++)
+#pragma unroll
+                for (int j = 0; j < KS - 1; j++) fs[e * (KS - 1) + j] = (T)hist[j][e];
+        }
+    } else {
+        // cur = row s, hist[j] = row s - (KS - 1) + j; stepping down shifts the window the other way
+        float cur[VEC];
+        load_row(s_end - 1, cur);
+#pragma unroll
+        for (int j = 0; j < KS - 1; j++) load_any(s_end - 1 - (KS - 1) + j, hist[j]);
+        if (p.final_state != nullptr && s_end == p.S) {  // the last kernel_size - 1 inputs: hist[1..], cur
+            T* fs = reinterpret_cast<T*>(p.final_state) + ((int64_t)b * p.C + c0) * (KS - 1);
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+#pragma unroll
+                for (int j = 0; j + 1 < KS - 1; j++) fs[e * (KS - 1) + j] = (T)hist[j + 1][e];
+                fs[e * (KS - 1) + KS - 2] = (T)cur[e];
+            }
+        }
+#pragma unroll 8
+        for (int s = s_end - 1; s >= s_begin; s--) {
+            emit(s, cur, hist);
+            float next[VEC] = {};  // row s - KS, the new oldest row of the window around s - 1
+            if (s > s_begin) load_any(s - KS, next);
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+                cur[e] = hist[KS - 2][e];
+#pragma unroll
+                for (int j = KS - 2; j > 0; j--) hist[j][e] = hist[j - 1][e];
+                hist[0][e] = next[e];
+            }
+        }
     }
 }
 
