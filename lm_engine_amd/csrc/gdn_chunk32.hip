@@ -255,24 +255,36 @@ __global__ __launch_bounds__(PREP_THREADS, 3) void chunk_prepare32_kernel(const 
                     acc = mfma32_bf16(a, b, acc);
                     if (s % 2 == 1) __builtin_amdgcn_sched_barrier(0);  // keeps the operand reads from piling up in registers
                 }
+                // register quad q of the tile holds rows 32 trow + 8 q + 4 h + 0..3: their per-token values in one read
                 if (!is_p) {
                     const int j = 32 * tcol + l32;
                     const float gj = s_gam[j], rkj = s_rk[j];
 #pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const int i = 32 * trow + 8 * (r / 4) + 4 * lh + r % 4;
-                        const float val = s_beta[i] * s_rk[i] * rkj * __expf(s_gam[i] - gj) * acc[r];
-                        sA[i * LDA + j] = (i > j) ? val : 0.f;
+                    for (int q = 0; q < 4; q++) {
+                        const int i0 = 32 * trow + 8 * q + 4 * lh;
+                        const f32x4 bi = *reinterpret_cast<const f32x4*>(&s_beta[i0]);
+                        const f32x4 ri = *reinterpret_cast<const f32x4*>(&s_rk[i0]);
+                        const f32x4 gi = *reinterpret_cast<const f32x4*>(&s_gam[i0]);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const float val = bi[e] * ri[e] * rkj * __expf(gi[e] - gj) * acc[4 * q + e];
+                            sA[(i0 + e) * LDA + j] = (i0 + e > j) ? val : 0.f;
+                        }
                     }
                 } else {
                     const int i = 32 * tcol + l32;
                     const float gi = s_gam[i], qi = p.scale * s_rq[i];
                     f32x16 pv;
 #pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const int j = 32 * trow + 8 * (r / 4) + 4 * lh + r % 4;
-                        const float val = qi * s_rk[j] * __expf(gi - s_gam[j]) * acc[r];
-                        pv[r] = (i >= j) ? val : 0.f;
+                    for (int q = 0; q < 4; q++) {
+                        const int j0 = 32 * trow + 8 * q + 4 * lh;
+                        const f32x4 rj = *reinterpret_cast<const f32x4*>(&s_rk[j0]);
+                        const f32x4 gj = *reinterpret_cast<const f32x4*>(&s_gam[j0]);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const float val = qi * rj[e] * __expf(gi - gj[e]) * acc[4 * q + e];
+                            pv[4 * q + e] = (i >= j0 + e) ? val : 0.f;
+                        }
                     }
                     // fragments (tcol, 2 trow + s); the all-zero pair (tcol 0, trow 1) has no place in the record
                     bf16x8* pf = reinterpret_cast<bf16x8*>(rec + p.off_p);
