@@ -526,12 +526,11 @@ struct ScanScheduleRules {
     static constexpr int t_tile(int j) { return j < 2 ? 0 : 1; }
     static constexpr int t_slab(int j) { return j < 2 ? j : j - 2; }
 
-    // pieces: X (4 registers; every second one also packs half a tile of X) | output hand-over (half a tile) | q row
-    // scale (4 registers) | decay (4 registers) | scaled V~ (half a fragment) | plain V~ (a fragment) | new state
-    // (a fragment)
-    static constexpr int N_XC = 8, N_OUT = 4, N_AS = 8, N_DEC = 4 * KD, N_VS = 8, N_VB = 4, N_SB = 2 * KD;
+    // pieces: X (4 registers) | output hand-over (half a tile) | q row scale (4 registers) | decay (4 registers) |
+    // scaled V~ (half a fragment) | plain V~ (a fragment) | new state (a fragment) | X as operand (a fragment)
+    static constexpr int N_XC = 8, N_OUT = 4, N_AS = 8, N_DEC = 4 * KD, N_VS = 8, N_VB = 4, N_SB = 2 * KD, N_XB = 4;
     static constexpr int P_XC = 0, P_OUT = P_XC + N_XC, P_AS = P_OUT + N_OUT, P_DEC = P_AS + N_AS, P_VS = P_DEC + N_DEC,
-                         P_VB = P_VS + N_VS, P_SB = P_VB + N_VB, NPIECES = P_SB + N_SB;
+                         P_VB = P_VS + N_VS, P_SB = P_VB + N_VB, P_XB = P_SB + N_SB, NPIECES = P_XB + N_XB;
 
     struct Window {
         int first, end;  // the piece runs before the MFMA of an op in [first, end)
@@ -541,9 +540,7 @@ struct ScanScheduleRules {
             const int tt = (pc - P_XC) / 4;
             return {KS16 * (tt + 1) + 1, OP_T + 2 * tt};
         }
-        if (pc < P_AS) {  // tile 0: this chunk's, after its two P ops; tile 1: the previous chunk's, before q overwrites it
-            return (pc - P_OUT) / 2 == 0 ? Window{OP_P + 3, NOPS} : Window{1, OP_Q + KS16};
-        }
+        if (pc < P_AS) return {1, OP_Q + KS16 * ((pc - P_OUT) / 2)};  // the previous chunk's tile, before q overwrites it
         if (pc < P_DEC) {
             const int tt = (pc - P_AS) / 4;
             const int end = OP_P + 2 * tt;
@@ -555,7 +552,9 @@ struct ScanScheduleRules {
             return {OP_T + (x / 2 == 0 ? 2 : 6) + 1, x < 2 ? OP_K + x : OP_K + NKF / 2 + (x - 2)};
         }
         if (pc < P_SB) return {OP_T + ((pc - P_VB) / 2 == 0 ? 2 : 6) + 1, OP_P};
-        return {OP_K + NKF / 2 + 2 * ((pc - P_SB) / 2) + 3, NOPS};
+        if (pc < P_XB) return {OP_K + NKF / 2 + 2 * ((pc - P_SB) / 2) + 3, NOPS};
+        const int tt = (pc - P_XB) / 2;  // after the two X pieces of its half tile (checked in make)
+        return {KS16 * (tt + 1) + 2, OP_T + 2 * tt};
     }
 
     struct Table {
@@ -580,9 +579,9 @@ struct ScanScheduleRules {
             }
         }
         if (left != 0) t.ok = false;
-        // the X pieces of a tile run in order (the odd ones pack what the even ones left)
-        for (int i = 1; i < N_XC; i++)
-            if (i % 4 != 0 && t.op[P_XC + i] < t.op[P_XC + i - 1]) t.ok = false;
+        // a half tile of X is packed after its two pieces (within an op the pieces run in index order: X before the pack)
+        for (int i = 0; i < N_XB; i++)
+            if (t.op[P_XB + i] < t.op[P_XC + 2 * i] || t.op[P_XB + i] < t.op[P_XC + 2 * i + 1]) t.ok = false;
         // a ring register (rings of four) is refilled only after the piece four places earlier has used it
         for (int i = 4; i < N_VS; i++)
             if (t.op[P_VS + i] - AHEAD <= t.op[P_VS + i - 4]) t.ok = false;
@@ -892,7 +891,7 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
 #pragma unroll
     for (int s = 0; s < KS16; s++) sb[s] = pack8_16(S[s / 2], s % 2, 1.f);
 
-    int valid_prev = 0;  // tokens of the previous chunk, the second half of whose output is still in acco[1]
+    int valid_prev = 0;  // tokens of the previous chunk, whose output is still in acco
     for (int c = 0; c < nchunks; c++) {
         const uint8_t* st = stage[c & 1];
         const uint8_t* stn = stage[(c + 1) & 1];
@@ -911,26 +910,19 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
                 constexpr int i = pc - SCH::P_XC, tt = i / 4, q4 = i % 4;
 #pragma unroll
                 for (int e = 0; e < 4; e++) accv[tt][4 * q4 + e] = (float)xvr[i % 4][e] - csr[i % 4][e] * accv[tt][4 * q4 + e];
-                if constexpr (q4 % 2 == 1) xb[2 * tt + q4 / 2] = pack8_16(accv[tt], q4 / 2, 1.f);
+            } else if constexpr (pc >= SCH::P_XB) {
+                constexpr int i = pc - SCH::P_XB;  // X as operand of T' X
+                xb[i] = pack8_16(accv[i / 2], i % 2, 1.f);
             } else if constexpr (pc >= SCH::P_OUT && pc < SCH::P_OUT + SCH::N_OUT) {
-                // output tile tt, registers 8 half .. 8 half + 7: tile 0 belongs to this chunk (its P terms are
-                // complete), tile 1 to the previous one
+                // output tile tt of the previous chunk, registers 8 half .. 8 half + 7
                 constexpr int i = pc - SCH::P_OUT, tt = i / 2, half = i % 2;
-                if constexpr (tt == 0) {
-                    if (OS) {
-                        *reinterpret_cast<bf16x8*>(ostage_at(wave, c & 1, l32, 2 * half + lh)) = pack8_16(acco[0], half, 1.f);
-                    } else if (l32 < valid) {
-                        *reinterpret_cast<bf16x8*>(og + 16 * half) = pack8_16(acco[0], half, 1.f);
-                    }
-                } else {
-                    if (OS) {
-                        if (c > 0)
-                            *reinterpret_cast<bf16x8*>(ostage_at(wave, (c - 1) & 1, 32 + l32, 2 * half + lh)) =
-                                pack8_16(acco[1], half, 1.f);
-                    } else if (32 + l32 < valid_prev) {
-                        *reinterpret_cast<bf16x8*>(og - og_step + (int64_t)32 * p.o_stride_t + 16 * half) =
-                            pack8_16(acco[1], half, 1.f);
-                    }
+                if (OS) {
+                    if (c > 0)
+                        *reinterpret_cast<bf16x8*>(ostage_at(wave, (c - 1) & 1, 32 * tt + l32, 2 * half + lh)) =
+                            pack8_16(acco[tt], half, 1.f);
+                } else if (32 * tt + l32 < valid_prev) {
+                    *reinterpret_cast<bf16x8*>(og - og_step + (int64_t)(32 * tt) * p.o_stride_t + 16 * half) =
+                        pack8_16(acco[tt], half, 1.f);
                 }
             } else if constexpr (pc >= SCH::P_AS && pc < SCH::P_AS + SCH::N_AS) {
                 // O^T = (q S0)^T so far: its columns (tokens) take the row scale of q before the P terms are added
@@ -1033,16 +1025,20 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
         og += og_step;
     }
 
-    // the second half of the output of the last chunk
+    // the output of the last chunk
 #pragma unroll
-    for (int half = 0; half < 2; half++) {
-        if (OS) {
-            if (nchunks > 0)
-                *reinterpret_cast<bf16x8*>(ostage_at(wave, (nchunks - 1) & 1, 32 + l32, 2 * half + lh)) = pack8_16(acco[1], half, 1.f);
-        } else if (32 + l32 < valid_prev) {
-            *reinterpret_cast<bf16x8*>(og - og_step + (int64_t)32 * p.o_stride_t + 16 * half) = pack8_16(acco[1], half, 1.f);
+    for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            if (OS) {
+                if (nchunks > 0)
+                    *reinterpret_cast<bf16x8*>(ostage_at(wave, (nchunks - 1) & 1, 32 * tt + l32, 2 * half + lh)) =
+                        pack8_16(acco[tt], half, 1.f);
+            } else if (32 * tt + l32 < valid_prev) {
+                *reinterpret_cast<bf16x8*>(og - og_step + (int64_t)(32 * tt) * p.o_stride_t + 16 * half) =
+                    pack8_16(acco[tt], half, 1.f);
+            }
         }
-    }
     if (OS) __syncthreads();
 
     if (p.ht != nullptr) {
