@@ -117,7 +117,7 @@ __global__ __launch_bounds__(PREP_THREADS, 3) void chunk_prepare32_kernel(const 
     // the slot number and the heads rotate with the rest: every XCD works on all heads.  The rows of one head
     // lie a whole token row (a multiple of 2 KiB) apart, so they fall on few channels of an XCD's L2; an XCD
     // that only ever sees one or two heads would send all its q, k, v traffic there.
-    const int64_t items = (int64_t)((p.TC + 7) / 8) * 8 * p.H;
+    const uint32_t items = (uint32_t)((p.TC + 7) / 8) * 8u * (uint32_t)p.H;  // the launcher rejects more than 2^31
 
     // ---- register prefetch of one item's inputs ----
     bf16x8 kx[NPASS], qx[NPASS];
@@ -125,10 +125,10 @@ __global__ __launch_bounds__(PREP_THREADS, 3) void chunk_prepare32_kernel(const 
     uint32_t bx_raw = 0;  // beta of the prefetched item, raw bits: any arithmetic on it here would wait for every load in flight
     ChunkCoord ncc;  // coordinates of the prefetched item
     int nh = 0, nslot = 0;
-    auto locate = [&](int64_t w) {
-        const int64_t j = w / 8;
-        nh = (int)(j % p.H);
-        nslot = (int)(j / p.H) * 8 + (int)(w % 8);
+    auto locate = [&](uint32_t w) {  // wave-uniform 32-bit arithmetic
+        const uint32_t j = w / 8u, jh = j / (uint32_t)p.H;
+        nh = (int)(j - jh * (uint32_t)p.H);
+        nslot = (int)(jh * 8u + w % 8u);
         ncc = locate_chunk(p, nslot);
     };
     // Loads are written as (workgroup-uniform base pointer) + (32-bit per-lane element offset) so that the
@@ -162,7 +162,7 @@ __global__ __launch_bounds__(PREP_THREADS, 3) void chunk_prepare32_kernel(const 
             }
         }
     };
-    int64_t w = blockIdx.x;
+    uint32_t w = blockIdx.x;
     if (w >= items) return;
     locate(w);
     prefetch_kq();
@@ -1056,6 +1056,7 @@ template <int K>
 static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int num_cus) {
     const int64_t items = (int64_t)((p.TC + 7) / 8) * 8 * p.H;  // a multiple of 8, see the kernel
     const int64_t cap = (int64_t)(3 * num_cus + 7) / 8 * 8;      // three workgroups per CU (LDS and registers allow it)
+    if (items >= ((int64_t)1 << 31)) return GDN_ERR_UNSUPPORTED;  // the kernel counts items in 32 bits
     const int grid_prep = (int)(items < cap ? items : cap);
     hipLaunchKernelGGL((chunk_prepare32_kernel<K>), dim3(grid_prep), dim3(PREP_THREADS), 0, stream, p);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
