@@ -61,6 +61,40 @@ def test_many_chains_share_records_in_a_workgroup(B, T, H, K, V, slices_per_work
     _check(inp, f"B={B} H={H} K={K} V={V}: {slices_per_workgroup} slice(s) per workgroup")
 
 
+def _sweep_case(i):
+    gen = torch.Generator("cpu").manual_seed(9000 + i)
+    pick = lambda xs: xs[int(torch.randint(len(xs), (1,), generator=gen))]  # noqa: E731
+    K = pick([64, 128])
+    V = pick([32, 64, 96, 128, 160, 192, 256])
+    H = pick([1, 2, 3, 4, 8])
+    T = int(torch.randint(1, 400, (1,), generator=gen))
+    B = pick([1, 1, 2, 3, 5])
+    return dict(
+        B=B, T=T, H=H, K=K, V=V,
+        l2norm=pick([False, True]), h0=pick([False, True]), gated=pick([True, True, False]),
+        g_mean=pick([-1.0, 1.0, 3.0]), packed=B == 1 and T >= 8 and pick([False, True]),
+    )  # fmt: skip
+
+
+@pytest.mark.parametrize("i", range(16))
+def test_seeded_sweep_of_shapes_and_options(i):
+    # shapes and switches drawn from a seeded generator: head dims, column tiles that do not divide evenly over
+    # the workgroup sizes, ragged lengths, packed sequences, state in / no state, ungated, in-kernel l2norm
+    c = _sweep_case(i)
+    kwargs = dict(use_qk_l2norm_in_kernel=True) if c["l2norm"] else {}
+    n_seq, cu = None, None
+    if c["packed"]:
+        gen = torch.Generator("cpu").manual_seed(9100 + i)
+        cuts = sorted(set(int(x) for x in torch.randint(1, c["T"], (3,), generator=gen)))
+        cu = torch.tensor([0] + cuts + [c["T"]], dtype=torch.int32)
+        n_seq = cu.numel() - 1
+    inp = random_inputs(B=c["B"], T=c["T"], H=c["H"], K=c["K"], V=c["V"], dtype=BF16, seed=9200 + i, gated=c["gated"],
+                        h0=c["h0"], g_mean=c["g_mean"], normalize=not c["l2norm"], N=n_seq)  # fmt: skip
+    if cu is not None:
+        inp = dict(inp, cu_seqlens=cu)
+    _check(inp, f"sweep {i}: {c}", **kwargs)
+
+
 def test_short_sequence_single_partial_chunk():
     _check(random_inputs(B=3, T=17, H=2, K=128, V=128, dtype=BF16, seed=70), "T=17")
 
