@@ -73,6 +73,13 @@ __device__ __forceinline__ bf16x4 lds_read_tr4x16(const bf16_t* m, int ld, int r
 // register pair (2 m, 2 m + 1) of a transposed accumulator tile covers 8 consecutive columns per lane.
 __device__ __forceinline__ int slice_col(int l32) { return (l32 & 0x13) | ((l32 & 4) << 1) | ((l32 & 8) >> 1); }
 
+// x of another lane as named by a DPP control word; lanes the move does not write (outside ROW_MASK, or shifted in
+// from outside their row) get 0
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_move(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, ROW_MASK, 0xF, false));
+}
+
 __device__ __forceinline__ void split_hi_lo(float x, bf16_t& hi, bf16_t& lo) {
     hi = (bf16_t)x;
     lo = (bf16_t)(x - (float)hi);
@@ -206,12 +213,16 @@ __global__ __launch_bounds__(PREP_THREADS, 3) void chunk_prepare32_kernel(const 
                 }
             }
             if (wave == 0) {
+                // inclusive prefix sum over the 64 lanes in data-parallel-primitive moves (shifts inside a row of 16
+                // lanes with zero fill, then the last lane of a row broadcast to the rows above): six dependent adds
+                // instead of six round trips through the LDS crossbar
                 float gv = gx;
-#pragma unroll
-                for (int off = 1; off < WAVE; off <<= 1) {
-                    const float up = __shfl_up(gv, off, WAVE);
-                    if (lane >= off) gv += up;
-                }
+                gv += dpp_move<0x111, 0xF>(gv);  // row_shr:1
+                gv += dpp_move<0x112, 0xF>(gv);  // row_shr:2
+                gv += dpp_move<0x114, 0xF>(gv);  // row_shr:4
+                gv += dpp_move<0x118, 0xF>(gv);  // row_shr:8
+                gv += dpp_move<0x142, 0xA>(gv);  // row_bcast:15 into rows 1 and 3
+                gv += dpp_move<0x143, 0xC>(gv);  // row_bcast:31 into rows 2 and 3
                 s_gam[lane] = gv;
                 s_beta[lane] = __builtin_bit_cast(float, (p.beta != nullptr && p.beta_dtype == GDN_BF16) ? bx_raw << 16 : bx_raw);
             }
