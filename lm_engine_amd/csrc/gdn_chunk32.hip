@@ -99,22 +99,19 @@ __global__ __launch_bounds__(PREP_THREADS, 3) void chunk_prepare32_kernel(const 
     constexpr int CPR = K / 8;  // 16 B pieces per row of K / Q
     constexpr int RPP = PREP_THREADS / CPR;  // rows per pass of the K / Q copy
     constexpr int NPASS = C / RPP;
-    constexpr int QT_BYTES = (C * LDK * 2 > C * LDA * 4) ? C * LDK * 2 : C * LDA * 4;
-
-    // K is dead once A and P are formed; the scratch blocks of the inverse take its place
-    constexpr int SCRATCH_FLOATS = 32 * LDT + 16 * LDM + 2 * 16 * LDM + 32 * LDT;
+    // K is dead once A and P are formed; the scratch blocks of the block merges take its place.  T is built in
+    // place of A, block by block.
+    constexpr int SCRATCH_FLOATS = 32 * LDT + 2 * 16 * LDM + 32 * LDT;
     constexpr int KM_BYTES = (C * LDK * 2 > SCRATCH_FLOATS * 4) ? C * LDK * 2 : SCRATCH_FLOATS * 4;
     __shared__ __attribute__((aligned(16))) uint8_t sKM[KM_BYTES];
-    __shared__ __attribute__((aligned(16))) uint8_t sQT[QT_BYTES];  // Q (bf16), then T (fp32)
+    __shared__ __attribute__((aligned(16))) bf16_t sQ[C * LDK];
     __shared__ __attribute__((aligned(16))) float sA[C * LDA];
     __shared__ __attribute__((aligned(16))) float s_gam[C], s_beta[C], s_ssk[C], s_ssq[C];
     __shared__ __attribute__((aligned(16))) float s_rk[C], s_rq[C];
-    bf16_t* const sQ = reinterpret_cast<bf16_t*>(sQT);
-    float* const sT = reinterpret_cast<float*>(sQT);
+    float* const sT = sA;
     bf16_t* const sK = reinterpret_cast<bf16_t*>(sKM);
     float* const sTtA = reinterpret_cast<float*>(sKM);  // transpose of the top-left 32 x 32 of T
-    float* const sTt2 = sTtA + 32 * LDT;                // transpose of diagonal block 2 of T
-    float* const sMt = sTt2 + 16 * LDM;                 // transposed products
+    float* const sMt = sTtA + 32 * LDT;                 // transposed products
     float* const sMtB = sMt + 2 * 16 * LDM;
 
     const int tid = threadIdx.x;
@@ -304,25 +301,23 @@ __global__ __launch_bounds__(PREP_THREADS, 3) void chunk_prepare32_kernel(const 
                     pf[(first + 1) * WAVE + lane] = pack8_16(pv, 1, 1.f);
                 }
             };
-            if (wave == 0) {
-                tile_job(false, 1, 0);
-                tile_job(false, 0, 0);
-            } else if (wave == 1) {
-                tile_job(true, 0, 1);
-                tile_job(true, 0, 0);
-            } else if (wave == 2) {
-                tile_job(false, 1, 1);
-            } else {
-                tile_job(true, 1, 1);  // P[i < 32][j >= 32] = 0 is not stored
-            }
+            // first the two diagonal tiles of A, which the inverse starts from, and two of the three tiles of P
+            if (wave == 0) tile_job(false, 0, 0);
+            else if (wave == 1) tile_job(true, 0, 0);
+            else if (wave == 2) tile_job(false, 1, 1);
+            else tile_job(true, 1, 1);  // P[i < 32][j >= 32] = 0 is not stored
+            __syncthreads();  // #3: the diagonal tiles of A are complete
+            // then wave 0 inverts the diagonal blocks (a long dependent chain on one wave) while two others
+            // finish the tiles: K and Q stay in place until barrier #4
+            if (wave == 1) tile_job(false, 1, 0);
+            else if (wave == 2) tile_job(true, 0, 1);
         }
-        __syncthreads();  // #3: A complete, Q consumed (its region becomes T)
 
-        // ---- wave 0: inverses of the four 16 x 16 diagonal blocks ----
+        // ---- wave 0: inverses of the four 16 x 16 diagonal blocks, written over the blocks of A ----
+        float x[16];  // column l16 of the inverse of block lq (wave 0)
         if (wave == 0) {
             const int blk = lq, j = l16;  // lane owns column j of block `blk`
             const float* a = &sA[(16 * blk) * LDA + 16 * blk];
-            float x[16];
 #pragma unroll
             for (int i = 0; i < 16; i++) {
                 f32x4 row[4];
@@ -333,39 +328,16 @@ __global__ __launch_bounds__(PREP_THREADS, 3) void chunk_prepare32_kernel(const 
                 for (int kk = 0; kk < i; kk++) part[kk % 4] -= row[kk / 4][kk % 4] * x[kk];
                 x[i] = (part[0] + part[1]) + (part[2] + part[3]);
             }
+            // every lane of the wave has read its block of A by now (one wave, program order)
 #pragma unroll
             for (int i = 0; i < 16; i++) sT[(16 * blk + i) * LDA + 16 * blk + j] = x[i];
-            // transposes used as B operands below; zero blocks above the diagonal where a product reads them
-            if (blk == 0) {
-#pragma unroll
-                for (int i = 0; i < 16; i++) sT[i * LDA + 16 + j] = 0.f;  // T block (0, 1)
-            }
-            if (blk < 2) {
-#pragma unroll
-                for (int c4 = 0; c4 < 4; c4++)
-                    *reinterpret_cast<f32x4*>(&sTtA[(16 * blk + j) * LDT + 16 * blk + 4 * c4]) =
-                        f32x4{x[4 * c4], x[4 * c4 + 1], x[4 * c4 + 2], x[4 * c4 + 3]};
-                if (blk == 1) {
-#pragma unroll
-                    for (int c4 = 0; c4 < 4; c4++)
-                        *reinterpret_cast<f32x4*>(&sTtA[(16 + j) * LDT + 4 * c4]) = f32x4{0.f, 0.f, 0.f, 0.f};
-                }
-            } else if (blk == 2) {
-#pragma unroll
-                for (int c4 = 0; c4 < 4; c4++)
-                    *reinterpret_cast<f32x4*>(&sTt2[j * LDM + 4 * c4]) = f32x4{x[4 * c4], x[4 * c4 + 1], x[4 * c4 + 2], x[4 * c4 + 3]};
-#pragma unroll
-                for (int i = 0; i < 16; i++) sT[(32 + i) * LDA + 48 + j] = 0.f;  // T block (2, 3)
-            }
         }
-        __syncthreads();  // #4: diagonal blocks of T
+        __syncthreads();  // #4: diagonal blocks of T, all of A and P; K and Q are dead
 
         // 16 x 16 x 16 product on one 16x16x32 MFMA pair with hi/lo split operands.
         // x = rows of X (8 consecutive reduction entries k' = 8 (lq % 2) + e of row l16),
         // y = rows of Y^T (same entries of column l16 of Y).  Returns X Y.
-        auto mm16 = [&](const float* xrow, const float* ytrow) -> f32x4 {
-            const f32x4 x0 = *reinterpret_cast<const f32x4*>(xrow), x1 = *reinterpret_cast<const f32x4*>(xrow + 4);
-            const f32x4 y0 = *reinterpret_cast<const f32x4*>(ytrow), y1 = *reinterpret_cast<const f32x4*>(ytrow + 4);
+        auto mm16v = [&](const f32x4 x0, const f32x4 x1, const f32x4 y0, const f32x4 y1) -> f32x4 {
             bf16x8 a1, b1, a2, b2;
 #pragma unroll
             for (int e = 0; e < 8; e++) {
@@ -381,6 +353,10 @@ __global__ __launch_bounds__(PREP_THREADS, 3) void chunk_prepare32_kernel(const 
             acc = mfma_bf16(a1, b1, acc);
             acc = mfma_bf16(a2, b2, acc);
             return acc;
+        };
+        auto mm16 = [&](const float* xrow, const float* ytrow) -> f32x4 {
+            return mm16v(*reinterpret_cast<const f32x4*>(xrow), *reinterpret_cast<const f32x4*>(xrow + 4),
+                         *reinterpret_cast<const f32x4*>(ytrow), *reinterpret_cast<const f32x4*>(ytrow + 4));
         };
         // 16 x 16 output tile of a product with 32 reduction entries (k = 8 lq + e), hi/lo split: 3 MFMAs
         auto mm16x32 = [&](const float* xrow, const float* ytrow) -> f32x4 {
@@ -406,12 +382,32 @@ __global__ __launch_bounds__(PREP_THREADS, 3) void chunk_prepare32_kernel(const 
             const int bi = 2 * wave + 1, bj = 2 * wave;
             const int kk = 8 * (lq % 2);
             float* const mt = &sMt[wave * 16 * LDM];
-            const float* ttrow = (wave == 0) ? &sTtA[l16 * LDT + kk] : &sTt2[l16 * LDM + kk];  // (T_bj,bj)^T row l16
-            const f32x4 m = mm16(&sA[(16 * bi + l16) * LDA + 16 * bj + kk], ttrow);
+            // column l16 of T_bj,bj, entries kk .. kk + 7 (a row of its transpose)
+            f32x4 y0, y1;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                y0[e] = sT[(16 * bj + kk + e) * LDA + 16 * bj + l16];
+                y1[e] = sT[(16 * bj + kk + 4 + e) * LDA + 16 * bj + l16];
+            }
+            const float* arow = &sA[(16 * bi + l16) * LDA + 16 * bj + kk];
+            const f32x4 m = mm16v(*reinterpret_cast<const f32x4*>(arow), *reinterpret_cast<const f32x4*>(arow + 4), y0, y1);
+            if (wave == 0 && lq < 2) {
+                // K's region is free now: the transposes of T_00 and T_11 for level B, from the registers of the inverse,
+                // and the zero block (T_01)^T
+#pragma unroll
+                for (int c4 = 0; c4 < 4; c4++)
+                    *reinterpret_cast<f32x4*>(&sTtA[(16 * lq + l16) * LDT + 16 * lq + 4 * c4]) =
+                        f32x4{x[4 * c4], x[4 * c4 + 1], x[4 * c4 + 2], x[4 * c4 + 3]};
+                if (lq == 1) {
+#pragma unroll
+                    for (int c4 = 0; c4 < 4; c4++)
+                        *reinterpret_cast<f32x4*>(&sTtA[(16 + l16) * LDT + 4 * c4]) = f32x4{0.f, 0.f, 0.f, 0.f};
+                }
+            }
             *reinterpret_cast<f32x4*>(&mt[l16 * LDM + 4 * lq]) = m;  // M^T[n][4 lq + e]
             const f32x4 t = mm16(&sT[(16 * bi + l16) * LDA + 16 * bi + kk], &mt[l16 * LDM + kk]);
 #pragma unroll
-            for (int e = 0; e < 4; e++) sT[(16 * bi + 4 * lq + e) * LDA + 16 * bj + l16] = -t[e];
+            for (int e = 0; e < 4; e++) sT[(16 * bi + 4 * lq + e) * LDA + 16 * bj + l16] = -t[e];  // over A_bi,bj, read above
             if (wave == 0) *reinterpret_cast<f32x4*>(&sTtA[l16 * LDT + 16 + 4 * lq]) = -t;  // (T_10)^T
         }
         __syncthreads();  // #5
