@@ -157,15 +157,16 @@ def bench_decode(steps, warmup):
     for i in range(warmup):
         call(i)
     torch.cuda.synchronize()
-    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    # one pair of events around all the launches: a pair per launch adds its own handling (~5 us) to every bracket
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
-    for i, (start, stop) in enumerate(events):
-        start.record()
+    start.record()
+    for i in range(steps):
         call(i)
-        stop.record()
+    stop.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) / steps * 1e3
-    kernel_ms = sum(start.elapsed_time(stop) for start, stop in events) / steps
+    kernel_ms = start.elapsed_time(stop) / steps
     nbytes = decode_bytes_per_seq_head(w.K, w.V) * w.B * w.H
     gbs = nbytes / (kernel_ms * 1e-3) / 1e9
     return {
@@ -197,13 +198,13 @@ def bench_conv(w, steps, warmup):
     for _ in range(warmup):
         call()
     torch.cuda.synchronize()
-    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
-    for start, stop in events:
-        start.record()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
         call()
-        stop.record()
+    stop.record()
     torch.cuda.synchronize()
-    kernel_ms = sum(start.elapsed_time(stop) for start, stop in events) / steps
+    kernel_ms = start.elapsed_time(stop) / steps  # back-to-back launches, one pair of events around all of them
     nbytes = 2 * x.numel() * x.element_size()
     gbs = nbytes / (kernel_ms * 1e-3) / 1e9
     return {
