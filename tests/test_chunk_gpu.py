@@ -4,6 +4,8 @@ Every case feeds the GPU and the oracle the same bf16-rounded tensors; the gate 
 the benchmark contract for bf16 inputs: max-abs <= 2e-2 and relative-L2 <= 1e-2 on both the
 output and the final state."""
 
+import os
+
 import pytest
 import torch
 
@@ -76,7 +78,7 @@ def _sweep_case(i):
     )  # fmt: skip
 
 
-@pytest.mark.parametrize("i", range(16))
+@pytest.mark.parametrize("i", range(int(os.environ.get("GDN_SWEEP_CASES", "16"))))
 def test_seeded_sweep_of_shapes_and_options(i):
     # shapes and switches drawn from a seeded generator: head dims, column tiles that do not divide evenly over
     # the workgroup sizes, ragged lengths, packed sequences, state in / no state, ungated, in-kernel l2norm
