@@ -11,7 +11,7 @@ use_qk_l2norm_in_kernel`` and both returning ``(o, final_state)``:
 Both are provided here with the same names, argument meaning and return convention, on top
 of the HIP library (``libgdn_hip.so``, C ABI in include/gdn_hip.h).  PyTorch only owns the
 device memory and the stream; there is no eager or CPU fallback: without the library every
-call raises.
+call raises.  Both are differentiable (``backward.py``).
 
     q, k            [B, T, H, K]   bf16 (or fp32), last dim contiguous
     v               [B, T, H, V]
@@ -29,6 +29,7 @@ import ctypes
 import torch
 
 from . import _lib
+from .backward import gated_delta_rule_backward
 from .kernels import Kernel, is_kernel_allowed
 
 
@@ -196,26 +197,37 @@ def chunk_forward_kernel_times(
     return dict(zip(_lib.CHUNK_KERNEL_NAMES, (float(x) for x in times)))
 
 
-class _ForwardOnly(torch.autograd.Function):
-    """The operator has no backward yet; differentiating through it must fail, not pass silently."""
+class _GatedDeltaRule(torch.autograd.Function):
+    """Forward on the HIP kernels; backward by ``backward.gated_delta_rule_backward`` from the saved
+    inputs (the forward keeps no intermediate results)."""
 
     @staticmethod
     def forward(ctx, mode, scale, output_final_state, l2norm, inplace_state, left_padded, q, k, v, g, beta,
                 initial_state, cu_seqlens):  # fmt: skip
+        if inplace_state:
+            raise ValueError("inplace_state overwrites the initial state the backward needs; it is for inference")
         o, ht = _run(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm,
                      inplace_state, left_padded)  # fmt: skip
+        ctx.save_for_backward(q, k, v, g, beta, initial_state, cu_seqlens)
+        ctx.options = (scale, l2norm, left_padded)
         return o, ht
 
     @staticmethod
-    def backward(ctx, *grads):
-        raise NotImplementedError("the HIP gated delta rule is forward-only; its backward is not implemented")
+    def backward(ctx, do, dht):
+        q, k, v, g, beta, initial_state, cu_seqlens = ctx.saved_tensors
+        scale, l2norm, left_padded = ctx.options
+        dq, dk, dv, dg, dbeta, dh0 = gated_delta_rule_backward(
+            q, k, v, g, beta, do, dht, scale=scale, initial_state=initial_state, cu_seqlens=cu_seqlens,
+            use_qk_l2norm_in_kernel=l2norm, left_padded=left_padded,
+        )  # fmt: skip
+        return None, None, None, None, None, None, dq, dk, dv, dg, dbeta, dh0, None
 
 
 def _dispatch(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm, inplace_state,
               left_padded=False):
     tensors = (q, k, v, g, beta, initial_state)
     if torch.is_grad_enabled() and any(x is not None and x.requires_grad for x in tensors):
-        return _ForwardOnly.apply(mode, scale, output_final_state, l2norm, inplace_state, left_padded, q, k, v, g,
+        return _GatedDeltaRule.apply(mode, scale, output_final_state, l2norm, inplace_state, left_padded, q, k, v, g,
                                   beta, initial_state, cu_seqlens)  # fmt: skip
     return _run(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm, inplace_state,
                 left_padded)  # fmt: skip

@@ -155,9 +155,8 @@ def test_output_final_state_false_returns_none_and_runs_are_bitwise_repeatable()
     assert torch.equal(o1, o2)
 
 
-def test_backward_is_refused():
+def test_inplace_state_is_refused_when_gradients_are_needed():
     inp = _to_gpu(random_inputs(B=1, T=4, H=1, K=64, V=64, dtype=torch.float32, seed=47))
     inp["v"].requires_grad_(True)
-    o, _ = lm_engine_amd.fused_recurrent_gated_delta_rule(**inp)
-    with pytest.raises(NotImplementedError):
-        o.sum().backward()
+    with pytest.raises(ValueError, match="inplace_state"):
+        lm_engine_amd.fused_recurrent_gated_delta_rule(**inp, output_final_state=True, inplace_state=True)
