@@ -119,6 +119,27 @@ int gdn_chunk_fwd(const gdn_args *args, void *stream);
 int gdn_recurrent_fwd(const gdn_args *args, void *stream);
 
 /*
+ * Training support.  The reference differentiates through chunk_gated_delta_rule (chunk mode is asserted
+ * while training, gated_deltanet/module.py:194-209); a backward pass needs the state every chunk starts
+ * from and the chunk's V~ (the values written into the state), which gdn_chunk_fwd does not keep.
+ * gdn_chunk_fwd_saving is gdn_chunk_fwd (K <= 128) with a scan that also writes them, fp32:
+ *     states [N * H][chunks_per_chain][K][V]     chain n * H + h, chunk c of its sequence
+ *     v_new  [N * H][chunks_per_chain][64][V]    rows past the end of a sequence are not meaningful
+ * Either may be NULL.  Chunks c >= chunks_per_chain are computed but not saved.
+ * With records_given != 0 the prepare kernel is skipped: args->workspace then holds the chunk records
+ * themselves, [H][B * ceil(T / 64)] records in the layout prepare writes (fixed-length batches only;
+ * g, beta and the l2norm flag are not used, the records carry every scale).  The backward pass of this
+ * package runs its reverse sweep over the chunks that way.
+ */
+typedef struct gdn_chunk_saves {
+    float *states;
+    float *v_new;
+    int32_t chunks_per_chain;
+    int32_t records_given;
+} gdn_chunk_saves;
+int gdn_chunk_fwd_saving(const gdn_args *args, const gdn_chunk_saves *saves, void *stream);
+
+/*
  * Measurement aid, no counterpart in the reference: runs exactly what gdn_chunk_fwd runs, with a
  * HIP event recorded on `stream` before and after every kernel, waits for the last one and
  * returns each kernel's duration in milliseconds in kernel_ms[GDN_CHUNK_KERNELS], in launch

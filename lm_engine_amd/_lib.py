@@ -31,6 +31,7 @@ EXPORTED_SYMBOLS = (
     "gdn_chunk_fwd",
     "gdn_recurrent_fwd",
     "gdn_chunk_fwd_profile",
+    "gdn_chunk_fwd_saving",
     "gdn_causal_conv1d_fwd",
     "gdn_gates_fwd",
     "gdn_gated_rmsnorm_fwd",
@@ -38,6 +39,15 @@ EXPORTED_SYMBOLS = (
 
 GDN_CHUNK_KERNELS = 3
 CHUNK_KERNEL_NAMES = ("chunk_offsets", "chunk_prepare", "chunk_scan")
+
+
+class GdnChunkSaves(ctypes.Structure):
+    _fields_ = [
+        ("states", ctypes.c_void_p),
+        ("v_new", ctypes.c_void_p),
+        ("chunks_per_chain", ctypes.c_int32),
+        ("records_given", ctypes.c_int32),
+    ]
 
 
 class GdnArgs(ctypes.Structure):
@@ -121,6 +131,8 @@ def load_library() -> ctypes.CDLL:
     lib.gdn_recurrent_fwd.restype = ctypes.c_int
     lib.gdn_chunk_fwd_profile.argtypes = [ctypes.POINTER(GdnArgs), ctypes.c_void_p, ctypes.POINTER(ctypes.c_float)]
     lib.gdn_chunk_fwd_profile.restype = ctypes.c_int
+    lib.gdn_chunk_fwd_saving.argtypes = [ctypes.POINTER(GdnArgs), ctypes.POINTER(GdnChunkSaves), ctypes.c_void_p]
+    lib.gdn_chunk_fwd_saving.restype = ctypes.c_int
     lib.gdn_causal_conv1d_fwd.argtypes = [ctypes.POINTER(GdnConvArgs), ctypes.c_void_p]
     lib.gdn_causal_conv1d_fwd.restype = ctypes.c_int
     lib.gdn_gates_fwd.argtypes = [ctypes.POINTER(GdnGateArgs), ctypes.c_void_p]

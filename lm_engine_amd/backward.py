@@ -4,11 +4,22 @@ The reference trains through ``chunk_gated_delta_rule`` (chunk mode is asserted 
 lm_engine/modeling_utils/sequence_mixer_blocks/gated_deltanet/module.py:194-209), so autograd needs
 the gradients of ``(o, final_state)`` with respect to ``(q, k, v, g, beta, initial_state)``.
 
-This is the first, functional version: the per-chunk products are batched library GEMMs (fp32,
-``torch.bmm`` on the tensors' device) and the two sweeps over the chunks of a chain - forward to
-rebuild the chunk states, backward to carry the state gradient - are loops of such GEMMs.  It keeps
-the shape a fused kernel pipeline has (a state-saving forward scan, a reverse scan, one chunk-local
-gradient kernel); those kernels replace the corresponding blocks below one at a time.
+The chunk-local products are batched library GEMMs (fp32, ``torch.bmm`` on the tensors' device).  The
+two sweeps over the chunks of a chain - forward to rebuild the state every chunk starts from, backward
+to carry the state gradient - run on the HIP scan kernel for bf16 inputs with K <= 128
+(``gdn_chunk_fwd_saving``: the forward's scan in a variant that also writes the chunk states and V~),
+and as loops of batched GEMMs otherwise.
+
+The reverse sweep is the same recurrence as the forward one on other data, which is how it gets onto
+that kernel: with the tokens of a chain in reverse order (a transposed lower-triangular matrix is
+lower-triangular again), chunk c becomes two chunks of a "mirror" problem,
+
+    A:  v := P^T dO,  k := k,  T' := T^T,  row scales -(Kd's) and -(Kb's)       =>  V~ = Y = T^T dV~,
+        state: exp(gamma_C) dS1 - Kb^T Y
+    B:  v := dO,      k := q,  T' := I,    row scale Qe's, no decay             =>  state += Qe^T dO
+
+whose records are written here (``_mirror_problem``) instead of by the prepare kernel; the states the
+scan saves at the A chunks are dS1, its output there is Y.
 
 Chunk-local quantities (C = 64 tokens, gamma = prefix sum of g inside the chunk, e = exp(gamma),
 E_ij = exp(gamma_i - gamma_j) for j <= i):
@@ -19,8 +30,10 @@ E_ij = exp(gamma_i - gamma_j) for j <= i):
     P  = tril(Q K^T . E)                    Qe = diag(e) Q         Kd = diag(exp(gamma_C - gamma)) K
 
     forward sweep     V~ = U - W S0         S1 = exp(gamma_C) S0 + Kd^T V~        (O = Qe S0 + P V~)
-    reverse sweep     dV~ = P^T dO + Kd dS1
-                      dS0 = exp(gamma_C) dS1 + Qe^T dO - W^T dV~
+    reverse sweep     dV~ = P^T dO + Kd dS1       Y = T^T dV~
+                      dS0 = exp(gamma_C) dS1 + Qe^T dO - Kb^T Y
+    chunk-local       dP = tril(dO V~^T)    dQe = dO S0^T    dKd = V~ dS1^T    Z = Y S0^T
+                      dA = -stril(Y V~^T)   (the gradients with respect to Kb and Vb are -Z and Y)
 """
 
 from __future__ import annotations
@@ -89,6 +102,120 @@ def _l2norm_grad(y, r, dy):
     return r * (dy - y * (y * dy).sum(dim=-1, keepdim=True))
 
 
+def _sweeps_as_gemm_loops(S_init, dS_init, egl, Kd, Qe, Kb, Tm, Vb, P, doc):
+    """Both sweeps as loops of batched GEMMs (any dtype, any K).  Returns S0, V~, dS1, Y, dS0 of chunk 0."""
+    Bt, NC = egl.shape
+    K, V = S_init.shape[-2:]
+    dev = egl.device
+    W, U, Tt = Tm @ Kb, Tm @ Vb, Tm.transpose(-1, -2)
+    S = S_init.clone()
+    S0 = torch.empty(Bt, NC, K, V, device=dev)
+    Vn = torch.empty(Bt, NC, CHUNK, V, device=dev)
+    for c in range(NC):
+        S0[:, c] = S
+        Vn[:, c] = U[:, c] - W[:, c] @ S
+        S = egl[:, c, None, None] * S + Kd[:, c].transpose(-1, -2) @ Vn[:, c]
+    dS = dS_init.clone()
+    dS1 = torch.empty(Bt, NC, K, V, device=dev)
+    Y = torch.empty(Bt, NC, CHUNK, V, device=dev)
+    for c in reversed(range(NC)):
+        dS1[:, c] = dS
+        Y[:, c] = Tt[:, c] @ (P[:, c].transpose(-1, -2) @ doc[:, c] + Kd[:, c] @ dS)
+        dS = (egl[:, c, None, None] * dS + Qe[:, c].transpose(-1, -2) @ doc[:, c]
+              - Kb[:, c].transpose(-1, -2) @ Y[:, c])  # fmt: skip
+    return S0, Vn, dS1, Y, dS
+
+
+_FRAGMENT_INDEX = {}
+
+
+def _fragment_index(device):
+    """Where the entries of a lower-triangular 64 x 64 matrix sit in its six MFMA operand fragments of a chunk
+    record (the layout the prepare kernel writes for T diag(beta) and for P): fragment f < 2 covers rows
+    0..31 and columns 16 f .. 16 f + 15, fragment f >= 2 rows 32..63 and columns 16 (f - 2) ..; lane
+    l = l32 + 32 h holds, of row 32 (f >= 2) + l32, the columns 16 s + 4 h + 0..3 and 16 s + 8 + 4 h + 0..3."""
+    if device not in _FRAGMENT_INDEX:
+        f = torch.arange(6).view(6, 1, 1)
+        lane = torch.arange(64).view(1, 64, 1)
+        e = torch.arange(8).view(1, 1, 8)
+        tile = (f >= 2).long()
+        slab = torch.where(f < 2, f, f - 2)
+        rows = (32 * tile + lane % 32).expand(6, 64, 8)
+        cols = 16 * slab + 4 * (lane // 32) + torch.where(e < 4, e, e + 4)
+        _FRAGMENT_INDEX[device] = (rows.to(device), cols.to(device))
+    return _FRAGMENT_INDEX[device]
+
+
+RECORD_BYTES = 13312  # record of the 32x32x16 kernels (K <= 128): 12 fragments, 3 x 64 row scales, e^{gamma_C}
+
+
+def _mirror_problem(N, H, kraw, qraw, doc, Tm, P, egl, cs_a, ks_a, ks_b):
+    """Tensors and chunk records of the reverse sweep as a forward scan (see the module docstring).
+
+    Inputs are packed [N * H, NC, C, ...] fp32; ``cs_a``, ``ks_a``, ``ks_b`` are the row scales of the A and
+    B chunks in forward token order.  Returns k, v ``[N, 2 NC C, H, D]`` bf16 and the records as a uint8
+    tensor ``[H, N * 2 NC, RECORD_BYTES]``."""
+    Bt, NC = egl.shape
+    dev = egl.device
+    K, V = kraw.size(-1), doc.size(-1)
+    bf = torch.bfloat16
+
+    def mirrored(a_rows, b_rows):  # [Bt, NC, C, D] x 2 -> [N, 2 NC C, H, D]: chunks and tokens reversed, A before B
+        x = torch.stack((a_rows, b_rows), dim=2).flip(1, 3)  # [Bt, NC, 2, C, D]
+        D = x.size(-1)
+        return x.reshape(N, H, 2 * NC * CHUNK, D).transpose(1, 2).to(bf).contiguous()
+
+    U_bar = P.transpose(-1, -2) @ doc
+    k_m = mirrored(kraw, qraw)
+    v_m = mirrored(U_bar, doc)
+
+    rows, cols = _fragment_index(dev)
+    eye = torch.eye(CHUNK, device=dev)
+    # T^T with rows and columns reversed is lower-triangular again: entry (i', j') is T[63 - j', 63 - i']
+    Tmir = Tm.transpose(-1, -2).flip(-1, -2)
+    frag_t = Tmir[..., rows, cols].to(bf).reshape(Bt, NC, 6 * 512)
+    frag_i = eye[rows, cols].to(bf).reshape(6 * 512)
+
+    rec = torch.zeros(Bt, NC, 2, RECORD_BYTES // 2, dtype=bf, device=dev)
+    rec[:, :, 0, :3072] = frag_t.flip(1)          # A: T' := mirrored T^T
+    rec[:, :, 0, 3072:6144] = frag_i              #    P  := I, so that the output of the chunk is Y
+    rec[:, :, 1, :3072] = frag_i                  # B: T' := I; P stays 0
+    scal = rec.view(torch.float32)                # [Bt, NC, 2, 3328]: row scales of q | k (update) | k S0 | e^{gamma_C}
+    base = 6144 // 2
+    scal[:, :, 0, base + 64 : base + 128] = ks_a.flip(1, 2)
+    scal[:, :, 0, base + 128 : base + 192] = cs_a.flip(1, 2)
+    scal[:, :, 0, base + 192] = egl.flip(1)
+    scal[:, :, 1, base + 64 : base + 128] = ks_b.flip(1, 2)
+    scal[:, :, 1, base + 192] = 1.0
+    rec = rec.view(N, H, NC * 2, RECORD_BYTES // 2).transpose(0, 1).contiguous()
+    return k_m, v_m, rec.view(torch.uint8).reshape(H, N * NC * 2, RECORD_BYTES)
+
+
+def _sweeps_on_scan_kernel(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2norm, left_padded, pk, dht,
+                           kraw, qraw, doc, Tm, P, egl, cs_a, ks_a, ks_b):  # fmt: skip
+    """Both sweeps on the HIP scan kernel.  Returns S0, V~, dS1, Y, dS0 of chunk 0 (packed, fp32)."""
+    from . import ops  # late: ops imports this module
+
+    N, H, NC = pk.N, pk.H, pk.NC
+    Bt = N * H
+    K, V = q.size(-1), v.size(-1)
+    dev = q.device
+    S0 = torch.zeros(Bt, NC, K, V, device=dev)
+    Vn = torch.zeros(Bt, NC, CHUNK, V, device=dev)
+    ops.chunk_forward_saving(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2norm, left_padded, S0, Vn, NC)
+    live = pk.valid.reshape(N, 1, NC, CHUNK, 1).expand(N, H, NC, CHUNK, 1).reshape(Bt, NC, CHUNK, 1)
+    Vn = torch.where(live, Vn, torch.zeros_like(Vn))  # rows past the end of a sequence hold whatever the kernel left
+
+    k_m, v_m, rec = _mirror_problem(N, H, kraw, qraw, doc, Tm, P, egl, cs_a, ks_a, ks_b)
+    states = torch.empty(Bt, 2 * NC, K, V, device=dev)
+    dht32 = None if dht is None else dht.to(torch.float32).contiguous()
+    o_m, dS = ops.chunk_scan_given_records(k_m, v_m, rec, dht32, states, 2 * NC)
+    dS1 = states[:, 0::2].flip(1)
+    # the A chunks' output, back in forward order: [N, NC, 2, C, H, V] -> [Bt, NC, C, V]
+    Y = o_m.view(N, NC, 2, CHUNK, H, V)[:, :, 0].flip(1, 2).permute(0, 3, 1, 2, 4).reshape(Bt, NC, CHUNK, V).float()
+    return S0, Vn, dS1, Y, dS.reshape(Bt, K, V)
+
+
 def gated_delta_rule_backward(
     q, k, v, g, beta, do, dht=None, scale=None, initial_state=None, cu_seqlens=None,
     use_qk_l2norm_in_kernel=False, left_padded=False,
@@ -117,6 +244,7 @@ def gated_delta_rule_backward(
         kn, rk = _l2norm(kc)
     else:
         qn, kn = qc, kc
+        rq = rk = torch.ones(Bt, NC, CHUNK, 1, device=dev)
     qs = qn * scale
 
     incl = torch.ones(CHUNK, CHUNK, dtype=torch.bool, device=dev).tril(0)
@@ -134,58 +262,48 @@ def gated_delta_rule_backward(
     KK = kn @ kT
     A = bc[..., None] * E * KK * strict
     Tm = torch.linalg.solve_triangular(eye + A, eye.expand_as(A), upper=False)
-    Tt = Tm.transpose(-1, -2)
     Kb = kn * (bc * e)[..., None]
     Vb = vc * bc[..., None]
-    W = Tm @ Kb
-    U = Tm @ Vb
     P = E * (qs @ kT)
     Qe = qs * e[..., None]
     Kd = kn * tail[..., None]
 
-    # forward sweep: the state every chunk starts from, and V~
-    S = torch.zeros(Bt, K, V, device=dev)
-    if initial_state is not None:
-        S = initial_state.to(torch.float32).reshape(Bt, K, V).clone()
-    S0 = torch.empty(Bt, NC, K, V, device=dev)
-    Vn = torch.empty(Bt, NC, CHUNK, V, device=dev)
-    for c in range(NC):
-        S0[:, c] = S
-        Vn[:, c] = U[:, c] - W[:, c] @ S
-        S = egl[:, c, None, None] * S + Kd[:, c].transpose(-1, -2) @ Vn[:, c]
-
-    # reverse sweep: the gradient of the state every chunk ends with, and dV~
-    dS = torch.zeros(Bt, K, V, device=dev) if dht is None else dht.to(torch.float32).reshape(Bt, K, V).clone()
-    dS1 = torch.empty(Bt, NC, K, V, device=dev)
-    dVn = torch.empty(Bt, NC, CHUNK, V, device=dev)
-    for c in reversed(range(NC)):
-        dS1[:, c] = dS
-        dVn[:, c] = P[:, c].transpose(-1, -2) @ doc[:, c] + Kd[:, c] @ dS
-        dS = (egl[:, c, None, None] * dS + Qe[:, c].transpose(-1, -2) @ doc[:, c]
-              - W[:, c].transpose(-1, -2) @ dVn[:, c])  # fmt: skip
+    on_kernel = q.is_cuda and q.dtype == torch.bfloat16 and K <= 128 and V % 32 == 0
+    if on_kernel:
+        # the scan reads the raw rows of k and q; their norms and e^{gamma} go into the row scales
+        S0, Vn, dS1, Y, dS = _sweeps_on_scan_kernel(
+            q, k, v, g, beta, scale, initial_state, cu_seqlens, use_qk_l2norm_in_kernel, left_padded, pk, dht,
+            kc, qc, doc, Tm, P, egl,
+            cs_a=-(tail * rk[..., 0]), ks_a=-(bc * e * rk[..., 0]), ks_b=e * rq[..., 0] * scale,
+        )  # fmt: skip
+    else:
+        S_init = torch.zeros(Bt, K, V, device=dev)
+        if initial_state is not None:
+            S_init = initial_state.to(torch.float32).reshape(Bt, K, V)
+        dS_init = torch.zeros(Bt, K, V, device=dev) if dht is None else dht.to(torch.float32).reshape(Bt, K, V)
+        S0, Vn, dS1, Y, dS = _sweeps_as_gemm_loops(S_init, dS_init, egl, Kd, Qe, Kb, Tm, Vb, P, doc)
     dh0 = dS.reshape(N, H, K, V) if initial_state is not None else None
 
     # chunk-local gradients, all chunks at once
     S0t = S0.transpose(-1, -2)
-    dP = (doc @ Vn.transpose(-1, -2)) * incl
+    VnT = Vn.transpose(-1, -2)
+    dP = (doc @ VnT) * incl
     dQe = doc @ S0t
     dKd = Vn @ dS1.transpose(-1, -2)
-    dW = -(dVn @ S0t)
-    dKb = Tt @ dW
-    dVb = Tt @ dVn
-    dA = -(Tt @ (dW @ Kb.transpose(-1, -2) + dVn @ Vb.transpose(-1, -2)) @ Tt) * strict
+    Z = Y @ S0t          # the gradient with respect to Kb is -Z, the one with respect to Vb is Y
+    dA = -(Y @ VnT) * strict
 
     G = dP * E
     Hm = dA * bc[..., None] * E
     dqs = G @ kn + dQe * e[..., None]
-    dkn = (G.transpose(-1, -2) @ qs + dKd * tail[..., None] + dKb * (bc * e)[..., None]
+    dkn = (G.transpose(-1, -2) @ qs + dKd * tail[..., None] - Z * (bc * e)[..., None]
            + (Hm + Hm.transpose(-1, -2)) @ kn)  # fmt: skip
-    dvc = dVb * bc[..., None]
-    dbc = (dKb * kn * e[..., None]).sum(-1) + (dVb * vc).sum(-1) + (dA * E * KK).sum(-1)
+    dvc = Y * bc[..., None]
+    dbc = -(Z * kn * e[..., None]).sum(-1) + (Y * vc).sum(-1) + (dA * E * KK).sum(-1)
     MP = dP * P
     MA = dA * A
     n_kd = (dKd * Kd).sum(-1)
-    dgam = MP.sum(-1) - MP.sum(-2) + (dQe * Qe).sum(-1) - n_kd + (dKb * Kb).sum(-1) + MA.sum(-1) - MA.sum(-2)
+    dgam = MP.sum(-1) - MP.sum(-2) + (dQe * Qe).sum(-1) - n_kd - (Z * Kb).sum(-1) + MA.sum(-1) - MA.sum(-2)
     dgam[..., -1] += egl * (dS1 * S0).sum(dim=(-1, -2)) + n_kd.sum(-1)
     dgc = dgam.flip(-1).cumsum(-1).flip(-1)
 

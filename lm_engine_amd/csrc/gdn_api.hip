@@ -93,6 +93,23 @@ int gdn_chunk_fwd(const gdn_args* a, void* stream) {
     return gdn::launch_chunk_fwd(*a, static_cast<hipStream_t>(stream));
 }
 
+int gdn_chunk_fwd_saving(const gdn_args* a, const gdn_chunk_saves* saves, void* stream) {
+    if (saves == nullptr) return GDN_ERR_NULL;
+    const int rc = validate_common(a);
+    if (rc != GDN_OK) return rc;
+    if (!gdn::chunk_shape_supported(*a) || a->K > 128) return GDN_ERR_UNSUPPORTED;
+    if (saves->states == nullptr && saves->v_new == nullptr) return GDN_ERR_NULL;
+    if ((saves->states && !aligned(saves->states, 16)) || (saves->v_new && !aligned(saves->v_new, 16))) return GDN_ERR_ALIGN;
+    if (saves->chunks_per_chain <= 0) return GDN_ERR_SHAPE;  // chunks beyond it are computed but not saved
+    uint64_t need = gdn::chunk_workspace_bytes(*a);
+    if (saves->records_given) {
+        if (a->cu_seqlens != nullptr) return GDN_ERR_VARLEN;  // records are given for fixed-length batches only
+        need = gdn::chunk_record_bytes(*a);
+    }
+    if (a->workspace == nullptr || a->workspace_bytes < need || !aligned(a->workspace, 256)) return GDN_ERR_WORKSPACE;
+    return gdn::launch_chunk_fwd(*a, static_cast<hipStream_t>(stream), nullptr, saves);
+}
+
 int gdn_chunk_fwd_profile(const gdn_args* a, void* stream, float* kernel_ms) {
     if (kernel_ms == nullptr) return GDN_ERR_NULL;
     int rc = validate_chunk(a);

@@ -62,6 +62,10 @@ bool chunk_shape_supported(const gdn_args& a) {
     return true;
 }
 
+uint64_t chunk_record_bytes(const gdn_args& a) {
+    return (uint64_t)a.H * chunk_slots(a) * record_layout(a.K, a.V).bytes;
+}
+
 uint64_t chunk_workspace_bytes(const gdn_args& a) {
     const RecordLayout r = record_layout(a.K, a.V);
     return chunk_off_bytes(a) + (uint64_t)a.H * chunk_slots(a) * r.bytes;
@@ -594,7 +598,7 @@ static int launch_chunk_256(ChunkParams& p, hipStream_t stream, hipEvent_t* even
     return (int)hipGetLastError();
 }
 
-int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events) {
+int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events, const gdn_chunk_saves* saves) {
     const RecordLayout r = record_layout(a.K, a.V);
     ChunkParams p;
     p.q = static_cast<const bf16_t*>(a.q);
@@ -610,6 +614,12 @@ int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events) 
     p.pad_lens = left_padded ? a.cu_seqlens : nullptr;
     p.chunk_off = static_cast<int32_t*>(a.workspace);
     p.rec = static_cast<uint8_t*>(a.workspace) + chunk_off_bytes(a);
+    p.save_state = nullptr, p.save_vnew = nullptr, p.save_nc = 0, p.records_given = 0;
+    if (saves != nullptr) {
+        p.save_state = saves->states, p.save_vnew = saves->v_new, p.save_nc = saves->chunks_per_chain;
+        p.records_given = saves->records_given;
+        if (p.records_given) p.chunk_off = nullptr, p.rec = static_cast<uint8_t*>(a.workspace);
+    }
     p.q_stride_b = a.q_stride_b, p.q_stride_t = a.q_stride_t, p.q_stride_h = a.q_stride_h;
     p.k_stride_b = a.k_stride_b, p.k_stride_t = a.k_stride_t, p.k_stride_h = a.k_stride_h;
     p.v_stride_b = a.v_stride_b, p.v_stride_t = a.v_stride_t, p.v_stride_h = a.v_stride_h;

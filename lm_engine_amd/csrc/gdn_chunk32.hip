@@ -609,7 +609,7 @@ struct ScanSchedule : ScanScheduleRules<K> {
 
 // NT: the loaders use non-temporal loads.  Right when no other workgroup reads the same lines (one workgroup per
 // chain; measured 7 % faster at 1024 chains), wrong when column groups share them through the L2 (8 % slower).
-template <int K, int NW, bool NT = false>
+template <int K, int NW, bool NT = false, bool SAVE = false>
 __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(const ChunkParams p) {
     constexpr int NL = SCAN_LOADERS;
     // a separate wave writes the output (see below); with four compute waves the LDS has no room for its staging
@@ -903,6 +903,22 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
         const uint8_t* st = stage[c & 1];
         const uint8_t* stn = stage[(c + 1) & 1];
         const int valid = (int)min((int64_t)C, seq_len - (int64_t)c * C);
+        if constexpr (SAVE) {
+            // the state this chunk starts from, for the backward pass (stores from a compute wave: this variant
+            // is not the one the forward is timed on)
+            // (one wave-uniform base per store plus one per-lane byte offset: 64-bit per-lane addresses for
+            // all of them would not fit the register file)
+            if (p.save_state != nullptr && c < p.save_nc) {
+                char* base = reinterpret_cast<char*>(p.save_state + ((int64_t)chain * p.save_nc + c) * K * p.V);
+                const uint32_t lane_off = (uint32_t)((8 * lh) * p.V + 32 * tn + slice_col(l32)) * 4u;
+                const uint32_t row_bytes = (uint32_t)p.V * 4u;
+#pragma unroll
+                for (int td = 0; td < KD; td++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+                        *reinterpret_cast<float*>(base + (size_t)(st_row(td, r) * row_bytes) + lane_off) = S[td][r];
+            }
+        }
         bf16x8 fr[NOPS];
 #pragma unroll
         for (int i = 0; i < LA; i++) fr[i] = fnext[i];
@@ -1028,6 +1044,19 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
             }
             __builtin_amdgcn_sched_barrier(0);
         });
+        if constexpr (SAVE) {
+            // V~ of this chunk: tile tt, register r holds token 32 tt + 8 (r/4) + 4 h + r%4 of this lane's column
+            if (p.save_vnew != nullptr && c < p.save_nc) {
+                char* base = reinterpret_cast<char*>(p.save_vnew + ((int64_t)chain * p.save_nc + c) * C * p.V);
+                const uint32_t lane_off = (uint32_t)((4 * lh) * p.V + 32 * tn + slice_col(l32)) * 4u;
+                const uint32_t row_bytes = (uint32_t)p.V * 4u;
+#pragma unroll
+                for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+                        *reinterpret_cast<float*>(base + (size_t)((32 * tt + 8 * (r / 4) + r % 4) * row_bytes) + lane_off) = accv[tt][r];
+            }
+        }
         valid_prev = valid;
         og += og_step;
     }
@@ -1065,8 +1094,10 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     const int64_t cap = (int64_t)(3 * num_cus + 7) / 8 * 8;      // three workgroups per CU (LDS and registers allow it)
     if (items >= ((int64_t)1 << 31)) return GDN_ERR_UNSUPPORTED;  // the kernel counts items in 32 bits
     const int grid_prep = (int)(items < cap ? items : cap);
-    hipLaunchKernelGGL((chunk_prepare32_kernel<K>), dim3(grid_prep), dim3(PREP_THREADS), 0, stream, p);
-    if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
+    if (!p.records_given) {
+        hipLaunchKernelGGL((chunk_prepare32_kernel<K>), dim3(grid_prep), dim3(PREP_THREADS), 0, stream, p);
+        if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
+    }
     if (events != nullptr) (void)hipEventRecord(events[2], stream);
 
     // Compute waves (32-column slices) per scan workgroup: one while that gives no more workgroups than CUs, so
@@ -1077,8 +1108,15 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     const int vtiles = p.V / 32;
     int nw = 1;
     while (nw < 4 && vtiles % (2 * nw) == 0 && chains * (vtiles / nw) > (int64_t)num_cus) nw *= 2;
+    const bool save = p.save_state != nullptr || p.save_vnew != nullptr;
+    if (save && nw == 2) nw = 1;  // the saving variant exists for 1 and 4 slices per workgroup
     p.scan_groups = vtiles / nw;
     const dim3 grid((unsigned)(chains8 * p.scan_groups));
+    if (save) {
+        if (nw == 4) hipLaunchKernelGGL((chunk_scan32_kernel<K, 4, false, true>), grid, dim3(scan_waves(4) * WAVE), 0, stream, p);
+        else hipLaunchKernelGGL((chunk_scan32_kernel<K, 1, false, true>), grid, dim3(scan_waves(1) * WAVE), 0, stream, p);
+        return (int)hipGetLastError();
+    }
     if (nw == 4 && p.scan_groups == 1) hipLaunchKernelGGL((chunk_scan32_kernel<K, 4, true>), grid, dim3(scan_waves(4) * WAVE), 0, stream, p);
     else if (nw == 4) hipLaunchKernelGGL((chunk_scan32_kernel<K, 4>), grid, dim3(scan_waves(4) * WAVE), 0, stream, p);
     else if (nw == 2) hipLaunchKernelGGL((chunk_scan32_kernel<K, 2>), grid, dim3(scan_waves(2) * WAVE), 0, stream, p);

@@ -34,6 +34,12 @@ struct ChunkParams {
     float scale;
     uint32_t rec_bytes, off_qs, off_kt, off_ks, off_cs, off_p, off_u, off_eg;
     int scan_groups;  // workgroups per (sequence, head) in the scan kernel
+    // training support (scan of the 32x32x16 kernels only): when set, the scan also writes the fp32 state every
+    // chunk starts from, [N * H][save_nc][K][V], and V~ of every chunk, [N * H][save_nc][64][V]
+    float* save_state;
+    float* save_vnew;
+    int save_nc;
+    int records_given;  // the records are already in place: prepare is not run
 };
 
 struct RecordLayout {

@@ -10,8 +10,10 @@ namespace gdn {
 // Arguments are validated by the caller (gdn_api.hip); these only pick an instantiation and launch.
 int launch_recurrent(const gdn_args& a, hipStream_t stream);
 // `events`, when not null, holds GDN_CHUNK_KERNELS + 1 events recorded around the kernels.
-int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events = nullptr);
+// `saves`, when not null, selects the state-saving scan (see gdn_chunk_fwd_saving).
+int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events = nullptr, const gdn_chunk_saves* saves = nullptr);
 uint64_t chunk_workspace_bytes(const gdn_args& a);
+uint64_t chunk_record_bytes(const gdn_args& a);  // the records alone, [H][chunk slots]
 bool chunk_shape_supported(const gdn_args& a);
 
 }  // namespace gdn

@@ -197,6 +197,61 @@ def chunk_forward_kernel_times(
     return dict(zip(_lib.CHUNK_KERNEL_NAMES, (float(x) for x in times)))
 
 
+def chunk_forward_saving(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2norm, left_padded, states, v_new,
+                         chunks_per_chain):  # fmt: skip
+    """The chunked forward once more, for the backward pass: through ``gdn_chunk_fwd_saving`` it writes the
+    state every chunk starts from into ``states`` ``[N * H, chunks_per_chain, K, V]`` and V~ into ``v_new``
+    ``[N * H, chunks_per_chain, 64, V]`` (both fp32, contiguous).  The output itself is discarded."""
+    _require_hip_path()
+    lib = _lib.load_library()
+    dims = _check_inputs(q, k, v, g, beta, initial_state, cu_seqlens, left_padded)
+    B, T, H, K, V, N = dims
+    q, k, v = _last_dim_contiguous(q), _last_dim_contiguous(k), _last_dim_contiguous(v)
+    g = None if g is None else g.to(torch.float32).contiguous()
+    if beta is not None:
+        beta = beta.contiguous() if beta.dtype in (torch.bfloat16, torch.float32) else beta.float().contiguous()
+    cu_seqlens = None if cu_seqlens is None else cu_seqlens.to(torch.int32).contiguous()
+    h0 = None if initial_state is None else initial_state.contiguous()
+    for x, rows in ((states, K), (v_new, 64)):
+        if x.dtype != torch.float32 or not x.is_contiguous() or tuple(x.shape) != (N * H, chunks_per_chain, rows, V):
+            raise ValueError(f"save array must be contiguous fp32 {(N * H, chunks_per_chain, rows, V)}")
+    o = torch.empty(B, T, H, V, dtype=v.dtype, device=v.device)
+    args = _fill_args(q, k, v, g, beta, h0, None, o, cu_seqlens, scale, l2norm, False, dims, left_padded)
+    saves = _lib.GdnChunkSaves(states.data_ptr(), v_new.data_ptr(), chunks_per_chain, 0)
+    with torch.cuda.device(q.device):
+        nbytes = lib.gdn_workspace_bytes(ctypes.byref(args))
+        workspace = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=q.device)
+        args.workspace, args.workspace_bytes = workspace.data_ptr(), workspace.numel()
+        stream = ctypes.c_void_p(torch.cuda.current_stream(q.device).cuda_stream)
+        _lib.check_status(lib.gdn_chunk_fwd_saving(ctypes.byref(args), ctypes.byref(saves), stream),
+                          "gdn_chunk_fwd_saving")  # fmt: skip
+
+
+def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_chain):
+    """The scan kernel alone over a fixed-length batch whose chunk records the caller has written
+    (``records`` uint8 ``[H, B * T / 64, record bytes]``, T a multiple of 64); it reads the rows of ``k`` (also
+    in the place of q: such records carry zero row scales for q) and of ``v``.  Returns ``(o, final_state)``
+    and writes the state every chunk starts from into ``states`` ``[B * H, chunks_per_chain, K, V]``."""
+    _require_hip_path()
+    lib = _lib.load_library()
+    dims = _check_inputs(k, k, v, None, None, initial_state, None)
+    B, T, H, K, V, N = dims
+    if T % 64 != 0 or not records.is_contiguous() or records.dtype != torch.uint8 or tuple(records.shape[:2]) != (H, B * T // 64):
+        raise ValueError("records must be contiguous uint8 [H, B * T / 64, record bytes] with T a multiple of 64")
+    if states.dtype != torch.float32 or not states.is_contiguous() or tuple(states.shape) != (B * H, chunks_per_chain, K, V):
+        raise ValueError(f"states must be contiguous fp32 {(B * H, chunks_per_chain, K, V)}")
+    o = torch.empty(B, T, H, V, dtype=v.dtype, device=v.device)
+    ht = torch.empty(N, H, K, V, dtype=torch.float32, device=v.device)
+    args = _fill_args(k, k, v, None, None, initial_state, ht, o, None, 1.0, False, False, dims)
+    args.workspace, args.workspace_bytes = records.data_ptr(), records.numel()
+    saves = _lib.GdnChunkSaves(states.data_ptr(), None, chunks_per_chain, 1)
+    with torch.cuda.device(k.device):
+        stream = ctypes.c_void_p(torch.cuda.current_stream(k.device).cuda_stream)
+        _lib.check_status(lib.gdn_chunk_fwd_saving(ctypes.byref(args), ctypes.byref(saves), stream),
+                          "gdn_chunk_fwd_saving")  # fmt: skip
+    return o, ht
+
+
 class _GatedDeltaRule(torch.autograd.Function):
     """Forward on the HIP kernels; backward by ``backward.gated_delta_rule_backward`` from the saved
     inputs (the forward keeps no intermediate results)."""
