@@ -10,7 +10,7 @@ import torch
 import lm_engine_amd
 from oracle.gdn_backward_oracle import gated_delta_rule_grads_autograd
 
-from .helpers import max_abs, random_inputs, rel_l2
+from .helpers import assert_parity, max_abs, random_inputs, rel_l2
 
 
 pytestmark = pytest.mark.gpu
@@ -69,3 +69,74 @@ def test_chunk_bf16_packed():
 def test_recurrent_fp32():
     inp = random_inputs(B=2, T=40, H=2, K=64, V=64, dtype=torch.float32, seed=8, normalize=False)
     _run_case(lm_engine_amd.fused_recurrent_gated_delta_rule, inp, torch.float32)
+
+
+def test_chunk_bf16_k64_and_wide_v():
+    inp = random_inputs(B=1, T=130, H=3, K=64, V=256, dtype=torch.bfloat16, seed=9, normalize=False)
+    _run_case(lm_engine_amd.chunk_gated_delta_rule, inp, torch.bfloat16)
+
+
+def test_chunk_bf16_many_chains():
+    # more than 128 chains at V = 128: the saving scan runs with four column slices per workgroup
+    inp = random_inputs(B=9, T=128, H=16, K=128, V=128, dtype=torch.bfloat16, seed=10, normalize=False)
+    _run_case(lm_engine_amd.chunk_gated_delta_rule, inp, torch.bfloat16)
+
+
+def test_chunk_bf16_left_padded_batch():
+    B, T, H, K, V = 3, 200, 2, 128, 128
+    lens = [200, 70, 1]
+    inp = random_inputs(B=B, T=T, H=H, K=K, V=V, dtype=torch.bfloat16, seed=11, normalize=False)
+    cu = torch.tensor([0, 200, 270, 271], dtype=torch.int32)
+    leaves = _leaves(inp)
+    o, ht = lm_engine_amd.chunk_gated_delta_rule(**leaves, output_final_state=True, cu_seqlens=cu.cuda(),
+                                                 use_qk_l2norm_in_kernel=True, left_padded=True)  # fmt: skip
+    gen = torch.Generator().manual_seed(5)
+    do = torch.randn(o.shape, generator=gen).to(torch.bfloat16)
+    dht = torch.randn(ht.shape, generator=gen)
+    ((o.float() * do.cuda().float()).sum() + (ht * dht.cuda()).sum()).backward()
+    for b, n in enumerate(lens):
+        sl = lambda x: x[b : b + 1, T - n :]
+        want = gated_delta_rule_grads_autograd(
+            sl(inp["q"]), sl(inp["k"]), sl(inp["v"]), sl(inp["g"]), sl(inp["beta"]), sl(do), dht[b : b + 1],
+            initial_state=inp["initial_state"][b : b + 1], use_qk_l2norm_in_kernel=True,
+        )  # fmt: skip
+        got = [sl(leaves[x].grad.cpu()) for x in ("q", "k", "v", "g", "beta")] + [leaves["initial_state"].grad[b : b + 1]]
+        _assert_grads(got, want, torch.bfloat16)
+        for x in ("q", "k", "v", "g", "beta"):
+            assert not leaves[x].grad[b, : T - n].any(), f"gradient of {x} at the padding"
+
+
+def test_ungated_without_beta():
+    inp = random_inputs(B=2, T=100, H=2, K=128, V=64, dtype=torch.bfloat16, seed=12, normalize=False, gated=False)
+    inp["beta"] = None
+    q, k, v = (inp[x].cuda().requires_grad_(True) for x in ("q", "k", "v"))
+    h0 = inp["initial_state"].cuda()
+    o, _ = lm_engine_amd.chunk_gated_delta_rule(q, k, v, initial_state=h0, use_qk_l2norm_in_kernel=True)
+    do = torch.randn(o.shape, generator=torch.Generator().manual_seed(6)).to(torch.bfloat16)
+    (o.float() * do.cuda().float()).sum().backward()
+    zero, one = torch.zeros(2, 100, 2), torch.ones(2, 100, 2)
+    want = gated_delta_rule_grads_autograd(inp["q"], inp["k"], inp["v"], zero, one, do, None,
+                                           initial_state=inp["initial_state"], use_qk_l2norm_in_kernel=True)  # fmt: skip
+    _assert_grads([q.grad, k.grad, v.grad], want[:3], torch.bfloat16)
+
+
+def test_saved_chunk_states_are_the_states_of_the_prefixes():
+    """``gdn_chunk_fwd_saving``: the state saved for chunk c is the final state of the first 64 c tokens."""
+    from lm_engine_amd import ops
+    from oracle.gdn_oracle import recurrent_gated_delta_rule_ref
+
+    B, T, H, K, V = 2, 200, 2, 128, 128
+    inp = random_inputs(B=B, T=T, H=H, K=K, V=V, dtype=torch.bfloat16, seed=13)
+    dev = {n: (None if x is None else x.cuda()) for n, x in inp.items()}
+    NC = 4
+    states = torch.zeros(B * H, NC, K, V, device="cuda")
+    v_new = torch.zeros(B * H, NC, 64, V, device="cuda")
+    ops.chunk_forward_saving(dev["q"], dev["k"], dev["v"], dev["g"], dev["beta"], None, dev["initial_state"], None,
+                             True, False, states, v_new, NC)  # fmt: skip
+    states = states.cpu().reshape(B, H, NC, K, V)
+    assert torch.equal(states[:, :, 0], inp["initial_state"])
+    for c in range(1, NC):
+        cut = {n: inp[n][:, : 64 * c] for n in ("q", "k", "v", "g", "beta")}
+        _, want = recurrent_gated_delta_rule_ref(**cut, initial_state=inp["initial_state"], output_final_state=True,
+                                                 use_qk_l2norm_in_kernel=True)  # fmt: skip
+        assert_parity(states[:, :, c], want, torch.bfloat16, f"state at the start of chunk {c}")
