@@ -65,17 +65,23 @@ class _Packing:
         starts, lens = _chains(B, T, cu_seqlens, left_padded)
         self.N, self.H = len(lens), H
         self.NC = max(1, -(-max(lens + [1]) // CHUNK))
+        self.shape = (B, T)
+        # whole chunks, one sequence per row: packing is a change of layout, no gather
+        self.aligned = cu_seqlens is None and T % CHUNK == 0
         Tp = self.NC * CHUNK
         t = torch.arange(Tp, device=device)
         lens_t = torch.tensor(lens, device=device)
         self.valid = t[None, :] < lens_t[:, None]  # [N, Tp]
-        index = torch.tensor(starts, device=device)[:, None] + t[None, :]
-        self.index = torch.where(self.valid, index, torch.zeros_like(index))
-        self.shape = (B, T)
+        if not self.aligned:
+            index = torch.tensor(starts, device=device)[:, None] + t[None, :]
+            self.index = torch.where(self.valid, index, torch.zeros_like(index))
 
     def pack(self, x):
         """[B, T, H, *D] -> fp32 [N * H, NC, C, *D], zero at the padding."""
         tail = x.shape[3:]
+        if self.aligned:
+            y = x.reshape(self.N, self.NC, CHUNK, self.H, *tail).movedim(3, 1)
+            return y.to(torch.float32, memory_format=torch.contiguous_format).reshape(self.N * self.H, self.NC, CHUNK, *tail)
         flat = x.reshape(x.shape[0] * x.shape[1], self.H, *tail)
         y = flat[self.index].to(torch.float32)  # [N, Tp, H, *D]
         y = y * self.valid.reshape(self.N, -1, 1, *([1] * len(tail)))
@@ -86,7 +92,10 @@ class _Packing:
         """fp32 [N * H, NC, C, *D] -> [B, T, H, *D] in ``dtype``, zero where no sequence lives."""
         tail = y.shape[3:]
         B, T = self.shape
-        y = y.reshape(self.N, self.H, self.NC, CHUNK, *tail).movedim(1, 3).reshape(self.N, -1, self.H, *tail)
+        y = y.reshape(self.N, self.H, self.NC, CHUNK, *tail).movedim(1, 3)
+        if self.aligned:
+            return y.to(dtype, memory_format=torch.contiguous_format).reshape(B, T, self.H, *tail)
+        y = y.reshape(self.N, -1, self.H, *tail)
         out = torch.zeros(B * T, self.H, *tail, dtype=dtype, device=y.device)
         out[self.index[self.valid]] = y[self.valid].to(dtype)
         return out.reshape(B, T, self.H, *tail)
@@ -161,9 +170,9 @@ def _mirror_problem(N, H, kraw, qraw, doc, Tm, P, egl, cs_a, ks_a, ks_b):
     bf = torch.bfloat16
 
     def mirrored(a_rows, b_rows):  # [Bt, NC, C, D] x 2 -> [N, 2 NC C, H, D]: chunks and tokens reversed, A before B
-        x = torch.stack((a_rows, b_rows), dim=2).flip(1, 3)  # [Bt, NC, 2, C, D]
+        x = torch.stack((a_rows.to(bf), b_rows.to(bf)), dim=2).flip(1, 3)  # [Bt, NC, 2, C, D]
         D = x.size(-1)
-        return x.reshape(N, H, 2 * NC * CHUNK, D).transpose(1, 2).to(bf).contiguous()
+        return x.reshape(N, H, 2 * NC * CHUNK, D).transpose(1, 2).contiguous()
 
     U_bar = P.transpose(-1, -2) @ doc
     k_m = mirrored(kraw, qraw)
@@ -200,8 +209,9 @@ def _sweeps_on_scan_kernel(q, k, v, g, beta, scale, initial_state, cu_seqlens, l
     Bt = N * H
     K, V = q.size(-1), v.size(-1)
     dev = q.device
-    S0 = torch.zeros(Bt, NC, K, V, device=dev)
-    Vn = torch.zeros(Bt, NC, CHUNK, V, device=dev)
+    alloc = torch.empty if pk.aligned else torch.zeros  # chains shorter than NC chunks leave entries unwritten
+    S0 = alloc(Bt, NC, K, V, device=dev)
+    Vn = alloc(Bt, NC, CHUNK, V, device=dev)
     ops.chunk_forward_saving(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2norm, left_padded, S0, Vn, NC)
     live = pk.valid.reshape(N, 1, NC, CHUNK, 1).expand(N, H, NC, CHUNK, 1).reshape(Bt, NC, CHUNK, 1)
     Vn = torch.where(live, Vn, torch.zeros_like(Vn))  # rows past the end of a sequence hold whatever the kernel left
