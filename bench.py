@@ -61,7 +61,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", type=int, default=1, choices=(1, 2, 4))
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-decode", action="store_true", help="skip the decode, convolution and epilogue legs")
+    ap.add_argument("--no-decode", action="store_true", help="skip the decode, convolution, epilogue and backward legs")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target duration of the CPU baseline sample")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, the known-size kernel the HBM counters are scaled by")
@@ -328,6 +328,37 @@ def calibrate_copy():
     torch.cuda.synchronize()
 
 
+def bench_backward(w, inp, steps, warmup):
+    """One backward pass of the chunked operator on the same workload (``lm_engine_amd.backward``: both sweeps
+    over the chunks on the scan kernel, the chunk-local products as batched library GEMMs), gradient of the
+    output only.  Wall time per call with the device idle before and after."""
+    import torch
+
+    from lm_engine_amd.backward import gated_delta_rule_backward
+
+    gen = torch.Generator("cpu").manual_seed(555)
+    do = torch.randn(inp["v"].shape, generator=gen).to(inp["v"].dtype).cuda()
+    call = lambda: gated_delta_rule_backward(  # noqa: E731
+        inp["q"], inp["k"], inp["v"], inp["g"], inp["beta"], do, None, scale=inp["scale"],
+        initial_state=inp["initial_state"], cu_seqlens=inp["cu_seqlens"])  # fmt: skip
+    steps, warmup = max(1, min(steps, 5)), max(1, min(warmup, 2))
+    for _ in range(warmup):
+        call()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        call()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    return {
+        "workload": w.name,
+        "steps": steps,
+        "ms_per_backward": round(ms, 3),
+        "tokens_per_s": round(w.B * w.T / (ms * 1e-3), 1),
+        "composition": "2 scan launches (state-saving variant) + rocBLAS batched GEMMs + elementwise torch ops",
+    }
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -350,6 +381,7 @@ def main():
     decode = None if args.no_decode else bench_decode(args.steps, args.warmup)
     conv = None if args.no_decode else bench_conv(w, args.steps, args.warmup)
     epilogue = None if args.no_decode else bench_epilogue(w, args.steps, args.warmup)
+    backward = None if args.no_decode else bench_backward(w, inp, args.steps, args.warmup)
     baseline = None if args.no_cpu_baseline else cpu_baseline(w, inp, args.cpu_seconds)
     if args.calibrate_copy:
         calibrate_copy()
@@ -374,6 +406,7 @@ def main():
         "decode": decode,
         "conv": conv,
         "epilogue": epilogue,
+        "backward": backward,
         "device": torch.cuda.get_device_name(0),
     }
     print(json.dumps(line))
