@@ -4,6 +4,7 @@ Functional form of the reference's ``DepthwiseCausalConvolution.forward``
 (lm_engine/modeling_utils/depthwise_causal_convolution.py:103-241): same arguments, same three
 modes (fresh prefill, one-token update, multi-token continuation), same return ``(y, final_state)``.
 It runs one HIP kernel (``gdn_causal_conv1d_fwd`` of libgdn_hip.so); there is no torch fallback.
+Under autograd the backward differentiates the same formula written in torch (``_autograd.py``).
 
     x             [B, S, C]          bf16 or fp32, channels contiguous
     weight        [C, 1, ks] or [C, ks]   nn.Conv1d's depthwise weight, ks in 2..4
@@ -21,6 +22,7 @@ import ctypes
 import torch
 
 from . import _lib
+from ._autograd import kernel_with_formula_backward
 from .kernels import Kernel, is_kernel_allowed
 
 
@@ -44,6 +46,29 @@ def depthwise_causal_convolution(
     output_state: bool = False,
     activation: str | None = "silu",
 ) -> tuple[torch.Tensor, torch.Tensor | None]:
+    def formula(x, weight, bias, input_state):
+        # y[s] = act(bias + sum_j w[j] xx[s + j]) over xx = [state or zeros | x * mask], y masked again
+        w = (weight.squeeze(1) if weight.dim() == 3 else weight).float()
+        B, S, C = x.shape
+        ks = w.size(1)
+        use_mask = attention_mask is not None and attention_mask.shape[1] > 1 and attention_mask.shape[0] > 1
+        xm = x.float() * attention_mask[:, :, None].float() if use_mask else x.float()
+        head = torch.zeros(B, C, ks - 1, device=x.device) if input_state is None else input_state.float()
+        xx = torch.cat([head, xm.transpose(1, 2)], dim=-1)
+        y = torch.nn.functional.conv1d(xx, w[:, None, :], None if bias is None else bias.float(), groups=C)
+        if activation is not None:
+            y = torch.nn.functional.silu(y)
+        y = y.transpose(1, 2)
+        if use_mask:
+            y = y * attention_mask[:, :, None].float()
+        return y.to(x.dtype), (xx[..., -(ks - 1):].to(x.dtype) if output_state else None)
+
+    kernel = lambda x, weight, bias, input_state: _depthwise_causal_convolution(  # noqa: E731
+        x, weight, bias, input_state, attention_mask, output_state, activation)  # fmt: skip
+    return kernel_with_formula_backward(kernel, formula, x, weight, bias, input_state)
+
+
+def _depthwise_causal_convolution(x, weight, bias, input_state, attention_mask, output_state, activation):
     if not is_kernel_allowed(Kernel.gated_delta_rule):
         raise RuntimeError("Kernel.gated_delta_rule is disabled and this package ships no other implementation")
     if activation not in _IN_KERNEL_ACTIVATIONS:

@@ -7,6 +7,7 @@
   lm_engine/modeling_utils/normalization.py:69-124.
 
 Both take the (strided) slices of the layer's projections as they are; there is no torch fallback.
+Under autograd their backward differentiates the same formulas written in torch (``_autograd.py``).
 """
 
 from __future__ import annotations
@@ -16,6 +17,7 @@ import ctypes
 import torch
 
 from . import _lib
+from ._autograd import kernel_with_formula_backward
 from .kernels import Kernel, is_kernel_allowed
 
 
@@ -50,6 +52,17 @@ def delta_rule_gates(
     a: torch.Tensor, b: torch.Tensor, A_log: torch.Tensor, dt_bias: torch.Tensor, allow_neg_eigval: bool = False
 ) -> tuple[torch.Tensor, torch.Tensor]:
     """a, b ``[..., H]`` (activation dtype, may be slices of one projection) -> ``(g fp32, beta)`` of the same shape."""
+
+    def formula(a, b, A_log, dt_bias):
+        g = -torch.exp(A_log.float()) * torch.nn.functional.softplus(a.float() + dt_bias.float())
+        beta = torch.sigmoid(b.float()) * (2.0 if allow_neg_eigval else 1.0)
+        return g, beta.to(b.dtype)
+
+    kernel = lambda a, b, A_log, dt_bias: _delta_rule_gates(a, b, A_log, dt_bias, allow_neg_eigval)  # noqa: E731
+    return kernel_with_formula_backward(kernel, formula, a, b, A_log, dt_bias)
+
+
+def _delta_rule_gates(a, b, A_log, dt_bias, allow_neg_eigval):
     _require(a, "a")
     H = a.size(-1)
     if b.shape != a.shape or b.dtype != a.dtype:
@@ -82,6 +95,22 @@ def gated_rmsnorm(
     """o ``[..., H, V]``; gate the same shape or ``[..., H * V]`` (a slice of a projection) or None;
     weight ``[V]`` or None.  Returns ``rmsnorm(o * silu(gate)) * weight`` over V, shape and dtype of o.
     ``eps=None`` is torch's default for nn.RMSNorm: the machine epsilon of o's dtype."""
+    eps_value = float(torch.finfo(o.dtype).eps if eps is None else eps)
+
+    def formula(o, gate, weight):
+        x = o.float()
+        if gate is not None:
+            x = x * torch.nn.functional.silu(gate.float().reshape(o.shape))
+        y = x * torch.rsqrt(x.square().mean(dim=-1, keepdim=True) + eps_value)
+        if weight is not None:
+            y = y * weight.float()
+        return (y.to(o.dtype),)
+
+    kernel = lambda o, gate, weight: (_gated_rmsnorm(o, gate, weight, eps),)  # noqa: E731
+    return kernel_with_formula_backward(kernel, formula, o, gate, weight)[0]
+
+
+def _gated_rmsnorm(o, gate, weight, eps):
     _require(o, "o")
     if o.dim() < 2:
         raise ValueError("o must be [..., H, V]")

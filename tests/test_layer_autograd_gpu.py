@@ -1,0 +1,116 @@
+"""Gradients through the layer's single-kernel steps and through the whole chain
+(convolution -> gates -> operator -> gated norm), against autograd through the fp64 CPU oracles."""
+
+import pytest
+import torch
+
+import lm_engine_amd
+from oracle import recurrent_gated_delta_rule_ref
+from oracle.conv_oracle import depthwise_causal_convolution_ref
+from oracle.layer_oracle import delta_rule_gates_ref, gated_rmsnorm_ref
+from tests.helpers import rel_l2
+
+
+pytestmark = pytest.mark.gpu
+BF16, F32, F64 = torch.bfloat16, torch.float32, torch.float64
+
+
+def _grads(fn, tensors, cotangents):
+    leaves = [x.detach().clone().requires_grad_(True) for x in tensors]
+    outs = fn(*leaves)
+    outs = [o for o in outs if o is not None]
+    loss = sum((o.to(c.dtype) * c).sum() for o, c in zip(outs, cotangents))
+    return torch.autograd.grad(loss, leaves)
+
+
+def _compare(got, want, tol, names):
+    for name, a, b in zip(names, got, want):
+        err = rel_l2(a, b)
+        assert err <= tol, f"{name}: rel-L2 {err:.3e} > {tol}"
+
+
+def test_gates_gradients():
+    gen = torch.Generator().manual_seed(1)
+    H = 8
+    a, b = torch.randn(3, 50, H, generator=gen), torch.randn(3, 50, H, generator=gen)
+    A_log, dt_bias = torch.randn(H, generator=gen), torch.randn(H, generator=gen)
+    cg, cb = torch.randn(3, 50, H, generator=gen), torch.randn(3, 50, H, generator=gen)
+    want = _grads(lambda *t: delta_rule_gates_ref(*t, True), [x.to(F64) for x in (a, b, A_log, dt_bias)], [cg.to(F64), cb.to(F64)])
+    got = _grads(lambda *t: lm_engine_amd.delta_rule_gates(*t, True), [x.cuda() for x in (a, b, A_log, dt_bias)], [cg.cuda(), cb.cuda()])
+    _compare(got, want, 1e-5, ("da", "db", "dA_log", "ddt_bias"))
+
+
+@pytest.mark.parametrize("gated", [False, True])
+def test_gated_rmsnorm_gradients(gated):
+    gen = torch.Generator().manual_seed(2)
+    o, gate, w = torch.randn(2, 40, 4, 64, generator=gen), torch.randn(2, 40, 4, 64, generator=gen), torch.randn(64, generator=gen)
+    c = torch.randn(2, 40, 4, 64, generator=gen)
+    if gated:
+        want = _grads(lambda o, g, w: (gated_rmsnorm_ref(o, g, w, 1e-5),), [x.to(F64) for x in (o, gate, w)], [c.to(F64)])
+        got = _grads(lambda o, g, w: (lm_engine_amd.gated_rmsnorm(o, g, w, 1e-5),), [x.cuda() for x in (o, gate, w)], [c.cuda()])
+        _compare(got, want, 1e-5, ("do", "dgate", "dweight"))
+    else:
+        want = _grads(lambda o, w: (gated_rmsnorm_ref(o, None, w, 1e-5),), [x.to(F64) for x in (o, w)], [c.to(F64)])
+        got = _grads(lambda o, w: (lm_engine_amd.gated_rmsnorm(o, None, w, 1e-5),), [x.cuda() for x in (o, w)], [c.cuda()])
+        _compare(got, want, 1e-5, ("do", "dweight"))
+
+
+@pytest.mark.parametrize("with_state, masked", [(False, False), (True, False), (False, True)])
+def test_convolution_gradients(with_state, masked):
+    gen = torch.Generator().manual_seed(3)
+    B, S, C, ks = 3, 37, 64, 4
+    x, w, bias = torch.randn(B, S, C, generator=gen), 0.5 * torch.randn(C, 1, ks, generator=gen), torch.randn(C, generator=gen)
+    state = torch.randn(B, C, ks - 1, generator=gen)
+    mask = torch.ones(B, S)
+    if masked:
+        mask[1, :10] = 0
+        mask[2, :36] = 0
+    cy, cs = torch.randn(B, S, C, generator=gen), torch.randn(B, C, ks - 1, generator=gen)
+    m = mask if masked else None
+    if with_state:
+        want = _grads(lambda x, w, b, s: depthwise_causal_convolution_ref(x, w, b, s, m, True), [t.to(F64) for t in (x, w, bias, state)], [cy.to(F64), cs.to(F64)])
+        got = _grads(lambda x, w, b, s: lm_engine_amd.depthwise_causal_convolution(x, w, b, s, None if m is None else m.cuda(), True),
+                     [t.cuda() for t in (x, w, bias, state)], [cy.cuda(), cs.cuda()])  # fmt: skip
+        _compare(got, want, 1e-5, ("dx", "dweight", "dbias", "dstate"))
+    else:
+        want = _grads(lambda x, w, b: depthwise_causal_convolution_ref(x, w, b, None, m, True), [t.to(F64) for t in (x, w, bias)], [cy.to(F64), cs.to(F64)])
+        got = _grads(lambda x, w, b: lm_engine_amd.depthwise_causal_convolution(x, w, b, None, None if m is None else m.cuda(), True),
+                     [t.cuda() for t in (x, w, bias)], [cy.cuda(), cs.cuda()])  # fmt: skip
+        _compare(got, want, 1e-5, ("dx", "dweight", "dbias"))
+
+
+def test_layer_chain_gradients():
+    B, S, HK, HV, DK, DV = 2, 130, 2, 4, 128, 128
+    key_dim, value_dim = HK * DK, HV * DV
+    gen = torch.Generator().manual_seed(4)
+    qkv = torch.randn(B, S, 2 * key_dim + value_dim, generator=gen).to(BF16)
+    ab = torch.randn(B, S, 2 * HV + value_dim, generator=gen).to(BF16)
+    conv_w = (0.4 * torch.randn(2 * key_dim + value_dim, 1, 4, generator=gen)).to(BF16)
+    conv_b = (0.1 * torch.randn(2 * key_dim + value_dim, generator=gen)).to(BF16)
+    A_log = torch.log(torch.rand(HV, generator=gen) * 4 + 0.1)
+    dt_bias = torch.randn(HV, generator=gen) - 2.0
+    norm_w = (1 + 0.1 * torch.randn(DV, generator=gen)).to(BF16)
+    c = torch.randn(B, S, value_dim, generator=gen)
+
+    def oracle(qkv, ab, conv_w, conv_b, A_log, dt_bias, norm_w):
+        y, _ = depthwise_causal_convolution_ref(qkv, conv_w, conv_b, None, None, False)
+        q, k, v = y.split((key_dim, key_dim, value_dim), dim=-1)
+        q = q.reshape(B, S, HK, DK).repeat_interleave(HV // HK, dim=-2)
+        k = k.reshape(B, S, HK, DK).repeat_interleave(HV // HK, dim=-2)
+        v = v.reshape(B, S, HV, DV)
+        a, b, gate = ab[..., :HV], ab[..., HV : 2 * HV], ab[..., 2 * HV :]
+        g, beta = delta_rule_gates_ref(a, b, A_log, dt_bias, False)
+        o, _ = recurrent_gated_delta_rule_ref(q, k, v, g=g, beta=beta, use_qk_l2norm_in_kernel=True, state_dtype=F64)
+        return (gated_rmsnorm_ref(o, gate, norm_w, 1e-5).flatten(-2),)
+
+    def kernels(qkv, ab, conv_w, conv_b, A_log, dt_bias, norm_w):
+        a, b, gate = ab[..., :HV], ab[..., HV : 2 * HV], ab[..., 2 * HV :]
+        out, _ = lm_engine_amd.gated_deltanet_mixing(qkv, a, b, gate, conv_w, conv_b, A_log, dt_bias, norm_w, 1e-5,
+                                                     HK, HV, DK, DV)  # fmt: skip
+        return (out,)
+
+    tensors = (qkv, ab, conv_w, conv_b, A_log, dt_bias, norm_w)
+    want = _grads(oracle, [t.to(F64) for t in tensors], [c.to(F64)])
+    got = _grads(kernels, [t.cuda() for t in tensors], [c.cuda()])
+    assert [g.dtype for g in got] == [t.dtype for t in tensors]
+    _compare(got, want, 3e-2, ("dqkv", "dab", "dconv_weight", "dconv_bias", "dA_log", "ddt_bias", "dnorm_weight"))
