@@ -125,7 +125,9 @@ int gdn_recurrent_fwd(const gdn_args *args, void *stream);
  * gdn_chunk_fwd_saving is gdn_chunk_fwd (K <= 128) with a scan that also writes them, fp32:
  *     states [N * H][chunks_per_chain][K][V]     chain n * H + h, chunk c of its sequence
  *     v_new  [N * H][chunks_per_chain][64][V]    rows past the end of a sequence are not meaningful
- * Either may be NULL.  Chunks c >= chunks_per_chain are computed but not saved.
+ * Either may be NULL.  Only chunks c with c % save_every == 0 are saved (save_every <= 0 means 1), as entry
+ * e = c / save_every, or as entry chunks_per_chain - 1 - e when save_reverse != 0; entries outside
+ * [0, chunks_per_chain) are computed but not saved.
  * With records_given != 0 the prepare kernel is skipped: args->workspace then holds the chunk records
  * themselves, [H][B * ceil(T / 64)] records in the layout prepare writes (fixed-length batches only;
  * g, beta and the l2norm flag are not used, the records carry every scale).  The backward pass of this
@@ -136,6 +138,8 @@ typedef struct gdn_chunk_saves {
     float *v_new;
     int32_t chunks_per_chain;
     int32_t records_given;
+    int32_t save_every;
+    int32_t save_reverse;
 } gdn_chunk_saves;
 int gdn_chunk_fwd_saving(const gdn_args *args, const gdn_chunk_saves *saves, void *stream);
 

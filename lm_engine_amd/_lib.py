@@ -47,6 +47,8 @@ class GdnChunkSaves(ctypes.Structure):
         ("v_new", ctypes.c_void_p),
         ("chunks_per_chain", ctypes.c_int32),
         ("records_given", ctypes.c_int32),
+        ("save_every", ctypes.c_int32),
+        ("save_reverse", ctypes.c_int32),
     ]
 
 

@@ -217,10 +217,10 @@ def _sweeps_on_scan_kernel(q, k, v, g, beta, scale, initial_state, cu_seqlens, l
     Vn = torch.where(live, Vn, torch.zeros_like(Vn))  # rows past the end of a sequence hold whatever the kernel left
 
     k_m, v_m, rec = _mirror_problem(N, H, kraw, qraw, doc, Tm, P, egl, cs_a, ks_a, ks_b)
-    states = torch.empty(Bt, 2 * NC, K, V, device=dev)
+    dS1 = torch.empty(Bt, NC, K, V, device=dev)
     dht32 = None if dht is None else dht.to(torch.float32).contiguous()
-    o_m, dS = ops.chunk_scan_given_records(k_m, v_m, rec, dht32, states, 2 * NC)
-    dS1 = states[:, 0::2].flip(1)
+    # the A chunks are the even ones; mirror chunk 2 r is chunk NC - 1 - r of the forward order
+    o_m, dS = ops.chunk_scan_given_records(k_m, v_m, rec, dht32, dS1, NC, save_every=2, save_reverse=True)
     # the A chunks' output, back in forward order: [N, NC, 2, C, H, V] -> [Bt, NC, C, V]
     Y = o_m.view(N, NC, 2, CHUNK, H, V)[:, :, 0].flip(1, 2).permute(0, 3, 1, 2, 4).reshape(Bt, NC, CHUNK, V).float()
     return S0, Vn, dS1, Y, dS.reshape(Bt, K, V)

@@ -614,9 +614,10 @@ int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events, 
     p.pad_lens = left_padded ? a.cu_seqlens : nullptr;
     p.chunk_off = static_cast<int32_t*>(a.workspace);
     p.rec = static_cast<uint8_t*>(a.workspace) + chunk_off_bytes(a);
-    p.save_state = nullptr, p.save_vnew = nullptr, p.save_nc = 0, p.records_given = 0;
+    p.save_state = nullptr, p.save_vnew = nullptr, p.save_nc = 0, p.records_given = 0, p.save_every = 1, p.save_reverse = 0;
     if (saves != nullptr) {
         p.save_state = saves->states, p.save_vnew = saves->v_new, p.save_nc = saves->chunks_per_chain;
+        p.save_every = saves->save_every > 0 ? saves->save_every : 1, p.save_reverse = saves->save_reverse ? 1 : 0;
         p.records_given = saves->records_given;
         if (p.records_given) p.chunk_off = nullptr, p.rec = static_cast<uint8_t*>(a.workspace);
     }

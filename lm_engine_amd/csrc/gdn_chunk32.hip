@@ -908,8 +908,9 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
             // is not the one the forward is timed on)
             // (one wave-uniform base per store plus one per-lane byte offset: 64-bit per-lane addresses for
             // all of them would not fit the register file)
-            if (p.save_state != nullptr && c < p.save_nc) {
-                char* base = reinterpret_cast<char*>(p.save_state + ((int64_t)chain * p.save_nc + c) * K * p.V);
+            if (p.save_state != nullptr && c % p.save_every == 0 && c / p.save_every < p.save_nc) {
+                const int entry = p.save_reverse ? p.save_nc - 1 - c / p.save_every : c / p.save_every;
+                char* base = reinterpret_cast<char*>(p.save_state + ((int64_t)chain * p.save_nc + entry) * K * p.V);
                 const uint32_t lane_off = (uint32_t)((8 * lh) * p.V + 32 * tn + slice_col(l32)) * 4u;
                 const uint32_t row_bytes = (uint32_t)p.V * 4u;
 #pragma unroll
@@ -1046,8 +1047,9 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
         });
         if constexpr (SAVE) {
             // V~ of this chunk: tile tt, register r holds token 32 tt + 8 (r/4) + 4 h + r%4 of this lane's column
-            if (p.save_vnew != nullptr && c < p.save_nc) {
-                char* base = reinterpret_cast<char*>(p.save_vnew + ((int64_t)chain * p.save_nc + c) * C * p.V);
+            if (p.save_vnew != nullptr && c % p.save_every == 0 && c / p.save_every < p.save_nc) {
+                const int entry = p.save_reverse ? p.save_nc - 1 - c / p.save_every : c / p.save_every;
+                char* base = reinterpret_cast<char*>(p.save_vnew + ((int64_t)chain * p.save_nc + entry) * C * p.V);
                 const uint32_t lane_off = (uint32_t)((4 * lh) * p.V + 32 * tn + slice_col(l32)) * 4u;
                 const uint32_t row_bytes = (uint32_t)p.V * 4u;
 #pragma unroll

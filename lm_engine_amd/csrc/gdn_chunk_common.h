@@ -39,6 +39,8 @@ struct ChunkParams {
     float* save_state;
     float* save_vnew;
     int save_nc;
+    int save_every;    // only chunks c with c % save_every == 0 are saved, as entry c / save_every ...
+    int save_reverse;  // ... or, when set, as entry save_nc - 1 - c / save_every
     int records_given;  // the records are already in place: prepare is not run
 };
 

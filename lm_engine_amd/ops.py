@@ -217,7 +217,7 @@ def chunk_forward_saving(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2n
             raise ValueError(f"save array must be contiguous fp32 {(N * H, chunks_per_chain, rows, V)}")
     o = torch.empty(B, T, H, V, dtype=v.dtype, device=v.device)
     args = _fill_args(q, k, v, g, beta, h0, None, o, cu_seqlens, scale, l2norm, False, dims, left_padded)
-    saves = _lib.GdnChunkSaves(states.data_ptr(), v_new.data_ptr(), chunks_per_chain, 0)
+    saves = _lib.GdnChunkSaves(states.data_ptr(), v_new.data_ptr(), chunks_per_chain, 0, 1, 0)
     with torch.cuda.device(q.device):
         nbytes = lib.gdn_workspace_bytes(ctypes.byref(args))
         workspace = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=q.device)
@@ -227,11 +227,13 @@ def chunk_forward_saving(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2n
                           "gdn_chunk_fwd_saving")  # fmt: skip
 
 
-def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_chain):
+def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_chain, save_every=1, save_reverse=False):
     """The scan kernel alone over a fixed-length batch whose chunk records the caller has written
     (``records`` uint8 ``[H, B * T / 64, record bytes]``, T a multiple of 64); it reads the rows of ``k`` (also
     in the place of q: such records carry zero row scales for q) and of ``v``.  Returns ``(o, final_state)``
-    and writes the state every chunk starts from into ``states`` ``[B * H, chunks_per_chain, K, V]``."""
+    and writes the state that chunk ``c`` starts from, for every ``c`` divisible by ``save_every``, into entry
+    ``c / save_every`` of ``states`` ``[B * H, chunks_per_chain, K, V]`` (counted from the end with
+    ``save_reverse``)."""
     _require_hip_path()
     lib = _lib.load_library()
     dims = _check_inputs(k, k, v, None, None, initial_state, None)
@@ -244,7 +246,7 @@ def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_ch
     ht = torch.empty(N, H, K, V, dtype=torch.float32, device=v.device)
     args = _fill_args(k, k, v, None, None, initial_state, ht, o, None, 1.0, False, False, dims)
     args.workspace, args.workspace_bytes = records.data_ptr(), records.numel()
-    saves = _lib.GdnChunkSaves(states.data_ptr(), None, chunks_per_chain, 1)
+    saves = _lib.GdnChunkSaves(states.data_ptr(), None, chunks_per_chain, 1, save_every, 1 if save_reverse else 0)
     with torch.cuda.device(k.device):
         stream = ctypes.c_void_p(torch.cuda.current_stream(k.device).cuda_stream)
         _lib.check_status(lib.gdn_chunk_fwd_saving(ctypes.byref(args), ctypes.byref(saves), stream),
