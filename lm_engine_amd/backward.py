@@ -158,12 +158,13 @@ def _fragment_index(device):
 RECORD_BYTES = 13312  # record of the 32x32x16 kernels (K <= 128): 12 fragments, 3 x 64 row scales, e^{gamma_C}
 
 
-def _mirror_problem(N, H, kraw, qraw, doc, Tm, P, egl, cs_a, ks_a, ks_b):
+def _mirror_problem(N, H, kraw, qraw, doc, Tm, P, egl, cs_a, ks_a, ks_b, aligned_inputs=None):
     """Tensors and chunk records of the reverse sweep as a forward scan (see the module docstring).
 
     Inputs are packed [N * H, NC, C, ...] fp32; ``cs_a``, ``ks_a``, ``ks_b`` are the row scales of the A and
-    B chunks in forward token order.  Returns k, v ``[N, 2 NC C, H, D]`` bf16 and the records as a uint8
-    tensor ``[H, N * 2 NC, RECORD_BYTES]``."""
+    B chunks in forward token order.  ``aligned_inputs`` = the caller's ``(q, k, do)`` when they are whole
+    chunks with one sequence per row (the mirrored rows are then taken from them directly).  Returns k, v
+    ``[N, 2 NC C, H, D]`` bf16 and the records as a uint8 tensor ``[H, N * 2 NC, RECORD_BYTES]``."""
     Bt, NC = egl.shape
     dev = egl.device
     K, V = kraw.size(-1), doc.size(-1)
@@ -175,32 +176,43 @@ def _mirror_problem(N, H, kraw, qraw, doc, Tm, P, egl, cs_a, ks_a, ks_b):
         return x.reshape(N, H, 2 * NC * CHUNK, D).transpose(1, 2).contiguous()
 
     U_bar = P.transpose(-1, -2) @ doc
-    k_m = mirrored(kraw, qraw)
-    v_m = mirrored(U_bar, doc)
+    if aligned_inputs is None:
+        k_m = mirrored(kraw, qraw)
+        v_m = mirrored(U_bar, doc)
+    else:
+        # reversing the token axis of [N, T, H, D] reverses the chunks and the tokens inside them at once
+        q, k, do = (x.to(bf).flip(1).view(N, NC, CHUNK, H, -1) for x in aligned_inputs)
+        k_m = torch.stack((k, q), dim=2).view(N, 2 * NC * CHUNK, H, K)
+        v_m = torch.empty(N, NC, 2, CHUNK, H, V, dtype=bf, device=dev)
+        v_m[:, :, 0] = U_bar.view(N, H, NC, CHUNK, V).flip(2, 3).permute(0, 2, 3, 1, 4)
+        v_m[:, :, 1] = do
+        v_m = v_m.view(N, 2 * NC * CHUNK, H, V)
 
     rows, cols = _fragment_index(dev)
     eye = torch.eye(CHUNK, device=dev)
     # T^T with rows and columns reversed is lower-triangular again: entry (i', j') is T[63 - j', 63 - i']
     Tmir = Tm.transpose(-1, -2).flip(-1, -2)
-    frag_t = Tmir[..., rows, cols].to(bf).reshape(Bt, NC, 6 * 512)
+    frag_t = Tmir[..., rows, cols].to(bf).reshape(N, H, NC, 6 * 512)
     frag_i = eye[rows, cols].to(bf).reshape(6 * 512)
 
-    rec = torch.zeros(Bt, NC, 2, RECORD_BYTES // 2, dtype=bf, device=dev)
-    rec[:, :, 0, :3072] = frag_t.flip(1)          # A: T' := mirrored T^T
-    rec[:, :, 0, 3072:6144] = frag_i              #    P  := I, so that the output of the chunk is Y
-    rec[:, :, 1, :3072] = frag_i                  # B: T' := I; P stays 0
-    scal = rec.view(torch.float32)                # [Bt, NC, 2, 3328]: row scales of q | k (update) | k S0 | e^{gamma_C}
+    def by_head(x):  # [N * H, NC, ...] in forward chunk order -> [H, N, NC, ...] in mirror order
+        return x.reshape(N, H, NC, *x.shape[2:]).flip(2).transpose(0, 1)
+
+    rec = torch.zeros(H, N, NC, 2, RECORD_BYTES // 2, dtype=bf, device=dev)
+    rec[:, :, :, 0, :3072] = frag_t.flip(2).transpose(0, 1)  # A: T' := mirrored T^T
+    rec[:, :, :, 0, 3072:6144] = frag_i                      #    P  := I, so that the output of the chunk is Y
+    rec[:, :, :, 1, :3072] = frag_i                          # B: T' := I; P stays 0
+    scal = rec.view(torch.float32)  # [H, N, NC, 2, 3328]: row scales of q | of k (update) | of k S0 | e^{gamma_C}
     base = 6144 // 2
-    scal[:, :, 0, base + 64 : base + 128] = ks_a.flip(1, 2)
-    scal[:, :, 0, base + 128 : base + 192] = cs_a.flip(1, 2)
-    scal[:, :, 0, base + 192] = egl.flip(1)
-    scal[:, :, 1, base + 64 : base + 128] = ks_b.flip(1, 2)
-    scal[:, :, 1, base + 192] = 1.0
-    rec = rec.view(N, H, NC * 2, RECORD_BYTES // 2).transpose(0, 1).contiguous()
+    scal[:, :, :, 0, base + 64 : base + 128] = by_head(ks_a).flip(-1)
+    scal[:, :, :, 0, base + 128 : base + 192] = by_head(cs_a).flip(-1)
+    scal[:, :, :, 0, base + 192] = by_head(egl)
+    scal[:, :, :, 1, base + 64 : base + 128] = by_head(ks_b).flip(-1)
+    scal[:, :, :, 1, base + 192] = 1.0
     return k_m, v_m, rec.view(torch.uint8).reshape(H, N * NC * 2, RECORD_BYTES)
 
 
-def _sweeps_on_scan_kernel(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2norm, left_padded, pk, dht,
+def _sweeps_on_scan_kernel(q, k, v, do, g, beta, scale, initial_state, cu_seqlens, l2norm, left_padded, pk, dht,
                            kraw, qraw, doc, Tm, P, egl, cs_a, ks_a, ks_b):  # fmt: skip
     """Both sweeps on the HIP scan kernel.  Returns S0, V~, dS1, Y, dS0 of chunk 0 (packed, fp32)."""
     from . import ops  # late: ops imports this module
@@ -216,7 +228,8 @@ def _sweeps_on_scan_kernel(q, k, v, g, beta, scale, initial_state, cu_seqlens, l
     live = pk.valid.reshape(N, 1, NC, CHUNK, 1).expand(N, H, NC, CHUNK, 1).reshape(Bt, NC, CHUNK, 1)
     Vn = torch.where(live, Vn, torch.zeros_like(Vn))  # rows past the end of a sequence hold whatever the kernel left
 
-    k_m, v_m, rec = _mirror_problem(N, H, kraw, qraw, doc, Tm, P, egl, cs_a, ks_a, ks_b)
+    k_m, v_m, rec = _mirror_problem(N, H, kraw, qraw, doc, Tm, P, egl, cs_a, ks_a, ks_b,
+                                    aligned_inputs=(q, k, do) if pk.aligned else None)  # fmt: skip
     dS1 = torch.empty(Bt, NC, K, V, device=dev)
     dht32 = None if dht is None else dht.to(torch.float32).contiguous()
     # the A chunks are the even ones; mirror chunk 2 r is chunk NC - 1 - r of the forward order
@@ -282,7 +295,7 @@ def gated_delta_rule_backward(
     if on_kernel:
         # the scan reads the raw rows of k and q; their norms and e^{gamma} go into the row scales
         S0, Vn, dS1, Y, dS = _sweeps_on_scan_kernel(
-            q, k, v, g, beta, scale, initial_state, cu_seqlens, use_qk_l2norm_in_kernel, left_padded, pk, dht,
+            q, k, v, do, g, beta, scale, initial_state, cu_seqlens, use_qk_l2norm_in_kernel, left_padded, pk, dht,
             kc, qc, doc, Tm, P, egl,
             cs_a=-(tail * rk[..., 0]), ks_a=-(bc * e * rk[..., 0]), ks_b=e * rq[..., 0] * scale,
         )  # fmt: skip
