@@ -318,9 +318,10 @@ def gated_delta_rule_backward(
 
     G = dP * E
     Hm = dA * bc[..., None] * E
-    dqs = G @ kn + dQe * e[..., None]
-    dkn = (G.transpose(-1, -2) @ qs + dKd * tail[..., None] - Z * (bc * e)[..., None]
-           + (Hm + Hm.transpose(-1, -2)) @ kn)  # fmt: skip
+    dqs = torch.baddbmm((dQe * e[..., None]).flatten(0, 1), G.flatten(0, 1), kn.flatten(0, 1)).view_as(dQe)
+    dkn = (dKd * tail[..., None]).addcmul_(Z, (bc * e)[..., None], value=-1.0).flatten(0, 1)
+    dkn = dkn.baddbmm_(G.transpose(-1, -2).flatten(0, 1), qs.flatten(0, 1))
+    dkn = dkn.baddbmm_((Hm + Hm.transpose(-1, -2)).flatten(0, 1), kn.flatten(0, 1)).view_as(dKd)
     dvc = Y * bc[..., None]
     dbc = -(Z * kn * e[..., None]).sum(-1) + (Y * vc).sum(-1) + (dA * E * KK).sum(-1)
     MP = dP * P
