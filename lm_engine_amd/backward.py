@@ -286,7 +286,6 @@ def gated_delta_rule_backward(
     A = bc[..., None] * E * KK * strict
     Tm = torch.linalg.solve_triangular(eye + A, eye.expand_as(A), upper=False)
     Kb = kn * (bc * e)[..., None]
-    Vb = vc * bc[..., None]
     P = E * (qs @ kT)
     Qe = qs * e[..., None]
     Kd = kn * tail[..., None]
@@ -304,7 +303,7 @@ def gated_delta_rule_backward(
         if initial_state is not None:
             S_init = initial_state.to(torch.float32).reshape(Bt, K, V)
         dS_init = torch.zeros(Bt, K, V, device=dev) if dht is None else dht.to(torch.float32).reshape(Bt, K, V)
-        S0, Vn, dS1, Y, dS = _sweeps_as_gemm_loops(S_init, dS_init, egl, Kd, Qe, Kb, Tm, Vb, P, doc)
+        S0, Vn, dS1, Y, dS = _sweeps_as_gemm_loops(S_init, dS_init, egl, Kd, Qe, Kb, Tm, vc * bc[..., None], P, doc)
     dh0 = dS.reshape(N, H, K, V) if initial_state is not None else None
 
     # chunk-local gradients, all chunks at once
