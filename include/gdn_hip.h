@@ -144,6 +144,28 @@ typedef struct gdn_chunk_saves {
 int gdn_chunk_fwd_saving(const gdn_args *args, const gdn_chunk_saves *saves, void *stream);
 
 /*
+ * Training support, second part: the chunk-local gradients, one workgroup per (sequence, head, chunk), once
+ * the two sweeps over the chunks (gdn_chunk_fwd_saving, forward and mirrored) have delivered per chunk the
+ * state it starts from, the gradient of the state it ends with, V~ and Y = T^T dV~.  All arrays fp32,
+ * contiguous, chunk-major ("packed": sequences padded with zeros to whole chunks):
+ *     qs, kn        [chunks][64][K]   q normalised and scaled, k normalised
+ *     v, dout, y, v_new  [chunks][64][V]
+ *     states, dstates    [chunks][K][V]
+ *     gamma, beta   [chunks][64]      prefix sum of g inside the chunk, beta
+ * Outputs: dqs, dkn [chunks][64][K] (gradients with respect to qs and kn), dbeta [chunks][64], and
+ * dgamma [chunks][64], the gradient with respect to gamma (dg is its reverse prefix sum inside the chunk).
+ * K = V = 128 only (GDN_ERR_UNSUPPORTED otherwise).  Counterpart upstream: the chunk-local kernels of fla's
+ * backward of chunk_gated_delta_rule, reached from gated_deltanet/module.py:197-209 under autograd.
+ */
+typedef struct gdn_chunk_local_args {
+    const float *qs, *kn, *v, *dout, *y, *v_new, *states, *dstates, *gamma, *beta;
+    float *dqs, *dkn, *dbeta, *dgamma;
+    int64_t chunks;
+    int32_t K, V;
+} gdn_chunk_local_args;
+int gdn_chunk_bwd_local(const gdn_chunk_local_args *args, void *stream);
+
+/*
  * Measurement aid, no counterpart in the reference: runs exactly what gdn_chunk_fwd runs, with a
  * HIP event recorded on `stream` before and after every kernel, waits for the last one and
  * returns each kernel's duration in milliseconds in kernel_ms[GDN_CHUNK_KERNELS], in launch

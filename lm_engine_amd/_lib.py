@@ -32,6 +32,7 @@ EXPORTED_SYMBOLS = (
     "gdn_recurrent_fwd",
     "gdn_chunk_fwd_profile",
     "gdn_chunk_fwd_saving",
+    "gdn_chunk_bwd_local",
     "gdn_causal_conv1d_fwd",
     "gdn_gates_fwd",
     "gdn_gated_rmsnorm_fwd",
@@ -50,6 +51,12 @@ class GdnChunkSaves(ctypes.Structure):
         ("save_every", ctypes.c_int32),
         ("save_reverse", ctypes.c_int32),
     ]
+
+
+class GdnChunkLocalArgs(ctypes.Structure):
+    _fields_ = [(name, ctypes.c_void_p) for name in (
+        "qs", "kn", "v", "dout", "y", "v_new", "states", "dstates", "gamma", "beta", "dqs", "dkn", "dbeta", "dgamma",
+    )] + [("chunks", ctypes.c_int64), ("K", ctypes.c_int32), ("V", ctypes.c_int32)]  # fmt: skip
 
 
 class GdnArgs(ctypes.Structure):
@@ -135,6 +142,8 @@ def load_library() -> ctypes.CDLL:
     lib.gdn_chunk_fwd_profile.restype = ctypes.c_int
     lib.gdn_chunk_fwd_saving.argtypes = [ctypes.POINTER(GdnArgs), ctypes.POINTER(GdnChunkSaves), ctypes.c_void_p]
     lib.gdn_chunk_fwd_saving.restype = ctypes.c_int
+    lib.gdn_chunk_bwd_local.argtypes = [ctypes.POINTER(GdnChunkLocalArgs), ctypes.c_void_p]
+    lib.gdn_chunk_bwd_local.restype = ctypes.c_int
     lib.gdn_causal_conv1d_fwd.argtypes = [ctypes.POINTER(GdnConvArgs), ctypes.c_void_p]
     lib.gdn_causal_conv1d_fwd.restype = ctypes.c_int
     lib.gdn_gates_fwd.argtypes = [ctypes.POINTER(GdnGateArgs), ctypes.c_void_p]

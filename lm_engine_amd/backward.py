@@ -239,6 +239,56 @@ def _sweeps_on_scan_kernel(q, k, v, do, g, beta, scale, initial_state, cu_seqlen
     return S0, Vn, dS1, Y, dS.reshape(Bt, K, V)
 
 
+def _chunk_local_kv():
+    from . import ops  # late: ops imports this module
+
+    return ops.CHUNK_LOCAL_KV
+
+
+def _chunk_local_grads(qs, kn, vc, doc, Y, Vn, S0, dS1, gam, bc):
+    """The chunk-local gradients with batched GEMMs and elementwise torch operations (any shape, any device):
+    what ``gdn_chunk_bwd_local`` computes in one kernel.  Packed fp32 tensors in; returns the gradients with
+    respect to qs and kn, dbeta, and the gradient with respect to gamma (before the reverse prefix sum)."""
+    dev = qs.device
+    incl = torch.ones(CHUNK, CHUNK, dtype=torch.bool, device=dev).tril(0)
+    strict = incl.tril(-1)
+    e = gam.exp()
+    gl = gam[..., -1]
+    egl = gl.exp()
+    tail = (gl[..., None] - gam).exp()
+    diff = gam[..., :, None] - gam[..., None, :]
+    E = torch.where(incl, diff, torch.zeros_like(diff)).exp() * incl
+    kT = kn.transpose(-1, -2)
+    KK = kn @ kT
+    A = bc[..., None] * E * KK * strict
+    P = E * (qs @ kT)
+    Kb = kn * (bc * e)[..., None]
+    Qe = qs * e[..., None]
+    Kd = kn * tail[..., None]
+
+    S0t = S0.transpose(-1, -2)
+    VnT = Vn.transpose(-1, -2)
+    dP = (doc @ VnT) * incl
+    dQe = doc @ S0t
+    dKd = Vn @ dS1.transpose(-1, -2)
+    Z = Y @ S0t          # the gradient with respect to Kb is -Z, the one with respect to Vb is Y
+    dA = -(Y @ VnT) * strict
+
+    G = dP * E
+    Hm = dA * bc[..., None] * E
+    dqs = torch.baddbmm((dQe * e[..., None]).flatten(0, 1), G.flatten(0, 1), kn.flatten(0, 1)).view_as(dQe)
+    dkn = (dKd * tail[..., None]).addcmul_(Z, (bc * e)[..., None], value=-1.0).flatten(0, 1)
+    dkn = dkn.baddbmm_(G.transpose(-1, -2).flatten(0, 1), qs.flatten(0, 1))
+    dkn = dkn.baddbmm_((Hm + Hm.transpose(-1, -2)).flatten(0, 1), kn.flatten(0, 1)).view_as(dKd)
+    dbc = -(Z * kn * e[..., None]).sum(-1) + (Y * vc).sum(-1) + (dA * E * KK).sum(-1)
+    MP = dP * P
+    MA = dA * A
+    n_kd = (dKd * Kd).sum(-1)
+    dgam = MP.sum(-1) - MP.sum(-2) + (dQe * Qe).sum(-1) - n_kd - (Z * Kb).sum(-1) + MA.sum(-1) - MA.sum(-2)
+    dgam[..., -1] += egl * (dS1 * S0).sum(dim=(-1, -2)) + n_kd.sum(-1)
+    return dqs, dkn, dbc, dgam
+
+
 def gated_delta_rule_backward(
     q, k, v, g, beta, do, dht=None, scale=None, initial_state=None, cu_seqlens=None,
     use_qk_l2norm_in_kernel=False, left_padded=False,
@@ -285,10 +335,7 @@ def gated_delta_rule_backward(
     KK = kn @ kT
     A = bc[..., None] * E * KK * strict
     Tm = torch.linalg.solve_triangular(eye + A, eye.expand_as(A), upper=False)
-    Kb = kn * (bc * e)[..., None]
     P = E * (qs @ kT)
-    Qe = qs * e[..., None]
-    Kd = kn * tail[..., None]
 
     on_kernel = q.is_cuda and q.dtype == torch.bfloat16 and K <= 128 and V % 32 == 0
     if on_kernel:
@@ -303,31 +350,19 @@ def gated_delta_rule_backward(
         if initial_state is not None:
             S_init = initial_state.to(torch.float32).reshape(Bt, K, V)
         dS_init = torch.zeros(Bt, K, V, device=dev) if dht is None else dht.to(torch.float32).reshape(Bt, K, V)
-        S0, Vn, dS1, Y, dS = _sweeps_as_gemm_loops(S_init, dS_init, egl, Kd, Qe, Kb, Tm, vc * bc[..., None], P, doc)
+        S0, Vn, dS1, Y, dS = _sweeps_as_gemm_loops(
+            S_init, dS_init, egl, kn * tail[..., None], qs * e[..., None], kn * (bc * e)[..., None], Tm,
+            vc * bc[..., None], P, doc,
+        )  # fmt: skip
     dh0 = dS.reshape(N, H, K, V) if initial_state is not None else None
 
-    # chunk-local gradients, all chunks at once
-    S0t = S0.transpose(-1, -2)
-    VnT = Vn.transpose(-1, -2)
-    dP = (doc @ VnT) * incl
-    dQe = doc @ S0t
-    dKd = Vn @ dS1.transpose(-1, -2)
-    Z = Y @ S0t          # the gradient with respect to Kb is -Z, the one with respect to Vb is Y
-    dA = -(Y @ VnT) * strict
+    if on_kernel and (K, V) == _chunk_local_kv():
+        from . import ops
 
-    G = dP * E
-    Hm = dA * bc[..., None] * E
-    dqs = torch.baddbmm((dQe * e[..., None]).flatten(0, 1), G.flatten(0, 1), kn.flatten(0, 1)).view_as(dQe)
-    dkn = (dKd * tail[..., None]).addcmul_(Z, (bc * e)[..., None], value=-1.0).flatten(0, 1)
-    dkn = dkn.baddbmm_(G.transpose(-1, -2).flatten(0, 1), qs.flatten(0, 1))
-    dkn = dkn.baddbmm_((Hm + Hm.transpose(-1, -2)).flatten(0, 1), kn.flatten(0, 1)).view_as(dKd)
+        dqs, dkn, dbc, dgam = ops.chunk_local_grads(qs, kn, vc, doc, Y, Vn, S0, dS1, gam, bc)
+    else:
+        dqs, dkn, dbc, dgam = _chunk_local_grads(qs, kn, vc, doc, Y, Vn, S0, dS1, gam, bc)
     dvc = Y * bc[..., None]
-    dbc = -(Z * kn * e[..., None]).sum(-1) + (Y * vc).sum(-1) + (dA * E * KK).sum(-1)
-    MP = dP * P
-    MA = dA * A
-    n_kd = (dKd * Kd).sum(-1)
-    dgam = MP.sum(-1) - MP.sum(-2) + (dQe * Qe).sum(-1) - n_kd - (Z * Kb).sum(-1) + MA.sum(-1) - MA.sum(-2)
-    dgam[..., -1] += egl * (dS1 * S0).sum(dim=(-1, -2)) + n_kd.sum(-1)
     dgc = dgam.flip(-1).cumsum(-1).flip(-1)
 
     dqn = dqs * scale

@@ -15,5 +15,7 @@ int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events =
 uint64_t chunk_workspace_bytes(const gdn_args& a);
 uint64_t chunk_record_bytes(const gdn_args& a);  // the records alone, [H][chunk slots]
 bool chunk_shape_supported(const gdn_args& a);
+int launch_chunk_bwd_local(const gdn_chunk_local_args& a, hipStream_t stream);  // gdn_chunk_bwd.hip
+bool chunk_bwd_local_supported(const gdn_chunk_local_args& a);
 
 }  // namespace gdn

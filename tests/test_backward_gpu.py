@@ -140,3 +140,26 @@ def test_saved_chunk_states_are_the_states_of_the_prefixes():
         _, want = recurrent_gated_delta_rule_ref(**cut, initial_state=inp["initial_state"], output_final_state=True,
                                                  use_qk_l2norm_in_kernel=True)  # fmt: skip
         assert_parity(states[:, :, c], want, torch.bfloat16, f"state at the start of chunk {c}")
+
+
+def test_chunk_local_kernel_matches_the_batched_gemm_version():
+    """``gdn_chunk_bwd_local`` against the same stage written with torch operations, on random packed inputs."""
+    from lm_engine_amd import ops
+    from lm_engine_amd.backward import _chunk_local_grads
+
+    gen = torch.Generator().manual_seed(21)
+    Bt, NC, C, K, V = 3, 5, 64, 128, 128
+    rnd = lambda *shape: torch.randn(*shape, generator=gen)  # noqa: E731
+    qs = torch.nn.functional.normalize(rnd(Bt, NC, C, K), dim=-1) * K**-0.5
+    kn = torch.nn.functional.normalize(rnd(Bt, NC, C, K), dim=-1)
+    v, dout, y, v_new = rnd(Bt, NC, C, V), rnd(Bt, NC, C, V), rnd(Bt, NC, C, V), rnd(Bt, NC, C, V)
+    s0, ds1 = 0.3 * rnd(Bt, NC, K, V), 0.3 * rnd(Bt, NC, K, V)
+    gam = torch.nn.functional.logsigmoid(rnd(Bt, NC, C) + 2.0).cumsum(-1)
+    beta = torch.sigmoid(rnd(Bt, NC, C))
+    args = [x.cuda() for x in (qs, kn, v, dout, y, v_new, s0, ds1, gam, beta)]
+    got = ops.chunk_local_grads(*args)
+    want = _chunk_local_grads(*[x.double() for x in (qs, kn, v, dout, y, v_new, s0, ds1, gam, beta)])
+    for name, a, b in zip(("dqs", "dkn", "dbeta", "dgamma"), got, want):
+        err = rel_l2(a, b)
+        print(f"   {name}: rel-L2 {err:.3e}", flush=True)
+        assert err <= 1e-2, f"{name}: rel-L2 {err:.3e}"
