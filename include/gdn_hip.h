@@ -152,16 +152,21 @@ int gdn_chunk_fwd_saving(const gdn_args *args, const gdn_chunk_saves *saves, voi
  *     v, dout, y, v_new  [chunks][64][V]
  *     states, dstates    [chunks][K][V]
  *     gamma, beta   [chunks][64]      prefix sum of g inside the chunk, beta
- * Outputs: dqs, dkn [chunks][64][K] (gradients with respect to qs and kn), dbeta [chunks][64], and
- * dgamma [chunks][64], the gradient with respect to gamma (dg is its reverse prefix sum inside the chunk).
+ *     rq, rk        [chunks][64]      1 / sqrt(|q|^2 + 1e-6), likewise for k, when q and k were normalised
+ *                                     (the l2norm flag of the forward); both NULL otherwise
+ * qs = scale * q (* rq), kn = k (* rk).  Outputs: dq, dk [chunks][64][K], the gradients with respect to q and
+ * k themselves (through the scale and the normalisation), dbeta [chunks][64], and dgamma [chunks][64], the
+ * gradient with respect to gamma (dg is its reverse prefix sum inside the chunk).
  * K = V = 128 only (GDN_ERR_UNSUPPORTED otherwise).  Counterpart upstream: the chunk-local kernels of fla's
  * backward of chunk_gated_delta_rule, reached from gated_deltanet/module.py:197-209 under autograd.
  */
 typedef struct gdn_chunk_local_args {
-    const float *qs, *kn, *v, *dout, *y, *v_new, *states, *dstates, *gamma, *beta;
-    float *dqs, *dkn, *dbeta, *dgamma;
+    const float *qs, *kn, *v, *dout, *y, *v_new, *states, *dstates, *gamma, *beta, *rq, *rk;
+    float *dq, *dk, *dbeta, *dgamma;
     int64_t chunks;
     int32_t K, V;
+    float scale;
+    int32_t reserved;
 } gdn_chunk_local_args;
 int gdn_chunk_bwd_local(const gdn_chunk_local_args *args, void *stream);
 

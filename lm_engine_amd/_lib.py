@@ -55,8 +55,10 @@ class GdnChunkSaves(ctypes.Structure):
 
 class GdnChunkLocalArgs(ctypes.Structure):
     _fields_ = [(name, ctypes.c_void_p) for name in (
-        "qs", "kn", "v", "dout", "y", "v_new", "states", "dstates", "gamma", "beta", "dqs", "dkn", "dbeta", "dgamma",
-    )] + [("chunks", ctypes.c_int64), ("K", ctypes.c_int32), ("V", ctypes.c_int32)]  # fmt: skip
+        "qs", "kn", "v", "dout", "y", "v_new", "states", "dstates", "gamma", "beta", "rq", "rk",
+        "dq", "dk", "dbeta", "dgamma",
+    )] + [("chunks", ctypes.c_int64), ("K", ctypes.c_int32), ("V", ctypes.c_int32), ("scale", ctypes.c_float),
+          ("reserved", ctypes.c_int32)]  # fmt: skip
 
 
 class GdnArgs(ctypes.Structure):

@@ -359,17 +359,17 @@ def gated_delta_rule_backward(
     if on_kernel and (K, V) == _chunk_local_kv():
         from . import ops
 
-        dqs, dkn, dbc, dgam = ops.chunk_local_grads(qs, kn, vc, doc, Y, Vn, S0, dS1, gam, bc)
+        norms = dict(rq=rq[..., 0], rk=rk[..., 0]) if use_qk_l2norm_in_kernel else {}
+        dqc, dkc, dbc, dgam = ops.chunk_local_grads(qs, kn, vc, doc, Y, Vn, S0, dS1, gam, bc, scale, **norms)
     else:
         dqs, dkn, dbc, dgam = _chunk_local_grads(qs, kn, vc, doc, Y, Vn, S0, dS1, gam, bc)
+        dqn = dqs * scale
+        if use_qk_l2norm_in_kernel:
+            dqc, dkc = _l2norm_grad(qn, rq, dqn), _l2norm_grad(kn, rk, dkn)
+        else:
+            dqc, dkc = dqn, dkn
     dvc = Y * bc[..., None]
     dgc = dgam.flip(-1).cumsum(-1).flip(-1)
-
-    dqn = dqs * scale
-    if use_qk_l2norm_in_kernel:
-        dqc, dkc = _l2norm_grad(qn, rq, dqn), _l2norm_grad(kn, rk, dkn)
-    else:
-        dqc, dkc = dqn, dkn
     return (
         pk.unpack(dqc, q.dtype),
         pk.unpack(dkc, k.dtype),

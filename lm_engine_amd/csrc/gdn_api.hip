@@ -113,11 +113,14 @@ int gdn_chunk_fwd_saving(const gdn_args* a, const gdn_chunk_saves* saves, void* 
 int gdn_chunk_bwd_local(const gdn_chunk_local_args* a, void* stream) {
     if (a == nullptr) return GDN_ERR_NULL;
     const void* ptrs[] = {a->qs, a->kn, a->v, a->dout, a->y, a->v_new, a->states, a->dstates, a->gamma, a->beta,
-                          a->dqs, a->dkn, a->dbeta, a->dgamma};
+                          a->dq, a->dk, a->dbeta, a->dgamma};
     for (const void* x : ptrs) {
         if (x == nullptr) return GDN_ERR_NULL;
         if (!aligned(x, 16)) return GDN_ERR_ALIGN;
     }
+    if ((a->rq == nullptr) != (a->rk == nullptr)) return GDN_ERR_NULL;
+    if (a->rq != nullptr && (!aligned(a->rq, 4) || !aligned(a->rk, 4))) return GDN_ERR_ALIGN;
+    if (!(a->scale > 0.f)) return GDN_ERR_SHAPE;
     if (a->chunks <= 0 || a->chunks > 0x7fffffff) return GDN_ERR_SHAPE;
     if (!gdn::chunk_bwd_local_supported(*a)) return GDN_ERR_UNSUPPORTED;
     return gdn::launch_chunk_bwd_local(*a, static_cast<hipStream_t>(stream));

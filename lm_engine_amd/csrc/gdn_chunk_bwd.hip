@@ -47,8 +47,11 @@ struct ChunkLocalParams {
     const float* ds1;
     const float* gam;
     const float* beta;
-    float* dqs;
-    float* dkn;
+    const float* rq;  // 1 / |q|, 1 / |k| per token when q and k were normalised, else NULL
+    const float* rk;
+    float scale;
+    float* dq;
+    float* dk;
     float* dbeta;
     float* dgam;
 };
@@ -80,7 +83,7 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
     __shared__ __attribute__((aligned(16))) bf16_t sVN[C * LDR];
     __shared__ __attribute__((aligned(16))) bf16_t sY[C * LDR];
     __shared__ __attribute__((aligned(16))) bf16_t sST[K * LDR];  // S0, then dS1, then G | G^T | Hm + Hm^T
-    __shared__ float s_gam[C], s_beta[C], s_e[C], s_tail[C], s_dgam[C], s_dbeta[C], s_red[4];
+    __shared__ float s_gam[C], s_beta[C], s_e[C], s_tail[C], s_dgam[C], s_dbeta[C], s_dotq[C], s_dotk[C], s_red[4];
     bf16_t* const sG = sST;
     bf16_t* const sGT = sST + C * LDS64;
     bf16_t* const sH = sST + 2 * C * LDS64;
@@ -107,6 +110,8 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
         s_tail[t] = __expf(p.gam[chunk * C + C - 1] - g);
         s_dgam[t] = 0.f;
         s_dbeta[t] = 0.f;
+        s_dotq[t] = 0.f;
+        s_dotk[t] = 0.f;
     }
     if (t < 4) s_red[t] = 0.f;
     auto put4 = [](bf16_t* dst, f32x4 x) {
@@ -224,6 +229,7 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
 
     // ---- per-token sums over the key dim, then dQ^T and dK^T ----
     float nkd = 0.f;
+    f32x16 accq[2], acck[2];
 #pragma unroll
     for (int tt = 0; tt < 2; tt++) {
         const int i = 32 * tt + l32;
@@ -241,26 +247,53 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
         atomicAdd(&s_dbeta[i], -ei * s_zk);
         nkd += tl * s_kd;
 
-        f32x16 accq, acck;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            accq[r] = dQeT[tt][r] * ei;
-            acck[r] = dKdT[tt][r] * tl - ZT[tt][r] * (bi * ei);
+            accq[tt][r] = dQeT[tt][r] * ei;
+            acck[tt][r] = dKdT[tt][r] * tl - ZT[tt][r] * (bi * ei);
         }
-        accq = mma_nt(sKT + 32 * wave * LDS64, LDS64, sG + 32 * tt * LDS64, LDS64, C, accq, l32, lh);
-        acck = mma_nt(sQT + 32 * wave * LDS64, LDS64, sGT + 32 * tt * LDS64, LDS64, C, acck, l32, lh);
-        acck = mma_nt(sKT + 32 * wave * LDS64, LDS64, sH + 32 * tt * LDS64, LDS64, C, acck, l32, lh);
-        float* dq = p.dqs + (chunk * C + i) * K + 32 * wave + 4 * lh;
-        float* dk = p.dkn + (chunk * C + i) * K + 32 * wave + 4 * lh;
+        accq[tt] = mma_nt(sKT + 32 * wave * LDS64, LDS64, sG + 32 * tt * LDS64, LDS64, C, accq[tt], l32, lh);
+        acck[tt] = mma_nt(sQT + 32 * wave * LDS64, LDS64, sGT + 32 * tt * LDS64, LDS64, C, acck[tt], l32, lh);
+        acck[tt] = mma_nt(sKT + 32 * wave * LDS64, LDS64, sH + 32 * tt * LDS64, LDS64, C, acck[tt], l32, lh);
+        if (p.rq != nullptr) {  // <dQs_i, Qs_i> and <dK_i, K_i> for the backward of the normalisation
+            float dq_q = 0.f, dk_k = 0.f;
 #pragma unroll
-        for (int r4 = 0; r4 < 4; r4++) {
-            *reinterpret_cast<f32x4*>(dq + 8 * r4) = f32x4{accq[4 * r4], accq[4 * r4 + 1], accq[4 * r4 + 2], accq[4 * r4 + 3]};
-            *reinterpret_cast<f32x4*>(dk + 8 * r4) = f32x4{acck[4 * r4], acck[4 * r4 + 1], acck[4 * r4 + 2], acck[4 * r4 + 3]};
+            for (int r = 0; r < 16; r++) {
+                const int d = 32 * wave + 8 * (r / 4) + 4 * lh + r % 4;
+                dq_q += accq[tt][r] * (float)sQT[d * LDS64 + i];
+                dk_k += acck[tt][r] * (float)sKT[d * LDS64 + i];
+            }
+            atomicAdd(&s_dotq[i], dq_q);
+            atomicAdd(&s_dotk[i], dk_k);
         }
     }
     nkd = wave_sum(nkd);
     if (lane == 0) atomicAdd(&s_red[1], nkd);
     __syncthreads();
+
+    // With x = y / r the normalised row (y: input, r = |y|^-1 incl. epsilon): dy = r (dx - x <x, dx>); the scale of
+    // q moves through: Qs = scale Qn, so dQn = scale dQs and Qn <Qn, dQn> = Qs <Qs, dQs> / scale.
+#pragma unroll
+    for (int tt = 0; tt < 2; tt++) {
+        const int i = 32 * tt + l32;
+        float* dq = p.dq + (chunk * C + i) * K + 32 * wave + 4 * lh;
+        float* dk = p.dk + (chunk * C + i) * K + 32 * wave + 4 * lh;
+        const bool norm = p.rq != nullptr;
+        const float rq = norm ? p.rq[chunk * C + i] : 1.f, rk = norm ? p.rk[chunk * C + i] : 1.f;
+        const float cq = norm ? s_dotq[i] / p.scale : 0.f, ck = norm ? s_dotk[i] : 0.f;
+#pragma unroll
+        for (int r4 = 0; r4 < 4; r4++) {
+            f32x4 oq, ok;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int r = 4 * r4 + e, d = 32 * wave + 8 * r4 + 4 * lh + e;
+                oq[e] = rq * (accq[tt][r] * p.scale - cq * (float)sQT[d * LDS64 + i]);
+                ok[e] = rk * (acck[tt][r] - ck * (float)sKT[d * LDS64 + i]);
+            }
+            *reinterpret_cast<f32x4*>(dq + 8 * r4) = oq;
+            *reinterpret_cast<f32x4*>(dk + 8 * r4) = ok;
+        }
+    }
 
     if (t < C) {
         float dg = s_dgam[t];
@@ -276,7 +309,8 @@ int launch_chunk_bwd_local(const gdn_chunk_local_args& a, hipStream_t stream) {
     ChunkLocalParams p;
     p.qs = a.qs, p.kn = a.kn, p.v = a.v, p.dout = a.dout, p.y = a.y, p.vnew = a.v_new;
     p.s0 = a.states, p.ds1 = a.dstates, p.gam = a.gamma, p.beta = a.beta;
-    p.dqs = a.dqs, p.dkn = a.dkn, p.dbeta = a.dbeta, p.dgam = a.dgamma;
+    p.rq = a.rq, p.rk = a.rk, p.scale = a.scale;
+    p.dq = a.dq, p.dk = a.dk, p.dbeta = a.dbeta, p.dgam = a.dgamma;
     hipLaunchKernelGGL(chunk_local_grads_kernel, dim3((unsigned)a.chunks), dim3(BWD_THREADS), 0, stream, p);
     return (int)hipGetLastError();
 }

@@ -257,33 +257,38 @@ def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_ch
 CHUNK_LOCAL_KV = (128, 128)  # head dims gdn_chunk_bwd_local is built for
 
 
-def chunk_local_grads(qs, kn, v, dout, y, v_new, states, dstates, gamma, beta):
+def chunk_local_grads(qs, kn, v, dout, y, v_new, states, dstates, gamma, beta, scale, rq=None, rk=None):
     """``gdn_chunk_bwd_local`` on packed fp32 tensors (``[Bt, NC, 64, K or V]``, states ``[Bt, NC, K, V]``,
-    gamma and beta ``[Bt, NC, 64]``).  Returns ``dqs, dkn`` (like qs), ``dbeta, dgamma`` (like gamma)."""
+    gamma, beta and the inverse norms rq, rk ``[Bt, NC, 64]``; ``qs = scale * q * rq``, ``kn = k * rk``, without
+    rq and rk q and k were not normalised).  Returns ``dq, dk`` (like qs), ``dbeta, dgamma`` (like gamma)."""
     _require_hip_path()
     lib = _lib.load_library()
     Bt, NC, C, K = qs.shape
     V = v.size(-1)
     shapes = {"qs": (Bt, NC, C, K), "kn": (Bt, NC, C, K), "v": (Bt, NC, C, V), "dout": (Bt, NC, C, V),
               "y": (Bt, NC, C, V), "v_new": (Bt, NC, C, V), "states": (Bt, NC, K, V), "dstates": (Bt, NC, K, V),
-              "gamma": (Bt, NC, C), "beta": (Bt, NC, C)}  # fmt: skip
+              "gamma": (Bt, NC, C), "beta": (Bt, NC, C), "rq": (Bt, NC, C), "rk": (Bt, NC, C)}  # fmt: skip
     tensors = dict(qs=qs, kn=kn, v=v, dout=dout, y=y, v_new=v_new, states=states, dstates=dstates, gamma=gamma, beta=beta)
+    if (rq is None) != (rk is None):
+        raise ValueError("rq and rk come together")
+    if rq is not None:
+        tensors.update(rq=rq, rk=rk)
     for name, x in tensors.items():
         if tuple(x.shape) != shapes[name] or x.dtype != torch.float32 or not x.is_cuda:
             raise ValueError(f"{name} must be a device fp32 tensor of shape {shapes[name]}, got {tuple(x.shape)} {x.dtype}")
         tensors[name] = x.contiguous()
     if C != 64 or (K, V) != CHUNK_LOCAL_KV:
         raise ValueError(f"chunk-local gradients are built for chunk 64 and K, V = {CHUNK_LOCAL_KV}")
-    out = dict(dqs=torch.empty_like(tensors["qs"]), dkn=torch.empty_like(tensors["kn"]),
+    out = dict(dq=torch.empty_like(tensors["qs"]), dk=torch.empty_like(tensors["kn"]),
                dbeta=torch.empty_like(tensors["gamma"]), dgamma=torch.empty_like(tensors["gamma"]))  # fmt: skip
     a = _lib.GdnChunkLocalArgs()
     for name, x in {**tensors, **out}.items():
         setattr(a, name, x.data_ptr())
-    a.chunks, a.K, a.V = Bt * NC, K, V
+    a.chunks, a.K, a.V, a.scale = Bt * NC, K, V, float(scale)
     with torch.cuda.device(qs.device):
         stream = ctypes.c_void_p(torch.cuda.current_stream(qs.device).cuda_stream)
         _lib.check_status(lib.gdn_chunk_bwd_local(ctypes.byref(a), stream), "gdn_chunk_bwd_local")
-    return out["dqs"], out["dkn"], out["dbeta"], out["dgamma"]
+    return out["dq"], out["dk"], out["dbeta"], out["dgamma"]
 
 
 class _GatedDeltaRule(torch.autograd.Function):

@@ -157,9 +157,22 @@ def test_chunk_local_kernel_matches_the_batched_gemm_version():
     gam = torch.nn.functional.logsigmoid(rnd(Bt, NC, C) + 2.0).cumsum(-1)
     beta = torch.sigmoid(rnd(Bt, NC, C))
     args = [x.cuda() for x in (qs, kn, v, dout, y, v_new, s0, ds1, gam, beta)]
-    got = ops.chunk_local_grads(*args)
-    want = _chunk_local_grads(*[x.double() for x in (qs, kn, v, dout, y, v_new, s0, ds1, gam, beta)])
-    for name, a, b in zip(("dqs", "dkn", "dbeta", "dgamma"), got, want):
+    dqs, dkn, dbeta, dgamma = _chunk_local_grads(*[x.double() for x in (qs, kn, v, dout, y, v_new, s0, ds1, gam, beta)])
+    scale = K**-0.5
+    # without the normalisation the kernel returns the gradients with respect to q = qs / scale and k = kn ...
+    got = ops.chunk_local_grads(*args, scale)
+    want = (dqs * scale, dkn, dbeta, dgamma)
+    for name, a, b in zip(("dq", "dk", "dbeta", "dgamma"), got, want):
         err = rel_l2(a, b)
         print(f"   {name}: rel-L2 {err:.3e}", flush=True)
+        assert err <= 1e-2, f"{name}: rel-L2 {err:.3e}"
+    # ... and with it, of the rows before they were normalised: x = y r, dy = r (dx - x <x, dx>)
+    rq, rk = torch.rand(Bt, NC, C, generator=gen) + 0.5, torch.rand(Bt, NC, C, generator=gen) + 0.5
+    got = ops.chunk_local_grads(*args, scale, rq=rq.cuda(), rk=rk.cuda())
+    qn, dqn = (qs / scale).double(), dqs * scale
+    want_q = rq[..., None] * (dqn - qn * (qn * dqn).sum(-1, keepdim=True))
+    want_k = rk[..., None] * (dkn - kn.double() * (kn.double() * dkn).sum(-1, keepdim=True))
+    for name, a, b in zip(("dq", "dk"), got[:2], (want_q, want_k)):
+        err = rel_l2(a, b)
+        print(f"   normalised {name}: rel-L2 {err:.3e}", flush=True)
         assert err <= 1e-2, f"{name}: rel-L2 {err:.3e}"
