@@ -33,6 +33,7 @@ EXPORTED_SYMBOLS = (
     "gdn_chunk_fwd_profile",
     "gdn_chunk_fwd_saving",
     "gdn_chunk_bwd_local",
+    "gdn_chunk_bwd_prepare",
     "gdn_causal_conv1d_fwd",
     "gdn_gates_fwd",
     "gdn_gated_rmsnorm_fwd",
@@ -59,6 +60,18 @@ class GdnChunkLocalArgs(ctypes.Structure):
         "dq", "dk", "dbeta", "dgamma",
     )] + [("chunks", ctypes.c_int64), ("K", ctypes.c_int32), ("V", ctypes.c_int32), ("scale", ctypes.c_float),
           ("reserved", ctypes.c_int32)]  # fmt: skip
+
+
+class GdnChunkBwdPrepareArgs(ctypes.Structure):
+    _fields_ = (
+        [(name, ctypes.c_void_p) for name in ("q", "k", "v", "dout", "g", "beta")]
+        + [(f"{x}_stride_{d}", ctypes.c_int64) for x in ("q", "k", "v", "dout") for d in ("b", "t", "h")]
+        + [(name, ctypes.c_int32) for name in ("N", "T", "H", "K", "V", "beta_dtype", "flags")]
+        + [("scale", ctypes.c_float)]
+        + [(name, ctypes.c_void_p) for name in ("qs", "kn", "v_packed", "dout_packed", "gamma", "beta_packed", "rq", "rk",
+                                                "k_mirror", "v_mirror", "records")]
+        + [("records_bytes", ctypes.c_uint64)]
+    )  # fmt: skip
 
 
 class GdnArgs(ctypes.Structure):
@@ -146,6 +159,8 @@ def load_library() -> ctypes.CDLL:
     lib.gdn_chunk_fwd_saving.restype = ctypes.c_int
     lib.gdn_chunk_bwd_local.argtypes = [ctypes.POINTER(GdnChunkLocalArgs), ctypes.c_void_p]
     lib.gdn_chunk_bwd_local.restype = ctypes.c_int
+    lib.gdn_chunk_bwd_prepare.argtypes = [ctypes.POINTER(GdnChunkBwdPrepareArgs), ctypes.c_void_p]
+    lib.gdn_chunk_bwd_prepare.restype = ctypes.c_int
     lib.gdn_causal_conv1d_fwd.argtypes = [ctypes.POINTER(GdnConvArgs), ctypes.c_void_p]
     lib.gdn_causal_conv1d_fwd.restype = ctypes.c_int
     lib.gdn_gates_fwd.argtypes = [ctypes.POINTER(GdnGateArgs), ctypes.c_void_p]

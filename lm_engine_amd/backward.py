@@ -289,6 +289,40 @@ def _chunk_local_grads(qs, kn, vc, doc, Y, Vn, S0, dS1, gam, bc):
     return dqs, dkn, dbc, dgam
 
 
+def _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, l2norm):
+    """The whole backward on four kernel launches (bf16, K = V = 128, whole chunks, one sequence per row):
+    ``gdn_chunk_bwd_prepare`` (packed operands + mirror problem), the saving forward sweep, the scan over the
+    mirror problem, ``gdn_chunk_bwd_local``; torch only reorders Y and unpacks the results."""
+    from . import ops  # late: ops imports this module
+
+    N, T, H, K = q.shape
+    V = v.size(-1)
+    NC, Bt, dev = T // CHUNK, N * H, q.device
+    prep = ops.chunk_bwd_prepare(q, k, v, do, g, beta, scale, l2norm)
+    S0 = torch.empty(Bt, NC, K, V, device=dev)
+    Vn = torch.empty(Bt, NC, CHUNK, V, device=dev)
+    ops.chunk_forward_saving(q, k, v, g, beta, scale, initial_state, None, l2norm, False, S0, Vn, NC)
+    dS1 = torch.empty(Bt, NC, K, V, device=dev)
+    dht32 = None if dht is None else dht.to(torch.float32).contiguous()
+    o_m, dS = ops.chunk_scan_given_records(prep["k_mirror"], prep["v_mirror"], prep["records"], dht32, dS1, NC,
+                                           save_every=2, save_reverse=True)  # fmt: skip
+    Y = o_m.view(N, NC, 2, CHUNK, H, V)[:, :, 0].flip(1, 2).permute(0, 3, 1, 2, 4).reshape(Bt, NC, CHUNK, V).float()
+    norms = dict(rq=prep["rq"], rk=prep["rk"]) if l2norm else {}
+    dqc, dkc, dbc, dgam = ops.chunk_local_grads(prep["qs"], prep["kn"], prep["v"], prep["dout"], Y, Vn, S0, dS1,
+                                                prep["gamma"], prep["beta"], scale, **norms)  # fmt: skip
+    dvc = Y * prep["beta"][..., None]
+    dgc = dgam.flip(-1).cumsum(-1).flip(-1)
+    pk = _Packing(N, T, H, None, False, dev)
+    return (
+        pk.unpack(dqc, q.dtype),
+        pk.unpack(dkc, k.dtype),
+        pk.unpack(dvc, v.dtype),
+        pk.unpack(dgc, g.dtype) if g is not None else None,
+        pk.unpack(dbc, beta.dtype) if beta is not None else None,
+        dS if initial_state is not None else None,
+    )
+
+
 def gated_delta_rule_backward(
     q, k, v, g, beta, do, dht=None, scale=None, initial_state=None, cu_seqlens=None,
     use_qk_l2norm_in_kernel=False, left_padded=False,
@@ -303,6 +337,9 @@ def gated_delta_rule_backward(
     V = v.size(-1)
     dev = q.device
     scale = K**-0.5 if scale is None else scale
+    if (q.is_cuda and q.dtype == torch.bfloat16 and (K, V) == _chunk_local_kv() and cu_seqlens is None
+            and T % CHUNK == 0):  # fmt: skip
+        return _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, use_qk_l2norm_in_kernel)
     pk = _Packing(B, T, H, cu_seqlens, left_padded, dev)
     N, NC, Bt = pk.N, pk.NC, pk.N * H
 

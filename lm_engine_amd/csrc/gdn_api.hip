@@ -126,6 +126,27 @@ int gdn_chunk_bwd_local(const gdn_chunk_local_args* a, void* stream) {
     return gdn::launch_chunk_bwd_local(*a, static_cast<hipStream_t>(stream));
 }
 
+int gdn_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args* a, void* stream) {
+    if (a == nullptr) return GDN_ERR_NULL;
+    const void* ptrs[] = {a->q, a->k, a->v, a->dout, a->qs, a->kn, a->v_packed, a->dout_packed, a->gamma,
+                          a->beta_packed, a->rq, a->rk, a->k_mirror, a->v_mirror, a->records};
+    for (const void* x : ptrs) {
+        if (x == nullptr) return GDN_ERR_NULL;
+        if (!aligned(x, 16)) return GDN_ERR_ALIGN;
+    }
+    if (a->N <= 0 || a->T <= 0 || a->H <= 0 || a->N > 65535 || a->H > 65535) return GDN_ERR_SHAPE;
+    if (!gdn::chunk_bwd_prepare_supported(*a)) return GDN_ERR_UNSUPPORTED;
+    if (a->beta && a->beta_dtype != GDN_BF16 && a->beta_dtype != GDN_F32) return GDN_ERR_UNSUPPORTED;
+    if (!(a->scale > 0.f)) return GDN_ERR_SHAPE;
+    const int64_t strides[] = {a->q_stride_b, a->q_stride_t, a->q_stride_h, a->k_stride_b, a->k_stride_t, a->k_stride_h,
+                               a->v_stride_b, a->v_stride_t, a->v_stride_h, a->dout_stride_b, a->dout_stride_t, a->dout_stride_h};
+    for (int64_t s : strides)
+        if (s < 0 || s % 8 != 0) return GDN_ERR_ALIGN;
+    if ((int64_t)a->N * a->H * (a->T / 64) > 0x7fffffff) return GDN_ERR_UNSUPPORTED;
+    if (!aligned(a->records, 256) || a->records_bytes < gdn::chunk_bwd_record_bytes(*a)) return GDN_ERR_WORKSPACE;
+    return gdn::launch_chunk_bwd_prepare(*a, static_cast<hipStream_t>(stream));
+}
+
 int gdn_chunk_fwd_profile(const gdn_args* a, void* stream, float* kernel_ms) {
     if (kernel_ms == nullptr) return GDN_ERR_NULL;
     int rc = validate_chunk(a);

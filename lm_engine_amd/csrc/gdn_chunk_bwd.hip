@@ -303,6 +303,224 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
     }
 }
 
+
+// ------------------------------------------------------------------------------------------
+// Everything the backward needs per chunk before its two sweeps, one workgroup per (sequence, head, chunk),
+// for batches of whole chunks (one sequence per row, T a multiple of 64):
+//   * the packed fp32 operands of chunk_local_grads_kernel: Qs = scale Q / |Q|, Kn = K / |K|, V, dO, gamma,
+//     beta and the inverse norms;
+//   * the "mirror" problem that turns the reverse sweep into a forward scan (tokens in reverse order; chunk c
+//     becomes chunks A, B = 2 r, 2 r + 1 with r = NC - 1 - c):
+//         A:  v := P^T dO, k := k, T' := T^T mirrored, P := I, row scales of k: -tail / |k| before T',
+//             -beta e / |k| for the state update, e^{gamma_C} decay
+//         B:  v := dO, k := q, T' := I, P := 0, row scale e scale / |q| for the state update, no decay
+//     i.e. the rows of k_m and v_m and both records, in the layout chunk_prepare32_kernel writes.
+// T = (I + A)^-1 is formed by forward substitution in one wave (a lane owns a column, 2016 multiply-adds).
+// ------------------------------------------------------------------------------------------
+constexpr int LDA = 68;  // floats per LDS row of A / T
+
+struct BwdPrepareParams {
+    const bf16_t* q;
+    const bf16_t* k;
+    const bf16_t* v;
+    const bf16_t* dout;
+    const float* g;  // [N][T][H], NULL = 0
+    const void* beta;  // [N][T][H], NULL = 1
+    int beta_dtype;
+    int64_t q_stride_b, q_stride_t, q_stride_h;
+    int64_t k_stride_b, k_stride_t, k_stride_h;
+    int64_t v_stride_b, v_stride_t, v_stride_h;
+    int64_t d_stride_b, d_stride_t, d_stride_h;
+    int N, H, NC;
+    int l2norm;
+    float scale;
+    float* qs;
+    float* kn;
+    float* vc;
+    float* doc;
+    float* gam;
+    float* bc;
+    float* rq;
+    float* rk;
+    bf16_t* k_m;
+    bf16_t* v_m;
+    uint8_t* rec;
+    uint32_t rec_bytes, off_p, off_qs, off_ks, off_cs, off_eg;
+};
+
+__global__ __launch_bounds__(BWD_THREADS) void chunk_bwd_prepare_kernel(const BwdPrepareParams p) {
+    constexpr int K = BWD_K, V = BWD_V;
+    __shared__ __attribute__((aligned(16))) bf16_t sQ[C * LDR];
+    __shared__ __attribute__((aligned(16))) bf16_t sK[C * LDR];
+    __shared__ __attribute__((aligned(16))) bf16_t sDOT[V * LDS64];  // dO^T
+    __shared__ __attribute__((aligned(16))) bf16_t sPT[C * LDS64];   // P^T
+    __shared__ __attribute__((aligned(16))) float sA[C * LDA];       // A, then T in its place
+    __shared__ float s_gam[C], s_beta[C], s_e[C], s_tail[C], s_rq[C], s_rk[C];
+
+    const int t = threadIdx.x;
+    const int lane = t % WAVE, wave = t / WAVE;
+    const int l32 = lane % 32, lh = lane / 32;
+    const int64_t chunk = blockIdx.x;
+    const int ci = (int)(chunk % p.NC);
+    const int chain = (int)(chunk / p.NC);
+    const int n = chain / p.H, h = chain % p.H;
+    const int64_t T = (int64_t)p.NC * C, TM = 2 * T;
+    const int64_t tok0 = (int64_t)ci * C;
+    const int64_t mir0 = (int64_t)(p.NC - 1 - ci) * 2 * C;  // first token of chunk A in the mirror problem
+
+    // ---- gamma (prefix sum of g inside the chunk) and beta: wave 0 ----
+    if (wave == 0) {
+        const int64_t at = ((int64_t)n * T + tok0 + lane) * p.H + h;
+        float x = p.g == nullptr ? 0.f : p.g[at];
+#pragma unroll
+        for (int off = 1; off < WAVE; off <<= 1) {
+            const float y = __shfl_up(x, off, WAVE);
+            if (lane >= off) x += y;
+        }
+        const float gl = __shfl(x, WAVE - 1, WAVE);
+        const float b = load_beta(p.beta, p.beta_dtype, at);
+        s_gam[lane] = x, s_beta[lane] = b, s_e[lane] = __expf(x), s_tail[lane] = __expf(gl - x);
+        p.gam[chunk * C + lane] = x;
+        p.bc[chunk * C + lane] = b;
+    }
+
+    // ---- rows of q, k, v, dO: 16-byte pieces, 16 lanes per row ----
+    const int p8 = t % 16;
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const int row = t / 16 + 16 * it;
+        const int64_t tok = tok0 + row;
+        const bf16x8 qr = *reinterpret_cast<const bf16x8*>(p.q + n * p.q_stride_b + tok * p.q_stride_t + (int64_t)h * p.q_stride_h + 8 * p8);
+        const bf16x8 kr = *reinterpret_cast<const bf16x8*>(p.k + n * p.k_stride_b + tok * p.k_stride_t + (int64_t)h * p.k_stride_h + 8 * p8);
+        const bf16x8 vr = *reinterpret_cast<const bf16x8*>(p.v + n * p.v_stride_b + tok * p.v_stride_t + (int64_t)h * p.v_stride_h + 8 * p8);
+        const bf16x8 dr = *reinterpret_cast<const bf16x8*>(p.dout + n * p.d_stride_b + tok * p.d_stride_t + (int64_t)h * p.d_stride_h + 8 * p8);
+        float ssq = 0.f, ssk = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) ssq += (float)qr[e] * (float)qr[e], ssk += (float)kr[e] * (float)kr[e];
+#pragma unroll
+        for (int off = 8; off >= 1; off >>= 1) ssq += __shfl_xor(ssq, off, WAVE), ssk += __shfl_xor(ssk, off, WAVE);
+        const float rq = p.l2norm ? rsqrtf(ssq + L2NORM_EPS) : 1.f, rk = p.l2norm ? rsqrtf(ssk + L2NORM_EPS) : 1.f;
+        if (p8 == 0) {
+            s_rq[row] = rq, s_rk[row] = rk;
+            p.rq[chunk * C + row] = rq, p.rk[chunk * C + row] = rk;
+        }
+        bf16x8 qb, kb;
+        f32x4 q0, q1, k0, k1, v0, v1, d0, d1;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            q0[e] = (float)qr[e] * rq * p.scale, q1[e] = (float)qr[4 + e] * rq * p.scale;
+            k0[e] = (float)kr[e] * rk, k1[e] = (float)kr[4 + e] * rk;
+            v0[e] = (float)vr[e], v1[e] = (float)vr[4 + e];
+            d0[e] = (float)dr[e], d1[e] = (float)dr[4 + e];
+            qb[e] = (bf16_t)q0[e], qb[4 + e] = (bf16_t)q1[e];
+            kb[e] = (bf16_t)k0[e], kb[4 + e] = (bf16_t)k1[e];
+        }
+        *reinterpret_cast<bf16x8*>(sQ + row * LDR + 8 * p8) = qb;
+        *reinterpret_cast<bf16x8*>(sK + row * LDR + 8 * p8) = kb;
+#pragma unroll
+        for (int e = 0; e < 8; e++) sDOT[(8 * p8 + e) * LDS64 + row] = dr[e];
+        const int64_t packed = (chunk * C + row) * K + 8 * p8;  // K == V
+        *reinterpret_cast<f32x4*>(p.qs + packed) = q0, *reinterpret_cast<f32x4*>(p.qs + packed + 4) = q1;
+        *reinterpret_cast<f32x4*>(p.kn + packed) = k0, *reinterpret_cast<f32x4*>(p.kn + packed + 4) = k1;
+        *reinterpret_cast<f32x4*>(p.vc + packed) = v0, *reinterpret_cast<f32x4*>(p.vc + packed + 4) = v1;
+        *reinterpret_cast<f32x4*>(p.doc + packed) = d0, *reinterpret_cast<f32x4*>(p.doc + packed + 4) = d1;
+        // mirror rows: token `row` of this chunk is token 63 - row of chunks A and B
+        const int64_t rowA = (((int64_t)n * TM + mir0 + (C - 1 - row)) * p.H + h) * K + 8 * p8;
+        const int64_t rowB = rowA + (int64_t)C * p.H * K;
+        *reinterpret_cast<bf16x8*>(p.k_m + rowA) = kr;
+        *reinterpret_cast<bf16x8*>(p.k_m + rowB) = qr;
+        *reinterpret_cast<bf16x8*>(p.v_m + rowB) = dr;
+    }
+    __syncthreads();
+
+    f32x16 zero;
+#pragma unroll
+    for (int r = 0; r < 16; r++) zero[r] = 0.f;
+
+    // ---- A = stril(beta_i E . K K^T) and P^T = tril(E . Q K^T)^T: wave -> tile (ti, tj) ----
+    {
+        const int ti = wave / 2, tj = wave % 2;
+        const f32x16 KK = mma_nt(sK + 32 * ti * LDR, LDR, sK + 32 * tj * LDR, LDR, K, zero, l32, lh);
+        const f32x16 QK = mma_nt(sQ + 32 * ti * LDR, LDR, sK + 32 * tj * LDR, LDR, K, zero, l32, lh);
+        const int j = 32 * tj + l32;
+        const float gj = s_gam[j];
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int i = 32 * ti + 8 * (r / 4) + 4 * lh + r % 4;
+            const float E = i >= j ? __expf(s_gam[i] - gj) : 0.f;
+            sA[i * LDA + j] = i > j ? s_beta[i] * E * KK[r] : 0.f;
+            sPT[j * LDS64 + i] = (bf16_t)(E * QK[r]);
+        }
+    }
+    __syncthreads();
+
+    // ---- P^T dO -> rows of v_m for chunk A: rows j = 32 tj + .., columns v = 32 wave + l32 ----
+#pragma unroll
+    for (int tj = 0; tj < 2; tj++) {
+        const f32x16 u = mma_nt(sPT + 32 * tj * LDS64, LDS64, sDOT + 32 * wave * LDS64, LDS64, C, zero, l32, lh);
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int j = 32 * tj + 8 * (r / 4) + 4 * lh + r % 4;
+            p.v_m[(((int64_t)n * TM + mir0 + (C - 1 - j)) * p.H + h) * V + 32 * wave + l32] = (bf16_t)u[r];
+        }
+    }
+
+    // ---- T = (I + A)^-1 in place of A: lane = column, row i needs rows 0 .. i - 1 ----
+    if (wave == 0) {
+        float Tc[C];
+#pragma unroll
+        for (int i = 0; i < C; i++) {
+            float x = (i == lane) ? 1.f : 0.f;
+#pragma unroll
+            for (int j4 = 0; j4 < (i + 3) / 4; j4++) {
+                const f32x4 a = *reinterpret_cast<const f32x4*>(sA + i * LDA + 4 * j4);  // same address in every lane
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (4 * j4 + e < i) x -= a[e] * Tc[4 * j4 + e];
+            }
+            Tc[i] = x;
+        }
+#pragma unroll
+        for (int i = 0; i < C; i++) sA[i * LDA + lane] = Tc[i];
+    }
+    __syncthreads();
+
+    // ---- the two records ----
+    uint8_t* recA = p.rec + ((int64_t)h * ((int64_t)p.N * 2 * p.NC) + (int64_t)n * 2 * p.NC + 2 * (p.NC - 1 - ci)) * p.rec_bytes;
+    uint8_t* recB = recA + p.rec_bytes;
+    for (int fl = t; fl < 6 * WAVE; fl += BWD_THREADS) {
+        const int f = fl / WAVE, L = fl % WAVE;
+        const int row = 32 * (f < 2 ? 0 : 1) + L % 32;
+        const int col0 = 16 * (f < 2 ? f : f - 2) + 4 * (L / 32);
+        bf16x8 tm, id, zz;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const int col = col0 + (e < 4 ? e : e + 4);
+            // mirrored transpose: entry (row, col) is T[63 - col][63 - row], zero above the diagonal
+            tm[e] = (bf16_t)(row >= col ? sA[(C - 1 - col) * LDA + (C - 1 - row)] : 0.f);
+            id[e] = (bf16_t)(row == col ? 1.f : 0.f);
+            zz[e] = (bf16_t)0.f;
+        }
+        reinterpret_cast<bf16x8*>(recA)[fl] = tm;
+        reinterpret_cast<bf16x8*>(recA + p.off_p)[fl] = id;
+        reinterpret_cast<bf16x8*>(recB)[fl] = id;
+        reinterpret_cast<bf16x8*>(recB + p.off_p)[fl] = zz;
+    }
+    if (t < C) {
+        const int src = C - 1 - t;
+        reinterpret_cast<float*>(recA + p.off_qs)[t] = 0.f;
+        reinterpret_cast<float*>(recA + p.off_ks)[t] = -(s_beta[src] * s_e[src] * s_rk[src]);
+        reinterpret_cast<float*>(recA + p.off_cs)[t] = -(s_tail[src] * s_rk[src]);
+        reinterpret_cast<float*>(recB + p.off_qs)[t] = 0.f;
+        reinterpret_cast<float*>(recB + p.off_ks)[t] = s_e[src] * s_rq[src] * p.scale;
+        reinterpret_cast<float*>(recB + p.off_cs)[t] = 0.f;
+        if (t == 0) {
+            *reinterpret_cast<float*>(recA + p.off_eg) = s_e[C - 1];
+            *reinterpret_cast<float*>(recB + p.off_eg) = 1.f;
+        }
+    }
+}
+
 }  // namespace
 
 int launch_chunk_bwd_local(const gdn_chunk_local_args& a, hipStream_t stream) {
@@ -316,5 +534,36 @@ int launch_chunk_bwd_local(const gdn_chunk_local_args& a, hipStream_t stream) {
 }
 
 bool chunk_bwd_local_supported(const gdn_chunk_local_args& a) { return a.K == BWD_K && a.V == BWD_V; }
+
+bool chunk_bwd_prepare_supported(const gdn_chunk_bwd_prepare_args& a) {
+    return a.K == BWD_K && a.V == BWD_V && a.T > 0 && a.T % C == 0;
+}
+
+uint64_t chunk_bwd_record_bytes(const gdn_chunk_bwd_prepare_args& a) {
+    return (uint64_t)a.H * a.N * 2 * (a.T / C) * record_layout(a.K, a.V).bytes;
+}
+
+int launch_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args& a, hipStream_t stream) {
+    const RecordLayout r = record_layout(a.K, a.V);
+    BwdPrepareParams p;
+    p.q = static_cast<const bf16_t*>(a.q), p.k = static_cast<const bf16_t*>(a.k);
+    p.v = static_cast<const bf16_t*>(a.v), p.dout = static_cast<const bf16_t*>(a.dout);
+    p.g = a.g, p.beta = a.beta, p.beta_dtype = a.beta_dtype;
+    p.q_stride_b = a.q_stride_b, p.q_stride_t = a.q_stride_t, p.q_stride_h = a.q_stride_h;
+    p.k_stride_b = a.k_stride_b, p.k_stride_t = a.k_stride_t, p.k_stride_h = a.k_stride_h;
+    p.v_stride_b = a.v_stride_b, p.v_stride_t = a.v_stride_t, p.v_stride_h = a.v_stride_h;
+    p.d_stride_b = a.dout_stride_b, p.d_stride_t = a.dout_stride_t, p.d_stride_h = a.dout_stride_h;
+    p.N = a.N, p.H = a.H, p.NC = a.T / C;
+    p.l2norm = (a.flags & GDN_FLAG_L2NORM) ? 1 : 0;
+    p.scale = a.scale;
+    p.qs = a.qs, p.kn = a.kn, p.vc = a.v_packed, p.doc = a.dout_packed, p.gam = a.gamma, p.bc = a.beta_packed;
+    p.rq = a.rq, p.rk = a.rk;
+    p.k_m = static_cast<bf16_t*>(a.k_mirror), p.v_m = static_cast<bf16_t*>(a.v_mirror);
+    p.rec = static_cast<uint8_t*>(a.records);
+    p.rec_bytes = r.bytes, p.off_p = r.off_p, p.off_qs = r.off_qs, p.off_ks = r.off_ks, p.off_cs = r.off_cs, p.off_eg = r.off_eg;
+    const int64_t chunks = (int64_t)a.N * a.H * p.NC;
+    hipLaunchKernelGGL(chunk_bwd_prepare_kernel, dim3((unsigned)chunks), dim3(BWD_THREADS), 0, stream, p);
+    return (int)hipGetLastError();
+}
 
 }  // namespace gdn

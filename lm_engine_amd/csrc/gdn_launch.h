@@ -17,5 +17,8 @@ uint64_t chunk_record_bytes(const gdn_args& a);  // the records alone, [H][chunk
 bool chunk_shape_supported(const gdn_args& a);
 int launch_chunk_bwd_local(const gdn_chunk_local_args& a, hipStream_t stream);  // gdn_chunk_bwd.hip
 bool chunk_bwd_local_supported(const gdn_chunk_local_args& a);
+int launch_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args& a, hipStream_t stream);
+bool chunk_bwd_prepare_supported(const gdn_chunk_bwd_prepare_args& a);
+uint64_t chunk_bwd_record_bytes(const gdn_chunk_bwd_prepare_args& a);
 
 }  // namespace gdn

@@ -291,6 +291,57 @@ def chunk_local_grads(qs, kn, v, dout, y, v_new, states, dstates, gamma, beta, s
     return out["dq"], out["dk"], out["dbeta"], out["dgamma"]
 
 
+RECORD_BYTES = 13312  # chunk record of the 32x32x16 kernels (K <= 128)
+
+
+def chunk_bwd_prepare(q, k, v, dout, g, beta, scale, l2norm):
+    """``gdn_chunk_bwd_prepare`` for a batch of whole chunks (``[N, T, H, 128]`` bf16, T a multiple of 64).
+    Returns a dict: the packed fp32 operands of ``chunk_local_grads`` (``qs, kn, v, dout`` ``[N H, T/64, 64, D]``;
+    ``gamma, beta, rq, rk`` ``[N H, T/64, 64]``) and the mirror problem ``k_mirror, v_mirror``
+    ``[N, 2 T, H, D]`` bf16, ``records`` uint8 ``[H, N * 2 T/64, RECORD_BYTES]``."""
+    _require_hip_path()
+    lib = _lib.load_library()
+    N, T, H, K = q.shape
+    V = v.size(-1)
+    if (K, V) != CHUNK_LOCAL_KV or T % 64 != 0 or q.dtype != torch.bfloat16:
+        raise ValueError(f"built for bf16, K, V = {CHUNK_LOCAL_KV} and T a multiple of 64")
+    q, k, v, dout = (_last_dim_contiguous(x) for x in (q, k, v, dout.to(torch.bfloat16)))
+    g = None if g is None else g.to(torch.float32).contiguous()
+    if beta is not None:
+        beta = beta.contiguous() if beta.dtype in (torch.bfloat16, torch.float32) else beta.float().contiguous()
+    dev, NC, Bt = q.device, T // 64, N * H
+    f32 = dict(dtype=torch.float32, device=dev)
+    out = dict(
+        qs=torch.empty(Bt, NC, 64, K, **f32), kn=torch.empty(Bt, NC, 64, K, **f32),
+        v=torch.empty(Bt, NC, 64, V, **f32), dout=torch.empty(Bt, NC, 64, V, **f32),
+        gamma=torch.empty(Bt, NC, 64, **f32), beta=torch.empty(Bt, NC, 64, **f32),
+        rq=torch.empty(Bt, NC, 64, **f32), rk=torch.empty(Bt, NC, 64, **f32),
+        k_mirror=torch.empty(N, 2 * T, H, K, dtype=torch.bfloat16, device=dev),
+        v_mirror=torch.empty(N, 2 * T, H, V, dtype=torch.bfloat16, device=dev),
+        records=torch.empty(H, N * 2 * NC, RECORD_BYTES, dtype=torch.uint8, device=dev),
+    )  # fmt: skip
+    a = _lib.GdnChunkBwdPrepareArgs()
+    a.q, a.k, a.v, a.dout = q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr()
+    a.g = None if g is None else g.data_ptr()
+    a.beta = None if beta is None else beta.data_ptr()
+    for name, x in (("q", q), ("k", k), ("v", v), ("dout", dout)):
+        setattr(a, f"{name}_stride_b", x.stride(0))
+        setattr(a, f"{name}_stride_t", x.stride(1))
+        setattr(a, f"{name}_stride_h", x.stride(2))
+    a.N, a.T, a.H, a.K, a.V = N, T, H, K, V
+    a.beta_dtype = _lib.GDN_F32 if beta is None else _dtype_code(beta.dtype, "beta")
+    a.flags = _lib.GDN_FLAG_L2NORM if l2norm else 0
+    a.scale = float(scale)
+    a.qs, a.kn, a.v_packed, a.dout_packed = (out[n].data_ptr() for n in ("qs", "kn", "v", "dout"))
+    a.gamma, a.beta_packed, a.rq, a.rk = (out[n].data_ptr() for n in ("gamma", "beta", "rq", "rk"))
+    a.k_mirror, a.v_mirror, a.records = (out[n].data_ptr() for n in ("k_mirror", "v_mirror", "records"))
+    a.records_bytes = out["records"].numel()
+    with torch.cuda.device(dev):
+        stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+        _lib.check_status(lib.gdn_chunk_bwd_prepare(ctypes.byref(a), stream), "gdn_chunk_bwd_prepare")
+    return out
+
+
 class _GatedDeltaRule(torch.autograd.Function):
     """Forward on the HIP kernels; backward by ``backward.gated_delta_rule_backward`` from the saved
     inputs (the forward keeps no intermediate results)."""
