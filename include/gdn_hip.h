@@ -167,6 +167,17 @@ typedef struct gdn_chunk_local_args {
     int32_t K, V;
     float scale;
     int32_t reserved;
+    /*
+     * "Final" mode, for batches of whole chunks (chunk index = (n * H + h) * NC + c), when y_mirror != NULL:
+     * Y is read from the output of the scan over the mirror problem of gdn_chunk_bwd_prepare
+     * (bf16 [N, 2 * NC * 64, H, V]) instead of `y`, and the gradients are written in the caller's layout instead
+     * of dq, dk, dbeta, dgamma: dq_out, dk_out [N, NC * 64, H, K] and dv_out [N, NC * 64, H, V] = beta Y (bf16,
+     * contiguous), dg_out and dbeta_out fp32 [N, NC * 64, H] (dg_out is the gradient with respect to g).
+     */
+    const void *y_mirror;
+    void *dq_out, *dk_out, *dv_out;
+    float *dg_out, *dbeta_out;
+    int32_t H, NC;
 } gdn_chunk_local_args;
 int gdn_chunk_bwd_local(const gdn_chunk_local_args *args, void *stream);
 

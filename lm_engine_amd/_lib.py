@@ -59,7 +59,9 @@ class GdnChunkLocalArgs(ctypes.Structure):
         "qs", "kn", "v", "dout", "y", "v_new", "states", "dstates", "gamma", "beta", "rq", "rk",
         "dq", "dk", "dbeta", "dgamma",
     )] + [("chunks", ctypes.c_int64), ("K", ctypes.c_int32), ("V", ctypes.c_int32), ("scale", ctypes.c_float),
-          ("reserved", ctypes.c_int32)]  # fmt: skip
+          ("reserved", ctypes.c_int32)] + [(name, ctypes.c_void_p) for name in (
+        "y_mirror", "dq_out", "dk_out", "dv_out", "dg_out", "dbeta_out",
+    )] + [("H", ctypes.c_int32), ("NC", ctypes.c_int32)]  # fmt: skip
 
 
 class GdnChunkBwdPrepareArgs(ctypes.Structure):

@@ -292,7 +292,7 @@ def _chunk_local_grads(qs, kn, vc, doc, Y, Vn, S0, dS1, gam, bc):
 def _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, l2norm):
     """The whole backward on four kernel launches (bf16, K = V = 128, whole chunks, one sequence per row):
     ``gdn_chunk_bwd_prepare`` (packed operands + mirror problem), the saving forward sweep, the scan over the
-    mirror problem, ``gdn_chunk_bwd_local``; torch only reorders Y and unpacks the results."""
+    mirror problem, ``gdn_chunk_bwd_local`` writing the gradients in the caller's layout."""
     from . import ops  # late: ops imports this module
 
     N, T, H, K = q.shape
@@ -306,19 +306,13 @@ def _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, l2norm
     dht32 = None if dht is None else dht.to(torch.float32).contiguous()
     o_m, dS = ops.chunk_scan_given_records(prep["k_mirror"], prep["v_mirror"], prep["records"], dht32, dS1, NC,
                                            save_every=2, save_reverse=True)  # fmt: skip
-    Y = o_m.view(N, NC, 2, CHUNK, H, V)[:, :, 0].flip(1, 2).permute(0, 3, 1, 2, 4).reshape(Bt, NC, CHUNK, V).float()
-    norms = dict(rq=prep["rq"], rk=prep["rk"]) if l2norm else {}
-    dqc, dkc, dbc, dgam = ops.chunk_local_grads(prep["qs"], prep["kn"], prep["v"], prep["dout"], Y, Vn, S0, dS1,
-                                                prep["gamma"], prep["beta"], scale, **norms)  # fmt: skip
-    dvc = Y * prep["beta"][..., None]
-    dgc = dgam.flip(-1).cumsum(-1).flip(-1)
-    pk = _Packing(N, T, H, None, False, dev)
+    dq, dk, dv, dg, dbeta = ops.chunk_local_grads_final(prep, o_m, Vn, S0, dS1, scale, l2norm, N, H)
     return (
-        pk.unpack(dqc, q.dtype),
-        pk.unpack(dkc, k.dtype),
-        pk.unpack(dvc, v.dtype),
-        pk.unpack(dgc, g.dtype) if g is not None else None,
-        pk.unpack(dbc, beta.dtype) if beta is not None else None,
+        dq,
+        dk,
+        dv,
+        dg.to(g.dtype) if g is not None else None,
+        dbeta.to(beta.dtype) if beta is not None else None,
         dS if initial_state is not None else None,
     )
 

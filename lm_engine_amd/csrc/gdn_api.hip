@@ -112,11 +112,22 @@ int gdn_chunk_fwd_saving(const gdn_args* a, const gdn_chunk_saves* saves, void* 
 
 int gdn_chunk_bwd_local(const gdn_chunk_local_args* a, void* stream) {
     if (a == nullptr) return GDN_ERR_NULL;
-    const void* ptrs[] = {a->qs, a->kn, a->v, a->dout, a->y, a->v_new, a->states, a->dstates, a->gamma, a->beta,
-                          a->dq, a->dk, a->dbeta, a->dgamma};
-    for (const void* x : ptrs) {
+    const bool final_mode = a->y_mirror != nullptr;
+    const void* common[] = {a->qs, a->kn, a->v, a->dout, a->v_new, a->states, a->dstates, a->gamma, a->beta};
+    const void* packed[] = {a->y, a->dq, a->dk, a->dbeta, a->dgamma};
+    const void* final_[] = {a->y_mirror, a->dq_out, a->dk_out, a->dv_out, a->dg_out, a->dbeta_out};
+    for (const void* x : common)
         if (x == nullptr) return GDN_ERR_NULL;
-        if (!aligned(x, 16)) return GDN_ERR_ALIGN;
+        else if (!aligned(x, 16)) return GDN_ERR_ALIGN;
+    if (final_mode) {
+        for (const void* x : final_)
+            if (x == nullptr) return GDN_ERR_NULL;
+            else if (!aligned(x, 16)) return GDN_ERR_ALIGN;
+        if (a->H <= 0 || a->NC <= 0 || a->chunks % ((int64_t)a->H * a->NC) != 0) return GDN_ERR_SHAPE;
+    } else {
+        for (const void* x : packed)
+            if (x == nullptr) return GDN_ERR_NULL;
+            else if (!aligned(x, 16)) return GDN_ERR_ALIGN;
     }
     if ((a->rq == nullptr) != (a->rk == nullptr)) return GDN_ERR_NULL;
     if (a->rq != nullptr && (!aligned(a->rq, 4) || !aligned(a->rk, 4))) return GDN_ERR_ALIGN;

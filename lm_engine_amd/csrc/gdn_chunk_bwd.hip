@@ -54,6 +54,16 @@ struct ChunkLocalParams {
     float* dk;
     float* dbeta;
     float* dgam;
+    // "final" mode (whole-chunk batches; chunk = (n H + h) NC + c): Y is read from the output of the scan over
+    // the mirror problem, and the gradients go out in the caller's layout, [N, NC 64, H, .] bf16 for q, k, v and
+    // fp32 [N, NC 64, H] for g (reverse prefix sum of dgamma done here) and beta
+    const bf16_t* y_mirror;  // [N][2 NC 64][H][V], NULL = packed mode
+    bf16_t* dq_out;
+    bf16_t* dk_out;
+    bf16_t* dv_out;
+    float* dg_out;
+    float* dbeta_out;
+    int H, NC;
 };
 
 // acc[r] += sum_k A[8 (r/4) + 4 h + r%4][k] B[l32][k] over k < kd: A, B point at the first of 32 rows
@@ -96,7 +106,14 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
     const float* kn = p.kn + chunk * C * K;
     const float* vv = p.v + chunk * C * V;
     const float* dout = p.dout + chunk * C * V;
-    const float* yy = p.y + chunk * C * V;
+    const bool final_mode = p.y_mirror != nullptr;
+    const int ci = final_mode ? (int)(chunk % p.NC) : 0;
+    const int chain = final_mode ? (int)(chunk / p.NC) : 0;
+    const int n = final_mode ? chain / p.H : 0, h = final_mode ? chain % p.H : 0;
+    const int64_t T = (int64_t)p.NC * C;
+    const int64_t tok0 = (int64_t)n * T + (int64_t)ci * C;                                  // first token, caller's layout
+    const int64_t mirA = (int64_t)n * 2 * T + (int64_t)(p.NC - 1 - ci) * 2 * C;             // first token of mirror chunk A
+    const float* yy = final_mode ? nullptr : p.y + chunk * C * V;
     const float* vnew = p.vnew + chunk * C * V;
     const float* s0 = p.s0 + chunk * K * V;
     const float* ds1 = p.ds1 + chunk * K * V;
@@ -134,7 +151,14 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
         }
         const f32x4 d = *reinterpret_cast<const f32x4*>(dout + row * V + 4 * c4);
         const f32x4 n = *reinterpret_cast<const f32x4*>(vnew + row * V + 4 * c4);
-        const f32x4 y = *reinterpret_cast<const f32x4*>(yy + row * V + 4 * c4);
+        f32x4 y;
+        if (final_mode) {  // token `row` is token 63 - row of mirror chunk A; dV = beta Y goes out right away
+            y = load4<bf16_t>(p.y_mirror + ((mirA + (C - 1 - row)) * p.H + h) * V + 4 * c4);
+            const float b = p.beta[chunk * C + row];
+            store4<bf16_t>(p.dv_out + ((tok0 + row) * p.H + h) * V + 4 * c4, f32x4{y.x * b, y.y * b, y.z * b, y.w * b});
+        } else {
+            y = *reinterpret_cast<const f32x4*>(yy + row * V + 4 * c4);
+        }
         const f32x4 x = *reinterpret_cast<const f32x4*>(vv + row * V + 4 * c4);
         put4(sDO + row * LDR + 4 * c4, d);
         put4(sVN + row * LDR + 4 * c4, n);
@@ -276,8 +300,7 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
 #pragma unroll
     for (int tt = 0; tt < 2; tt++) {
         const int i = 32 * tt + l32;
-        float* dq = p.dq + (chunk * C + i) * K + 32 * wave + 4 * lh;
-        float* dk = p.dk + (chunk * C + i) * K + 32 * wave + 4 * lh;
+        const int64_t at = final_mode ? ((tok0 + i) * p.H + h) * K + 32 * wave + 4 * lh : (chunk * C + i) * K + 32 * wave + 4 * lh;
         const bool norm = p.rq != nullptr;
         const float rq = norm ? p.rq[chunk * C + i] : 1.f, rk = norm ? p.rk[chunk * C + i] : 1.f;
         const float cq = norm ? s_dotq[i] / p.scale : 0.f, ck = norm ? s_dotk[i] : 0.f;
@@ -290,16 +313,32 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
                 oq[e] = rq * (accq[tt][r] * p.scale - cq * (float)sQT[d * LDS64 + i]);
                 ok[e] = rk * (acck[tt][r] - ck * (float)sKT[d * LDS64 + i]);
             }
-            *reinterpret_cast<f32x4*>(dq + 8 * r4) = oq;
-            *reinterpret_cast<f32x4*>(dk + 8 * r4) = ok;
+            if (final_mode) {
+                store4<bf16_t>(p.dq_out + at + 8 * r4, oq);
+                store4<bf16_t>(p.dk_out + at + 8 * r4, ok);
+            } else {
+                *reinterpret_cast<f32x4*>(p.dq + at + 8 * r4) = oq;
+                *reinterpret_cast<f32x4*>(p.dk + at + 8 * r4) = ok;
+            }
         }
     }
 
-    if (t < C) {
+    if (t < C) {  // wave 0
         float dg = s_dgam[t];
         if (t == C - 1) dg += s_e[C - 1] * s_red[0] + s_red[1];
-        p.dgam[chunk * C + t] = dg;
-        p.dbeta[chunk * C + t] = s_dbeta[t];
+        if (final_mode) {
+            // dg_t = sum of dgamma over the tokens t .. 63 of the chunk
+#pragma unroll
+            for (int off = 1; off < WAVE; off <<= 1) {
+                const float y = __shfl_down(dg, off, WAVE);
+                if (t + off < C) dg += y;
+            }
+            p.dg_out[(tok0 + t) * p.H + h] = dg;
+            p.dbeta_out[(tok0 + t) * p.H + h] = s_dbeta[t];
+        } else {
+            p.dgam[chunk * C + t] = dg;
+            p.dbeta[chunk * C + t] = s_dbeta[t];
+        }
     }
 }
 
@@ -529,6 +568,10 @@ int launch_chunk_bwd_local(const gdn_chunk_local_args& a, hipStream_t stream) {
     p.s0 = a.states, p.ds1 = a.dstates, p.gam = a.gamma, p.beta = a.beta;
     p.rq = a.rq, p.rk = a.rk, p.scale = a.scale;
     p.dq = a.dq, p.dk = a.dk, p.dbeta = a.dbeta, p.dgam = a.dgamma;
+    p.y_mirror = static_cast<const bf16_t*>(a.y_mirror);
+    p.dq_out = static_cast<bf16_t*>(a.dq_out), p.dk_out = static_cast<bf16_t*>(a.dk_out), p.dv_out = static_cast<bf16_t*>(a.dv_out);
+    p.dg_out = a.dg_out, p.dbeta_out = a.dbeta_out;
+    p.H = a.H, p.NC = a.NC;
     hipLaunchKernelGGL(chunk_local_grads_kernel, dim3((unsigned)a.chunks), dim3(BWD_THREADS), 0, stream, p);
     return (int)hipGetLastError();
 }

@@ -291,6 +291,43 @@ def chunk_local_grads(qs, kn, v, dout, y, v_new, states, dstates, gamma, beta, s
     return out["dq"], out["dk"], out["dbeta"], out["dgamma"]
 
 
+def chunk_local_grads_final(prep, y_mirror, v_new, states, dstates, scale, l2norm, N, H):
+    """``gdn_chunk_bwd_local`` in its final mode, for a batch of whole chunks: ``prep`` is what
+    ``chunk_bwd_prepare`` returned, ``y_mirror`` the output of the scan over its mirror problem.  Returns
+    ``dq, dk, dv`` bf16 ``[N, T, H, D]`` and ``dg, dbeta`` fp32 ``[N, T, H]``."""
+    _require_hip_path()
+    lib = _lib.load_library()
+    Bt, NC, C, K = prep["qs"].shape
+    V = prep["v"].size(-1)
+    T, dev = NC * C, y_mirror.device
+    if Bt != N * H or tuple(y_mirror.shape) != (N, 2 * T, H, V) or y_mirror.dtype != torch.bfloat16 or not y_mirror.is_contiguous():
+        raise ValueError("y_mirror must be the contiguous bf16 [N, 2 T, H, V] output of the scan over the mirror problem")
+    for name, x, shape in (("v_new", v_new, (Bt, NC, C, V)), ("states", states, (Bt, NC, K, V)), ("dstates", dstates, (Bt, NC, K, V))):
+        if tuple(x.shape) != shape or x.dtype != torch.float32 or not x.is_contiguous():
+            raise ValueError(f"{name} must be contiguous fp32 {shape}")
+    out = dict(
+        dq_out=torch.empty(N, T, H, K, dtype=torch.bfloat16, device=dev),
+        dk_out=torch.empty(N, T, H, K, dtype=torch.bfloat16, device=dev),
+        dv_out=torch.empty(N, T, H, V, dtype=torch.bfloat16, device=dev),
+        dg_out=torch.empty(N, T, H, dtype=torch.float32, device=dev),
+        dbeta_out=torch.empty(N, T, H, dtype=torch.float32, device=dev),
+    )
+    a = _lib.GdnChunkLocalArgs()
+    a.qs, a.kn, a.v, a.dout = (prep[n].data_ptr() for n in ("qs", "kn", "v", "dout"))
+    a.gamma, a.beta = prep["gamma"].data_ptr(), prep["beta"].data_ptr()
+    if l2norm:
+        a.rq, a.rk = prep["rq"].data_ptr(), prep["rk"].data_ptr()
+    a.v_new, a.states, a.dstates = v_new.data_ptr(), states.data_ptr(), dstates.data_ptr()
+    a.y_mirror = y_mirror.data_ptr()
+    for name, x in out.items():
+        setattr(a, name, x.data_ptr())
+    a.chunks, a.K, a.V, a.scale, a.H, a.NC = Bt * NC, K, V, float(scale), H, NC
+    with torch.cuda.device(dev):
+        stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+        _lib.check_status(lib.gdn_chunk_bwd_local(ctypes.byref(a), stream), "gdn_chunk_bwd_local")
+    return out["dq_out"], out["dk_out"], out["dv_out"], out["dg_out"], out["dbeta_out"]
+
+
 RECORD_BYTES = 13312  # chunk record of the 32x32x16 kernels (K <= 128)
 
 
