@@ -329,9 +329,8 @@ def calibrate_copy():
 
 
 def bench_backward(w, inp, steps, warmup):
-    """One backward pass of the chunked operator on the same workload (``lm_engine_amd.backward``: both sweeps
-    over the chunks on the scan kernel, the chunk-local products as batched library GEMMs), gradient of the
-    output only.  Wall time per call with the device idle before and after."""
+    """One backward pass of the chunked operator on the same workload (``lm_engine_amd.backward``), gradient
+    of the output only.  Wall time per call with the device idle before and after."""
     import torch
 
     from lm_engine_amd.backward import gated_delta_rule_backward
@@ -355,7 +354,9 @@ def bench_backward(w, inp, steps, warmup):
         "steps": steps,
         "ms_per_backward": round(ms, 3),
         "tokens_per_s": round(w.B * w.T / (ms * 1e-3), 1),
-        "composition": "2 scan launches (state-saving variant) + rocBLAS batched GEMMs + elementwise torch ops",
+        "composition": ("5 kernel launches: backward prepare, forward prepare + saving scan, saving scan over the "
+                        "mirror problem, chunk-local gradients" if (w.K, w.V) == (128, 128) and not w.varlen else
+                        "2 saving scans + rocBLAS batched GEMMs + elementwise torch ops"),
     }
 
 
