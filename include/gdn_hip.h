@@ -178,15 +178,21 @@ typedef struct gdn_chunk_local_args {
     void *dq_out, *dk_out, *dv_out;
     float *dg_out, *dbeta_out;
     int32_t H, NC;
+    /* final mode reads the caller's bf16 q, k, v, dout ([N, NC * 64, H, D], element strides) instead of qs, kn, v,
+     * dout, which may then be NULL; rq and rk (or NULL), gamma, beta stay packed fp32 */
+    const void *q_raw, *k_raw, *v_raw, *dout_raw;
+    int64_t q_stride_b, q_stride_t, q_stride_h;
+    int64_t k_stride_b, k_stride_t, k_stride_h;
+    int64_t v_stride_b, v_stride_t, v_stride_h;
+    int64_t dout_stride_b, dout_stride_t, dout_stride_h;
 } gdn_chunk_local_args;
 int gdn_chunk_bwd_local(const gdn_chunk_local_args *args, void *stream);
 
 /*
  * Training support, third part: everything the backward needs per chunk before its two sweeps, for batches
- * of whole chunks (no cu_seqlens, T a multiple of 64; bf16 q, k, v, dout as [N, T, H, D] with element
+ * of whole chunks (no cu_seqlens, T a multiple of 64; bf16 q, k, dout as [N, T, H, D] with element
  * strides; K = V = 128, GDN_ERR_UNSUPPORTED otherwise).  One workgroup per (sequence, head, chunk) writes
- *   - the packed fp32 operands of gdn_chunk_bwd_local: qs, kn [N H T/64][64][K], v_packed, dout_packed
- *     [..][64][V], gamma, beta_packed, rq, rk [..][64];
+ *   - gamma, beta_packed, rq, rk: fp32 [N H T/64][64], operands of gdn_chunk_bwd_local;
  *   - the reverse sweep as a forward scan over 2 T tokens per sequence ("mirror" problem: tokens in reverse
  *     order, chunk c becomes chunks 2 r and 2 r + 1, r = T/64 - 1 - c): k_mirror [N, 2 T, H, K] and
  *     v_mirror [N, 2 T, H, V] (bf16, contiguous) and the chunk records [H][N * 2 T/64], records_bytes >=
@@ -196,18 +202,17 @@ int gdn_chunk_bwd_local(const gdn_chunk_local_args *args, void *stream);
  * flags: GDN_FLAG_L2NORM only.  g (fp32 [N, T, H]) and beta ([N, T, H], beta_dtype) may be NULL (0 and 1).
  */
 typedef struct gdn_chunk_bwd_prepare_args {
-    const void *q, *k, *v, *dout;
+    const void *q, *k, *dout;
     const float *g;
     const void *beta;
     int64_t q_stride_b, q_stride_t, q_stride_h;
     int64_t k_stride_b, k_stride_t, k_stride_h;
-    int64_t v_stride_b, v_stride_t, v_stride_h;
     int64_t dout_stride_b, dout_stride_t, dout_stride_h;
     int32_t N, T, H, K, V;
     int32_t beta_dtype;
     int32_t flags;
     float scale;
-    float *qs, *kn, *v_packed, *dout_packed, *gamma, *beta_packed, *rq, *rk;
+    float *gamma, *beta_packed, *rq, *rk;
     void *k_mirror, *v_mirror, *records;
     uint64_t records_bytes;
 } gdn_chunk_bwd_prepare_args;

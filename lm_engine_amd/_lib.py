@@ -61,17 +61,18 @@ class GdnChunkLocalArgs(ctypes.Structure):
     )] + [("chunks", ctypes.c_int64), ("K", ctypes.c_int32), ("V", ctypes.c_int32), ("scale", ctypes.c_float),
           ("reserved", ctypes.c_int32)] + [(name, ctypes.c_void_p) for name in (
         "y_mirror", "dq_out", "dk_out", "dv_out", "dg_out", "dbeta_out",
-    )] + [("H", ctypes.c_int32), ("NC", ctypes.c_int32)]  # fmt: skip
+    )] + [("H", ctypes.c_int32), ("NC", ctypes.c_int32)] + [(name, ctypes.c_void_p) for name in (
+        "q_raw", "k_raw", "v_raw", "dout_raw",
+    )] + [(f"{x}_stride_{d}", ctypes.c_int64) for x in ("q", "k", "v", "dout") for d in ("b", "t", "h")]  # fmt: skip
 
 
 class GdnChunkBwdPrepareArgs(ctypes.Structure):
     _fields_ = (
-        [(name, ctypes.c_void_p) for name in ("q", "k", "v", "dout", "g", "beta")]
-        + [(f"{x}_stride_{d}", ctypes.c_int64) for x in ("q", "k", "v", "dout") for d in ("b", "t", "h")]
+        [(name, ctypes.c_void_p) for name in ("q", "k", "dout", "g", "beta")]
+        + [(f"{x}_stride_{d}", ctypes.c_int64) for x in ("q", "k", "dout") for d in ("b", "t", "h")]
         + [(name, ctypes.c_int32) for name in ("N", "T", "H", "K", "V", "beta_dtype", "flags")]
         + [("scale", ctypes.c_float)]
-        + [(name, ctypes.c_void_p) for name in ("qs", "kn", "v_packed", "dout_packed", "gamma", "beta_packed", "rq", "rk",
-                                                "k_mirror", "v_mirror", "records")]
+        + [(name, ctypes.c_void_p) for name in ("gamma", "beta_packed", "rq", "rk", "k_mirror", "v_mirror", "records")]
         + [("records_bytes", ctypes.c_uint64)]
     )  # fmt: skip
 

@@ -298,7 +298,8 @@ def _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, l2norm
     N, T, H, K = q.shape
     V = v.size(-1)
     NC, Bt, dev = T // CHUNK, N * H, q.device
-    prep = ops.chunk_bwd_prepare(q, k, v, do, g, beta, scale, l2norm)
+    q, k, v, do = (x if x.stride(-1) == 1 else x.contiguous() for x in (q, k, v, do.to(torch.bfloat16)))
+    prep = ops.chunk_bwd_prepare(q, k, do, g, beta, scale, l2norm, V)
     S0 = torch.empty(Bt, NC, K, V, device=dev)
     Vn = torch.empty(Bt, NC, CHUNK, V, device=dev)
     ops.chunk_forward_saving(q, k, v, g, beta, scale, initial_state, None, l2norm, False, S0, Vn, NC)
@@ -306,7 +307,7 @@ def _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, l2norm
     dht32 = None if dht is None else dht.to(torch.float32).contiguous()
     o_m, dS = ops.chunk_scan_given_records(prep["k_mirror"], prep["v_mirror"], prep["records"], dht32, dS1, NC,
                                            save_every=2, save_reverse=True)  # fmt: skip
-    dq, dk, dv, dg, dbeta = ops.chunk_local_grads_final(prep, o_m, Vn, S0, dS1, scale, l2norm, N, H)
+    dq, dk, dv, dg, dbeta = ops.chunk_local_grads_final(q, k, v, do, prep, o_m, Vn, S0, dS1, scale, l2norm)
     return (
         dq,
         dk,

@@ -113,9 +113,10 @@ int gdn_chunk_fwd_saving(const gdn_args* a, const gdn_chunk_saves* saves, void* 
 int gdn_chunk_bwd_local(const gdn_chunk_local_args* a, void* stream) {
     if (a == nullptr) return GDN_ERR_NULL;
     const bool final_mode = a->y_mirror != nullptr;
-    const void* common[] = {a->qs, a->kn, a->v, a->dout, a->v_new, a->states, a->dstates, a->gamma, a->beta};
-    const void* packed[] = {a->y, a->dq, a->dk, a->dbeta, a->dgamma};
-    const void* final_[] = {a->y_mirror, a->dq_out, a->dk_out, a->dv_out, a->dg_out, a->dbeta_out};
+    const void* common[] = {a->v_new, a->states, a->dstates, a->gamma, a->beta};
+    const void* packed[] = {a->qs, a->kn, a->v, a->dout, a->y, a->dq, a->dk, a->dbeta, a->dgamma};
+    const void* final_[] = {a->y_mirror, a->dq_out, a->dk_out, a->dv_out, a->dg_out, a->dbeta_out,
+                            a->q_raw, a->k_raw, a->v_raw, a->dout_raw};
     for (const void* x : common)
         if (x == nullptr) return GDN_ERR_NULL;
         else if (!aligned(x, 16)) return GDN_ERR_ALIGN;
@@ -124,6 +125,10 @@ int gdn_chunk_bwd_local(const gdn_chunk_local_args* a, void* stream) {
             if (x == nullptr) return GDN_ERR_NULL;
             else if (!aligned(x, 16)) return GDN_ERR_ALIGN;
         if (a->H <= 0 || a->NC <= 0 || a->chunks % ((int64_t)a->H * a->NC) != 0) return GDN_ERR_SHAPE;
+        const int64_t raw_strides[] = {a->q_stride_b, a->q_stride_t, a->q_stride_h, a->k_stride_b, a->k_stride_t, a->k_stride_h,
+                                       a->v_stride_b, a->v_stride_t, a->v_stride_h, a->dout_stride_b, a->dout_stride_t, a->dout_stride_h};
+        for (int64_t st : raw_strides)
+            if (st < 0 || st % 8 != 0) return GDN_ERR_ALIGN;
     } else {
         for (const void* x : packed)
             if (x == nullptr) return GDN_ERR_NULL;
@@ -139,8 +144,7 @@ int gdn_chunk_bwd_local(const gdn_chunk_local_args* a, void* stream) {
 
 int gdn_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args* a, void* stream) {
     if (a == nullptr) return GDN_ERR_NULL;
-    const void* ptrs[] = {a->q, a->k, a->v, a->dout, a->qs, a->kn, a->v_packed, a->dout_packed, a->gamma,
-                          a->beta_packed, a->rq, a->rk, a->k_mirror, a->v_mirror, a->records};
+    const void* ptrs[] = {a->q, a->k, a->dout, a->gamma, a->beta_packed, a->rq, a->rk, a->k_mirror, a->v_mirror, a->records};
     for (const void* x : ptrs) {
         if (x == nullptr) return GDN_ERR_NULL;
         if (!aligned(x, 16)) return GDN_ERR_ALIGN;
@@ -150,7 +154,7 @@ int gdn_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args* a, void* stream) {
     if (a->beta && a->beta_dtype != GDN_BF16 && a->beta_dtype != GDN_F32) return GDN_ERR_UNSUPPORTED;
     if (!(a->scale > 0.f)) return GDN_ERR_SHAPE;
     const int64_t strides[] = {a->q_stride_b, a->q_stride_t, a->q_stride_h, a->k_stride_b, a->k_stride_t, a->k_stride_h,
-                               a->v_stride_b, a->v_stride_t, a->v_stride_h, a->dout_stride_b, a->dout_stride_t, a->dout_stride_h};
+                               a->dout_stride_b, a->dout_stride_t, a->dout_stride_h};
     for (int64_t s : strides)
         if (s < 0 || s % 8 != 0) return GDN_ERR_ALIGN;
     if ((int64_t)a->N * a->H * (a->T / 64) > 0x7fffffff) return GDN_ERR_UNSUPPORTED;

@@ -58,6 +58,15 @@ struct ChunkLocalParams {
     // the mirror problem, and the gradients go out in the caller's layout, [N, NC 64, H, .] bf16 for q, k, v and
     // fp32 [N, NC 64, H] for g (reverse prefix sum of dgamma done here) and beta
     const bf16_t* y_mirror;  // [N][2 NC 64][H][V], NULL = packed mode
+    // final mode reads the caller's q, k, v, dO (bf16, element strides) instead of the packed qs, kn, v, dout
+    const bf16_t* q_raw;
+    const bf16_t* k_raw;
+    const bf16_t* v_raw;
+    const bf16_t* d_raw;
+    int64_t q_stride_b, q_stride_t, q_stride_h;
+    int64_t k_stride_b, k_stride_t, k_stride_h;
+    int64_t v_stride_b, v_stride_t, v_stride_h;
+    int64_t d_stride_b, d_stride_t, d_stride_h;
     bf16_t* dq_out;
     bf16_t* dk_out;
     bf16_t* dv_out;
@@ -102,7 +111,7 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
     const int lane = t % WAVE, wave = t / WAVE;
     const int l32 = lane % 32, lh = lane / 32;
     const int64_t chunk = blockIdx.x;
-    const float* qs = p.qs + chunk * C * K;
+    const float* qs = p.qs + chunk * C * K;  // packed mode only
     const float* kn = p.kn + chunk * C * K;
     const float* vv = p.v + chunk * C * V;
     const float* dout = p.dout + chunk * C * V;
@@ -138,32 +147,68 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
     };
     float yv[8];  // <Y_i, V_i> pieces, reduced after the barrier (s_dbeta is being cleared above)
 #pragma unroll
-    for (int i = 0; i < 8; i++) {  // [64][128] fp32: 2048 groups of 4, row = 8 i + t / 32
-        const int idx = t + BWD_THREADS * i, row = idx / 32, c4 = idx % 32;
-        const f32x4 a = *reinterpret_cast<const f32x4*>(qs + row * K + 4 * c4);
-        const f32x4 b = *reinterpret_cast<const f32x4*>(kn + row * K + 4 * c4);
-        put4(sQ + row * LDR + 4 * c4, a);
-        put4(sK + row * LDR + 4 * c4, b);
+    for (int i = 0; i < 8; i++) yv[i] = 0.f;
+    if (final_mode) {
+        // rows of the caller's q, k, v, dO and of Y (token `row` is token 63 - row of mirror chunk A) as 16-byte
+        // pieces, 16 lanes per row; V~ below
+        const int p8 = t % 16;
+        const int64_t tl = (int64_t)ci * C;  // first token of the chunk inside its sequence
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-            sQT[(4 * c4 + e) * LDS64 + row] = (bf16_t)a[e];
-            sKT[(4 * c4 + e) * LDS64 + row] = (bf16_t)b[e];
-        }
-        const f32x4 d = *reinterpret_cast<const f32x4*>(dout + row * V + 4 * c4);
-        const f32x4 n = *reinterpret_cast<const f32x4*>(vnew + row * V + 4 * c4);
-        f32x4 y;
-        if (final_mode) {  // token `row` is token 63 - row of mirror chunk A; dV = beta Y goes out right away
-            y = load4<bf16_t>(p.y_mirror + ((mirA + (C - 1 - row)) * p.H + h) * V + 4 * c4);
+        for (int it = 0; it < 4; it++) {
+            const int row = t / 16 + 16 * it;
+            const bf16x8 qr = *reinterpret_cast<const bf16x8*>(p.q_raw + n * p.q_stride_b + (tl + row) * p.q_stride_t + (int64_t)h * p.q_stride_h + 8 * p8);
+            const bf16x8 kr = *reinterpret_cast<const bf16x8*>(p.k_raw + n * p.k_stride_b + (tl + row) * p.k_stride_t + (int64_t)h * p.k_stride_h + 8 * p8);
+            const bf16x8 vr = *reinterpret_cast<const bf16x8*>(p.v_raw + n * p.v_stride_b + (tl + row) * p.v_stride_t + (int64_t)h * p.v_stride_h + 8 * p8);
+            const bf16x8 dr = *reinterpret_cast<const bf16x8*>(p.d_raw + n * p.d_stride_b + (tl + row) * p.d_stride_t + (int64_t)h * p.d_stride_h + 8 * p8);
+            const bf16x8 yr = *reinterpret_cast<const bf16x8*>(p.y_mirror + ((mirA + (C - 1 - row)) * p.H + h) * V + 8 * p8);
+            const float fq = (p.rq != nullptr ? p.rq[chunk * C + row] : 1.f) * p.scale;
+            const float fk = p.rk != nullptr ? p.rk[chunk * C + row] : 1.f;
             const float b = p.beta[chunk * C + row];
-            store4<bf16_t>(p.dv_out + ((tok0 + row) * p.H + h) * V + 4 * c4, f32x4{y.x * b, y.y * b, y.z * b, y.w * b});
-        } else {
-            y = *reinterpret_cast<const f32x4*>(yy + row * V + 4 * c4);
+            bf16x8 qb, kb, dv;
+            float acc = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                qb[e] = (bf16_t)((float)qr[e] * fq);
+                kb[e] = (bf16_t)((float)kr[e] * fk);
+                dv[e] = (bf16_t)((float)yr[e] * b);
+                acc += (float)yr[e] * (float)vr[e];
+                sQT[(8 * p8 + e) * LDS64 + row] = qb[e];
+                sKT[(8 * p8 + e) * LDS64 + row] = kb[e];
+            }
+            *reinterpret_cast<bf16x8*>(sQ + row * LDR + 8 * p8) = qb;
+            *reinterpret_cast<bf16x8*>(sK + row * LDR + 8 * p8) = kb;
+            *reinterpret_cast<bf16x8*>(sDO + row * LDR + 8 * p8) = dr;
+            *reinterpret_cast<bf16x8*>(sY + row * LDR + 8 * p8) = yr;
+            *reinterpret_cast<bf16x8*>(p.dv_out + ((tok0 + row) * p.H + h) * V + 8 * p8) = dv;  // dV = beta Y
+            yv[it] = acc;
         }
-        const f32x4 x = *reinterpret_cast<const f32x4*>(vv + row * V + 4 * c4);
-        put4(sDO + row * LDR + 4 * c4, d);
-        put4(sVN + row * LDR + 4 * c4, n);
-        put4(sY + row * LDR + 4 * c4, y);
-        yv[i] = y.x * x.x + y.y * x.y + y.z * x.z + y.w * x.w;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int idx = t + BWD_THREADS * i, row = idx / 32, c4 = idx % 32;
+            put4(sVN + row * LDR + 4 * c4, *reinterpret_cast<const f32x4*>(vnew + row * V + 4 * c4));
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {  // [64][128] fp32: 2048 groups of 4, row = 8 i + t / 32
+            const int idx = t + BWD_THREADS * i, row = idx / 32, c4 = idx % 32;
+            const f32x4 a = *reinterpret_cast<const f32x4*>(qs + row * K + 4 * c4);
+            const f32x4 b = *reinterpret_cast<const f32x4*>(kn + row * K + 4 * c4);
+            put4(sQ + row * LDR + 4 * c4, a);
+            put4(sK + row * LDR + 4 * c4, b);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                sQT[(4 * c4 + e) * LDS64 + row] = (bf16_t)a[e];
+                sKT[(4 * c4 + e) * LDS64 + row] = (bf16_t)b[e];
+            }
+            const f32x4 d = *reinterpret_cast<const f32x4*>(dout + row * V + 4 * c4);
+            const f32x4 n4 = *reinterpret_cast<const f32x4*>(vnew + row * V + 4 * c4);
+            const f32x4 y = *reinterpret_cast<const f32x4*>(yy + row * V + 4 * c4);
+            const f32x4 x = *reinterpret_cast<const f32x4*>(vv + row * V + 4 * c4);
+            put4(sDO + row * LDR + 4 * c4, d);
+            put4(sVN + row * LDR + 4 * c4, n4);
+            put4(sY + row * LDR + 4 * c4, y);
+            yv[i] = y.x * x.x + y.y * x.y + y.z * x.z + y.w * x.w;
+        }
     }
 #pragma unroll
     for (int i = 0; i < 16; i++) {  // S0 [128][128] fp32: row = 8 i + t / 32
@@ -171,10 +216,20 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
         put4(sST + row * LDR + 4 * c4, *reinterpret_cast<const f32x4*>(s0 + row * V + 4 * c4));
     }
     __syncthreads();
+    if (final_mode) {
 #pragma unroll
-    for (int i = 0; i < 8; i++) {  // the 32 lanes of a wave half hold one row
-        const float s = half_sum(yv[i]);
-        if (l32 == 0) atomicAdd(&s_dbeta[8 * i + t / 32], s);
+        for (int it = 0; it < 4; it++) {  // 16 lanes hold one row
+            float x = yv[it];
+#pragma unroll
+            for (int off = 8; off >= 1; off >>= 1) x += __shfl_xor(x, off, WAVE);
+            if (t % 16 == 0) atomicAdd(&s_dbeta[t / 16 + 16 * it], x);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {  // the 32 lanes of a wave half hold one row
+            const float x = half_sum(yv[i]);
+            if (l32 == 0) atomicAdd(&s_dbeta[8 * i + t / 32], x);
+        }
     }
 
     f32x16 zero;
@@ -346,8 +401,8 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
 // ------------------------------------------------------------------------------------------
 // Everything the backward needs per chunk before its two sweeps, one workgroup per (sequence, head, chunk),
 // for batches of whole chunks (one sequence per row, T a multiple of 64):
-//   * the packed fp32 operands of chunk_local_grads_kernel: Qs = scale Q / |Q|, Kn = K / |K|, V, dO, gamma,
-//     beta and the inverse norms;
+//   * gamma, beta (fp32) and the inverse norms of the rows of q and k, packed per chunk, for
+//     chunk_local_grads_kernel;
 //   * the "mirror" problem that turns the reverse sweep into a forward scan (tokens in reverse order; chunk c
 //     becomes chunks A, B = 2 r, 2 r + 1 with r = NC - 1 - c):
 //         A:  v := P^T dO, k := k, T' := T^T mirrored, P := I, row scales of k: -tail / |k| before T',
@@ -361,22 +416,16 @@ constexpr int LDA = 68;  // floats per LDS row of A / T
 struct BwdPrepareParams {
     const bf16_t* q;
     const bf16_t* k;
-    const bf16_t* v;
     const bf16_t* dout;
     const float* g;  // [N][T][H], NULL = 0
     const void* beta;  // [N][T][H], NULL = 1
     int beta_dtype;
     int64_t q_stride_b, q_stride_t, q_stride_h;
     int64_t k_stride_b, k_stride_t, k_stride_h;
-    int64_t v_stride_b, v_stride_t, v_stride_h;
     int64_t d_stride_b, d_stride_t, d_stride_h;
     int N, H, NC;
     int l2norm;
     float scale;
-    float* qs;
-    float* kn;
-    float* vc;
-    float* doc;
     float* gam;
     float* bc;
     float* rq;
@@ -431,7 +480,6 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_bwd_prepare_kernel(const Bw
         const int64_t tok = tok0 + row;
         const bf16x8 qr = *reinterpret_cast<const bf16x8*>(p.q + n * p.q_stride_b + tok * p.q_stride_t + (int64_t)h * p.q_stride_h + 8 * p8);
         const bf16x8 kr = *reinterpret_cast<const bf16x8*>(p.k + n * p.k_stride_b + tok * p.k_stride_t + (int64_t)h * p.k_stride_h + 8 * p8);
-        const bf16x8 vr = *reinterpret_cast<const bf16x8*>(p.v + n * p.v_stride_b + tok * p.v_stride_t + (int64_t)h * p.v_stride_h + 8 * p8);
         const bf16x8 dr = *reinterpret_cast<const bf16x8*>(p.dout + n * p.d_stride_b + tok * p.d_stride_t + (int64_t)h * p.d_stride_h + 8 * p8);
         float ssq = 0.f, ssk = 0.f;
 #pragma unroll
@@ -444,25 +492,15 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_bwd_prepare_kernel(const Bw
             p.rq[chunk * C + row] = rq, p.rk[chunk * C + row] = rk;
         }
         bf16x8 qb, kb;
-        f32x4 q0, q1, k0, k1, v0, v1, d0, d1;
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-            q0[e] = (float)qr[e] * rq * p.scale, q1[e] = (float)qr[4 + e] * rq * p.scale;
-            k0[e] = (float)kr[e] * rk, k1[e] = (float)kr[4 + e] * rk;
-            v0[e] = (float)vr[e], v1[e] = (float)vr[4 + e];
-            d0[e] = (float)dr[e], d1[e] = (float)dr[4 + e];
-            qb[e] = (bf16_t)q0[e], qb[4 + e] = (bf16_t)q1[e];
-            kb[e] = (bf16_t)k0[e], kb[4 + e] = (bf16_t)k1[e];
+        for (int e = 0; e < 8; e++) {
+            qb[e] = (bf16_t)((float)qr[e] * rq * p.scale);
+            kb[e] = (bf16_t)((float)kr[e] * rk);
         }
         *reinterpret_cast<bf16x8*>(sQ + row * LDR + 8 * p8) = qb;
         *reinterpret_cast<bf16x8*>(sK + row * LDR + 8 * p8) = kb;
 #pragma unroll
         for (int e = 0; e < 8; e++) sDOT[(8 * p8 + e) * LDS64 + row] = dr[e];
-        const int64_t packed = (chunk * C + row) * K + 8 * p8;  // K == V
-        *reinterpret_cast<f32x4*>(p.qs + packed) = q0, *reinterpret_cast<f32x4*>(p.qs + packed + 4) = q1;
-        *reinterpret_cast<f32x4*>(p.kn + packed) = k0, *reinterpret_cast<f32x4*>(p.kn + packed + 4) = k1;
-        *reinterpret_cast<f32x4*>(p.vc + packed) = v0, *reinterpret_cast<f32x4*>(p.vc + packed + 4) = v1;
-        *reinterpret_cast<f32x4*>(p.doc + packed) = d0, *reinterpret_cast<f32x4*>(p.doc + packed + 4) = d1;
         // mirror rows: token `row` of this chunk is token 63 - row of chunks A and B
         const int64_t rowA = (((int64_t)n * TM + mir0 + (C - 1 - row)) * p.H + h) * K + 8 * p8;
         const int64_t rowB = rowA + (int64_t)C * p.H * K;
@@ -572,6 +610,12 @@ int launch_chunk_bwd_local(const gdn_chunk_local_args& a, hipStream_t stream) {
     p.dq_out = static_cast<bf16_t*>(a.dq_out), p.dk_out = static_cast<bf16_t*>(a.dk_out), p.dv_out = static_cast<bf16_t*>(a.dv_out);
     p.dg_out = a.dg_out, p.dbeta_out = a.dbeta_out;
     p.H = a.H, p.NC = a.NC;
+    p.q_raw = static_cast<const bf16_t*>(a.q_raw), p.k_raw = static_cast<const bf16_t*>(a.k_raw);
+    p.v_raw = static_cast<const bf16_t*>(a.v_raw), p.d_raw = static_cast<const bf16_t*>(a.dout_raw);
+    p.q_stride_b = a.q_stride_b, p.q_stride_t = a.q_stride_t, p.q_stride_h = a.q_stride_h;
+    p.k_stride_b = a.k_stride_b, p.k_stride_t = a.k_stride_t, p.k_stride_h = a.k_stride_h;
+    p.v_stride_b = a.v_stride_b, p.v_stride_t = a.v_stride_t, p.v_stride_h = a.v_stride_h;
+    p.d_stride_b = a.dout_stride_b, p.d_stride_t = a.dout_stride_t, p.d_stride_h = a.dout_stride_h;
     hipLaunchKernelGGL(chunk_local_grads_kernel, dim3((unsigned)a.chunks), dim3(BWD_THREADS), 0, stream, p);
     return (int)hipGetLastError();
 }
@@ -590,16 +634,15 @@ int launch_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args& a, hipStream_t st
     const RecordLayout r = record_layout(a.K, a.V);
     BwdPrepareParams p;
     p.q = static_cast<const bf16_t*>(a.q), p.k = static_cast<const bf16_t*>(a.k);
-    p.v = static_cast<const bf16_t*>(a.v), p.dout = static_cast<const bf16_t*>(a.dout);
+    p.dout = static_cast<const bf16_t*>(a.dout);
     p.g = a.g, p.beta = a.beta, p.beta_dtype = a.beta_dtype;
     p.q_stride_b = a.q_stride_b, p.q_stride_t = a.q_stride_t, p.q_stride_h = a.q_stride_h;
     p.k_stride_b = a.k_stride_b, p.k_stride_t = a.k_stride_t, p.k_stride_h = a.k_stride_h;
-    p.v_stride_b = a.v_stride_b, p.v_stride_t = a.v_stride_t, p.v_stride_h = a.v_stride_h;
     p.d_stride_b = a.dout_stride_b, p.d_stride_t = a.dout_stride_t, p.d_stride_h = a.dout_stride_h;
     p.N = a.N, p.H = a.H, p.NC = a.T / C;
     p.l2norm = (a.flags & GDN_FLAG_L2NORM) ? 1 : 0;
     p.scale = a.scale;
-    p.qs = a.qs, p.kn = a.kn, p.vc = a.v_packed, p.doc = a.dout_packed, p.gam = a.gamma, p.bc = a.beta_packed;
+    p.gam = a.gamma, p.bc = a.beta_packed;
     p.rq = a.rq, p.rk = a.rk;
     p.k_m = static_cast<bf16_t*>(a.k_mirror), p.v_m = static_cast<bf16_t*>(a.v_mirror);
     p.rec = static_cast<uint8_t*>(a.records);

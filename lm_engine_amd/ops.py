@@ -291,16 +291,18 @@ def chunk_local_grads(qs, kn, v, dout, y, v_new, states, dstates, gamma, beta, s
     return out["dq"], out["dk"], out["dbeta"], out["dgamma"]
 
 
-def chunk_local_grads_final(prep, y_mirror, v_new, states, dstates, scale, l2norm, N, H):
-    """``gdn_chunk_bwd_local`` in its final mode, for a batch of whole chunks: ``prep`` is what
-    ``chunk_bwd_prepare`` returned, ``y_mirror`` the output of the scan over its mirror problem.  Returns
-    ``dq, dk, dv`` bf16 ``[N, T, H, D]`` and ``dg, dbeta`` fp32 ``[N, T, H]``."""
+def chunk_local_grads_final(q, k, v, dout, prep, y_mirror, v_new, states, dstates, scale, l2norm):
+    """``gdn_chunk_bwd_local`` in its final mode, for a batch of whole chunks: q, k, v, dout are the caller's bf16
+    tensors (last dim contiguous), ``prep`` what ``chunk_bwd_prepare`` returned, ``y_mirror`` the output of the
+    scan over its mirror problem.  Returns ``dq, dk, dv`` bf16 ``[N, T, H, D]`` and ``dg, dbeta`` fp32
+    ``[N, T, H]``."""
     _require_hip_path()
     lib = _lib.load_library()
-    Bt, NC, C, K = prep["qs"].shape
-    V = prep["v"].size(-1)
-    T, dev = NC * C, y_mirror.device
-    if Bt != N * H or tuple(y_mirror.shape) != (N, 2 * T, H, V) or y_mirror.dtype != torch.bfloat16 or not y_mirror.is_contiguous():
+    N, T, H, K = q.shape
+    V = v.size(-1)
+    Bt, NC, C = prep["gamma"].shape
+    dev = y_mirror.device
+    if Bt != N * H or NC * C != T or tuple(y_mirror.shape) != (N, 2 * T, H, V) or y_mirror.dtype != torch.bfloat16 or not y_mirror.is_contiguous():
         raise ValueError("y_mirror must be the contiguous bf16 [N, 2 T, H, V] output of the scan over the mirror problem")
     for name, x, shape in (("v_new", v_new, (Bt, NC, C, V)), ("states", states, (Bt, NC, K, V)), ("dstates", dstates, (Bt, NC, K, V))):
         if tuple(x.shape) != shape or x.dtype != torch.float32 or not x.is_contiguous():
@@ -313,12 +315,18 @@ def chunk_local_grads_final(prep, y_mirror, v_new, states, dstates, scale, l2nor
         dbeta_out=torch.empty(N, T, H, dtype=torch.float32, device=dev),
     )
     a = _lib.GdnChunkLocalArgs()
-    a.qs, a.kn, a.v, a.dout = (prep[n].data_ptr() for n in ("qs", "kn", "v", "dout"))
     a.gamma, a.beta = prep["gamma"].data_ptr(), prep["beta"].data_ptr()
     if l2norm:
         a.rq, a.rk = prep["rq"].data_ptr(), prep["rk"].data_ptr()
     a.v_new, a.states, a.dstates = v_new.data_ptr(), states.data_ptr(), dstates.data_ptr()
     a.y_mirror = y_mirror.data_ptr()
+    for name, x in (("q", q), ("k", k), ("v", v), ("dout", dout)):
+        if x.dtype != torch.bfloat16 or x.stride(-1) != 1:
+            raise ValueError(f"{name} must be bf16 with a contiguous last dim")
+        setattr(a, f"{name}_raw", x.data_ptr())
+        setattr(a, f"{name}_stride_b", x.stride(0))
+        setattr(a, f"{name}_stride_t", x.stride(1))
+        setattr(a, f"{name}_stride_h", x.stride(2))
     for name, x in out.items():
         setattr(a, name, x.data_ptr())
     a.chunks, a.K, a.V, a.scale, a.H, a.NC = Bt * NC, K, V, float(scale), H, NC
@@ -331,26 +339,22 @@ def chunk_local_grads_final(prep, y_mirror, v_new, states, dstates, scale, l2nor
 RECORD_BYTES = 13312  # chunk record of the 32x32x16 kernels (K <= 128)
 
 
-def chunk_bwd_prepare(q, k, v, dout, g, beta, scale, l2norm):
+def chunk_bwd_prepare(q, k, dout, g, beta, scale, l2norm, V):
     """``gdn_chunk_bwd_prepare`` for a batch of whole chunks (``[N, T, H, 128]`` bf16, T a multiple of 64).
-    Returns a dict: the packed fp32 operands of ``chunk_local_grads`` (``qs, kn, v, dout`` ``[N H, T/64, 64, D]``;
-    ``gamma, beta, rq, rk`` ``[N H, T/64, 64]``) and the mirror problem ``k_mirror, v_mirror``
-    ``[N, 2 T, H, D]`` bf16, ``records`` uint8 ``[H, N * 2 T/64, RECORD_BYTES]``."""
+    Returns a dict: ``gamma, beta, rq, rk`` (fp32 ``[N H, T/64, 64]``: prefix sums of g inside the chunks, beta,
+    inverse norms of the rows of q and k) and the mirror problem ``k_mirror, v_mirror`` ``[N, 2 T, H, D]`` bf16,
+    ``records`` uint8 ``[H, N * 2 T/64, RECORD_BYTES]``."""
     _require_hip_path()
     lib = _lib.load_library()
     N, T, H, K = q.shape
-    V = v.size(-1)
     if (K, V) != CHUNK_LOCAL_KV or T % 64 != 0 or q.dtype != torch.bfloat16:
         raise ValueError(f"built for bf16, K, V = {CHUNK_LOCAL_KV} and T a multiple of 64")
-    q, k, v, dout = (_last_dim_contiguous(x) for x in (q, k, v, dout.to(torch.bfloat16)))
     g = None if g is None else g.to(torch.float32).contiguous()
     if beta is not None:
         beta = beta.contiguous() if beta.dtype in (torch.bfloat16, torch.float32) else beta.float().contiguous()
     dev, NC, Bt = q.device, T // 64, N * H
     f32 = dict(dtype=torch.float32, device=dev)
     out = dict(
-        qs=torch.empty(Bt, NC, 64, K, **f32), kn=torch.empty(Bt, NC, 64, K, **f32),
-        v=torch.empty(Bt, NC, 64, V, **f32), dout=torch.empty(Bt, NC, 64, V, **f32),
         gamma=torch.empty(Bt, NC, 64, **f32), beta=torch.empty(Bt, NC, 64, **f32),
         rq=torch.empty(Bt, NC, 64, **f32), rk=torch.empty(Bt, NC, 64, **f32),
         k_mirror=torch.empty(N, 2 * T, H, K, dtype=torch.bfloat16, device=dev),
@@ -358,10 +362,10 @@ def chunk_bwd_prepare(q, k, v, dout, g, beta, scale, l2norm):
         records=torch.empty(H, N * 2 * NC, RECORD_BYTES, dtype=torch.uint8, device=dev),
     )  # fmt: skip
     a = _lib.GdnChunkBwdPrepareArgs()
-    a.q, a.k, a.v, a.dout = q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr()
+    a.q, a.k, a.dout = q.data_ptr(), k.data_ptr(), dout.data_ptr()
     a.g = None if g is None else g.data_ptr()
     a.beta = None if beta is None else beta.data_ptr()
-    for name, x in (("q", q), ("k", k), ("v", v), ("dout", dout)):
+    for name, x in (("q", q), ("k", k), ("dout", dout)):
         setattr(a, f"{name}_stride_b", x.stride(0))
         setattr(a, f"{name}_stride_t", x.stride(1))
         setattr(a, f"{name}_stride_h", x.stride(2))
@@ -369,7 +373,6 @@ def chunk_bwd_prepare(q, k, v, dout, g, beta, scale, l2norm):
     a.beta_dtype = _lib.GDN_F32 if beta is None else _dtype_code(beta.dtype, "beta")
     a.flags = _lib.GDN_FLAG_L2NORM if l2norm else 0
     a.scale = float(scale)
-    a.qs, a.kn, a.v_packed, a.dout_packed = (out[n].data_ptr() for n in ("qs", "kn", "v", "dout"))
     a.gamma, a.beta_packed, a.rq, a.rk = (out[n].data_ptr() for n in ("gamma", "beta", "rq", "rk"))
     a.k_mirror, a.v_mirror, a.records = (out[n].data_ptr() for n in ("k_mirror", "v_mirror", "records"))
     a.records_bytes = out["records"].numel()
