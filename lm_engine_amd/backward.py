@@ -332,7 +332,7 @@ def gated_delta_rule_backward(
     V = v.size(-1)
     dev = q.device
     scale = K**-0.5 if scale is None else scale
-    if (q.is_cuda and q.dtype == torch.bfloat16 and (K, V) == _chunk_local_kv() and cu_seqlens is None
+    if (q.is_cuda and q.dtype == torch.bfloat16 and (K, V) in _chunk_local_kv() and cu_seqlens is None
             and T % CHUNK == 0):  # fmt: skip
         return _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, use_qk_l2norm_in_kernel)
     pk = _Packing(B, T, H, cu_seqlens, left_padded, dev)
@@ -388,7 +388,7 @@ def gated_delta_rule_backward(
         )  # fmt: skip
     dh0 = dS.reshape(N, H, K, V) if initial_state is not None else None
 
-    if on_kernel and (K, V) == _chunk_local_kv():
+    if on_kernel and (K, V) in _chunk_local_kv():
         from . import ops
 
         norms = dict(rq=rq[..., 0], rk=rk[..., 0]) if use_qk_l2norm_in_kernel else {}

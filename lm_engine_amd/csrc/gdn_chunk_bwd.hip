@@ -21,7 +21,8 @@
 // Every matrix product is an "A B^T" of two row-major bf16 matrices staged in LDS (the transposes of Q and K
 // are staged next to them), on 32x32x16 MFMA with fp32 accumulation.  The 64 x K results are kept transposed
 // ([key dim][token]) so that a lane owns one token: the per-token scales are per-lane scalars and the sums
-// over the key dim stay inside a lane.  Built for K = V = 128 (157 KiB of LDS: one workgroup per CU).
+// over the key dim stay inside a lane.  Built for K = 128 and V = 128 or 256 (the value dim is staged 128 columns
+// at a time; 157 KiB of LDS: one workgroup per CU).
 #include <hip/hip_runtime.h>
 
 #include "gdn_chunk_common.h"
@@ -31,7 +32,7 @@ namespace gdn {
 
 namespace {
 
-constexpr int BWD_K = 128, BWD_V = 128;
+constexpr int BWD_K = 128;  // the kernels of this file are built for K = 128 and V = 128 or 256
 constexpr int BWD_THREADS = 256;
 constexpr int LDR = 136;  // bf16 per LDS row of a [.][128] matrix: 16 bytes of padding
 constexpr int LDS64 = 72;  // bf16 per LDS row of a [.][64] matrix
@@ -92,8 +93,9 @@ __device__ __forceinline__ float half_sum(float x) {
     return x;
 }
 
+template <int V>
 __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const ChunkLocalParams p) {
-    constexpr int K = BWD_K, V = BWD_V;
+    constexpr int K = BWD_K, VW = 128;  // VW: columns of the value dim staged at a time
     __shared__ __attribute__((aligned(16))) bf16_t sQ[C * LDR];
     __shared__ __attribute__((aligned(16))) bf16_t sK[C * LDR];
     __shared__ __attribute__((aligned(16))) bf16_t sQT[K * LDS64];
@@ -145,49 +147,8 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
         r.x = (bf16_t)x.x, r.y = (bf16_t)x.y, r.z = (bf16_t)x.z, r.w = (bf16_t)x.w;
         *reinterpret_cast<bf16x4*>(dst) = r;
     };
-    float yv[8];  // <Y_i, V_i> pieces, reduced after the barrier (s_dbeta is being cleared above)
-#pragma unroll
-    for (int i = 0; i < 8; i++) yv[i] = 0.f;
-    if (final_mode) {
-        // rows of the caller's q, k, v, dO and of Y (token `row` is token 63 - row of mirror chunk A) as 16-byte
-        // pieces, 16 lanes per row; V~ below
-        const int p8 = t % 16;
-        const int64_t tl = (int64_t)ci * C;  // first token of the chunk inside its sequence
-#pragma unroll
-        for (int it = 0; it < 4; it++) {
-            const int row = t / 16 + 16 * it;
-            const bf16x8 qr = *reinterpret_cast<const bf16x8*>(p.q_raw + n * p.q_stride_b + (tl + row) * p.q_stride_t + (int64_t)h * p.q_stride_h + 8 * p8);
-            const bf16x8 kr = *reinterpret_cast<const bf16x8*>(p.k_raw + n * p.k_stride_b + (tl + row) * p.k_stride_t + (int64_t)h * p.k_stride_h + 8 * p8);
-            const bf16x8 vr = *reinterpret_cast<const bf16x8*>(p.v_raw + n * p.v_stride_b + (tl + row) * p.v_stride_t + (int64_t)h * p.v_stride_h + 8 * p8);
-            const bf16x8 dr = *reinterpret_cast<const bf16x8*>(p.d_raw + n * p.d_stride_b + (tl + row) * p.d_stride_t + (int64_t)h * p.d_stride_h + 8 * p8);
-            const bf16x8 yr = *reinterpret_cast<const bf16x8*>(p.y_mirror + ((mirA + (C - 1 - row)) * p.H + h) * V + 8 * p8);
-            const float fq = (p.rq != nullptr ? p.rq[chunk * C + row] : 1.f) * p.scale;
-            const float fk = p.rk != nullptr ? p.rk[chunk * C + row] : 1.f;
-            const float b = p.beta[chunk * C + row];
-            bf16x8 qb, kb, dv;
-            float acc = 0.f;
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                qb[e] = (bf16_t)((float)qr[e] * fq);
-                kb[e] = (bf16_t)((float)kr[e] * fk);
-                dv[e] = (bf16_t)((float)yr[e] * b);
-                acc += (float)yr[e] * (float)vr[e];
-                sQT[(8 * p8 + e) * LDS64 + row] = qb[e];
-                sKT[(8 * p8 + e) * LDS64 + row] = kb[e];
-            }
-            *reinterpret_cast<bf16x8*>(sQ + row * LDR + 8 * p8) = qb;
-            *reinterpret_cast<bf16x8*>(sK + row * LDR + 8 * p8) = kb;
-            *reinterpret_cast<bf16x8*>(sDO + row * LDR + 8 * p8) = dr;
-            *reinterpret_cast<bf16x8*>(sY + row * LDR + 8 * p8) = yr;
-            *reinterpret_cast<bf16x8*>(p.dv_out + ((tok0 + row) * p.H + h) * V + 8 * p8) = dv;  // dV = beta Y
-            yv[it] = acc;
-        }
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const int idx = t + BWD_THREADS * i, row = idx / 32, c4 = idx % 32;
-            put4(sVN + row * LDR + 4 * c4, *reinterpret_cast<const f32x4*>(vnew + row * V + 4 * c4));
-        }
-    } else {
+    // ---- q, k and their transposes (final mode: with the first half of v, dO, Y below, one batch of loads) ----
+    if (!final_mode) {
 #pragma unroll
         for (int i = 0; i < 8; i++) {  // [64][128] fp32: 2048 groups of 4, row = 8 i + t / 32
             const int idx = t + BWD_THREADS * i, row = idx / 32, c4 = idx % 32;
@@ -200,35 +161,6 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
                 sQT[(4 * c4 + e) * LDS64 + row] = (bf16_t)a[e];
                 sKT[(4 * c4 + e) * LDS64 + row] = (bf16_t)b[e];
             }
-            const f32x4 d = *reinterpret_cast<const f32x4*>(dout + row * V + 4 * c4);
-            const f32x4 n4 = *reinterpret_cast<const f32x4*>(vnew + row * V + 4 * c4);
-            const f32x4 y = *reinterpret_cast<const f32x4*>(yy + row * V + 4 * c4);
-            const f32x4 x = *reinterpret_cast<const f32x4*>(vv + row * V + 4 * c4);
-            put4(sDO + row * LDR + 4 * c4, d);
-            put4(sVN + row * LDR + 4 * c4, n4);
-            put4(sY + row * LDR + 4 * c4, y);
-            yv[i] = y.x * x.x + y.y * x.y + y.z * x.z + y.w * x.w;
-        }
-    }
-#pragma unroll
-    for (int i = 0; i < 16; i++) {  // S0 [128][128] fp32: row = 8 i + t / 32
-        const int idx = t + BWD_THREADS * i, row = idx / 32, c4 = idx % 32;
-        put4(sST + row * LDR + 4 * c4, *reinterpret_cast<const f32x4*>(s0 + row * V + 4 * c4));
-    }
-    __syncthreads();
-    if (final_mode) {
-#pragma unroll
-        for (int it = 0; it < 4; it++) {  // 16 lanes hold one row
-            float x = yv[it];
-#pragma unroll
-            for (int off = 8; off >= 1; off >>= 1) x += __shfl_xor(x, off, WAVE);
-            if (t % 16 == 0) atomicAdd(&s_dbeta[t / 16 + 16 * it], x);
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < 8; i++) {  // the 32 lanes of a wave half hold one row
-            const float x = half_sum(yv[i]);
-            if (l32 == 0) atomicAdd(&s_dbeta[8 * i + t / 32], x);
         }
     }
 
@@ -236,41 +168,136 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
 #pragma unroll
     for (int r = 0; r < 16; r++) zero[r] = 0.f;
 
-    // ---- products with S0, transposed: rows = key dims 32 wave .., columns = tokens 32 tt + l32 ----
-    f32x16 dQeT[2], ZT[2], dKdT[2];
+    // Everything that contracts over the value dim runs over V in halves of 128 columns (VW), accumulating:
+    // the products with the states, transposed (rows = key dims 32 wave .., columns = tokens 32 tt + l32), and
+    // the 64 x 64 products dO V~^T and Y V~^T (wave -> tile (wave / 2, wave % 2)).
+    f32x16 dQeT[2] = {zero, zero}, ZT[2] = {zero, zero}, dKdT[2] = {zero, zero}, DP = zero, DA = zero;
 #pragma unroll
-    for (int tt = 0; tt < 2; tt++) {
-        dQeT[tt] = mma_nt(sST + 32 * wave * LDR, LDR, sDO + 32 * tt * LDR, LDR, V, zero, l32, lh);
-        ZT[tt] = mma_nt(sST + 32 * wave * LDR, LDR, sY + 32 * tt * LDR, LDR, V, zero, l32, lh);
-    }
-    __syncthreads();  // S0 has been read by every wave
-
-    // ---- dS1 takes the place of S0; <dS1, S0> on the way ----
-    {
-        float dot = 0.f;
+    for (int hv = 0; hv < V / VW; hv++) {
+        const int v0 = VW * hv;
+        float yv[8];  // <Y_i, V_i> pieces, reduced after the barrier (s_dbeta is cleared before the first one)
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int idx = t + BWD_THREADS * i, row = idx / 32, c4 = idx % 32;
-            const f32x4 x = *reinterpret_cast<const f32x4*>(ds1 + row * V + 4 * c4);
-            const bf16x4 s = *reinterpret_cast<const bf16x4*>(sST + row * LDR + 4 * c4);
-            dot += x.x * (float)s.x + x.y * (float)s.y + x.z * (float)s.z + x.w * (float)s.w;
-            put4(sST + row * LDR + 4 * c4, x);
+        for (int i = 0; i < 8; i++) yv[i] = 0.f;
+        if (final_mode) {
+            // v, dO and Y (token `row` is token 63 - row of mirror chunk A); dV = beta Y goes out right away
+            const int p8 = t % 16;
+            const int64_t tl = (int64_t)ci * C;
+#pragma unroll
+            for (int it = 0; it < 4; it++) {
+                const int row = t / 16 + 16 * it;
+                if (hv == 0) {
+                    const bf16x8 qr = *reinterpret_cast<const bf16x8*>(p.q_raw + n * p.q_stride_b + (tl + row) * p.q_stride_t + (int64_t)h * p.q_stride_h + 8 * p8);
+                    const bf16x8 kr = *reinterpret_cast<const bf16x8*>(p.k_raw + n * p.k_stride_b + (tl + row) * p.k_stride_t + (int64_t)h * p.k_stride_h + 8 * p8);
+                    const float fq = (p.rq != nullptr ? p.rq[chunk * C + row] : 1.f) * p.scale;
+                    const float fk = p.rk != nullptr ? p.rk[chunk * C + row] : 1.f;
+                    bf16x8 qb, kb;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        qb[e] = (bf16_t)((float)qr[e] * fq);
+                        kb[e] = (bf16_t)((float)kr[e] * fk);
+                        sQT[(8 * p8 + e) * LDS64 + row] = qb[e];
+                        sKT[(8 * p8 + e) * LDS64 + row] = kb[e];
+                    }
+                    *reinterpret_cast<bf16x8*>(sQ + row * LDR + 8 * p8) = qb;
+                    *reinterpret_cast<bf16x8*>(sK + row * LDR + 8 * p8) = kb;
+                }
+                const bf16x8 vr = *reinterpret_cast<const bf16x8*>(p.v_raw + n * p.v_stride_b + (tl + row) * p.v_stride_t + (int64_t)h * p.v_stride_h + v0 + 8 * p8);
+                const bf16x8 dr = *reinterpret_cast<const bf16x8*>(p.d_raw + n * p.d_stride_b + (tl + row) * p.d_stride_t + (int64_t)h * p.d_stride_h + v0 + 8 * p8);
+                const bf16x8 yr = *reinterpret_cast<const bf16x8*>(p.y_mirror + ((mirA + (C - 1 - row)) * p.H + h) * V + v0 + 8 * p8);
+                const float b = p.beta[chunk * C + row];
+                bf16x8 dv;
+                float acc = 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    dv[e] = (bf16_t)((float)yr[e] * b);
+                    acc += (float)yr[e] * (float)vr[e];
+                }
+                *reinterpret_cast<bf16x8*>(sDO + row * LDR + 8 * p8) = dr;
+                *reinterpret_cast<bf16x8*>(sY + row * LDR + 8 * p8) = yr;
+                *reinterpret_cast<bf16x8*>(p.dv_out + ((tok0 + row) * p.H + h) * V + v0 + 8 * p8) = dv;
+                yv[it] = acc;
+            }
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int idx = t + BWD_THREADS * i, row = idx / 32, c4 = idx % 32;
+                put4(sVN + row * LDR + 4 * c4, *reinterpret_cast<const f32x4*>(vnew + row * V + v0 + 4 * c4));
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int idx = t + BWD_THREADS * i, row = idx / 32, c4 = idx % 32;
+                const f32x4 d = *reinterpret_cast<const f32x4*>(dout + row * V + v0 + 4 * c4);
+                const f32x4 n4 = *reinterpret_cast<const f32x4*>(vnew + row * V + v0 + 4 * c4);
+                const f32x4 y = *reinterpret_cast<const f32x4*>(yy + row * V + v0 + 4 * c4);
+                const f32x4 x = *reinterpret_cast<const f32x4*>(vv + row * V + v0 + 4 * c4);
+                put4(sDO + row * LDR + 4 * c4, d);
+                put4(sVN + row * LDR + 4 * c4, n4);
+                put4(sY + row * LDR + 4 * c4, y);
+                yv[i] = y.x * x.x + y.y * x.y + y.z * x.z + y.w * x.w;
+            }
         }
-        dot = wave_sum(dot);
-        if (lane == 0) atomicAdd(&s_red[0], dot);
-    }
-    __syncthreads();
 #pragma unroll
-    for (int tt = 0; tt < 2; tt++) dKdT[tt] = mma_nt(sST + 32 * wave * LDR, LDR, sVN + 32 * tt * LDR, LDR, V, zero, l32, lh);
-    __syncthreads();  // the state's region is free
+        for (int i = 0; i < 16; i++) {  // S0[:, v0 .. v0 + 127] fp32: row = 8 i + t / 32
+            const int idx = t + BWD_THREADS * i, row = idx / 32, c4 = idx % 32;
+            put4(sST + row * LDR + 4 * c4, *reinterpret_cast<const f32x4*>(s0 + row * V + v0 + 4 * c4));
+        }
+        __syncthreads();
+        if (final_mode) {
+#pragma unroll
+            for (int it = 0; it < 4; it++) {  // 16 lanes hold one row
+                float x = yv[it];
+#pragma unroll
+                for (int off = 8; off >= 1; off >>= 1) x += __shfl_xor(x, off, WAVE);
+                if (t % 16 == 0) atomicAdd(&s_dbeta[t / 16 + 16 * it], x);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {  // the 32 lanes of a wave half hold one row
+                const float x = half_sum(yv[i]);
+                if (l32 == 0) atomicAdd(&s_dbeta[8 * i + t / 32], x);
+            }
+        }
+
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++) {
+            dQeT[tt] = mma_nt(sST + 32 * wave * LDR, LDR, sDO + 32 * tt * LDR, LDR, VW, dQeT[tt], l32, lh);
+            ZT[tt] = mma_nt(sST + 32 * wave * LDR, LDR, sY + 32 * tt * LDR, LDR, VW, ZT[tt], l32, lh);
+        }
+        if constexpr (V > VW) {  // with a single half they wait until the 64 x 64 stage below (dO, V~, Y stay staged)
+            DP = mma_nt(sDO + 32 * (wave / 2) * LDR, LDR, sVN + 32 * (wave % 2) * LDR, LDR, VW, DP, l32, lh);
+            DA = mma_nt(sY + 32 * (wave / 2) * LDR, LDR, sVN + 32 * (wave % 2) * LDR, LDR, VW, DA, l32, lh);
+        }
+        __syncthreads();  // S0 has been read by every wave
+
+        // dS1 takes the place of S0; <dS1, S0> on the way
+        {
+            float dot = 0.f;
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int idx = t + BWD_THREADS * i, row = idx / 32, c4 = idx % 32;
+                const f32x4 x = *reinterpret_cast<const f32x4*>(ds1 + row * V + v0 + 4 * c4);
+                const bf16x4 sv = *reinterpret_cast<const bf16x4*>(sST + row * LDR + 4 * c4);
+                dot += x.x * (float)sv.x + x.y * (float)sv.y + x.z * (float)sv.z + x.w * (float)sv.w;
+                put4(sST + row * LDR + 4 * c4, x);
+            }
+            dot = wave_sum(dot);
+            if (lane == 0) atomicAdd(&s_red[0], dot);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++) dKdT[tt] = mma_nt(sST + 32 * wave * LDR, LDR, sVN + 32 * tt * LDR, LDR, VW, dKdT[tt], l32, lh);
+        __syncthreads();  // the staged half is free
+    }
 
     // ---- the 64 x 64 products: wave -> tile (ti, tj); rows i = 32 ti + 8 (r/4) + 4 h + r%4, column j = 32 tj + l32 ----
     {
         const int ti = wave / 2, tj = wave % 2;
         const f32x16 QK = mma_nt(sQ + 32 * ti * LDR, LDR, sK + 32 * tj * LDR, LDR, K, zero, l32, lh);
         const f32x16 KK = mma_nt(sK + 32 * ti * LDR, LDR, sK + 32 * tj * LDR, LDR, K, zero, l32, lh);
-        const f32x16 DP = mma_nt(sDO + 32 * ti * LDR, LDR, sVN + 32 * tj * LDR, LDR, V, zero, l32, lh);
-        const f32x16 DA = mma_nt(sY + 32 * ti * LDR, LDR, sVN + 32 * tj * LDR, LDR, V, zero, l32, lh);
+        if constexpr (V == VW) {
+            DP = mma_nt(sDO + 32 * ti * LDR, LDR, sVN + 32 * tj * LDR, LDR, VW, zero, l32, lh);
+            DA = mma_nt(sY + 32 * ti * LDR, LDR, sVN + 32 * tj * LDR, LDR, VW, zero, l32, lh);
+        }
         const int j = 32 * tj + l32;
         const float gj = s_gam[j];
         float colsum = 0.f;
@@ -436,8 +463,9 @@ struct BwdPrepareParams {
     uint32_t rec_bytes, off_p, off_qs, off_ks, off_cs, off_eg;
 };
 
+template <int V>
 __global__ __launch_bounds__(BWD_THREADS) void chunk_bwd_prepare_kernel(const BwdPrepareParams p) {
-    constexpr int K = BWD_K, V = BWD_V;
+    constexpr int K = BWD_K;
     __shared__ __attribute__((aligned(16))) bf16_t sQ[C * LDR];
     __shared__ __attribute__((aligned(16))) bf16_t sK[C * LDR];
     __shared__ __attribute__((aligned(16))) bf16_t sDOT[V * LDS64];  // dO^T
@@ -480,7 +508,6 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_bwd_prepare_kernel(const Bw
         const int64_t tok = tok0 + row;
         const bf16x8 qr = *reinterpret_cast<const bf16x8*>(p.q + n * p.q_stride_b + tok * p.q_stride_t + (int64_t)h * p.q_stride_h + 8 * p8);
         const bf16x8 kr = *reinterpret_cast<const bf16x8*>(p.k + n * p.k_stride_b + tok * p.k_stride_t + (int64_t)h * p.k_stride_h + 8 * p8);
-        const bf16x8 dr = *reinterpret_cast<const bf16x8*>(p.dout + n * p.d_stride_b + tok * p.d_stride_t + (int64_t)h * p.d_stride_h + 8 * p8);
         float ssq = 0.f, ssk = 0.f;
 #pragma unroll
         for (int e = 0; e < 8; e++) ssq += (float)qr[e] * (float)qr[e], ssk += (float)kr[e] * (float)kr[e];
@@ -499,14 +526,17 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_bwd_prepare_kernel(const Bw
         }
         *reinterpret_cast<bf16x8*>(sQ + row * LDR + 8 * p8) = qb;
         *reinterpret_cast<bf16x8*>(sK + row * LDR + 8 * p8) = kb;
-#pragma unroll
-        for (int e = 0; e < 8; e++) sDOT[(8 * p8 + e) * LDS64 + row] = dr[e];
         // mirror rows: token `row` of this chunk is token 63 - row of chunks A and B
-        const int64_t rowA = (((int64_t)n * TM + mir0 + (C - 1 - row)) * p.H + h) * K + 8 * p8;
-        const int64_t rowB = rowA + (int64_t)C * p.H * K;
-        *reinterpret_cast<bf16x8*>(p.k_m + rowA) = kr;
-        *reinterpret_cast<bf16x8*>(p.k_m + rowB) = qr;
-        *reinterpret_cast<bf16x8*>(p.v_m + rowB) = dr;
+        const int64_t tokA = ((int64_t)n * TM + mir0 + (C - 1 - row)) * p.H + h, tokB = tokA + (int64_t)C * p.H;
+        *reinterpret_cast<bf16x8*>(p.k_m + tokA * K + 8 * p8) = kr;
+        *reinterpret_cast<bf16x8*>(p.k_m + tokB * K + 8 * p8) = qr;
+#pragma unroll
+        for (int hv = 0; hv < V / 128; hv++) {
+            const bf16x8 dr = *reinterpret_cast<const bf16x8*>(p.dout + n * p.d_stride_b + tok * p.d_stride_t + (int64_t)h * p.d_stride_h + 128 * hv + 8 * p8);
+#pragma unroll
+            for (int e = 0; e < 8; e++) sDOT[(128 * hv + 8 * p8 + e) * LDS64 + row] = dr[e];
+            *reinterpret_cast<bf16x8*>(p.v_m + tokB * V + 128 * hv + 8 * p8) = dr;
+        }
     }
     __syncthreads();
 
@@ -531,16 +561,18 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_bwd_prepare_kernel(const Bw
     }
     __syncthreads();
 
-    // ---- P^T dO -> rows of v_m for chunk A: rows j = 32 tj + .., columns v = 32 wave + l32 ----
+    // ---- P^T dO -> rows of v_m for chunk A: rows j = 32 tj + .., columns v = 32 tv + l32, tv = wave, wave + 4, .. ----
 #pragma unroll
-    for (int tj = 0; tj < 2; tj++) {
-        const f32x16 u = mma_nt(sPT + 32 * tj * LDS64, LDS64, sDOT + 32 * wave * LDS64, LDS64, C, zero, l32, lh);
+    for (int tv = wave; tv < V / 32; tv += BWD_THREADS / WAVE)
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int j = 32 * tj + 8 * (r / 4) + 4 * lh + r % 4;
-            p.v_m[(((int64_t)n * TM + mir0 + (C - 1 - j)) * p.H + h) * V + 32 * wave + l32] = (bf16_t)u[r];
+        for (int tj = 0; tj < 2; tj++) {
+            const f32x16 u = mma_nt(sPT + 32 * tj * LDS64, LDS64, sDOT + 32 * tv * LDS64, LDS64, C, zero, l32, lh);
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int j = 32 * tj + 8 * (r / 4) + 4 * lh + r % 4;
+                p.v_m[(((int64_t)n * TM + mir0 + (C - 1 - j)) * p.H + h) * V + 32 * tv + l32] = (bf16_t)u[r];
+            }
         }
-    }
 
     // ---- T = (I + A)^-1 in place of A: lane = column, row i needs rows 0 .. i - 1 ----
     if (wave == 0) {
@@ -616,14 +648,15 @@ int launch_chunk_bwd_local(const gdn_chunk_local_args& a, hipStream_t stream) {
     p.k_stride_b = a.k_stride_b, p.k_stride_t = a.k_stride_t, p.k_stride_h = a.k_stride_h;
     p.v_stride_b = a.v_stride_b, p.v_stride_t = a.v_stride_t, p.v_stride_h = a.v_stride_h;
     p.d_stride_b = a.dout_stride_b, p.d_stride_t = a.dout_stride_t, p.d_stride_h = a.dout_stride_h;
-    hipLaunchKernelGGL(chunk_local_grads_kernel, dim3((unsigned)a.chunks), dim3(BWD_THREADS), 0, stream, p);
+    if (a.V == 256) hipLaunchKernelGGL(chunk_local_grads_kernel<256>, dim3((unsigned)a.chunks), dim3(BWD_THREADS), 0, stream, p);
+    else hipLaunchKernelGGL(chunk_local_grads_kernel<128>, dim3((unsigned)a.chunks), dim3(BWD_THREADS), 0, stream, p);
     return (int)hipGetLastError();
 }
 
-bool chunk_bwd_local_supported(const gdn_chunk_local_args& a) { return a.K == BWD_K && a.V == BWD_V; }
+bool chunk_bwd_local_supported(const gdn_chunk_local_args& a) { return a.K == BWD_K && (a.V == 128 || a.V == 256); }
 
 bool chunk_bwd_prepare_supported(const gdn_chunk_bwd_prepare_args& a) {
-    return a.K == BWD_K && a.V == BWD_V && a.T > 0 && a.T % C == 0;
+    return a.K == BWD_K && (a.V == 128 || a.V == 256) && a.T > 0 && a.T % C == 0;
 }
 
 uint64_t chunk_bwd_record_bytes(const gdn_chunk_bwd_prepare_args& a) {
@@ -648,7 +681,8 @@ int launch_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args& a, hipStream_t st
     p.rec = static_cast<uint8_t*>(a.records);
     p.rec_bytes = r.bytes, p.off_p = r.off_p, p.off_qs = r.off_qs, p.off_ks = r.off_ks, p.off_cs = r.off_cs, p.off_eg = r.off_eg;
     const int64_t chunks = (int64_t)a.N * a.H * p.NC;
-    hipLaunchKernelGGL(chunk_bwd_prepare_kernel, dim3((unsigned)chunks), dim3(BWD_THREADS), 0, stream, p);
+    if (a.V == 256) hipLaunchKernelGGL(chunk_bwd_prepare_kernel<256>, dim3((unsigned)chunks), dim3(BWD_THREADS), 0, stream, p);
+    else hipLaunchKernelGGL(chunk_bwd_prepare_kernel<128>, dim3((unsigned)chunks), dim3(BWD_THREADS), 0, stream, p);
     return (int)hipGetLastError();
 }
 

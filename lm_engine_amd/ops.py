@@ -254,7 +254,7 @@ def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_ch
     return o, ht
 
 
-CHUNK_LOCAL_KV = (128, 128)  # head dims gdn_chunk_bwd_local is built for
+CHUNK_LOCAL_KV = ((128, 128), (128, 256))  # head dims gdn_chunk_bwd_local and gdn_chunk_bwd_prepare are built for
 
 
 def chunk_local_grads(qs, kn, v, dout, y, v_new, states, dstates, gamma, beta, scale, rq=None, rk=None):
@@ -277,7 +277,7 @@ def chunk_local_grads(qs, kn, v, dout, y, v_new, states, dstates, gamma, beta, s
         if tuple(x.shape) != shapes[name] or x.dtype != torch.float32 or not x.is_cuda:
             raise ValueError(f"{name} must be a device fp32 tensor of shape {shapes[name]}, got {tuple(x.shape)} {x.dtype}")
         tensors[name] = x.contiguous()
-    if C != 64 or (K, V) != CHUNK_LOCAL_KV:
+    if C != 64 or (K, V) not in CHUNK_LOCAL_KV:
         raise ValueError(f"chunk-local gradients are built for chunk 64 and K, V = {CHUNK_LOCAL_KV}")
     out = dict(dq=torch.empty_like(tensors["qs"]), dk=torch.empty_like(tensors["kn"]),
                dbeta=torch.empty_like(tensors["gamma"]), dgamma=torch.empty_like(tensors["gamma"]))  # fmt: skip
@@ -347,7 +347,7 @@ def chunk_bwd_prepare(q, k, dout, g, beta, scale, l2norm, V):
     _require_hip_path()
     lib = _lib.load_library()
     N, T, H, K = q.shape
-    if (K, V) != CHUNK_LOCAL_KV or T % 64 != 0 or q.dtype != torch.bfloat16:
+    if (K, V) not in CHUNK_LOCAL_KV or T % 64 != 0 or q.dtype != torch.bfloat16:
         raise ValueError(f"built for bf16, K, V = {CHUNK_LOCAL_KV} and T a multiple of 64")
     g = None if g is None else g.to(torch.float32).contiguous()
     if beta is not None:

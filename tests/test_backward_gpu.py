@@ -76,6 +76,13 @@ def test_chunk_bf16_k64_and_wide_v():
     _run_case(lm_engine_amd.chunk_gated_delta_rule, inp, torch.bfloat16)
 
 
+@pytest.mark.parametrize("V", [128, 256])
+def test_chunk_bf16_whole_chunks_all_on_kernels(V):
+    # whole chunks, K = 128: prepare, both sweeps and the chunk-local gradients are kernel launches
+    inp = random_inputs(B=2, T=192, H=3, K=128, V=V, dtype=torch.bfloat16, seed=30 + V, normalize=False)
+    _run_case(lm_engine_amd.chunk_gated_delta_rule, inp, torch.bfloat16)
+
+
 def test_chunk_bf16_many_chains():
     # more than 128 chains at V = 128: the saving scan runs with four column slices per workgroup
     inp = random_inputs(B=9, T=128, H=16, K=128, V=128, dtype=torch.bfloat16, seed=10, normalize=False)
@@ -142,13 +149,14 @@ def test_saved_chunk_states_are_the_states_of_the_prefixes():
         assert_parity(states[:, :, c], want, torch.bfloat16, f"state at the start of chunk {c}")
 
 
-def test_chunk_local_kernel_matches_the_batched_gemm_version():
+@pytest.mark.parametrize("V", [128, 256])
+def test_chunk_local_kernel_matches_the_batched_gemm_version(V):
     """``gdn_chunk_bwd_local`` against the same stage written with torch operations, on random packed inputs."""
     from lm_engine_amd import ops
     from lm_engine_amd.backward import _chunk_local_grads
 
     gen = torch.Generator().manual_seed(21)
-    Bt, NC, C, K, V = 3, 5, 64, 128, 128
+    Bt, NC, C, K = 3, 5, 64, 128
     rnd = lambda *shape: torch.randn(*shape, generator=gen)  # noqa: E731
     qs = torch.nn.functional.normalize(rnd(Bt, NC, C, K), dim=-1) * K**-0.5
     kn = torch.nn.functional.normalize(rnd(Bt, NC, C, K), dim=-1)
