@@ -4,11 +4,16 @@ The reference trains through ``chunk_gated_delta_rule`` (chunk mode is asserted 
 lm_engine/modeling_utils/sequence_mixer_blocks/gated_deltanet/module.py:194-209), so autograd needs
 the gradients of ``(o, final_state)`` with respect to ``(q, k, v, g, beta, initial_state)``.
 
-The chunk-local products are batched library GEMMs (fp32, ``torch.bmm`` on the tensors' device).  The
-two sweeps over the chunks of a chain - forward to rebuild the state every chunk starts from, backward
-to carry the state gradient - run on the HIP scan kernel for bf16 inputs with K <= 128
-(``gdn_chunk_fwd_saving``: the forward's scan in a variant that also writes the chunk states and V~),
-and as loops of batched GEMMs otherwise.
+Three ways through, same formulas:
+
+* bf16, K = 128, V = 128 or 256, batches of whole chunks (no cu_seqlens, T a multiple of 64): five kernel
+  launches (``_backward_on_kernels``) - ``gdn_chunk_bwd_prepare``, ``gdn_chunk_fwd_saving`` for the forward
+  sweep and again over the mirror problem for the reverse sweep, ``gdn_chunk_bwd_local``;
+* other bf16 shapes with K <= 128, packed, ragged or left-padded batches: the two sweeps over the chunks of a
+  chain on the scan kernel (``gdn_chunk_fwd_saving``: the forward's scan in a variant that also writes the chunk
+  states and V~), everything chunk-local as batched library GEMMs (fp32, ``torch.bmm``) and elementwise torch
+  operations on sequences padded to whole chunks;
+* fp32 inputs, K = 256, CPU tensors: the sweeps as loops of batched GEMMs as well.
 
 The reverse sweep is the same recurrence as the forward one on other data, which is how it gets onto
 that kernel: with the tokens of a chain in reverse order (a transposed lower-triangular matrix is
@@ -18,8 +23,8 @@ lower-triangular again), chunk c becomes two chunks of a "mirror" problem,
         state: exp(gamma_C) dS1 - Kb^T Y
     B:  v := dO,      k := q,  T' := I,    row scale Qe's, no decay             =>  state += Qe^T dO
 
-whose records are written here (``_mirror_problem``) instead of by the prepare kernel; the states the
-scan saves at the A chunks are dS1, its output there is Y.
+whose rows and records ``gdn_chunk_bwd_prepare`` writes (``_mirror_problem`` on the second way); the states
+the scan saves at the A chunks are dS1, its output there is Y.
 
 Chunk-local quantities (C = 64 tokens, gamma = prefix sum of g inside the chunk, e = exp(gamma),
 E_ij = exp(gamma_i - gamma_j) for j <= i):
