@@ -185,12 +185,19 @@ typedef struct gdn_chunk_local_args {
     int64_t k_stride_b, k_stride_t, k_stride_h;
     int64_t v_stride_b, v_stride_t, v_stride_h;
     int64_t dout_stride_b, dout_stride_t, dout_stride_h;
+    /* final mode for packed or left-padded batches: sequence n starts at token seq_start[n] (a flat index over the
+     * rows of the caller's tensors, T_rows tokens per row) and has seq_len[n] tokens; its chunks c * 64 >= seq_len[n]
+     * are skipped, tokens past its end are not written.  NULL: sequence n is row n, NC * 64 tokens. */
+    const int32_t *seq_start, *seq_len;
+    int32_t T_rows;
+    int32_t reserved2;
 } gdn_chunk_local_args;
 int gdn_chunk_bwd_local(const gdn_chunk_local_args *args, void *stream);
 
 /*
- * Training support, third part: everything the backward needs per chunk before its two sweeps, for batches
- * of whole chunks (no cu_seqlens, T a multiple of 64; bf16 q, k, dout as [N, T, H, D] with element
+ * Training support, third part: everything the backward needs per chunk before its two sweeps (batches of
+ * whole chunks: T a multiple of 64, one sequence per row; other batches through seq_start / seq_len below;
+ * bf16 q, k, dout as [N, T, H, D] with element
  * strides; K = 128 and V = 128 or 256, GDN_ERR_UNSUPPORTED otherwise).  One workgroup per (sequence, head, chunk) writes
  *   - gamma, beta_packed, rq, rk: fp32 [N H T/64][64], operands of gdn_chunk_bwd_local;
  *   - the reverse sweep as a forward scan over 2 T tokens per sequence ("mirror" problem: tokens in reverse
@@ -215,6 +222,12 @@ typedef struct gdn_chunk_bwd_prepare_args {
     float *gamma, *beta_packed, *rq, *rk;
     void *k_mirror, *v_mirror, *records;
     uint64_t records_bytes;
+    /* packed or left-padded batches: as in gdn_chunk_local_args, with T the tokens per row of q, k, dout (N need not
+     * be their number of rows) and NC the chunks per sequence of the packed arrays and of the mirror problem
+     * (>= ceil(max seq_len / 64)); T / 64 is read as NC when seq_start is NULL */
+    const int32_t *seq_start, *seq_len;
+    int32_t NC;
+    int32_t reserved;
 } gdn_chunk_bwd_prepare_args;
 int gdn_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args *args, void *stream);
 

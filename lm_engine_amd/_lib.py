@@ -63,7 +63,9 @@ class GdnChunkLocalArgs(ctypes.Structure):
         "y_mirror", "dq_out", "dk_out", "dv_out", "dg_out", "dbeta_out",
     )] + [("H", ctypes.c_int32), ("NC", ctypes.c_int32)] + [(name, ctypes.c_void_p) for name in (
         "q_raw", "k_raw", "v_raw", "dout_raw",
-    )] + [(f"{x}_stride_{d}", ctypes.c_int64) for x in ("q", "k", "v", "dout") for d in ("b", "t", "h")]  # fmt: skip
+    )] + [(f"{x}_stride_{d}", ctypes.c_int64) for x in ("q", "k", "v", "dout") for d in ("b", "t", "h")] + [
+        ("seq_start", ctypes.c_void_p), ("seq_len", ctypes.c_void_p), ("T_rows", ctypes.c_int32), ("reserved2", ctypes.c_int32),
+    ]  # fmt: skip
 
 
 class GdnChunkBwdPrepareArgs(ctypes.Structure):
@@ -73,7 +75,8 @@ class GdnChunkBwdPrepareArgs(ctypes.Structure):
         + [(name, ctypes.c_int32) for name in ("N", "T", "H", "K", "V", "beta_dtype", "flags")]
         + [("scale", ctypes.c_float)]
         + [(name, ctypes.c_void_p) for name in ("gamma", "beta_packed", "rq", "rk", "k_mirror", "v_mirror", "records")]
-        + [("records_bytes", ctypes.c_uint64)]
+        + [("records_bytes", ctypes.c_uint64), ("seq_start", ctypes.c_void_p), ("seq_len", ctypes.c_void_p),
+           ("NC", ctypes.c_int32), ("reserved", ctypes.c_int32)]
     )  # fmt: skip
 
 

@@ -294,25 +294,34 @@ def _chunk_local_grads(qs, kn, vc, doc, Y, Vn, S0, dS1, gam, bc):
     return dqs, dkn, dbc, dgam
 
 
-def _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, l2norm):
-    """The whole backward on four kernel launches (bf16, K = V = 128, whole chunks, one sequence per row):
-    ``gdn_chunk_bwd_prepare`` (packed operands + mirror problem), the saving forward sweep, the scan over the
-    mirror problem, ``gdn_chunk_bwd_local`` writing the gradients in the caller's layout."""
+def _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, l2norm, cu_seqlens, left_padded):
+    """The whole backward on five kernel launches (bf16, K = 128, V = 128 or 256): ``gdn_chunk_bwd_prepare``
+    (mirror problem and per-chunk scalars), the saving forward sweep, the saving scan over the mirror problem,
+    ``gdn_chunk_bwd_local`` writing the gradients in the caller's layout.  Packed and left-padded batches are laid
+    out with the chunk count of their longest sequence."""
     from . import ops  # late: ops imports this module
 
-    N, T, H, K = q.shape
+    B, T, H, K = q.shape
     V = v.size(-1)
-    NC, Bt, dev = T // CHUNK, N * H, q.device
+    dev = q.device
+    if cu_seqlens is None and T % CHUNK == 0:
+        N, NC, sequences = B, T // CHUNK, None
+    else:
+        starts, lens = _chains(B, T, cu_seqlens, left_padded)
+        N, NC = len(lens), max(1, -(-max(lens + [1]) // CHUNK))
+        as_i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)  # noqa: E731
+        sequences = (as_i32(starts), as_i32(lens), NC)
+    Bt = N * H
     q, k, v, do = (x if x.stride(-1) == 1 else x.contiguous() for x in (q, k, v, do.to(torch.bfloat16)))
-    prep = ops.chunk_bwd_prepare(q, k, do, g, beta, scale, l2norm, V)
+    prep = ops.chunk_bwd_prepare(q, k, do, g, beta, scale, l2norm, V, sequences)
     S0 = torch.empty(Bt, NC, K, V, device=dev)
     Vn = torch.empty(Bt, NC, CHUNK, V, device=dev)
-    ops.chunk_forward_saving(q, k, v, g, beta, scale, initial_state, None, l2norm, False, S0, Vn, NC)
+    ops.chunk_forward_saving(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2norm, left_padded, S0, Vn, NC)
     dS1 = torch.empty(Bt, NC, K, V, device=dev)
     dht32 = None if dht is None else dht.to(torch.float32).contiguous()
     o_m, dS = ops.chunk_scan_given_records(prep["k_mirror"], prep["v_mirror"], prep["records"], dht32, dS1, NC,
                                            save_every=2, save_reverse=True)  # fmt: skip
-    dq, dk, dv, dg, dbeta = ops.chunk_local_grads_final(q, k, v, do, prep, o_m, Vn, S0, dS1, scale, l2norm)
+    dq, dk, dv, dg, dbeta = ops.chunk_local_grads_final(q, k, v, do, prep, o_m, Vn, S0, dS1, scale, l2norm, sequences)
     return (
         dq,
         dk,
@@ -337,9 +346,9 @@ def gated_delta_rule_backward(
     V = v.size(-1)
     dev = q.device
     scale = K**-0.5 if scale is None else scale
-    if (q.is_cuda and q.dtype == torch.bfloat16 and (K, V) in _chunk_local_kv() and cu_seqlens is None
-            and T % CHUNK == 0):  # fmt: skip
-        return _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, use_qk_l2norm_in_kernel)
+    if q.is_cuda and q.dtype == torch.bfloat16 and (K, V) in _chunk_local_kv():
+        return _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, use_qk_l2norm_in_kernel,
+                                    cu_seqlens, left_padded)  # fmt: skip
     pk = _Packing(B, T, H, cu_seqlens, left_padded, dev)
     N, NC, Bt = pk.N, pk.NC, pk.N * H
 

@@ -125,6 +125,7 @@ int gdn_chunk_bwd_local(const gdn_chunk_local_args* a, void* stream) {
             if (x == nullptr) return GDN_ERR_NULL;
             else if (!aligned(x, 16)) return GDN_ERR_ALIGN;
         if (a->H <= 0 || a->NC <= 0 || a->chunks % ((int64_t)a->H * a->NC) != 0) return GDN_ERR_SHAPE;
+        if (a->seq_start != nullptr && (a->seq_len == nullptr || a->T_rows <= 0)) return GDN_ERR_SHAPE;
         const int64_t raw_strides[] = {a->q_stride_b, a->q_stride_t, a->q_stride_h, a->k_stride_b, a->k_stride_t, a->k_stride_h,
                                        a->v_stride_b, a->v_stride_t, a->v_stride_h, a->dout_stride_b, a->dout_stride_t, a->dout_stride_h};
         for (int64_t st : raw_strides)
@@ -157,7 +158,7 @@ int gdn_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args* a, void* stream) {
                                a->dout_stride_b, a->dout_stride_t, a->dout_stride_h};
     for (int64_t s : strides)
         if (s < 0 || s % 8 != 0) return GDN_ERR_ALIGN;
-    if ((int64_t)a->N * a->H * (a->T / 64) > 0x7fffffff) return GDN_ERR_UNSUPPORTED;
+    if ((int64_t)a->N * a->H * (a->seq_start != nullptr ? a->NC : a->T / 64) > 0x7fffffff) return GDN_ERR_UNSUPPORTED;
     if (!aligned(a->records, 256) || a->records_bytes < gdn::chunk_bwd_record_bytes(*a)) return GDN_ERR_WORKSPACE;
     return gdn::launch_chunk_bwd_prepare(*a, static_cast<hipStream_t>(stream));
 }

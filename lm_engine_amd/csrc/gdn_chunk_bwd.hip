@@ -74,6 +74,11 @@ struct ChunkLocalParams {
     float* dg_out;
     float* dbeta_out;
     int H, NC;
+    // sequences that are not whole rows of whole chunks (packed or left-padded batches): first token (flat index
+    // over the rows of the caller's tensors) and length of every sequence; NULL = sequence n is row n
+    const int32_t* seq_start;
+    const int32_t* seq_len;
+    int T_rows;  // tokens per row of the caller's tensors
 };
 
 // acc[r] += sum_k A[8 (r/4) + 4 h + r%4][k] B[l32][k] over k < kd: A, B point at the first of 32 rows
@@ -121,9 +126,27 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
     const int ci = final_mode ? (int)(chunk % p.NC) : 0;
     const int chain = final_mode ? (int)(chunk / p.NC) : 0;
     const int n = final_mode ? chain / p.H : 0, h = final_mode ? chain % p.H : 0;
-    const int64_t T = (int64_t)p.NC * C;
-    const int64_t tok0 = (int64_t)n * T + (int64_t)ci * C;                                  // first token, caller's layout
-    const int64_t mirA = (int64_t)n * 2 * T + (int64_t)(p.NC - 1 - ci) * 2 * C;             // first token of mirror chunk A
+    // first token of the chunk as a flat index over the rows of the caller's tensors, and its number of tokens
+    int valid = C;
+    int64_t tok0 = 0;
+    if (final_mode) {
+        if (p.seq_start != nullptr) {
+            valid = min(max(p.seq_len[n] - ci * C, 0), C);
+            tok0 = (int64_t)p.seq_start[n] + (int64_t)ci * C;
+        } else {
+            tok0 = (int64_t)n * p.T_rows + (int64_t)ci * C;
+        }
+        if (valid == 0) return;  // a chunk past the end of its sequence (whole workgroup)
+    }
+    const int64_t mirA = ((int64_t)n * p.NC + (p.NC - 1 - ci)) * 2 * C;  // first token of mirror chunk A
+    // row `row` of the chunk in one of the caller's tensors; rows past the end read token 0 and are zeroed
+    auto row_of = [&](const bf16_t* base, int64_t sb, int64_t st, int64_t sh, int row) -> const bf16_t* {
+        const int64_t f = row < valid ? tok0 + row : 0;
+        return base + (f / p.T_rows) * sb + (f % p.T_rows) * st + (int64_t)h * sh;
+    };
+    bf16x8 zero8;
+#pragma unroll
+    for (int e = 0; e < 8; e++) zero8[e] = (bf16_t)0.f;
     const float* yy = final_mode ? nullptr : p.y + chunk * C * V;
     const float* vnew = p.vnew + chunk * C * V;
     const float* s0 = p.s0 + chunk * K * V;
@@ -181,13 +204,14 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
         if (final_mode) {
             // v, dO and Y (token `row` is token 63 - row of mirror chunk A); dV = beta Y goes out right away
             const int p8 = t % 16;
-            const int64_t tl = (int64_t)ci * C;
 #pragma unroll
             for (int it = 0; it < 4; it++) {
                 const int row = t / 16 + 16 * it;
+                const bool live = row < valid;
                 if (hv == 0) {
-                    const bf16x8 qr = *reinterpret_cast<const bf16x8*>(p.q_raw + n * p.q_stride_b + (tl + row) * p.q_stride_t + (int64_t)h * p.q_stride_h + 8 * p8);
-                    const bf16x8 kr = *reinterpret_cast<const bf16x8*>(p.k_raw + n * p.k_stride_b + (tl + row) * p.k_stride_t + (int64_t)h * p.k_stride_h + 8 * p8);
+                    bf16x8 qr = *reinterpret_cast<const bf16x8*>(row_of(p.q_raw, p.q_stride_b, p.q_stride_t, p.q_stride_h, row) + 8 * p8);
+                    bf16x8 kr = *reinterpret_cast<const bf16x8*>(row_of(p.k_raw, p.k_stride_b, p.k_stride_t, p.k_stride_h, row) + 8 * p8);
+                    if (!live) qr = zero8, kr = zero8;
                     const float fq = (p.rq != nullptr ? p.rq[chunk * C + row] : 1.f) * p.scale;
                     const float fk = p.rk != nullptr ? p.rk[chunk * C + row] : 1.f;
                     bf16x8 qb, kb;
@@ -201,8 +225,9 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
                     *reinterpret_cast<bf16x8*>(sQ + row * LDR + 8 * p8) = qb;
                     *reinterpret_cast<bf16x8*>(sK + row * LDR + 8 * p8) = kb;
                 }
-                const bf16x8 vr = *reinterpret_cast<const bf16x8*>(p.v_raw + n * p.v_stride_b + (tl + row) * p.v_stride_t + (int64_t)h * p.v_stride_h + v0 + 8 * p8);
-                const bf16x8 dr = *reinterpret_cast<const bf16x8*>(p.d_raw + n * p.d_stride_b + (tl + row) * p.d_stride_t + (int64_t)h * p.d_stride_h + v0 + 8 * p8);
+                bf16x8 vr = *reinterpret_cast<const bf16x8*>(row_of(p.v_raw, p.v_stride_b, p.v_stride_t, p.v_stride_h, row) + v0 + 8 * p8);
+                bf16x8 dr = *reinterpret_cast<const bf16x8*>(row_of(p.d_raw, p.d_stride_b, p.d_stride_t, p.d_stride_h, row) + v0 + 8 * p8);
+                if (!live) vr = zero8, dr = zero8;
                 const bf16x8 yr = *reinterpret_cast<const bf16x8*>(p.y_mirror + ((mirA + (C - 1 - row)) * p.H + h) * V + v0 + 8 * p8);
                 const float b = p.beta[chunk * C + row];
                 bf16x8 dv;
@@ -214,13 +239,14 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
                 }
                 *reinterpret_cast<bf16x8*>(sDO + row * LDR + 8 * p8) = dr;
                 *reinterpret_cast<bf16x8*>(sY + row * LDR + 8 * p8) = yr;
-                *reinterpret_cast<bf16x8*>(p.dv_out + ((tok0 + row) * p.H + h) * V + v0 + 8 * p8) = dv;
+                if (live) *reinterpret_cast<bf16x8*>(p.dv_out + ((tok0 + row) * p.H + h) * V + v0 + 8 * p8) = dv;
                 yv[it] = acc;
             }
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
+            for (int i = 0; i < 8; i++) {  // rows of V~ past the end of the sequence hold whatever the scan left
                 const int idx = t + BWD_THREADS * i, row = idx / 32, c4 = idx % 32;
-                put4(sVN + row * LDR + 4 * c4, *reinterpret_cast<const f32x4*>(vnew + row * V + v0 + 4 * c4));
+                const f32x4 x = *reinterpret_cast<const f32x4*>(vnew + row * V + v0 + 4 * c4);
+                put4(sVN + row * LDR + 4 * c4, row < valid ? x : f32x4{0.f, 0.f, 0.f, 0.f});
             }
         } else {
 #pragma unroll
@@ -396,8 +422,10 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
                 ok[e] = rk * (acck[tt][r] - ck * (float)sKT[d * LDS64 + i]);
             }
             if (final_mode) {
-                store4<bf16_t>(p.dq_out + at + 8 * r4, oq);
-                store4<bf16_t>(p.dk_out + at + 8 * r4, ok);
+                if (i < valid) {
+                    store4<bf16_t>(p.dq_out + at + 8 * r4, oq);
+                    store4<bf16_t>(p.dk_out + at + 8 * r4, ok);
+                }
             } else {
                 *reinterpret_cast<f32x4*>(p.dq + at + 8 * r4) = oq;
                 *reinterpret_cast<f32x4*>(p.dk + at + 8 * r4) = ok;
@@ -415,8 +443,10 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
                 const float y = __shfl_down(dg, off, WAVE);
                 if (t + off < C) dg += y;
             }
-            p.dg_out[(tok0 + t) * p.H + h] = dg;
-            p.dbeta_out[(tok0 + t) * p.H + h] = s_dbeta[t];
+            if (t < valid) {
+                p.dg_out[(tok0 + t) * p.H + h] = dg;
+                p.dbeta_out[(tok0 + t) * p.H + h] = s_dbeta[t];
+            }
         } else {
             p.dgam[chunk * C + t] = dg;
             p.dbeta[chunk * C + t] = s_dbeta[t];
@@ -457,6 +487,9 @@ struct BwdPrepareParams {
     float* bc;
     float* rq;
     float* rk;
+    const int32_t* seq_start;  // as in ChunkLocalParams
+    const int32_t* seq_len;
+    int T_rows;
     bf16_t* k_m;
     bf16_t* v_m;
     uint8_t* rec;
@@ -480,21 +513,35 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_bwd_prepare_kernel(const Bw
     const int ci = (int)(chunk % p.NC);
     const int chain = (int)(chunk / p.NC);
     const int n = chain / p.H, h = chain % p.H;
-    const int64_t T = (int64_t)p.NC * C, TM = 2 * T;
-    const int64_t tok0 = (int64_t)ci * C;
+    const int64_t TM = (int64_t)p.NC * 2 * C;  // tokens per sequence of the mirror problem
+    // first token of the chunk as a flat index over the rows of the caller's tensors, and its number of tokens;
+    // a chunk past the end of its sequence (valid = 0) still gets its (neutral) records and zero rows
+    int valid = C;
+    int64_t tok0 = (int64_t)n * p.T_rows + (int64_t)ci * C;
+    if (p.seq_start != nullptr) {
+        valid = min(max(p.seq_len[n] - ci * C, 0), C);
+        tok0 = (int64_t)p.seq_start[n] + (int64_t)ci * C;
+    }
+    auto row_of = [&](const bf16_t* base, int64_t sb, int64_t st, int64_t sh, int row) -> const bf16_t* {
+        const int64_t f = row < valid ? tok0 + row : 0;
+        return base + (f / p.T_rows) * sb + (f % p.T_rows) * st + (int64_t)h * sh;
+    };
+    bf16x8 zero8;
+#pragma unroll
+    for (int e = 0; e < 8; e++) zero8[e] = (bf16_t)0.f;
     const int64_t mir0 = (int64_t)(p.NC - 1 - ci) * 2 * C;  // first token of chunk A in the mirror problem
 
     // ---- gamma (prefix sum of g inside the chunk) and beta: wave 0 ----
     if (wave == 0) {
-        const int64_t at = ((int64_t)n * T + tok0 + lane) * p.H + h;
-        float x = p.g == nullptr ? 0.f : p.g[at];
+        const int64_t at = (lane < valid ? tok0 + lane : 0) * p.H + h;
+        float x = (p.g == nullptr || lane >= valid) ? 0.f : p.g[at];
 #pragma unroll
         for (int off = 1; off < WAVE; off <<= 1) {
             const float y = __shfl_up(x, off, WAVE);
             if (lane >= off) x += y;
         }
         const float gl = __shfl(x, WAVE - 1, WAVE);
-        const float b = load_beta(p.beta, p.beta_dtype, at);
+        const float b = lane < valid ? load_beta(p.beta, p.beta_dtype, at) : 0.f;
         s_gam[lane] = x, s_beta[lane] = b, s_e[lane] = __expf(x), s_tail[lane] = __expf(gl - x);
         p.gam[chunk * C + lane] = x;
         p.bc[chunk * C + lane] = b;
@@ -505,9 +552,10 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_bwd_prepare_kernel(const Bw
 #pragma unroll
     for (int it = 0; it < 4; it++) {
         const int row = t / 16 + 16 * it;
-        const int64_t tok = tok0 + row;
-        const bf16x8 qr = *reinterpret_cast<const bf16x8*>(p.q + n * p.q_stride_b + tok * p.q_stride_t + (int64_t)h * p.q_stride_h + 8 * p8);
-        const bf16x8 kr = *reinterpret_cast<const bf16x8*>(p.k + n * p.k_stride_b + tok * p.k_stride_t + (int64_t)h * p.k_stride_h + 8 * p8);
+        const bool live = row < valid;
+        bf16x8 qr = *reinterpret_cast<const bf16x8*>(row_of(p.q, p.q_stride_b, p.q_stride_t, p.q_stride_h, row) + 8 * p8);
+        bf16x8 kr = *reinterpret_cast<const bf16x8*>(row_of(p.k, p.k_stride_b, p.k_stride_t, p.k_stride_h, row) + 8 * p8);
+        if (!live) qr = zero8, kr = zero8;
         float ssq = 0.f, ssk = 0.f;
 #pragma unroll
         for (int e = 0; e < 8; e++) ssq += (float)qr[e] * (float)qr[e], ssk += (float)kr[e] * (float)kr[e];
@@ -532,7 +580,8 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_bwd_prepare_kernel(const Bw
         *reinterpret_cast<bf16x8*>(p.k_m + tokB * K + 8 * p8) = qr;
 #pragma unroll
         for (int hv = 0; hv < V / 128; hv++) {
-            const bf16x8 dr = *reinterpret_cast<const bf16x8*>(p.dout + n * p.d_stride_b + tok * p.d_stride_t + (int64_t)h * p.d_stride_h + 128 * hv + 8 * p8);
+            bf16x8 dr = *reinterpret_cast<const bf16x8*>(row_of(p.dout, p.d_stride_b, p.d_stride_t, p.d_stride_h, row) + 128 * hv + 8 * p8);
+            if (!live) dr = zero8;
 #pragma unroll
             for (int e = 0; e < 8; e++) sDOT[(128 * hv + 8 * p8 + e) * LDS64 + row] = dr[e];
             *reinterpret_cast<bf16x8*>(p.v_m + tokB * V + 128 * hv + 8 * p8) = dr;
@@ -648,6 +697,7 @@ int launch_chunk_bwd_local(const gdn_chunk_local_args& a, hipStream_t stream) {
     p.k_stride_b = a.k_stride_b, p.k_stride_t = a.k_stride_t, p.k_stride_h = a.k_stride_h;
     p.v_stride_b = a.v_stride_b, p.v_stride_t = a.v_stride_t, p.v_stride_h = a.v_stride_h;
     p.d_stride_b = a.dout_stride_b, p.d_stride_t = a.dout_stride_t, p.d_stride_h = a.dout_stride_h;
+    p.seq_start = a.seq_start, p.seq_len = a.seq_len, p.T_rows = a.seq_start != nullptr ? a.T_rows : a.NC * C;
     if (a.V == 256) hipLaunchKernelGGL(chunk_local_grads_kernel<256>, dim3((unsigned)a.chunks), dim3(BWD_THREADS), 0, stream, p);
     else hipLaunchKernelGGL(chunk_local_grads_kernel<128>, dim3((unsigned)a.chunks), dim3(BWD_THREADS), 0, stream, p);
     return (int)hipGetLastError();
@@ -656,11 +706,13 @@ int launch_chunk_bwd_local(const gdn_chunk_local_args& a, hipStream_t stream) {
 bool chunk_bwd_local_supported(const gdn_chunk_local_args& a) { return a.K == BWD_K && (a.V == 128 || a.V == 256); }
 
 bool chunk_bwd_prepare_supported(const gdn_chunk_bwd_prepare_args& a) {
-    return a.K == BWD_K && (a.V == 128 || a.V == 256) && a.T > 0 && a.T % C == 0;
+    if (a.K != BWD_K || (a.V != 128 && a.V != 256) || a.T <= 0) return false;
+    return a.seq_start != nullptr ? (a.seq_len != nullptr && a.NC > 0) : a.T % C == 0;
 }
 
 uint64_t chunk_bwd_record_bytes(const gdn_chunk_bwd_prepare_args& a) {
-    return (uint64_t)a.H * a.N * 2 * (a.T / C) * record_layout(a.K, a.V).bytes;
+    const uint64_t nc = a.seq_start != nullptr ? a.NC : a.T / C;
+    return (uint64_t)a.H * a.N * 2 * nc * record_layout(a.K, a.V).bytes;
 }
 
 int launch_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args& a, hipStream_t stream) {
@@ -672,7 +724,8 @@ int launch_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args& a, hipStream_t st
     p.q_stride_b = a.q_stride_b, p.q_stride_t = a.q_stride_t, p.q_stride_h = a.q_stride_h;
     p.k_stride_b = a.k_stride_b, p.k_stride_t = a.k_stride_t, p.k_stride_h = a.k_stride_h;
     p.d_stride_b = a.dout_stride_b, p.d_stride_t = a.dout_stride_t, p.d_stride_h = a.dout_stride_h;
-    p.N = a.N, p.H = a.H, p.NC = a.T / C;
+    p.N = a.N, p.H = a.H, p.NC = a.seq_start != nullptr ? a.NC : a.T / C;
+    p.seq_start = a.seq_start, p.seq_len = a.seq_len, p.T_rows = a.T;
     p.l2norm = (a.flags & GDN_FLAG_L2NORM) ? 1 : 0;
     p.scale = a.scale;
     p.gam = a.gamma, p.bc = a.beta_packed;

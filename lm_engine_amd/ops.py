@@ -291,28 +291,31 @@ def chunk_local_grads(qs, kn, v, dout, y, v_new, states, dstates, gamma, beta, s
     return out["dq"], out["dk"], out["dbeta"], out["dgamma"]
 
 
-def chunk_local_grads_final(q, k, v, dout, prep, y_mirror, v_new, states, dstates, scale, l2norm):
-    """``gdn_chunk_bwd_local`` in its final mode, for a batch of whole chunks: q, k, v, dout are the caller's bf16
-    tensors (last dim contiguous), ``prep`` what ``chunk_bwd_prepare`` returned, ``y_mirror`` the output of the
-    scan over its mirror problem.  Returns ``dq, dk, dv`` bf16 ``[N, T, H, D]`` and ``dg, dbeta`` fp32
-    ``[N, T, H]``."""
+def chunk_local_grads_final(q, k, v, dout, prep, y_mirror, v_new, states, dstates, scale, l2norm, sequences=None):
+    """``gdn_chunk_bwd_local`` in its final mode: q, k, v, dout are the caller's bf16 ``[B, T, H, D]`` tensors (last
+    dim contiguous), ``prep`` what ``chunk_bwd_prepare`` returned (same ``sequences``), ``y_mirror`` the output of
+    the scan over its mirror problem.  Returns ``dq, dk, dv`` bf16 ``[B, T, H, D]`` and ``dg, dbeta`` fp32
+    ``[B, T, H]`` (zero where no sequence lives)."""
     _require_hip_path()
     lib = _lib.load_library()
-    N, T, H, K = q.shape
+    B, T, H, K = q.shape
     V = v.size(-1)
     Bt, NC, C = prep["gamma"].shape
+    N = Bt // H
     dev = y_mirror.device
-    if Bt != N * H or NC * C != T or tuple(y_mirror.shape) != (N, 2 * T, H, V) or y_mirror.dtype != torch.bfloat16 or not y_mirror.is_contiguous():
-        raise ValueError("y_mirror must be the contiguous bf16 [N, 2 T, H, V] output of the scan over the mirror problem")
+    if (sequences is None and (N != B or NC * C != T)) or tuple(y_mirror.shape) != (N, 2 * NC * C, H, V) \
+            or y_mirror.dtype != torch.bfloat16 or not y_mirror.is_contiguous():  # fmt: skip
+        raise ValueError("y_mirror must be the contiguous bf16 [N, 2 NC 64, H, V] output of the scan over the mirror problem")
     for name, x, shape in (("v_new", v_new, (Bt, NC, C, V)), ("states", states, (Bt, NC, K, V)), ("dstates", dstates, (Bt, NC, K, V))):
         if tuple(x.shape) != shape or x.dtype != torch.float32 or not x.is_contiguous():
             raise ValueError(f"{name} must be contiguous fp32 {shape}")
+    alloc = torch.empty if sequences is None else torch.zeros  # tokens outside every sequence are not written
     out = dict(
-        dq_out=torch.empty(N, T, H, K, dtype=torch.bfloat16, device=dev),
-        dk_out=torch.empty(N, T, H, K, dtype=torch.bfloat16, device=dev),
-        dv_out=torch.empty(N, T, H, V, dtype=torch.bfloat16, device=dev),
-        dg_out=torch.empty(N, T, H, dtype=torch.float32, device=dev),
-        dbeta_out=torch.empty(N, T, H, dtype=torch.float32, device=dev),
+        dq_out=alloc(B, T, H, K, dtype=torch.bfloat16, device=dev),
+        dk_out=alloc(B, T, H, K, dtype=torch.bfloat16, device=dev),
+        dv_out=alloc(B, T, H, V, dtype=torch.bfloat16, device=dev),
+        dg_out=alloc(B, T, H, dtype=torch.float32, device=dev),
+        dbeta_out=alloc(B, T, H, dtype=torch.float32, device=dev),
     )
     a = _lib.GdnChunkLocalArgs()
     a.gamma, a.beta = prep["gamma"].data_ptr(), prep["beta"].data_ptr()
@@ -330,6 +333,8 @@ def chunk_local_grads_final(q, k, v, dout, prep, y_mirror, v_new, states, dstate
     for name, x in out.items():
         setattr(a, name, x.data_ptr())
     a.chunks, a.K, a.V, a.scale, a.H, a.NC = Bt * NC, K, V, float(scale), H, NC
+    if sequences is not None:
+        a.seq_start, a.seq_len, a.T_rows = sequences[0].data_ptr(), sequences[1].data_ptr(), T
     with torch.cuda.device(dev):
         stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
         _lib.check_status(lib.gdn_chunk_bwd_local(ctypes.byref(a), stream), "gdn_chunk_bwd_local")
@@ -339,26 +344,35 @@ def chunk_local_grads_final(q, k, v, dout, prep, y_mirror, v_new, states, dstate
 RECORD_BYTES = 13312  # chunk record of the 32x32x16 kernels (K <= 128)
 
 
-def chunk_bwd_prepare(q, k, dout, g, beta, scale, l2norm, V):
-    """``gdn_chunk_bwd_prepare`` for a batch of whole chunks (``[N, T, H, 128]`` bf16, T a multiple of 64).
-    Returns a dict: ``gamma, beta, rq, rk`` (fp32 ``[N H, T/64, 64]``: prefix sums of g inside the chunks, beta,
-    inverse norms of the rows of q and k) and the mirror problem ``k_mirror, v_mirror`` ``[N, 2 T, H, D]`` bf16,
-    ``records`` uint8 ``[H, N * 2 T/64, RECORD_BYTES]``."""
+def chunk_bwd_prepare(q, k, dout, g, beta, scale, l2norm, V, sequences=None):
+    """``gdn_chunk_bwd_prepare``.  ``q, k, dout`` are the caller's bf16 ``[B, T, H, D]`` tensors; without
+    ``sequences`` every row is one sequence of whole chunks, else ``sequences = (seq_start, seq_len, NC)``: int32
+    device tensors ``[N]`` (first token as a flat index over the rows, length) and the chunks per sequence to lay
+    the results out with.  Returns a dict: ``gamma, beta, rq, rk`` (fp32 ``[N H, NC, 64]``: prefix sums of g inside
+    the chunks, beta, inverse norms of the rows of q and k) and the mirror problem ``k_mirror, v_mirror``
+    ``[N, 2 NC 64, H, D]`` bf16, ``records`` uint8 ``[H, N * 2 NC, RECORD_BYTES]``."""
     _require_hip_path()
     lib = _lib.load_library()
-    N, T, H, K = q.shape
-    if (K, V) not in CHUNK_LOCAL_KV or T % 64 != 0 or q.dtype != torch.bfloat16:
-        raise ValueError(f"built for bf16, K, V = {CHUNK_LOCAL_KV} and T a multiple of 64")
+    B, T, H, K = q.shape
+    if (K, V) not in CHUNK_LOCAL_KV or q.dtype != torch.bfloat16:
+        raise ValueError(f"built for bf16 and K, V in {CHUNK_LOCAL_KV}")
+    if sequences is None:
+        if T % 64 != 0:
+            raise ValueError("without `sequences` T must be a multiple of 64")
+        N, NC = B, T // 64
+    else:
+        seq_start, seq_len, NC = sequences
+        N = seq_start.numel()
     g = None if g is None else g.to(torch.float32).contiguous()
     if beta is not None:
         beta = beta.contiguous() if beta.dtype in (torch.bfloat16, torch.float32) else beta.float().contiguous()
-    dev, NC, Bt = q.device, T // 64, N * H
+    dev, Bt = q.device, N * H
     f32 = dict(dtype=torch.float32, device=dev)
     out = dict(
         gamma=torch.empty(Bt, NC, 64, **f32), beta=torch.empty(Bt, NC, 64, **f32),
         rq=torch.empty(Bt, NC, 64, **f32), rk=torch.empty(Bt, NC, 64, **f32),
-        k_mirror=torch.empty(N, 2 * T, H, K, dtype=torch.bfloat16, device=dev),
-        v_mirror=torch.empty(N, 2 * T, H, V, dtype=torch.bfloat16, device=dev),
+        k_mirror=torch.empty(N, 2 * NC * 64, H, K, dtype=torch.bfloat16, device=dev),
+        v_mirror=torch.empty(N, 2 * NC * 64, H, V, dtype=torch.bfloat16, device=dev),
         records=torch.empty(H, N * 2 * NC, RECORD_BYTES, dtype=torch.uint8, device=dev),
     )  # fmt: skip
     a = _lib.GdnChunkBwdPrepareArgs()
@@ -376,6 +390,8 @@ def chunk_bwd_prepare(q, k, dout, g, beta, scale, l2norm, V):
     a.gamma, a.beta_packed, a.rq, a.rk = (out[n].data_ptr() for n in ("gamma", "beta", "rq", "rk"))
     a.k_mirror, a.v_mirror, a.records = (out[n].data_ptr() for n in ("k_mirror", "v_mirror", "records"))
     a.records_bytes = out["records"].numel()
+    if sequences is not None:
+        a.seq_start, a.seq_len, a.NC = seq_start.data_ptr(), seq_len.data_ptr(), NC
     with torch.cuda.device(dev):
         stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
         _lib.check_status(lib.gdn_chunk_bwd_prepare(ctypes.byref(a), stream), "gdn_chunk_bwd_prepare")

@@ -60,9 +60,10 @@ def test_chunk_bf16(T):
     _run_case(lm_engine_amd.chunk_gated_delta_rule, inp, torch.bfloat16)
 
 
-def test_chunk_bf16_packed():
+@pytest.mark.parametrize("V", [64, 128])  # V = 64: chunk-local part as batched GEMMs; V = 128: all on kernels
+def test_chunk_bf16_packed(V):
     cu = torch.tensor([0, 70, 71, 300], dtype=torch.int32)
-    inp = random_inputs(B=1, T=300, H=2, K=128, V=64, dtype=torch.bfloat16, seed=7, normalize=False, N=3)
+    inp = random_inputs(B=1, T=300, H=2, K=128, V=V, dtype=torch.bfloat16, seed=7, normalize=False, N=3)
     _run_case(lm_engine_amd.chunk_gated_delta_rule, inp, torch.bfloat16, cu=cu)
 
 
