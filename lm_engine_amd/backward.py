@@ -6,13 +6,13 @@ the gradients of ``(o, final_state)`` with respect to ``(q, k, v, g, beta, initi
 
 Three ways through, same formulas:
 
-* bf16, K = 128, V = 128 or 256, batches of whole chunks (no cu_seqlens, T a multiple of 64): five kernel
-  launches (``_backward_on_kernels``) - ``gdn_chunk_bwd_prepare``, ``gdn_chunk_fwd_saving`` for the forward
-  sweep and again over the mirror problem for the reverse sweep, ``gdn_chunk_bwd_local``;
-* other bf16 shapes with K <= 128, packed, ragged or left-padded batches: the two sweeps over the chunks of a
-  chain on the scan kernel (``gdn_chunk_fwd_saving``: the forward's scan in a variant that also writes the chunk
-  states and V~), everything chunk-local as batched library GEMMs (fp32, ``torch.bmm``) and elementwise torch
-  operations on sequences padded to whole chunks;
+* bf16, K = 128, V = 128 or 256 (whole rows, packed or left-padded batches): five kernel launches
+  (``_backward_on_kernels``) - ``gdn_chunk_bwd_prepare``, ``gdn_chunk_fwd_saving`` for the forward sweep and
+  again over the mirror problem for the reverse sweep, ``gdn_chunk_bwd_local``;
+* other bf16 shapes with K <= 128: the two sweeps over the chunks of a chain on the scan kernel
+  (``gdn_chunk_fwd_saving``: the forward's scan in a variant that also writes the chunk states and V~),
+  everything chunk-local as batched library GEMMs (fp32, ``torch.bmm``) and elementwise torch operations on
+  sequences padded to whole chunks;
 * fp32 inputs, K = 256, CPU tensors: the sweeps as loops of batched GEMMs as well.
 
 The reverse sweep is the same recurrence as the forward one on other data, which is how it gets onto
