@@ -4,6 +4,8 @@ through the fp64 token loop of the oracle on the same (rounded) inputs.
 Gate for a gradient: relative-L2 <= 1e-2 and max-abs <= 2e-2 x max(1, max |reference|) for bf16 inputs
 (the gradients come back rounded to bf16), 1e-4 on both for fp32 inputs."""
 
+import os
+
 import pytest
 import torch
 
@@ -185,3 +187,69 @@ def test_chunk_local_kernel_matches_the_batched_gemm_version(V):
         err = rel_l2(a, b)
         print(f"   normalised {name}: rel-L2 {err:.3e}", flush=True)
         assert err <= 1e-2, f"{name}: rel-L2 {err:.3e}"
+
+
+def _backward_sweep_case(i):
+    """Case ``i`` of a seeded sweep over batch layouts and options (K = 128: prepare, sweeps and chunk-local
+    gradients all run as kernels)."""
+    gen = torch.Generator().manual_seed(9000 + i)
+    pick = lambda *xs: xs[int(torch.randint(len(xs), (1,), generator=gen))]  # noqa: E731
+    layout = pick("rows", "packed", "left_padded")
+    H, V = pick(1, 2, 3), pick(128, 256)
+    l2norm, with_state, with_dht, gated = pick(True, False), pick(True, False), pick(True, False), pick(True, True, False)
+    if layout == "rows":
+        B, T = pick(1, 2), pick(64, 70, 128, 191)
+        lens, cu = [T] * B, None
+    elif layout == "packed":
+        lens = [int(x) for x in torch.randint(1, 150, (pick(1, 2, 4),), generator=gen)]
+        B, T = 1, sum(lens)
+        cu = torch.tensor([0] + lens).cumsum(0).to(torch.int32)
+    else:
+        B, T = pick(2, 3), pick(96, 130)
+        lens = [T] + [int(x) for x in torch.randint(1, T + 1, (B - 1,), generator=gen)]
+        cu = torch.tensor([0] + lens).cumsum(0).to(torch.int32)
+    N = len(lens)
+    inp = random_inputs(B=B, T=T, H=H, K=128, V=V, dtype=torch.bfloat16, seed=9100 + i, normalize=not l2norm, gated=gated, N=N)
+    if not with_state:
+        inp["initial_state"] = None
+    return dict(layout=layout, lens=lens, cu=cu, inp=inp, l2norm=l2norm, with_dht=with_dht, B=B, T=T, H=H, V=V)
+
+
+@pytest.mark.parametrize("i", range(int(os.environ.get("GDN_SWEEP_CASES", "10"))))
+def test_seeded_sweep_of_layouts_and_options(i):
+    c = _backward_sweep_case(i)
+    inp, cu, T = c["inp"], c["cu"], c["T"]
+    print(f"case {i}: {c['layout']} lens={c['lens']} H={c['H']} V={c['V']} l2norm={c['l2norm']} "
+          f"h0={inp['initial_state'] is not None} dht={c['with_dht']} gated={inp['g'] is not None}", flush=True)  # fmt: skip
+    leaves = {n: x.cuda().requires_grad_(True) for n, x in inp.items() if x is not None}
+    o, ht = lm_engine_amd.chunk_gated_delta_rule(
+        **leaves, output_final_state=True, cu_seqlens=None if cu is None else cu.cuda(),
+        use_qk_l2norm_in_kernel=c["l2norm"], left_padded=c["layout"] == "left_padded")  # fmt: skip
+    gen = torch.Generator().manual_seed(9200 + i)
+    do = torch.randn(o.shape, generator=gen).to(torch.bfloat16)
+    dht = torch.randn(ht.shape, generator=gen) if c["with_dht"] else None
+    loss = (o.float() * do.cuda().float()).sum()
+    if dht is not None:
+        loss = loss + (ht * dht.cuda()).sum()
+    loss.backward()
+    names = [n for n in ("q", "k", "v", "g", "beta", "initial_state") if n in leaves]
+    zero_g = torch.zeros(c["B"], T, c["H"])
+    for n, length in enumerate(c["lens"]):  # sequence by sequence against the oracle
+        if c["layout"] == "rows":
+            sl = lambda x: x[n : n + 1]  # noqa: E731
+        elif c["layout"] == "packed":
+            t0 = int(cu[n])
+            sl = lambda x: x[:, t0 : t0 + length]  # noqa: E731
+        else:
+            sl = lambda x: x[n : n + 1, T - length :]  # noqa: E731
+        h0 = None if inp["initial_state"] is None else inp["initial_state"][n : n + 1]
+        want = gated_delta_rule_grads_autograd(
+            sl(inp["q"]), sl(inp["k"]), sl(inp["v"]), sl(inp["g"] if inp["g"] is not None else zero_g), sl(inp["beta"]),
+            sl(do), None if dht is None else dht[n : n + 1], initial_state=h0, use_qk_l2norm_in_kernel=c["l2norm"])  # fmt: skip
+        want = dict(zip(("q", "k", "v", "g", "beta", "initial_state"), want))
+        got = [sl(leaves[x].grad.cpu()) if x != "initial_state" else leaves[x].grad[n : n + 1] for x in names]
+        _assert_grads(got, [want[x] for x in names], torch.bfloat16)
+    if c["layout"] == "left_padded":
+        for b, length in enumerate(c["lens"]):
+            for x in ("q", "k", "v"):
+                assert not leaves[x].grad[b, : T - length].any(), f"gradient of {x} at the padding"
