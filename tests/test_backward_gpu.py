@@ -253,3 +253,9 @@ def test_seeded_sweep_of_layouts_and_options(i):
         for b, length in enumerate(c["lens"]):
             for x in ("q", "k", "v"):
                 assert not leaves[x].grad[b, : T - length].any(), f"gradient of {x} at the padding"
+
+
+def test_recurrent_bf16_short_sequences():
+    # T <= 64: the layer calls the recurrent operator; its backward runs the chunk kernels on one ragged chunk
+    inp = random_inputs(B=2, T=40, H=2, K=128, V=128, dtype=torch.bfloat16, seed=14, normalize=False)
+    _run_case(lm_engine_amd.fused_recurrent_gated_delta_rule, inp, torch.bfloat16)
