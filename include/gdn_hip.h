@@ -284,6 +284,28 @@ typedef struct gdn_conv_args {
 int gdn_causal_conv1d_fwd(const gdn_conv_args *args, void *stream);
 
 /*
+ * Backward of gdn_causal_conv1d_fwd for bf16 x (what autograd computes through
+ * DepthwiseCausalConvolution.forward, depthwise_causal_convolution.py:103-241, when the layer trains):
+ * given dy [B, S, C] (element strides) it recomputes the pre-activation from x and writes dx [B, S, C]
+ * (bf16, contiguous), dstate [B, C, kernel_size - 1] (bf16; NULL when there was no input_state) and, per
+ * block of 64 tokens of a row, the partial sums of the gradients of weight and bias:
+ * dweight_partial [B * ceil(S / 64)][C][kernel_size] and dbias_partial [B * ceil(S / 64)][C], fp32, which
+ * the caller adds up over the first dim.  The gradient flowing into final_state is not handled (the layer
+ * does not differentiate through its cache).
+ */
+typedef struct gdn_conv_bwd_args {
+    const void *x, *dy, *weight, *bias, *input_state, *mask;
+    void *dx, *dstate;
+    float *dweight_partial, *dbias_partial;
+    int64_t x_stride_b, x_stride_s;
+    int64_t dy_stride_b, dy_stride_s;
+    int32_t B, S, C, kernel_size;
+    int32_t w_dtype;    /* gdn_dtype of weight and bias */
+    int32_t activation; /* gdn_activation */
+} gdn_conv_bwd_args;
+int gdn_causal_conv1d_bwd(const gdn_conv_bwd_args *args, void *stream);
+
+/*
  * The operator's scalar inputs from the layer's projections, one pass:
  *   g    = -exp(A_log[h]) * softplus(a + dt_bias[h])     fp32   SoftplusDecayGate.forward with
  *          final_exponential=False, lm_engine/modeling_utils/softplus_decay_gate/module.py:69-96

@@ -35,6 +35,7 @@ EXPORTED_SYMBOLS = (
     "gdn_chunk_bwd_local",
     "gdn_chunk_bwd_prepare",
     "gdn_causal_conv1d_fwd",
+    "gdn_causal_conv1d_bwd",
     "gdn_gates_fwd",
     "gdn_gated_rmsnorm_fwd",
 )
@@ -77,6 +78,15 @@ class GdnChunkBwdPrepareArgs(ctypes.Structure):
         + [(name, ctypes.c_void_p) for name in ("gamma", "beta_packed", "rq", "rk", "k_mirror", "v_mirror", "records")]
         + [("records_bytes", ctypes.c_uint64), ("seq_start", ctypes.c_void_p), ("seq_len", ctypes.c_void_p),
            ("NC", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+    )  # fmt: skip
+
+
+class GdnConvBwdArgs(ctypes.Structure):
+    _fields_ = (
+        [(name, ctypes.c_void_p) for name in ("x", "dy", "weight", "bias", "input_state", "mask", "dx", "dstate",
+                                              "dweight_partial", "dbias_partial")]
+        + [(name, ctypes.c_int64) for name in ("x_stride_b", "x_stride_s", "dy_stride_b", "dy_stride_s")]
+        + [(name, ctypes.c_int32) for name in ("B", "S", "C", "kernel_size", "w_dtype", "activation")]
     )  # fmt: skip
 
 
@@ -169,6 +179,8 @@ def load_library() -> ctypes.CDLL:
     lib.gdn_chunk_bwd_prepare.restype = ctypes.c_int
     lib.gdn_causal_conv1d_fwd.argtypes = [ctypes.POINTER(GdnConvArgs), ctypes.c_void_p]
     lib.gdn_causal_conv1d_fwd.restype = ctypes.c_int
+    lib.gdn_causal_conv1d_bwd.argtypes = [ctypes.POINTER(GdnConvBwdArgs), ctypes.c_void_p]
+    lib.gdn_causal_conv1d_bwd.restype = ctypes.c_int
     lib.gdn_gates_fwd.argtypes = [ctypes.POINTER(GdnGateArgs), ctypes.c_void_p]
     lib.gdn_gates_fwd.restype = ctypes.c_int
     lib.gdn_gated_rmsnorm_fwd.argtypes = [ctypes.POINTER(GdnNormArgs), ctypes.c_void_p]

@@ -4,7 +4,8 @@ Functional form of the reference's ``DepthwiseCausalConvolution.forward``
 (lm_engine/modeling_utils/depthwise_causal_convolution.py:103-241): same arguments, same three
 modes (fresh prefill, one-token update, multi-token continuation), same return ``(y, final_state)``.
 It runs one HIP kernel (``gdn_causal_conv1d_fwd`` of libgdn_hip.so); there is no torch fallback.
-Under autograd the backward differentiates the same formula written in torch (``_autograd.py``).
+Under autograd the backward of bf16 inputs is one more HIP kernel (``gdn_causal_conv1d_bwd``); other inputs
+differentiate the same formula written in torch (``_autograd.py``).
 
     x             [B, S, C]          bf16 or fp32, channels contiguous
     weight        [C, 1, ks] or [C, ks]   nn.Conv1d's depthwise weight, ks in 2..4
@@ -65,7 +66,80 @@ def depthwise_causal_convolution(
 
     kernel = lambda x, weight, bias, input_state: _depthwise_causal_convolution(  # noqa: E731
         x, weight, bias, input_state, attention_mask, output_state, activation)  # fmt: skip
+    needs_grad = torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (x, weight, bias, input_state))
+    if needs_grad and _backward_kernel_applies(x, weight, activation):
+        return _ConvolutionOnKernels.apply(x, weight, bias, input_state, attention_mask, output_state, activation)
     return kernel_with_formula_backward(kernel, formula, x, weight, bias, input_state)
+
+
+def _backward_kernel_applies(x, weight, activation) -> bool:
+    if not x.is_cuda or x.dtype != torch.bfloat16 or activation not in _IN_KERNEL_ACTIVATIONS or x.dim() != 3:
+        return False
+    B, S, C = x.shape
+    return C % 8 == 0 and weight.dtype in (torch.bfloat16, torch.float32) and B * (-(-S // 64)) <= 65535
+
+
+class _ConvolutionOnKernels(torch.autograd.Function):
+    """Forward and backward on the HIP kernels (bf16 x).  The gradient that flows into the returned state is
+    not propagated: the layer's cache is not differentiated through."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, input_state, attention_mask, output_state, activation):
+        y, final_state = _depthwise_causal_convolution(x, weight, bias, input_state, attention_mask, output_state,
+                                                       activation)  # fmt: skip
+        ctx.save_for_backward(x, weight, bias, input_state, attention_mask)
+        ctx.activation = activation
+        if final_state is not None:
+            ctx.mark_non_differentiable(final_state)
+        return y, final_state
+
+    @staticmethod
+    def backward(ctx, dy, _dstate_out):
+        x, weight, bias, input_state, attention_mask = ctx.saved_tensors
+        dx, dweight, dbias, dstate = _convolution_backward(x, weight, bias, input_state, attention_mask, dy,
+                                                           ctx.activation)  # fmt: skip
+        return dx, dweight, dbias, dstate, None, None, None
+
+
+def _convolution_backward(x, weight, bias, input_state, attention_mask, dy, activation):
+    """``gdn_causal_conv1d_bwd``: dx, dweight, dbias, dinput_state for bf16 x (see include/gdn_hip.h)."""
+    lib = _lib.load_library()
+    B, S, C = x.shape
+    w2 = (weight.squeeze(1) if weight.dim() == 3 else weight).contiguous()
+    ks = w2.size(1)
+    if x.stride(-1) != 1:
+        x = x.contiguous()
+    dy = dy.to(torch.bfloat16)
+    if dy.stride(-1) != 1:
+        dy = dy.contiguous()
+    b2 = None if bias is None else bias.to(w2.dtype).contiguous()
+    state = None if input_state is None else input_state.to(x.dtype).contiguous()
+    mask = None
+    if attention_mask is not None and attention_mask.shape[1] > 1 and attention_mask.shape[0] > 1:
+        mask = attention_mask.to(x.dtype).contiguous()
+    blocks = B * (-(-S // 64))
+    dx = torch.empty(B, S, C, dtype=x.dtype, device=x.device)
+    dstate = None if state is None else torch.empty(B, C, ks - 1, dtype=x.dtype, device=x.device)
+    dw_part = torch.empty(blocks, C, ks, dtype=torch.float32, device=x.device)
+    db_part = torch.empty(blocks, C, dtype=torch.float32, device=x.device)
+    a = _lib.GdnConvBwdArgs()
+    a.x, a.dy, a.weight, a.dx = x.data_ptr(), dy.data_ptr(), w2.data_ptr(), dx.data_ptr()
+    a.bias = None if b2 is None else b2.data_ptr()
+    a.input_state = None if state is None else state.data_ptr()
+    a.mask = None if mask is None else mask.data_ptr()
+    a.dstate = None if dstate is None else dstate.data_ptr()
+    a.dweight_partial, a.dbias_partial = dw_part.data_ptr(), db_part.data_ptr()
+    a.x_stride_b, a.x_stride_s, a.dy_stride_b, a.dy_stride_s = x.stride(0), x.stride(1), dy.stride(0), dy.stride(1)
+    a.B, a.S, a.C, a.kernel_size = B, S, C, ks
+    a.w_dtype = _dtype_code(w2.dtype, "weight")
+    a.activation = _IN_KERNEL_ACTIVATIONS[activation]
+    with torch.cuda.device(x.device):
+        stream = ctypes.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)
+        _lib.check_status(lib.gdn_causal_conv1d_bwd(ctypes.byref(a), stream), "gdn_causal_conv1d_bwd")
+    dweight = dw_part.sum(dim=0).to(weight.dtype).reshape(weight.shape)
+    dbias = None if bias is None else db_part.sum(dim=0).to(bias.dtype)
+    dstate = None if dstate is None else dstate.to(input_state.dtype)
+    return dx, dweight, dbias, dstate
 
 
 def _depthwise_causal_convolution(x, weight, bias, input_state, attention_mask, output_state, activation):

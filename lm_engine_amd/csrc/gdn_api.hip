@@ -163,6 +163,21 @@ int gdn_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args* a, void* stream) {
     return gdn::launch_chunk_bwd_prepare(*a, static_cast<hipStream_t>(stream));
 }
 
+int gdn_causal_conv1d_bwd(const gdn_conv_bwd_args* a, void* stream) {
+    if (a == nullptr) return GDN_ERR_NULL;
+    if (!a->x || !a->dy || !a->weight || !a->dx || !a->dweight_partial || !a->dbias_partial) return GDN_ERR_NULL;
+    if (a->B <= 0 || a->S <= 0 || a->C <= 0) return GDN_ERR_SHAPE;
+    if (a->C % 8 != 0 || a->kernel_size < 2 || a->kernel_size > 4) return GDN_ERR_UNSUPPORTED;
+    if (a->w_dtype != GDN_BF16 && a->w_dtype != GDN_F32) return GDN_ERR_UNSUPPORTED;
+    if (a->activation != GDN_ACT_NONE && a->activation != GDN_ACT_SILU) return GDN_ERR_UNSUPPORTED;
+    if (!aligned(a->x, 16) || !aligned(a->dy, 16) || !aligned(a->dx, 16)) return GDN_ERR_ALIGN;
+    const int64_t strides[] = {a->x_stride_b, a->x_stride_s, a->dy_stride_b, a->dy_stride_s};
+    for (int64_t s : strides)
+        if (s < 0 || s % 8 != 0) return GDN_ERR_ALIGN;
+    if ((int64_t)a->B * ((a->S + 63) / 64) > 65535) return GDN_ERR_UNSUPPORTED;  // one grid row per 64 tokens
+    return gdn::launch_conv_bwd(*a, static_cast<hipStream_t>(stream));
+}
+
 int gdn_chunk_fwd_profile(const gdn_args* a, void* stream, float* kernel_ms) {
     if (kernel_ms == nullptr) return GDN_ERR_NULL;
     int rc = validate_chunk(a);

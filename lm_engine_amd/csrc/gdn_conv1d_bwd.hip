@@ -1,0 +1,198 @@
+// Backward of the depthwise causal convolution (kernel size 2..4, bias, optional SiLU, optional padding mask,
+// optional carried-in state): what autograd computes through DepthwiseCausalConvolution.forward,
+// lm_engine/modeling_utils/depthwise_causal_convolution.py:103-241, when the layer trains.
+//
+// Forward, per channel: xx = [state or zeros (KS - 1 rows) | x * mask], z[s] = bias + sum_j w[j] xx[s + j],
+// y[s] = act(z[s]) * mask[s].  Backward with dz[s] = dy[s] mask[s] act'(z[s]):
+//     dxx[u]  = sum_j w[j] dz[u - j]           dx[t] = mask[t] dxx[t + KS - 1]      dstate[i] = dxx[i]
+//     dw[j]   = sum_{b, s} dz[s] xx[s + j]     dbias = sum_{b, s} dz[s]
+// One pass: a thread owns 8 consecutive channels and walks a block of tokens upward, recomputing z from a
+// sliding window of xx (nothing was saved by the forward), keeping KS partial sums of dxx in flight, and
+// accumulating dw and dbias for its block in registers; the KS - 1 rows of dz past the block's end are recomputed
+// for dx only.  The per-block partial sums of dw and dbias go to a [blocks][C] array each that the caller adds up.
+#include <hip/hip_runtime.h>
+
+#include "gdn_common.h"
+#include "gdn_launch.h"
+
+namespace gdn {
+
+namespace {
+
+constexpr int CB_THREADS = 256;
+constexpr int CB_TOKENS = 64;  // tokens per block of the walk
+constexpr int CB_VEC = 8;
+
+struct ConvBwdParams {
+    const bf16_t* x;
+    const bf16_t* dy;
+    const void* weight;
+    const void* bias;
+    const bf16_t* input_state;
+    const bf16_t* mask;
+    bf16_t* dx;
+    bf16_t* dstate;
+    float* dw_part;  // [B * blocks per row][C][KS]
+    float* db_part;  // [B * blocks per row][C]
+    int64_t x_stride_b, x_stride_s, dy_stride_b, dy_stride_s;
+    int B, S, C;
+    int w_is_bf16;
+};
+
+__device__ __forceinline__ float load_w(const void* w, int is_bf16, int64_t i) {
+    return is_bf16 ? (float)reinterpret_cast<const bf16_t*>(w)[i] : reinterpret_cast<const float*>(w)[i];
+}
+
+template <int KS, bool SILU>
+__global__ __launch_bounds__(CB_THREADS) void causal_conv1d_bwd_kernel(const ConvBwdParams p) {
+    constexpr int VEC = CB_VEC;
+    const int c0 = (blockIdx.x * CB_THREADS + threadIdx.x) * VEC;
+    if (c0 >= p.C) return;
+    const int blocks_per_row = (p.S + CB_TOKENS - 1) / CB_TOKENS;
+    const int b = blockIdx.y / blocks_per_row, blk = blockIdx.y % blocks_per_row;
+    const int s_begin = blk * CB_TOKENS;
+    const int s_own = min(s_begin + CB_TOKENS, p.S);      // dz of [s_begin, s_own) belongs to this block
+    const int s_end = min(s_own + KS - 1, p.S);           // dz up to here feeds dx of this block
+
+    const bf16_t* xb = p.x + (int64_t)b * p.x_stride_b + c0;
+    const bf16_t* dyb = p.dy + (int64_t)b * p.dy_stride_b + c0;
+    const bf16_t* mb = p.mask == nullptr ? nullptr : p.mask + (int64_t)b * p.S;
+    bf16_t* dxb = p.dx + ((int64_t)b * p.S) * p.C + c0;
+
+    float w[VEC][KS], bias[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+#pragma unroll
+        for (int j = 0; j < KS; j++) w[e][j] = load_w(p.weight, p.w_is_bf16, (int64_t)(c0 + e) * KS + j);
+        bias[e] = p.bias == nullptr ? 0.f : load_w(p.bias, p.w_is_bf16, c0 + e);
+    }
+
+    // row s of xx in x's index (s < 0: carried state or zeros)
+    auto load_xx = [&](int s, float (&row)[VEC]) {
+        if (s >= 0) {
+            const bf16x8 v = *reinterpret_cast<const bf16x8*>(xb + (int64_t)s * p.x_stride_s);
+            const float m = mb == nullptr ? 1.f : (float)mb[s];
+#pragma unroll
+            for (int e = 0; e < VEC; e++) row[e] = (float)v[e] * m;
+        } else {
+#pragma unroll
+            for (int e = 0; e < VEC; e++)
+                row[e] = p.input_state == nullptr ? 0.f : (float)p.input_state[((int64_t)b * p.C + c0 + e) * (KS - 1) + (KS - 1) + s];
+        }
+    };
+
+    float win[KS][VEC];   // win[j] = xx row (s - (KS - 1) + j) for the current s
+    float pend[KS][VEC];  // pend[j] = partial dxx of x index (s - (KS - 1) + j)
+    float dw[VEC][KS], db[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+        db[e] = 0.f;
+#pragma unroll
+        for (int j = 0; j < KS; j++) dw[e][j] = 0.f, pend[j][e] = 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < KS - 1; j++) load_xx(s_begin - (KS - 1) + j, win[j + 1]);  // shifted into place by the first step
+
+    for (int s = s_begin; s < s_end; s++) {
+        // slide: win[j] <- win[j + 1], pend likewise (pend[0] of the last step was emitted below)
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+#pragma unroll
+            for (int j = 0; j + 1 < KS; j++) win[j][e] = win[j + 1][e], pend[j][e] = pend[j + 1][e];
+            pend[KS - 1][e] = 0.f;
+        }
+        load_xx(s, win[KS - 1]);
+        const bf16x8 g = *reinterpret_cast<const bf16x8*>(dyb + (int64_t)s * p.dy_stride_s);
+        const float m = mb == nullptr ? 1.f : (float)mb[s];
+        const bool own = s < s_own;
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            float z = bias[e];
+#pragma unroll
+            for (int j = 0; j < KS; j++) z += w[e][j] * win[j][e];
+            float dz = (float)g[e] * m;
+            if (SILU) {
+                const float sg = __builtin_amdgcn_rcpf(1.f + __expf(-z));
+                dz *= sg * (1.f + z * (1.f - sg));
+            }
+#pragma unroll
+            for (int j = 0; j < KS; j++) pend[j][e] += w[e][j] * dz;  // x index s - (KS - 1) + j
+            if (own) {
+                db[e] += dz;
+#pragma unroll
+                for (int j = 0; j < KS; j++) dw[e][j] += dz * win[j][e];
+            }
+        }
+        // x index t = s - (KS - 1) is complete now
+        const int t = s - (KS - 1);
+        if (t >= s_begin) {
+            const float mt = mb == nullptr ? 1.f : (float)mb[t];
+            bf16x8 out;
+#pragma unroll
+            for (int e = 0; e < VEC; e++) out[e] = (bf16_t)(pend[0][e] * mt);
+            *reinterpret_cast<bf16x8*>(dxb + (int64_t)t * p.C) = out;
+        } else if (t < 0 && p.dstate != nullptr) {  // only in the first block of a row
+#pragma unroll
+            for (int e = 0; e < VEC; e++) p.dstate[((int64_t)b * p.C + c0 + e) * (KS - 1) + (KS - 1) + t] = (bf16_t)pend[0][e];
+        }
+    }
+    // the rows still in flight: x indices s_end - (KS - 1) + 1 .. s_end - 1 (complete only at the end of the sequence;
+    // inside it they belong to the next block, which recomputes them)
+    if (s_end == p.S) {
+#pragma unroll
+        for (int j = 1; j < KS; j++) {
+            const int t = s_end - 1 - (KS - 1) + j;
+            if (t >= s_begin && t < s_own) {
+                const float mt = mb == nullptr ? 1.f : (float)mb[t];
+                bf16x8 out;
+#pragma unroll
+                for (int e = 0; e < VEC; e++) out[e] = (bf16_t)(pend[j][e] * mt);
+                *reinterpret_cast<bf16x8*>(dxb + (int64_t)t * p.C) = out;
+            } else if (t < 0 && t >= -(KS - 1) && s_begin == 0 && p.dstate != nullptr) {
+#pragma unroll
+                for (int e = 0; e < VEC; e++) p.dstate[((int64_t)b * p.C + c0 + e) * (KS - 1) + (KS - 1) + t] = (bf16_t)pend[j][e];
+            }
+        }
+    }
+    const int64_t part = (int64_t)blockIdx.y * p.C + c0;
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+        p.db_part[part + e] = db[e];
+#pragma unroll
+        for (int j = 0; j < KS; j++) p.dw_part[(part + e) * KS + j] = dw[e][j];
+    }
+}
+
+template <int KS>
+int launch_ks(const ConvBwdParams& p, bool silu, hipStream_t stream) {
+    const int blocks_per_row = (p.S + CB_TOKENS - 1) / CB_TOKENS;
+    const dim3 grid((unsigned)((p.C / CB_VEC + CB_THREADS - 1) / CB_THREADS), (unsigned)(p.B * blocks_per_row));
+    if (silu) hipLaunchKernelGGL((causal_conv1d_bwd_kernel<KS, true>), grid, dim3(CB_THREADS), 0, stream, p);
+    else hipLaunchKernelGGL((causal_conv1d_bwd_kernel<KS, false>), grid, dim3(CB_THREADS), 0, stream, p);
+    return (int)hipGetLastError();
+}
+
+}  // namespace
+
+int conv_bwd_blocks(int B, int S) { return B * ((S + CB_TOKENS - 1) / CB_TOKENS); }
+
+int launch_conv_bwd(const gdn_conv_bwd_args& a, hipStream_t stream) {
+    ConvBwdParams p;
+    p.x = static_cast<const bf16_t*>(a.x), p.dy = static_cast<const bf16_t*>(a.dy);
+    p.weight = a.weight, p.bias = a.bias;
+    p.input_state = static_cast<const bf16_t*>(a.input_state), p.mask = static_cast<const bf16_t*>(a.mask);
+    p.dx = static_cast<bf16_t*>(a.dx), p.dstate = static_cast<bf16_t*>(a.dstate);
+    p.dw_part = a.dweight_partial, p.db_part = a.dbias_partial;
+    p.x_stride_b = a.x_stride_b, p.x_stride_s = a.x_stride_s, p.dy_stride_b = a.dy_stride_b, p.dy_stride_s = a.dy_stride_s;
+    p.B = a.B, p.S = a.S, p.C = a.C;
+    p.w_is_bf16 = a.w_dtype == GDN_BF16 ? 1 : 0;
+    const bool silu = a.activation == GDN_ACT_SILU;
+    switch (a.kernel_size) {
+        case 2: return launch_ks<2>(p, silu, stream);
+        case 3: return launch_ks<3>(p, silu, stream);
+        case 4: return launch_ks<4>(p, silu, stream);
+        default: return GDN_ERR_UNSUPPORTED;
+    }
+}
+
+}  // namespace gdn

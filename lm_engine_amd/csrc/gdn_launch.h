@@ -20,5 +20,6 @@ bool chunk_bwd_local_supported(const gdn_chunk_local_args& a);
 int launch_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args& a, hipStream_t stream);
 bool chunk_bwd_prepare_supported(const gdn_chunk_bwd_prepare_args& a);
 uint64_t chunk_bwd_record_bytes(const gdn_chunk_bwd_prepare_args& a);
+int launch_conv_bwd(const gdn_conv_bwd_args& a, hipStream_t stream);  // gdn_conv1d_bwd.hip
 
 }  // namespace gdn

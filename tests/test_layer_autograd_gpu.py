@@ -55,6 +55,38 @@ def test_gated_rmsnorm_gradients(gated):
         _compare(got, want, 1e-5, ("do", "dweight"))
 
 
+@pytest.mark.parametrize("S, ks", [(1, 4), (2, 3), (64, 4), (130, 2), (200, 4)])
+@pytest.mark.parametrize("with_state, masked, silu", [(False, False, True), (True, False, True), (False, True, True), (True, True, False)])
+def test_convolution_gradients_bf16_kernel(with_state, masked, silu, S, ks):
+    """bf16 x: the backward is ``gdn_causal_conv1d_bwd``; against autograd through the fp64 oracle on the same
+    (rounded) inputs.  The gradient is taken of y only (the cache state is not differentiated through)."""
+    gen = torch.Generator().manual_seed(100 * S + ks)
+    B, C = 3, 72
+    rt = lambda t: t.to(BF16)  # noqa: E731
+    x, w = rt(torch.randn(B, S, C, generator=gen)), rt(0.5 * torch.randn(C, 1, ks, generator=gen))
+    bias, state = rt(torch.randn(C, generator=gen)), rt(torch.randn(B, C, ks - 1, generator=gen))
+    cy = rt(torch.randn(B, S, C, generator=gen))
+    mask = torch.ones(B, S)
+    if masked and S > 1:
+        mask[1, : S // 3] = 0
+        mask[2, : S - 1] = 0
+    m = mask if masked else None
+    act = "silu" if silu else None
+    tensors = [x, w, bias] + ([state] if with_state else [])
+    oracle = lambda x, w, b, s=None: (depthwise_causal_convolution_ref(x, w, b, s, m, False, act)[0],)  # noqa: E731
+    kernels = lambda x, w, b, s=None: (lm_engine_amd.depthwise_causal_convolution(  # noqa: E731
+        x, w, b, s, None if m is None else m.cuda(), True, act)[0],)  # fmt: skip
+    want = _grads(oracle, [t.to(F64) for t in tensors], [cy.to(F64)])
+    got = _grads(kernels, [t.cuda() for t in tensors], [cy.cuda()])
+    assert [g.dtype for g in got] == [t.dtype for t in tensors]
+    names = ("dx", "dweight", "dbias", "dstate")
+    for name, a, b in zip(names, got, want):
+        if float(b.abs().max()) == 0.0:
+            assert not a.any(), name
+        else:
+            assert rel_l2(a, b) <= 1e-2, f"{name}: rel-L2 {rel_l2(a, b):.3e}"
+
+
 @pytest.mark.parametrize("with_state, masked", [(False, False), (True, False), (False, True)])
 def test_convolution_gradients(with_state, masked):
     gen = torch.Generator().manual_seed(3)
