@@ -356,6 +356,26 @@ typedef struct gdn_norm_args {
 
 int gdn_gated_rmsnorm_fwd(const gdn_norm_args *args, void *stream);
 
+/*
+ * Backward of gdn_gated_rmsnorm_fwd (autograd through `o = o * silu(g)`, `o = self.o_norm(o)`,
+ * module.py:238-242, when the layer trains): given dy [tokens, H, V] (contiguous) it writes d_o and, with a
+ * gate, d_gate (both [tokens, H, V] contiguous, dtype of o), and the partial sums of the gradient of weight
+ * left by each of its `partial_blocks` workgroups, dweight_partial [partial_blocks][V] fp32, which the
+ * caller adds up (also when weight is NULL).
+ */
+typedef struct gdn_norm_bwd_args {
+    const void *o, *gate, *weight, *dy;
+    void *d_o, *d_gate;
+    float *dweight_partial;
+    int64_t o_stride_t, gate_stride_t;
+    int64_t tokens;
+    int32_t H, V;
+    int32_t dtype, w_dtype;
+    float eps;
+    int32_t partial_blocks;
+} gdn_norm_bwd_args;
+int gdn_gated_rmsnorm_bwd(const gdn_norm_bwd_args *args, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

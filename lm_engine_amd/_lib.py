@@ -38,6 +38,7 @@ EXPORTED_SYMBOLS = (
     "gdn_causal_conv1d_bwd",
     "gdn_gates_fwd",
     "gdn_gated_rmsnorm_fwd",
+    "gdn_gated_rmsnorm_bwd",
 )
 
 GDN_CHUNK_KERNELS = 3
@@ -87,6 +88,15 @@ class GdnConvBwdArgs(ctypes.Structure):
                                               "dweight_partial", "dbias_partial")]
         + [(name, ctypes.c_int64) for name in ("x_stride_b", "x_stride_s", "dy_stride_b", "dy_stride_s")]
         + [(name, ctypes.c_int32) for name in ("B", "S", "C", "kernel_size", "w_dtype", "activation")]
+    )  # fmt: skip
+
+
+class GdnNormBwdArgs(ctypes.Structure):
+    _fields_ = (
+        [(name, ctypes.c_void_p) for name in ("o", "gate", "weight", "dy", "d_o", "d_gate", "dweight_partial")]
+        + [(name, ctypes.c_int64) for name in ("o_stride_t", "gate_stride_t", "tokens")]
+        + [(name, ctypes.c_int32) for name in ("H", "V", "dtype", "w_dtype")]
+        + [("eps", ctypes.c_float), ("partial_blocks", ctypes.c_int32)]
     )  # fmt: skip
 
 
@@ -179,6 +189,8 @@ def load_library() -> ctypes.CDLL:
     lib.gdn_chunk_bwd_prepare.restype = ctypes.c_int
     lib.gdn_causal_conv1d_fwd.argtypes = [ctypes.POINTER(GdnConvArgs), ctypes.c_void_p]
     lib.gdn_causal_conv1d_fwd.restype = ctypes.c_int
+    lib.gdn_gated_rmsnorm_bwd.argtypes = [ctypes.POINTER(GdnNormBwdArgs), ctypes.c_void_p]
+    lib.gdn_gated_rmsnorm_bwd.restype = ctypes.c_int
     lib.gdn_causal_conv1d_bwd.argtypes = [ctypes.POINTER(GdnConvBwdArgs), ctypes.c_void_p]
     lib.gdn_causal_conv1d_bwd.restype = ctypes.c_int
     lib.gdn_gates_fwd.argtypes = [ctypes.POINTER(GdnGateArgs), ctypes.c_void_p]

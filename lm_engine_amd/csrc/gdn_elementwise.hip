@@ -126,6 +126,103 @@ static int launch_norm(const NormParams& p, hipStream_t stream) {
     return (int)hipGetLastError();
 }
 
+// Backward of gated_rmsnorm_kernel: with x = o silu(g), r = (mean(x^2) + eps)^-1/2, y = x r w,
+//     dx = r (dy w) - (r^3 / V) x <dy w, x>     do = dx silu(g)     dg = dx o silu'(g)     dw = sum_rows dy x r
+// Same lane mapping; a workgroup walks over row groups with a stride of the grid and leaves its partial sum of
+// dw in dw_part[blockIdx.x][V] (fp32), which the caller adds up.
+struct NormBwdParams {
+    const void* o;
+    const void* gate;
+    const void* weight;
+    const void* dy;
+    void* d_o;
+    void* d_gate;
+    float* dw_part;
+    int64_t o_stride_t, gate_stride_t;
+    int64_t rows;
+    int H, V;
+    float eps;
+};
+
+template <typename T, typename WT, int LPR>
+__global__ __launch_bounds__(256) void gated_rmsnorm_bwd_kernel(const NormBwdParams p) {
+    constexpr int ROWS_PER_BLOCK = 256 / LPR;
+    __shared__ float s_dw[ROWS_PER_BLOCK][LPR * 8];
+    const int sub = threadIdx.x % LPR, slot = threadIdx.x / LPR;
+    const int c = sub * 8;
+    const bool col_live = c < p.V;
+    float w[8], dw[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) w[e] = 1.f, dw[e] = 0.f;
+    if (col_live && p.weight != nullptr) load8(reinterpret_cast<const WT*>(p.weight) + c, w);
+    const int64_t groups = (p.rows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
+    for (int64_t grp = blockIdx.x; grp < groups; grp += gridDim.x) {
+        const int64_t row = grp * ROWS_PER_BLOCK + slot;
+        const bool live = row < p.rows && col_live;
+        const int64_t t = live ? row / p.H : 0;
+        const int h = live ? (int)(row % p.H) : 0;
+        float o[8], g[8], dy[8], x[8], sg[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) o[e] = 0.f, g[e] = 0.f, dy[e] = 0.f, sg[e] = 1.f;
+        if (live) {
+            load8(reinterpret_cast<const T*>(p.o) + t * p.o_stride_t + (int64_t)h * p.V + c, o);
+            load8(reinterpret_cast<const T*>(p.dy) + row * p.V + c, dy);
+            if (p.gate != nullptr) load8(reinterpret_cast<const T*>(p.gate) + t * p.gate_stride_t + (int64_t)h * p.V + c, g);
+        }
+        float ss = 0.f, dot = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            if (p.gate != nullptr) sg[e] = __builtin_amdgcn_rcpf(1.f + __expf(-g[e]));
+            x[e] = p.gate != nullptr ? o[e] * g[e] * sg[e] : o[e];
+            ss += x[e] * x[e];
+            dot += dy[e] * w[e] * x[e];
+        }
+#pragma unroll
+        for (int off = 1; off < LPR; off <<= 1) ss += __shfl_xor(ss, off, WAVE), dot += __shfl_xor(dot, off, WAVE);
+        if (live) {
+            const float r = rsqrtf(ss / (float)p.V + p.eps);
+            const float k = r * r * r * dot / (float)p.V;
+            float d_o[8], d_g[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float dx = r * dy[e] * w[e] - k * x[e];
+                dw[e] += dy[e] * x[e] * r;
+                if (p.gate != nullptr) {
+                    d_o[e] = dx * g[e] * sg[e];
+                    d_g[e] = dx * o[e] * sg[e] * (1.f + g[e] * (1.f - sg[e]));
+                } else {
+                    d_o[e] = dx;
+                }
+            }
+            store8(reinterpret_cast<T*>(p.d_o) + row * p.V + c, d_o);
+            if (p.gate != nullptr) store8(reinterpret_cast<T*>(p.d_gate) + row * p.V + c, d_g);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; e++) s_dw[slot][c + e] = dw[e];
+    __syncthreads();
+    if (slot == 0 && col_live) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            float acc = 0.f;
+            for (int q = 0; q < ROWS_PER_BLOCK; q++) acc += s_dw[q][c + e];
+            p.dw_part[(int64_t)blockIdx.x * p.V + c + e] = acc;
+        }
+    }
+}
+
+template <typename T, typename WT>
+static int launch_norm_bwd(const NormBwdParams& p, int blocks, hipStream_t stream) {
+    int lpr = 8;
+    while (lpr * 8 < p.V) lpr *= 2;
+    const dim3 grid((unsigned)blocks);
+    if (lpr == 8) hipLaunchKernelGGL((gated_rmsnorm_bwd_kernel<T, WT, 8>), grid, dim3(256), 0, stream, p);
+    else if (lpr == 16) hipLaunchKernelGGL((gated_rmsnorm_bwd_kernel<T, WT, 16>), grid, dim3(256), 0, stream, p);
+    else if (lpr == 32) hipLaunchKernelGGL((gated_rmsnorm_bwd_kernel<T, WT, 32>), grid, dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL((gated_rmsnorm_bwd_kernel<T, WT, 64>), grid, dim3(256), 0, stream, p);
+    return (int)hipGetLastError();
+}
+
 }  // namespace gdn
 
 namespace {
@@ -169,4 +266,32 @@ extern "C" int gdn_gated_rmsnorm_fwd(const gdn_norm_args* a, void* stream) {
     const bool wf32 = a->weight == nullptr || a->w_dtype == GDN_F32;
     if (a->dtype == GDN_BF16) return wf32 ? gdn::launch_norm<gdn::bf16_t, float>(p, st) : gdn::launch_norm<gdn::bf16_t, gdn::bf16_t>(p, st);
     return wf32 ? gdn::launch_norm<float, float>(p, st) : gdn::launch_norm<float, gdn::bf16_t>(p, st);
+}
+
+extern "C" int gdn_gated_rmsnorm_bwd(const gdn_norm_bwd_args* a, void* stream) {
+    if (a == nullptr || !a->o || !a->dy || !a->d_o || !a->dweight_partial) return GDN_ERR_NULL;
+    if ((a->gate == nullptr) != (a->d_gate == nullptr)) return GDN_ERR_NULL;
+    if (a->tokens <= 0 || a->H <= 0 || a->V <= 0 || a->partial_blocks <= 0) return GDN_ERR_SHAPE;
+    if (a->V % 8 != 0 || a->V > 512) return GDN_ERR_UNSUPPORTED;
+    if (a->dtype != GDN_BF16 && a->dtype != GDN_F32) return GDN_ERR_UNSUPPORTED;
+    if (a->weight && a->w_dtype != GDN_BF16 && a->w_dtype != GDN_F32) return GDN_ERR_UNSUPPORTED;
+    const int64_t row_elems = (int64_t)a->H * a->V;
+    if (a->o_stride_t < row_elems || (a->gate && a->gate_stride_t < row_elems)) return GDN_ERR_SHAPE;
+    const size_t esz = a->dtype == GDN_BF16 ? 2 : 4;
+    const void* ptrs[] = {a->o, a->dy, a->d_o, a->gate, a->d_gate, a->weight};
+    for (const void* x : ptrs)
+        if (x != nullptr && !aligned_to(x, 16)) return GDN_ERR_ALIGN;
+    if ((a->o_stride_t * esz) % 16 || (a->gate && (a->gate_stride_t * esz) % 16)) return GDN_ERR_ALIGN;
+    gdn::NormBwdParams p;
+    p.o = a->o, p.gate = a->gate, p.weight = a->weight, p.dy = a->dy, p.d_o = a->d_o, p.d_gate = a->d_gate;
+    p.dw_part = a->dweight_partial;
+    p.o_stride_t = a->o_stride_t, p.gate_stride_t = a->gate_stride_t;
+    p.rows = a->tokens * (int64_t)a->H, p.H = a->H, p.V = a->V, p.eps = a->eps;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const bool wf32 = a->weight == nullptr || a->w_dtype == GDN_F32;
+    if (a->dtype == GDN_BF16)
+        return wf32 ? gdn::launch_norm_bwd<gdn::bf16_t, float>(p, a->partial_blocks, st)
+                    : gdn::launch_norm_bwd<gdn::bf16_t, gdn::bf16_t>(p, a->partial_blocks, st);
+    return wf32 ? gdn::launch_norm_bwd<float, float>(p, a->partial_blocks, st)
+                : gdn::launch_norm_bwd<float, gdn::bf16_t>(p, a->partial_blocks, st);
 }

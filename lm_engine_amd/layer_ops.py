@@ -7,7 +7,8 @@
   lm_engine/modeling_utils/normalization.py:69-124.
 
 Both take the (strided) slices of the layer's projections as they are; there is no torch fallback.
-Under autograd their backward differentiates the same formulas written in torch (``_autograd.py``).
+Under autograd the gated norm's backward is one more HIP kernel (``gdn_gated_rmsnorm_bwd``); the gates'
+backward differentiates the same formula written in torch (``_autograd.py``).
 """
 
 from __future__ import annotations
@@ -107,10 +108,58 @@ def gated_rmsnorm(
         return (y.to(o.dtype),)
 
     kernel = lambda o, gate, weight: (_gated_rmsnorm(o, gate, weight, eps),)  # noqa: E731
+    needs_grad = torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (o, gate, weight))
+    if needs_grad and o.is_cuda and o.dtype in (torch.bfloat16, torch.float32):
+        return _GatedRMSNormOnKernels.apply(o, gate, weight, eps)
     return kernel_with_formula_backward(kernel, formula, o, gate, weight)[0]
 
 
-def _gated_rmsnorm(o, gate, weight, eps):
+class _GatedRMSNormOnKernels(torch.autograd.Function):
+    """Forward and backward on the HIP kernels."""
+
+    @staticmethod
+    def forward(ctx, o, gate, weight, eps):
+        ctx.save_for_backward(o, gate, weight)
+        ctx.eps = eps
+        return _gated_rmsnorm(o, gate, weight, eps)
+
+    @staticmethod
+    def backward(ctx, dy):
+        o, gate, weight = ctx.saved_tensors
+        d_o, d_gate, d_weight = _gated_rmsnorm_backward(o, gate, weight, ctx.eps, dy)
+        return d_o, d_gate, d_weight, None
+
+
+def _gated_rmsnorm_backward(o, gate, weight, eps, dy):
+    """``gdn_gated_rmsnorm_bwd``: gradients with respect to o, gate (shaped like gate) and weight."""
+    o2, o_stride, g2, g_stride, H, V = _norm_operands(o, gate)
+    tokens = o2.size(0)
+    dy = dy.to(o.dtype).contiguous()
+    d_o = torch.empty(o.shape, dtype=o.dtype, device=o.device)
+    d_gate = None if gate is None else torch.empty(o.shape, dtype=o.dtype, device=o.device)
+    blocks = min(2048, max(1, (tokens * H * max(V // 8, 8) + 255) // 256))
+    dw_part = torch.empty(blocks, V, dtype=torch.float32, device=o.device)
+    w = None if weight is None else weight.contiguous()
+    args = _lib.GdnNormBwdArgs()
+    args.o, args.dy, args.d_o, args.dweight_partial = o2.data_ptr(), dy.data_ptr(), d_o.data_ptr(), dw_part.data_ptr()
+    args.gate = None if g2 is None else g2.data_ptr()
+    args.d_gate = None if d_gate is None else d_gate.data_ptr()
+    args.weight = None if w is None else w.data_ptr()
+    args.o_stride_t, args.gate_stride_t, args.tokens, args.H, args.V = o_stride, g_stride, tokens, H, V
+    args.dtype = _dtype_code(o.dtype, "o")
+    args.w_dtype = _lib.GDN_F32 if w is None else _dtype_code(w.dtype, "weight")
+    args.eps = float(torch.finfo(o.dtype).eps if eps is None else eps)
+    args.partial_blocks = blocks
+    lib = _lib.load_library()
+    with torch.cuda.device(o.device):
+        stream = ctypes.c_void_p(torch.cuda.current_stream(o.device).cuda_stream)
+        _lib.check_status(lib.gdn_gated_rmsnorm_bwd(ctypes.byref(args), stream), "gdn_gated_rmsnorm_bwd")
+    d_weight = None if weight is None else dw_part.sum(dim=0).to(weight.dtype)
+    return d_o, (None if gate is None else d_gate.reshape(gate.shape)), d_weight
+
+
+def _norm_operands(o, gate):
+    """Token-row views of o and gate for the norm kernels: ``(o2, o_stride, g2, g_stride, H, V)``."""
     _require(o, "o")
     if o.dim() < 2:
         raise ValueError("o must be [..., H, V]")
@@ -129,6 +178,11 @@ def _gated_rmsnorm(o, gate, weight, eps):
             # a slice that starts off a 16-byte boundary (e.g. behind 2 * H gate scalars with H = 2) is compacted
             g2 = g2.contiguous()
             g_stride = H * V
+    return o2, o_stride, g2, g_stride, H, V
+
+
+def _gated_rmsnorm(o, gate, weight, eps):
+    o2, o_stride, g2, g_stride, H, V = _norm_operands(o, gate)
     if weight is not None and tuple(weight.shape) != (V,):
         raise ValueError(f"weight must be [V] = {(V,)}")
     weight = None if weight is None else weight.contiguous()

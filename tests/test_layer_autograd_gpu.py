@@ -23,6 +23,13 @@ def _grads(fn, tensors, cotangents):
     return torch.autograd.grad(loss, leaves)
 
 
+def _grads_allow_unused(fn, tensors, cotangents):
+    leaves = [x.detach().clone().requires_grad_(True) for x in tensors]
+    outs = [o for o in fn(*leaves) if o is not None]
+    loss = sum((o.to(c.dtype) * c).sum() for o, c in zip(outs, cotangents))
+    return torch.autograd.grad(loss, leaves, allow_unused=True)
+
+
 def _compare(got, want, tol, names):
     for name, a, b in zip(names, got, want):
         err = rel_l2(a, b)
@@ -53,6 +60,33 @@ def test_gated_rmsnorm_gradients(gated):
         want = _grads(lambda o, w: (gated_rmsnorm_ref(o, None, w, 1e-5),), [x.to(F64) for x in (o, w)], [c.to(F64)])
         got = _grads(lambda o, w: (lm_engine_amd.gated_rmsnorm(o, None, w, 1e-5),), [x.cuda() for x in (o, w)], [c.cuda()])
         _compare(got, want, 1e-5, ("do", "dweight"))
+
+
+@pytest.mark.parametrize("V, gated, weighted", [(128, True, True), (256, True, False), (64, False, True), (72, True, True)])
+def test_gated_rmsnorm_gradients_bf16(V, gated, weighted):
+    """bf16, gate as a strided slice of a wider projection: the backward is ``gdn_gated_rmsnorm_bwd``."""
+    gen = torch.Generator().manual_seed(V)
+    B, S, H = 2, 33, 3
+    o = torch.randn(B, S, H, V, generator=gen).to(BF16)
+    proj = torch.randn(B, S, 2 * H + H * V, generator=gen).to(BF16)
+    w = (1 + 0.1 * torch.randn(V, generator=gen)).to(BF16)
+    c = torch.randn(B, S, H, V, generator=gen).to(BF16)
+
+    def oracle(o, proj, w):
+        gate = proj[..., 2 * H :] if gated else None
+        return (gated_rmsnorm_ref(o, gate, w if weighted else None, 1e-5),)
+
+    def kernels(o, proj, w):
+        gate = proj[..., 2 * H :] if gated else None
+        return (lm_engine_amd.gated_rmsnorm(o, gate, w if weighted else None, 1e-5),)
+
+    want = _grads_allow_unused(oracle, [t.to(F64) for t in (o, proj, w)], [c.to(F64)])
+    got = _grads_allow_unused(kernels, [t.cuda() for t in (o, proj, w)], [c.cuda()])
+    for name, a, b in zip(("do", "dproj", "dweight"), got, want):
+        if b is None:
+            assert a is None, name
+        else:
+            assert rel_l2(a, b) <= 1e-2, f"{name}: rel-L2 {rel_l2(a, b):.3e}"
 
 
 @pytest.mark.parametrize("S, ks", [(1, 4), (2, 3), (64, 4), (130, 2), (200, 4)])
