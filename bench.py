@@ -328,6 +328,53 @@ def calibrate_copy():
     torch.cuda.synchronize()
 
 
+def bench_layer_backward_kernels(w, steps, warmup):
+    """The backward kernels of the convolution and of the gated norm on the shapes of ``bench_conv`` and
+    ``bench_epilogue``.  HBM-bound: algorithmic bytes = x and dy in, dx out (convolution); o, gate and dy in, d_o and
+    d_gate out (norm).  One pair of events around back-to-back launches, the partial sums' reduction included."""
+    import torch
+
+    from lm_engine_amd.conv import _convolution_backward
+    from lm_engine_amd.layer_ops import _gated_rmsnorm_backward
+
+    def timed(call):
+        for _ in range(warmup):
+            call()
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(steps):
+            call()
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) / steps
+
+    gen = torch.Generator("cpu").manual_seed(4322)
+    C = w.H * (2 * w.K + w.V)
+    x = torch.randn(w.B, w.T, C, generator=gen).to(torch.bfloat16).cuda()
+    dy = torch.randn(w.B, w.T, C, generator=gen).to(torch.bfloat16).cuda()
+    weight = (0.5 * torch.randn(C, 1, 4, generator=gen)).to(torch.bfloat16).cuda()
+    bias = (0.1 * torch.randn(C, generator=gen)).to(torch.bfloat16).cuda()
+    conv_ms = timed(lambda: _convolution_backward(x, weight, bias, None, None, dy, "silu"))
+    conv_gbs = 3 * x.numel() * 2 / (conv_ms * 1e-3) / 1e9
+
+    o = torch.randn(w.B, w.T, w.H, w.V, generator=gen).to(torch.bfloat16).cuda()
+    proj = torch.randn(w.B, w.T, 2 * w.H + w.H * w.V, generator=gen).to(torch.bfloat16).cuda()
+    gate = proj[..., 2 * w.H:]
+    do = torch.randn(w.B, w.T, w.H, w.V, generator=gen).to(torch.bfloat16).cuda()
+    nweight = torch.ones(w.V, dtype=torch.bfloat16, device="cuda")
+    norm_ms = timed(lambda: _gated_rmsnorm_backward(o, gate, nweight, 1e-5, do))
+    norm_gbs = 5 * o.numel() * 2 / (norm_ms * 1e-3) / 1e9
+    return {
+        "conv": {"workload": f"conv1d_k4_silu_bf16 backward B={w.B} S={w.T} C={C}", "ms": round(conv_ms, 4),
+                 "roofline": {"kernel": "causal_conv1d_bwd_kernel", "bound": "hbm", "achieved": round(conv_gbs, 1),
+                              "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(conv_gbs / HBM_PEAK_GBS, 4), "traffic": None}},
+        "norm": {"workload": f"gated_rmsnorm_bf16 backward B={w.B} T={w.T} H={w.H} V={w.V}", "ms": round(norm_ms, 4),
+                 "roofline": {"kernel": "gated_rmsnorm_bwd_kernel", "bound": "hbm", "achieved": round(norm_gbs, 1),
+                              "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(norm_gbs / HBM_PEAK_GBS, 4), "traffic": None}},
+    }  # fmt: skip
+
+
 def bench_backward(w, inp, steps, warmup):
     """One backward pass of the chunked operator on the same workload (``lm_engine_amd.backward``), gradient
     of the output only.  Wall time per call with the device idle before and after."""
@@ -383,6 +430,8 @@ def main():
     conv = None if args.no_decode else bench_conv(w, args.steps, args.warmup)
     epilogue = None if args.no_decode else bench_epilogue(w, args.steps, args.warmup)
     backward = None if args.no_decode else bench_backward(w, inp, args.steps, args.warmup)
+    if backward is not None:
+        backward["layer_kernels"] = bench_layer_backward_kernels(w, args.steps, args.warmup)
     baseline = None if args.no_cpu_baseline else cpu_baseline(w, inp, args.cpu_seconds)
     if args.calibrate_copy:
         calibrate_copy()
