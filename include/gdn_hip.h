@@ -288,8 +288,8 @@ int gdn_causal_conv1d_fwd(const gdn_conv_args *args, void *stream);
  * DepthwiseCausalConvolution.forward, depthwise_causal_convolution.py:103-241, when the layer trains):
  * given dy [B, S, C] (element strides) it recomputes the pre-activation from x and writes dx [B, S, C]
  * (bf16, contiguous), dstate [B, C, kernel_size - 1] (bf16; NULL when there was no input_state) and, per
- * block of 64 tokens of a row, the partial sums of the gradients of weight and bias:
- * dweight_partial [B * ceil(S / 64)][C][kernel_size] and dbias_partial [B * ceil(S / 64)][C], fp32, which
+ * block of tokens_per_block (8 .. 4096) tokens of a row, the partial sums of the gradients of weight and bias:
+ * dweight_partial [B * ceil(S / tokens_per_block)][C][kernel_size] and dbias_partial [same][C], fp32, which
  * the caller adds up over the first dim.  The gradient flowing into final_state is not handled (the layer
  * does not differentiate through its cache).
  */
@@ -302,6 +302,8 @@ typedef struct gdn_conv_bwd_args {
     int32_t B, S, C, kernel_size;
     int32_t w_dtype;    /* gdn_dtype of weight and bias */
     int32_t activation; /* gdn_activation */
+    int32_t tokens_per_block;
+    int32_t reserved;
 } gdn_conv_bwd_args;
 int gdn_causal_conv1d_bwd(const gdn_conv_bwd_args *args, void *stream);
 

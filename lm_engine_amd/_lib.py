@@ -87,7 +87,8 @@ class GdnConvBwdArgs(ctypes.Structure):
         [(name, ctypes.c_void_p) for name in ("x", "dy", "weight", "bias", "input_state", "mask", "dx", "dstate",
                                               "dweight_partial", "dbias_partial")]
         + [(name, ctypes.c_int64) for name in ("x_stride_b", "x_stride_s", "dy_stride_b", "dy_stride_s")]
-        + [(name, ctypes.c_int32) for name in ("B", "S", "C", "kernel_size", "w_dtype", "activation")]
+        + [(name, ctypes.c_int32) for name in ("B", "S", "C", "kernel_size", "w_dtype", "activation", "tokens_per_block",
+                                               "reserved")]
     )  # fmt: skip
 
 

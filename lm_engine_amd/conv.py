@@ -72,11 +72,14 @@ def depthwise_causal_convolution(
     return kernel_with_formula_backward(kernel, formula, x, weight, bias, input_state)
 
 
+_BWD_TOKENS_PER_BLOCK = 64  # tokens a thread of the backward kernel walks over (16: 0.36 ms, 32: 0.27, 64: 0.22, 128: 0.28 at 4 x 4096 x 6144)
+
+
 def _backward_kernel_applies(x, weight, activation) -> bool:
     if not x.is_cuda or x.dtype != torch.bfloat16 or activation not in _IN_KERNEL_ACTIVATIONS or x.dim() != 3:
         return False
     B, S, C = x.shape
-    return C % 8 == 0 and weight.dtype in (torch.bfloat16, torch.float32) and B * (-(-S // 64)) <= 65535
+    return C % 8 == 0 and weight.dtype in (torch.bfloat16, torch.float32) and B * (-(-S // _BWD_TOKENS_PER_BLOCK)) <= 65535
 
 
 class _ConvolutionOnKernels(torch.autograd.Function):
@@ -117,7 +120,7 @@ def _convolution_backward(x, weight, bias, input_state, attention_mask, dy, acti
     mask = None
     if attention_mask is not None and attention_mask.shape[1] > 1 and attention_mask.shape[0] > 1:
         mask = attention_mask.to(x.dtype).contiguous()
-    blocks = B * (-(-S // 64))
+    blocks = B * (-(-S // _BWD_TOKENS_PER_BLOCK))
     dx = torch.empty(B, S, C, dtype=x.dtype, device=x.device)
     dstate = None if state is None else torch.empty(B, C, ks - 1, dtype=x.dtype, device=x.device)
     dw_part = torch.empty(blocks, C, ks, dtype=torch.float32, device=x.device)
@@ -130,7 +133,7 @@ def _convolution_backward(x, weight, bias, input_state, attention_mask, dy, acti
     a.dstate = None if dstate is None else dstate.data_ptr()
     a.dweight_partial, a.dbias_partial = dw_part.data_ptr(), db_part.data_ptr()
     a.x_stride_b, a.x_stride_s, a.dy_stride_b, a.dy_stride_s = x.stride(0), x.stride(1), dy.stride(0), dy.stride(1)
-    a.B, a.S, a.C, a.kernel_size = B, S, C, ks
+    a.B, a.S, a.C, a.kernel_size, a.tokens_per_block = B, S, C, ks, _BWD_TOKENS_PER_BLOCK
     a.w_dtype = _dtype_code(w2.dtype, "weight")
     a.activation = _IN_KERNEL_ACTIVATIONS[activation]
     with torch.cuda.device(x.device):

@@ -174,7 +174,8 @@ int gdn_causal_conv1d_bwd(const gdn_conv_bwd_args* a, void* stream) {
     const int64_t strides[] = {a->x_stride_b, a->x_stride_s, a->dy_stride_b, a->dy_stride_s};
     for (int64_t s : strides)
         if (s < 0 || s % 8 != 0) return GDN_ERR_ALIGN;
-    if ((int64_t)a->B * ((a->S + 63) / 64) > 65535) return GDN_ERR_UNSUPPORTED;  // one grid row per 64 tokens
+    if (a->tokens_per_block < 8 || a->tokens_per_block > 4096) return GDN_ERR_SHAPE;
+    if ((int64_t)a->B * ((a->S + a->tokens_per_block - 1) / a->tokens_per_block) > 65535) return GDN_ERR_UNSUPPORTED;  // one grid row per block
     return gdn::launch_conv_bwd(*a, static_cast<hipStream_t>(stream));
 }
 

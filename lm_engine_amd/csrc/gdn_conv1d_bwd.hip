@@ -20,7 +20,6 @@ namespace gdn {
 namespace {
 
 constexpr int CB_THREADS = 256;
-constexpr int CB_TOKENS = 64;  // tokens per block of the walk
 constexpr int CB_VEC = 8;
 
 struct ConvBwdParams {
@@ -37,6 +36,7 @@ struct ConvBwdParams {
     int64_t x_stride_b, x_stride_s, dy_stride_b, dy_stride_s;
     int B, S, C;
     int w_is_bf16;
+    int tokens_per_block;  // tokens per block of the walk
 };
 
 __device__ __forceinline__ float load_w(const void* w, int is_bf16, int64_t i) {
@@ -48,10 +48,10 @@ __global__ __launch_bounds__(CB_THREADS) void causal_conv1d_bwd_kernel(const Con
     constexpr int VEC = CB_VEC;
     const int c0 = (blockIdx.x * CB_THREADS + threadIdx.x) * VEC;
     if (c0 >= p.C) return;
-    const int blocks_per_row = (p.S + CB_TOKENS - 1) / CB_TOKENS;
+    const int blocks_per_row = (p.S + p.tokens_per_block - 1) / p.tokens_per_block;
     const int b = blockIdx.y / blocks_per_row, blk = blockIdx.y % blocks_per_row;
-    const int s_begin = blk * CB_TOKENS;
-    const int s_own = min(s_begin + CB_TOKENS, p.S);      // dz of [s_begin, s_own) belongs to this block
+    const int s_begin = blk * p.tokens_per_block;
+    const int s_own = min(s_begin + p.tokens_per_block, p.S);      // dz of [s_begin, s_own) belongs to this block
     const int s_end = min(s_own + KS - 1, p.S);           // dz up to here feeds dx of this block
 
     const bf16_t* xb = p.x + (int64_t)b * p.x_stride_b + c0;
@@ -165,7 +165,7 @@ __global__ __launch_bounds__(CB_THREADS) void causal_conv1d_bwd_kernel(const Con
 
 template <int KS>
 int launch_ks(const ConvBwdParams& p, bool silu, hipStream_t stream) {
-    const int blocks_per_row = (p.S + CB_TOKENS - 1) / CB_TOKENS;
+    const int blocks_per_row = (p.S + p.tokens_per_block - 1) / p.tokens_per_block;
     const dim3 grid((unsigned)((p.C / CB_VEC + CB_THREADS - 1) / CB_THREADS), (unsigned)(p.B * blocks_per_row));
     if (silu) hipLaunchKernelGGL((causal_conv1d_bwd_kernel<KS, true>), grid, dim3(CB_THREADS), 0, stream, p);
     else hipLaunchKernelGGL((causal_conv1d_bwd_kernel<KS, false>), grid, dim3(CB_THREADS), 0, stream, p);
@@ -173,8 +173,6 @@ int launch_ks(const ConvBwdParams& p, bool silu, hipStream_t stream) {
 }
 
 }  // namespace
-
-int conv_bwd_blocks(int B, int S) { return B * ((S + CB_TOKENS - 1) / CB_TOKENS); }
 
 int launch_conv_bwd(const gdn_conv_bwd_args& a, hipStream_t stream) {
     ConvBwdParams p;
@@ -186,6 +184,7 @@ int launch_conv_bwd(const gdn_conv_bwd_args& a, hipStream_t stream) {
     p.x_stride_b = a.x_stride_b, p.x_stride_s = a.x_stride_s, p.dy_stride_b = a.dy_stride_b, p.dy_stride_s = a.dy_stride_s;
     p.B = a.B, p.S = a.S, p.C = a.C;
     p.w_is_bf16 = a.w_dtype == GDN_BF16 ? 1 : 0;
+    p.tokens_per_block = a.tokens_per_block;
     const bool silu = a.activation == GDN_ACT_SILU;
     switch (a.kernel_size) {
         case 2: return launch_ks<2>(p, silu, stream);
