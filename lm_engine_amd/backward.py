@@ -54,8 +54,16 @@ def _chains(B, T, cu_seqlens, left_padded):
     """Start (in the flattened [B * T] token axis) and length of every sequence."""
     if cu_seqlens is None:
         return [b * T for b in range(B)], [T] * B
+    # The layout of the packed gradients depends on the longest sequence, so the prefix has to come to the host
+    # (one copy of N + 1 integers per backward).  It is checked here, where it is visible: the forward kernels
+    # clamp a malformed prefix, the index arithmetic below would not.
     cu = cu_seqlens.detach().to("cpu", torch.int64).tolist()
+    limit = B * T if left_padded else T
+    if cu[0] != 0 or any(cu[n + 1] < cu[n] for n in range(len(cu) - 1)) or cu[-1] > limit:
+        raise ValueError(f"cu_seqlens must start at 0, be non-decreasing and end at or below {limit}, got {cu}")
     lens = [cu[n + 1] - cu[n] for n in range(len(cu) - 1)]
+    if left_padded and max(lens) > T:
+        raise ValueError(f"a left-padded row holds at most T = {T} tokens, got lengths {lens}")
     if left_padded:
         return [b * T + T - lens[b] for b in range(B)], lens
     return cu[:-1], lens

@@ -74,14 +74,22 @@ uint64_t chunk_workspace_bytes(const gdn_args& a) {
 // ------------------------------------------------------------------------------------------
 // chunk offsets of packed sequences: chunk_off[n] = sum_{m < n} ceil(len_m / C)
 // ------------------------------------------------------------------------------------------
+// Lengths are taken through packed_bounds, and the running total is capped at the number of record slots
+// the workspace holds (`slots`): whatever cu_seqlens contains, no chunk gets a slot outside the workspace
+// (sequences past the cap get none; a well-formed prefix never reaches it).
 __global__ __launch_bounds__(256) void chunk_offsets_kernel(const int32_t* __restrict__ cu, int32_t* __restrict__ off,
-                                                            int N) {
+                                                            int N, int total, int slots) {
     __shared__ int s_part[256];
     const int tid = threadIdx.x;
     const int per = (N + 255) / 256;
     const int begin = min(tid * per, N), end = min(begin + per, N);
+    auto chunks_of = [&](int n) {
+        int t0, len;
+        packed_bounds(cu, n, total, t0, len);
+        return (len + C - 1) / C;
+    };
     int sum = 0;
-    for (int n = begin; n < end; n++) sum += (cu[n + 1] - cu[n] + C - 1) / C;
+    for (int n = begin; n < end; n++) sum = min(sum + chunks_of(n), slots);
     s_part[tid] = sum;
     __syncthreads();
     if (tid == 0) {
@@ -89,7 +97,7 @@ __global__ __launch_bounds__(256) void chunk_offsets_kernel(const int32_t* __res
         for (int i = 0; i < 256; i++) {
             const int x = s_part[i];
             s_part[i] = run;
-            run += x;
+            run = min(run + x, slots);
         }
         off[N] = run;
     }
@@ -97,7 +105,7 @@ __global__ __launch_bounds__(256) void chunk_offsets_kernel(const int32_t* __res
     int run = s_part[tid];
     for (int n = begin; n < end; n++) {
         off[n] = run;
-        run += (cu[n + 1] - cu[n] + C - 1) / C;
+        run = min(run + chunks_of(n), slots);
     }
 }
 
@@ -468,7 +476,9 @@ __global__ __launch_bounds__(NW* WAVE) void chunk_scan_kernel(const ChunkParams 
         b = n, seq_t0 = p.T - seq_len;
     } else {
         slot_begin = p.chunk_off[n], slot_end = p.chunk_off[n + 1];
-        b = 0, seq_t0 = p.cu_seqlens[n], seq_len = p.cu_seqlens[n + 1] - seq_t0;
+        int t0, len;
+        packed_bounds(p.cu_seqlens, n, p.T, t0, len);
+        b = 0, seq_t0 = t0, seq_len = min(len, (slot_end - slot_begin) * C);
     }
 
     // state: tile t holds rows 16 t + 4 lq + e, column 16 tn + l16
@@ -640,7 +650,7 @@ int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events, 
     };
     mark(0);
     if (p.cu_seqlens != nullptr) {
-        hipLaunchKernelGGL(chunk_offsets_kernel, dim3(1), dim3(256), 0, stream, p.cu_seqlens, p.chunk_off, p.N);
+        hipLaunchKernelGGL(chunk_offsets_kernel, dim3(1), dim3(256), 0, stream, p.cu_seqlens, p.chunk_off, p.N, p.T, p.TC);
         if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
     }
     mark(1);

@@ -667,7 +667,9 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
         b = n, seq_t0 = p.T - seq_len;
     } else {
         slot_begin = p.chunk_off[n], slot_end = p.chunk_off[n + 1];
-        b = 0, seq_t0 = p.cu_seqlens[n], seq_len = p.cu_seqlens[n + 1] - seq_t0;
+        int t0, len;
+        packed_bounds(p.cu_seqlens, n, p.T, t0, len);
+        b = 0, seq_t0 = t0, seq_len = min(len, (slot_end - slot_begin) * C);
     }
     const int nchunks = slot_end - slot_begin;
     const uint8_t* rec = p.rec + ((int64_t)h * p.TC + slot_begin) * p.rec_bytes;

@@ -115,8 +115,10 @@ __device__ __forceinline__ ChunkCoord locate_chunk(const ChunkParams& p, int slo
     }
     cc.n = lo;
     const int c = slot - p.chunk_off[lo];
-    cc.t0 = (int64_t)p.cu_seqlens[lo] + (int64_t)c * C;
-    cc.len = min(C, p.cu_seqlens[lo + 1] - (int)cc.t0);
+    int t0, len;
+    packed_bounds(p.cu_seqlens, lo, p.T, t0, len);
+    cc.t0 = (int64_t)t0 + (int64_t)c * C;
+    cc.len = min(C, len - c * C);
     return cc;
 }
 

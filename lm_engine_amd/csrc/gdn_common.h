@@ -73,6 +73,15 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, f32x4 x) {
     *reinterpret_cast<bf16x4*>(p) = r;
 }
 
+// Packed sequences: first token and length of sequence n from cu_seqlens, which lives on the device and is
+// never seen by the host-side checks: clamped into [0, total] and made non-negative, so that a malformed
+// prefix (decreasing, or running past the packed token count) gives short or empty sequences and never
+// an address outside the tensors.
+__device__ __forceinline__ void packed_bounds(const int32_t* cu, int n, int total, int& t0, int& len) {
+    t0 = min(max(cu[n], 0), total);
+    len = min(max(cu[n + 1], t0), total) - t0;
+}
+
 // beta / g are per (token, head) scalars; beta may be bf16 or fp32, NULL means 1.
 __device__ __forceinline__ float load_beta(const void* beta, int beta_dtype, int64_t idx) {
     if (beta == nullptr) return 1.0f;

@@ -53,7 +53,10 @@ __global__ __launch_bounds__(REC_THREADS) void recurrent_kernel(const RecurrentP
     static_assert(K % ROWG == 0 && RPT >= 1, "tile does not divide over the workgroup");
     static_assert(K % WAVE == 0, "K must be a multiple of the wave size");
 
-    __shared__ __attribute__((aligned(16))) float s_k[K];
+    // k^ is read again after the second barrier of a token (the rank-1 update) while wave 0 may already be
+    // staging the next token: two buffers, alternating by token.  q^ and k^ . q^ are only read between the
+    // two barriers, where wave 0 cannot have moved on.
+    __shared__ __attribute__((aligned(16))) float s_k2[2][K];
     __shared__ __attribute__((aligned(16))) float s_q[K];
     __shared__ float s_kq[1];
     __shared__ __attribute__((aligned(16))) float s_red[REC_WAVES][LANES_V][8];
@@ -70,9 +73,9 @@ __global__ __launch_bounds__(REC_THREADS) void recurrent_kernel(const RecurrentP
     int64_t b = n, t_begin = 0, t_end = p.T;
     if (p.pad_lens != nullptr) t_begin = p.T - min(max(p.pad_lens[n + 1] - p.pad_lens[n], 0), p.T);  // the last tokens of row n
     if (p.cu_seqlens != nullptr) {
-        b = 0;
-        t_begin = p.cu_seqlens[n];
-        t_end = p.cu_seqlens[n + 1];
+        int t0, len;
+        packed_bounds(p.cu_seqlens, n, p.T, t0, len);
+        b = 0, t_begin = t0, t_end = t0 + len;
     }
 
     const int64_t state_off = (((int64_t)n * p.H + h) * K + (int64_t)rg * RPT) * p.V + v0;
@@ -92,6 +95,7 @@ __global__ __launch_bounds__(REC_THREADS) void recurrent_kernel(const RecurrentP
     T* op = reinterpret_cast<T*>(p.o) + b * p.o_stride_b + h * p.o_stride_h + v0;
 
     for (int64_t t = t_begin; t < t_end; t++) {
+        float* const s_k = s_k2[(t - t_begin) & 1];
         // ---- wave 0 stages k^ and q^ (normalised, q scaled) in LDS; others go straight on ----
         if (wave == 0) {
             float kx[KPL], qx[KPL];
