@@ -110,6 +110,20 @@ uint64_t gdn_workspace_bytes(const gdn_args *args);
 int gdn_chunk_fwd(const gdn_args *args, void *stream);
 
 /*
+ * gdn_chunk_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  args->workspace and
+ * args->workspace_bytes are ignored: the chunk records go to a scratch array that is part of the library's
+ * device code (GDN_NOALLOC_SCRATCH_BYTES per device the library runs on, held until the process ends), and the
+ * call makes no hipMalloc, hipFree or other allocating call.  Shapes with gdn_workspace_bytes(args) above that
+ * size are rejected with GDN_ERR_WORKSPACE.  Results are bit-identical to gdn_chunk_fwd's.  Every call on a
+ * device shares that device's array: calls that overlap on one device (different streams or threads) race;
+ * calls on one stream are ordered and safe.  The first call on a device looks the array's address up
+ * (hipGetSymbolAddress), which may load the code object: make that call outside any capture.
+ */
+#define GDN_NOALLOC_SCRATCH_BYTES (64u << 20)
+int gdn_chunk_fwd_noalloc(const gdn_args *args, void *stream);
+
+/*
  * Token-by-token recurrence with the state tile held in registers; T may be any length and
  * q/k/v may be bf16 or fp32.  With T == 1 this is the decode step: one read and one write
  * of the fp32 state, in place when GDN_FLAG_STATE_INPLACE is set and ht == h0.

@@ -19,6 +19,8 @@ GDN_FLAG_L2NORM = 1
 GDN_FLAG_STATE_INPLACE = 2
 GDN_FLAG_LEFT_PADDED = 4
 
+GDN_NOALLOC_SCRATCH_BYTES = 64 << 20  # built-in workspace of gdn_chunk_fwd_noalloc
+
 GDN_ACT_NONE = 0
 GDN_ACT_SILU = 1
 
@@ -29,6 +31,7 @@ EXPORTED_SYMBOLS = (
     "gdn_strerror",
     "gdn_workspace_bytes",
     "gdn_chunk_fwd",
+    "gdn_chunk_fwd_noalloc",
     "gdn_recurrent_fwd",
     "gdn_chunk_fwd_profile",
     "gdn_chunk_fwd_saving",
@@ -178,6 +181,8 @@ def load_library() -> ctypes.CDLL:
     lib.gdn_workspace_bytes.restype = ctypes.c_uint64
     lib.gdn_chunk_fwd.argtypes = [ctypes.POINTER(GdnArgs), ctypes.c_void_p]
     lib.gdn_chunk_fwd.restype = ctypes.c_int
+    lib.gdn_chunk_fwd_noalloc.argtypes = [ctypes.POINTER(GdnArgs), ctypes.c_void_p]
+    lib.gdn_chunk_fwd_noalloc.restype = ctypes.c_int
     lib.gdn_recurrent_fwd.argtypes = [ctypes.POINTER(GdnArgs), ctypes.c_void_p]
     lib.gdn_recurrent_fwd.restype = ctypes.c_int
     lib.gdn_chunk_fwd_profile.argtypes = [ctypes.POINTER(GdnArgs), ctypes.c_void_p, ctypes.POINTER(ctypes.c_float)]

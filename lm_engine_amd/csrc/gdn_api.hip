@@ -1,13 +1,43 @@
 // C ABI of libgdn_hip.so (declared in include/gdn_hip.h): argument validation and dispatch.
-// Everything that can fault a kernel (shapes, strides, alignment, workspace size) is checked
-// here on the host before any launch.
+// Everything the host can see that could fault a kernel (shapes, strides, alignment, workspace size) is
+// checked here before any launch.  The contents of cu_seqlens live on the device and are not: the kernels
+// clamp them (packed_bounds, and the slot cap of chunk_offsets_kernel), so a malformed prefix gives wrong
+// sequences but no access outside the caller's tensors or the workspace.
 
 #include <hip/hip_runtime.h>
+
+#include <mutex>
 
 #include "gdn_hip.h"
 #include "gdn_launch.h"
 
+// Workspace of gdn_chunk_fwd_noalloc: device memory that belongs to the library's code object, so that the entry
+// point has nothing to allocate.  Every device the library runs on holds its own copy, at its own address, until
+// the process ends.  Host code never passes this name to a kernel (on the host it is a stand-in, not a device
+// address): noalloc_scratch() below asks the runtime for the address once per device and hands that out.
+static __device__ __align__(256) unsigned char scratch[GDN_NOALLOC_SCRATCH_BYTES];
+
 namespace {
+
+constexpr int MAX_DEVICES = 64;
+std::mutex scratch_mutex;
+void* scratch_ptr[MAX_DEVICES] = {};
+
+// Address of `scratch` on the calling thread's current device; looked up on the first call per device.
+int noalloc_scratch(void** out) {
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= MAX_DEVICES) return GDN_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        if (hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)); e != hipSuccess) return (int)e;
+        if (ptr == nullptr) return (int)hipErrorInvalidSymbol;
+        scratch_ptr[dev] = ptr;
+    }
+    *out = scratch_ptr[dev];
+    return GDN_OK;
+}
 
 inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
@@ -59,7 +89,8 @@ const char* gdn_strerror(int status) {
             return "unsupported configuration (need K in {64,128,256}, V % 32 == 0, bf16/fp32; chunked forward: "
                    "bf16, chunk 64)";
         case GDN_ERR_ALIGN: return "pointer or stride not 16-byte aligned";
-        case GDN_ERR_WORKSPACE: return "workspace missing or too small";
+        case GDN_ERR_WORKSPACE:
+            return "workspace missing or too small (gdn_chunk_fwd_noalloc: the shape needs more than its built-in scratch)";
         case GDN_ERR_VARLEN: return "cu_seqlens requires B == 1 (packed) or GDN_FLAG_LEFT_PADDED";
         default: break;
     }
@@ -91,6 +122,22 @@ int gdn_chunk_fwd(const gdn_args* a, void* stream) {
     const int rc = validate_chunk(a);
     if (rc != GDN_OK) return rc;
     return gdn::launch_chunk_fwd(*a, static_cast<hipStream_t>(stream));
+}
+
+int gdn_chunk_fwd_noalloc(const gdn_args* a, void* stream) {
+    int rc = validate_common(a);
+    if (rc != GDN_OK) return rc;
+    if (!gdn::chunk_shape_supported(*a)) return GDN_ERR_UNSUPPORTED;
+    if (gdn::chunk_workspace_bytes(*a) > (uint64_t)GDN_NOALLOC_SCRATCH_BYTES) return GDN_ERR_WORKSPACE;
+    void* ptr = nullptr;
+    rc = noalloc_scratch(&ptr);
+    if (rc != GDN_OK) return rc;
+    // Nothing in the workspace has to start at zero: the offsets kernel and prepare write every word the
+    // scan reads.  The same array serves every call on this device.
+    gdn_args b = *a;
+    b.workspace = ptr;
+    b.workspace_bytes = (uint64_t)GDN_NOALLOC_SCRATCH_BYTES;
+    return gdn::launch_chunk_fwd(b, static_cast<hipStream_t>(stream));
 }
 
 int gdn_chunk_fwd_saving(const gdn_args* a, const gdn_chunk_saves* saves, void* stream) {

@@ -221,3 +221,17 @@ def test_fla_shim_resolves_the_reference_imports():
     finally:
         uninstall_fla_shim()
     assert "fla" not in sys.modules
+
+
+def test_noalloc_entry_point_rejects_shapes_beyond_its_scratch():
+    lib = _lib.load_library()
+    args = _lib.GdnArgs()
+    args.q = args.k = args.v = args.o = 0x1000
+    args.B, args.T, args.H, args.K, args.V, args.N = 8, 8192, 16, 128, 128, 8
+    args.chunk, args.dtype, args.beta_dtype, args.scale = 64, _lib.GDN_BF16, _lib.GDN_BF16, 1.0
+    for name in ("q", "k", "v", "o"):
+        setattr(args, f"{name}_stride_b", 8192 * 16 * 128)
+        setattr(args, f"{name}_stride_t", 16 * 128)
+        setattr(args, f"{name}_stride_h", 128)
+    assert lib.gdn_workspace_bytes(ctypes.byref(args)) > _lib.GDN_NOALLOC_SCRATCH_BYTES
+    assert lib.gdn_chunk_fwd_noalloc(ctypes.byref(args), None) == -5  # GDN_ERR_WORKSPACE, before any launch
