@@ -42,36 +42,12 @@
 
 #include <type_traits>
 
-#include "gdn_chunk_common.h"
+#include <stdlib.h>
+
+#include "gdn_chunk32_common.h"
 #include "gdn_launch.h"
 
 namespace gdn {
-
-typedef __attribute__((ext_vector_type(4))) short s16x4;
-
-__device__ __forceinline__ bf16x8 pack8_16(const f32x16& d, int s, float sign) {
-    bf16x8 r;
-#pragma unroll
-    for (int e = 0; e < 8; e++) r[e] = (bf16_t)(sign * d[8 * s + e]);
-    return r;
-}
-
-// 4 consecutive rows x 16 consecutive columns of a row-major bf16 LDS matrix, transposed on the
-// way in: lane i of each 16-lane group receives M[row0 + 0..3][col0 + i].
-// With SWAP, the two middle groups of 4 columns change places: lane i receives column col0 + sigma(i),
-// sigma(4 q + b) = 4 swap(q) + b, swap(1) = 2, swap(2) = 1 (the column order of the scan's state slices).
-template <bool SWAP = false>
-__device__ __forceinline__ bf16x4 lds_read_tr4x16(const bf16_t* m, int ld, int row0, int col0, int l16) {
-    const int q = l16 % 4;
-    const int piece = SWAP ? ((q & 1) << 1 | (q >> 1)) : q;
-    const bf16_t* p = m + (row0 + l16 / 4) * ld + col0 + 4 * piece;
-    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p);
-    return __builtin_bit_cast(bf16x4, v);
-}
-
-// Column of a 32-column state slice held by lane l32 (the order lds_read_tr4x16<true> produces): with it,
-// register pair (2 m, 2 m + 1) of a transposed accumulator tile covers 8 consecutive columns per lane.
-__device__ __forceinline__ int slice_col(int l32) { return (l32 & 0x13) | ((l32 & 4) << 1) | ((l32 & 8) >> 1); }
 
 // x of another lane as named by a DPP control word; lanes the move does not write (outside ROW_MASK, or shifted in
 // from outside their row) get 0
@@ -486,23 +462,6 @@ constexpr int SCAN_LOADERS = 4;
 //   NW = 2:  0 1 compute | 2 3 loaders | 4 output store | 5 exits at once | 6 7 loaders
 //   NW = 4:  0..3 compute | 4..7 loaders (each compute wave shares with one loader; no output wave)
 __host__ __device__ constexpr int scan_waves(int nw) { return nw == 1 ? 6 : 8; }
-
-// compile-time loop: f(std::integral_constant<int, I>{}) for I = B .. E - 1
-template <int B, int E, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-    if constexpr (B < E) {
-        f(std::integral_constant<int, B>{});
-        static_for<B + 1, E>(f);
-    }
-}
-
-// keeps the computation of x at this point of the program
-__device__ __forceinline__ void pin_regs(bf16x8& x) {
-    typedef __attribute__((ext_vector_type(4))) int i32x4;
-    i32x4 t = __builtin_bit_cast(i32x4, x);
-    asm volatile("" : "+v"(t));
-    x = __builtin_bit_cast(bf16x8, t);
-}
 
 // Order of the MFMAs of one chunk in the scan's compute wave, and where its side work goes.
 //
@@ -1092,13 +1051,16 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
 // ------------------------------------------------------------------------------------------
 // launch
 // ------------------------------------------------------------------------------------------
+int launch_scan_pair(ChunkParams& p, int K, hipStream_t stream, int ns, bool save);  // gdn_chunk_pair.hip
+bool scan_pair_supported(int K, int V, int ns);
+
 template <int K>
 static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int num_cus) {
     const int64_t items = (int64_t)((p.TC + 7) / 8) * 8 * p.H;  // a multiple of 8, see the kernel
     const int64_t cap = (int64_t)(3 * num_cus + 7) / 8 * 8;      // three workgroups per CU (LDS and registers allow it)
     if (items >= ((int64_t)1 << 31)) return GDN_ERR_UNSUPPORTED;  // the kernel counts items in 32 bits
     const int grid_prep = (int)(items < cap ? items : cap);
-    if (!p.records_given) {
+    if (!p.records_given && getenv("GDN_SKIP_PREPARE") == nullptr) {
         hipLaunchKernelGGL((chunk_prepare32_kernel<K>), dim3(grid_prep), dim3(PREP_THREADS), 0, stream, p);
         if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
     }
@@ -1113,6 +1075,15 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     int nw = 1;
     while (nw < 4 && vtiles % (2 * nw) == 0 && chains * (vtiles / nw) > (int64_t)num_cus) nw *= 2;
     const bool save = p.save_state != nullptr || p.save_vnew != nullptr;
+    {
+        // experiment switch: GDN_SCAN=p1 / p2 runs the scan with two compute waves per slice, 1 or 2 slices per workgroup
+        const char* mode = getenv("GDN_SCAN");
+        if (mode != nullptr && mode[0] == 'n') return (int)hipGetLastError();  // prepare only
+        if (mode != nullptr && mode[0] == 'p') {
+            const int ns = mode[1] == '2' ? 2 : 1;
+            if (scan_pair_supported(K, p.V, ns)) return launch_scan_pair(p, K, stream, ns, save);
+        }
+    }
     if (save && nw == 2) nw = 1;  // the saving variant exists for 1 and 4 slices per workgroup
     p.scan_groups = vtiles / nw;
     const dim3 grid((unsigned)(chains8 * p.scan_groups));
