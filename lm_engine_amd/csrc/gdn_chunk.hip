@@ -66,9 +66,12 @@ uint64_t chunk_record_bytes(const gdn_args& a) {
     return (uint64_t)a.H * chunk_slots(a) * record_layout(a.K, a.V).bytes;
 }
 
+// one int32 flag per record (used when prepare and scan run in one launch)
+static uint64_t chunk_flag_bytes(const gdn_args& a) { return ((uint64_t)a.H * chunk_slots(a) * 4 + 255u) & ~(uint64_t)255u; }
+
 uint64_t chunk_workspace_bytes(const gdn_args& a) {
     const RecordLayout r = record_layout(a.K, a.V);
-    return chunk_off_bytes(a) + (uint64_t)a.H * chunk_slots(a) * r.bytes;
+    return chunk_off_bytes(a) + chunk_flag_bytes(a) + (uint64_t)a.H * chunk_slots(a) * r.bytes;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -623,13 +626,14 @@ int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events, 
     p.cu_seqlens = left_padded ? nullptr : a.cu_seqlens;
     p.pad_lens = left_padded ? a.cu_seqlens : nullptr;
     p.chunk_off = static_cast<int32_t*>(a.workspace);
-    p.rec = static_cast<uint8_t*>(a.workspace) + chunk_off_bytes(a);
+    p.ready = reinterpret_cast<int32_t*>(static_cast<uint8_t*>(a.workspace) + chunk_off_bytes(a));
+    p.rec = static_cast<uint8_t*>(a.workspace) + chunk_off_bytes(a) + chunk_flag_bytes(a);
     p.save_state = nullptr, p.save_vnew = nullptr, p.save_nc = 0, p.records_given = 0, p.save_every = 1, p.save_reverse = 0;
     if (saves != nullptr) {
         p.save_state = saves->states, p.save_vnew = saves->v_new, p.save_nc = saves->chunks_per_chain;
         p.save_every = saves->save_every > 0 ? saves->save_every : 1, p.save_reverse = saves->save_reverse ? 1 : 0;
         p.records_given = saves->records_given;
-        if (p.records_given) p.chunk_off = nullptr, p.rec = static_cast<uint8_t*>(a.workspace);
+        if (p.records_given) p.chunk_off = nullptr, p.ready = nullptr, p.rec = static_cast<uint8_t*>(a.workspace);
     }
     p.q_stride_b = a.q_stride_b, p.q_stride_t = a.q_stride_t, p.q_stride_h = a.q_stride_h;
     p.k_stride_b = a.k_stride_b, p.k_stride_t = a.k_stride_t, p.k_stride_h = a.k_stride_h;

@@ -42,6 +42,7 @@ struct ChunkParams {
     int save_every;    // only chunks c with c % save_every == 0 are saved, as entry c / save_every ...
     int save_reverse;  // ... or, when set, as entry save_nc - 1 - c / save_every
     int records_given;  // the records are already in place: prepare is not run
+    int32_t* ready;     // [H][TC] one flag per record, for the launch that runs prepare and scan together
 };
 
 struct RecordLayout {

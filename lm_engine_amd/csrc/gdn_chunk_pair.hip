@@ -34,6 +34,7 @@
 #include <stdlib.h>
 
 #include "gdn_chunk32_common.h"
+#include "gdn_chunk_prepare32.h"
 #include "gdn_launch.h"
 
 namespace gdn {
@@ -94,8 +95,18 @@ __device__ long long pair_timing[1024][2][16];
 // pure MFMA intrinsic is not and would be placed wherever its result is first needed.
 __device__ __forceinline__ void pin_acc(f32x16& acc) { asm volatile("" : "+v"(acc)); }
 
-template <int K, int NS, bool NT = false, bool SAVE = false>
-__global__ __launch_bounds__(PAIR_THREADS) void chunk_scan_pair_kernel(const ChunkParams p) {
+// LDS bytes of a scan workgroup: two stage halves, exchange buffers and output staging per slice, the flags
+template <int K, int NS>
+constexpr int scan_pair_lds_bytes() {
+    constexpr int STAGE = 12 * FRAG_BYTES + C * (64 * NS + 16) + 2 * C * (2 * K + 16) + 3 * C * 4 + 16;
+    constexpr int XF = K / 32 > 4 ? K / 32 : 4;
+    return 2 * STAGE + NS * ((2 * XF + 2) * FRAG_BYTES + 2 * C * 64) + 64;
+}
+
+// WAIT: the records are written by prepare workgroups of the same launch; a loader asks p.ready before it loads one.
+// `id` numbers the scan workgroups (blockIdx.x when the scan is a kernel of its own).
+template <int K, int NS, bool NT, bool SAVE, bool WAIT>
+__device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* lds, const int id) {
     constexpr int NL = PAIR_LOADERS;
     constexpr int NB = GDN_PAIR_NB;  // register buffers of a loader wave: chunks in flight
     constexpr int KD = K / 32;    // 32-row tiles of the state
@@ -131,17 +142,17 @@ __global__ __launch_bounds__(PAIR_THREADS) void chunk_scan_pair_kernel(const Chu
     constexpr int OBYTES = 2 * C * 64;  // output staging of a slice: [chunk parity][64 tokens][64 bytes]
     static_assert(2 * STAGE_BYTES + NS * (XBYTES + OBYTES) + 64 <= 160 * 1024, "stage exceeds LDS");
 
-    __shared__ __attribute__((aligned(16))) uint8_t stage[2][STAGE_BYTES];
-    __shared__ __attribute__((aligned(16))) uint8_t xbuf[NS][XBYTES];
-    __shared__ __attribute__((aligned(16))) uint8_t ostage[NS][OBYTES];
-    __shared__ int flags[NS][2];
+    static_assert(2 * STAGE_BYTES + NS * (XBYTES + OBYTES) + 64 == scan_pair_lds_bytes<K, NS>(), "LDS layout and its size disagree");
+    uint8_t (*const stage)[STAGE_BYTES] = reinterpret_cast<uint8_t (*)[STAGE_BYTES]>(lds);
+    uint8_t (*const xbuf)[XBYTES] = reinterpret_cast<uint8_t (*)[XBYTES]>(lds + 2 * STAGE_BYTES);
+    uint8_t (*const ostage)[OBYTES] = reinterpret_cast<uint8_t (*)[OBYTES]>(lds + 2 * STAGE_BYTES + NS * XBYTES);
+    int (*const flags)[2] = reinterpret_cast<int (*)[2]>(lds + 2 * STAGE_BYTES + NS * (XBYTES + OBYTES));
 
     const int lane = threadIdx.x % WAVE;
     const int wave = threadIdx.x / WAVE;
     const int l32 = lane % 32, lh = lane / 32;
 
     // workgroup -> (sequence-head chain, column group); the groups of a chain stay on one XCD (id % 8)
-    const int id = blockIdx.x;
     const int xcd = id % 8, rest = id / 8;
     const int vgroup = rest % p.scan_groups;
     const int per_xcd = (p.N * p.H + 7) / 8;
@@ -304,14 +315,38 @@ __global__ __launch_bounds__(PAIR_THREADS) void chunk_scan_pair_kernel(const Chu
                 for (int sl = 0; sl < NS; sl++) *reinterpret_cast<bf16x8*>(og + (int64_t)c * C * p.o_stride_t + 32 * sl) = rows[sl];
             }
         };
+        // Records written in this very launch: chunks below ready_upto are known to be complete.  One poll reads the
+        // flags of the next 64 chunks, one per lane, with loads that bypass the caches; it also waits for every load
+        // this wave has in flight (they return in order), so polls should be rare: prepare normally runs well ahead.
+        int ready_upto = WAIT ? 0 : nchunks;
+        auto ensure_ready = [&](int c) {
+            if constexpr (WAIT) {
+                if (c < ready_upto || c >= nchunks) return;
+                const int32_t* flag = p.ready + (int64_t)h * p.TC + slot_begin + c;
+                for (uint32_t spin = 0;; spin++) {
+                    const int32_t got = c + lane < nchunks ? __hip_atomic_load(flag + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 1;
+                    const uint64_t pending = __ballot(got == 0);
+                    const int n = pending == 0 ? 64 : __builtin_ctzll(pending);
+                    if (n > 0 || spin >= (1u << 22)) {  // bounded: a launch without its prepare half must still end
+                        ready_upto = c + (n > 0 ? n : 1);
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(32);
+                }
+                asm volatile("" ::: "memory");
+            }
+        };
         constexpr std::true_type yes{};
         constexpr std::false_type no{};
         // Chunk c travels in register buffer c % NB: NB chunks are in flight or on their way into LDS at any time.
+        ensure_ready(0);
+        ensure_ready(NB - 1);
         static_for<0, NB>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
             if (j < nchunks) load(buf[j], sc[j], j);
         });
         if (nchunks > 0) {
+            ensure_ready(NB);
             if (nchunks > NB) store_and_reload(buf[0], sc[0], 0, NB, yes);
             else store_and_reload(buf[0], sc[0], 0, 0, no);
         }
@@ -323,6 +358,7 @@ __global__ __launch_bounds__(PAIR_THREADS) void chunk_scan_pair_kernel(const Chu
         for (; c + 2 * NB < nchunks; c += NB) {  // steady state: straight-line code, every reload exists
             static_for<0, NB>([&](auto jc) {
                 constexpr int j = decltype(jc)::value, bi = (j + 1) % NB;
+                ensure_ready(c + j + 1 + NB);
                 store_and_reload(buf[bi], sc[bi], c + j + 1, c + j + 1 + NB, yes);
                 __syncthreads();
                 if (c + j > 0) flush(c + j - 1);
@@ -334,6 +370,7 @@ __global__ __launch_bounds__(PAIR_THREADS) void chunk_scan_pair_kernel(const Chu
                 const int cc = c + j;
                 if (cc < nchunks) {
                     if (cc + 1 < nchunks) {
+                        ensure_ready(cc + 1 + NB);
                         if (cc + 1 + NB < nchunks) store_and_reload(buf[bi], sc[bi], cc + 1, cc + 1 + NB, yes);
                         else store_and_reload(buf[bi], sc[bi], cc + 1, 0, no);
                     }
@@ -667,6 +704,55 @@ __global__ __launch_bounds__(PAIR_THREADS) void chunk_scan_pair_kernel(const Chu
 }
 
 // ------------------------------------------------------------------------------------------
+// kernels
+// ------------------------------------------------------------------------------------------
+template <int K, int NS, bool NT = false, bool SAVE = false>
+__global__ __launch_bounds__(PAIR_THREADS) void chunk_scan_pair_kernel(const ChunkParams p) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[scan_pair_lds_bytes<K, NS>()];
+    scan_pair_body<K, NS, NT, SAVE, false>(p, lds, blockIdx.x);
+}
+
+// Prepare and scan in one launch (fixed-length batches whose scan needs at most ~3/4 of the CUs).  Every workgroup
+// takes a CU to itself (by its LDS size).  The first `prep_wgs` workgroups are producers: two groups of four waves
+// each run the prepare step on items of the chains that are scanned on their XCD, earliest chunks first, and set a
+// flag per finished record.  The others are scan workgroups whose loaders wait for those flags.  A producer never
+// waits for anything and the producers have the lowest workgroup ids, which are dispatched first: the launch cannot
+// block itself whatever part of it is resident.  What this buys: the prepare step runs beside the scan instead of
+// before it, and the scan finds q, k and the records of a chain in the L2 of its XCD shortly after they were used.
+constexpr int FUSED_GROUPS = 2;
+
+template <int K, int NS>
+__global__ __launch_bounds__(PAIR_THREADS) void chunk_fused_kernel(const ChunkParams p, const int prep_wgs) {
+    constexpr int SCAN_LDS = scan_pair_lds_bytes<K, NS>(), PREP_LDS = FUSED_GROUPS * prepare32_lds_bytes<K>();
+    __shared__ __attribute__((aligned(16))) uint8_t lds[SCAN_LDS > PREP_LDS ? SCAN_LDS : PREP_LDS];
+    if ((int)blockIdx.x >= prep_wgs) {
+        scan_pair_body<K, NS, false, false, true>(p, lds, (int)blockIdx.x - prep_wgs);  // prep_wgs is a multiple of 8: same XCD numbering
+        return;
+    }
+    // producer: items of XCD x are (chunk c, chain) for the chains x * per_xcd .. the scan puts on that XCD, chunk-major
+    const int xcd = blockIdx.x % 8, rank = blockIdx.x / 8, per = prep_wgs / 8;
+    const int chains = p.N * p.H, per_xcd = (chains + 7) / 8;
+    const int first_chain = xcd * per_xcd;
+    const int nch = max(0, min(per_xcd, chains - first_chain));
+    const uint32_t items = (uint32_t)nch * (uint32_t)p.NT;
+    const int H = p.H, NT = p.NT;
+    auto item_of = [=](uint32_t i, int& h, int& slot) {
+        const int c = (int)(i / (uint32_t)nch), chain = first_chain + (int)(i % (uint32_t)nch);
+        h = chain % H;
+        slot = (chain / H) * NT + c;
+    };
+    const uint32_t step = (uint32_t)(per * FUSED_GROUPS);
+    const uint32_t rounds = (items + step - 1) / step;
+    const uint32_t group = threadIdx.x / PREP_THREADS;
+    if (group >= (uint32_t)FUSED_GROUPS) return;
+    chunk_prepare32_body<K, FUSED_GROUPS, true>(p, lds, item_of, items, (uint32_t)rank * FUSED_GROUPS + group, step, rounds, p.ready, 1);
+}
+
+__global__ void fill_zero_kernel(int32_t* x, int64_t n) {
+    for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) x[i] = 0;
+}
+
+// ------------------------------------------------------------------------------------------
 // launch
 // ------------------------------------------------------------------------------------------
 bool scan_pair_supported(int K, int V, int ns) { return (K == 64 || K == 128) && V % (32 * ns) == 0; }
@@ -684,6 +770,33 @@ static int launch_pair_k(ChunkParams& p, hipStream_t stream, int ns, bool save) 
         else hipLaunchKernelGGL((chunk_scan_pair_kernel<K, 1>), grid, block, 0, stream, p);
     }
     return (int)hipGetLastError();
+}
+
+// The fused launch: scan workgroups of two slices each beside the producers.  Returns GDN_ERR_UNSUPPORTED (before any
+// launch) when the shape does not qualify; the caller then runs prepare and scan as two kernels.
+template <int K>
+static int launch_fused_k(ChunkParams& p, hipStream_t stream, int num_cus) {
+    const int64_t chains8 = ((int64_t)p.N * p.H + 7) / 8 * 8;
+    p.scan_groups = p.V / 64;
+    const int64_t scan_wgs = chains8 * p.scan_groups;
+    const int prep_wgs = (int)((num_cus - scan_wgs) / 8 * 8);
+    if (scan_wgs > (int64_t)num_cus * 3 / 4 || prep_wgs < num_cus / 4) return GDN_ERR_UNSUPPORTED;
+    const int64_t nflags = (int64_t)p.H * p.TC;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((nflags + 255) / 256 < 64 ? (nflags + 255) / 256 : 64)), dim3(256), 0, stream, p.ready, nflags);
+    if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
+    hipLaunchKernelGGL((chunk_fused_kernel<K, 2>), dim3((unsigned)(prep_wgs + scan_wgs)), dim3(PAIR_THREADS), 0, stream, p, prep_wgs);
+    return (int)hipGetLastError();
+}
+
+bool chunk_fused_supported(const ChunkParams& p, int K) {
+    return (K == 64 || K == 128) && p.V % 64 == 0 && p.cu_seqlens == nullptr && p.pad_lens == nullptr && p.ready != nullptr &&
+           !p.records_given && p.save_state == nullptr && p.save_vnew == nullptr;
+}
+
+int launch_chunk_fused(ChunkParams& p, int K, hipStream_t stream, int num_cus) {
+    if (!chunk_fused_supported(p, K)) return GDN_ERR_UNSUPPORTED;
+    if (K == 64) return launch_fused_k<64>(p, stream, num_cus);
+    return launch_fused_k<128>(p, stream, num_cus);
 }
 
 int launch_scan_pair(ChunkParams& p, int K, hipStream_t stream, int ns, bool save) {
