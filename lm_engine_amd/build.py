@@ -21,7 +21,7 @@ CSRC_DIR = os.path.join(PACKAGE_DIR, "csrc")
 INCLUDE_DIR = os.path.join(os.path.dirname(PACKAGE_DIR), "include")
 LIBRARY_PATH = os.path.join(PACKAGE_DIR, "libgdn_hip.so")
 
-SOURCES = ("gdn_api.hip", "gdn_recurrent.hip", "gdn_chunk.hip", "gdn_chunk32.hip", "gdn_chunk_pair.hip", "gdn_chunk_bwd.hip", "gdn_conv1d.hip", "gdn_conv1d_bwd.hip", "gdn_elementwise.hip")
+SOURCES = ("gdn_api.hip", "gdn_recurrent.hip", "gdn_chunk.hip", "gdn_chunk32.hip", "gdn_chunk_fused.hip", "gdn_chunk_bwd.hip", "gdn_conv1d.hip", "gdn_conv1d_bwd.hip", "gdn_elementwise.hip")
 
 HIPCC_FLAGS = (
     "--offload-arch=gfx950",

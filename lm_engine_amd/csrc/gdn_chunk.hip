@@ -648,6 +648,7 @@ int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events, 
     p.rec_bytes = r.bytes, p.off_qs = r.off_qs, p.off_kt = r.off_kt, p.off_ks = r.off_ks, p.off_cs = r.off_cs, p.off_p = r.off_p, p.off_u = r.off_u;
     p.off_eg = r.off_eg;
     p.scan_groups = 1;
+    p.fused = (a.flags & GDN_FLAG_FUSED_LAUNCH) ? 1 : 0;
 
     auto mark = [&](int i) {
         if (events != nullptr) (void)hipEventRecord(events[i], stream);

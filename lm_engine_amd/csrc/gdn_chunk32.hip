@@ -42,8 +42,6 @@
 
 #include <type_traits>
 
-#include <stdlib.h>
-
 #include "gdn_chunk32_common.h"
 #include "gdn_chunk_prepare32.h"
 #include "gdn_launch.h"
@@ -312,7 +310,7 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
 #pragma unroll
                 for (int i = 0; i < 4; i++)
                     if (row0 + 16 * i < valid)
-                        *reinterpret_cast<bf16x8*>(og + ((int64_t)c * C + 16 * i) * p.o_stride_t + 32 * w) = rows[i];
+                        __builtin_nontemporal_store(rows[i], reinterpret_cast<bf16x8*>(og + ((int64_t)c * C + 16 * i) * p.o_stride_t + 32 * w));
             }
         };
         __syncthreads();
@@ -702,9 +700,7 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
 // ------------------------------------------------------------------------------------------
 // launch
 // ------------------------------------------------------------------------------------------
-int launch_scan_pair(ChunkParams& p, int K, hipStream_t stream, int ns, bool save);  // gdn_chunk_pair.hip
-int launch_chunk_fused(ChunkParams& p, int K, hipStream_t stream, int num_cus);
-bool scan_pair_supported(int K, int V, int ns);
+int launch_chunk_fused(ChunkParams& p, int K, hipStream_t stream, int num_cus);  // gdn_chunk_fused.hip
 
 template <int K>
 static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int num_cus) {
@@ -712,12 +708,12 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     const int64_t cap = (int64_t)(3 * num_cus + 7) / 8 * 8;      // three workgroups per CU (LDS and registers allow it)
     if (items >= ((int64_t)1 << 31)) return GDN_ERR_UNSUPPORTED;  // the kernel counts items in 32 bits
     const int grid_prep = (int)(items < cap ? items : cap);
-    if (const char* mode = getenv("GDN_SCAN"); mode != nullptr && mode[0] == 'f') {
+    if (p.fused) {  // prepare and scan in one launch, when the shape qualifies
         if (events != nullptr) (void)hipEventRecord(events[2], stream);
         const int rc = launch_chunk_fused(p, K, stream, num_cus);
         if (rc != GDN_ERR_UNSUPPORTED) return rc;
     }
-    if (!p.records_given && getenv("GDN_SKIP_PREPARE") == nullptr) {
+    if (!p.records_given) {
         hipLaunchKernelGGL((chunk_prepare32_kernel<K>), dim3(grid_prep), dim3(PREP_THREADS), 0, stream, p);
         if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
     }
@@ -732,15 +728,6 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     int nw = 1;
     while (nw < 4 && vtiles % (2 * nw) == 0 && chains * (vtiles / nw) > (int64_t)num_cus) nw *= 2;
     const bool save = p.save_state != nullptr || p.save_vnew != nullptr;
-    {
-        // experiment switch: GDN_SCAN=p1 / p2 runs the scan with two compute waves per slice, 1 or 2 slices per workgroup
-        const char* mode = getenv("GDN_SCAN");
-        if (mode != nullptr && mode[0] == 'n') return (int)hipGetLastError();  // prepare only
-        if (mode != nullptr && mode[0] == 'p') {
-            const int ns = mode[1] == '2' ? 2 : 1;
-            if (scan_pair_supported(K, p.V, ns)) return launch_scan_pair(p, K, stream, ns, save);
-        }
-    }
     if (save && nw == 2) nw = 1;  // the saving variant exists for 1 and 4 slices per workgroup
     p.scan_groups = vtiles / nw;
     const dim3 grid((unsigned)(chains8 * p.scan_groups));

@@ -43,6 +43,7 @@ struct ChunkParams {
     int save_reverse;  // ... or, when set, as entry save_nc - 1 - c / save_every
     int records_given;  // the records are already in place: prepare is not run
     int32_t* ready;     // [H][TC] one flag per record, for the launch that runs prepare and scan together
+    int fused;          // that launch was asked for (GDN_FLAG_FUSED_LAUNCH)
 };
 
 struct RecordLayout {

@@ -1,8 +1,10 @@
-// Scan of the chunked forward with TWO compute waves per 32-column slice of the state (K <= 128).
+// The chunked forward as ONE launch (K <= 128, fixed-length batches whose scan needs at most about half of the CUs):
+// producer workgroups run the prepare step and scan workgroups consume its records as they appear.
 //
-// gdn_chunk32.hip's scan gives one wave a whole slice: 60 MFMAs and ~480 other instructions per chunk on a
-// single SIMD, whose matrix pipe alone needs 60 x 32 cycles for them, while the other three SIMDs of the CU
-// feed it.  Here a slice is shared by a pair of waves on two SIMDs.  Wave tt (0 or 1) of a pair owns
+// Scan workgroups.  gdn_chunk32.hip's scan gives one wave a whole 32-column slice of the state, and a slice a CU.
+// Here a workgroup holds two slices of a chain (64 columns: whole 128-byte lines of the output) and each slice is
+// shared by a PAIR of compute waves on two SIMDs, so the scan of a batch needs half as many CUs and leaves the
+// others to the producers.  Wave tt (0 or 1) of a pair owns
 //   * token tile tt (tokens 32 tt .. 32 tt + 31 of the chunk) in every product whose rows are tokens:
 //     K S0, X, V~ = T' X, and the output O = diag(qs) Q S0 + P V~;
 //   * key half tt (state rows K/2 tt .. K/2 tt + K/2 - 1) of the state, as MFMA accumulators, in the update
@@ -18,20 +20,21 @@
 // epoch number to an LDS word of its own; the partner polls that word.  (LDS operations of a wave execute
 // in order, so whoever reads the new epoch reads the data written before it.)  Each wave starts on the
 // half of a product that needs only its own operand and picks the partner's up when it gets there, which
-// hides most of the hand-over.  Per chunk and wave (K = 128): 28 (tile 0) or 32 (tile 1) MFMAs.
-//
+// hides part of the hand-over.  Per chunk and wave (K = 128): 28 (tile 0) or 32 (tile 1) MFMAs.
 // The exchange buffers overlap: a wave's tile of V~ is written over the partner's half of S0, which that
 // wave alone reads and has finished with by then; the partner overwrites it with its next half of S0 only
 // after it has read V~ from it.
+// Loaders (4 waves) and the LDS double buffer are those of gdn_chunk32.hip; the loaders also write the output
+// (a compute wave leaves its bf16 output tile in LDS at the start of the next chunk).  One workgroup barrier
+// per chunk hands the stage halves over.  Waves of a scan workgroup with two slices: 0..3 compute (pairs 0-1,
+// 2-3), 4..7 loaders.  (With one slice: 0 1 compute | 2 3 6 7 loaders | 4 output store | 5 exits at once.)
 //
-// Loaders (4 waves) and the LDS double buffer are those of gdn_chunk32.hip; the loaders also write the
-// output (a compute wave leaves its bf16 output tile in LDS at the start of the next chunk).  One workgroup
-// barrier per chunk hands the stage halves over.  A workgroup holds NS = 1 or 2 slices of one chain:
-//   NS = 1:  waves 0 1 compute | 2 3 6 7 loaders | 4 output store | 5 exits at once   (loaders on the SIMDs without compute waves)
-//   NS = 2:  waves 0..3 compute (pairs 0-1, 2-3) | 4..7 loaders
-
-#include <stdio.h>
-#include <stdlib.h>
+// What a wave pays, measured with one wave alone on a SIMD: 4.5 cycles per VALU instruction, 32 per MFMA (hidden
+// behind up to ~7 independent VALU instructions), ~17 per ds_read_b128, ~29 per ds_write_b128, ~120 for an LDS write
+// followed by a read of it.  The operand fragments (one ds_read_b128 per MFMA) and the bf16 conversions therefore
+// cost a compute wave more than its MFMAs, in this scan as in the one-wave scan, and the hand-overs between the
+// waves of a pair (~300 cycles each, three per chunk) eat what the second SIMD brings: a pair runs a slice in
+// ~2750 cycles per chunk, the single wave in ~2850.
 
 #include "gdn_chunk32_common.h"
 #include "gdn_chunk_prepare32.h"
@@ -39,15 +42,8 @@
 
 namespace gdn {
 
-#ifdef GDN_PAIR_NS2_STOREWAVE
-constexpr int PAIR_THREADS = 9 * WAVE;
-#else
 constexpr int PAIR_THREADS = 8 * WAVE;
-#endif
 constexpr int PAIR_LOADERS = 4;
-#ifndef GDN_PAIR_NB
-#define GDN_PAIR_NB 2
-#endif
 
 // Epochs: a wave stores 3 c + 1 once its half of the state chunk c starts from is in LDS, 3 c + 2 (wave 0
 // only) after X of token tile 0, 3 c + 3 after its tile of V~.
@@ -78,16 +74,6 @@ __device__ __forceinline__ void pair_wait(lds_flag_t* flag, int epoch) {
         : "memory", "scc");
 }
 
-#ifdef GDN_PAIR_TIMING
-__device__ long long pair_timing[1024][2][16];
-#define PT_NOW() clock64()
-#define PT_ADD(i, t0) tacc[i] += clock64() - (t0)
-#define PT_SEG(i) { long long n_ = clock64(); tacc[8 + (i)] += n_ - t_seg; t_seg = n_; }
-#else
-#define PT_NOW() 0
-#define PT_ADD(i, t0) (void)(t0)
-#define PT_SEG(i)
-#endif
 
 #define PIN() __builtin_amdgcn_sched_barrier(0)
 
@@ -104,11 +90,11 @@ constexpr int scan_pair_lds_bytes() {
 }
 
 // WAIT: the records are written by prepare workgroups of the same launch; a loader asks p.ready before it loads one.
-// `id` numbers the scan workgroups (blockIdx.x when the scan is a kernel of its own).
-template <int K, int NS, bool NT, bool SAVE, bool WAIT>
+// `id` numbers the scan workgroups.
+template <int K, int NS, bool WAIT>
 __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* lds, const int id) {
     constexpr int NL = PAIR_LOADERS;
-    constexpr int NB = GDN_PAIR_NB;  // register buffers of a loader wave: chunks in flight
+    constexpr int NB = 2;       // register buffers of a loader wave: chunks in flight
     constexpr int KD = K / 32;    // 32-row tiles of the state
     constexpr int KS16 = K / 16;  // 16-wide slabs over the key dim
     constexpr int KDH = KD / 2;   // state tiles per wave
@@ -185,11 +171,7 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
     // With one slice a separate wave writes the output: a store in a loader wave sits in the same in-order
     // memory counter as its loads, and every wait for a load then also waits for the store's acknowledgement
     // (measured: the loaders alone 59 us for configuration 1 without the stores, 93 us with them).
-#ifdef GDN_PAIR_NS2_STOREWAVE
-    constexpr bool STORE_WAVE = true;
-#else
     constexpr bool STORE_WAVE = NS == 1;
-#endif
     const bool is_compute = wave < 2 * NS;
     const bool is_loader = NS == 2 ? (wave >= 4 && wave < 8) : (wave == 2 || wave == 3 || wave == 6 || wave == 7);
     const bool is_store = STORE_WAVE && wave == (NS == 2 ? 8 : 4);
@@ -211,12 +193,7 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
 #pragma unroll
                 for (int i = 0; i < 4; i++)
                     if (row0 + 16 * i < valid) {
-#if defined(GDN_PAIR_NOSTORE)
-#elif defined(GDN_PAIR_NTSTORE)
                         __builtin_nontemporal_store(rows[i], reinterpret_cast<bf16x8*>(og + ((int64_t)c * C + 16 * i) * p.o_stride_t + 32 * sl));
-#else
-                        *reinterpret_cast<bf16x8*>(og + ((int64_t)c * C + 16 * i) * p.o_stride_t + 32 * sl) = rows[i];
-#endif
                     }
             }
         };
@@ -251,9 +228,6 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
         };
         Scalars sc[NB] = {};
         auto src_of = [&](int c, int i) -> const uint8_t* {
-#ifdef GDN_PAIR_SAMECHUNK
-            c = 0;
-#endif
             if (i < NF) return rec + ((int64_t)c * p.rec_bytes + (int64_t)frag_of(i) * FRAG_BYTES) + lane * 16;
             if (i < NF + NV) {  // a row past the end of the sequence is read from the last token instead: never used
                 const int tok = min(c * C + vunit_of(i - NF) * V_ROWS + v_row, (int)seq_len - 1);
@@ -276,10 +250,7 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
             sc.cs = reinterpret_cast<const float*>(r + p.off_cs)[lane];
             sc.eg = *reinterpret_cast<const float*>(r + p.off_eg);
         };
-        auto fetch = [&](const uint8_t* src) -> bf16x8 {
-            if constexpr (NT) return __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(src));
-            else return *reinterpret_cast<const bf16x8*>(src);
-        };
+        auto fetch = [&](const uint8_t* src) -> bf16x8 { return *reinterpret_cast<const bf16x8*>(src); };
         auto load = [&](bf16x8(&buf)[NLOAD], Scalars& sc, int c) {
 #pragma unroll
             for (int i = 0; i < NLOAD; i++) buf[i] = fetch(src_of(c, i));
@@ -312,7 +283,7 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
             for (int sl = 0; sl < NS; sl++) rows[sl] = *reinterpret_cast<const bf16x8*>(ostage_at(sl, c & 1, o_row, o_piece));
             if (o_row < valid) {
 #pragma unroll
-                for (int sl = 0; sl < NS; sl++) *reinterpret_cast<bf16x8*>(og + (int64_t)c * C * p.o_stride_t + 32 * sl) = rows[sl];
+                for (int sl = 0; sl < NS; sl++) __builtin_nontemporal_store(rows[sl], reinterpret_cast<bf16x8*>(og + (int64_t)c * C * p.o_stride_t + 32 * sl));
             }
         };
         // Records written in this very launch: chunks below ready_upto are known to be complete.  One poll reads the
@@ -436,15 +407,7 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
 #pragma unroll
         for (int i = 0; i < SH; i++)
             kfn[i] = *reinterpret_cast<const bf16x8*>(stage[0] + K_OFF + (32 * TT + l32) * QLD + (16 * (SH * TT + i) + 8 * lh) * 2);
-#ifdef GDN_PAIR_TIMING
-        long long tacc[16] = {};
-        const long long t_loop = clock64();
-#endif
 
-#ifdef GDN_PAIR_NOCOMPUTE
-        for (int c = 0; c < nchunks; c++) __syncthreads();
-        if (false)
-#endif
         for (int c = 0; c < nchunks; c++) {
             const uint8_t* st = stage[c & 1];
             const bf16_t* km = reinterpret_cast<const bf16_t*>(st + K_OFF);
@@ -463,20 +426,6 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
                 return r;
             };
             auto rec_frag = [&](int f) { return reinterpret_cast<const bf16x8*>(st)[f * WAVE + lane]; };  // T' 0..5 | P 6..11
-
-            if constexpr (SAVE) {
-                if (p.save_state != nullptr && c % p.save_every == 0 && c / p.save_every < p.save_nc) {
-                    const int entry = p.save_reverse ? p.save_nc - 1 - c / p.save_every : c / p.save_every;
-                    char* base = reinterpret_cast<char*>(p.save_state + ((int64_t)chain * p.save_nc + entry) * K * p.V);
-                    const uint32_t lane_off = (uint32_t)((8 * lh) * p.V + 32 * tn + slice_col(l32)) * 4u;
-                    const uint32_t row_bytes = (uint32_t)p.V * 4u;
-#pragma unroll
-                    for (int t = 0; t < KDH; t++)
-#pragma unroll
-                        for (int r = 0; r < 16; r++)
-                            *reinterpret_cast<float*>(base + (size_t)(st_row(KDH * TT + t, r) * row_bytes) + lane_off) = S[t][r];
-                }
-            }
 
             // The order below is the schedule: what stands between two PIN()s stays there.  A wave issues in order and
             // an MFMA holds the matrix pipe for 32 cycles, so every MFMA is followed by a handful of instructions that do
@@ -501,9 +450,6 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
 #pragma unroll
                 for (int e = 0; e < 4; e++) vbs[x][4 * sub + e] = (bf16_t)(vt[8 * x + 4 * sub + e] * ksr[2 * x + sub][e]);
             };
-#ifdef GDN_PAIR_TIMING
-            long long t_seg = clock64();
-#endif
 #pragma unroll
             for (int i = 0; i < SH; i++) kf[i] = kfn[i];
             const float egc = *reinterpret_cast<const float*>(st + EG_OFF);
@@ -524,7 +470,6 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
                 qf[i] = q_frag(SH * TT + i);
                 PIN();
             });
-            PT_SEG(0);
             // ---- the previous chunk's output leaves the accumulators; first product of (Q S0)^T ----
             write_out((c - 1) & 1);  // (chunk 0 hands over zeros, which nobody writes out)
 #pragma unroll
@@ -537,14 +482,10 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
                 xvr[q4] = lds_read_tr4x16<true>(reinterpret_cast<const bf16_t*>(st + V_OFF), VLD / 2, 32 * TT + 8 * q4 + 4 * lh, 32 * sl + 16 * g16, l16);
             }
             PIN();
-            PT_SEG(1);
-            { auto t_ = PT_NOW(); pair_wait(other_flag, 3 * c + 1); PT_ADD(0, t_); }
+            pair_wait(other_flag, 3 * c + 1);
 #pragma unroll
             for (int i = 0; i < SH; i++) sbo[i] = xs_other[i * WAVE];
             PIN();
-#ifdef GDN_PAIR_TIMING
-            t_seg = clock64();
-#endif
             // ---- K S0, the partner's half | operand reads ----
             static_for<0, SH>([&](auto ic) {
                 constexpr int i = decltype(ic)::value;
@@ -561,7 +502,6 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
                 }
                 PIN();
             });
-            PT_SEG(2);
             // ---- X, with (Q S0)^T in the matrix pipe ----
             g2(std::integral_constant<int, 1>{});
             PIN();
@@ -575,8 +515,6 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
             });
             if constexpr (TT == 0) pair_publish(my_flag, 3 * c + 2);
             PIN();
-
-            PT_SEG(3);
             // ---- V~ = T' X (tile 1: its own X first, then tile 0's) ----
             vt = mfma32_bf16(tf[0], xb[0], vt);
             vt = mfma32_bf16(tf[1], xb[1], vt);
@@ -590,7 +528,7 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
             if constexpr (TT == 1) {
                 static_for<4, G2_BEFORE_V>([&](auto jc) { g2(jc); });
                 PIN();
-                { auto t_ = PT_NOW(); pair_wait(other_flag, 3 * c + 2); PT_ADD(1, t_); }
+                pair_wait(other_flag, 3 * c + 2);
                 const bf16x8 x0 = xx[0], x1 = xx[WAVE];
                 vt = mfma32_bf16(tf[2], x0, vt);
                 vt = mfma32_bf16(tf[3], x1, vt);
@@ -603,19 +541,6 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
             const bf16x8 pm0 = rec_frag(TT == 0 ? 6 : 10), pm1 = rec_frag(TT == 0 ? 7 : 11);
             PIN();
 
-            if constexpr (SAVE) {
-                if (p.save_vnew != nullptr && c % p.save_every == 0 && c / p.save_every < p.save_nc) {
-                    const int entry = p.save_reverse ? p.save_nc - 1 - c / p.save_every : c / p.save_every;
-                    char* base = reinterpret_cast<char*>(p.save_vnew + ((int64_t)chain * p.save_nc + entry) * C * p.V);
-                    const uint32_t lane_off = (uint32_t)((4 * lh) * p.V + 32 * tn + slice_col(l32)) * 4u;
-                    const uint32_t row_bytes = (uint32_t)p.V * 4u;
-#pragma unroll
-                    for (int r = 0; r < 16; r++)
-                        *reinterpret_cast<float*>(base + (size_t)((32 * TT + 8 * (r / 4) + r % 4) * row_bytes) + lane_off) = vt[r];
-                }
-            }
-
-            PT_SEG(4);
             // ---- V~ as operands (rows scaled by ks for the state update, plain for P V~), the rest of (Q S0)^T between ----
             static_for<0, 2>([&](auto xc) {
                 constexpr int x = decltype(xc)::value;
@@ -628,8 +553,6 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
             if constexpr (TT == 0) xs_other[2 * WAVE] = vb[0], xs_other[3 * WAVE] = vb[1];
             pair_publish(my_flag, 3 * c + 3);
             PIN();
-
-            PT_SEG(5);
             // ---- S += k^T V~', my token tile's slabs | q's row scale on (Q S0)^T, complete by now ----
             static_for<0, 2 * KDH>([&](auto uc) {
                 constexpr int u = decltype(uc)::value, t = u / 2, j = u % 2;
@@ -648,8 +571,7 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
             bf16x8 po0 = {}, po1 = {};
             if constexpr (TT == 1) po0 = rec_frag(8), po1 = rec_frag(9);
             PIN();
-            PT_SEG(6);
-            { auto t_ = PT_NOW(); pair_wait(other_flag, 3 * c + 3); PT_ADD(2, t_); }
+            pair_wait(other_flag, 3 * c + 3);
             const bf16x8 vo0 = xs_mine[0], vo1 = xs_mine[WAVE];
             bf16x8 pv0 = {}, pv1 = {};
             if constexpr (TT == 1) pv0 = xs_mine[2 * WAVE], pv1 = xs_mine[3 * WAVE];
@@ -661,7 +583,7 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
                 S[t] = mfma32_bf16(ktf[t][3], vo1, S[t]);
             }
             PIN();
-            { auto t_ = PT_NOW(); __syncthreads(); PT_ADD(3, t_); }  // this wave has read all it needs of chunk c's half; chunk c + 1 is in the other one
+            __syncthreads();  // this wave has read all it needs of chunk c's half; chunk c + 1 is in the other one
             if constexpr (TT == 1) {
                 acco = mfma32_bf16(pv0, po0, acco);
                 acco = mfma32_bf16(pv1, po1, acco);
@@ -680,15 +602,9 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
                 sbm[i] = pack8_16(S[i / 2], i % 2, 1.f);
                 xs_mine[i * WAVE] = sbm[i];
             }
-            PT_SEG(7);
             pair_publish(my_flag, 3 * (c + 1) + 1);
         }
 
-#ifdef GDN_PAIR_TIMING
-        tacc[4] = clock64() - t_loop;
-        if (lane == 0 && sl == 0 && blockIdx.x < 1024)
-            for (int i = 0; i < 16; i++) pair_timing[blockIdx.x][TT][i] = tacc[i];
-#endif
         if (nchunks > 0) write_out((nchunks - 1) & 1);
         __syncthreads();  // the loaders write the last output tile
 
@@ -706,12 +622,6 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
 // ------------------------------------------------------------------------------------------
 // kernels
 // ------------------------------------------------------------------------------------------
-template <int K, int NS, bool NT = false, bool SAVE = false>
-__global__ __launch_bounds__(PAIR_THREADS) void chunk_scan_pair_kernel(const ChunkParams p) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[scan_pair_lds_bytes<K, NS>()];
-    scan_pair_body<K, NS, NT, SAVE, false>(p, lds, blockIdx.x);
-}
-
 // Prepare and scan in one launch (fixed-length batches whose scan needs at most ~3/4 of the CUs).  Every workgroup
 // takes a CU to itself (by its LDS size).  The first `prep_wgs` workgroups are producers: two groups of four waves
 // each run the prepare step on items of the chains that are scanned on their XCD, earliest chunks first, and set a
@@ -726,7 +636,7 @@ __global__ __launch_bounds__(PAIR_THREADS) void chunk_fused_kernel(const ChunkPa
     constexpr int SCAN_LDS = scan_pair_lds_bytes<K, NS>(), PREP_LDS = FUSED_GROUPS * prepare32_lds_bytes<K>();
     __shared__ __attribute__((aligned(16))) uint8_t lds[SCAN_LDS > PREP_LDS ? SCAN_LDS : PREP_LDS];
     if ((int)blockIdx.x >= prep_wgs) {
-        scan_pair_body<K, NS, false, false, true>(p, lds, (int)blockIdx.x - prep_wgs);  // prep_wgs is a multiple of 8: same XCD numbering
+        scan_pair_body<K, NS, true>(p, lds, (int)blockIdx.x - prep_wgs);  // prep_wgs is a multiple of 8: same XCD numbering
         return;
     }
     // producer: items of XCD x are (chunk c, chain) for the chains x * per_xcd .. the scan puts on that XCD, chunk-major
@@ -755,23 +665,6 @@ __global__ void fill_zero_kernel(int32_t* x, int64_t n) {
 // ------------------------------------------------------------------------------------------
 // launch
 // ------------------------------------------------------------------------------------------
-bool scan_pair_supported(int K, int V, int ns) { return (K == 64 || K == 128) && V % (32 * ns) == 0; }
-
-template <int K>
-static int launch_pair_k(ChunkParams& p, hipStream_t stream, int ns, bool save) {
-    const int64_t chains8 = ((int64_t)p.N * p.H + 7) / 8 * 8;
-    p.scan_groups = p.V / 32 / ns;
-    const dim3 grid((unsigned)(chains8 * p.scan_groups)), block(PAIR_THREADS);
-    if (save) {
-        if (ns == 2) hipLaunchKernelGGL((chunk_scan_pair_kernel<K, 2, false, true>), grid, block, 0, stream, p);
-        else hipLaunchKernelGGL((chunk_scan_pair_kernel<K, 1, false, true>), grid, block, 0, stream, p);
-    } else {
-        if (ns == 2) hipLaunchKernelGGL((chunk_scan_pair_kernel<K, 2>), grid, block, 0, stream, p);
-        else hipLaunchKernelGGL((chunk_scan_pair_kernel<K, 1>), grid, block, 0, stream, p);
-    }
-    return (int)hipGetLastError();
-}
-
 // The fused launch: scan workgroups of two slices each beside the producers.  Returns GDN_ERR_UNSUPPORTED (before any
 // launch) when the shape does not qualify; the caller then runs prepare and scan as two kernels.
 template <int K>
@@ -797,26 +690,6 @@ int launch_chunk_fused(ChunkParams& p, int K, hipStream_t stream, int num_cus) {
     if (!chunk_fused_supported(p, K)) return GDN_ERR_UNSUPPORTED;
     if (K == 64) return launch_fused_k<64>(p, stream, num_cus);
     return launch_fused_k<128>(p, stream, num_cus);
-}
-
-int launch_scan_pair(ChunkParams& p, int K, hipStream_t stream, int ns, bool save) {
-    int rc = GDN_ERR_UNSUPPORTED;
-    if (K == 64) rc = launch_pair_k<64>(p, stream, ns, save);
-    if (K == 128) rc = launch_pair_k<128>(p, stream, ns, save);
-#ifdef GDN_PAIR_TIMING
-    if (getenv("GDN_PAIR_PRINT") != nullptr) {
-        static long long host[1024][2][16];
-        (void)hipDeviceSynchronize();
-        (void)hipMemcpyFromSymbol(host, HIP_SYMBOL(pair_timing), sizeof(host));
-        for (int wg = 0; wg < 1024; wg += 37)
-            if (host[wg][0][4] != 0)
-                for (int tt = 0; tt < 2; tt++)
-                    printf("wg %4d wave %d: loop %lld spin1 %lld spin2 %lld spin3 %lld barrier %lld | segs %lld %lld %lld %lld %lld %lld %lld %lld\n", wg, tt, host[wg][tt][4] / 64,
-                           host[wg][tt][0] / 64, host[wg][tt][1] / 64, host[wg][tt][2] / 64, host[wg][tt][3] / 64, host[wg][tt][8] / 64, host[wg][tt][9] / 64,
-                           host[wg][tt][10] / 64, host[wg][tt][11] / 64, host[wg][tt][12] / 64, host[wg][tt][13] / 64, host[wg][tt][14] / 64, host[wg][tt][15] / 64);
-    }
-#endif
-    return rc;
 }
 
 }  // namespace gdn

@@ -88,7 +88,9 @@ __device__ __forceinline__ void chunk_prepare32_body(const ChunkParams& p, uint8
     float* const sMtB = sMt + 2 * 16 * LDM;
 
     const int tid = threadIdx.x % PREP_THREADS;
-    const int wave = tid / WAVE;
+    // role of this wave in its group; the hardware puts wave w of a workgroup on SIMD w % 4, so with several groups the
+    // roles are rotated from group to group: the one-wave steps of the inverse then run on different SIMDs
+    const int wave = (tid / WAVE + group) % 4;
     // ---- register prefetch of one item's inputs ----
     bf16x8 kx[NPASS], qx[NPASS];
     float gx = 0.f;

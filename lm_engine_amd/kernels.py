@@ -7,8 +7,14 @@ environment variables.  Its GatedDeltaNet layer is the one mixer without an entr
 module adds that entry, ``Kernel.gated_delta_rule``, with the same interface so the layer can
 guard the HIP operator the way the other mixers guard theirs.
 
-Difference from the reference: the flag is ON by default, and switching it off makes the
-operator raise: this package ships no second implementation to fall back to.
+Difference from the reference: ``gated_delta_rule`` is ON by default, and switching it off makes
+the operator raise: this package ships no second implementation to fall back to.
+
+``Kernel.gated_delta_rule_fused_launch`` (off by default, as every flag of the reference is) asks the
+chunked forward to run its prepare and scan steps as one launch where the shape allows it
+(``GDN_FLAG_FUSED_LAUNCH`` of the C ABI).  Results stay within the same parity gates, but they are not
+bit-identical to the two-kernel path, which batches that do not qualify (packed, left-padded, many
+sequences) still take: leave it off where runs are compared bit for bit.
 """
 
 from __future__ import annotations
@@ -20,9 +26,11 @@ from enum import Enum
 
 class Kernel(Enum):
     gated_delta_rule = "gated_delta_rule"
+    gated_delta_rule_fused_launch = "gated_delta_rule_fused_launch"
 
 
-_KERNELS: dict[Kernel, bool] = {kernel: True for kernel in Kernel}
+_ON_BY_DEFAULT = (Kernel.gated_delta_rule,)
+_KERNELS: dict[Kernel, bool] = {kernel: kernel in _ON_BY_DEFAULT for kernel in Kernel}
 
 
 def enable_kernels_from_env_variable() -> None:

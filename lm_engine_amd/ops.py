@@ -121,7 +121,8 @@ def _fill_args(q, k, v, g, beta, h0, ht, o, cu_seqlens, scale, l2norm, inplace, 
     a.dtype = _dtype_code(q.dtype, "q, k, v")
     a.beta_dtype = _lib.GDN_F32 if beta is None else _dtype_code(beta.dtype, "beta")
     a.flags = ((_lib.GDN_FLAG_L2NORM if l2norm else 0) | (_lib.GDN_FLAG_STATE_INPLACE if inplace else 0)
-               | (_lib.GDN_FLAG_LEFT_PADDED if left_padded else 0))  # fmt: skip
+               | (_lib.GDN_FLAG_LEFT_PADDED if left_padded else 0)
+               | (_lib.GDN_FLAG_FUSED_LAUNCH if is_kernel_allowed(Kernel.gated_delta_rule_fused_launch) else 0))  # fmt: skip
     a.scale = float(K**-0.5 if scale is None else scale)
     return a
 

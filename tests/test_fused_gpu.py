@@ -1,0 +1,116 @@
+"""The chunked forward as one launch (Kernel.gated_delta_rule_fused_launch / GDN_FLAG_FUSED_LAUNCH): producer
+workgroups run the prepare step while scan workgroups with two compute waves per state slice consume the records.
+Same parity gates against the CPU oracle as the two-kernel path (bf16: max-abs 2e-2 and relative-L2 1e-2 on the
+output and on the final state); shapes that do not qualify must fall back to the two-kernel path unchanged."""
+
+import pytest
+import torch
+
+import lm_engine_amd
+from lm_engine_amd.kernels import Kernel, enable_kernels
+from lm_engine_amd.ops import chunk_forward_kernel_times
+from lm_engine_amd.workloads import get_workload, make_inputs
+from oracle.c_oracle import recurrent_gated_delta_rule_c
+from tests.helpers import assert_parity, max_abs, random_inputs, rel_l2
+
+
+pytestmark = pytest.mark.gpu
+BF16 = torch.bfloat16
+FUSED = [Kernel.gated_delta_rule_fused_launch]
+
+
+def _to_gpu(inp):
+    return {n: (x.cuda() if isinstance(x, torch.Tensor) else x) for n, x in inp.items()}
+
+
+def _check(inp, label, **kwargs):
+    print(f"case: fused launch {label} q={tuple(inp['q'].shape)} v={tuple(inp['v'].shape)} {kwargs}", flush=True)
+    o_ref, h_ref = recurrent_gated_delta_rule_c(**inp, output_final_state=True, **kwargs)
+    with enable_kernels(FUSED):
+        o, ht = lm_engine_amd.chunk_gated_delta_rule(**_to_gpu(inp), output_final_state=True, **kwargs)
+    torch.cuda.synchronize()
+    print(f"   o: max-abs {max_abs(o.float(), o_ref):.3e} rel-L2 {rel_l2(o.float(), o_ref):.3e}   "
+          f"ht: max-abs {max_abs(ht, h_ref):.3e} rel-L2 {rel_l2(ht, h_ref):.3e}", flush=True)  # fmt: skip
+    assert_parity(o.float(), o_ref, BF16, "o")
+    assert_parity(ht, h_ref, BF16, "final_state")
+    return o, ht
+
+
+def test_the_flag_selects_the_single_launch():
+    # with the flag the prepare kernel is not launched: the interval between the events around it holds no kernel
+    inp = _to_gpu(random_inputs(B=2, T=4096, H=32, K=128, V=128, dtype=BF16, seed=149))
+    for _ in range(2):  # the first call of each loads its kernels
+        split = chunk_forward_kernel_times(**inp, output_final_state=True)
+        with enable_kernels(FUSED):
+            fused = chunk_forward_kernel_times(**inp, output_final_state=True)
+    print(f"kernel times, ms: two kernels {split}, one launch {fused}", flush=True)
+    assert fused["chunk_prepare"] < 0.5 * split["chunk_prepare"] and fused["chunk_scan"] > split["chunk_scan"]
+
+
+@pytest.mark.parametrize("T", [65, 128, 130, 321])
+def test_sequence_lengths_with_tail_chunks(T):
+    _check(random_inputs(B=2, T=T, H=2, K=128, V=128, dtype=BF16, seed=150 + T), f"T={T}")
+
+
+@pytest.mark.parametrize("K, V", [(64, 64), (64, 128), (128, 64), (128, 256)])
+def test_head_dims(K, V):
+    _check(random_inputs(B=1, T=200, H=3, K=K, V=V, dtype=BF16, seed=160 + K + V), f"K={K} V={V}")
+
+
+def test_options_l2norm_scale_no_state_ungated():
+    inp = random_inputs(B=2, T=257, H=2, K=128, V=128, dtype=BF16, seed=171, normalize=False)
+    _check(inp, "in-kernel l2norm, scale 0.3", use_qk_l2norm_in_kernel=True, scale=0.3)
+    inp = random_inputs(B=1, T=192, H=2, K=128, V=128, dtype=BF16, seed=172, gated=False, h0=False)
+    _check(dict(inp, beta=None), "ungated, beta = 1, zero state")
+
+
+def test_strided_projection_slices():
+    # q, k, v as slices of one fused projection, the way the layer passes them
+    gen = torch.Generator("cpu").manual_seed(173)
+    B, T, H, K, V = 1, 300, 4, 128, 128
+    proj = torch.randn(B, T, H * (2 * K + V), generator=gen).to(BF16)
+    q, k, v = (x.reshape(B, T, H, -1) for x in proj.split([H * K, H * K, H * V], dim=-1))
+    q = torch.nn.functional.normalize(q.float(), dim=-1).to(BF16)  # contiguous copy: only k and v stay strided
+    inp = dict(random_inputs(B, T, H, K, V, dtype=BF16, seed=174), q=q, k=k, v=v)
+    _check(inp, "strided k, v", use_qk_l2norm_in_kernel=True)
+
+
+def test_config1_full_size():
+    _check(make_inputs(get_workload(1)), "cfg1 full size")
+
+
+def test_config4_long_context_and_the_split_property():
+    # H=32, K=128, V=256, random initial state, T=8192 (128 chunks per chain; the full length is checked on the default path)
+    inp = make_inputs(get_workload(4, T=8192))
+    o, ht = _check(inp, "cfg4 at T=8192")
+    gpu = _to_gpu(inp)
+    cut = 64 * 45
+    with enable_kernels(FUSED):
+        first = {n: (x[:, :cut] if n in ("q", "k", "v", "g", "beta") else x) for n, x in gpu.items()}
+        o1, h1 = lm_engine_amd.chunk_gated_delta_rule(**first, output_final_state=True)
+        second = {n: (x[:, cut:] if n in ("q", "k", "v", "g", "beta") else x) for n, x in gpu.items()}
+        second["initial_state"] = h1
+        o2, h2 = lm_engine_amd.chunk_gated_delta_rule(**second, output_final_state=True)
+        o_again, h_again = lm_engine_amd.chunk_gated_delta_rule(**gpu, output_final_state=True)
+    torch.cuda.synchronize()
+    assert torch.equal(torch.cat([o1, o2], dim=1), o) and torch.equal(h2, ht), "split run differs from the full run"
+    assert torch.equal(o_again, o) and torch.equal(h_again, ht), "two runs of the same launch differ"
+
+
+def test_close_to_the_two_kernel_path_and_fallback_is_unchanged():
+    inp = _to_gpu(random_inputs(B=3, T=500, H=4, K=128, V=128, dtype=BF16, seed=180))
+    o_split, h_split = lm_engine_amd.chunk_gated_delta_rule(**inp, output_final_state=True)
+    with enable_kernels(FUSED):
+        o_fused, h_fused = lm_engine_amd.chunk_gated_delta_rule(**inp, output_final_state=True)
+    assert rel_l2(o_fused.float(), o_split.float()) < 5e-3 and rel_l2(h_fused, h_split) < 1e-3
+    # shapes that do not qualify take the two-kernel path whatever the flag says: packed sequences, V not a multiple of 64,
+    # more scan workgroups than three quarters of the CUs
+    packed = _to_gpu(random_inputs(B=1, T=300, H=2, K=128, V=128, dtype=BF16, seed=181, N=3))
+    cu = torch.tensor([0, 70, 71, 300], dtype=torch.int32, device="cuda")
+    odd_v = _to_gpu(random_inputs(B=1, T=130, H=2, K=128, V=96, dtype=BF16, seed=182))
+    many = _to_gpu(random_inputs(B=20, T=130, H=16, K=128, V=128, dtype=BF16, seed=183))
+    for case, extra in ((packed, dict(cu_seqlens=cu)), (odd_v, {}), (many, {})):
+        a = lm_engine_amd.chunk_gated_delta_rule(**case, output_final_state=True, **extra)
+        with enable_kernels(FUSED):
+            b = lm_engine_amd.chunk_gated_delta_rule(**case, output_final_state=True, **extra)
+        assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])

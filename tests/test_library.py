@@ -199,6 +199,15 @@ def test_kernel_flag_registry_follows_the_reference_convention():
     assert is_kernel_allowed(Kernel.gated_delta_rule)
 
 
+def test_fused_launch_flag_is_off_by_default():
+    fused = Kernel.gated_delta_rule_fused_launch
+    assert not is_kernel_allowed(fused)
+    with enable_kernels([fused]):
+        assert is_kernel_allowed(fused) and is_kernel_allowed(Kernel.gated_delta_rule)
+    assert not is_kernel_allowed(fused)
+    assert _lib.GDN_FLAG_FUSED_LAUNCH == 8
+
+
 def test_kernel_flag_env_variable():
     code = "from lm_engine_amd.kernels import Kernel, is_kernel_allowed; print(is_kernel_allowed(Kernel.gated_delta_rule))"
     run = lambda env: subprocess.run([sys.executable, "-c", code], env={**os.environ, **env}, cwd=ROOT,
