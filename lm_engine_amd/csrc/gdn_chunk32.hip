@@ -42,6 +42,8 @@
 
 #include <type_traits>
 
+#include <stdio.h>
+
 #include "gdn_chunk32_common.h"
 #include "gdn_chunk_prepare32.h"
 #include "gdn_launch.h"
@@ -102,6 +104,12 @@ __global__ __launch_bounds__(PREP_THREADS, 3) void chunk_prepare32_kernel(const 
 // asking).
 // ------------------------------------------------------------------------------------------
 constexpr int SCAN_LOADERS = 4;
+#ifdef GDN_EXP_TIMING
+__device__ unsigned long long g_dbg[64];
+#define STAMP(k) { const unsigned long long t1 = clock64(); tacc[k] += t1 - t0; t0 = t1; }
+#else
+#define STAMP(k)
+#endif
 
 // Waves of a scan workgroup.  The hardware deals the waves of a workgroup round over the four SIMDs (wave w runs on
 // SIMD w % 4), and a wave that shares a SIMD with a compute wave takes instruction-issue slots from it (measured:
@@ -110,7 +118,9 @@ constexpr int SCAN_LOADERS = 4;
 //   NW = 1:  0 compute | 1 2 3 loaders | 4 output store | 5 loader
 //   NW = 2:  0 1 compute | 2 3 loaders | 4 output store | 5 exits at once | 6 7 loaders
 //   NW = 4:  0..3 compute | 4..7 loaders (each compute wave shares with one loader; no output wave)
-__host__ __device__ constexpr int scan_waves(int nw) { return nw == 1 ? 6 : 8; }
+//   NW = 1, SPLIT:  0 state | 1 output | 2 3 loaders | 4 output store | 5 exits at once | 6 7 loaders
+//   NW = 1, HALF:   0 1 compute (16 columns each) | the rest as above
+__host__ __device__ constexpr int scan_waves(int nw, bool split = false) { return nw == 1 && !split ? 6 : 8; }
 
 // Order of the MFMAs of one chunk in the scan's compute wave, and where its side work goes.
 //
@@ -124,15 +134,20 @@ __host__ __device__ constexpr int scan_waves(int nw) { return nw == 1 ? 6 : 8; }
 // and the op that needs its result.  A lone wave issues an instruction every four to five cycles and an MFMA
 // occupies the matrix pipe for 33, so more than about six instructions between two MFMAs idle the pipe: the pieces
 // are spread one per op, earliest deadline first, as far as their windows allow.
-template <int K>
+//
+// SPLIT: the schedule of the state wave when a second wave of the workgroup computes the output (see the kernel):
+// no O^T groups, no output pieces; V~ goes to accumulators of its own (X of token tile 1 then has until the fifth
+// op of T' X), and the bf16 copy of the last state tile, which nothing in this chunk waits for any more, runs in a
+// tail slot behind the last MFMA.
+template <int K, bool SPLIT = false>
 struct ScanScheduleRules {
     static constexpr int KD = K / 32, KS16 = K / 16;
-    static constexpr int NSF = 2 * KS16, NQF = 2 * KS16, NTF = 6, NKF = 4 * KD, NPF = 6;
+    static constexpr int NSF = 2 * KS16, NQF = SPLIT ? 0 : 2 * KS16, NTF = 6, NKF = 4 * KD, NPF = SPLIT ? 0 : 6;
     static constexpr int NOPS = NSF + NQF + NTF + NKF + NPF;
-    static constexpr int LA = 6;
+    static constexpr int LA = SPLIT && K == 64 ? 3 : 6;
     static constexpr int OP_Q = NSF, OP_T = OP_Q + NQF, OP_K = OP_T + NTF, OP_P = OP_K + NKF, OP_BAR = NOPS - LA;
     static constexpr int AHEAD = 2;  // scales and rows of v are read this many ops before their piece
-    static_assert(OP_BAR >= OP_P, "the scales and v of this chunk are used before the barrier");
+    static_assert(SPLIT || OP_BAR >= OP_P, "the scales and v of this chunk are used before the barrier");
 
     // op j of the fourth group -> key tile, token slab
     static constexpr int k_tile(int j) { return (j % (2 * KD)) / 2; }
@@ -143,17 +158,17 @@ struct ScanScheduleRules {
 
     // pieces: X (4 registers) | output hand-over (half a tile) | q row scale (4 registers) | decay (4 registers) |
     // scaled V~ (half a fragment) | plain V~ (a fragment) | new state (a fragment) | X as operand (a fragment)
-    static constexpr int N_XC = 8, N_OUT = 4, N_AS = 8, N_DEC = 4 * KD, N_VS = 8, N_VB = 4, N_SB = 2 * KD, N_XB = 4;
+    static constexpr int N_XC = 8, N_OUT = SPLIT ? 0 : 4, N_AS = SPLIT ? 0 : 8, N_DEC = 4 * KD, N_VS = 8, N_VB = 4, N_SB = 2 * KD, N_XB = 4;
     static constexpr int P_XC = 0, P_OUT = P_XC + N_XC, P_AS = P_OUT + N_OUT, P_DEC = P_AS + N_AS, P_VS = P_DEC + N_DEC,
                          P_VB = P_VS + N_VS, P_SB = P_VB + N_VB, P_XB = P_SB + N_SB, NPIECES = P_XB + N_XB;
 
     struct Window {
-        int first, end;  // the piece runs before the MFMA of an op in [first, end)
+        int first, end;  // the piece runs before the MFMA of an op in [first, end); first >= NOPS: in the tail slot
     };
     static constexpr Window window(int pc) {
         if (pc < P_OUT) {  // K S0 of tile tt is complete after op KS16 (tt + 1) - 1; T' X overwrites tile 1 at its third op
             const int tt = (pc - P_XC) / 4;
-            return {KS16 * (tt + 1) + 1, OP_T + 2 * tt};
+            return {KS16 * (tt + 1) + 1, SPLIT ? OP_T + 4 * tt : OP_T + 2 * tt};
         }
         if (pc < P_AS) return {1, OP_Q + KS16 * ((pc - P_OUT) / 2)};  // the previous chunk's tile, before q overwrites it
         if (pc < P_DEC) {
@@ -166,10 +181,10 @@ struct ScanScheduleRules {
             const int x = (pc - P_VS) / 2;
             return {OP_T + (x / 2 == 0 ? 2 : 6) + 1, x < 2 ? OP_K + x : OP_K + NKF / 2 + (x - 2)};
         }
-        if (pc < P_SB) return {OP_T + ((pc - P_VB) / 2 == 0 ? 2 : 6) + 1, OP_P};
+        if (pc < P_SB) return {OP_T + ((pc - P_VB) / 2 == 0 ? 2 : 6) + 1, SPLIT ? OP_BAR : OP_P};  // (SPLIT: the output wave waits for it)
         if (pc < P_XB) return {OP_K + NKF / 2 + 2 * ((pc - P_SB) / 2) + 3, NOPS};
         const int tt = (pc - P_XB) / 2;  // after the two X pieces of its half tile (checked in make)
-        return {KS16 * (tt + 1) + 2, OP_T + 2 * tt};
+        return SPLIT ? Window{KS16 * (tt + 1) + 1, OP_T + 4 * tt} : Window{KS16 * (tt + 1) + 2, OP_T + 2 * tt};
     }
 
     struct Table {
@@ -193,6 +208,8 @@ struct ScanScheduleRules {
                 t.op[best] = op, done[best] = true, left--;
             }
         }
+        for (int pc = 0; pc < NPIECES; pc++)  // the tail slot
+            if (!done[pc] && window(pc).first >= NOPS) t.op[pc] = NOPS, done[pc] = true, left--;
         if (left != 0) t.ok = false;
         // a half tile of X is packed after its two pieces (within an op the pieces run in index order: X before the pack)
         for (int i = 0; i < N_XB; i++)
@@ -204,21 +221,156 @@ struct ScanScheduleRules {
             if (t.op[P_XC + i] - AHEAD <= t.op[P_XC + i - 4]) t.ok = false;
         for (int i = 0; i < N_VS; i++)
             if (t.op[P_VS + i] - AHEAD < 0) t.ok = false;
+        // the scales of this chunk are read before the barrier that releases its half of the stage
+        for (int i = 0; i < N_VS; i++)
+            if (t.op[P_VS + i] >= OP_BAR) t.ok = false;
+        for (int i = 0; i < N_XC; i++)
+            if (t.op[P_XC + i] >= OP_BAR) t.ok = false;
+        return t;
+    }
+};
+
+template <int K, bool SPLIT = false>
+struct ScanSchedule : ScanScheduleRules<K, SPLIT> {
+    static constexpr typename ScanScheduleRules<K, SPLIT>::Table TABLE = ScanScheduleRules<K, SPLIT>::make();
+    static_assert(TABLE.ok, "no placement of the side work satisfies the windows");
+    static constexpr int op_of(int pc) { return TABLE.op[pc]; }
+};
+
+// Schedule of the half-slice scan (HALF, see the kernel): the same five groups on v_mfma_f32_16x16x32_bf16, whose
+// tiles are 16 tokens or 16 keys by this wave's 16 columns: K S0 (K/32 slabs x 4 token tiles) | O^T (as many) |
+// V~ = T' X (6) | S += k^T V~' (2 token slabs x K/16 key tiles) | O^T += V~^T P^T (6).  Within a group consecutive
+// MFMAs go to different accumulators (the instruction has 4 passes: a dependent one right behind it would wait).
+// The pieces are half as large as in the whole-slice schedule; placement is the same earliest-deadline walk.  With
+// MFMAs this short an op can be over in 16 cycles, so results are taken DIST ops after their MFMA and LDS data
+// LA ops (operand fragments) or AHEAD ops (scales, rows of v) after the read was issued.
+template <int K>
+struct Scan16Rules {
+    static constexpr int KS = K / 32, KT = K / 16;
+    static constexpr int NSF = 4 * KS, NQF = 4 * KS, NTF = 6, NKF = 2 * KT, NPF = 6;
+    static constexpr int NOPS = NSF + NQF + NTF + NKF + NPF;
+    static constexpr int LA = 10;
+    static constexpr int OP_Q = NSF, OP_T = OP_Q + NQF, OP_K = OP_T + NTF, OP_P = OP_K + NKF, OP_BAR = NOPS - LA;
+    static constexpr int AHEAD = 4, DIST = 3;
+
+    // op j of the first two groups -> token tile, key slab
+    static constexpr int s_tile(int j) { return j % 4; }
+    static constexpr int s_slab(int j) { return j / 4; }
+    static constexpr int s_last(int tt) { return 4 * (KS - 1) + tt; }  // last op of tile tt
+    // op j of the third and fifth group -> token tile (16 tokens), slab of 32 reduction tokens: the non-zero blocks of a
+    // lower triangular 64 x 64 matrix, (0,0) (1,0) (2,0) (3,0) (2,1) (3,1); fragment (tile, slab) is number
+    // t_frag(j) of the record, where they are stored tile by tile
+    static constexpr int t_tile(int j) { return j < 4 ? j : j - 2; }
+    static constexpr int t_slab(int j) { return j < 4 ? 0 : 1; }
+    static constexpr int t_frag(int j) { return j < 2 ? j : j == 2 ? 2 : j == 3 ? 4 : j == 4 ? 3 : 5; }
+    static constexpr int t_first(int tt) { return tt; }                   // first op of tile tt ...
+    static constexpr int t_last(int tt) { return tt < 2 ? tt : tt + 2; }  // ... and its last
+    static constexpr int s_first(int s) { return s == 0 ? 0 : 4; }        // first op that reads slab s
+    static constexpr int k_tile(int j) { return j % KT; }
+    static constexpr int k_slab(int j) { return j / KT; }
+
+    // pieces: X of a token tile | X of a slab as operand | previous output tile to LDS | q row scale of a tile |
+    // decay of a state tile | scaled V~ of a token tile (half an operand) | plain V~ of a slab | new state slab
+    static constexpr int N_XC = 4, N_XB = 2, N_OUT = 4, N_AS = 4, N_DEC = KT, N_VS = 4, N_VB = 2, N_SB = KS;
+    static constexpr int P_XC = 0, P_XB = P_XC + N_XC, P_OUT = P_XB + N_XB, P_AS = P_OUT + N_OUT, P_DEC = P_AS + N_AS,
+                         P_VS = P_DEC + N_DEC, P_VB = P_VS + N_VS, P_SB = P_VB + N_VB, NPIECES = P_SB + N_SB;
+    struct Window {
+        int first, end;
+    };
+    static constexpr Window window(int pc) {
+        if (pc < P_XB) {
+            const int tt = pc - P_XC;
+            return {s_last(tt) + DIST, OP_T + s_first(tt / 2)};
+        }
+        if (pc < P_OUT) {
+            const int s = pc - P_XB;
+            return {s_last(2 * s + 1) + DIST, OP_T + s_first(s)};
+        }
+        if (pc < P_AS) return {DIST - 1, OP_Q + (pc - P_OUT)};  // (the last MFMA of the previous chunk was its last op)
+        if (pc < P_DEC) {
+            const int it = pc - P_AS;
+            const int end = OP_P + t_first(it);
+            return {OP_Q + s_last(it) + DIST, end < OP_BAR ? end : OP_BAR};
+        }
+        if (pc < P_VS) return {OP_Q, OP_K + (pc - P_DEC)};  // (not among the K S0 products: the X pieces and the output are there)
+        if (pc < P_VB) {
+            const int tt = pc - P_VS;
+            return {OP_T + t_last(tt) + DIST, OP_K + KT * (tt / 2)};
+        }
+        if (pc < P_SB) {
+            const int s = pc - P_VB;
+            return {OP_T + t_last(2 * s + 1) + DIST, OP_P + s_first(s)};
+        }
+        const int s = pc - P_SB;
+        return {OP_K + KT + 2 * s + 1 + DIST, NOPS};
+    }
+    struct Table {
+        int op[NPIECES];
+        bool ok;
+    };
+    static constexpr Table make() {
+        Table t{};
+        bool done[NPIECES] = {};
+        int left = NPIECES;
+        t.ok = true;
+        for (int op = 0; op < NOPS; op++) {
+            const int quota = (left + (NOPS - op) - 1) / (NOPS - op);
+            for (int n = 0;; n++) {
+                int best = -1;
+                for (int pc = 0; pc < NPIECES; pc++)
+                    if (!done[pc] && window(pc).first <= op && (best < 0 || window(pc).end < window(best).end)) best = pc;
+                if (best < 0) break;
+                if (n >= quota && window(best).end > op + 1) break;
+                if (window(best).end <= op) t.ok = false;  // window missed
+                t.op[best] = op, done[best] = true, left--;
+            }
+        }
+        if (left != 0) t.ok = false;
+        // a slab of X is packed after the X of both its tiles (within an op the pieces run in index order)
+        for (int s = 0; s < N_XB; s++)
+            if (t.op[P_XB + s] < t.op[P_XC + 2 * s] || t.op[P_XB + s] < t.op[P_XC + 2 * s + 1]) t.ok = false;
+        // what a piece reads of this chunk's half of the stage is read before the barrier; the decay and the row scale
+        // of q use values that the barrier op replaces
+        for (int i = 0; i < N_VS; i++)
+            if (t.op[P_VS + i] - AHEAD < 0 || t.op[P_VS + i] >= OP_BAR) t.ok = false;
+        for (int i = 0; i < N_XC; i++)
+            if (t.op[P_XC + i] - AHEAD < 0 || t.op[P_XC + i] >= OP_BAR) t.ok = false;
+        for (int i = 0; i < N_DEC; i++)
+            if (t.op[P_DEC + i] >= OP_BAR) t.ok = false;
+        for (int i = 0; i < N_AS; i++)
+            if (t.op[P_AS + i] >= OP_BAR) t.ok = false;
         return t;
     }
 };
 
 template <int K>
-struct ScanSchedule : ScanScheduleRules<K> {
-    static constexpr typename ScanScheduleRules<K>::Table TABLE = ScanScheduleRules<K>::make();
+struct Scan16Schedule : Scan16Rules<K> {
+    static constexpr typename Scan16Rules<K>::Table TABLE = Scan16Rules<K>::make();
     static_assert(TABLE.ok, "no placement of the side work satisfies the windows");
     static constexpr int op_of(int pc) { return TABLE.op[pc]; }
 };
 
 // NT: the loaders use non-temporal loads.  Right when no other workgroup reads the same lines (one workgroup per
 // chain; measured 7 % faster at 1024 chains), wrong when column groups share them through the L2 (8 % slower).
-template <int K, int NW, bool NT = false, bool SAVE = false>
-__global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(const ChunkParams p) {
+//
+// SPLIT (one slice per workgroup): the slice has two waves on two SIMDs.  A lone wave issues in order, and what
+// bounds the one-wave scan is its instruction count (per chunk and K = 128: 60 MFMAs at 8 issue cycles, 280 vector
+// instructions at 4.3, 97 LDS instructions at 7), not the matrix pipe.  So the products that nothing in the
+// recurrence waits for, O^T = S0^T q^T and O^T += V~^T P^T, their operand reads, the row scale of q and the bf16
+// output move to an output wave.  The state wave hands it the operands it has made anyway - the bf16 copy of the
+// state a chunk starts from and V~ - through a double-buffered LDS area, publishing each with an epoch word; nothing
+// flows back, so the state wave never waits for its partner (the workgroup barrier of a chunk, which the output
+// wave reaches first, also tells the state wave that the area's other half has been read).  Same arithmetic in the
+// same order as the one-wave scan: the results are bit-identical.
+//
+// HALF (one slice per workgroup): the slice has two waves, each with 16 of its columns, on v_mfma_f32_16x16x32_bf16.
+// A wave has the same number of MFMAs and operand reads as a whole-slice wave but half the accumulators, so half the
+// vector work on them (decay, X, the bf16 copies), and the two halves need nothing from each other.  The records must
+// hold the fragments of T diag(beta) and P in the layout of that instruction (ChunkParams::rec16).
+template <int K, int NW, bool NT = false, bool SAVE = false, bool SPLIT = false, bool HALF = false>
+__global__ __launch_bounds__(scan_waves(NW, SPLIT || HALF) * WAVE) void chunk_scan32_kernel(const ChunkParams p) {
+    static_assert(!SPLIT || (NW == 1 && !SAVE), "the split scan has one slice per workgroup and saves nothing");
+    static_assert(!HALF || (NW == 1 && !SAVE && !SPLIT), "the half-slice scan has one slice per workgroup and saves nothing");
     constexpr int NL = SCAN_LOADERS;
     // a separate wave writes the output (see below); with four compute waves the LDS has no room for its staging
     constexpr bool OS = NW < 4;
@@ -249,8 +401,14 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
     static_assert(SHARED_FRAGS % NL == 0 && V_UNITS % NL == 0 && (2 * Q_UNITS) % NL == 0, "the pieces must divide over the loader waves");
     static_assert(2 * STAGE_BYTES + (OS ? NW * 2 * C * 64 : 16) <= 160 * 1024, "stage exceeds LDS");
 
+    // SPLIT: what the state wave hands to the output wave, [chunk parity][state KS16 | V~ 4] fragments, and two epochs
+    constexpr int XCH_FRAGS = KS16 + 4;
+    static_assert(2 * STAGE_BYTES + (OS ? NW * 2 * C * 64 : 16) + (SPLIT ? 2 * XCH_FRAGS * FRAG_BYTES + 16 : 0) <= 160 * 1024, "stage exceeds LDS");
+
     __shared__ __attribute__((aligned(16))) uint8_t stage[2][STAGE_BYTES];
     __shared__ __attribute__((aligned(16))) uint8_t ostage[OS ? NW * 2 * C * 64 : 16];
+    __shared__ __attribute__((aligned(16))) uint8_t xch[SPLIT ? 2 : 1][SPLIT ? XCH_FRAGS * FRAG_BYTES : 16];
+    __shared__ int xch_epoch[2];  // chunks whose state copy / whose V~ the state wave has published
 
     const int lane = threadIdx.x % WAVE;
     const int wave = threadIdx.x / WAVE;
@@ -289,8 +447,10 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
     };
     // role of this wave (see scan_waves)
     const bool is_store = OS && wave == 4;
-    const bool is_loader = NW == 4 ? wave >= 4 : NW == 2 ? (wave == 2 || wave == 3 || wave >= 6) : (wave >= 1 && wave != 4);
-    if (NW == 2 && wave == 5) return;
+    constexpr bool EIGHT = NW == 2 || SPLIT || HALF;  // the wave layout of two compute waves
+    const bool is_loader = NW == 4 ? wave >= 4 : EIGHT ? (wave == 2 || wave == 3 || wave >= 6) : (wave >= 1 && wave != 4);
+    if (EIGHT && wave == 5) return;
+    if (SPLIT && threadIdx.x < 2) xch_epoch[threadIdx.x] = 0;  // (visible after the barrier below that every wave passes)
     if (is_store) {
         // ------------------------------ output store ------------------------------
         // The compute waves leave the bf16 output tile of chunk c in LDS while they work on chunk c + 1; this
@@ -325,7 +485,7 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
     if (is_loader) {
         // ------------------------------ loader ------------------------------
         // loader number 0..3, wave-uniform: unit numbers and bases stay scalar
-        const int lw = __builtin_amdgcn_readfirstlane(NW == 4 ? wave - 4 : NW == 2 ? (wave < 4 ? wave - 2 : wave - 4) : (wave < 4 ? wave - 1 : 3));
+        const int lw = __builtin_amdgcn_readfirstlane(NW == 4 ? wave - 4 : EIGHT ? (wave < 4 ? wave - 2 : wave - 4) : (wave < 4 ? wave - 1 : 3));
         // Slots 0 .. NF - 1 of this wave move record fragments lw * NF + (rotated slot), the next NV slots 1 KiB
         // pieces of the v rows, the last NQ slots pieces of the q and k rows.  Which kind a slot is, is known at
         // compile time, so there is no branch in these loops (a branch makes the compiler wait for every load in
@@ -418,6 +578,9 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
         // c - 1) and refill the freed registers with chunk c + 3.
         int c = 0;
         for (; c + 4 < nchunks; c += 2) {  // steady state: straight-line code, both reloads exist
+#ifdef GDN_EXP_NO_LOAD
+            if (c > 2) { __syncthreads(); __syncthreads(); continue; }
+#endif
             store_and_reload(buf1, sc1, c + 1, c + 3, yes);
             __syncthreads();
             store_and_reload(buf0, sc0, c + 2, c + 4, yes);
@@ -435,6 +598,274 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
             }
         }
         if (OS) __syncthreads();  // the hand-over of the last output tile
+        return;
+    }
+
+    [[maybe_unused]] lds_flag_t* const ep_state = (lds_flag_t*)&xch_epoch[0];
+    [[maybe_unused]] lds_flag_t* const ep_v = (lds_flag_t*)&xch_epoch[1];
+    if constexpr (SPLIT) {
+        if (wave == 1) {
+            // ------------------------------ output (SPLIT) ------------------------------
+            // O^T tile tt, register r: token 32 tt + l32, column 16 (r/8) + 8 h + r%8 of the slice (slice_col order)
+            constexpr int NQF = 2 * KS16, LAQ = 4;
+            auto q_frag = [&](const uint8_t* st, int j) {  // rows of q, token tile j / KS16, key slab j % KS16: B operand of S0^T q^T
+                return *reinterpret_cast<const bf16x8*>(st + Q_OFF + (32 * (j / KS16) + l32) * QLD + (16 * (j % KS16) + 8 * lh) * 2);
+            };
+            f32x16 acco[2];
+            __syncthreads();  // stage[0] holds chunk 0
+            for (int c = 0; c < nchunks; c++) {
+#ifdef GDN_EXP_NO_O
+                if (c > 0) { __syncthreads(); continue; }
+#endif
+                const uint8_t* st = stage[c & 1];
+                const bf16x8* xc = reinterpret_cast<const bf16x8*>(xch[c & 1]) + lane;
+                bf16x8 qf[NQF], so[KS16], pf[6], vo[4];
+#pragma unroll
+                for (int j = 0; j < LAQ; j++) qf[j] = q_frag(st, j);
+                const float qs0 = reinterpret_cast<const float*>(st + QS_OFF)[l32], qs1 = reinterpret_cast<const float*>(st + QS_OFF)[32 + l32];
+                pair_wait(ep_state, c + 1);  // the bf16 copy of the state this chunk starts from
+#pragma unroll
+                for (int i = 0; i < KS16; i++) so[i] = xc[i * WAVE];
+                __builtin_amdgcn_sched_barrier(0);
+                static_for<0, NQF>([&](auto jc) {
+                    constexpr int j = decltype(jc)::value, s = j % KS16, tt = j / KS16;
+                    if constexpr (j + LAQ < NQF) qf[j + LAQ] = q_frag(st, j + LAQ);
+                    else pf[j + LAQ - NQF] = reinterpret_cast<const bf16x8*>(st)[(6 + j + LAQ - NQF) * WAVE + lane];
+                    if constexpr (s == 0) {
+                        f32x16 zero;
+#pragma unroll
+                        for (int r = 0; r < 16; r++) zero[r] = 0.f;
+                        acco[tt] = mfma32_bf16(so[s], qf[j], zero);
+                    } else {
+                        acco[tt] = mfma32_bf16(so[s], qf[j], acco[tt]);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                });
+                static_assert(LAQ <= 6, "the six fragments of P are read behind the last rows of q");
+#pragma unroll
+                for (int f = LAQ; f < 6; f++) pf[f] = reinterpret_cast<const bf16x8*>(st)[(6 + f) * WAVE + lane];
+                __syncthreads();  // this wave has read what it needs of chunk c's half of the stage
+#pragma unroll
+                for (int r = 0; r < 16; r++) acco[0][r] *= qs0, acco[1][r] *= qs1;
+                pair_wait(ep_v, c + 1);  // V~ of this chunk
+#pragma unroll
+                for (int i = 0; i < 4; i++) vo[i] = xc[(KS16 + i) * WAVE];
+                __builtin_amdgcn_sched_barrier(0);
+                acco[0] = mfma32_bf16(vo[0], pf[0], acco[0]);  // O^T += V~^T P^T; P[i < 32][j >= 32] = 0 is skipped
+                acco[1] = mfma32_bf16(vo[0], pf[2], acco[1]);
+                acco[0] = mfma32_bf16(vo[1], pf[1], acco[0]);
+                acco[1] = mfma32_bf16(vo[1], pf[3], acco[1]);
+                acco[1] = mfma32_bf16(vo[2], pf[4], acco[1]);
+                acco[1] = mfma32_bf16(vo[3], pf[5], acco[1]);
+#pragma unroll
+                for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+                    for (int half = 0; half < 2; half++)
+                        *reinterpret_cast<bf16x8*>(ostage_at(0, c & 1, 32 * tt + l32, 2 * half + lh)) = pack8_16(acco[tt], half, 1.f);
+            }
+            __syncthreads();  // the store wave writes the last output tile
+            return;
+        }
+    }
+
+    if constexpr (HALF) {
+        // ------------------------------ compute (HALF) ------------------------------
+        // Lane (j, g) = (lane % 16, lane / 16).  Operands of the 16x16x32 MFMA: A[j][8 g + 0..7], B[8 g + 0..7][j]; its
+        // accumulator: D[4 g + r][j], r = 0..3.  This wave owns the 16 columns c0 + j of the slice.
+        //   state tile t (K / 16 of them), register r: key 32 (t / 2) + 8 g + 4 (t % 2) + r.  Tiles 2 s and 2 s + 1 together
+        //     hand a lane the 8 consecutive keys 32 s + 8 g + 0..7: one operand register set, usable as B of K S0 (rows
+        //     of k are read as they lie) and as A of O^T = S0^T q^T.
+        //   token tile tt of K S0, X, V~ (16 tokens each), register r: token 16 tt + 4 g + r.  Tiles 2 s and 2 s + 1 hand
+        //     over the tokens 32 s + 4 g + 0..3 and 32 s + 16 + 4 g + 0..3: the reduction order of every fragment of
+        //     T diag(beta), P and k^T that multiplies them.
+        //   O^T tile it, register r: column c0 + 4 g + r of token 16 it + j.
+        typedef Scan16Schedule<K> SCH;
+        constexpr int NOPS = SCH::NOPS, OP_Q = SCH::OP_Q, OP_T = SCH::OP_T, OP_K = SCH::OP_K, OP_P = SCH::OP_P, OP_BAR = SCH::OP_BAR;
+        constexpr int LA = SCH::LA, KS = SCH::KS, KT = SCH::KT;
+        const int j16 = lane % 16, g = lane / 16;
+        const int half = wave;  // 0 or 1
+        const int c0 = 32 * vgroup + 16 * half;
+        f32x4 S[KT];
+        auto st_key = [&](int t, int r) { return 32 * (t / 2) + 8 * g + 4 * (t % 2) + r; };
+        const int64_t st_off = ((int64_t)n * p.H + h) * K * p.V + c0 + j16;
+#pragma unroll
+        for (int t = 0; t < KT; t++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) S[t][r] = p.h0 != nullptr ? p.h0[st_off + (int64_t)st_key(t, r) * p.V] : 0.f;
+
+        auto lds_frag = [&](const uint8_t* st, auto opc) -> bf16x8 {
+            constexpr int op = decltype(opc)::value;
+            if constexpr (op < OP_T) {  // rows of k (A of K S0) or of q (B of S0^T q^T): token tile, 32-key slab
+                constexpr int jj = op < OP_Q ? op : op - OP_Q, sl = SCH::s_slab(jj), tt = SCH::s_tile(jj);
+                return *reinterpret_cast<const bf16x8*>(st + (op < OP_Q ? K_OFF : Q_OFF) + (16 * tt + j16) * QLD + (32 * sl + 8 * g) * 2);
+            } else if constexpr (op >= OP_K && op < OP_P) {
+                // k^T: row j of key tile t is key 32 (t / 2) + 8 (j / 4) + 4 (t % 2) + j % 4; tokens 32 s + 4 g + 0..3 and
+                // 32 s + 16 + 4 g + 0..3.  Two transposing loads; lane (4 r' + q) supplies keys base + 8 q + 0..3 of token row r'.
+                constexpr int sl = SCH::k_slab(op - OP_K), t = SCH::k_tile(op - OP_K);
+                const bf16_t* km = reinterpret_cast<const bf16_t*>(st + K_OFF) + (32 * sl + 4 * g + j16 / 4) * (QLD / 2) + 32 * (t / 2) + 4 * (t % 2) + 8 * (j16 % 4);
+                const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)km);
+                const s16x4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(km + 16 * (QLD / 2)));
+                const bf16x4 a4 = __builtin_bit_cast(bf16x4, a), b4 = __builtin_bit_cast(bf16x4, b);
+                bf16x8 r;
+#pragma unroll
+                for (int e = 0; e < 4; e++) r[e] = a4[e], r[4 + e] = b4[e];
+                return r;
+            } else {
+                constexpr int f = op < OP_K ? SCH::t_frag(op - OP_T) : 6 + SCH::t_frag(op - OP_P);  // T' | P are contiguous in the stage
+                return reinterpret_cast<const bf16x8*>(st)[f * WAVE + lane];
+            }
+        };
+        auto lds_eg = [&](const uint8_t* st) -> float { return *reinterpret_cast<const float*>(st + EG_OFF); };
+        auto lds_qs = [&](const uint8_t* st, int it) -> float { return reinterpret_cast<const float*>(st + QS_OFF)[16 * it + j16]; };
+        auto pack4x2 = [](const f32x4& a, const f32x4& b) {
+            bf16x8 r;
+#pragma unroll
+            for (int e = 0; e < 4; e++) r[e] = (bf16_t)a[e], r[4 + e] = (bf16_t)b[e];
+            return r;
+        };
+
+        f32x4 accv[4], vt[4], acco[4];
+        bf16x8 sb[KS], xb[2], vb[2], vbs[2], fnext[LA];
+        f32x4 ksr[4], csr[4];
+        bf16x4 xvr[4];
+        float egc, qsc[4];
+#pragma unroll
+        for (int it = 0; it < 4; it++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) acco[it][r] = 0.f;
+
+        __syncthreads();  // stage[0] holds chunk 0
+        egc = lds_eg(stage[0]);
+#pragma unroll
+        for (int it = 0; it < 4; it++) qsc[it] = lds_qs(stage[0], it);
+        static_for<0, LA>([&](auto i) { fnext[decltype(i)::value] = lds_frag(stage[0], i); });
+#pragma unroll
+        for (int sl = 0; sl < KS; sl++) sb[sl] = pack4x2(S[2 * sl], S[2 * sl + 1]);
+
+#ifdef GDN_EXP_TIMING
+        unsigned long long tacc[8] = {0, 0, 0, 0, 0, 0, 0, 0}, t0 = clock64();
+#endif
+        for (int c = 0; c < nchunks; c++) {
+            const uint8_t* st = stage[c & 1];
+            const uint8_t* stn = stage[(c + 1) & 1];
+            bf16x8 fr[NOPS];
+#pragma unroll
+            for (int i = 0; i < LA; i++) fr[i] = fnext[i];
+            __builtin_amdgcn_sched_barrier(0);
+
+            auto run_piece = [&](auto pcc) {
+                constexpr int pc = decltype(pcc)::value;
+                if constexpr (pc < SCH::P_XB) {  // X = V - diag(cs) (K S0), token tile tt
+                    constexpr int tt = pc - SCH::P_XC;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) accv[tt][e] = (float)xvr[tt][e] - csr[tt][e] * accv[tt][e];
+                } else if constexpr (pc < SCH::P_OUT) {
+                    constexpr int sl = pc - SCH::P_XB;
+                    xb[sl] = pack4x2(accv[2 * sl], accv[2 * sl + 1]);
+                } else if constexpr (pc < SCH::P_AS) {  // output tile `it` of the previous chunk: 4 columns of token 16 it + j
+                    constexpr int it = pc - SCH::P_OUT;
+                    if (c > 0) {
+                        bf16x4 o4;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) o4[e] = (bf16_t)acco[it][e];
+                        *reinterpret_cast<bf16x4*>(ostage_at(0, (c - 1) & 1, 16 * it + j16, 2 * half + g / 2) + 8 * (g % 2)) = o4;
+                    }
+                } else if constexpr (pc < SCH::P_DEC) {
+                    constexpr int it = pc - SCH::P_AS;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) acco[it][e] *= qsc[it];
+                } else if constexpr (pc < SCH::P_VS) {
+                    constexpr int t = pc - SCH::P_DEC;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) S[t][e] *= egc;
+                } else if constexpr (pc < SCH::P_VB) {  // V~ of token tile tt with its rows scaled for the state update
+                    constexpr int tt = pc - SCH::P_VS;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) vbs[tt / 2][4 * (tt % 2) + e] = (bf16_t)(vt[tt][e] * ksr[tt][e]);
+                } else if constexpr (pc < SCH::P_SB) {
+                    constexpr int sl = pc - SCH::P_VB;
+                    vb[sl] = pack4x2(vt[2 * sl], vt[2 * sl + 1]);
+                } else {
+                    constexpr int sl = pc - SCH::P_SB;
+                    sb[sl] = pack4x2(S[2 * sl], S[2 * sl + 1]);
+                    pin_regs(sb[sl]);
+                }
+            };
+
+            static_for<0, NOPS>([&](auto opc) {
+                constexpr int op = decltype(opc)::value;
+                if constexpr (op + LA < NOPS) fr[op + LA] = lds_frag(st, std::integral_constant<int, (op + LA < NOPS ? op + LA : 0)>{});
+                if constexpr (op == OP_BAR) {
+                    __syncthreads();  // this wave is done with chunk c's half; chunk c + 1 is in the other one
+                    egc = lds_eg(stn);
+#pragma unroll
+                    for (int it = 0; it < 4; it++) qsc[it] = lds_qs(stn, it);
+                }
+                if constexpr (op >= OP_BAR) fnext[op >= OP_BAR ? op - OP_BAR : 0] = lds_frag(stn, std::integral_constant<int, (op >= OP_BAR ? op - OP_BAR : 0)>{});
+                static_for<0, SCH::N_VS>([&](auto ic) {
+                    constexpr int i = decltype(ic)::value;
+                    if constexpr (SCH::op_of(SCH::P_VS + i) - SCH::AHEAD == op)
+                        ksr[i] = *reinterpret_cast<const f32x4*>(st + KS_OFF + (16 * i + 4 * g) * 4);
+                });
+                static_for<0, SCH::N_XC>([&](auto ic) {
+                    constexpr int i = decltype(ic)::value;
+                    if constexpr (SCH::op_of(SCH::P_XC + i) - SCH::AHEAD == op) {
+                        csr[i] = *reinterpret_cast<const f32x4*>(st + CS_OFF + (16 * i + 4 * g) * 4);
+                        xvr[i] = lds_read_tr4x16<false>(reinterpret_cast<const bf16_t*>(st + V_OFF), VLD / 2, 16 * i + 4 * g, 16 * half, j16);
+                    }
+                });
+                static_for<0, SCH::NPIECES>([&](auto pcc) {
+                    if constexpr (SCH::op_of(decltype(pcc)::value) == op) run_piece(pcc);
+                });
+
+#ifdef GDN_EXP_TIMING
+                if constexpr (op == 0) STAMP(0)
+                if constexpr (op == OP_Q) STAMP(1)
+                if constexpr (op == OP_T) STAMP(2)
+                if constexpr (op == OP_K) STAMP(3)
+                if constexpr (op == OP_K + KT) STAMP(4)
+                if constexpr (op == OP_P) STAMP(5)
+                if constexpr (op == OP_BAR + 1) STAMP(6)
+#endif
+                const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+                if constexpr (op < OP_Q) {  // K S0
+                    constexpr int sl = SCH::s_slab(op), tt = SCH::s_tile(op);
+                    accv[tt] = mfma_bf16(fr[op], sb[sl], sl == 0 ? zero : accv[tt]);
+                } else if constexpr (op < OP_T) {  // O^T = S0^T q^T, scaled per token by a later piece
+                    constexpr int jj = op - OP_Q, sl = SCH::s_slab(jj), it = SCH::s_tile(jj);
+                    acco[it] = mfma_bf16(sb[sl], fr[op], sl == 0 ? zero : acco[it]);
+                } else if constexpr (op < OP_K) {  // V~ = T' X
+                    constexpr int jj = op - OP_T, tt = SCH::t_tile(jj), sl = SCH::t_slab(jj);
+                    vt[tt] = mfma_bf16(fr[op], xb[sl], sl == 0 ? zero : vt[tt]);
+                } else if constexpr (op < OP_P) {  // S = e^{gamma_C} S + k^T (row-scaled V~)
+                    constexpr int sl = SCH::k_slab(op - OP_K), t = SCH::k_tile(op - OP_K);
+                    S[t] = mfma_bf16(fr[op], vbs[sl], S[t]);
+                } else {  // O^T += V~^T P^T
+                    constexpr int jj = op - OP_P, it = SCH::t_tile(jj), sl = SCH::t_slab(jj);
+                    acco[it] = mfma_bf16(vb[sl], fr[op], acco[it]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            });
+        }
+        if (nchunks > 0) {
+#pragma unroll
+            for (int it = 0; it < 4; it++) {
+                bf16x4 o4;
+#pragma unroll
+                for (int e = 0; e < 4; e++) o4[e] = (bf16_t)acco[it][e];
+                *reinterpret_cast<bf16x4*>(ostage_at(0, (nchunks - 1) & 1, 16 * it + j16, 2 * half + g / 2) + 8 * (g % 2)) = o4;
+            }
+        }
+        __syncthreads();  // the store wave writes the last output tile
+#ifdef GDN_EXP_TIMING
+        if (lane == 0 && blockIdx.x == 40 && wave == 0) for (int i = 0; i < 8; i++) g_dbg[i] = tacc[i] / (nchunks > 0 ? nchunks : 1);
+#endif
+        if (p.ht != nullptr) {
+#pragma unroll
+            for (int t = 0; t < KT; t++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) p.ht[st_off + (int64_t)st_key(t, r) * p.V] = S[t][r];
+        }
         return;
     }
 
@@ -463,7 +894,7 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
 
     // MFMA schedule of one chunk: K S0 | q | T' X | k^T | P; the side work sits between the MFMAs at the ops
     // ScanSchedule<K> assigns.
-    typedef ScanSchedule<K> SCH;
+    typedef ScanSchedule<K, SPLIT> SCH;
     constexpr int NOPS = SCH::NOPS, OP_Q = SCH::OP_Q, OP_T = SCH::OP_T, OP_K = SCH::OP_K, OP_P = SCH::OP_P, OP_BAR = SCH::OP_BAR;
     constexpr int LA = SCH::LA;  // LDS reads are issued this many MFMAs ahead of their use
     const int l16 = lane % 16, g16 = l32 / 16;
@@ -494,6 +925,8 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
     auto lds_qs = [&](const uint8_t* st, int tt) -> float { return reinterpret_cast<const float*>(st + QS_OFF)[32 * tt + l32]; };
 
     f32x16 accv[2], acco[2];
+    [[maybe_unused]] f32x16 vts[2];             // SPLIT: V~ has accumulators of its own
+    f32x16(&vt)[2] = SPLIT ? vts : accv;
     bf16x8 sb[KS16], xb[4], vb[4], vbs[4], fnext[LA];  // xb: X, vb: V~, vbs: V~ with its rows scaled for the state update
     f32x4 ksr[4], csr[4];                              // row scales on their way to the pieces that use them
     bf16x4 xvr[4];                                     // and rows of v
@@ -503,12 +936,26 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
 
     // what the tail of a chunk does for the next one, for chunk 0
     egc = lds_eg(stage[0]);
-    qsc[0] = lds_qs(stage[0], 0), qsc[1] = lds_qs(stage[0], 1);
+    if constexpr (!SPLIT) qsc[0] = lds_qs(stage[0], 0), qsc[1] = lds_qs(stage[0], 1);
     static_for<0, LA>([&](auto i) { fnext[decltype(i)::value] = lds_frag(stage[0], i); });
 #pragma unroll
     for (int s = 0; s < KS16; s++) sb[s] = pack8_16(S[s / 2], s % 2, 1.f);
+    if constexpr (SPLIT) {  // the output wave's copy of the state chunk 0 starts from
+#pragma unroll
+        for (int s = 0; s < KS16; s++) reinterpret_cast<bf16x8*>(xch[0])[s * WAVE + lane] = sb[s];
+        pair_publish(ep_state, 1);
+    }
+    // SPLIT: the op whose pieces complete V~ for the output wave
+    constexpr int LAST_VB_OP = [] {
+        int m = 0;
+        for (int i = 0; i < SCH::N_VB; i++) m = SCH::op_of(SCH::P_VB + i) > m ? SCH::op_of(SCH::P_VB + i) : m;
+        return m;
+    }();
 
     int valid_prev = 0;  // tokens of the previous chunk, whose output is still in acco
+#ifdef GDN_EXP_TIMING
+    unsigned long long tacc[8] = {0, 0, 0, 0, 0, 0, 0, 0}, t0 = clock64();
+#endif
     for (int c = 0; c < nchunks; c++) {
         const uint8_t* st = stage[c & 1];
         const uint8_t* stn = stage[(c + 1) & 1];
@@ -572,16 +1019,18 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
                 // V~ as operand of k^T V~: each row (token) scaled by e^{gamma_C - gamma} / |k|; half a fragment
                 constexpr int i = pc - SCH::P_VS, x = i / 2, sub = i % 2, tt = x / 2, half = x % 2;
 #pragma unroll
-                for (int e = 0; e < 4; e++) vbs[x][4 * sub + e] = (bf16_t)(accv[tt][8 * half + 4 * sub + e] * ksr[i % 4][e]);
+                for (int e = 0; e < 4; e++) vbs[x][4 * sub + e] = (bf16_t)(vt[tt][8 * half + 4 * sub + e] * ksr[i % 4][e]);
             } else if constexpr (pc >= SCH::P_VB && pc < SCH::P_VB + SCH::N_VB) {
                 constexpr int i = pc - SCH::P_VB;  // V~ as operand of P V~
-                vb[i] = pack8_16(accv[i / 2], i % 2, 1.f);
+                vb[i] = pack8_16(vt[i / 2], i % 2, 1.f);
+                if constexpr (SPLIT) reinterpret_cast<bf16x8*>(xch[c & 1])[(KS16 + i) * WAVE + lane] = vb[i];
             } else {
                 // the new state tile as operand of the next chunk; pinned here, or the compiler moves all of them
                 // behind the last MFMA of the loop
                 constexpr int i = pc - SCH::P_SB;
                 sb[i] = pack8_16(S[i / 2], i % 2, 1.f);
                 pin_regs(sb[i]);
+                if constexpr (SPLIT) reinterpret_cast<bf16x8*>(xch[(c + 1) & 1])[i * WAVE + lane] = sb[i];  // (freed by the barrier of this chunk)
             }
         };
 
@@ -592,7 +1041,7 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
             if constexpr (op == OP_BAR) {
                 __syncthreads();  // this wave is done with chunk c's half; chunk c + 1 is in the other one
                 egc = lds_eg(stn);
-                qsc[0] = lds_qs(stn, 0), qsc[1] = lds_qs(stn, 1);  // this chunk's scales were applied before the barrier
+                if constexpr (!SPLIT) qsc[0] = lds_qs(stn, 0), qsc[1] = lds_qs(stn, 1);  // this chunk's scales were applied before the barrier
             }
             if constexpr (op >= OP_BAR) fnext[op >= OP_BAR ? op - OP_BAR : 0] = lds_frag(stn, std::integral_constant<int, (op >= OP_BAR ? op - OP_BAR : 0)>{});
             // row scales and rows of v, a few ops ahead of the piece that uses them
@@ -613,7 +1062,17 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
             static_for<0, SCH::NPIECES>([&](auto pcc) {
                 if constexpr (SCH::op_of(decltype(pcc)::value) == op) run_piece(pcc);
             });
+            if constexpr (SPLIT && op == LAST_VB_OP) pair_publish(ep_v, c + 1);
 
+#ifdef GDN_EXP_TIMING
+            if constexpr (op == 0) STAMP(0)
+            if constexpr (op == KS16) STAMP(1)
+            if constexpr (op == OP_T) STAMP(2)
+            if constexpr (op == OP_T + 4) STAMP(3)
+            if constexpr (op == OP_K) STAMP(4)
+            if constexpr (op == OP_K + SCH::NKF / 2) STAMP(5)
+            if constexpr (op == OP_BAR + 1) STAMP(6)
+#endif
             // ---- the MFMA ----
             if constexpr (op < OP_Q) {  // K S0, fragment (tt, s): rows = tokens
                 constexpr int s = op % KS16, tt = op / KS16;
@@ -641,9 +1100,9 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
                     f32x16 zero;
 #pragma unroll
                     for (int r = 0; r < 16; r++) zero[r] = 0.f;
-                    accv[tt] = mfma32_bf16(fr[op], xb[s], zero);
+                    vt[tt] = mfma32_bf16(fr[op], xb[s], zero);
                 } else {
-                    accv[tt] = mfma32_bf16(fr[op], xb[s], accv[tt]);
+                    vt[tt] = mfma32_bf16(fr[op], xb[s], vt[tt]);
                 }
             } else if constexpr (op < OP_P) {  // S = e^{gamma_C} S + k^T (row-scaled V~), fragment (td, s)
                 constexpr int s = SCH::k_slab(op - OP_K), td = SCH::k_tile(op - OP_K);
@@ -655,6 +1114,12 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
             }
             __builtin_amdgcn_sched_barrier(0);
         });
+        if constexpr (SPLIT) {  // the tail slot, and the state the next chunk starts from is complete in LDS
+            static_for<0, SCH::NPIECES>([&](auto pcc) {
+                if constexpr (SCH::op_of(decltype(pcc)::value) == NOPS) run_piece(pcc);
+            });
+            pair_publish(ep_state, c + 2);
+        }
         if constexpr (SAVE) {
             // V~ of this chunk: tile tt, register r holds token 32 tt + 8 (r/4) + 4 h + r%4 of this lane's column
             if (p.save_vnew != nullptr && c % p.save_every == 0 && c / p.save_every < p.save_nc) {
@@ -675,7 +1140,7 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
 
     // the output of the last chunk
 #pragma unroll
-    for (int tt = 0; tt < 2; tt++)
+    for (int tt = 0; tt < 2 && !SPLIT; tt++)
 #pragma unroll
         for (int half = 0; half < 2; half++) {
             if (OS) {
@@ -688,6 +1153,9 @@ __global__ __launch_bounds__(scan_waves(NW) * WAVE) void chunk_scan32_kernel(con
             }
         }
     if (OS) __syncthreads();
+#ifdef GDN_EXP_TIMING
+    if (lane == 0 && blockIdx.x == 40) for (int i = 0; i < 8; i++) g_dbg[i] = tacc[i] / (nchunks > 0 ? nchunks : 1);
+#endif
 
     if (p.ht != nullptr) {
 #pragma unroll
@@ -708,17 +1176,12 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     const int64_t cap = (int64_t)(3 * num_cus + 7) / 8 * 8;      // three workgroups per CU (LDS and registers allow it)
     if (items >= ((int64_t)1 << 31)) return GDN_ERR_UNSUPPORTED;  // the kernel counts items in 32 bits
     const int grid_prep = (int)(items < cap ? items : cap);
+    p.rec16 = 0;
     if (p.fused) {  // prepare and scan in one launch, when the shape qualifies
         if (events != nullptr) (void)hipEventRecord(events[2], stream);
         const int rc = launch_chunk_fused(p, K, stream, num_cus);
         if (rc != GDN_ERR_UNSUPPORTED) return rc;
     }
-    if (!p.records_given) {
-        hipLaunchKernelGGL((chunk_prepare32_kernel<K>), dim3(grid_prep), dim3(PREP_THREADS), 0, stream, p);
-        if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
-    }
-    if (events != nullptr) (void)hipEventRecord(events[2], stream);
-
     // Compute waves (32-column slices) per scan workgroup: one while that gives no more workgroups than CUs, so
     // that every slice has a CU's load bandwidth to itself; otherwise 2 or 4 slices of a chain share the
     // records through one workgroup's LDS (they must divide the V / 32 tiles).
@@ -729,6 +1192,18 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     while (nw < 4 && vtiles % (2 * nw) == 0 && chains * (vtiles / nw) > (int64_t)num_cus) nw *= 2;
     const bool save = p.save_state != nullptr || p.save_vnew != nullptr;
     if (save && nw == 2) nw = 1;  // the saving variant exists for 1 and 4 slices per workgroup
+    // a slice with a CU to itself is scanned by two waves of 16 columns each; the records are laid out for them
+#if defined(GDN_NO_SPLIT) || defined(GDN_SPLIT)
+    const bool half = false;
+#else
+    const bool half = nw == 1 && !save && !p.records_given;
+#endif
+    p.rec16 = half ? 1 : 0;
+    if (!p.records_given) {
+        hipLaunchKernelGGL((chunk_prepare32_kernel<K>), dim3(grid_prep), dim3(PREP_THREADS), 0, stream, p);
+        if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
+    }
+    if (events != nullptr) (void)hipEventRecord(events[2], stream);
     p.scan_groups = vtiles / nw;
     const dim3 grid((unsigned)(chains8 * p.scan_groups));
     if (save) {
@@ -739,10 +1214,28 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     if (nw == 4 && p.scan_groups == 1) hipLaunchKernelGGL((chunk_scan32_kernel<K, 4, true>), grid, dim3(scan_waves(4) * WAVE), 0, stream, p);
     else if (nw == 4) hipLaunchKernelGGL((chunk_scan32_kernel<K, 4>), grid, dim3(scan_waves(4) * WAVE), 0, stream, p);
     else if (nw == 2) hipLaunchKernelGGL((chunk_scan32_kernel<K, 2>), grid, dim3(scan_waves(2) * WAVE), 0, stream, p);
+#if defined(GDN_NO_SPLIT)
     else hipLaunchKernelGGL((chunk_scan32_kernel<K, 1>), grid, dim3(scan_waves(1) * WAVE), 0, stream, p);
+#elif defined(GDN_SPLIT)
+    else hipLaunchKernelGGL((chunk_scan32_kernel<K, 1, false, false, true>), grid, dim3(scan_waves(1, true) * WAVE), 0, stream, p);
+#else
+    else if (half) hipLaunchKernelGGL((chunk_scan32_kernel<K, 1, false, false, false, true>), grid, dim3(scan_waves(1, true) * WAVE), 0, stream, p);
+    else hipLaunchKernelGGL((chunk_scan32_kernel<K, 1>), grid, dim3(scan_waves(1) * WAVE), 0, stream, p);
+#endif
     return (int)hipGetLastError();
 }
 
+#ifdef GDN_EXP_TIMING
+extern "C" void gdn_dbg_dump() {
+    unsigned long long h[8];
+    (void)hipDeviceSynchronize();
+    (void)hipMemcpyFromSymbol(h, HIP_SYMBOL(g_dbg), sizeof(h));
+    printf("cycles per chunk up to op 0 | KS16 | OP_T | OP_T+4 | OP_K | OP_K+NKF/2 | OP_BAR+1 :");
+    unsigned long long sum = 0;
+    for (int i = 0; i < 7; i++) printf(" %llu", h[i]), sum += h[i];
+    printf("  total %llu\n", sum);
+}
+#endif
 int launch_chunk32(ChunkParams& p, int K, hipStream_t stream, hipEvent_t* events, int num_cus) {
     if (K == 64) return launch32<64>(p, stream, events, num_cus);
     if (K == 128) return launch32<128>(p, stream, events, num_cus);

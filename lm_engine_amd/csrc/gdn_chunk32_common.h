@@ -1,4 +1,4 @@
-// Device helpers shared by the kernels built on v_mfma_f32_32x32x16_bf16 (gdn_chunk32.hip, gdn_chunk_pair.hip).
+// Device helpers shared by the kernels built on v_mfma_f32_32x32x16_bf16 (gdn_chunk32.hip, gdn_chunk_fused.hip).
 #pragma once
 
 #include <type_traits>
@@ -48,6 +48,36 @@ __device__ __forceinline__ void pin_regs(bf16x8& x) {
     i32x4 t = __builtin_bit_cast(i32x4, x);
     asm volatile("" : "+v"(t));
     x = __builtin_bit_cast(bf16x8, t);
+}
+
+// ---- hand-over between two waves of a workgroup through LDS ----
+// A wave publishes what it wrote to LDS by storing a running epoch number to an LDS word of its own; the other wave
+// polls that word.  LDS operations of a wave execute in order, so whoever reads the new epoch reads the data written
+// before it.  The words are addressed as LDS explicitly: through a generic pointer the compiler emits FLAT accesses,
+// which take the vector-memory path and are not ordered with the DS instructions around them.
+typedef __attribute__((address_space(3))) volatile int lds_flag_t;
+
+__device__ __forceinline__ void pair_publish(lds_flag_t* flag, int epoch) {
+    asm volatile("" ::: "memory");
+    *flag = epoch;
+    asm volatile("" ::: "memory");
+}
+
+// The wait is one asm statement, loop included, so that the chunk loop of a compute wave stays a single basic
+// block: with a branch in it the compiler sinks work that is not needed until after the wait past it, out of the
+// slots it was written into.  All lanes read the same word.
+__device__ __forceinline__ void pair_wait(lds_flag_t* flag, int epoch) {
+    int seen, uniform;
+    asm volatile(
+        "pair_wait_%=:\n\t"
+        "ds_read_b32 %0, %2\n\t"
+        "s_waitcnt lgkmcnt(0)\n\t"
+        "v_readfirstlane_b32 %1, %0\n\t"
+        "s_cmp_lt_i32 %1, %3\n\t"
+        "s_cbranch_scc1 pair_wait_%="
+        : "=&v"(seen), "=&s"(uniform)
+        : "v"((uint32_t)(uintptr_t)flag), "s"(epoch)
+        : "memory", "scc");
 }
 
 }  // namespace gdn

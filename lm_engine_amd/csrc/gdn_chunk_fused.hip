@@ -46,34 +46,7 @@ constexpr int PAIR_THREADS = 8 * WAVE;
 constexpr int PAIR_LOADERS = 4;
 
 // Epochs: a wave stores 3 c + 1 once its half of the state chunk c starts from is in LDS, 3 c + 2 (wave 0
-// only) after X of token tile 0, 3 c + 3 after its tile of V~.
-// The flags are addressed as LDS explicitly: through a generic pointer the compiler emits FLAT accesses, which
-// take the vector-memory path and are not ordered with the DS instructions around them.
-typedef __attribute__((address_space(3))) volatile int lds_flag_t;
-
-__device__ __forceinline__ void pair_publish(lds_flag_t* flag, int epoch) {
-    asm volatile("" ::: "memory");
-    *flag = epoch;
-    asm volatile("" ::: "memory");
-}
-
-// The wait is one asm statement, loop included, so that the chunk loop of a compute wave stays a single basic
-// block: with a branch in it the compiler sinks work that is not needed until after the wait (the decay, the output
-// products) past it, out of the slots they were written into.  All lanes read the same word.
-__device__ __forceinline__ void pair_wait(lds_flag_t* flag, int epoch) {
-    int seen, uniform;
-    asm volatile(
-        "pair_wait_%=:\n\t"
-        "ds_read_b32 %0, %2\n\t"
-        "s_waitcnt lgkmcnt(0)\n\t"
-        "v_readfirstlane_b32 %1, %0\n\t"
-        "s_cmp_lt_i32 %1, %3\n\t"
-        "s_cbranch_scc1 pair_wait_%="
-        : "=&v"(seen), "=&s"(uniform)
-        : "v"((uint32_t)(uintptr_t)flag), "s"(epoch)
-        : "memory", "scc");
-}
-
+// only) after X of token tile 0, 3 c + 3 after its tile of V~ (pair_publish / pair_wait).
 
 #define PIN() __builtin_amdgcn_sched_barrier(0)
 

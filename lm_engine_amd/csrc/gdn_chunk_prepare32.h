@@ -31,6 +31,13 @@ __device__ __forceinline__ void record_store(uint8_t* rec, uint32_t bytes, uint3
         __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), __builtin_amdgcn_make_buffer_rsrc(rec, 0, bytes, 0x00020000), offset, 0, 16);
     else *reinterpret_cast<bf16x8*>(rec + offset) = v;
 }
+typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
+template <bool DEVICE_SCOPE>
+__device__ __forceinline__ void record_store(uint8_t* rec, uint32_t bytes, uint32_t offset, bf16x4 v) {
+    if constexpr (DEVICE_SCOPE)
+        __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, v), __builtin_amdgcn_make_buffer_rsrc(rec, 0, bytes, 0x00020000), offset, 0, 16);
+    else *reinterpret_cast<bf16x4*>(rec + offset) = v;
+}
 template <bool DEVICE_SCOPE>
 __device__ __forceinline__ void record_store(uint8_t* rec, uint32_t bytes, uint32_t offset, float v) {
     if constexpr (DEVICE_SCOPE)
@@ -270,10 +277,27 @@ __device__ __forceinline__ void chunk_prepare32_body(const ChunkParams& p, uint8
                             pv[4 * q + e] = (i >= j0 + e) ? val : 0.f;
                         }
                     }
-                    // fragments (tcol, 2 trow + s); the all-zero pair (tcol 0, trow 1) has no place in the record
-                    const int first = tcol == 0 ? 0 : 2 + 2 * trow;
-                    record_store<FLAGS>(rec, p.rec_bytes, p.off_p + ((first + 0) * WAVE + lane) * 16, pack8_16(pv, 0, 1.f));
-                    record_store<FLAGS>(rec, p.rec_bytes, p.off_p + ((first + 1) * WAVE + lane) * 16, pack8_16(pv, 1, 1.f));
+                    if (p.rec16) {
+                        // 16x16x32 fragments (it, s): 16 output tokens 16 it .. of P, 32 reduction tokens 32 s ..; lane
+                        // (i, g) of a fragment holds P[16 it + i][32 s + 4 g + 0..3] and P[16 it + i][32 s + 16 + 4 g + 0..3].
+                        // This lane has token i = 32 tcol + l32 and, in register quad q, tokens j = 32 trow + 8 q + 4 h + 0..3:
+                        // a half of lane (l32 % 16, 2 (q % 2) + h) of fragment (2 tcol + l32 / 16, trow).
+                        const int it = 2 * tcol + l32 / 16;
+                        const int frag = it < 2 ? it : 2 * it - 2 + trow;  // (0,0) (1,0) (2,0) (2,1) (3,0) (3,1)
+#pragma unroll
+                        for (int q = 0; q < 4; q++) {
+                            bf16x4 piece;
+#pragma unroll
+                            for (int e = 0; e < 4; e++) piece[e] = (bf16_t)pv[4 * q + e];
+                            const int g = 2 * (q % 2) + lh;
+                            record_store<FLAGS>(rec, p.rec_bytes, p.off_p + (frag * WAVE + 16 * g + l32 % 16) * 16 + 8 * (q / 2), piece);
+                        }
+                    } else {
+                        // fragments (tcol, 2 trow + s); the all-zero pair (tcol 0, trow 1) has no place in the record
+                        const int first = tcol == 0 ? 0 : 2 + 2 * trow;
+                        record_store<FLAGS>(rec, p.rec_bytes, p.off_p + ((first + 0) * WAVE + lane) * 16, pack8_16(pv, 0, 1.f));
+                        record_store<FLAGS>(rec, p.rec_bytes, p.off_p + ((first + 1) * WAVE + lane) * 16, pack8_16(pv, 1, 1.f));
+                    }
                 }
             };
             // first the two diagonal tiles of A, which the inverse starts from, and two of the three tiles of P
@@ -402,13 +426,19 @@ __device__ __forceinline__ void chunk_prepare32_body(const ChunkParams& p, uint8
         // ---- T diag(beta) as A operands of V~ = T' X: tiles (0, 0), (1, 0), (1, 1), two 16-token slabs each ----
         // The reduction index (token j of X) runs in the order in which an accumulator tile of the scan hands its
         // rows over as a B operand: lane half h supplies tokens 16 s + 4 h + 0..3 and 16 s + 8 + 4 h + 0..3.
+        // (16x16x32 layout: fragments (tt, s) = (0,0) (1,0) (2,0) (2,1) (3,0) (3,1), 16 rows 16 tt .., lane (i, g) holds
+        // columns 32 s + 4 g + 0..3 and 32 s + 16 + 4 g + 0..3: the order in which two 16 x 16 accumulator tiles hand
+        // their rows over)
         for (int f = wave; f < 6; f += 4) {
             const int ti = f < 2 ? 0 : 1, tj = f < 4 ? 0 : 1, sl = f % 2;
-            const int i = 32 * ti + l32, j0 = 32 * tj + 16 * sl + 4 * lh;
+            const int tt16 = f < 2 ? f : 2 + (f - 2) / 2, s16 = f < 2 ? 0 : f % 2;
+            const int i = p.rec16 ? 16 * tt16 + l16 : 32 * ti + l32;
+            const int j0 = p.rec16 ? 32 * s16 + 4 * lq : 32 * tj + 16 * sl + 4 * lh;
+            const int j1 = p.rec16 ? j0 + 16 : j0 + 8;
             const f32x4 t0 = *reinterpret_cast<const f32x4*>(&sT[i * LDA + j0]);
-            const f32x4 t1 = *reinterpret_cast<const f32x4*>(&sT[i * LDA + j0 + 8]);
+            const f32x4 t1 = *reinterpret_cast<const f32x4*>(&sT[i * LDA + j1]);
             const f32x4 c0 = *reinterpret_cast<const f32x4*>(&s_beta[j0]);
-            const f32x4 c1 = *reinterpret_cast<const f32x4*>(&s_beta[j0 + 8]);
+            const f32x4 c1 = *reinterpret_cast<const f32x4*>(&s_beta[j1]);
             bf16x8 r;
 #pragma unroll
             for (int e = 0; e < 4; e++) {  // sT holds the whole of T here: unit diagonal, zeros above it
