@@ -42,8 +42,6 @@
 
 #include <type_traits>
 
-#include <stdio.h>
-
 #include "gdn_chunk32_common.h"
 #include "gdn_chunk_prepare32.h"
 #include "gdn_launch.h"
@@ -104,12 +102,6 @@ __global__ __launch_bounds__(PREP_THREADS, 3) void chunk_prepare32_kernel(const 
 // asking).
 // ------------------------------------------------------------------------------------------
 constexpr int SCAN_LOADERS = 4;
-#ifdef GDN_EXP_TIMING
-__device__ unsigned long long g_dbg[64];
-#define STAMP(k) { const unsigned long long t1 = clock64(); tacc[k] += t1 - t0; t0 = t1; }
-#else
-#define STAMP(k)
-#endif
 
 // Waves of a scan workgroup.  The hardware deals the waves of a workgroup round over the four SIMDs (wave w runs on
 // SIMD w % 4), and a wave that shares a SIMD with a compute wave takes instruction-issue slots from it (measured:
@@ -118,9 +110,8 @@ __device__ unsigned long long g_dbg[64];
 //   NW = 1:  0 compute | 1 2 3 loaders | 4 output store | 5 loader
 //   NW = 2:  0 1 compute | 2 3 loaders | 4 output store | 5 exits at once | 6 7 loaders
 //   NW = 4:  0..3 compute | 4..7 loaders (each compute wave shares with one loader; no output wave)
-//   NW = 1, SPLIT:  0 state | 1 output | 2 3 loaders | 4 output store | 5 exits at once | 6 7 loaders
-//   NW = 1, HALF:   0 1 compute (16 columns each) | the rest as above
-__host__ __device__ constexpr int scan_waves(int nw, bool split = false) { return nw == 1 && !split ? 6 : 8; }
+//   NW = 1, HALF:  0 1 compute (16 columns each) | the rest as for NW = 2
+__host__ __device__ constexpr int scan_waves(int nw, bool half = false) { return nw == 1 && !half ? 6 : 8; }
 
 // Order of the MFMAs of one chunk in the scan's compute wave, and where its side work goes.
 //
@@ -134,20 +125,15 @@ __host__ __device__ constexpr int scan_waves(int nw, bool split = false) { retur
 // and the op that needs its result.  A lone wave issues an instruction every four to five cycles and an MFMA
 // occupies the matrix pipe for 33, so more than about six instructions between two MFMAs idle the pipe: the pieces
 // are spread one per op, earliest deadline first, as far as their windows allow.
-//
-// SPLIT: the schedule of the state wave when a second wave of the workgroup computes the output (see the kernel):
-// no O^T groups, no output pieces; V~ goes to accumulators of its own (X of token tile 1 then has until the fifth
-// op of T' X), and the bf16 copy of the last state tile, which nothing in this chunk waits for any more, runs in a
-// tail slot behind the last MFMA.
-template <int K, bool SPLIT = false>
+template <int K>
 struct ScanScheduleRules {
     static constexpr int KD = K / 32, KS16 = K / 16;
-    static constexpr int NSF = 2 * KS16, NQF = SPLIT ? 0 : 2 * KS16, NTF = 6, NKF = 4 * KD, NPF = SPLIT ? 0 : 6;
+    static constexpr int NSF = 2 * KS16, NQF = 2 * KS16, NTF = 6, NKF = 4 * KD, NPF = 6;
     static constexpr int NOPS = NSF + NQF + NTF + NKF + NPF;
-    static constexpr int LA = SPLIT && K == 64 ? 3 : 6;
+    static constexpr int LA = 6;
     static constexpr int OP_Q = NSF, OP_T = OP_Q + NQF, OP_K = OP_T + NTF, OP_P = OP_K + NKF, OP_BAR = NOPS - LA;
     static constexpr int AHEAD = 2;  // scales and rows of v are read this many ops before their piece
-    static_assert(SPLIT || OP_BAR >= OP_P, "the scales and v of this chunk are used before the barrier");
+    static_assert(OP_BAR >= OP_P, "the scales and v of this chunk are used before the barrier");
 
     // op j of the fourth group -> key tile, token slab
     static constexpr int k_tile(int j) { return (j % (2 * KD)) / 2; }
@@ -158,17 +144,17 @@ struct ScanScheduleRules {
 
     // pieces: X (4 registers) | output hand-over (half a tile) | q row scale (4 registers) | decay (4 registers) |
     // scaled V~ (half a fragment) | plain V~ (a fragment) | new state (a fragment) | X as operand (a fragment)
-    static constexpr int N_XC = 8, N_OUT = SPLIT ? 0 : 4, N_AS = SPLIT ? 0 : 8, N_DEC = 4 * KD, N_VS = 8, N_VB = 4, N_SB = 2 * KD, N_XB = 4;
+    static constexpr int N_XC = 8, N_OUT = 4, N_AS = 8, N_DEC = 4 * KD, N_VS = 8, N_VB = 4, N_SB = 2 * KD, N_XB = 4;
     static constexpr int P_XC = 0, P_OUT = P_XC + N_XC, P_AS = P_OUT + N_OUT, P_DEC = P_AS + N_AS, P_VS = P_DEC + N_DEC,
                          P_VB = P_VS + N_VS, P_SB = P_VB + N_VB, P_XB = P_SB + N_SB, NPIECES = P_XB + N_XB;
 
     struct Window {
-        int first, end;  // the piece runs before the MFMA of an op in [first, end); first >= NOPS: in the tail slot
+        int first, end;  // the piece runs before the MFMA of an op in [first, end)
     };
     static constexpr Window window(int pc) {
         if (pc < P_OUT) {  // K S0 of tile tt is complete after op KS16 (tt + 1) - 1; T' X overwrites tile 1 at its third op
             const int tt = (pc - P_XC) / 4;
-            return {KS16 * (tt + 1) + 1, SPLIT ? OP_T + 4 * tt : OP_T + 2 * tt};
+            return {KS16 * (tt + 1) + 1, OP_T + 2 * tt};
         }
         if (pc < P_AS) return {1, OP_Q + KS16 * ((pc - P_OUT) / 2)};  // the previous chunk's tile, before q overwrites it
         if (pc < P_DEC) {
@@ -181,10 +167,10 @@ struct ScanScheduleRules {
             const int x = (pc - P_VS) / 2;
             return {OP_T + (x / 2 == 0 ? 2 : 6) + 1, x < 2 ? OP_K + x : OP_K + NKF / 2 + (x - 2)};
         }
-        if (pc < P_SB) return {OP_T + ((pc - P_VB) / 2 == 0 ? 2 : 6) + 1, SPLIT ? OP_BAR : OP_P};  // (SPLIT: the output wave waits for it)
+        if (pc < P_SB) return {OP_T + ((pc - P_VB) / 2 == 0 ? 2 : 6) + 1, OP_P};
         if (pc < P_XB) return {OP_K + NKF / 2 + 2 * ((pc - P_SB) / 2) + 3, NOPS};
         const int tt = (pc - P_XB) / 2;  // after the two X pieces of its half tile (checked in make)
-        return SPLIT ? Window{KS16 * (tt + 1) + 1, OP_T + 4 * tt} : Window{KS16 * (tt + 1) + 2, OP_T + 2 * tt};
+        return {KS16 * (tt + 1) + 2, OP_T + 2 * tt};
     }
 
     struct Table {
@@ -208,8 +194,6 @@ struct ScanScheduleRules {
                 t.op[best] = op, done[best] = true, left--;
             }
         }
-        for (int pc = 0; pc < NPIECES; pc++)  // the tail slot
-            if (!done[pc] && window(pc).first >= NOPS) t.op[pc] = NOPS, done[pc] = true, left--;
         if (left != 0) t.ok = false;
         // a half tile of X is packed after its two pieces (within an op the pieces run in index order: X before the pack)
         for (int i = 0; i < N_XB; i++)
@@ -221,18 +205,13 @@ struct ScanScheduleRules {
             if (t.op[P_XC + i] - AHEAD <= t.op[P_XC + i - 4]) t.ok = false;
         for (int i = 0; i < N_VS; i++)
             if (t.op[P_VS + i] - AHEAD < 0) t.ok = false;
-        // the scales of this chunk are read before the barrier that releases its half of the stage
-        for (int i = 0; i < N_VS; i++)
-            if (t.op[P_VS + i] >= OP_BAR) t.ok = false;
-        for (int i = 0; i < N_XC; i++)
-            if (t.op[P_XC + i] >= OP_BAR) t.ok = false;
         return t;
     }
 };
 
-template <int K, bool SPLIT = false>
-struct ScanSchedule : ScanScheduleRules<K, SPLIT> {
-    static constexpr typename ScanScheduleRules<K, SPLIT>::Table TABLE = ScanScheduleRules<K, SPLIT>::make();
+template <int K>
+struct ScanSchedule : ScanScheduleRules<K> {
+    static constexpr typename ScanScheduleRules<K>::Table TABLE = ScanScheduleRules<K>::make();
     static_assert(TABLE.ok, "no placement of the side work satisfies the windows");
     static constexpr int op_of(int pc) { return TABLE.op[pc]; }
 };
@@ -253,10 +232,12 @@ struct Scan16Rules {
     static constexpr int OP_Q = NSF, OP_T = OP_Q + NQF, OP_K = OP_T + NTF, OP_P = OP_K + NKF, OP_BAR = NOPS - LA;
     static constexpr int AHEAD = 4, DIST = 3;
 
-    // op j of the first two groups -> token tile, key slab
-    static constexpr int s_tile(int j) { return j % 4; }
-    static constexpr int s_slab(int j) { return j / 4; }
-    static constexpr int s_last(int tt) { return 4 * (KS - 1) + tt; }  // last op of tile tt
+    // op j of the first two groups -> token tile, key slab: tiles 0 and 1 alternate through all slabs, then tiles 2 and 3
+    // (X of the first two tiles can then be formed while the products of the other two run)
+    static constexpr int s_tile(int j) { return 2 * (j / (2 * KS)) + j % 2; }
+    static constexpr int s_slab(int j) { return (j % (2 * KS)) / 2; }
+    static constexpr int s_last(int tt) { return (tt / 2) * 2 * KS + 2 * (KS - 1) + tt % 2; }  // last op of tile tt
+    static constexpr int s_begin(int tt) { return (tt / 2) * 2 * KS + tt % 2; }                // and its first
     // op j of the third and fifth group -> token tile (16 tokens), slab of 32 reduction tokens: the non-zero blocks of a
     // lower triangular 64 x 64 matrix, (0,0) (1,0) (2,0) (3,0) (2,1) (3,1); fragment (tile, slab) is number
     // t_frag(j) of the record, where they are stored tile by tile
@@ -277,6 +258,7 @@ struct Scan16Rules {
     struct Window {
         int first, end;
     };
+    static constexpr int before_barrier(int op) { return op < OP_BAR ? op : OP_BAR; }
     static constexpr Window window(int pc) {
         if (pc < P_XB) {
             const int tt = pc - P_XC;
@@ -286,16 +268,15 @@ struct Scan16Rules {
             const int s = pc - P_XB;
             return {s_last(2 * s + 1) + DIST, OP_T + s_first(s)};
         }
-        if (pc < P_AS) return {DIST - 1, OP_Q + (pc - P_OUT)};  // (the last MFMA of the previous chunk was its last op)
+        if (pc < P_AS) return {DIST - 1, OP_Q + s_begin(pc - P_OUT)};  // (the last MFMA of the previous chunk was its last op)
         if (pc < P_DEC) {
             const int it = pc - P_AS;
-            const int end = OP_P + t_first(it);
-            return {OP_Q + s_last(it) + DIST, end < OP_BAR ? end : OP_BAR};
+            return {OP_Q + s_last(it) + DIST, before_barrier(OP_P + t_first(it))};
         }
-        if (pc < P_VS) return {OP_Q, OP_K + (pc - P_DEC)};  // (not among the K S0 products: the X pieces and the output are there)
+        if (pc < P_VS) return {OP_Q, before_barrier(OP_K + (pc - P_DEC))};
         if (pc < P_VB) {
             const int tt = pc - P_VS;
-            return {OP_T + t_last(tt) + DIST, OP_K + KT * (tt / 2)};
+            return {OP_T + t_last(tt) + DIST, before_barrier(OP_K + KT * (tt / 2))};
         }
         if (pc < P_SB) {
             const int s = pc - P_VB;
@@ -353,24 +334,13 @@ struct Scan16Schedule : Scan16Rules<K> {
 // NT: the loaders use non-temporal loads.  Right when no other workgroup reads the same lines (one workgroup per
 // chain; measured 7 % faster at 1024 chains), wrong when column groups share them through the L2 (8 % slower).
 //
-// SPLIT (one slice per workgroup): the slice has two waves on two SIMDs.  A lone wave issues in order, and what
-// bounds the one-wave scan is its instruction count (per chunk and K = 128: 60 MFMAs at 8 issue cycles, 280 vector
-// instructions at 4.3, 97 LDS instructions at 7), not the matrix pipe.  So the products that nothing in the
-// recurrence waits for, O^T = S0^T q^T and O^T += V~^T P^T, their operand reads, the row scale of q and the bf16
-// output move to an output wave.  The state wave hands it the operands it has made anyway - the bf16 copy of the
-// state a chunk starts from and V~ - through a double-buffered LDS area, publishing each with an epoch word; nothing
-// flows back, so the state wave never waits for its partner (the workgroup barrier of a chunk, which the output
-// wave reaches first, also tells the state wave that the area's other half has been read).  Same arithmetic in the
-// same order as the one-wave scan: the results are bit-identical.
-//
 // HALF (one slice per workgroup): the slice has two waves, each with 16 of its columns, on v_mfma_f32_16x16x32_bf16.
 // A wave has the same number of MFMAs and operand reads as a whole-slice wave but half the accumulators, so half the
 // vector work on them (decay, X, the bf16 copies), and the two halves need nothing from each other.  The records must
 // hold the fragments of T diag(beta) and P in the layout of that instruction (ChunkParams::rec16).
-template <int K, int NW, bool NT = false, bool SAVE = false, bool SPLIT = false, bool HALF = false>
-__global__ __launch_bounds__(scan_waves(NW, SPLIT || HALF) * WAVE) void chunk_scan32_kernel(const ChunkParams p) {
-    static_assert(!SPLIT || (NW == 1 && !SAVE), "the split scan has one slice per workgroup and saves nothing");
-    static_assert(!HALF || (NW == 1 && !SAVE && !SPLIT), "the half-slice scan has one slice per workgroup and saves nothing");
+template <int K, int NW, bool NT = false, bool SAVE = false, bool HALF = false>
+__global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kernel(const ChunkParams p) {
+    static_assert(!HALF || (NW == 1 && !SAVE), "the half-slice scan has one slice per workgroup and saves nothing");
     constexpr int NL = SCAN_LOADERS;
     // a separate wave writes the output (see below); with four compute waves the LDS has no room for its staging
     constexpr bool OS = NW < 4;
@@ -401,14 +371,8 @@ __global__ __launch_bounds__(scan_waves(NW, SPLIT || HALF) * WAVE) void chunk_sc
     static_assert(SHARED_FRAGS % NL == 0 && V_UNITS % NL == 0 && (2 * Q_UNITS) % NL == 0, "the pieces must divide over the loader waves");
     static_assert(2 * STAGE_BYTES + (OS ? NW * 2 * C * 64 : 16) <= 160 * 1024, "stage exceeds LDS");
 
-    // SPLIT: what the state wave hands to the output wave, [chunk parity][state KS16 | V~ 4] fragments, and two epochs
-    constexpr int XCH_FRAGS = KS16 + 4;
-    static_assert(2 * STAGE_BYTES + (OS ? NW * 2 * C * 64 : 16) + (SPLIT ? 2 * XCH_FRAGS * FRAG_BYTES + 16 : 0) <= 160 * 1024, "stage exceeds LDS");
-
     __shared__ __attribute__((aligned(16))) uint8_t stage[2][STAGE_BYTES];
     __shared__ __attribute__((aligned(16))) uint8_t ostage[OS ? NW * 2 * C * 64 : 16];
-    __shared__ __attribute__((aligned(16))) uint8_t xch[SPLIT ? 2 : 1][SPLIT ? XCH_FRAGS * FRAG_BYTES : 16];
-    __shared__ int xch_epoch[2];  // chunks whose state copy / whose V~ the state wave has published
 
     const int lane = threadIdx.x % WAVE;
     const int wave = threadIdx.x / WAVE;
@@ -447,10 +411,9 @@ __global__ __launch_bounds__(scan_waves(NW, SPLIT || HALF) * WAVE) void chunk_sc
     };
     // role of this wave (see scan_waves)
     const bool is_store = OS && wave == 4;
-    constexpr bool EIGHT = NW == 2 || SPLIT || HALF;  // the wave layout of two compute waves
+    constexpr bool EIGHT = NW == 2 || HALF;  // the wave layout of two compute waves
     const bool is_loader = NW == 4 ? wave >= 4 : EIGHT ? (wave == 2 || wave == 3 || wave >= 6) : (wave >= 1 && wave != 4);
     if (EIGHT && wave == 5) return;
-    if (SPLIT && threadIdx.x < 2) xch_epoch[threadIdx.x] = 0;  // (visible after the barrier below that every wave passes)
     if (is_store) {
         // ------------------------------ output store ------------------------------
         // The compute waves leave the bf16 output tile of chunk c in LDS while they work on chunk c + 1; this
@@ -578,9 +541,6 @@ __global__ __launch_bounds__(scan_waves(NW, SPLIT || HALF) * WAVE) void chunk_sc
         // c - 1) and refill the freed registers with chunk c + 3.
         int c = 0;
         for (; c + 4 < nchunks; c += 2) {  // steady state: straight-line code, both reloads exist
-#ifdef GDN_EXP_NO_LOAD
-            if (c > 2) { __syncthreads(); __syncthreads(); continue; }
-#endif
             store_and_reload(buf1, sc1, c + 1, c + 3, yes);
             __syncthreads();
             store_and_reload(buf0, sc0, c + 2, c + 4, yes);
@@ -601,73 +561,6 @@ __global__ __launch_bounds__(scan_waves(NW, SPLIT || HALF) * WAVE) void chunk_sc
         return;
     }
 
-    [[maybe_unused]] lds_flag_t* const ep_state = (lds_flag_t*)&xch_epoch[0];
-    [[maybe_unused]] lds_flag_t* const ep_v = (lds_flag_t*)&xch_epoch[1];
-    if constexpr (SPLIT) {
-        if (wave == 1) {
-            // ------------------------------ output (SPLIT) ------------------------------
-            // O^T tile tt, register r: token 32 tt + l32, column 16 (r/8) + 8 h + r%8 of the slice (slice_col order)
-            constexpr int NQF = 2 * KS16, LAQ = 4;
-            auto q_frag = [&](const uint8_t* st, int j) {  // rows of q, token tile j / KS16, key slab j % KS16: B operand of S0^T q^T
-                return *reinterpret_cast<const bf16x8*>(st + Q_OFF + (32 * (j / KS16) + l32) * QLD + (16 * (j % KS16) + 8 * lh) * 2);
-            };
-            f32x16 acco[2];
-            __syncthreads();  // stage[0] holds chunk 0
-            for (int c = 0; c < nchunks; c++) {
-#ifdef GDN_EXP_NO_O
-                if (c > 0) { __syncthreads(); continue; }
-#endif
-                const uint8_t* st = stage[c & 1];
-                const bf16x8* xc = reinterpret_cast<const bf16x8*>(xch[c & 1]) + lane;
-                bf16x8 qf[NQF], so[KS16], pf[6], vo[4];
-#pragma unroll
-                for (int j = 0; j < LAQ; j++) qf[j] = q_frag(st, j);
-                const float qs0 = reinterpret_cast<const float*>(st + QS_OFF)[l32], qs1 = reinterpret_cast<const float*>(st + QS_OFF)[32 + l32];
-                pair_wait(ep_state, c + 1);  // the bf16 copy of the state this chunk starts from
-#pragma unroll
-                for (int i = 0; i < KS16; i++) so[i] = xc[i * WAVE];
-                __builtin_amdgcn_sched_barrier(0);
-                static_for<0, NQF>([&](auto jc) {
-                    constexpr int j = decltype(jc)::value, s = j % KS16, tt = j / KS16;
-                    if constexpr (j + LAQ < NQF) qf[j + LAQ] = q_frag(st, j + LAQ);
-                    else pf[j + LAQ - NQF] = reinterpret_cast<const bf16x8*>(st)[(6 + j + LAQ - NQF) * WAVE + lane];
-                    if constexpr (s == 0) {
-                        f32x16 zero;
-#pragma unroll
-                        for (int r = 0; r < 16; r++) zero[r] = 0.f;
-                        acco[tt] = mfma32_bf16(so[s], qf[j], zero);
-                    } else {
-                        acco[tt] = mfma32_bf16(so[s], qf[j], acco[tt]);
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
-                });
-                static_assert(LAQ <= 6, "the six fragments of P are read behind the last rows of q");
-#pragma unroll
-                for (int f = LAQ; f < 6; f++) pf[f] = reinterpret_cast<const bf16x8*>(st)[(6 + f) * WAVE + lane];
-                __syncthreads();  // this wave has read what it needs of chunk c's half of the stage
-#pragma unroll
-                for (int r = 0; r < 16; r++) acco[0][r] *= qs0, acco[1][r] *= qs1;
-                pair_wait(ep_v, c + 1);  // V~ of this chunk
-#pragma unroll
-                for (int i = 0; i < 4; i++) vo[i] = xc[(KS16 + i) * WAVE];
-                __builtin_amdgcn_sched_barrier(0);
-                acco[0] = mfma32_bf16(vo[0], pf[0], acco[0]);  // O^T += V~^T P^T; P[i < 32][j >= 32] = 0 is skipped
-                acco[1] = mfma32_bf16(vo[0], pf[2], acco[1]);
-                acco[0] = mfma32_bf16(vo[1], pf[1], acco[0]);
-                acco[1] = mfma32_bf16(vo[1], pf[3], acco[1]);
-                acco[1] = mfma32_bf16(vo[2], pf[4], acco[1]);
-                acco[1] = mfma32_bf16(vo[3], pf[5], acco[1]);
-#pragma unroll
-                for (int tt = 0; tt < 2; tt++)
-#pragma unroll
-                    for (int half = 0; half < 2; half++)
-                        *reinterpret_cast<bf16x8*>(ostage_at(0, c & 1, 32 * tt + l32, 2 * half + lh)) = pack8_16(acco[tt], half, 1.f);
-            }
-            __syncthreads();  // the store wave writes the last output tile
-            return;
-        }
-    }
-
     if constexpr (HALF) {
         // ------------------------------ compute (HALF) ------------------------------
         // Lane (j, g) = (lane % 16, lane / 16).  Operands of the 16x16x32 MFMA: A[j][8 g + 0..7], B[8 g + 0..7][j]; its
@@ -685,6 +578,12 @@ __global__ __launch_bounds__(scan_waves(NW, SPLIT || HALF) * WAVE) void chunk_sc
         const int j16 = lane % 16, g = lane / 16;
         const int half = wave;  // 0 or 1
         const int c0 = 32 * vgroup + 16 * half;
+        auto out_tile = [&](const f32x4& acc, int parity, int it) {  // 4 columns of token 16 it + j to the output staging
+            bf16x4 o4;
+#pragma unroll
+            for (int e = 0; e < 4; e++) o4[e] = (bf16_t)acc[e];
+            *reinterpret_cast<bf16x4*>(ostage_at(0, parity, 16 * it + j16, 2 * half + g / 2) + 8 * (g % 2)) = o4;
+        };
         f32x4 S[KT];
         auto st_key = [&](int t, int r) { return 32 * (t / 2) + 8 * g + 4 * (t % 2) + r; };
         const int64_t st_off = ((int64_t)n * p.H + h) * K * p.V + c0 + j16;
@@ -742,9 +641,6 @@ __global__ __launch_bounds__(scan_waves(NW, SPLIT || HALF) * WAVE) void chunk_sc
 #pragma unroll
         for (int sl = 0; sl < KS; sl++) sb[sl] = pack4x2(S[2 * sl], S[2 * sl + 1]);
 
-#ifdef GDN_EXP_TIMING
-        unsigned long long tacc[8] = {0, 0, 0, 0, 0, 0, 0, 0}, t0 = clock64();
-#endif
         for (int c = 0; c < nchunks; c++) {
             const uint8_t* st = stage[c & 1];
             const uint8_t* stn = stage[(c + 1) & 1];
@@ -764,12 +660,7 @@ __global__ __launch_bounds__(scan_waves(NW, SPLIT || HALF) * WAVE) void chunk_sc
                     xb[sl] = pack4x2(accv[2 * sl], accv[2 * sl + 1]);
                 } else if constexpr (pc < SCH::P_AS) {  // output tile `it` of the previous chunk: 4 columns of token 16 it + j
                     constexpr int it = pc - SCH::P_OUT;
-                    if (c > 0) {
-                        bf16x4 o4;
-#pragma unroll
-                        for (int e = 0; e < 4; e++) o4[e] = (bf16_t)acco[it][e];
-                        *reinterpret_cast<bf16x4*>(ostage_at(0, (c - 1) & 1, 16 * it + j16, 2 * half + g / 2) + 8 * (g % 2)) = o4;
-                    }
+                    if (c > 0) out_tile(acco[it], (c - 1) & 1, it);
                 } else if constexpr (pc < SCH::P_DEC) {
                     constexpr int it = pc - SCH::P_AS;
 #pragma unroll
@@ -818,15 +709,6 @@ __global__ __launch_bounds__(scan_waves(NW, SPLIT || HALF) * WAVE) void chunk_sc
                     if constexpr (SCH::op_of(decltype(pcc)::value) == op) run_piece(pcc);
                 });
 
-#ifdef GDN_EXP_TIMING
-                if constexpr (op == 0) STAMP(0)
-                if constexpr (op == OP_Q) STAMP(1)
-                if constexpr (op == OP_T) STAMP(2)
-                if constexpr (op == OP_K) STAMP(3)
-                if constexpr (op == OP_K + KT) STAMP(4)
-                if constexpr (op == OP_P) STAMP(5)
-                if constexpr (op == OP_BAR + 1) STAMP(6)
-#endif
                 const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
                 if constexpr (op < OP_Q) {  // K S0
                     constexpr int sl = SCH::s_slab(op), tt = SCH::s_tile(op);
@@ -849,17 +731,9 @@ __global__ __launch_bounds__(scan_waves(NW, SPLIT || HALF) * WAVE) void chunk_sc
         }
         if (nchunks > 0) {
 #pragma unroll
-            for (int it = 0; it < 4; it++) {
-                bf16x4 o4;
-#pragma unroll
-                for (int e = 0; e < 4; e++) o4[e] = (bf16_t)acco[it][e];
-                *reinterpret_cast<bf16x4*>(ostage_at(0, (nchunks - 1) & 1, 16 * it + j16, 2 * half + g / 2) + 8 * (g % 2)) = o4;
-            }
+            for (int it = 0; it < 4; it++) out_tile(acco[it], (nchunks - 1) & 1, it);
         }
         __syncthreads();  // the store wave writes the last output tile
-#ifdef GDN_EXP_TIMING
-        if (lane == 0 && blockIdx.x == 40 && wave == 0) for (int i = 0; i < 8; i++) g_dbg[i] = tacc[i] / (nchunks > 0 ? nchunks : 1);
-#endif
         if (p.ht != nullptr) {
 #pragma unroll
             for (int t = 0; t < KT; t++)
@@ -894,7 +768,7 @@ __global__ __launch_bounds__(scan_waves(NW, SPLIT || HALF) * WAVE) void chunk_sc
 
     // MFMA schedule of one chunk: K S0 | q | T' X | k^T | P; the side work sits between the MFMAs at the ops
     // ScanSchedule<K> assigns.
-    typedef ScanSchedule<K, SPLIT> SCH;
+    typedef ScanSchedule<K> SCH;
     constexpr int NOPS = SCH::NOPS, OP_Q = SCH::OP_Q, OP_T = SCH::OP_T, OP_K = SCH::OP_K, OP_P = SCH::OP_P, OP_BAR = SCH::OP_BAR;
     constexpr int LA = SCH::LA;  // LDS reads are issued this many MFMAs ahead of their use
     const int l16 = lane % 16, g16 = l32 / 16;
@@ -925,8 +799,6 @@ __global__ __launch_bounds__(scan_waves(NW, SPLIT || HALF) * WAVE) void chunk_sc
     auto lds_qs = [&](const uint8_t* st, int tt) -> float { return reinterpret_cast<const float*>(st + QS_OFF)[32 * tt + l32]; };
 
     f32x16 accv[2], acco[2];
-    [[maybe_unused]] f32x16 vts[2];             // SPLIT: V~ has accumulators of its own
-    f32x16(&vt)[2] = SPLIT ? vts : accv;
     bf16x8 sb[KS16], xb[4], vb[4], vbs[4], fnext[LA];  // xb: X, vb: V~, vbs: V~ with its rows scaled for the state update
     f32x4 ksr[4], csr[4];                              // row scales on their way to the pieces that use them
     bf16x4 xvr[4];                                     // and rows of v
@@ -936,26 +808,12 @@ __global__ __launch_bounds__(scan_waves(NW, SPLIT || HALF) * WAVE) void chunk_sc
 
     // what the tail of a chunk does for the next one, for chunk 0
     egc = lds_eg(stage[0]);
-    if constexpr (!SPLIT) qsc[0] = lds_qs(stage[0], 0), qsc[1] = lds_qs(stage[0], 1);
+    qsc[0] = lds_qs(stage[0], 0), qsc[1] = lds_qs(stage[0], 1);
     static_for<0, LA>([&](auto i) { fnext[decltype(i)::value] = lds_frag(stage[0], i); });
 #pragma unroll
     for (int s = 0; s < KS16; s++) sb[s] = pack8_16(S[s / 2], s % 2, 1.f);
-    if constexpr (SPLIT) {  // the output wave's copy of the state chunk 0 starts from
-#pragma unroll
-        for (int s = 0; s < KS16; s++) reinterpret_cast<bf16x8*>(xch[0])[s * WAVE + lane] = sb[s];
-        pair_publish(ep_state, 1);
-    }
-    // SPLIT: the op whose pieces complete V~ for the output wave
-    constexpr int LAST_VB_OP = [] {
-        int m = 0;
-        for (int i = 0; i < SCH::N_VB; i++) m = SCH::op_of(SCH::P_VB + i) > m ? SCH::op_of(SCH::P_VB + i) : m;
-        return m;
-    }();
 
     int valid_prev = 0;  // tokens of the previous chunk, whose output is still in acco
-#ifdef GDN_EXP_TIMING
-    unsigned long long tacc[8] = {0, 0, 0, 0, 0, 0, 0, 0}, t0 = clock64();
-#endif
     for (int c = 0; c < nchunks; c++) {
         const uint8_t* st = stage[c & 1];
         const uint8_t* stn = stage[(c + 1) & 1];
@@ -1019,18 +877,16 @@ __global__ __launch_bounds__(scan_waves(NW, SPLIT || HALF) * WAVE) void chunk_sc
                 // V~ as operand of k^T V~: each row (token) scaled by e^{gamma_C - gamma} / |k|; half a fragment
                 constexpr int i = pc - SCH::P_VS, x = i / 2, sub = i % 2, tt = x / 2, half = x % 2;
 #pragma unroll
-                for (int e = 0; e < 4; e++) vbs[x][4 * sub + e] = (bf16_t)(vt[tt][8 * half + 4 * sub + e] * ksr[i % 4][e]);
+                for (int e = 0; e < 4; e++) vbs[x][4 * sub + e] = (bf16_t)(accv[tt][8 * half + 4 * sub + e] * ksr[i % 4][e]);
             } else if constexpr (pc >= SCH::P_VB && pc < SCH::P_VB + SCH::N_VB) {
                 constexpr int i = pc - SCH::P_VB;  // V~ as operand of P V~
-                vb[i] = pack8_16(vt[i / 2], i % 2, 1.f);
-                if constexpr (SPLIT) reinterpret_cast<bf16x8*>(xch[c & 1])[(KS16 + i) * WAVE + lane] = vb[i];
+                vb[i] = pack8_16(accv[i / 2], i % 2, 1.f);
             } else {
                 // the new state tile as operand of the next chunk; pinned here, or the compiler moves all of them
                 // behind the last MFMA of the loop
                 constexpr int i = pc - SCH::P_SB;
                 sb[i] = pack8_16(S[i / 2], i % 2, 1.f);
                 pin_regs(sb[i]);
-                if constexpr (SPLIT) reinterpret_cast<bf16x8*>(xch[(c + 1) & 1])[i * WAVE + lane] = sb[i];  // (freed by the barrier of this chunk)
             }
         };
 
@@ -1041,7 +897,7 @@ __global__ __launch_bounds__(scan_waves(NW, SPLIT || HALF) * WAVE) void chunk_sc
             if constexpr (op == OP_BAR) {
                 __syncthreads();  // this wave is done with chunk c's half; chunk c + 1 is in the other one
                 egc = lds_eg(stn);
-                if constexpr (!SPLIT) qsc[0] = lds_qs(stn, 0), qsc[1] = lds_qs(stn, 1);  // this chunk's scales were applied before the barrier
+                qsc[0] = lds_qs(stn, 0), qsc[1] = lds_qs(stn, 1);  // this chunk's scales were applied before the barrier
             }
             if constexpr (op >= OP_BAR) fnext[op >= OP_BAR ? op - OP_BAR : 0] = lds_frag(stn, std::integral_constant<int, (op >= OP_BAR ? op - OP_BAR : 0)>{});
             // row scales and rows of v, a few ops ahead of the piece that uses them
@@ -1062,17 +918,7 @@ __global__ __launch_bounds__(scan_waves(NW, SPLIT || HALF) * WAVE) void chunk_sc
             static_for<0, SCH::NPIECES>([&](auto pcc) {
                 if constexpr (SCH::op_of(decltype(pcc)::value) == op) run_piece(pcc);
             });
-            if constexpr (SPLIT && op == LAST_VB_OP) pair_publish(ep_v, c + 1);
 
-#ifdef GDN_EXP_TIMING
-            if constexpr (op == 0) STAMP(0)
-            if constexpr (op == KS16) STAMP(1)
-            if constexpr (op == OP_T) STAMP(2)
-            if constexpr (op == OP_T + 4) STAMP(3)
-            if constexpr (op == OP_K) STAMP(4)
-            if constexpr (op == OP_K + SCH::NKF / 2) STAMP(5)
-            if constexpr (op == OP_BAR + 1) STAMP(6)
-#endif
             // ---- the MFMA ----
             if constexpr (op < OP_Q) {  // K S0, fragment (tt, s): rows = tokens
                 constexpr int s = op % KS16, tt = op / KS16;
@@ -1100,9 +946,9 @@ __global__ __launch_bounds__(scan_waves(NW, SPLIT || HALF) * WAVE) void chunk_sc
                     f32x16 zero;
 #pragma unroll
                     for (int r = 0; r < 16; r++) zero[r] = 0.f;
-                    vt[tt] = mfma32_bf16(fr[op], xb[s], zero);
+                    accv[tt] = mfma32_bf16(fr[op], xb[s], zero);
                 } else {
-                    vt[tt] = mfma32_bf16(fr[op], xb[s], vt[tt]);
+                    accv[tt] = mfma32_bf16(fr[op], xb[s], accv[tt]);
                 }
             } else if constexpr (op < OP_P) {  // S = e^{gamma_C} S + k^T (row-scaled V~), fragment (td, s)
                 constexpr int s = SCH::k_slab(op - OP_K), td = SCH::k_tile(op - OP_K);
@@ -1114,12 +960,6 @@ __global__ __launch_bounds__(scan_waves(NW, SPLIT || HALF) * WAVE) void chunk_sc
             }
             __builtin_amdgcn_sched_barrier(0);
         });
-        if constexpr (SPLIT) {  // the tail slot, and the state the next chunk starts from is complete in LDS
-            static_for<0, SCH::NPIECES>([&](auto pcc) {
-                if constexpr (SCH::op_of(decltype(pcc)::value) == NOPS) run_piece(pcc);
-            });
-            pair_publish(ep_state, c + 2);
-        }
         if constexpr (SAVE) {
             // V~ of this chunk: tile tt, register r holds token 32 tt + 8 (r/4) + 4 h + r%4 of this lane's column
             if (p.save_vnew != nullptr && c % p.save_every == 0 && c / p.save_every < p.save_nc) {
@@ -1140,7 +980,7 @@ __global__ __launch_bounds__(scan_waves(NW, SPLIT || HALF) * WAVE) void chunk_sc
 
     // the output of the last chunk
 #pragma unroll
-    for (int tt = 0; tt < 2 && !SPLIT; tt++)
+    for (int tt = 0; tt < 2; tt++)
 #pragma unroll
         for (int half = 0; half < 2; half++) {
             if (OS) {
@@ -1153,9 +993,6 @@ __global__ __launch_bounds__(scan_waves(NW, SPLIT || HALF) * WAVE) void chunk_sc
             }
         }
     if (OS) __syncthreads();
-#ifdef GDN_EXP_TIMING
-    if (lane == 0 && blockIdx.x == 40) for (int i = 0; i < 8; i++) g_dbg[i] = tacc[i] / (nchunks > 0 ? nchunks : 1);
-#endif
 
     if (p.ht != nullptr) {
 #pragma unroll
@@ -1193,11 +1030,7 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     const bool save = p.save_state != nullptr || p.save_vnew != nullptr;
     if (save && nw == 2) nw = 1;  // the saving variant exists for 1 and 4 slices per workgroup
     // a slice with a CU to itself is scanned by two waves of 16 columns each; the records are laid out for them
-#if defined(GDN_NO_SPLIT) || defined(GDN_SPLIT)
-    const bool half = false;
-#else
     const bool half = nw == 1 && !save && !p.records_given;
-#endif
     p.rec16 = half ? 1 : 0;
     if (!p.records_given) {
         hipLaunchKernelGGL((chunk_prepare32_kernel<K>), dim3(grid_prep), dim3(PREP_THREADS), 0, stream, p);
@@ -1214,28 +1047,11 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     if (nw == 4 && p.scan_groups == 1) hipLaunchKernelGGL((chunk_scan32_kernel<K, 4, true>), grid, dim3(scan_waves(4) * WAVE), 0, stream, p);
     else if (nw == 4) hipLaunchKernelGGL((chunk_scan32_kernel<K, 4>), grid, dim3(scan_waves(4) * WAVE), 0, stream, p);
     else if (nw == 2) hipLaunchKernelGGL((chunk_scan32_kernel<K, 2>), grid, dim3(scan_waves(2) * WAVE), 0, stream, p);
-#if defined(GDN_NO_SPLIT)
+    else if (half) hipLaunchKernelGGL((chunk_scan32_kernel<K, 1, false, false, true>), grid, dim3(scan_waves(1, true) * WAVE), 0, stream, p);
     else hipLaunchKernelGGL((chunk_scan32_kernel<K, 1>), grid, dim3(scan_waves(1) * WAVE), 0, stream, p);
-#elif defined(GDN_SPLIT)
-    else hipLaunchKernelGGL((chunk_scan32_kernel<K, 1, false, false, true>), grid, dim3(scan_waves(1, true) * WAVE), 0, stream, p);
-#else
-    else if (half) hipLaunchKernelGGL((chunk_scan32_kernel<K, 1, false, false, false, true>), grid, dim3(scan_waves(1, true) * WAVE), 0, stream, p);
-    else hipLaunchKernelGGL((chunk_scan32_kernel<K, 1>), grid, dim3(scan_waves(1) * WAVE), 0, stream, p);
-#endif
     return (int)hipGetLastError();
 }
 
-#ifdef GDN_EXP_TIMING
-extern "C" void gdn_dbg_dump() {
-    unsigned long long h[8];
-    (void)hipDeviceSynchronize();
-    (void)hipMemcpyFromSymbol(h, HIP_SYMBOL(g_dbg), sizeof(h));
-    printf("cycles per chunk up to op 0 | KS16 | OP_T | OP_T+4 | OP_K | OP_K+NKF/2 | OP_BAR+1 :");
-    unsigned long long sum = 0;
-    for (int i = 0; i < 7; i++) printf(" %llu", h[i]), sum += h[i];
-    printf("  total %llu\n", sum);
-}
-#endif
 int launch_chunk32(ChunkParams& p, int K, hipStream_t stream, hipEvent_t* events, int num_cus) {
     if (K == 64) return launch32<64>(p, stream, events, num_cus);
     if (K == 128) return launch32<128>(p, stream, events, num_cus);
