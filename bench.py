@@ -1,6 +1,7 @@
 """Benchmark of the gated delta-rule path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 1|2|4] [--no-cpu-baseline] [--no-decode]
+                    [--no-other-configs]
 
 A "step" is one chunked forward (``chunk_gated_delta_rule``) over one batch of synthetic input of
 the benchmark configuration (default: configuration 1, B=4, T=4096, H=16, K=V=128, bf16, chunk 64),
@@ -17,6 +18,8 @@ inputs already resident in HBM.  Prints ONE JSON line:
   epilogue     rmsnorm(o * silu(gate)) behind the operator, same batch, against the HBM peak
   cpu_baseline the naive token-by-token torch restatement of the operator (oracle/), timed on
                this host's cores on a bounded prefix of the same workload
+  forward_other the same forward on configurations 2 (packed sequences) and 4 (long context, V=256), and with
+               prepare and scan in one launch (an opt-in mode) on the headline configuration and on 4
 """
 
 from __future__ import annotations
@@ -35,23 +38,45 @@ if ROOT not in sys.path:
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 
-# HBM bytes per launch, (workload, kernel) -> bytes.  Not measurable from inside this process: these are
-# rocprofv3 --pmc readings of FETCH_SIZE and WRITE_SIZE (KiB per dispatch) for this very command, each scaled
-# by what the same counter reads for a plain 1 GiB copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the counter
-# summaries are kept under profiles/.  Workloads that were not profiled report null.
-_KIB = 1024
-MEASURED_HBM_TRAFFIC_BYTES = {
-    ("cfg1_chunk_fwd_bf16", "chunk_prepare"): (2.0 * 66468.2 + 52352.0) * _KIB,
-    ("cfg1_chunk_fwd_bf16", "chunk_scan"): (2.0 * 124827.2 + 69632.0) * _KIB,
-    ("cfg3_decode_bf16", "recurrent_kernel"): (2.0 * 265449.7 + 526881.4) * _KIB,
-    ("cfg1_chunk_fwd_bf16", "causal_conv1d_kernel"): (2.0 * 103205.2 + 196752.0) * _KIB,
-    ("cfg1_chunk_fwd_bf16", "gated_rmsnorm_kernel"): (2.0 * 66081.4 + 65536.0) * _KIB,
-}
+# HBM bytes per launch are not measurable from inside this process: they are rocprofv3 --pmc readings of
+# FETCH_SIZE and WRITE_SIZE (KiB per dispatch) for this very command, each scaled by what the same counter reads
+# for a plain 1 GiB copy.  The readings live in profiles/hbm_traffic_counters.json together with a digest of the
+# kernel sources they were taken on; with other sources (a kernel was changed since) every traffic figure is null.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_counters.json")
+_FUSED_MODE = []  # keeps the kernel-flag context of --fused-launch alive
+_traffic_table = None
+
+
+def kernel_sources_digest() -> str:
+    """sha256 over the HIP sources and headers the library is built from, in name order."""
+    import hashlib
+
+    digest = hashlib.sha256()
+    csrc = os.path.join(ROOT, "lm_engine_amd", "csrc")
+    names = sorted(n for n in os.listdir(csrc) if n.endswith((".hip", ".h")))
+    for path in [os.path.join(csrc, n) for n in names] + [os.path.join(ROOT, "include", "gdn_hip.h")]:
+        with open(path, "rb") as f:
+            digest.update(os.path.basename(path).encode() + b"\0" + f.read())
+    return digest.hexdigest()
 
 
 def measured_traffic(workload: str, kernel: str):
-    value = MEASURED_HBM_TRAFFIC_BYTES.get((workload, kernel))
-    return None if value is None else int(value)
+    """HBM bytes one launch of ``kernel`` moves on ``workload`` (counter readings, see above), or None."""
+    global _traffic_table
+    if _traffic_table is None:
+        _traffic_table = {}
+        try:
+            with open(TRAFFIC_FILE) as f:
+                table = json.load(f)
+            if table.get("sources_sha256") == kernel_sources_digest():
+                _traffic_table = table
+        except (OSError, ValueError):
+            pass
+    entry = _traffic_table.get("kernels", {}).get(f"{workload}/{kernel}")
+    if entry is None:
+        return None
+    kib = entry["fetch_size_kib"] * _traffic_table["fetch_size_scale"] + entry["write_size_kib"] * _traffic_table["write_size_scale"]
+    return int(kib * 1024)
 
 
 def parse_args():
@@ -63,18 +88,68 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true", help="skip the decode, convolution, epilogue and backward legs")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target duration of the CPU baseline sample")
+    ap.add_argument("--no-other-configs", action="store_true", help="skip the forward legs of configurations 2 and 4")
+    ap.add_argument("--fused-launch", action="store_true",
+                    help="run the headline step and everything after it with prepare and scan in one launch "
+                         "(Kernel.gated_delta_rule_fused_launch, an opt-in mode of the library)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, the known-size kernel the HBM counters are scaled by")
     return ap.parse_args()
 
 
-def bench_chunk(w, steps, warmup):
+def chunk_forward_leg(w, steps, warmup, fused_launch):
+    """Wall time per forward of workload ``w`` and the HIP-event durations of its kernels, one launch mode."""
+    import contextlib
+
     import torch
 
     import lm_engine_amd
+    from lm_engine_amd.kernels import Kernel, enable_kernels
+    from lm_engine_amd.ops import chunk_forward_kernel_times
+    from lm_engine_amd.workloads import chunk_fwd_flops_per_token_head, make_inputs
+
+    inp = make_inputs(w, device="cuda")
+    mode = enable_kernels([Kernel.gated_delta_rule_fused_launch]) if fused_launch else contextlib.nullcontext()
+    with mode:
+        for _ in range(warmup):
+            lm_engine_amd.chunk_gated_delta_rule(**inp, output_final_state=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            lm_engine_amd.chunk_gated_delta_rule(**inp, output_final_state=True)
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) / steps * 1e3
+        sums: dict[str, float] = {}
+        for _ in range(steps):
+            for name, t in chunk_forward_kernel_times(**inp, output_final_state=True).items():
+                sums[name] = sums.get(name, 0.0) + t
+    n_seq = w.B if inp["cu_seqlens"] is None else inp["cu_seqlens"].numel() - 1
+    tflops = w.B * w.T * w.H * chunk_fwd_flops_per_token_head(w.K, w.V)["dense"] / (ms * 1e-3) / 1e12
+    del inp
+    torch.cuda.empty_cache()
+    return {
+        "workload": w.name, "B": w.B, "T": w.T, "H": w.H, "K": w.K, "V": w.V, "sequences": n_seq,
+        "launch": "prepare and scan in one launch" if fused_launch else "prepare, then scan",
+        "ms_per_step": round(ms, 4),
+        "tokens_per_s": round(w.B * w.T / (ms * 1e-3), 1),
+        "tflops_dense": round(tflops, 1),
+        "mfma_frac_dense": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+        # (in the one-launch mode the whole launch is booked under chunk_scan)
+        "kernel_ms": {name: round(total / steps, 4) for name, total in sums.items()},
+    }  # fmt: skip
+
+
+def bench_chunk(w, steps, warmup, fused_launch=False):
+    import torch
+
+    import lm_engine_amd
+    from lm_engine_amd.kernels import Kernel, enable_kernels
     from lm_engine_amd.ops import chunk_forward_kernel_times
     from lm_engine_amd.workloads import chunk_fwd_bytes_per_token_head, chunk_fwd_flops_per_token_head, make_inputs
 
+    if fused_launch:  # for the rest of the run
+        _FUSED_MODE.append(enable_kernels([Kernel.gated_delta_rule_fused_launch]))
+        _FUSED_MODE[-1].__enter__()
     inp = make_inputs(w, device="cuda")
     call = lambda: lm_engine_amd.chunk_gated_delta_rule(**inp, output_final_state=True)  # noqa: E731
 
@@ -104,10 +179,18 @@ def bench_chunk(w, steps, warmup):
 
     per_kernel = {}
     for name, part in (("chunk_prepare", "prepare"), ("chunk_scan", "scan")):
+        if fused_launch:  # one launch does both parts; it is booked under chunk_scan
+            if name == "chunk_prepare":
+                continue
+            part = "dense"
         tflops = token_heads * flops[part] / (kernel_ms[name] * 1e-3) / 1e12
         per_kernel[name] = {"ms": round(kernel_ms[name], 4), "algorithmic_flop_per_token_head": flops[part],
-                            "tflops": round(tflops, 1), "mfma_frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4)}  # fmt: skip
+                            "tflops": round(tflops, 1), "mfma_frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+                            "traffic": measured_traffic(w.name, "chunk_fused" if fused_launch else name)}  # fmt: skip
     dominant = max(per_kernel, key=lambda name: per_kernel[name]["ms"])
+    # HBM bytes of the whole step (every kernel of it), or null when a kernel has no reading
+    step_traffic = [k["traffic"] for k in per_kernel.values()]
+    step_traffic = None if any(t is None for t in step_traffic) else sum(step_traffic)
     whole_tflops = token_heads * flops["dense"] / (ms_per_step * 1e-3) / 1e12
 
     result = {
@@ -117,7 +200,8 @@ def bench_chunk(w, steps, warmup):
         "ms_per_step": round(ms_per_step, 4),
         "dtype": "bf16",
         "config": {"workload": w.name, "B": w.B, "T": w.T, "H": w.H, "K": w.K, "V": w.V, "chunk": 64,
-                   "sequences": n_seq, "initial_state": inp["initial_state"] is not None},  # fmt: skip
+                   "sequences": n_seq, "initial_state": inp["initial_state"] is not None,
+                   "launch": "prepare and scan in one launch" if fused_launch else "prepare, then scan"},  # fmt: skip
         "roofline": {
             "kernel": dominant,
             "bound": "mfma",
@@ -125,7 +209,9 @@ def bench_chunk(w, steps, warmup):
             "peak": MFMA_BF16_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": per_kernel[dominant]["mfma_frac"],
-            "traffic": measured_traffic(w.name, dominant),
+            "traffic": step_traffic,
+            "traffic_scope": "whole step: " + " + ".join(per_kernel) + " (per kernel under step.kernels)",
+            "algorithmic_bytes": int(algo_bytes),
         },
         "step": {
             "tflops_dense": round(whole_tflops, 1),
@@ -425,13 +511,21 @@ def main():
     torch.cuda.set_device(0)
 
     w = get_workload(args.workload)
-    result, inp = bench_chunk(w, args.steps, args.warmup)
+    result, inp = bench_chunk(w, args.steps, args.warmup, args.fused_launch)
     decode = None if args.no_decode else bench_decode(args.steps, args.warmup)
     conv = None if args.no_decode else bench_conv(w, args.steps, args.warmup)
     epilogue = None if args.no_decode else bench_epilogue(w, args.steps, args.warmup)
     backward = None if args.no_decode else bench_backward(w, inp, args.steps, args.warmup)
     if backward is not None:
         backward["layer_kernels"] = bench_layer_backward_kernels(w, args.steps, args.warmup)
+    other = None
+    if not args.no_other_configs:
+        # the forward on the other chunked configurations, and with prepare and scan in one launch where that qualifies
+        other = [chunk_forward_leg(w, args.steps, args.warmup, fused_launch=True)]
+        for index in (2, 4):
+            if index != args.workload:
+                other.append(chunk_forward_leg(get_workload(index), args.steps, args.warmup, fused_launch=False))
+        other.append(chunk_forward_leg(get_workload(4), args.steps, args.warmup, fused_launch=True))
     baseline = None if args.no_cpu_baseline else cpu_baseline(w, inp, args.cpu_seconds)
     if args.calibrate_copy:
         calibrate_copy()
@@ -457,6 +551,7 @@ def main():
         "conv": conv,
         "epilogue": epilogue,
         "backward": backward,
+        "forward_other": other,
         "device": torch.cuda.get_device_name(0),
     }
     print(json.dumps(line))

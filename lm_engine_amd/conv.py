@@ -38,6 +38,26 @@ def _dtype_code(dtype: torch.dtype, what: str) -> int:
     raise ValueError(f"{what} must be bfloat16 or float32, got {dtype}")
 
 
+def convolution_formula(x, weight, bias, input_state, attention_mask, output_state, activation):
+    """The convolution in torch operations (fp32 arithmetic): what the backward differentiates when the backward
+    kernel does not apply."""
+    # y[s] = act(bias + sum_j w[j] xx[s + j]) over xx = [state or zeros | x * mask], y masked again
+    w = (weight.squeeze(1) if weight.dim() == 3 else weight).float()
+    B, S, C = x.shape
+    ks = w.size(1)
+    use_mask = attention_mask is not None and attention_mask.shape[1] > 1 and attention_mask.shape[0] > 1
+    xm = x.float() * attention_mask[:, :, None].float() if use_mask else x.float()
+    head = torch.zeros(B, C, ks - 1, device=x.device) if input_state is None else input_state.float()
+    xx = torch.cat([head, xm.transpose(1, 2)], dim=-1)
+    y = torch.nn.functional.conv1d(xx, w[:, None, :], None if bias is None else bias.float(), groups=C)
+    if activation is not None:
+        y = torch.nn.functional.silu(y)
+    y = y.transpose(1, 2)
+    if use_mask:
+        y = y * attention_mask[:, :, None].float()
+    return y.to(x.dtype), (xx[..., -(ks - 1):].to(x.dtype) if output_state else None)
+
+
 def depthwise_causal_convolution(
     x: torch.Tensor,
     weight: torch.Tensor,
@@ -47,22 +67,13 @@ def depthwise_causal_convolution(
     output_state: bool = False,
     activation: str | None = "silu",
 ) -> tuple[torch.Tensor, torch.Tensor | None]:
+    if torch.compiler.is_compiling():  # a graph is being captured: the kernel goes in as an opaque operator
+        from . import _opaque
+
+        return _opaque.depthwise_causal_convolution(x, weight, bias, input_state, attention_mask, output_state, activation)
+
     def formula(x, weight, bias, input_state):
-        # y[s] = act(bias + sum_j w[j] xx[s + j]) over xx = [state or zeros | x * mask], y masked again
-        w = (weight.squeeze(1) if weight.dim() == 3 else weight).float()
-        B, S, C = x.shape
-        ks = w.size(1)
-        use_mask = attention_mask is not None and attention_mask.shape[1] > 1 and attention_mask.shape[0] > 1
-        xm = x.float() * attention_mask[:, :, None].float() if use_mask else x.float()
-        head = torch.zeros(B, C, ks - 1, device=x.device) if input_state is None else input_state.float()
-        xx = torch.cat([head, xm.transpose(1, 2)], dim=-1)
-        y = torch.nn.functional.conv1d(xx, w[:, None, :], None if bias is None else bias.float(), groups=C)
-        if activation is not None:
-            y = torch.nn.functional.silu(y)
-        y = y.transpose(1, 2)
-        if use_mask:
-            y = y * attention_mask[:, :, None].float()
-        return y.to(x.dtype), (xx[..., -(ks - 1):].to(x.dtype) if output_state else None)
+        return convolution_formula(x, weight, bias, input_state, attention_mask, output_state, activation)
 
     kernel = lambda x, weight, bias, input_state: _depthwise_causal_convolution(  # noqa: E731
         x, weight, bias, input_state, attention_mask, output_state, activation)  # fmt: skip

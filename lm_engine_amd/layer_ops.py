@@ -49,15 +49,25 @@ def _token_rows(x: torch.Tensor, width: int, what: str) -> tuple[torch.Tensor, i
     return rows, rows.stride(0) if rows.size(0) > 1 else width
 
 
+def gates_formula(a, b, A_log, dt_bias, allow_neg_eigval):
+    """The gates in torch operations: what their backward differentiates."""
+    g = -torch.exp(A_log.float()) * torch.nn.functional.softplus(a.float() + dt_bias.float())
+    beta = torch.sigmoid(b.float()) * (2.0 if allow_neg_eigval else 1.0)
+    return g, beta.to(b.dtype)
+
+
 def delta_rule_gates(
     a: torch.Tensor, b: torch.Tensor, A_log: torch.Tensor, dt_bias: torch.Tensor, allow_neg_eigval: bool = False
 ) -> tuple[torch.Tensor, torch.Tensor]:
     """a, b ``[..., H]`` (activation dtype, may be slices of one projection) -> ``(g fp32, beta)`` of the same shape."""
 
+    if torch.compiler.is_compiling():  # a graph is being captured: the kernel goes in as an opaque operator
+        from . import _opaque
+
+        return _opaque.delta_rule_gates(a, b, A_log, dt_bias, allow_neg_eigval)
+
     def formula(a, b, A_log, dt_bias):
-        g = -torch.exp(A_log.float()) * torch.nn.functional.softplus(a.float() + dt_bias.float())
-        beta = torch.sigmoid(b.float()) * (2.0 if allow_neg_eigval else 1.0)
-        return g, beta.to(b.dtype)
+        return gates_formula(a, b, A_log, dt_bias, allow_neg_eigval)
 
     kernel = lambda a, b, A_log, dt_bias: _delta_rule_gates(a, b, A_log, dt_bias, allow_neg_eigval)  # noqa: E731
     return kernel_with_formula_backward(kernel, formula, a, b, A_log, dt_bias)
@@ -90,6 +100,17 @@ def _delta_rule_gates(a, b, A_log, dt_bias, allow_neg_eigval):
     return g, beta
 
 
+def gated_rmsnorm_formula(o, gate, weight, eps_value):
+    """The gated norm in torch operations: what its backward differentiates off the GPU."""
+    x = o.float()
+    if gate is not None:
+        x = x * torch.nn.functional.silu(gate.float().reshape(o.shape))
+    y = x * torch.rsqrt(x.square().mean(dim=-1, keepdim=True) + eps_value)
+    if weight is not None:
+        y = y * weight.float()
+    return (y.to(o.dtype),)
+
+
 def gated_rmsnorm(
     o: torch.Tensor, gate: torch.Tensor | None, weight: torch.Tensor | None, eps: float | None = None
 ) -> torch.Tensor:
@@ -98,14 +119,13 @@ def gated_rmsnorm(
     ``eps=None`` is torch's default for nn.RMSNorm: the machine epsilon of o's dtype."""
     eps_value = float(torch.finfo(o.dtype).eps if eps is None else eps)
 
+    if torch.compiler.is_compiling():  # a graph is being captured: the kernel goes in as an opaque operator
+        from . import _opaque
+
+        return _opaque.gated_rmsnorm(o, gate, weight, eps)
+
     def formula(o, gate, weight):
-        x = o.float()
-        if gate is not None:
-            x = x * torch.nn.functional.silu(gate.float().reshape(o.shape))
-        y = x * torch.rsqrt(x.square().mean(dim=-1, keepdim=True) + eps_value)
-        if weight is not None:
-            y = y * weight.float()
-        return (y.to(o.dtype),)
+        return gated_rmsnorm_formula(o, gate, weight, eps_value)
 
     kernel = lambda o, gate, weight: (_gated_rmsnorm(o, gate, weight, eps),)  # noqa: E731
     needs_grad = torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (o, gate, weight))

@@ -427,6 +427,11 @@ class _GatedDeltaRule(torch.autograd.Function):
 
 def _dispatch(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm, inplace_state,
               left_padded=False):
+    if torch.compiler.is_compiling():  # a graph is being captured: the kernels go in as opaque operators
+        from . import _opaque
+
+        return _opaque.gated_delta_rule(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens,
+                                        l2norm, inplace_state, left_padded)  # fmt: skip
     tensors = (q, k, v, g, beta, initial_state)
     if torch.is_grad_enabled() and any(x is not None and x.requires_grad for x in tensors):
         return _GatedDeltaRule.apply(mode, scale, output_final_state, l2norm, inplace_state, left_padded, q, k, v, g,

@@ -244,3 +244,37 @@ def test_noalloc_entry_point_rejects_shapes_beyond_its_scratch():
         setattr(args, f"{name}_stride_h", 128)
     assert lib.gdn_workspace_bytes(ctypes.byref(args)) > _lib.GDN_NOALLOC_SCRATCH_BYTES
     assert lib.gdn_chunk_fwd_noalloc(ctypes.byref(args), None) == -5  # GDN_ERR_WORKSPACE, before any launch
+
+
+def test_opaque_operators_are_registered_with_shape_only_implementations():
+    # what torch.compile captures in place of the ctypes launches: one torch.library operator per kernel, each with a
+    # fake implementation (run here on meta tensors: no kernel is launched)
+    import torch
+
+    from lm_engine_amd import _opaque  # noqa: F401
+
+    ops = torch.ops.lm_engine_amd
+    for name in ("gated_delta_rule_forward", "gated_delta_rule_backward", "gated_delta_rule_decode_",
+                 "causal_conv1d_forward", "causal_conv1d_backward", "delta_rule_gates_forward",
+                 "delta_rule_gates_backward", "gated_rmsnorm_forward", "gated_rmsnorm_backward"):  # fmt: skip
+        assert hasattr(ops, name), name
+    meta = lambda *shape, dtype=torch.bfloat16: torch.empty(*shape, dtype=dtype, device="meta")  # noqa: E731
+    B, T, H, K, V = 2, 130, 3, 128, 64
+    q, k, v = meta(B, T, H, K), meta(B, T, H, K), meta(B, T, H, V)
+    g, beta, h0 = meta(B, T, H, dtype=torch.float32), meta(B, T, H), meta(B, H, K, V, dtype=torch.float32)
+    o, ht = ops.gated_delta_rule_forward(q, k, v, g, beta, h0, None, "chunk", None, True, False, False)
+    assert tuple(o.shape) == (B, T, H, V) and o.dtype == torch.bfloat16
+    assert tuple(ht.shape) == (B, H, K, V) and ht.dtype == torch.float32
+    o, ht = ops.gated_delta_rule_forward(q, k, v, None, None, None, None, "chunk", 0.5, False, True, False)
+    assert ht.numel() == 0
+    cu = torch.empty(4, dtype=torch.int32, device="meta")
+    _, ht = ops.gated_delta_rule_forward(q[:1], k[:1], v[:1], None, None, None, cu, "chunk", None, True, False, False)
+    assert tuple(ht.shape) == (3, H, K, V)
+    grads = ops.gated_delta_rule_backward(q, k, v, g, None, h0, None, o, None, None, False, False)
+    assert [tuple(x.shape) for x in grads] == [(B, T, H, K), (B, T, H, K), (B, T, H, V), (B, T, H), (0,), (B, H, K, V)]
+    y, state = ops.causal_conv1d_forward(meta(B, T, 96), meta(96, 4), None, None, None, True, "silu")
+    assert tuple(y.shape) == (B, T, 96) and tuple(state.shape) == (B, 96, 3)
+    gg, bb = ops.delta_rule_gates_forward(meta(B, T, H), meta(B, T, H), meta(H, dtype=torch.float32),
+                                          meta(H, dtype=torch.float32), False)  # fmt: skip
+    assert gg.dtype == torch.float32 and bb.dtype == torch.bfloat16 and tuple(gg.shape) == (B, T, H)
+    assert tuple(ops.gated_rmsnorm_forward(meta(B, T, H, V), meta(B, T, H * V), meta(V), None).shape) == (B, T, H, V)
