@@ -18,8 +18,8 @@ inputs already resident in HBM.  Prints ONE JSON line:
   epilogue     rmsnorm(o * silu(gate)) behind the operator, same batch, against the HBM peak
   cpu_baseline the naive token-by-token torch restatement of the operator (oracle/), timed on
                this host's cores on a bounded prefix of the same workload
-  forward_other the same forward on configurations 2 (packed sequences) and 4 (long context, V=256), and with
-               prepare and scan in one launch (an opt-in mode) on the headline configuration and on 4
+  forward_other the same forward with prepare and scan as two kernels (the headline configuration runs them as one
+               launch by default), and on configurations 2 (packed sequences) and 4 (long context, V=256; both ways)
 """
 
 from __future__ import annotations
@@ -43,7 +43,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # for a plain 1 GiB copy.  The readings live in profiles/hbm_traffic_counters.json together with a digest of the
 # kernel sources they were taken on; with other sources (a kernel was changed since) every traffic figure is null.
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_counters.json")
-_FUSED_MODE = []  # keeps the kernel-flag context of --fused-launch alive
+_LAUNCH_MODE = []  # keeps the kernel-flag context of --two-kernels alive
 _traffic_table = None
 
 
@@ -89,28 +89,35 @@ def parse_args():
     ap.add_argument("--no-decode", action="store_true", help="skip the decode, convolution, epilogue and backward legs")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target duration of the CPU baseline sample")
     ap.add_argument("--no-other-configs", action="store_true", help="skip the forward legs of configurations 2 and 4")
-    ap.add_argument("--fused-launch", action="store_true",
-                    help="run the headline step and everything after it with prepare and scan in one launch "
-                         "(Kernel.gated_delta_rule_fused_launch, an opt-in mode of the library)")
+    ap.add_argument("--two-kernels", action="store_true",
+                    help="run the headline step and everything after it with prepare and scan as two kernels "
+                         "(Kernel.gated_delta_rule_fused_launch off) also where the library would use one launch")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, the known-size kernel the HBM counters are scaled by")
     return ap.parse_args()
 
 
-def chunk_forward_leg(w, steps, warmup, fused_launch):
-    """Wall time per forward of workload ``w`` and the HIP-event durations of its kernels, one launch mode."""
+def launch_mode(two_kernels: bool):
+    """Context of a leg: the library's default (prepare and scan in one launch for the shapes where that is faster), or
+    prepare and scan as two kernels whatever the shape."""
     import contextlib
 
+    from lm_engine_amd.kernels import Kernel, enable_kernels
+
+    return enable_kernels([Kernel.gated_delta_rule], reset=True) if two_kernels else contextlib.nullcontext()
+
+
+def chunk_forward_leg(w, steps, warmup, two_kernels):
+    """Wall time per forward of workload ``w`` and the HIP-event durations of its kernels, one launch mode."""
     import torch
 
     import lm_engine_amd
-    from lm_engine_amd.kernels import Kernel, enable_kernels
-    from lm_engine_amd.ops import chunk_forward_kernel_times
+    from lm_engine_amd.ops import chunk_forward_kernel_times, fused_launch_applies
     from lm_engine_amd.workloads import chunk_fwd_flops_per_token_head, make_inputs
 
     inp = make_inputs(w, device="cuda")
-    mode = enable_kernels([Kernel.gated_delta_rule_fused_launch]) if fused_launch else contextlib.nullcontext()
-    with mode:
+    with launch_mode(two_kernels):
+        one_launch = fused_launch_applies(inp["q"], inp["v"], inp["cu_seqlens"])
         for _ in range(warmup):
             lm_engine_amd.chunk_gated_delta_rule(**inp, output_final_state=True)
         torch.cuda.synchronize()
@@ -129,7 +136,7 @@ def chunk_forward_leg(w, steps, warmup, fused_launch):
     torch.cuda.empty_cache()
     return {
         "workload": w.name, "B": w.B, "T": w.T, "H": w.H, "K": w.K, "V": w.V, "sequences": n_seq,
-        "launch": "prepare and scan in one launch" if fused_launch else "prepare, then scan",
+        "launch": "prepare and scan in one launch" if one_launch else "prepare, then scan",
         "ms_per_step": round(ms, 4),
         "tokens_per_s": round(w.B * w.T / (ms * 1e-3), 1),
         "tflops_dense": round(tflops, 1),
@@ -139,18 +146,18 @@ def chunk_forward_leg(w, steps, warmup, fused_launch):
     }  # fmt: skip
 
 
-def bench_chunk(w, steps, warmup, fused_launch=False):
+def bench_chunk(w, steps, warmup, two_kernels=False):
     import torch
 
     import lm_engine_amd
-    from lm_engine_amd.kernels import Kernel, enable_kernels
-    from lm_engine_amd.ops import chunk_forward_kernel_times
+    from lm_engine_amd.ops import chunk_forward_kernel_times, fused_launch_applies
     from lm_engine_amd.workloads import chunk_fwd_bytes_per_token_head, chunk_fwd_flops_per_token_head, make_inputs
 
-    if fused_launch:  # for the rest of the run
-        _FUSED_MODE.append(enable_kernels([Kernel.gated_delta_rule_fused_launch]))
-        _FUSED_MODE[-1].__enter__()
+    if two_kernels:  # for the rest of the run
+        _LAUNCH_MODE.append(launch_mode(True))
+        _LAUNCH_MODE[-1].__enter__()
     inp = make_inputs(w, device="cuda")
+    fused_launch = fused_launch_applies(inp["q"], inp["v"], inp["cu_seqlens"])
     call = lambda: lm_engine_amd.chunk_gated_delta_rule(**inp, output_final_state=True)  # noqa: E731
 
     for _ in range(warmup):
@@ -184,9 +191,10 @@ def bench_chunk(w, steps, warmup, fused_launch=False):
                 continue
             part = "dense"
         tflops = token_heads * flops[part] / (kernel_ms[name] * 1e-3) / 1e12
-        per_kernel[name] = {"ms": round(kernel_ms[name], 4), "algorithmic_flop_per_token_head": flops[part],
-                            "tflops": round(tflops, 1), "mfma_frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
-                            "traffic": measured_traffic(w.name, "chunk_fused" if fused_launch else name)}  # fmt: skip
+        key = "chunk_fused" if fused_launch else name
+        per_kernel[key] = {"ms": round(kernel_ms[name], 4), "algorithmic_flop_per_token_head": flops[part],
+                           "tflops": round(tflops, 1), "mfma_frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+                           "traffic": measured_traffic(w.name, key)}  # fmt: skip
     dominant = max(per_kernel, key=lambda name: per_kernel[name]["ms"])
     # HBM bytes of the whole step (every kernel of it), or null when a kernel has no reading
     step_traffic = [k["traffic"] for k in per_kernel.values()]
@@ -511,7 +519,7 @@ def main():
     torch.cuda.set_device(0)
 
     w = get_workload(args.workload)
-    result, inp = bench_chunk(w, args.steps, args.warmup, args.fused_launch)
+    result, inp = bench_chunk(w, args.steps, args.warmup, args.two_kernels)
     decode = None if args.no_decode else bench_decode(args.steps, args.warmup)
     conv = None if args.no_decode else bench_conv(w, args.steps, args.warmup)
     epilogue = None if args.no_decode else bench_epilogue(w, args.steps, args.warmup)
@@ -521,11 +529,11 @@ def main():
     other = None
     if not args.no_other_configs:
         # the forward on the other chunked configurations, and with prepare and scan in one launch where that qualifies
-        other = [chunk_forward_leg(w, args.steps, args.warmup, fused_launch=True)]
+        other = [chunk_forward_leg(w, args.steps, args.warmup, two_kernels=True)]
         for index in (2, 4):
             if index != args.workload:
-                other.append(chunk_forward_leg(get_workload(index), args.steps, args.warmup, fused_launch=False))
-        other.append(chunk_forward_leg(get_workload(4), args.steps, args.warmup, fused_launch=True))
+                other.append(chunk_forward_leg(get_workload(index), args.steps, args.warmup, two_kernels=False))
+        other.append(chunk_forward_leg(get_workload(4), args.steps, args.warmup, two_kernels=True))
     baseline = None if args.no_cpu_baseline else cpu_baseline(w, inp, args.cpu_seconds)
     if args.calibrate_copy:
         calibrate_copy()

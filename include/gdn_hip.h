@@ -43,8 +43,9 @@ enum {
     GDN_FLAG_STATE_INPLACE = 2, /* decode: ht == h0 is allowed and expected */
     GDN_FLAG_LEFT_PADDED = 4,   /* cu_seqlens describes a left-padded batch, see gdn_args */
     GDN_FLAG_FUSED_LAUNCH = 8,  /* gdn_chunk_fwd: run prepare and scan as one launch when the shape allows it (fixed-length
-                                   batch, K <= 128, V a multiple of 64, N * H * V / 64 at most half of the CUs); results
-                                   stay within the same parity gates but are not bit-identical to the two-kernel path */
+                                   batch, K <= 128, V a multiple of 64, N * H * V / 64 between 3/8 and 1/2 of the CUs: where
+                                   it is the faster way; other shapes run as without the flag); results stay within the
+                                   same parity gates but are not bit-identical to the two-kernel path */
 };
 
 /*

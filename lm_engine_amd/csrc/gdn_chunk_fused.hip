@@ -1,4 +1,4 @@
-// The chunked forward as ONE launch (K <= 128, fixed-length batches whose scan needs at most about half of the CUs):
+// The chunked forward as ONE launch (K <= 128, fixed-length batches whose scan fills about half of the CUs):
 // producer workgroups run the prepare step and scan workgroups consume its records as they appear.
 //
 // Scan workgroups.  gdn_chunk32.hip's scan gives one wave a whole 32-column slice of the state, and a slice a CU.
@@ -595,7 +595,7 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
 // ------------------------------------------------------------------------------------------
 // kernels
 // ------------------------------------------------------------------------------------------
-// Prepare and scan in one launch (fixed-length batches whose scan needs at most ~3/4 of the CUs).  Every workgroup
+// Prepare and scan in one launch (fixed-length batches whose scan fills between 3/8 and 1/2 of the CUs).  Every workgroup
 // takes a CU to itself (by its LDS size).  The first `prep_wgs` workgroups are producers: two groups of four waves
 // each run the prepare step on items of the chains that are scanned on their XCD, earliest chunks first, and set a
 // flag per finished record.  The others are scan workgroups whose loaders wait for those flags.  A producer never
@@ -646,7 +646,9 @@ static int launch_fused_k(ChunkParams& p, hipStream_t stream, int num_cus) {
     p.scan_groups = p.V / 64;
     const int64_t scan_wgs = chains8 * p.scan_groups;
     const int prep_wgs = (int)((num_cus - scan_wgs) / 8 * 8);
-    if (scan_wgs > (int64_t)num_cus * 3 / 4 || prep_wgs < num_cus / 4) return GDN_ERR_UNSUPPORTED;
+    // Worth it only when the scan fills about half of the CUs: with fewer chains the two-kernel path's scan, one slice per
+    // CU, is the faster one and prepare is short; with more, too few CUs are left for the producers.
+    if (scan_wgs > (int64_t)num_cus / 2 || scan_wgs < (int64_t)num_cus * 3 / 8) return GDN_ERR_UNSUPPORTED;
     const int64_t nflags = (int64_t)p.H * p.TC;
     hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((nflags + 255) / 256 < 64 ? (nflags + 255) / 256 : 64)), dim3(256), 0, stream, p.ready, nflags);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;

@@ -14,11 +14,6 @@ __device__ __forceinline__ float dpp_move(float x) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, ROW_MASK, 0xF, false));
 }
 
-__device__ __forceinline__ void split_hi_lo(float x, bf16_t& hi, bf16_t& lo) {
-    hi = (bf16_t)x;
-    lo = (bf16_t)(x - (float)hi);
-}
-
 // Stores into a record, `offset` bytes from its start.  DEVICE_SCOPE: written through to memory (scope bit sc1), so that
 // a workgroup on another XCD, whose L2 is a different one, reads what was written once the flag of the record says so.
 // (The alternative, a release fence at device scope, writes back every dirty line of the XCD's L2: 13 us per record.
@@ -88,6 +83,7 @@ __device__ __forceinline__ void chunk_prepare32_body(const ChunkParams& p, uint8
     float* const sA = reinterpret_cast<float*>(lds + KM_BYTES + C * LDK * 2);
     float* const s_gam = sA + C * LDA;
     float* const s_beta = s_gam + C, * const s_ssk = s_beta + C, * const s_ssq = s_ssk + C, * const s_rk = s_ssq + C, * const s_rq = s_rk + C;
+    float* const s_bri = s_ssk, * const s_g2 = s_ssq;  // from barrier #2 on: beta / |k| and gamma log2(e) per token
     float* const sT = sA;
     bf16_t* const sK = reinterpret_cast<bf16_t*>(sKM);
     float* const sTtA = reinterpret_cast<float*>(sKM);  // transpose of the top-left 32 x 32 of T
@@ -221,6 +217,10 @@ __device__ __forceinline__ void chunk_prepare32_body(const ChunkParams& p, uint8
             const float rq = p.l2norm ? rsqrtf(s_ssq[tid] + L2NORM_EPS) : 1.f;
             s_rk[tid] = rk;
             s_rq[tid] = rq;
+            // what the tile epilogues below multiply with, once per token instead of once per matrix entry (the sums of
+            // squares are not needed any more): beta_i / |k_i| and gamma_i in units of log 2
+            s_ssk[tid] = s_beta[tid] * rk;
+            s_ssq[tid] = gam * 1.44269504088896341f;
             // row scales the scan applies: to q S0, to the rows of V~ in the state update, to k S0 (none for
             // the rows past the end of a short chunk: the scan reads some other token's k and v there)
             const bool valid = tid < len;
@@ -249,32 +249,31 @@ __device__ __forceinline__ void chunk_prepare32_body(const ChunkParams& p, uint8
                 // register quad q of the tile holds rows 32 trow + 8 q + 4 h + 0..3: their per-token values in one read
                 if (!is_p) {
                     const int j = 32 * tcol + l32;
-                    const float gj = s_gam[j], rkj = s_rk[j];
+                    const float gj = s_g2[j], rkj = s_rk[j];
 #pragma unroll
                     for (int q = 0; q < 4; q++) {
                         const int i0 = 32 * trow + 8 * q + 4 * lh;
-                        const f32x4 bi = *reinterpret_cast<const f32x4*>(&s_beta[i0]);
-                        const f32x4 ri = *reinterpret_cast<const f32x4*>(&s_rk[i0]);
-                        const f32x4 gi = *reinterpret_cast<const f32x4*>(&s_gam[i0]);
+                        const f32x4 bi = *reinterpret_cast<const f32x4*>(&s_bri[i0]);
+                        const f32x4 gi = *reinterpret_cast<const f32x4*>(&s_g2[i0]);
 #pragma unroll
                         for (int e = 0; e < 4; e++) {
-                            const float val = bi[e] * ri[e] * rkj * __expf(gi[e] - gj) * acc[4 * q + e];
-                            sA[(i0 + e) * LDA + j] = (i0 + e > j) ? val : 0.f;
+                            const float val = bi[e] * __builtin_amdgcn_exp2f(gi[e] - gj) * (rkj * acc[4 * q + e]);
+                            sA[(i0 + e) * LDA + j] = (trow > tcol || i0 + e > j) ? val : 0.f;
                         }
                     }
                 } else {
                     const int i = 32 * tcol + l32;
-                    const float gi = s_gam[i], qi = p.scale * s_rq[i];
+                    const float gi = s_g2[i], qi = p.scale * s_rq[i];
                     f32x16 pv;
 #pragma unroll
                     for (int q = 0; q < 4; q++) {
                         const int j0 = 32 * trow + 8 * q + 4 * lh;
                         const f32x4 rj = *reinterpret_cast<const f32x4*>(&s_rk[j0]);
-                        const f32x4 gj = *reinterpret_cast<const f32x4*>(&s_gam[j0]);
+                        const f32x4 gj = *reinterpret_cast<const f32x4*>(&s_g2[j0]);
 #pragma unroll
                         for (int e = 0; e < 4; e++) {
-                            const float val = qi * rj[e] * __expf(gi - gj[e]) * acc[4 * q + e];
-                            pv[4 * q + e] = (i >= j0 + e) ? val : 0.f;
+                            const float val = rj[e] * __builtin_amdgcn_exp2f(gi - gj[e]) * (qi * acc[4 * q + e]);
+                            pv[4 * q + e] = (tcol > trow || i >= j0 + e) ? val : 0.f;
                         }
                     }
                     if (p.rec16) {
@@ -333,63 +332,42 @@ __device__ __forceinline__ void chunk_prepare32_body(const ChunkParams& p, uint8
         }
         __syncthreads();  // #4: diagonal blocks of T, all of A and P; K and Q are dead
 
-        // 16 x 16 x 16 product on one 16x16x32 MFMA pair with hi/lo split operands.
-        // x = rows of X (8 consecutive reduction entries k' = 8 (lq % 2) + e of row l16),
-        // y = rows of Y^T (same entries of column l16 of Y).  Returns X Y.
-        auto mm16v = [&](const f32x4 x0, const f32x4 x1, const f32x4 y0, const f32x4 y1) -> f32x4 {
-            bf16x8 a1, b1, a2, b2;
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                bf16_t xh, xl, yh, yl;
-                split_hi_lo(e < 4 ? x0[e] : x1[e - 4], xh, xl);
-                split_hi_lo(e < 4 ? y0[e] : y1[e - 4], yh, yl);
-                a1[e] = lq < 2 ? xh : xl;  // [X_hi | X_lo]
-                b1[e] = yh;                // [Y_hi ; Y_hi]
-                a2[e] = lq < 2 ? xh : (bf16_t)0.f;  // [X_hi | 0]
-                b2[e] = lq < 2 ? yl : (bf16_t)0.f;  // [Y_lo ; 0]
-            }
+        // 16 x 16 output tile of a product X Y on the fp32 MFMA (16x16x4: no operand is rounded).  Lane (l16, lq) supplies
+        // reduction entries k = 4 n lq + e, e < 4 n, of row l16 of X and of column l16 of Y (a row of Y^T); MFMA e takes
+        // entry e of every lane, i.e. the four k = 4 n lq' + e, and the 4 n MFMAs together cover all 16 n.
+        auto mm16 = [&](const float* xrow, const float* ytrow) -> f32x4 {  // 16 reduction entries, k = 4 lq + e
+            const f32x4 x = *reinterpret_cast<const f32x4*>(xrow), y = *reinterpret_cast<const f32x4*>(ytrow);
             f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-            acc = mfma_bf16(a1, b1, acc);
-            acc = mfma_bf16(a2, b2, acc);
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc = mfma_f32(x[e], y[e], acc);
             return acc;
         };
-        auto mm16 = [&](const float* xrow, const float* ytrow) -> f32x4 {
-            return mm16v(*reinterpret_cast<const f32x4*>(xrow), *reinterpret_cast<const f32x4*>(xrow + 4),
-                         *reinterpret_cast<const f32x4*>(ytrow), *reinterpret_cast<const f32x4*>(ytrow + 4));
-        };
-        // 16 x 16 output tile of a product with 32 reduction entries (k = 8 lq + e), hi/lo split: 3 MFMAs
-        auto mm16x32 = [&](const float* xrow, const float* ytrow) -> f32x4 {
+        auto mm16x32 = [&](const float* xrow, const float* ytrow) -> f32x4 {  // 32 reduction entries, k = 8 lq + e
             const f32x4 x0 = *reinterpret_cast<const f32x4*>(xrow), x1 = *reinterpret_cast<const f32x4*>(xrow + 4);
             const f32x4 y0 = *reinterpret_cast<const f32x4*>(ytrow), y1 = *reinterpret_cast<const f32x4*>(ytrow + 4);
-            bf16x8 xh, xl, yh, yl;
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                bf16_t a, b, c, d;
-                split_hi_lo(e < 4 ? x0[e] : x1[e - 4], a, b);
-                split_hi_lo(e < 4 ? y0[e] : y1[e - 4], c, d);
-                xh[e] = a, xl[e] = b, yh[e] = c, yl[e] = d;
-            }
             f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-            acc = mfma_bf16(xh, yh, acc);
-            acc = mfma_bf16(xl, yh, acc);
-            acc = mfma_bf16(xh, yl, acc);
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc = mfma_f32(x0[e], y0[e], acc);
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc = mfma_f32(x1[e], y1[e], acc);
             return acc;
         };
 
         // ---- level A: T_10 = -T_11 (A_10 T_00) on wave 0, T_32 = -T_33 (A_32 T_22) on wave 1 ----
         if (wave < 2) {
             const int bi = 2 * wave + 1, bj = 2 * wave;
-            const int kk = 8 * (lq % 2);
+            const int kk = 4 * lq;
             float* const mt = &sMt[wave * 16 * LDM];
-            // column l16 of T_bj,bj, entries kk .. kk + 7 (a row of its transpose)
-            f32x4 y0, y1;
+            // column l16 of T_bj,bj, entries kk .. kk + 3 (a row of its transpose)
+            f32x4 y0;
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                y0[e] = sT[(16 * bj + kk + e) * LDA + 16 * bj + l16];
-                y1[e] = sT[(16 * bj + kk + 4 + e) * LDA + 16 * bj + l16];
+            for (int e = 0; e < 4; e++) y0[e] = sT[(16 * bj + kk + e) * LDA + 16 * bj + l16];
+            f32x4 m = {0.f, 0.f, 0.f, 0.f};
+            {
+                const f32x4 xa = *reinterpret_cast<const f32x4*>(&sA[(16 * bi + l16) * LDA + 16 * bj + kk]);
+#pragma unroll
+                for (int e = 0; e < 4; e++) m = mfma_f32(xa[e], y0[e], m);
             }
-            const float* arow = &sA[(16 * bi + l16) * LDA + 16 * bj + kk];
-            const f32x4 m = mm16v(*reinterpret_cast<const f32x4*>(arow), *reinterpret_cast<const f32x4*>(arow + 4), y0, y1);
             if (wave == 0 && lq < 2) {
                 // K's region is free now: the transposes of T_00 and T_11 for level B, from the registers of the inverse,
                 // and the zero block (T_01)^T

@@ -10,11 +10,12 @@ guard the HIP operator the way the other mixers guard theirs.
 Difference from the reference: ``gated_delta_rule`` is ON by default, and switching it off makes
 the operator raise: this package ships no second implementation to fall back to.
 
-``Kernel.gated_delta_rule_fused_launch`` (off by default, as every flag of the reference is) asks the
-chunked forward to run its prepare and scan steps as one launch where the shape allows it
-(``GDN_FLAG_FUSED_LAUNCH`` of the C ABI).  Results stay within the same parity gates, but they are not
-bit-identical to the two-kernel path, which batches that do not qualify (packed, left-padded, many
-sequences) still take: leave it off where runs are compared bit for bit.
+``Kernel.gated_delta_rule_fused_launch`` (on by default as well) lets the chunked forward run its prepare and
+scan steps as one launch for the shapes where that is the faster way (``GDN_FLAG_FUSED_LAUNCH`` of the C ABI:
+fixed-length batches whose scan fills about half of the GPU).  Results stay within the same parity gates, but
+they are not bit-identical to the two-kernel path, which every other batch takes (packed, left-padded, few or
+many sequences): switch it off - ``enable_kernels([Kernel.gated_delta_rule], reset=True)`` or
+``ENABLE_KERNELS=gated_delta_rule`` - where runs of different batch shapes are compared bit for bit.
 """
 
 from __future__ import annotations
@@ -29,7 +30,7 @@ class Kernel(Enum):
     gated_delta_rule_fused_launch = "gated_delta_rule_fused_launch"
 
 
-_ON_BY_DEFAULT = (Kernel.gated_delta_rule,)
+_ON_BY_DEFAULT = (Kernel.gated_delta_rule, Kernel.gated_delta_rule_fused_launch)
 _KERNELS: dict[Kernel, bool] = {kernel: kernel in _ON_BY_DEFAULT for kernel in Kernel}
 
 

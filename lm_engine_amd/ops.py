@@ -169,6 +169,22 @@ def _run(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_se
     return o, ht
 
 
+def fused_launch_applies(q, v, cu_seqlens=None) -> bool:
+    """Whether ``chunk_gated_delta_rule`` runs these inputs as one launch (prepare and scan together): the flag
+    ``Kernel.gated_delta_rule_fused_launch`` is on and the library's rule holds - bf16, a fixed-length batch, K 64 or
+    128, V a multiple of 64, and the scan's workgroups (one per 64 columns of every sequence-head chain, the chains
+    rounded up to a multiple of 8) fill between 3/8 and 1/2 of the compute units."""
+    if not is_kernel_allowed(Kernel.gated_delta_rule_fused_launch) or cu_seqlens is not None or q.dtype != torch.bfloat16:
+        return False
+    B, _, H, K = q.shape
+    V = v.size(-1)
+    if K not in (64, 128) or V % 64 != 0:
+        return False
+    cus = torch.cuda.get_device_properties(q.device).multi_processor_count
+    scan_workgroups = (B * H + 7) // 8 * 8 * (V // 64)
+    return cus * 3 // 8 <= scan_workgroups <= cus // 2
+
+
 def chunk_forward_kernel_times(
     q, k, v, g=None, beta=None, scale=None, initial_state=None, output_final_state=False, cu_seqlens=None,
     use_qk_l2norm_in_kernel=False,

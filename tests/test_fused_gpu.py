@@ -8,7 +8,7 @@ import torch
 
 import lm_engine_amd
 from lm_engine_amd.kernels import Kernel, enable_kernels
-from lm_engine_amd.ops import chunk_forward_kernel_times
+from lm_engine_amd.ops import chunk_forward_kernel_times, fused_launch_applies
 from lm_engine_amd.workloads import get_workload, make_inputs
 from oracle.c_oracle import recurrent_gated_delta_rule_c
 from tests.helpers import assert_parity, max_abs, random_inputs, rel_l2
@@ -19,11 +19,23 @@ BF16 = torch.bfloat16
 FUSED = [Kernel.gated_delta_rule_fused_launch]
 
 
+def two_kernels():
+    """Inside the block the forward runs prepare and scan as two kernels whatever the shape."""
+    return enable_kernels([Kernel.gated_delta_rule], reset=True)
+
+
 def _to_gpu(inp):
     return {n: (x.cuda() if isinstance(x, torch.Tensor) else x) for n, x in inp.items()}
 
 
+def _qualifies(inp):
+    """The rule of the library (ops.fused_launch_applies); inputs on the CPU or on the GPU."""
+    with enable_kernels(FUSED):
+        return fused_launch_applies(inp["q"].cuda(), inp["v"], inp.get("cu_seqlens"))
+
+
 def _check(inp, label, **kwargs):
+    assert _qualifies(inp), "this shape would take the two-kernel path"
     print(f"case: fused launch {label} q={tuple(inp['q'].shape)} v={tuple(inp['v'].shape)} {kwargs}", flush=True)
     o_ref, h_ref = recurrent_gated_delta_rule_c(**inp, output_final_state=True, **kwargs)
     with enable_kernels(FUSED):
@@ -40,34 +52,36 @@ def test_the_flag_selects_the_single_launch():
     # with the flag the prepare kernel is not launched: the interval between the events around it holds no kernel
     inp = _to_gpu(random_inputs(B=2, T=4096, H=32, K=128, V=128, dtype=BF16, seed=149))
     for _ in range(2):  # the first call of each loads its kernels
-        split = chunk_forward_kernel_times(**inp, output_final_state=True)
+        with two_kernels():
+            split = chunk_forward_kernel_times(**inp, output_final_state=True)
         with enable_kernels(FUSED):
             fused = chunk_forward_kernel_times(**inp, output_final_state=True)
+    assert fused_launch_applies(inp["q"], inp["v"]), "on by default"
     print(f"kernel times, ms: two kernels {split}, one launch {fused}", flush=True)
     assert fused["chunk_prepare"] < 0.5 * split["chunk_prepare"] and fused["chunk_scan"] > split["chunk_scan"]
 
 
 @pytest.mark.parametrize("T", [65, 128, 130, 321])
 def test_sequence_lengths_with_tail_chunks(T):
-    _check(random_inputs(B=2, T=T, H=2, K=128, V=128, dtype=BF16, seed=150 + T), f"T={T}")
+    _check(random_inputs(B=4, T=T, H=16, K=128, V=128, dtype=BF16, seed=150 + T), f"T={T}")
 
 
-@pytest.mark.parametrize("K, V", [(64, 64), (64, 128), (128, 64), (128, 256)])
-def test_head_dims(K, V):
-    _check(random_inputs(B=1, T=200, H=3, K=K, V=V, dtype=BF16, seed=160 + K + V), f"K={K} V={V}")
+@pytest.mark.parametrize("K, V, B", [(64, 64, 8), (64, 128, 4), (128, 64, 8), (128, 256, 2)])
+def test_head_dims(K, V, B):
+    _check(random_inputs(B=B, T=200, H=14, K=K, V=V, dtype=BF16, seed=160 + K + V), f"K={K} V={V}")
 
 
 def test_options_l2norm_scale_no_state_ungated():
-    inp = random_inputs(B=2, T=257, H=2, K=128, V=128, dtype=BF16, seed=171, normalize=False)
+    inp = random_inputs(B=4, T=257, H=14, K=128, V=128, dtype=BF16, seed=171, normalize=False)
     _check(inp, "in-kernel l2norm, scale 0.3", use_qk_l2norm_in_kernel=True, scale=0.3)
-    inp = random_inputs(B=1, T=192, H=2, K=128, V=128, dtype=BF16, seed=172, gated=False, h0=False)
+    inp = random_inputs(B=3, T=192, H=16, K=128, V=128, dtype=BF16, seed=172, gated=False, h0=False)
     _check(dict(inp, beta=None), "ungated, beta = 1, zero state")
 
 
 def test_strided_projection_slices():
     # q, k, v as slices of one fused projection, the way the layer passes them
     gen = torch.Generator("cpu").manual_seed(173)
-    B, T, H, K, V = 1, 300, 4, 128, 128
+    B, T, H, K, V = 4, 300, 16, 128, 128
     proj = torch.randn(B, T, H * (2 * K + V), generator=gen).to(BF16)
     q, k, v = (x.reshape(B, T, H, -1) for x in proj.split([H * K, H * K, H * V], dim=-1))
     q = torch.nn.functional.normalize(q.float(), dim=-1).to(BF16)  # contiguous copy: only k and v stay strided
@@ -98,19 +112,24 @@ def test_config4_long_context_and_the_split_property():
 
 
 def test_close_to_the_two_kernel_path_and_fallback_is_unchanged():
-    inp = _to_gpu(random_inputs(B=3, T=500, H=4, K=128, V=128, dtype=BF16, seed=180))
-    o_split, h_split = lm_engine_amd.chunk_gated_delta_rule(**inp, output_final_state=True)
+    inp = _to_gpu(random_inputs(B=4, T=500, H=16, K=128, V=128, dtype=BF16, seed=180))
+    assert _qualifies(inp)
+    with two_kernels():
+        o_split, h_split = lm_engine_amd.chunk_gated_delta_rule(**inp, output_final_state=True)
     with enable_kernels(FUSED):
         o_fused, h_fused = lm_engine_amd.chunk_gated_delta_rule(**inp, output_final_state=True)
     assert rel_l2(o_fused.float(), o_split.float()) < 5e-3 and rel_l2(h_fused, h_split) < 1e-3
     # shapes that do not qualify take the two-kernel path whatever the flag says: packed sequences, V not a multiple of 64,
-    # more scan workgroups than three quarters of the CUs
+    # more scan workgroups than half of the CUs, fewer than three eighths
     packed = _to_gpu(random_inputs(B=1, T=300, H=2, K=128, V=128, dtype=BF16, seed=181, N=3))
     cu = torch.tensor([0, 70, 71, 300], dtype=torch.int32, device="cuda")
     odd_v = _to_gpu(random_inputs(B=1, T=130, H=2, K=128, V=96, dtype=BF16, seed=182))
     many = _to_gpu(random_inputs(B=20, T=130, H=16, K=128, V=128, dtype=BF16, seed=183))
-    for case, extra in ((packed, dict(cu_seqlens=cu)), (odd_v, {}), (many, {})):
-        a = lm_engine_amd.chunk_gated_delta_rule(**case, output_final_state=True, **extra)
+    few = _to_gpu(random_inputs(B=1, T=300, H=16, K=128, V=128, dtype=BF16, seed=184))
+    assert not any(_qualifies(case) for case in (odd_v, many, few))
+    for case, extra in ((packed, dict(cu_seqlens=cu)), (odd_v, {}), (many, {}), (few, {})):
+        with two_kernels():
+            a = lm_engine_amd.chunk_gated_delta_rule(**case, output_final_state=True, **extra)
         with enable_kernels(FUSED):
             b = lm_engine_amd.chunk_gated_delta_rule(**case, output_final_state=True, **extra)
         assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])

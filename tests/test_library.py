@@ -199,12 +199,12 @@ def test_kernel_flag_registry_follows_the_reference_convention():
     assert is_kernel_allowed(Kernel.gated_delta_rule)
 
 
-def test_fused_launch_flag_is_off_by_default():
+def test_fused_launch_flag_is_on_by_default_and_can_be_switched_off():
     fused = Kernel.gated_delta_rule_fused_launch
-    assert not is_kernel_allowed(fused)
-    with enable_kernels([fused]):
-        assert is_kernel_allowed(fused) and is_kernel_allowed(Kernel.gated_delta_rule)
-    assert not is_kernel_allowed(fused)
+    assert is_kernel_allowed(fused)
+    with enable_kernels([Kernel.gated_delta_rule], reset=True):
+        assert not is_kernel_allowed(fused) and is_kernel_allowed(Kernel.gated_delta_rule)
+    assert is_kernel_allowed(fused)
     assert _lib.GDN_FLAG_FUSED_LAUNCH == 8
 
 
