@@ -43,6 +43,8 @@ E_ij = exp(gamma_i - gamma_j) for j <= i):
 
 from __future__ import annotations
 
+import weakref
+
 import torch
 
 
@@ -50,14 +52,30 @@ CHUNK = 64
 L2NORM_EPS = 1e-6  # the epsilon of the forward kernels' q/k normalisation
 
 
+# Host copies of the prefixes that backward passes have asked for, by tensor object: a model calls the operator once per
+# layer with the same cu_seqlens tensor, and only the first backward of a step should wait for the device.  An entry
+# is valid for that very object at that version (in-place writes bump it) and goes when the tensor does.
+_HOST_PREFIX: dict[int, tuple] = {}
+
+
+def _host_prefix(cu_seqlens) -> list[int]:
+    key = id(cu_seqlens)
+    hit = _HOST_PREFIX.get(key)
+    if hit is not None and hit[0]() is cu_seqlens and hit[1] == cu_seqlens._version:
+        return hit[2]
+    values = cu_seqlens.detach().to("cpu", torch.int64).tolist()
+    _HOST_PREFIX[key] = (weakref.ref(cu_seqlens, lambda _, key=key: _HOST_PREFIX.pop(key, None)), cu_seqlens._version, values)
+    return values
+
+
 def _chains(B, T, cu_seqlens, left_padded):
     """Start (in the flattened [B * T] token axis) and length of every sequence."""
     if cu_seqlens is None:
         return [b * T for b in range(B)], [T] * B
     # The layout of the packed gradients depends on the longest sequence, so the prefix has to come to the host
-    # (one copy of N + 1 integers per backward).  It is checked here, where it is visible: the forward kernels
-    # clamp a malformed prefix, the index arithmetic below would not.
-    cu = cu_seqlens.detach().to("cpu", torch.int64).tolist()
+    # (one copy of N + 1 integers, once per cu_seqlens tensor).  It is checked here, where it is visible: the forward
+    # kernels clamp a malformed prefix, the index arithmetic below would not.
+    cu = _host_prefix(cu_seqlens)
     limit = B * T if left_padded else T
     if cu[0] != 0 or any(cu[n + 1] < cu[n] for n in range(len(cu) - 1)) or cu[-1] > limit:
         raise ValueError(f"cu_seqlens must start at 0, be non-decreasing and end at or below {limit}, got {cu}")

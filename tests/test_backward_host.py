@@ -96,3 +96,18 @@ def test_gradients_come_back_in_the_input_dtypes():
     got = gated_delta_rule_backward(bf(q), bf(k), bf(v), g.float(), bf(beta), bf(do), dht.float(),
                                     initial_state=h0.float(), use_qk_l2norm_in_kernel=True)  # fmt: skip
     assert [x.dtype for x in got] == [torch.bfloat16] * 3 + [torch.float32, torch.bfloat16, torch.float32]
+
+
+def test_host_copy_of_cu_seqlens_is_made_once_per_tensor_and_version():
+    from lm_engine_amd import backward
+
+    cu = torch.tensor([0, 70, 130], dtype=torch.int32)
+    first = backward._host_prefix(cu)
+    assert first == [0, 70, 130] and backward._host_prefix(cu) is first  # the second call reuses the list
+    cu[1] = 64  # an in-place write makes the copy stale
+    assert backward._host_prefix(cu) == [0, 64, 130]
+    other = torch.tensor([0, 70, 130], dtype=torch.int32)
+    assert backward._host_prefix(other) is not first
+    key = id(cu)
+    del cu
+    assert key not in backward._HOST_PREFIX  # the entry goes with its tensor

@@ -1,7 +1,8 @@
 """gdn_chunk_fwd_noalloc, the entry point for callers that cannot allocate device memory, against
 gdn_chunk_fwd on the same inputs: both run the same kernels, so outputs and final states must be
 bit-identical.  Two calls in a row share the library's built-in scratch array; the second is smaller,
-so stale records of the first lie behind the ones it writes."""
+so stale records of the first lie behind the ones it writes.  (The arguments carry the library's default flags: the
+first shape qualifies for the one-launch forward, whose ready flags then live in the scratch array too.)"""
 
 import ctypes
 
@@ -43,7 +44,8 @@ def _both_entry_points(B, T, H, K, V, seed, cu_seqlens=None):
 
 def test_noalloc_entry_point_matches_chunk_fwd_on_two_calls_in_a_row():
     for B, T, H, K, V, seed, cu in [
-        (2, 1024, 8, 128, 128, 5, None),                 # first call: 128 chunk records per head
+        (4, 512, 16, 128, 128, 4, None),                 # a shape that runs prepare and scan as one launch (ready flags in the scratch)
+        (2, 1024, 8, 128, 128, 5, None),                 # 128 chunk records per head, two kernels
         (1, 200, 4, 128, 128, 6, None),                  # second, smaller call: 4 records, a partial last chunk
         (1, 512, 4, 128, 256, 7, [0, 130, 131, 512]),    # packed: the chunk offsets live in the scratch as well
     ]:  # fmt: skip
