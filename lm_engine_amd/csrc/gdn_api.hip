@@ -66,6 +66,10 @@ int validate_common(const gdn_args* a) {
         if (s < 0 || s % elems16 != 0) return GDN_ERR_ALIGN;
     if (a->q_stride_h < a->K || a->k_stride_h < a->K || a->v_stride_h < a->V || a->o_stride_h < a->V)
         return GDN_ERR_SHAPE;
+    // the kernels address the 64 rows of a chunk with 32-bit byte offsets from the chunk's first row
+    const int64_t token_strides[] = {a->q_stride_t, a->k_stride_t, a->v_stride_t, a->o_stride_t};
+    for (int64_t s : token_strides)
+        if (s > ((int64_t)1 << 24)) return GDN_ERR_UNSUPPORTED;
     if (!aligned(a->q, 16) || !aligned(a->k, 16) || !aligned(a->v, 16) || !aligned(a->o, 16)) return GDN_ERR_ALIGN;
     if ((a->h0 && !aligned(a->h0, 16)) || (a->ht && !aligned(a->ht, 16))) return GDN_ERR_ALIGN;
     if (a->g && !aligned(a->g, 4)) return GDN_ERR_ALIGN;

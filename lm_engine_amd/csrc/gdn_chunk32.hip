@@ -52,7 +52,7 @@ namespace gdn {
 // prepare as a kernel of its own: persistent workgroups of four waves, three per CU
 // ------------------------------------------------------------------------------------------
 template <int K>
-__global__ __launch_bounds__(PREP_THREADS, 3) void chunk_prepare32_kernel(const ChunkParams p) {
+__global__ __launch_bounds__(PREP_THREADS, (K > 128 ? 1 : 3)) void chunk_prepare32_kernel(const ChunkParams p) {
     __shared__ __attribute__((aligned(16))) uint8_t lds[prepare32_lds_bytes<K>()];
     // Work items: (chunk slot, head), the slots rounded up to a multiple of 8.  Workgroup i runs on XCD i % 8 and
     // takes items i, i + grid, ... with the grid a multiple of 8, so w % 8 names the XCD.  That digit goes into
@@ -341,6 +341,12 @@ struct Scan16Schedule : Scan16Rules<K> {
 template <int K, int NW, bool NT = false, bool SAVE = false, bool HALF = false>
 __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kernel(const ChunkParams p) {
     static_assert(!HALF || (NW == 1 && !SAVE), "the half-slice scan has one slice per workgroup and saves nothing");
+    // K = 256: two stage halves with the rows of q and k do not fit the LDS.  The rows of q, which a chunk needs for
+    // one group of MFMAs only, then get a single buffer and a second workgroup barrier per chunk ("barrier Q"), passed
+    // by a compute wave once it holds the last fragment of q: the loaders write the next chunk's rows of q between
+    // that barrier and the one at the end of the chunk.
+    constexpr bool QS = K > 128;
+    static_assert(!QS || HALF, "K = 256 runs as half slices");
     constexpr int NL = SCAN_LOADERS;
     // a separate wave writes the output (see below); with four compute waves the LDS has no room for its staging
     constexpr bool OS = NW < 4;
@@ -357,8 +363,8 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
     constexpr int QLD = 2 * K + 16;                  // bytes per staged row of q / k (16 bytes of padding against bank conflicts)
     constexpr int Q_UNITS = C * 2 * K / FRAG_BYTES;  // 1 KiB pieces of the q rows: 512 / K whole rows each; as many for k
     constexpr int V_OFF = SHARED_BYTES;
-    constexpr int Q_OFF = V_OFF + C * VLD;
-    constexpr int K_OFF = Q_OFF + C * QLD;
+    constexpr int Q_OFF = V_OFF + C * VLD;                 // not part of the stage halves when QS
+    constexpr int K_OFF = QS ? Q_OFF : Q_OFF + C * QLD;
     constexpr int QS_OFF = K_OFF + C * QLD;
     constexpr int KS_OFF = QS_OFF + C * 4;
     constexpr int CS_OFF = KS_OFF + C * 4;
@@ -369,9 +375,10 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
     constexpr int NQ = 2 * Q_UNITS / NL;   // q / k row slots per loader wave
     constexpr int NLOAD = NF + NV + NQ;    // 1 KiB moves per loader wave and chunk
     static_assert(SHARED_FRAGS % NL == 0 && V_UNITS % NL == 0 && (2 * Q_UNITS) % NL == 0, "the pieces must divide over the loader waves");
-    static_assert(2 * STAGE_BYTES + (OS ? NW * 2 * C * 64 : 16) <= 160 * 1024, "stage exceeds LDS");
+    static_assert(2 * STAGE_BYTES + (QS ? C * QLD : 0) + (OS ? NW * 2 * C * 64 : 16) <= 160 * 1024, "stage exceeds LDS");
 
     __shared__ __attribute__((aligned(16))) uint8_t stage[2][STAGE_BYTES];
+    __shared__ __attribute__((aligned(16))) uint8_t qstage[QS ? C * QLD : 16];  // the single buffer of q rows (QS)
     __shared__ __attribute__((aligned(16))) uint8_t ostage[OS ? NW * 2 * C * 64 : 16];
 
     const int lane = threadIdx.x % WAVE;
@@ -438,6 +445,7 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
         };
         __syncthreads();
         for (int c = 0; c < nchunks; c++) {
+            if constexpr (QS) __syncthreads();  // barrier Q
             __syncthreads();
             if (c > 0) flush(c - 1);
         }
@@ -458,7 +466,16 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
         const int rot_q = vgroup % NQ;
         auto frag_of = [&](int i) { return lw * NF + (i + rot_f < NF ? i + rot_f : i + rot_f - NF); };   // i < NF
         auto vunit_of = [&](int i) { return lw * NV + i; };                                              // i < NV
-        auto qunit_of = [&](int i) { return lw * NQ + (i + rot_q < NQ ? i + rot_q : i + rot_q - NQ); };  // i < NQ
+        // (QS: the first NQ / 2 slots of every wave are rows of q, the others rows of k, so that every wave writes its
+        // share of q after barrier Q; no rotation, so that a slot's place is the wave's first unit plus a constant)
+        constexpr int NQH = NQ / 2;
+        auto qunit_of = [&](int i) {  // i < NQ
+            if constexpr (QS) {
+                return (i < NQH ? 0 : Q_UNITS) + lw * NQH + i % NQH;
+            } else {
+                return lw * NQ + (i + rot_q < NQ ? i + rot_q : i + rot_q - NQ);
+            }
+        };
         // rows of q, k: lane -> (row within the unit, 16-byte piece); likewise for v
         constexpr int Q_ROWS = C / Q_UNITS, Q_PIECES = WAVE / Q_ROWS;
         constexpr int V_ROWS = C / V_UNITS, V_PIECES = WAVE / V_ROWS;
@@ -474,8 +491,28 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
             float qs, ks, cs, eg;
         };
         Scalars sc0 = {0.f, 0.f, 0.f, 0.f}, sc1 = {0.f, 0.f, 0.f, 0.f};
+        // (QS: wave-uniform 64-bit base of the chunk + 32-bit per-lane byte offset formed at the load, so that no
+        // per-slot 64-bit lane addresses stay live: with 20 slots per buffer they would not fit the registers)
+        const bf16_t* const qg0 = p.q + b * p.q_stride_b + seq_t0 * p.q_stride_t + (int64_t)h * p.q_stride_h;
+        const bf16_t* const kg0 = p.k + b * p.k_stride_b + seq_t0 * p.k_stride_t + (int64_t)h * p.k_stride_h;
+        const bf16_t* const vg0 = p.v + b * p.v_stride_b + seq_t0 * p.v_stride_t + (int64_t)h * p.v_stride_h + 32 * (vgroup * NW);
         auto src_of = [&](int c, int i) -> const uint8_t* {
             if (i < NF) return rec + ((int64_t)c * p.rec_bytes + (int64_t)frag_of(i) * FRAG_BYTES) + lane * 16;
+            if constexpr (QS) {
+                const int last = (int)min((int64_t)C, seq_len - (int64_t)c * C) - 1;  // wave-uniform
+                if (i < NF + NV) {
+                    const uint32_t off = (uint32_t)min(vunit_of(i - NF) * V_ROWS + v_row, last) * ((uint32_t)p.v_stride_t * 2u) + (uint32_t)v_piece * 16u;
+                    return reinterpret_cast<const uint8_t*>(vg0 + (int64_t)c * C * p.v_stride_t) + off;
+                }
+                // row of this lane in the wave's first unit; hidden from the optimiser at every use, or the offsets of
+                // all slots are formed ahead of the loop and held in registers
+                int row0 = lw * NQH * Q_ROWS + q_row;
+                asm volatile("" : "+v"(row0));
+                const bool is_k = i - NF - NV >= NQH;
+                const uint32_t stride = (uint32_t)(is_k ? p.k_stride_t : p.q_stride_t) * 2u;
+                const uint32_t off = (uint32_t)min(row0 + ((i - NF - NV) % NQH) * Q_ROWS, last) * stride + (uint32_t)q_piece * 16u;
+                return reinterpret_cast<const uint8_t*>((is_k ? kg0 : qg0) + (int64_t)c * C * (is_k ? p.k_stride_t : p.q_stride_t)) + off;
+            }
             // a row past the end of the sequence (tail chunk) is read from the last token instead: never used
             if (i < NF + NV) {
                 const int tok = min(c * C + vunit_of(i - NF) * V_ROWS + v_row, (int)seq_len - 1);
@@ -490,7 +527,15 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
         auto dst_of = [&](uint8_t* st, int i) -> uint8_t* {
             if (i < NF) return st + frag_of(i) * FRAG_BYTES + lane * 16;
             if (i < NF + NV) return st + V_OFF + (vunit_of(i - NF) * V_ROWS + v_row) * VLD + v_piece * 16;
-            return st + Q_OFF + (qunit_of(i - NF - NV) * Q_ROWS + q_row) * QLD + q_piece * 16;  // the k rows follow the q rows
+            if constexpr (QS) {
+                // the lane's place in the wave's first unit plus a compile-time constant
+                const int lane_off = (lw * NQH * Q_ROWS + q_row) * QLD + q_piece * 16;
+                const int slot_off = ((i - NF - NV) % NQH) * Q_ROWS * QLD;
+                if (i - NF - NV < NQH) return qstage + lane_off + slot_off;
+                return st + K_OFF + lane_off + slot_off;
+            } else {
+                return st + Q_OFF + (qunit_of(i - NF - NV) * Q_ROWS + q_row) * QLD + q_piece * 16;  // the k rows follow the q rows
+            }
         };
         // every loader wave carries the scales (identical values, identical LDS writes)
         auto load_scalars = [&](Scalars& sc, int c) {
@@ -511,8 +556,10 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
         };
         // write chunk c to LDS and refill each register with chunk c2 right behind its write, so the
         // LDS-write and the vector-memory queues fill together
-        auto store_and_reload = [&](bf16x8(&buf)[NLOAD], Scalars& sc, int c, int c2, auto reload_tag) {
+        // (QS: the rows of q, slots NF + NV .. NF + NV + NQH - 1, go last, after barrier Q when `barrier_q` is set)
+        auto store_and_reload = [&](bf16x8(&buf)[NLOAD], Scalars& sc, int c, int c2, auto reload_tag, auto barrier_q_tag) {
             constexpr bool reload = decltype(reload_tag)::value;
+            constexpr bool barrier_q = decltype(barrier_q_tag)::value;
             uint8_t* dst = stage[c & 1];
             reinterpret_cast<float*>(dst + QS_OFF)[lane] = sc.qs;
             reinterpret_cast<float*>(dst + KS_OFF)[lane] = sc.ks;
@@ -520,9 +567,19 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
             if (lane == 0) *reinterpret_cast<float*>(dst + EG_OFF) = sc.eg;
 #pragma unroll
             for (int i = 0; i < NLOAD; i++) {
+                if (QS && i >= NF + NV && i < NF + NV + NQH) continue;
                 *reinterpret_cast<bf16x8*>(dst_of(dst, i)) = buf[i];
                 if constexpr (reload) buf[i] = fetch(src_of(c2, i));
                 __builtin_amdgcn_sched_barrier(0);
+            }
+            if constexpr (QS) {
+                if constexpr (barrier_q) __syncthreads();  // barrier Q: the compute waves have read the rows of q in the buffer
+#pragma unroll
+                for (int i = NF + NV; i < NF + NV + NQH; i++) {
+                    *reinterpret_cast<bf16x8*>(dst_of(dst, i)) = buf[i];
+                    if constexpr (reload) buf[i] = fetch(src_of(c2, i));
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
             if constexpr (reload) load_scalars(sc, c2);
         };
@@ -532,28 +589,32 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
         if (nchunks > 0) {
             load(buf0, sc0, 0);
             if (nchunks > 1) load(buf1, sc1, 1);
-            if (nchunks > 2) store_and_reload(buf0, sc0, 0, 2, yes);
-            else store_and_reload(buf0, sc0, 0, 0, no);
+            if (nchunks > 2) store_and_reload(buf0, sc0, 0, 2, yes, no);
+            else store_and_reload(buf0, sc0, 0, 0, no, no);
         }
         __syncthreads();  // stage[0] holds chunk 0
         // Barrier of iteration c: the compute waves are done with stage[c & 1] and chunk c + 1 is in the
         // other half.  Before it: write chunk c + 1 (its half was released by the barrier of iteration
         // c - 1) and refill the freed registers with chunk c + 3.
         int c = 0;
+        // (QS: every iteration has barrier Q as well: inside store_and_reload, or on its own when nothing is left to write)
         for (; c + 4 < nchunks; c += 2) {  // steady state: straight-line code, both reloads exist
-            store_and_reload(buf1, sc1, c + 1, c + 3, yes);
+            store_and_reload(buf1, sc1, c + 1, c + 3, yes, yes);
             __syncthreads();
-            store_and_reload(buf0, sc0, c + 2, c + 4, yes);
+            store_and_reload(buf0, sc0, c + 2, c + 4, yes, yes);
             __syncthreads();
         }
         for (; c < nchunks; c += 2) {  // the last (at most four) chunks
             if (c + 1 < nchunks) {
-                if (c + 3 < nchunks) store_and_reload(buf1, sc1, c + 1, c + 3, yes);
-                else store_and_reload(buf1, sc1, c + 1, 0, no);
+                if (c + 3 < nchunks) store_and_reload(buf1, sc1, c + 1, c + 3, yes, yes);
+                else store_and_reload(buf1, sc1, c + 1, 0, no, yes);
+            } else if constexpr (QS) {
+                __syncthreads();
             }
             __syncthreads();
             if (c + 1 < nchunks) {
-                if (c + 2 < nchunks) store_and_reload(buf0, sc0, c + 2, 0, no);
+                if (c + 2 < nchunks) store_and_reload(buf0, sc0, c + 2, 0, no, yes);
+                else if constexpr (QS) __syncthreads();
                 __syncthreads();
             }
         }
@@ -596,7 +657,8 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
             constexpr int op = decltype(opc)::value;
             if constexpr (op < OP_T) {  // rows of k (A of K S0) or of q (B of S0^T q^T): token tile, 32-key slab
                 constexpr int jj = op < OP_Q ? op : op - OP_Q, sl = SCH::s_slab(jj), tt = SCH::s_tile(jj);
-                return *reinterpret_cast<const bf16x8*>(st + (op < OP_Q ? K_OFF : Q_OFF) + (16 * tt + j16) * QLD + (32 * sl + 8 * g) * 2);
+                const uint8_t* rows = op < OP_Q ? st + K_OFF : QS ? qstage : st + Q_OFF;
+                return *reinterpret_cast<const bf16x8*>(rows + (16 * tt + j16) * QLD + (32 * sl + 8 * g) * 2);
             } else if constexpr (op >= OP_K && op < OP_P) {
                 // k^T: row j of key tile t is key 32 (t / 2) + 8 (j / 4) + 4 (t % 2) + j % 4; tokens 32 s + 4 g + 0..3 and
                 // 32 s + 16 + 4 g + 0..3.  Two transposing loads; lane (4 r' + q) supplies keys base + 8 q + 0..3 of token row r'.
@@ -691,6 +753,13 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
                     egc = lds_eg(stn);
 #pragma unroll
                     for (int it = 0; it < 4; it++) qsc[it] = lds_qs(stn, it);
+                }
+                if constexpr (QS && op == OP_T) {
+                    // Barrier Q.  The MFMA before this point took the last fragment of q, and LDS reads return in order:
+                    // no read of the q buffer is outstanding, so the barrier needs no wait for the reads still in flight.
+                    static_assert(OP_T < OP_BAR && OP_Q >= LA, "barrier Q comes first and the prefetch across the chunk barrier holds no q");
+                    __builtin_amdgcn_s_barrier();
+                    __builtin_amdgcn_sched_barrier(0);
                 }
                 if constexpr (op >= OP_BAR) fnext[op >= OP_BAR ? op - OP_BAR : 0] = lds_frag(stn, std::integral_constant<int, (op >= OP_BAR ? op - OP_BAR : 0)>{});
                 static_for<0, SCH::N_VS>([&](auto ic) {
@@ -1029,6 +1098,10 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     while (nw < 4 && vtiles % (2 * nw) == 0 && chains * (vtiles / nw) > (int64_t)num_cus) nw *= 2;
     const bool save = p.save_state != nullptr || p.save_vnew != nullptr;
     if (save && nw == 2) nw = 1;  // the saving variant exists for 1 and 4 slices per workgroup
+    if constexpr (K > 128) {  // K = 256 has the half-slice scan only
+        if (save || p.records_given) return GDN_ERR_UNSUPPORTED;
+        nw = 1;
+    }
     // a slice with a CU to itself is scanned by two waves of 16 columns each; the records are laid out for them
     const bool half = nw == 1 && !save && !p.records_given;
     p.rec16 = half ? 1 : 0;
@@ -1039,6 +1112,10 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     if (events != nullptr) (void)hipEventRecord(events[2], stream);
     p.scan_groups = vtiles / nw;
     const dim3 grid((unsigned)(chains8 * p.scan_groups));
+    if constexpr (K > 128) {
+        hipLaunchKernelGGL((chunk_scan32_kernel<K, 1, false, false, true>), grid, dim3(scan_waves(1, true) * WAVE), 0, stream, p);
+        return (int)hipGetLastError();
+    } else {
     if (save) {
         if (nw == 4) hipLaunchKernelGGL((chunk_scan32_kernel<K, 4, false, true>), grid, dim3(scan_waves(4) * WAVE), 0, stream, p);
         else hipLaunchKernelGGL((chunk_scan32_kernel<K, 1, false, true>), grid, dim3(scan_waves(1) * WAVE), 0, stream, p);
@@ -1050,11 +1127,13 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     else if (half) hipLaunchKernelGGL((chunk_scan32_kernel<K, 1, false, false, true>), grid, dim3(scan_waves(1, true) * WAVE), 0, stream, p);
     else hipLaunchKernelGGL((chunk_scan32_kernel<K, 1>), grid, dim3(scan_waves(1) * WAVE), 0, stream, p);
     return (int)hipGetLastError();
+    }
 }
 
 int launch_chunk32(ChunkParams& p, int K, hipStream_t stream, hipEvent_t* events, int num_cus) {
     if (K == 64) return launch32<64>(p, stream, events, num_cus);
     if (K == 128) return launch32<128>(p, stream, events, num_cus);
+    if (K == 256) return launch32<256>(p, stream, events, num_cus);
     return GDN_ERR_UNSUPPORTED;
 }
 

@@ -32,9 +32,9 @@ struct ChunkParams {
     int beta_dtype;
     int l2norm;
     float scale;
-    uint32_t rec_bytes, off_qs, off_kt, off_ks, off_cs, off_p, off_u, off_eg;
+    uint32_t rec_bytes, off_qs, off_ks, off_cs, off_p, off_eg;
     int scan_groups;  // workgroups per (sequence, head) in the scan kernel
-    // training support (scan of the 32x32x16 kernels only): when set, the scan also writes the fp32 state every
+    // training support (K <= 128): when set, the scan also writes the fp32 state every
     // chunk starts from, [N * H][save_nc][K][V], and V~ of every chunk, [N * H][save_nc][64][V]
     float* save_state;
     float* save_vnew;
@@ -48,36 +48,22 @@ struct ChunkParams {
 };
 
 struct RecordLayout {
-    uint32_t off_wn, off_qs, off_kt, off_ks, off_cs, off_p, off_u, off_eg, bytes;
+    uint32_t off_p, off_qs, off_ks, off_cs, off_eg, bytes;
 };
 
-// Record of one (head, chunk).
-//   K = 256 (16x16x32 kernels): Wn (-W), Qs, Kt, P (8 fragments) as operand fragments, U as accumulator
-//   fragments, e^{gamma_C}.
-//   K <= 128 (32x32x16 kernels): the 6 non-zero fragments of T diag(beta) (T = (I + A)^-1) at 0, the 6 non-zero
-//   fragments of P, then three vectors of 64 fp32 row scales - of q at off_qs (e^{gamma} scale / |q|), of k for the
-//   state update at off_ks (e^{gamma_C - gamma} / |k|), of k S0 at off_cs (e^{gamma} / |k|) - and e^{gamma_C}.
-//   q, k and v themselves are read from the caller's tensors by the scan, which forms
-//   V~ = T diag(beta) (V - diag(cs) K S0) itself: the record does not depend on V.
+// Record of one (head, chunk), the same for every K and V: the 6 non-zero fragments of T diag(beta) (T = (I + A)^-1)
+// at 0, the 6 non-zero fragments of P, then three vectors of 64 fp32 row scales - of q at off_qs
+// (e^{gamma} scale / |q|), of k for the state update at off_ks (e^{gamma_C - gamma} / |k|), of k S0 at off_cs
+// (e^{gamma} / |k|) - and e^{gamma_C}.  q, k and v themselves are read from the caller's tensors by the scan, which
+// forms V~ = T diag(beta) (V - diag(cs) K S0) itself: the record depends neither on V nor on the key dim.
 inline RecordLayout record_layout(int K, int V) {
+    (void)K, (void)V;
     RecordLayout r;
-    const uint32_t kfrag = (uint32_t)(C / 16) * (K / 32) * FRAG_BYTES;  // [C x K] or [K x C] bf16
-    r.off_wn = 0;
-    if (K > 128) {
-        r.off_qs = kfrag;
-        r.off_kt = 2 * kfrag;
-        r.off_p = 3 * kfrag;
-        r.off_u = r.off_p + (C / 16) * (C / 32) * FRAG_BYTES;
-        r.off_eg = r.off_u + (uint32_t)C * V * 2;
-        r.off_ks = 0, r.off_cs = 0;  // unused
-    } else {
-        r.off_kt = 0, r.off_u = 0;  // unused
-        r.off_p = 6 * FRAG_BYTES;
-        r.off_qs = r.off_p + 6 * FRAG_BYTES;
-        r.off_ks = r.off_qs + C * 4;
-        r.off_cs = r.off_ks + C * 4;
-        r.off_eg = r.off_cs + C * 4;
-    }
+    r.off_p = 6 * FRAG_BYTES;
+    r.off_qs = r.off_p + 6 * FRAG_BYTES;
+    r.off_ks = r.off_qs + C * 4;
+    r.off_cs = r.off_ks + C * 4;
+    r.off_eg = r.off_cs + C * 4;
     r.bytes = (r.off_eg + 4 + 255u) & ~255u;
     return r;
 }

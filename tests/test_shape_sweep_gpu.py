@@ -18,12 +18,12 @@ pytestmark = pytest.mark.gpu
 BF16 = torch.bfloat16
 
 
-def _cases():
-    rng = random.Random(20240611)
+def _cases(seed=20240611, first=0, count=36, key_dims=(64, 128, 128), value_dims=(32, 64, 96, 128, 128, 256)):
+    rng = random.Random(seed)
     cases = []
-    for i in range(36):
-        K = rng.choice([64, 128, 128])
-        V = rng.choice([32, 64, 96, 128, 128, 256])
+    for i in range(first, first + count):
+        K = rng.choice(key_dims)
+        V = rng.choice(value_dims)
         kind = rng.choice(["batch", "batch", "packed", "padded"])
         H = rng.choice([1, 2, 3, 4, 8, 16])
         if i % 6 == 5:  # many chains: 2 or 4 slices per workgroup
@@ -40,7 +40,11 @@ def _cases():
     return cases
 
 
-@pytest.mark.parametrize("case", _cases(), ids=lambda c: f"{c['i']}-{c['kind']}-B{c['B']}T{c['T']}H{c['H']}K{c['K']}V{c['V']}")
+# the second batch: K = 256 (half-slice waves with a single buffer for the rows of q), V up to 512
+ALL_CASES = _cases() + _cases(seed=20240612, first=36, count=16, key_dims=(256,), value_dims=(32, 64, 128, 256, 512))
+
+
+@pytest.mark.parametrize("case", ALL_CASES, ids=lambda c: f"{c['i']}-{c['kind']}-B{c['B']}T{c['T']}H{c['H']}K{c['K']}V{c['V']}")
 def test_forward_parity(case):
     c = case
     gen = torch.Generator("cpu").manual_seed(1000 + c["i"])
