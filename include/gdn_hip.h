@@ -140,7 +140,7 @@ int gdn_recurrent_fwd(const gdn_args *args, void *stream);
  * Training support.  The reference differentiates through chunk_gated_delta_rule (chunk mode is asserted
  * while training, gated_deltanet/module.py:194-209); a backward pass needs the state every chunk starts
  * from and the chunk's V~ (the values written into the state), which gdn_chunk_fwd does not keep.
- * gdn_chunk_fwd_saving is gdn_chunk_fwd (K <= 128) with a scan that also writes them, fp32:
+ * gdn_chunk_fwd_saving is gdn_chunk_fwd with a scan that also writes them, fp32:
  *     states [N * H][chunks_per_chain][K][V]     chain n * H + h, chunk c of its sequence
  *     v_new  [N * H][chunks_per_chain][64][V]    rows past the end of a sequence are not meaningful
  * Either may be NULL.  Only chunks c with c % save_every == 0 are saved (save_every <= 0 means 1), as entry
@@ -148,8 +148,10 @@ int gdn_recurrent_fwd(const gdn_args *args, void *stream);
  * [0, chunks_per_chain) are computed but not saved.
  * With records_given != 0 the prepare kernel is skipped: args->workspace then holds the chunk records
  * themselves, [H][B * ceil(T / 64)] records in the layout prepare writes (fixed-length batches only;
- * g, beta and the l2norm flag are not used, the records carry every scale).  The backward pass of this
- * package runs its reverse sweep over the chunks that way.
+ * g, beta and the l2norm flag are not used, the records carry every scale).  The twelve operand fragments
+ * of a record are then expected in the lane order of the 32x32x16 MFMA for K <= 128 and of the 16x16x32
+ * MFMA for K = 256 (the scan that runs on them).  The backward pass of this package runs its reverse sweep
+ * over the chunks that way.
  */
 typedef struct gdn_chunk_saves {
     float *states;

@@ -9,11 +9,11 @@ Three ways through, same formulas:
 * bf16, K = 128, V = 128 or 256 (whole rows, packed or left-padded batches): five kernel launches
   (``_backward_on_kernels``) - ``gdn_chunk_bwd_prepare``, ``gdn_chunk_fwd_saving`` for the forward sweep and
   again over the mirror problem for the reverse sweep, ``gdn_chunk_bwd_local``;
-* other bf16 shapes with K <= 128: the two sweeps over the chunks of a chain on the scan kernel
+* other bf16 shapes: the two sweeps over the chunks of a chain on the scan kernel
   (``gdn_chunk_fwd_saving``: the forward's scan in a variant that also writes the chunk states and V~),
   everything chunk-local as batched library GEMMs (fp32, ``torch.bmm``) and elementwise torch operations on
   sequences padded to whole chunks;
-* fp32 inputs, K = 256, CPU tensors: the sweeps as loops of batched GEMMs as well.
+* fp32 inputs, CPU tensors: the sweeps as loops of batched GEMMs as well.
 
 The reverse sweep is the same recurrence as the forward one on other data, which is how it gets onto
 that kernel: with the tokens of a chain in reverse order (a transposed lower-triangular matrix is
@@ -169,24 +169,37 @@ def _sweeps_as_gemm_loops(S_init, dS_init, egl, Kd, Qe, Kb, Tm, Vb, P, doc):
 _FRAGMENT_INDEX = {}
 
 
-def _fragment_index(device):
+def _fragment_index(device, half_slices=False):
     """Where the entries of a lower-triangular 64 x 64 matrix sit in its six MFMA operand fragments of a chunk
-    record (the layout the prepare kernel writes for T diag(beta) and for P): fragment f < 2 covers rows
-    0..31 and columns 16 f .. 16 f + 15, fragment f >= 2 rows 32..63 and columns 16 (f - 2) ..; lane
-    l = l32 + 32 h holds, of row 32 (f >= 2) + l32, the columns 16 s + 4 h + 0..3 and 16 s + 8 + 4 h + 0..3."""
-    if device not in _FRAGMENT_INDEX:
+    record (the layouts the prepare kernel writes for T diag(beta) and for P).
+
+    For the 32x32x16 MFMA (K <= 128): fragment f < 2 covers rows 0..31 and columns 16 f .. 16 f + 15, fragment
+    f >= 2 rows 32..63 and columns 16 (f - 2) ..; lane l = l32 + 32 h holds, of row 32 (f >= 2) + l32, the columns
+    16 s + 4 h + 0..3 and 16 s + 8 + 4 h + 0..3.
+
+    For the 16x16x32 MFMA of the half-slice scan (``half_slices``, K = 256): the fragments are the non-zero blocks
+    of 16 rows x 32 columns - row tiles 0, 1 (column slab 0), then row tiles 2 and 3 with slabs 0 and 1 each; lane
+    l = l16 + 16 g holds, of row 16 tile + l16, the columns 32 s + 4 g + 0..3 and 32 s + 16 + 4 g + 0..3."""
+    key = (device, half_slices)
+    if key not in _FRAGMENT_INDEX:
         f = torch.arange(6).view(6, 1, 1)
         lane = torch.arange(64).view(1, 64, 1)
         e = torch.arange(8).view(1, 1, 8)
-        tile = (f >= 2).long()
-        slab = torch.where(f < 2, f, f - 2)
-        rows = (32 * tile + lane % 32).expand(6, 64, 8)
-        cols = 16 * slab + 4 * (lane // 32) + torch.where(e < 4, e, e + 4)
-        _FRAGMENT_INDEX[device] = (rows.to(device), cols.to(device))
-    return _FRAGMENT_INDEX[device]
+        if half_slices:
+            tile = torch.where(f < 2, f, 2 + (f - 2) // 2)
+            slab = torch.where(f < 2, torch.zeros_like(f), f % 2)
+            rows = (16 * tile + lane % 16).expand(6, 64, 8)
+            cols = 32 * slab + 4 * (lane // 16) + torch.where(e < 4, e, e + 12)
+        else:
+            tile = (f >= 2).long()
+            slab = torch.where(f < 2, f, f - 2)
+            rows = (32 * tile + lane % 32).expand(6, 64, 8)
+            cols = 16 * slab + 4 * (lane // 32) + torch.where(e < 4, e, e + 4)
+        _FRAGMENT_INDEX[key] = (rows.to(device), cols.to(device))
+    return _FRAGMENT_INDEX[key]
 
 
-RECORD_BYTES = 13312  # record of the 32x32x16 kernels (K <= 128): 12 fragments, 3 x 64 row scales, e^{gamma_C}
+RECORD_BYTES = 13312  # a chunk record: 12 fragments, 3 x 64 row scales, e^{gamma_C}
 
 
 def _mirror_problem(N, H, kraw, qraw, doc, Tm, P, egl, cs_a, ks_a, ks_b, aligned_inputs=None):
@@ -219,7 +232,7 @@ def _mirror_problem(N, H, kraw, qraw, doc, Tm, P, egl, cs_a, ks_a, ks_b, aligned
         v_m[:, :, 1] = do
         v_m = v_m.view(N, 2 * NC * CHUNK, H, V)
 
-    rows, cols = _fragment_index(dev)
+    rows, cols = _fragment_index(dev, half_slices=K > 128)  # the scan that runs on K = 256 is the half-slice one
     eye = torch.eye(CHUNK, device=dev)
     # T^T with rows and columns reversed is lower-triangular again: entry (i', j') is T[63 - j', 63 - i']
     Tmir = Tm.transpose(-1, -2).flip(-1, -2)
@@ -409,7 +422,7 @@ def gated_delta_rule_backward(
     Tm = torch.linalg.solve_triangular(eye + A, eye.expand_as(A), upper=False)
     P = E * (qs @ kT)
 
-    on_kernel = q.is_cuda and q.dtype == torch.bfloat16 and K <= 128 and V % 32 == 0
+    on_kernel = q.is_cuda and q.dtype == torch.bfloat16 and K in (64, 128, 256) and V % 32 == 0
     if on_kernel:
         # the scan reads the raw rows of k and q; their norms and e^{gamma} go into the row scales
         S0, Vn, dS1, Y, dS = _sweeps_on_scan_kernel(

@@ -148,7 +148,7 @@ int gdn_chunk_fwd_saving(const gdn_args* a, const gdn_chunk_saves* saves, void* 
     if (saves == nullptr) return GDN_ERR_NULL;
     const int rc = validate_common(a);
     if (rc != GDN_OK) return rc;
-    if (!gdn::chunk_shape_supported(*a) || a->K > 128) return GDN_ERR_UNSUPPORTED;
+    if (!gdn::chunk_shape_supported(*a)) return GDN_ERR_UNSUPPORTED;
     if (saves->states == nullptr && saves->v_new == nullptr) return GDN_ERR_NULL;
     if ((saves->states && !aligned(saves->states, 16)) || (saves->v_new && !aligned(saves->v_new, 16))) return GDN_ERR_ALIGN;
     if (saves->chunks_per_chain <= 0) return GDN_ERR_SHAPE;  // chunks beyond it are computed but not saved

@@ -340,7 +340,7 @@ struct Scan16Schedule : Scan16Rules<K> {
 // hold the fragments of T diag(beta) and P in the layout of that instruction (ChunkParams::rec16).
 template <int K, int NW, bool NT = false, bool SAVE = false, bool HALF = false>
 __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kernel(const ChunkParams p) {
-    static_assert(!HALF || (NW == 1 && !SAVE), "the half-slice scan has one slice per workgroup and saves nothing");
+    static_assert(!HALF || NW == 1, "the half-slice scan has one slice per workgroup");
     // K = 256: two stage halves with the rows of q and k do not fit the LDS.  The rows of q, which a chunk needs for
     // one group of MFMAs only, then get a single buffer and a second workgroup barrier per chunk ("barrier Q"), passed
     // by a compute wave once it holds the last fragment of q: the loaders write the next chunk's rows of q between
@@ -706,6 +706,21 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
         for (int c = 0; c < nchunks; c++) {
             const uint8_t* st = stage[c & 1];
             const uint8_t* stn = stage[(c + 1) & 1];
+            if constexpr (SAVE) {
+                // the state this chunk starts from, for the backward pass (one wave-uniform base plus one per-lane
+                // byte offset, as in the whole-slice scan)
+                if (p.save_state != nullptr && c % p.save_every == 0 && c / p.save_every < p.save_nc) {
+                    const int entry = p.save_reverse ? p.save_nc - 1 - c / p.save_every : c / p.save_every;
+                    char* base = reinterpret_cast<char*>(p.save_state + ((int64_t)chain * p.save_nc + entry) * K * p.V);
+                    const uint32_t lane_off = (uint32_t)((8 * g) * p.V + c0 + j16) * 4u;
+                    const uint32_t row_bytes = (uint32_t)p.V * 4u;
+#pragma unroll
+                    for (int t = 0; t < KT; t++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            *reinterpret_cast<float*>(base + (size_t)((32 * (t / 2) + 4 * (t % 2) + r) * row_bytes) + lane_off) = S[t][r];
+                }
+            }
             bf16x8 fr[NOPS];
 #pragma unroll
             for (int i = 0; i < LA; i++) fr[i] = fnext[i];
@@ -797,6 +812,20 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
                 }
                 __builtin_amdgcn_sched_barrier(0);
             });
+            if constexpr (SAVE) {
+                // V~ of this chunk: tile tt, register r holds token 16 tt + 4 g + r of this lane's column
+                if (p.save_vnew != nullptr && c % p.save_every == 0 && c / p.save_every < p.save_nc) {
+                    const int entry = p.save_reverse ? p.save_nc - 1 - c / p.save_every : c / p.save_every;
+                    char* base = reinterpret_cast<char*>(p.save_vnew + ((int64_t)chain * p.save_nc + entry) * C * p.V);
+                    const uint32_t lane_off = (uint32_t)((4 * g) * p.V + c0 + j16) * 4u;
+                    const uint32_t row_bytes = (uint32_t)p.V * 4u;
+#pragma unroll
+                    for (int tt = 0; tt < 4; tt++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            *reinterpret_cast<float*>(base + (size_t)((16 * tt + r) * row_bytes) + lane_off) = vt[tt][r];
+                }
+            }
         }
         if (nchunks > 0) {
 #pragma unroll
@@ -1098,12 +1127,9 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     while (nw < 4 && vtiles % (2 * nw) == 0 && chains * (vtiles / nw) > (int64_t)num_cus) nw *= 2;
     const bool save = p.save_state != nullptr || p.save_vnew != nullptr;
     if (save && nw == 2) nw = 1;  // the saving variant exists for 1 and 4 slices per workgroup
-    if constexpr (K > 128) {  // K = 256 has the half-slice scan only
-        if (save || p.records_given) return GDN_ERR_UNSUPPORTED;
-        nw = 1;
-    }
+    if constexpr (K > 128) nw = 1;  // K = 256 has the half-slice scan only, also as the saving variant and on given records
     // a slice with a CU to itself is scanned by two waves of 16 columns each; the records are laid out for them
-    const bool half = nw == 1 && !save && !p.records_given;
+    const bool half = K > 128 || (nw == 1 && !save && !p.records_given);
     p.rec16 = half ? 1 : 0;
     if (!p.records_given) {
         hipLaunchKernelGGL((chunk_prepare32_kernel<K>), dim3(grid_prep), dim3(PREP_THREADS), 0, stream, p);
@@ -1113,7 +1139,8 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     p.scan_groups = vtiles / nw;
     const dim3 grid((unsigned)(chains8 * p.scan_groups));
     if constexpr (K > 128) {
-        hipLaunchKernelGGL((chunk_scan32_kernel<K, 1, false, false, true>), grid, dim3(scan_waves(1, true) * WAVE), 0, stream, p);
+        if (save) hipLaunchKernelGGL((chunk_scan32_kernel<K, 1, false, true, true>), grid, dim3(scan_waves(1, true) * WAVE), 0, stream, p);
+        else hipLaunchKernelGGL((chunk_scan32_kernel<K, 1, false, false, true>), grid, dim3(scan_waves(1, true) * WAVE), 0, stream, p);
         return (int)hipGetLastError();
     } else {
     if (save) {

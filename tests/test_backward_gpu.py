@@ -109,6 +109,20 @@ def test_chunk_bf16_k64_and_wide_v():
     _run_case(lm_engine_amd.chunk_gated_delta_rule, inp, torch.bfloat16)
 
 
+@pytest.mark.parametrize("T, V", [(130, 64), (192, 512)])
+def test_chunk_bf16_k256(T, V):
+    # K = 256 (the head shape of the reference's shipped configurations is K = 256, V = 512): both sweeps on the
+    # half-slice scan in its saving variant, the reverse one on records written in that scan's fragment layout
+    inp = random_inputs(B=2, T=T, H=2, K=256, V=V, dtype=torch.bfloat16, seed=50 + V, normalize=False)
+    _run_case(lm_engine_amd.chunk_gated_delta_rule, inp, torch.bfloat16)
+
+
+def test_chunk_bf16_k256_packed():
+    cu = torch.tensor([0, 70, 71, 300], dtype=torch.int32)
+    inp = random_inputs(B=1, T=300, H=2, K=256, V=128, dtype=torch.bfloat16, seed=57, normalize=False, N=3)
+    _run_case(lm_engine_amd.chunk_gated_delta_rule, inp, torch.bfloat16, cu=cu)
+
+
 @pytest.mark.parametrize("V", [128, 256])
 def test_chunk_bf16_whole_chunks_all_on_kernels(V):
     # whole chunks, K = 128: prepare, both sweeps and the chunk-local gradients are kernel launches
@@ -160,12 +174,13 @@ def test_ungated_without_beta():
     _assert_grads([q.grad, k.grad, v.grad], want[:3], torch.bfloat16)
 
 
-def test_saved_chunk_states_are_the_states_of_the_prefixes():
+@pytest.mark.parametrize("K, V", [(128, 128), (256, 64)])
+def test_saved_chunk_states_are_the_states_of_the_prefixes(K, V):
     """``gdn_chunk_fwd_saving``: the state saved for chunk c is the final state of the first 64 c tokens."""
     from lm_engine_amd import ops
     from oracle.gdn_oracle import recurrent_gated_delta_rule_ref
 
-    B, T, H, K, V = 2, 200, 2, 128, 128
+    B, T, H = 2, 200, 2
     inp = random_inputs(B=B, T=T, H=H, K=K, V=V, dtype=torch.bfloat16, seed=13)
     dev = {n: (None if x is None else x.cuda()) for n, x in inp.items()}
     NC = 4
