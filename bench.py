@@ -19,7 +19,8 @@ inputs already resident in HBM.  Prints ONE JSON line:
   cpu_baseline the naive token-by-token torch restatement of the operator (oracle/), timed on
                this host's cores on a bounded prefix of the same workload
   forward_other the same forward with prepare and scan as two kernels (the headline configuration runs them as one
-               launch by default), and on configurations 2 (packed sequences) and 4 (long context, V=256; both ways)
+               launch by default), on configurations 2 (packed sequences) and 4 (long context, V=256; both ways), and
+               on the head shape of the reference's shipped configurations (B=8, T=4096, H=2, K=256, V=512)
 """
 
 from __future__ import annotations
@@ -29,6 +30,7 @@ import json
 import os
 import sys
 import time
+from dataclasses import replace
 
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
@@ -534,6 +536,9 @@ def main():
             if index != args.workload:
                 other.append(chunk_forward_leg(get_workload(index), args.steps, args.warmup, two_kernels=False))
         other.append(chunk_forward_leg(get_workload(4), args.steps, args.warmup, two_kernels=True))
+        # the head shape of the reference's shipped configurations (k_head_dim 256, v_head_dim 512, 2 heads, micro-batch 8)
+        shipped = get_workload(1, B=8, H=2, K=256, V=512)
+        other.append(chunk_forward_leg(replace(shipped, name="shipped_head_shape_k256_v512_bf16"), args.steps, args.warmup, two_kernels=False))
     baseline = None if args.no_cpu_baseline else cpu_baseline(w, inp, args.cpu_seconds)
     if args.calibrate_copy:
         calibrate_copy()

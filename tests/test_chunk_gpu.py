@@ -276,3 +276,23 @@ def test_config4_long_context_full_size():
     torch.cuda.synchronize()
     assert torch.equal(torch.cat([o1, o2], dim=1), o), "split run differs from the full run"
     assert torch.equal(h2, ht)
+
+
+def test_shipped_head_shape_full_size():
+    # the head shape of the reference's shipped configurations (k_head_dim 256, v_head_dim 512, 2 heads, micro-batch 8,
+    # T = 4096; configs/research/m2rnn/400m-normal/gated-deltanet.yml:60-73): the half-slice scan with a single buffer
+    # for the rows of q, 16 chains x 16 slices.  Inputs drawn like configuration 1's.
+    inp = make_inputs(get_workload(1, B=8, H=2, K=256, V=512))
+    assert tuple(inp["q"].shape) == (8, 4096, 2, 256) and tuple(inp["v"].shape) == (8, 4096, 2, 512)
+    o, ht = _check(inp, "K=256, V=512, B=8, T=4096, H=2")
+    # split at a chunk boundary with the state carried over == one run, bitwise
+    gpu = _to_gpu(inp)
+    cut = 64 * 23
+    first = {n: (x[:, :cut] if n in ("q", "k", "v", "g", "beta") else x) for n, x in gpu.items()}
+    o1, h1 = lm_engine_amd.chunk_gated_delta_rule(**first, output_final_state=True)
+    second = {n: (x[:, cut:] if n in ("q", "k", "v", "g", "beta") else x) for n, x in gpu.items()}
+    second["initial_state"] = h1
+    o2, h2 = lm_engine_amd.chunk_gated_delta_rule(**second, output_final_state=True)
+    torch.cuda.synchronize()
+    assert torch.equal(torch.cat([o1, o2], dim=1), o), "split run differs from the full run"
+    assert torch.equal(h2, ht)
