@@ -33,7 +33,8 @@ static int chunk_slots(const gdn_args& a) {
     return packed ? a.T / C + a.N : a.B * nt;
 }
 
-static uint64_t chunk_off_bytes(const gdn_args& a) { return (((uint64_t)a.N + 1) * 4 + 255u) & ~(uint64_t)255u; }
+// chunk offsets [N + 1] and the scan order of the sequences [N] (packed batches)
+static uint64_t chunk_off_bytes(const gdn_args& a) { return ((2 * (uint64_t)a.N + 1) * 4 + 255u) & ~(uint64_t)255u; }
 
 bool chunk_shape_supported(const gdn_args& a) {
     if (a.dtype != GDN_BF16) return false;
@@ -62,8 +63,14 @@ uint64_t chunk_workspace_bytes(const gdn_args& a) {
 // Lengths are taken through packed_bounds, and the running total is capped at the number of record slots
 // the workspace holds (`slots`): whatever cu_seqlens contains, no chunk gets a slot outside the workspace
 // (sequences past the cap get none; a well-formed prefix never reaches it).
+//
+// order[r] = the sequence with the r-th most chunks (ties by index): the scan starts its chains in that order, so that the
+// longest sequence of a ragged batch, which bounds the launch, is not the one that starts last.  Ranked by counting
+// (N^2 / 256 comparisons per thread) for up to ORDER_MAX sequences; larger batches, whose many sequences even out by
+// themselves, keep the order of the batch.
+constexpr int ORDER_MAX = 1024;
 __global__ __launch_bounds__(256) void chunk_offsets_kernel(const int32_t* __restrict__ cu, int32_t* __restrict__ off,
-                                                            int N, int total, int slots) {
+                                                            int32_t* __restrict__ order, int N, int total, int slots) {
     __shared__ int s_part[256];
     const int tid = threadIdx.x;
     const int per = (N + 255) / 256;
@@ -91,6 +98,19 @@ __global__ __launch_bounds__(256) void chunk_offsets_kernel(const int32_t* __res
     for (int n = begin; n < end; n++) {
         off[n] = run;
         run = min(run + chunks_of(n), slots);
+    }
+    if (N > ORDER_MAX) {
+        for (int n = tid; n < N; n += 256) order[n] = n;
+        return;
+    }
+    __shared__ int s_cnt[ORDER_MAX];
+    for (int n = tid; n < N; n += 256) s_cnt[n] = chunks_of(n);
+    __syncthreads();
+    for (int n = tid; n < N; n += 256) {
+        const int mine = s_cnt[n];
+        int rank = 0;
+        for (int m = 0; m < N; m++) rank += (s_cnt[m] > mine || (s_cnt[m] == mine && m < n)) ? 1 : 0;
+        order[rank] = n;  // the ranks are a permutation of 0 .. N - 1
     }
 }
 
@@ -126,6 +146,7 @@ int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events, 
     p.cu_seqlens = left_padded ? nullptr : a.cu_seqlens;
     p.pad_lens = left_padded ? a.cu_seqlens : nullptr;
     p.chunk_off = static_cast<int32_t*>(a.workspace);
+    p.seq_order = p.chunk_off + a.N + 1;
     p.ready = reinterpret_cast<int32_t*>(static_cast<uint8_t*>(a.workspace) + chunk_off_bytes(a));
     p.rec = static_cast<uint8_t*>(a.workspace) + chunk_off_bytes(a) + chunk_flag_bytes(a);
     p.save_state = nullptr, p.save_vnew = nullptr, p.save_nc = 0, p.records_given = 0, p.save_every = 1, p.save_reverse = 0;
@@ -133,7 +154,7 @@ int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events, 
         p.save_state = saves->states, p.save_vnew = saves->v_new, p.save_nc = saves->chunks_per_chain;
         p.save_every = saves->save_every > 0 ? saves->save_every : 1, p.save_reverse = saves->save_reverse ? 1 : 0;
         p.records_given = saves->records_given;
-        if (p.records_given) p.chunk_off = nullptr, p.ready = nullptr, p.rec = static_cast<uint8_t*>(a.workspace);
+        if (p.records_given) p.chunk_off = nullptr, p.seq_order = nullptr, p.ready = nullptr, p.rec = static_cast<uint8_t*>(a.workspace);
     }
     p.q_stride_b = a.q_stride_b, p.q_stride_t = a.q_stride_t, p.q_stride_h = a.q_stride_h;
     p.k_stride_b = a.k_stride_b, p.k_stride_t = a.k_stride_t, p.k_stride_h = a.k_stride_h;
@@ -155,7 +176,7 @@ int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events, 
     };
     mark(0);
     if (p.cu_seqlens != nullptr) {
-        hipLaunchKernelGGL(chunk_offsets_kernel, dim3(1), dim3(256), 0, stream, p.cu_seqlens, p.chunk_off, p.N, p.T, p.TC);
+        hipLaunchKernelGGL(chunk_offsets_kernel, dim3(1), dim3(256), 0, stream, p.cu_seqlens, p.chunk_off, p.seq_order, p.N, p.T, p.TC);
         if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
     }
     mark(1);

@@ -390,11 +390,24 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
     const int id = blockIdx.x;
     const int xcd = id % 8, rest = id / 8;
     const int vgroup = rest % p.scan_groups;
-    // XCD x takes the chains x * per_xcd .. : consecutive chains are different heads
     const int per_xcd = (p.N * p.H + 7) / 8;
-    const int chain = xcd * per_xcd + rest / p.scan_groups;
-    if (rest / p.scan_groups >= per_xcd || chain >= p.N * p.H) return;  // whole workgroup
-    const int n = chain / p.H, h = chain % p.H;
+    int n, h;
+    if (p.cu_seqlens == nullptr) {
+        // XCD x takes the chains x * per_xcd .. : consecutive chains are different heads
+        const int chain = xcd * per_xcd + rest / p.scan_groups;
+        if (rest / p.scan_groups >= per_xcd || chain >= p.N * p.H) return;  // whole workgroup
+        n = chain / p.H, h = chain % p.H;
+    } else {
+        // Packed batches: the chains in the order (sequence by decreasing length, head) are dealt out eight at a time, one
+        // per XCD, and workgroups start in the order of their ids: the longest chains first.  The deal is rotated from
+        // one eight to the next, so that an XCD does not keep getting the same heads (rows of one head lie a whole
+        // token row apart and fall on few channels of its L2).
+        const int i = rest / p.scan_groups;
+        const int rank = 8 * i + ((xcd - i) % 8 + 8) % 8;
+        if (i >= per_xcd || rank >= p.N * p.H) return;  // whole workgroup
+        n = p.seq_order[rank / p.H], h = rank % p.H;
+    }
+    const int chain = n * p.H + h;
 
     int slot_begin, slot_end;
     int64_t b, seq_t0, seq_len;
@@ -1126,6 +1139,11 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     int nw = 1;
     while (nw < 4 && vtiles % (2 * nw) == 0 && chains * (vtiles / nw) > (int64_t)num_cus) nw *= 2;
     const bool save = p.save_state != nullptr || p.save_vnew != nullptr;
+    // Packed batches are ragged as a rule, and their chains start longest first (chunk_offsets_kernel): the launch then
+    // takes as long as the longest chain, which runs faster the fewer slices share its workgroup, while the workgroups
+    // that do not fit at first fill in behind the short chains.  So up to two workgroups per CU are accepted there.
+    // (Configuration 2, 11 sequences of 202 .. 6350 tokens, H = 16: 246 us with four slices per workgroup, 193 us with two.)
+    if (p.cu_seqlens != nullptr && !save && nw > 1 && chains * (vtiles / (nw / 2)) <= 2 * (int64_t)num_cus) nw /= 2;
     if (save && nw == 2) nw = 1;  // the saving variant exists for 1 and 4 slices per workgroup
     if constexpr (K > 128) nw = 1;  // K = 256 has the half-slice scan only, also as the saving variant and on given records
     // a slice with a CU to itself is scanned by two waves of 16 columns each; the records are laid out for them

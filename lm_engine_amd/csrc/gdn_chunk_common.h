@@ -21,6 +21,7 @@ struct ChunkParams {
     const int32_t* cu_seqlens;  // packed sequences (B == 1), else NULL
     const int32_t* pad_lens;    // left-padded batch: prefix sums of the valid lengths, else NULL
     int32_t* chunk_off;  // [N + 1] prefix of chunks per sequence (packed input only)
+    int32_t* seq_order;  // [N] the sequences by decreasing number of chunks (packed input only)
     uint8_t* rec;        // workspace records, [H][TC]
     int64_t q_stride_b, q_stride_t, q_stride_h;
     int64_t k_stride_b, k_stride_t, k_stride_h;

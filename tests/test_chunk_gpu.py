@@ -140,6 +140,21 @@ def test_varlen_packed_sequences_match_and_equal_separate_runs():
         assert torch.equal(ht[n : n + 1], h_n)
 
 
+@pytest.mark.parametrize("count, H, V", [(40, 8, 128), (1100, 1, 32)])
+def test_varlen_many_sequences_start_longest_first(count, H, V):
+    # The scan starts the chains of a packed batch by decreasing length (ranked on the device; batches of more than
+    # 1024 sequences keep their order): sequences of equal and of very different lengths, empty ones, more chains
+    # than CUs in the first case (two workgroups per CU are accepted for packed batches).
+    gen = torch.Generator().manual_seed(count)
+    lengths = torch.randint(0, 4, (count,), generator=gen).tolist()
+    for i in range(0, count, 7):
+        lengths[i] = int(torch.randint(60, 200, (1,), generator=gen))
+    lengths[count // 2] = 700
+    inp = random_inputs(B=1, T=sum(lengths), H=H, K=64, V=V, dtype=BF16, seed=78, N=count)
+    cu = torch.tensor([0] + lengths).cumsum(0).to(torch.int32)
+    _check(dict(inp, cu_seqlens=cu), f"varlen, {count} sequences")
+
+
 @pytest.mark.parametrize("K, V", [(128, 128), (64, 64), (256, 128)])
 def test_varlen_with_an_empty_sequence(K, V):
     # a sequence of length 0 has no chunk: its final state is its initial state, and its neighbours are untouched
