@@ -46,6 +46,12 @@ enum {
                                    batch, K <= 128, V a multiple of 64, N * H * V / 64 between 3/8 and 1/2 of the CUs: where
                                    it is the faster way; other shapes run as without the flag); results stay within the
                                    same parity gates but are not bit-identical to the two-kernel path */
+    GDN_FLAG_READY_FLAGS_CLEAR = 16, /* gdn_chunk_fwd: the caller keeps this workspace between calls and every byte of it was
+                                   zero before its first use.  The one-launch forward keeps one ready flag per record
+                                   in the workspace; it clears them itself before it starts (a small kernel of its own)
+                                   unless this flag promises that they are clear.  Every call that returns success
+                                   leaves them clear again, with or without the flag, so a workspace that is used for
+                                   nothing else, by calls of one shape on one stream, keeps the promise by itself. */
 };
 
 /*

@@ -139,6 +139,7 @@ int gdn_chunk_fwd_noalloc(const gdn_args* a, void* stream) {
     // Nothing in the workspace has to start at zero: the offsets kernel and prepare write every word the
     // scan reads.  The same array serves every call on this device.
     gdn_args b = *a;
+    b.flags &= ~GDN_FLAG_READY_FLAGS_CLEAR;  // where the flags lie in the array depends on the shape: records of another call may have been there
     b.workspace = ptr;
     b.workspace_bytes = (uint64_t)GDN_NOALLOC_SCRATCH_BYTES;
     return gdn::launch_chunk_fwd(b, static_cast<hipStream_t>(stream));

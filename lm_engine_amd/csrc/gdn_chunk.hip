@@ -170,6 +170,7 @@ int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events, 
     p.off_eg = r.off_eg;
     p.scan_groups = 1;
     p.fused = (a.flags & GDN_FLAG_FUSED_LAUNCH) ? 1 : 0;
+    p.ready_clear = (a.flags & GDN_FLAG_READY_FLAGS_CLEAR) ? 1 : 0;
 
     auto mark = [&](int i) {
         if (events != nullptr) (void)hipEventRecord(events[i], stream);

@@ -45,6 +45,7 @@ struct ChunkParams {
     int records_given;  // the records are already in place: prepare is not run
     int32_t* ready;     // [H][TC] one flag per record, for the launch that runs prepare and scan together
     int fused;          // that launch was asked for (GDN_FLAG_FUSED_LAUNCH)
+    int ready_clear;    // the caller vouches that the ready flags are zero (GDN_FLAG_READY_FLAGS_CLEAR)
     int rec16;          // the fragments of T diag(beta) and P are laid out for v_mfma_f32_16x16x32_bf16 (the half-slice scan)
 };
 

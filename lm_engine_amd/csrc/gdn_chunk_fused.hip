@@ -325,6 +325,21 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
         }
         __syncthreads();  // the hand-over of the last output tile
         if (nchunks > 0) flush(nchunks - 1);
+        if constexpr (WAIT) {
+            // Leave the flags of this chain clear for the next launch on this workspace.  A producer set a flag to 1; every
+            // scan workgroup of the chain (p.scan_groups of them) adds 1 once none of its waves polls any more (they all
+            // passed the barrier above), and the one that finds 1 + (p.scan_groups - 1) there is the last: it stores 0.
+            if (lw == 0) {
+                int32_t* const flags_of_chain = p.ready + (int64_t)h * p.TC + slot_begin;
+                for (int c0 = 0; c0 < nchunks; c0 += WAVE) {
+                    if (c0 + lane < nchunks) {
+                        int32_t* const flag = flags_of_chain + c0 + lane;
+                        const int32_t before = __hip_atomic_fetch_add(flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        if (before == p.scan_groups) __hip_atomic_store(flag, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                }
+            }
+        }
         return;
     }
 
@@ -649,9 +664,11 @@ static int launch_fused_k(ChunkParams& p, hipStream_t stream, int num_cus) {
     // Worth it only when the scan fills about half of the CUs: with fewer chains the two-kernel path's scan, one slice per
     // CU, is the faster one and prepare is short; with more, too few CUs are left for the producers.
     if (scan_wgs > (int64_t)num_cus / 2 || scan_wgs < (int64_t)num_cus * 3 / 8) return GDN_ERR_UNSUPPORTED;
-    const int64_t nflags = (int64_t)p.H * p.TC;
-    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((nflags + 255) / 256 < 64 ? (nflags + 255) / 256 : 64)), dim3(256), 0, stream, p.ready, nflags);
-    if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
+    if (!p.ready_clear) {  // the scan waits for flags the producers set: they must start at zero (and end there: scan_pair_body)
+        const int64_t nflags = (int64_t)p.H * p.TC;
+        hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((nflags + 255) / 256 < 64 ? (nflags + 255) / 256 : 64)), dim3(256), 0, stream, p.ready, nflags);
+        if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
+    }
     hipLaunchKernelGGL((chunk_fused_kernel<K, 2>), dim3((unsigned)(prep_wgs + scan_wgs)), dim3(PAIR_THREADS), 0, stream, p, prep_wgs);
     return (int)hipGetLastError();
 }

@@ -25,6 +25,7 @@ call raises.  Both are differentiable (``backward.py``).
 from __future__ import annotations
 
 import ctypes
+from collections import OrderedDict
 
 import torch
 
@@ -127,6 +128,33 @@ def _fill_args(q, k, v, g, beta, h0, ht, o, cu_seqlens, scale, l2norm, inplace, 
     return a
 
 
+# Workspaces of the chunked forward, kept between calls: one per (device, stream, shape), zero-filled when it is made.
+# The library then need not clear the ready flags of its one-launch mode before every call (it leaves them clear
+# itself, GDN_FLAG_READY_FLAGS_CLEAR), and a step no longer asks the allocator for tens of megabytes.  Calls on one
+# stream run in order, so they can share a workspace; another stream gets its own.  The least recently used entries
+# go when there are more than _WORKSPACE_LIMIT; release_workspaces() drops them all.
+_WORKSPACES: "OrderedDict[tuple, torch.Tensor]" = OrderedDict()
+_WORKSPACE_LIMIT = 8
+
+
+def release_workspaces() -> None:
+    """Frees the workspaces that ``chunk_gated_delta_rule`` keeps between calls."""
+    _WORKSPACES.clear()
+
+
+def _kept_workspace(device, stream_handle, dims, packed, nbytes):
+    key = (device.index, stream_handle, dims, packed, nbytes)
+    workspace = _WORKSPACES.get(key)
+    if workspace is None:
+        workspace = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+        _WORKSPACES[key] = workspace
+        while len(_WORKSPACES) > _WORKSPACE_LIMIT:
+            _WORKSPACES.popitem(last=False)
+    else:
+        _WORKSPACES.move_to_end(key)
+    return key, workspace
+
+
 def _run(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, l2norm, inplace_state,
          left_padded=False):
     _require_hip_path()
@@ -160,10 +188,19 @@ def _run(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_se
 
     with torch.cuda.device(q.device):
         if mode == "chunk":
-            nbytes = lib.gdn_workspace_bytes(ctypes.byref(args))
-            workspace = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=q.device)
+            nbytes = max(int(lib.gdn_workspace_bytes(ctypes.byref(args))), 256)
+            if torch.cuda.is_current_stream_capturing():
+                # memory allocated under graph capture belongs to the graph: nothing of it is kept
+                key, workspace = None, torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+            else:
+                key, workspace = _kept_workspace(q.device, stream.value, dims, cu_seqlens is not None, nbytes)
+                args.flags |= _lib.GDN_FLAG_READY_FLAGS_CLEAR
             args.workspace, args.workspace_bytes = workspace.data_ptr(), workspace.numel()
-            _lib.check_status(lib.gdn_chunk_fwd(ctypes.byref(args), stream), "gdn_chunk_fwd")
+            try:
+                _lib.check_status(lib.gdn_chunk_fwd(ctypes.byref(args), stream), "gdn_chunk_fwd")
+            except Exception:
+                _WORKSPACES.pop(key, None)  # a call that failed may have left flags set
+                raise
         else:
             _lib.check_status(lib.gdn_recurrent_fwd(ctypes.byref(args), stream), "gdn_recurrent_fwd")
     return o, ht
@@ -206,11 +243,17 @@ def chunk_forward_kernel_times(
     args = _fill_args(q, k, v, g, beta, h0, ht, o, cu_seqlens, scale, use_qk_l2norm_in_kernel, False, dims)
     times = (ctypes.c_float * _lib.GDN_CHUNK_KERNELS)()
     with torch.cuda.device(q.device):
-        workspace = torch.empty(max(int(lib.gdn_workspace_bytes(ctypes.byref(args))), 256), dtype=torch.uint8,
-                                device=q.device)  # fmt: skip
-        args.workspace, args.workspace_bytes = workspace.data_ptr(), workspace.numel()
+        # the same kept workspace, and the same promise about its flags, as the operator itself
         stream = ctypes.c_void_p(torch.cuda.current_stream(q.device).cuda_stream)
-        _lib.check_status(lib.gdn_chunk_fwd_profile(ctypes.byref(args), stream, times), "gdn_chunk_fwd_profile")
+        nbytes = max(int(lib.gdn_workspace_bytes(ctypes.byref(args))), 256)
+        key, workspace = _kept_workspace(q.device, stream.value, dims, cu_seqlens is not None, nbytes)
+        args.flags |= _lib.GDN_FLAG_READY_FLAGS_CLEAR
+        args.workspace, args.workspace_bytes = workspace.data_ptr(), workspace.numel()
+        try:
+            _lib.check_status(lib.gdn_chunk_fwd_profile(ctypes.byref(args), stream, times), "gdn_chunk_fwd_profile")
+        except Exception:
+            _WORKSPACES.pop(key, None)
+            raise
     return dict(zip(_lib.CHUNK_KERNEL_NAMES, (float(x) for x in times)))
 
 

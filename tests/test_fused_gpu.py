@@ -133,3 +133,70 @@ def test_close_to_the_two_kernel_path_and_fallback_is_unchanged():
         with enable_kernels(FUSED):
             b = lm_engine_amd.chunk_gated_delta_rule(**case, output_final_state=True, **extra)
         assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
+def test_ready_flags_are_left_clear_and_need_no_clearing_when_the_caller_says_so():
+    """GDN_FLAG_READY_FLAGS_CLEAR through the C ABI: a workspace that was zero before its first use serves calls in a
+    row without the clearing kernel; each gives the bits of a call on a fresh workspace without the flag, and the
+    flag region is all zero after every call, with and without the flag."""
+    import ctypes
+
+    from lm_engine_amd import _lib, ops
+
+    lib = _lib.load_library()
+    B, T, H, K, V = 4, 512, 16, 128, 128  # inside the one-launch window
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    kept = None
+    for seed in (31, 32, 33):
+        inp = random_inputs(B, T, H, K, V, dtype=BF16, seed=seed)
+        q, k, v, g, beta, h0 = (inp[n].cuda() for n in ("q", "k", "v", "g", "beta", "initial_state"))
+        assert fused_launch_applies(q, v)
+        dims = ops._check_inputs(q, k, v, g, beta, h0, None)
+        outs = []
+        for promise in (False, True):
+            o = torch.full((B, T, H, V), float("nan"), dtype=BF16, device="cuda")
+            ht = torch.full((B, H, K, V), float("nan"), dtype=torch.float32, device="cuda")
+            args = ops._fill_args(q, k, v, g, beta, h0, ht, o, None, None, False, False, dims)
+            assert args.flags & _lib.GDN_FLAG_FUSED_LAUNCH
+            nbytes = int(lib.gdn_workspace_bytes(ctypes.byref(args)))
+            if promise:
+                kept = torch.zeros(nbytes, dtype=torch.uint8, device="cuda") if kept is None else kept
+                workspace = kept
+                args.flags |= _lib.GDN_FLAG_READY_FLAGS_CLEAR
+            else:
+                workspace = torch.full((nbytes,), 0xFF, dtype=torch.uint8, device="cuda")  # stale flags all set
+            args.workspace, args.workspace_bytes = workspace.data_ptr(), workspace.numel()
+            print(f"gdn_chunk_fwd seed={seed} ready flags promised clear: {promise}", flush=True)
+            _lib.check_status(lib.gdn_chunk_fwd(ctypes.byref(args), stream), "gdn_chunk_fwd")
+            torch.cuda.synchronize()
+            # workspace = [chunk offsets and order | flags | records]: everything in front of the records but the first region
+            records = H * B * (T // 64) * 13312
+            first = ((2 * B + 1) * 4 + 255) // 256 * 256
+            assert not workspace[first : nbytes - records].any(), "ready flags left set"
+            outs.append((o, ht))
+        assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+
+
+def test_operator_keeps_its_workspaces_between_calls():
+    from lm_engine_amd import ops
+
+    ops.release_workspaces()
+    inp = {n: (x.cuda() if isinstance(x, torch.Tensor) else x) for n, x in random_inputs(4, 512, 16, 128, 128, dtype=BF16, seed=34).items()}
+    first = lm_engine_amd.chunk_gated_delta_rule(**inp, output_final_state=True)
+    assert len(ops._WORKSPACES) == 1
+    again = lm_engine_amd.chunk_gated_delta_rule(**inp, output_final_state=True)
+    assert len(ops._WORKSPACES) == 1, "same device, stream and shape: same workspace"
+    assert torch.equal(first[0], again[0]) and torch.equal(first[1], again[1])
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        other = lm_engine_amd.chunk_gated_delta_rule(**inp, output_final_state=True)
+    side.synchronize()
+    assert len(ops._WORKSPACES) == 2, "another stream gets a workspace of its own"
+    assert torch.equal(first[0], other[0])
+    for t in range(2, 2 + ops._WORKSPACE_LIMIT + 2):
+        short = {n: (x[:, : 64 * t] if n in ("q", "k", "v", "g", "beta") else x) for n, x in inp.items()}
+        lm_engine_amd.chunk_gated_delta_rule(**short)
+    assert len(ops._WORKSPACES) == ops._WORKSPACE_LIMIT
+    ops.release_workspaces()
+    assert not ops._WORKSPACES

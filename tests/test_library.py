@@ -205,7 +205,7 @@ def test_fused_launch_flag_is_on_by_default_and_can_be_switched_off():
     with enable_kernels([Kernel.gated_delta_rule], reset=True):
         assert not is_kernel_allowed(fused) and is_kernel_allowed(Kernel.gated_delta_rule)
     assert is_kernel_allowed(fused)
-    assert _lib.GDN_FLAG_FUSED_LAUNCH == 8
+    assert _lib.GDN_FLAG_FUSED_LAUNCH == 8 and _lib.GDN_FLAG_READY_FLAGS_CLEAR == 16
 
 
 def test_kernel_flag_env_variable():
