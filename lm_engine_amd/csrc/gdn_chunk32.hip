@@ -1147,7 +1147,7 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     if (save && nw == 2) nw = 1;  // the saving variant exists for 1 and 4 slices per workgroup
     if constexpr (K > 128) nw = 1;  // K = 256 has the half-slice scan only, also as the saving variant and on given records
     // a slice with a CU to itself is scanned by two waves of 16 columns each; the records are laid out for them
-    const bool half = K > 128 || (nw == 1 && !save && !p.records_given);
+    const bool half = K > 128 || (nw == 1 && !p.records_given);
     p.rec16 = half ? 1 : 0;
     if (!p.records_given) {
         hipLaunchKernelGGL((chunk_prepare32_kernel<K>), dim3(grid_prep), dim3(PREP_THREADS), 0, stream, p);
@@ -1163,6 +1163,7 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     } else {
     if (save) {
         if (nw == 4) hipLaunchKernelGGL((chunk_scan32_kernel<K, 4, false, true>), grid, dim3(scan_waves(4) * WAVE), 0, stream, p);
+        else if (half) hipLaunchKernelGGL((chunk_scan32_kernel<K, 1, false, true, true>), grid, dim3(scan_waves(1, true) * WAVE), 0, stream, p);
         else hipLaunchKernelGGL((chunk_scan32_kernel<K, 1, false, true>), grid, dim3(scan_waves(1) * WAVE), 0, stream, p);
         return (int)hipGetLastError();
     }
