@@ -496,6 +496,105 @@ struct BwdPrepareParams {
     uint32_t rec_bytes, off_p, off_qs, off_ks, off_cs, off_eg;
 };
 
+// T = (I + A)^-1 for a strictly lower-triangular 64 x 64 matrix A (fp32 in LDS, rows LDA floats apart, zeros on and
+// above the diagonal), in place, by the four waves of the workgroup together; `scratch` holds INVERSE_SCRATCH_FLOATS.
+// The same blocked scheme as the forward's prepare step (gdn_chunk_prepare32.h, which interleaves it with its tile
+// products): wave 0 inverts the four 16 x 16 diagonal blocks by substitution (a lane owns a column: 120 dependent
+// multiply-adds instead of the 2016 of a substitution over all 64 rows), then the blocks below the diagonal follow
+// from T_BA = -T_BB (A_BA T_AA), first with 16 x 16 blocks on two waves, then with 32 x 32 blocks, one 16 x 16
+// output tile per wave, as products on the fp32 MFMA (16x16x4: no operand is rounded).  Ends with a barrier.
+constexpr int INV_LDT = 36, INV_LDM = 20;  // floats per row of the transposed 32 x 32 and 16 x 16 scratch blocks
+constexpr int INVERSE_SCRATCH_FLOATS = 32 * INV_LDT + 2 * 16 * INV_LDM + 32 * INV_LDT;
+template <int LDA_>
+__device__ __forceinline__ void invert_unit_lower_64(float* sA, float* scratch, const int wave, const int lane) {
+    constexpr int LDT = INV_LDT, LDM = INV_LDM;
+    float* const sT = sA;
+    float* const sTtA = scratch;           // transpose of the top-left 32 x 32 of T
+    float* const sMt = sTtA + 32 * LDT;    // transposed products of the first merge
+    float* const sMtB = sMt + 2 * 16 * LDM;  // transposed product of the second merge
+    const int l16 = lane % 16, lq = lane / 16;
+    __syncthreads();  // A is complete and the scratch is free
+    float x[16];  // column l16 of the inverse of diagonal block lq (wave 0)
+    if (wave == 0) {
+        const float* a = &sA[(16 * lq) * LDA_ + 16 * lq];
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            f32x4 row[4];
+#pragma unroll
+            for (int c4 = 0; c4 < (i + 3) / 4; c4++) row[c4] = *reinterpret_cast<const f32x4*>(&a[i * LDA_ + 4 * c4]);
+            float part[4] = {(i == l16) ? 1.f : 0.f, 0.f, 0.f, 0.f};  // four independent partial sums
+#pragma unroll
+            for (int kk = 0; kk < i; kk++) part[kk % 4] -= row[kk / 4][kk % 4] * x[kk];
+            x[i] = (part[0] + part[1]) + (part[2] + part[3]);
+        }
+        // every lane of the wave has read its block of A by now (one wave, program order)
+#pragma unroll
+        for (int i = 0; i < 16; i++) sT[(16 * lq + i) * LDA_ + 16 * lq + l16] = x[i];
+    }
+    __syncthreads();
+    // 16 x 16 output tile of a product X Y: lane (l16, lq) supplies reduction entries k = 4 n lq + e, e < 4 n, of row l16
+    // of X and of column l16 of Y (a row of Y^T); MFMA e takes entry e of every lane.
+    auto mm16 = [&](const float* xrow, const float* ytrow) -> f32x4 {
+        const f32x4 xv = *reinterpret_cast<const f32x4*>(xrow), yv = *reinterpret_cast<const f32x4*>(ytrow);
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc = mfma_f32(xv[e], yv[e], acc);
+        return acc;
+    };
+    auto mm16x32 = [&](const float* xrow, const float* ytrow) -> f32x4 {
+        const f32x4 x0 = *reinterpret_cast<const f32x4*>(xrow), x1 = *reinterpret_cast<const f32x4*>(xrow + 4);
+        const f32x4 y0 = *reinterpret_cast<const f32x4*>(ytrow), y1 = *reinterpret_cast<const f32x4*>(ytrow + 4);
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc = mfma_f32(x0[e], y0[e], acc);
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc = mfma_f32(x1[e], y1[e], acc);
+        return acc;
+    };
+    // first merge: T_10 = -T_11 (A_10 T_00) on wave 0, T_32 = -T_33 (A_32 T_22) on wave 1
+    if (wave < 2) {
+        const int bi = 2 * wave + 1, bj = 2 * wave;
+        const int kk = 4 * lq;
+        float* const mt = &sMt[wave * 16 * LDM];
+        f32x4 y0;  // column l16 of T_bj,bj, entries kk .. kk + 3 (a row of its transpose)
+#pragma unroll
+        for (int e = 0; e < 4; e++) y0[e] = sT[(16 * bj + kk + e) * LDA_ + 16 * bj + l16];
+        f32x4 m = {0.f, 0.f, 0.f, 0.f};
+        {
+            const f32x4 xa = *reinterpret_cast<const f32x4*>(&sA[(16 * bi + l16) * LDA_ + 16 * bj + kk]);
+#pragma unroll
+            for (int e = 0; e < 4; e++) m = mfma_f32(xa[e], y0[e], m);
+        }
+        if (wave == 0 && lq < 2) {
+            // the transposes of T_00 and T_11 for the second merge, from the registers of the inverse, and the zero block (T_01)^T
+#pragma unroll
+            for (int c4 = 0; c4 < 4; c4++)
+                *reinterpret_cast<f32x4*>(&sTtA[(16 * lq + l16) * LDT + 16 * lq + 4 * c4]) = f32x4{x[4 * c4], x[4 * c4 + 1], x[4 * c4 + 2], x[4 * c4 + 3]};
+            if (lq == 1) {
+#pragma unroll
+                for (int c4 = 0; c4 < 4; c4++) *reinterpret_cast<f32x4*>(&sTtA[(16 + l16) * LDT + 4 * c4]) = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+        }
+        *reinterpret_cast<f32x4*>(&mt[l16 * LDM + 4 * lq]) = m;  // M^T[n][4 lq + e]
+        const f32x4 t = mm16(&sT[(16 * bi + l16) * LDA_ + 16 * bi + kk], &mt[l16 * LDM + kk]);
+#pragma unroll
+        for (int e = 0; e < 4; e++) sT[(16 * bi + 4 * lq + e) * LDA_ + 16 * bj + l16] = -t[e];  // over A_bi,bj, read above
+        if (wave == 0) *reinterpret_cast<f32x4*>(&sTtA[l16 * LDT + 16 + 4 * lq]) = -t;  // (T_10)^T
+    }
+    __syncthreads();
+    // second merge: T_BA = -T_BB (A_BA T_AA) with 32 x 32 blocks; one 16 x 16 output tile per wave
+    {
+        const int ta = wave / 2, tb = wave % 2;
+        const f32x4 m = mm16x32(&sA[(32 + 16 * ta + l16) * LDA_ + 8 * lq], &sTtA[(16 * tb + l16) * LDT + 8 * lq]);
+        *reinterpret_cast<f32x4*>(&sMtB[(16 * tb + l16) * LDT + 16 * ta + 4 * lq]) = m;
+        __syncthreads();
+        const f32x4 t = mm16x32(&sT[(32 + 16 * ta + l16) * LDA_ + 32 + 8 * lq], &sMtB[(16 * tb + l16) * LDT + 8 * lq]);
+#pragma unroll
+        for (int e = 0; e < 4; e++) sT[(32 + 16 * ta + 4 * lq + e) * LDA_ + 16 * tb + l16] = -t[e];
+    }
+    __syncthreads();  // T is complete
+}
+
 template <int V>
 __global__ __launch_bounds__(BWD_THREADS) void chunk_bwd_prepare_kernel(const BwdPrepareParams p) {
     constexpr int K = BWD_K;
@@ -623,25 +722,9 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_bwd_prepare_kernel(const Bw
             }
         }
 
-    // ---- T = (I + A)^-1 in place of A: lane = column, row i needs rows 0 .. i - 1 ----
-    if (wave == 0) {
-        float Tc[C];
-#pragma unroll
-        for (int i = 0; i < C; i++) {
-            float x = (i == lane) ? 1.f : 0.f;
-#pragma unroll
-            for (int j4 = 0; j4 < (i + 3) / 4; j4++) {
-                const f32x4 a = *reinterpret_cast<const f32x4*>(sA + i * LDA + 4 * j4);  // same address in every lane
-#pragma unroll
-                for (int e = 0; e < 4; e++)
-                    if (4 * j4 + e < i) x -= a[e] * Tc[4 * j4 + e];
-            }
-            Tc[i] = x;
-        }
-#pragma unroll
-        for (int i = 0; i < C; i++) sA[i * LDA + lane] = Tc[i];
-    }
-    __syncthreads();
+    // ---- T = (I + A)^-1 in place of A (the rows of q and k in LDS are dead: their place is the scratch) ----
+    static_assert(INVERSE_SCRATCH_FLOATS * 4 <= C * LDR * 2, "the scratch of the inverse fits the rows of q");
+    invert_unit_lower_64<LDA>(sA, reinterpret_cast<float*>(sQ), wave, lane);
 
     // ---- the two records ----
     uint8_t* recA = p.rec + ((int64_t)h * ((int64_t)p.N * 2 * p.NC) + (int64_t)n * 2 * p.NC + 2 * (p.NC - 1 - ci)) * p.rec_bytes;
