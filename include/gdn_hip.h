@@ -52,6 +52,8 @@ enum {
                                    unless this flag promises that they are clear.  Every call that returns success
                                    leaves them clear again, with or without the flag, so a workspace that is used for
                                    nothing else, by calls of one shape on one stream, keeps the promise by itself. */
+    GDN_FLAG_RECORDS_16X16 = 32, /* gdn_chunk_bwd_prepare: write the operand fragments of the mirror problem's records in
+                                   the lane order of the 16x16x32 MFMA, for gdn_chunk_fwd_saving with records_given = 2 */
 };
 
 /*
@@ -154,10 +156,12 @@ int gdn_recurrent_fwd(const gdn_args *args, void *stream);
  * [0, chunks_per_chain) are computed but not saved.
  * With records_given != 0 the prepare kernel is skipped: args->workspace then holds the chunk records
  * themselves, [H][B * ceil(T / 64)] records in the layout prepare writes (fixed-length batches only;
- * g, beta and the l2norm flag are not used, the records carry every scale).  The twelve operand fragments
- * of a record are then expected in the lane order of the 32x32x16 MFMA for K <= 128 and of the 16x16x32
- * MFMA for K = 256 (the scan that runs on them).  The backward pass of this package runs its reverse sweep
- * over the chunks that way.
+ * g, beta and the l2norm flag are not used, the records carry every scale).  records_given = 1: the twelve
+ * operand fragments of a record are in the lane order of the 32x32x16 MFMA (K <= 128 only; the scan runs
+ * whole-slice waves, 1 or 4 slices per workgroup).  records_given = 2: they are in the lane order of the
+ * 16x16x32 MFMA (any K, required for K = 256); the scan then runs one slice per workgroup on two half-slice
+ * waves, which is the faster kernel as long as N * H * V / 32 does not exceed the number of compute units.
+ * The backward pass of this package runs its reverse sweep over the chunks that way.
  */
 typedef struct gdn_chunk_saves {
     float *states;

@@ -20,6 +20,7 @@ GDN_FLAG_STATE_INPLACE = 2
 GDN_FLAG_LEFT_PADDED = 4
 GDN_FLAG_FUSED_LAUNCH = 8
 GDN_FLAG_READY_FLAGS_CLEAR = 16
+GDN_FLAG_RECORDS_16X16 = 32
 
 GDN_NOALLOC_SCRATCH_BYTES = 64 << 20  # built-in workspace of gdn_chunk_fwd_noalloc
 

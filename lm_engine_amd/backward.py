@@ -202,7 +202,7 @@ def _fragment_index(device, half_slices=False):
 RECORD_BYTES = 13312  # a chunk record: 12 fragments, 3 x 64 row scales, e^{gamma_C}
 
 
-def _mirror_problem(N, H, kraw, qraw, doc, Tm, P, egl, cs_a, ks_a, ks_b, aligned_inputs=None):
+def _mirror_problem(N, H, kraw, qraw, doc, Tm, P, egl, cs_a, ks_a, ks_b, aligned_inputs=None, half_slices=False):
     """Tensors and chunk records of the reverse sweep as a forward scan (see the module docstring).
 
     Inputs are packed [N * H, NC, C, ...] fp32; ``cs_a``, ``ks_a``, ``ks_b`` are the row scales of the A and
@@ -232,7 +232,7 @@ def _mirror_problem(N, H, kraw, qraw, doc, Tm, P, egl, cs_a, ks_a, ks_b, aligned
         v_m[:, :, 1] = do
         v_m = v_m.view(N, 2 * NC * CHUNK, H, V)
 
-    rows, cols = _fragment_index(dev, half_slices=K > 128)  # the scan that runs on K = 256 is the half-slice one
+    rows, cols = _fragment_index(dev, half_slices=half_slices)
     eye = torch.eye(CHUNK, device=dev)
     # T^T with rows and columns reversed is lower-triangular again: entry (i', j') is T[63 - j', 63 - i']
     Tmir = Tm.transpose(-1, -2).flip(-1, -2)
@@ -272,12 +272,15 @@ def _sweeps_on_scan_kernel(q, k, v, do, g, beta, scale, initial_state, cu_seqlen
     live = pk.valid.reshape(N, 1, NC, CHUNK, 1).expand(N, H, NC, CHUNK, 1).reshape(Bt, NC, CHUNK, 1)
     Vn = torch.where(live, Vn, torch.zeros_like(Vn))  # rows past the end of a sequence hold whatever the kernel left
 
+    # K = 256 scans on half-slice waves only; smaller heads do when every slice gets a CU
+    half_slices = K > 128 or ops.half_slice_records_pay(Bt, V, dev)
     k_m, v_m, rec = _mirror_problem(N, H, kraw, qraw, doc, Tm, P, egl, cs_a, ks_a, ks_b,
-                                    aligned_inputs=(q, k, do) if pk.aligned else None)  # fmt: skip
+                                    aligned_inputs=(q, k, do) if pk.aligned else None, half_slices=half_slices)  # fmt: skip
     dS1 = torch.empty(Bt, NC, K, V, device=dev)
     dht32 = None if dht is None else dht.to(torch.float32).contiguous()
     # the A chunks are the even ones; mirror chunk 2 r is chunk NC - 1 - r of the forward order
-    o_m, dS = ops.chunk_scan_given_records(k_m, v_m, rec, dht32, dS1, NC, save_every=2, save_reverse=True)
+    o_m, dS = ops.chunk_scan_given_records(k_m, v_m, rec, dht32, dS1, NC, save_every=2, save_reverse=True,
+                                           half_slice_records=half_slices)  # fmt: skip
     # the A chunks' output, back in forward order: [N, NC, 2, C, H, V] -> [Bt, NC, C, V]
     Y = o_m.view(N, NC, 2, CHUNK, H, V)[:, :, 0].flip(1, 2).permute(0, 3, 1, 2, 4).reshape(Bt, NC, CHUNK, V).float()
     return S0, Vn, dS1, Y, dS.reshape(Bt, K, V)
@@ -352,14 +355,15 @@ def _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, l2norm
         sequences = (as_i32(starts), as_i32(lens), NC)
     Bt = N * H
     q, k, v, do = (x if x.stride(-1) == 1 else x.contiguous() for x in (q, k, v, do.to(torch.bfloat16)))
-    prep = ops.chunk_bwd_prepare(q, k, do, g, beta, scale, l2norm, V, sequences)
+    half_slices = ops.half_slice_records_pay(Bt, V, dev)
+    prep = ops.chunk_bwd_prepare(q, k, do, g, beta, scale, l2norm, V, sequences, half_slice_records=half_slices)
     S0 = torch.empty(Bt, NC, K, V, device=dev)
     Vn = torch.empty(Bt, NC, CHUNK, V, device=dev)
     ops.chunk_forward_saving(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2norm, left_padded, S0, Vn, NC)
     dS1 = torch.empty(Bt, NC, K, V, device=dev)
     dht32 = None if dht is None else dht.to(torch.float32).contiguous()
     o_m, dS = ops.chunk_scan_given_records(prep["k_mirror"], prep["v_mirror"], prep["records"], dht32, dS1, NC,
-                                           save_every=2, save_reverse=True)  # fmt: skip
+                                           save_every=2, save_reverse=True, half_slice_records=half_slices)  # fmt: skip
     dq, dk, dv, dg, dbeta = ops.chunk_local_grads_final(q, k, v, do, prep, o_m, Vn, S0, dS1, scale, l2norm, sequences)
     return (
         dq,

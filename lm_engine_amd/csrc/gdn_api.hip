@@ -154,6 +154,8 @@ int gdn_chunk_fwd_saving(const gdn_args* a, const gdn_chunk_saves* saves, void* 
     if ((saves->states && !aligned(saves->states, 16)) || (saves->v_new && !aligned(saves->v_new, 16))) return GDN_ERR_ALIGN;
     if (saves->chunks_per_chain <= 0) return GDN_ERR_SHAPE;  // chunks beyond it are computed but not saved
     uint64_t need = gdn::chunk_workspace_bytes(*a);
+    if (saves->records_given < 0 || saves->records_given > 2) return GDN_ERR_SHAPE;
+    if (saves->records_given == 1 && a->K > 128) return GDN_ERR_UNSUPPORTED;  // K = 256 scans on half-slice waves only
     if (saves->records_given) {
         if (a->cu_seqlens != nullptr) return GDN_ERR_VARLEN;  // records are given for fixed-length batches only
         need = gdn::chunk_record_bytes(*a);

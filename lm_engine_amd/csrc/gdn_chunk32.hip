@@ -1146,8 +1146,9 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     if (p.cu_seqlens != nullptr && !save && nw > 1 && chains * (vtiles / (nw / 2)) <= 2 * (int64_t)num_cus) nw /= 2;
     if (save && nw == 2) nw = 1;  // the saving variant exists for 1 and 4 slices per workgroup
     if constexpr (K > 128) nw = 1;  // K = 256 has the half-slice scan only, also as the saving variant and on given records
+    if (p.records_given == 2) nw = 1;  // records given in the half-slice scan's fragment order
     // a slice with a CU to itself is scanned by two waves of 16 columns each; the records are laid out for them
-    const bool half = K > 128 || (nw == 1 && !p.records_given);
+    const bool half = K > 128 || p.records_given == 2 || (nw == 1 && !p.records_given);
     p.rec16 = half ? 1 : 0;
     if (!p.records_given) {
         hipLaunchKernelGGL((chunk_prepare32_kernel<K>), dim3(grid_prep), dim3(PREP_THREADS), 0, stream, p);

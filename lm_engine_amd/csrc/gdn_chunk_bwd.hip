@@ -482,6 +482,7 @@ struct BwdPrepareParams {
     int64_t d_stride_b, d_stride_t, d_stride_h;
     int N, H, NC;
     int l2norm;
+    int rec16;  // fragments of the records in the lane order of the 16x16x32 MFMA (GDN_FLAG_RECORDS_16X16)
     float scale;
     float* gam;
     float* bc;
@@ -731,12 +732,17 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_bwd_prepare_kernel(const Bw
     uint8_t* recB = recA + p.rec_bytes;
     for (int fl = t; fl < 6 * WAVE; fl += BWD_THREADS) {
         const int f = fl / WAVE, L = fl % WAVE;
-        const int row = 32 * (f < 2 ? 0 : 1) + L % 32;
-        const int col0 = 16 * (f < 2 ? f : f - 2) + 4 * (L / 32);
+        // fragment f, lane L, element e -> entry (row, col) of the lower-triangular 64 x 64 matrix.  32x32x16 order:
+        // fragments (row tile, 16-column slab) = (0,0) (0,1) (1,0) (1,1) (1,2) (1,3); a lane holds columns 4 h + 0..3 and
+        // 8 + 4 h + 0..3 of the slab.  16x16x32 order: (16-row tile, 32-column slab) = (0,0) (1,0) (2,0) (2,1) (3,0) (3,1);
+        // a lane holds columns 4 g + 0..3 and 16 + 4 g + 0..3 of the slab.
+        const int row = p.rec16 ? 16 * (f < 2 ? f : 2 + (f - 2) / 2) + L % 16 : 32 * (f < 2 ? 0 : 1) + L % 32;
+        const int col0 = p.rec16 ? 32 * (f < 2 ? 0 : f % 2) + 4 * (L / 16) : 16 * (f < 2 ? f : f - 2) + 4 * (L / 32);
+        const int second = p.rec16 ? 12 : 4;  // elements 4..7 lie this many columns past e
         bf16x8 tm, id, zz;
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-            const int col = col0 + (e < 4 ? e : e + 4);
+            const int col = col0 + (e < 4 ? e : e + second);
             // mirrored transpose: entry (row, col) is T[63 - col][63 - row], zero above the diagonal
             tm[e] = (bf16_t)(row >= col ? sA[(C - 1 - col) * LDA + (C - 1 - row)] : 0.f);
             id[e] = (bf16_t)(row == col ? 1.f : 0.f);
@@ -810,6 +816,7 @@ int launch_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args& a, hipStream_t st
     p.N = a.N, p.H = a.H, p.NC = a.seq_start != nullptr ? a.NC : a.T / C;
     p.seq_start = a.seq_start, p.seq_len = a.seq_len, p.T_rows = a.T;
     p.l2norm = (a.flags & GDN_FLAG_L2NORM) ? 1 : 0;
+    p.rec16 = (a.flags & GDN_FLAG_RECORDS_16X16) ? 1 : 0;
     p.scale = a.scale;
     p.gam = a.gamma, p.bc = a.beta_packed;
     p.rq = a.rq, p.rk = a.rk;

@@ -287,13 +287,22 @@ def chunk_forward_saving(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2n
                           "gdn_chunk_fwd_saving")  # fmt: skip
 
 
-def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_chain, save_every=1, save_reverse=False):
+def half_slice_records_pay(chains: int, V: int, device) -> bool:
+    """Whether a scan over given records should get them in the fragment order of the half-slice scan (16x16x32
+    MFMA): that scan runs one 32-column slice per workgroup, the faster kernel while the slices of all chains
+    (``chains`` = sequences x heads) do not outnumber the compute units."""
+    return chains * (V // 32) <= torch.cuda.get_device_properties(device).multi_processor_count
+
+
+def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_chain, save_every=1, save_reverse=False,
+                             half_slice_records=False):
     """The scan kernel alone over a fixed-length batch whose chunk records the caller has written
     (``records`` uint8 ``[H, B * T / 64, record bytes]``, T a multiple of 64); it reads the rows of ``k`` (also
     in the place of q: such records carry zero row scales for q) and of ``v``.  Returns ``(o, final_state)``
     and writes the state that chunk ``c`` starts from, for every ``c`` divisible by ``save_every``, into entry
     ``c / save_every`` of ``states`` ``[B * H, chunks_per_chain, K, V]`` (counted from the end with
-    ``save_reverse``)."""
+    ``save_reverse``).  ``half_slice_records``: the fragments of the records are in the lane order of the
+    16x16x32 MFMA (K = 256 needs that) instead of the 32x32x16 one."""
     _require_hip_path()
     lib = _lib.load_library()
     dims = _check_inputs(k, k, v, None, None, initial_state, None)
@@ -306,7 +315,8 @@ def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_ch
     ht = torch.empty(N, H, K, V, dtype=torch.float32, device=v.device)
     args = _fill_args(k, k, v, None, None, initial_state, ht, o, None, 1.0, False, False, dims)
     args.workspace, args.workspace_bytes = records.data_ptr(), records.numel()
-    saves = _lib.GdnChunkSaves(states.data_ptr(), None, chunks_per_chain, 1, save_every, 1 if save_reverse else 0)
+    saves = _lib.GdnChunkSaves(states.data_ptr(), None, chunks_per_chain, 2 if half_slice_records else 1, save_every,
+                               1 if save_reverse else 0)  # fmt: skip
     with torch.cuda.device(k.device):
         stream = ctypes.c_void_p(torch.cuda.current_stream(k.device).cuda_stream)
         _lib.check_status(lib.gdn_chunk_fwd_saving(ctypes.byref(args), ctypes.byref(saves), stream),
@@ -404,13 +414,14 @@ def chunk_local_grads_final(q, k, v, dout, prep, y_mirror, v_new, states, dstate
 RECORD_BYTES = 13312  # chunk record of the 32x32x16 kernels (K <= 128)
 
 
-def chunk_bwd_prepare(q, k, dout, g, beta, scale, l2norm, V, sequences=None):
+def chunk_bwd_prepare(q, k, dout, g, beta, scale, l2norm, V, sequences=None, half_slice_records=False):
     """``gdn_chunk_bwd_prepare``.  ``q, k, dout`` are the caller's bf16 ``[B, T, H, D]`` tensors; without
     ``sequences`` every row is one sequence of whole chunks, else ``sequences = (seq_start, seq_len, NC)``: int32
     device tensors ``[N]`` (first token as a flat index over the rows, length) and the chunks per sequence to lay
     the results out with.  Returns a dict: ``gamma, beta, rq, rk`` (fp32 ``[N H, NC, 64]``: prefix sums of g inside
     the chunks, beta, inverse norms of the rows of q and k) and the mirror problem ``k_mirror, v_mirror``
-    ``[N, 2 NC 64, H, D]`` bf16, ``records`` uint8 ``[H, N * 2 NC, RECORD_BYTES]``."""
+    ``[N, 2 NC 64, H, D]`` bf16, ``records`` uint8 ``[H, N * 2 NC, RECORD_BYTES]`` (their fragments in the lane order
+    of the 16x16x32 MFMA with ``half_slice_records``, see ``chunk_scan_given_records``)."""
     _require_hip_path()
     lib = _lib.load_library()
     B, T, H, K = q.shape
@@ -445,7 +456,7 @@ def chunk_bwd_prepare(q, k, dout, g, beta, scale, l2norm, V, sequences=None):
         setattr(a, f"{name}_stride_h", x.stride(2))
     a.N, a.T, a.H, a.K, a.V = N, T, H, K, V
     a.beta_dtype = _lib.GDN_F32 if beta is None else _dtype_code(beta.dtype, "beta")
-    a.flags = _lib.GDN_FLAG_L2NORM if l2norm else 0
+    a.flags = (_lib.GDN_FLAG_L2NORM if l2norm else 0) | (_lib.GDN_FLAG_RECORDS_16X16 if half_slice_records else 0)
     a.scale = float(scale)
     a.gamma, a.beta_packed, a.rq, a.rk = (out[n].data_ptr() for n in ("gamma", "beta", "rq", "rk"))
     a.k_mirror, a.v_mirror, a.records = (out[n].data_ptr() for n in ("k_mirror", "v_mirror", "records"))
