@@ -222,6 +222,13 @@ def bench_chunk(w, steps, warmup, two_kernels=False):
             "traffic": step_traffic,
             "traffic_scope": "whole step: " + " + ".join(per_kernel) + " (per kernel under step.kernels)",
             "algorithmic_bytes": int(algo_bytes),
+            # the same step against the other roof: its algorithmic bytes over the sum of its kernels' durations
+            "hbm": {
+                "achieved": round(algo_bytes / (sum(k["ms"] for k in per_kernel.values()) * 1e-3) / 1e9, 1),
+                "peak": HBM_PEAK_GBS,
+                "unit": "GB/s",
+                "frac": round(algo_bytes / (sum(k["ms"] for k in per_kernel.values()) * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            },
         },
         "step": {
             "tflops_dense": round(whole_tflops, 1),
