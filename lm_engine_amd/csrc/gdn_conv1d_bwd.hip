@@ -93,47 +93,64 @@ __global__ __launch_bounds__(CB_THREADS) void causal_conv1d_bwd_kernel(const Con
 #pragma unroll
     for (int j = 0; j < KS - 1; j++) load_xx(s_begin - (KS - 1) + j, win[j + 1]);  // shifted into place by the first step
 
-    for (int s = s_begin; s < s_end; s++) {
-        // slide: win[j] <- win[j + 1], pend likewise (pend[0] of the last step was emitted below)
+    // The walk goes in steps of UNROLL tokens whose rows of x and dy are all requested before the first is used: a
+    // thread then has 2 UNROLL loads in flight instead of two, which is what a streaming kernel with this few waves
+    // per CU needs to keep the memory system busy.  (Rows past s_end are read again from row s_end - 1 and not used.)
+    constexpr int UNROLL = 4;
+    for (int s0 = s_begin; s0 < s_end; s0 += UNROLL) {
+        bf16x8 xr[UNROLL], gr[UNROLL];
 #pragma unroll
-        for (int e = 0; e < VEC; e++) {
-#pragma unroll
-            for (int j = 0; j + 1 < KS; j++) win[j][e] = win[j + 1][e], pend[j][e] = pend[j + 1][e];
-            pend[KS - 1][e] = 0.f;
+        for (int u = 0; u < UNROLL; u++) {
+            const int su = min(s0 + u, s_end - 1);
+            xr[u] = *reinterpret_cast<const bf16x8*>(xb + (int64_t)su * p.x_stride_s);
+            gr[u] = *reinterpret_cast<const bf16x8*>(dyb + (int64_t)su * p.dy_stride_s);
         }
-        load_xx(s, win[KS - 1]);
-        const bf16x8 g = *reinterpret_cast<const bf16x8*>(dyb + (int64_t)s * p.dy_stride_s);
-        const float m = mb == nullptr ? 1.f : (float)mb[s];
-        const bool own = s < s_own;
 #pragma unroll
-        for (int e = 0; e < VEC; e++) {
-            float z = bias[e];
+        for (int u = 0; u < UNROLL; u++) {
+            const int s = s0 + u;
+            if (s >= s_end) break;
+            // slide: win[j] <- win[j + 1], pend likewise (pend[0] of the last step was emitted below)
 #pragma unroll
-            for (int j = 0; j < KS; j++) z += w[e][j] * win[j][e];
-            float dz = (float)g[e] * m;
-            if (SILU) {
-                const float sg = __builtin_amdgcn_rcpf(1.f + __expf(-z));
-                dz *= sg * (1.f + z * (1.f - sg));
+            for (int e = 0; e < VEC; e++) {
+#pragma unroll
+                for (int j = 0; j + 1 < KS; j++) win[j][e] = win[j + 1][e], pend[j][e] = pend[j + 1][e];
+                pend[KS - 1][e] = 0.f;
             }
+            const float m = mb == nullptr ? 1.f : (float)mb[s];
 #pragma unroll
-            for (int j = 0; j < KS; j++) pend[j][e] += w[e][j] * dz;  // x index s - (KS - 1) + j
-            if (own) {
-                db[e] += dz;
+            for (int e = 0; e < VEC; e++) win[KS - 1][e] = (float)xr[u][e] * m;
+            const bf16x8 g = gr[u];
+            const bool own = s < s_own;
 #pragma unroll
-                for (int j = 0; j < KS; j++) dw[e][j] += dz * win[j][e];
+            for (int e = 0; e < VEC; e++) {
+                float z = bias[e];
+#pragma unroll
+                for (int j = 0; j < KS; j++) z += w[e][j] * win[j][e];
+                float dz = (float)g[e] * m;
+                if (SILU) {
+                    const float sg = __builtin_amdgcn_rcpf(1.f + __expf(-z));
+                    dz *= sg * (1.f + z * (1.f - sg));
+                }
+#pragma unroll
+                for (int j = 0; j < KS; j++) pend[j][e] += w[e][j] * dz;  // x index s - (KS - 1) + j
+                if (own) {
+                    db[e] += dz;
+#pragma unroll
+                    for (int j = 0; j < KS; j++) dw[e][j] += dz * win[j][e];
+                }
             }
-        }
-        // x index t = s - (KS - 1) is complete now
-        const int t = s - (KS - 1);
-        if (t >= s_begin) {
-            const float mt = mb == nullptr ? 1.f : (float)mb[t];
-            bf16x8 out;
+            // x index t = s - (KS - 1) is complete now
+            const int t = s - (KS - 1);
+            if (t >= s_begin) {
+                const float mt = mb == nullptr ? 1.f : (float)mb[t];
+                bf16x8 out;
 #pragma unroll
-            for (int e = 0; e < VEC; e++) out[e] = (bf16_t)(pend[0][e] * mt);
-            *reinterpret_cast<bf16x8*>(dxb + (int64_t)t * p.C) = out;
-        } else if (t < 0 && p.dstate != nullptr) {  // only in the first block of a row
+                for (int e = 0; e < VEC; e++) out[e] = (bf16_t)(pend[0][e] * mt);
+                *reinterpret_cast<bf16x8*>(dxb + (int64_t)t * p.C) = out;
+            } else if (t < 0 && p.dstate != nullptr) {  // only in the first block of a row
 #pragma unroll
-            for (int e = 0; e < VEC; e++) p.dstate[((int64_t)b * p.C + c0 + e) * (KS - 1) + (KS - 1) + t] = (bf16_t)pend[0][e];
+                for (int e = 0; e < VEC; e++) p.dstate[((int64_t)b * p.C + c0 + e) * (KS - 1) + (KS - 1) + t] = (bf16_t)pend[0][e];
+            }
         }
     }
     // the rows still in flight: x indices s_end - (KS - 1) + 1 .. s_end - 1 (complete only at the end of the sequence;
