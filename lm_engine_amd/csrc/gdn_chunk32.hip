@@ -380,6 +380,21 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
     __shared__ __attribute__((aligned(16))) uint8_t stage[2][STAGE_BYTES];
     __shared__ __attribute__((aligned(16))) uint8_t qstage[QS ? C * QLD : 16];  // the single buffer of q rows (QS)
     __shared__ __attribute__((aligned(16))) uint8_t ostage[OS ? NW * 2 * C * 64 : 16];
+    // LSAVE (the saving half-slice scan, K <= 128): the compute waves leave the state a chunk starts from and V~ in LDS, as
+    // rows of the slice's 32 fp32 columns, and the store wave writes them out in whole 128-byte lines.  Stores from the
+    // compute waves themselves are 64-byte halves of those lines from two waves, and a store that waits for room in the
+    // memory queue stalls the wave that feeds the matrix pipe.  Two buffers each, by chunk parity.  (K = 256 has no LDS
+    // left for them and stores from its compute waves.)
+    constexpr bool LSAVE = SAVE && HALF && !QS;
+    constexpr int SROW = 32 * 4;  // bytes per staged row
+    __shared__ __attribute__((aligned(16))) uint8_t sstage[LSAVE ? 2 : 1][LSAVE ? K * SROW : 16];
+    __shared__ __attribute__((aligned(16))) uint8_t vstage[LSAVE ? 2 : 1][LSAVE ? C * SROW : 16];
+    static_assert(!LSAVE || 2 * STAGE_BYTES + NW * 2 * C * 64 + 2 * (K + C) * SROW <= 160 * 1024, "the staging of the saves exceeds LDS");
+    // entry of the save arrays that chunk c goes to, or -1
+    auto save_entry = [&](int c) -> int {
+        if (c % p.save_every != 0 || c / p.save_every >= p.save_nc) return -1;
+        return p.save_reverse ? p.save_nc - 1 - c / p.save_every : c / p.save_every;
+    };
 
     const int lane = threadIdx.x % WAVE;
     const int wave = threadIdx.x / WAVE;
@@ -456,14 +471,41 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
                         __builtin_nontemporal_store(rows[i], reinterpret_cast<bf16x8*>(og + ((int64_t)c * C + 16 * i) * p.o_stride_t + 32 * w));
             }
         };
+        // LSAVE: rows of 32 fp32 columns, 8 lanes per row, 8 rows per instruction
+        auto flush_rows = [&](const uint8_t* staged, float* dst, int rows) {  // dst: row 0, column 0 of this slice
+            const int r0 = lane / 8, piece = lane % 8;
+            for (int r = 0; r < rows; r += 32) {
+                f32x4 x[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) x[i] = *reinterpret_cast<const f32x4*>(staged + (r + 8 * i + r0) * SROW + 16 * piece);
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    __builtin_nontemporal_store(x[i], reinterpret_cast<f32x4*>(dst + (int64_t)(r + 8 * i + r0) * p.V + 4 * piece));
+            }
+        };
+        auto flush_state = [&](int c) {  // the state chunk c starts from
+            if constexpr (LSAVE) {
+                const int entry = save_entry(c);
+                if (p.save_state != nullptr && entry >= 0)
+                    flush_rows(sstage[c & 1], p.save_state + ((int64_t)chain * p.save_nc + entry) * K * p.V + 32 * vgroup, K);
+            }
+        };
+        auto flush_vnew = [&](int c) {  // V~ of chunk c
+            if constexpr (LSAVE) {
+                const int entry = save_entry(c);
+                if (p.save_vnew != nullptr && entry >= 0)
+                    flush_rows(vstage[c & 1], p.save_vnew + ((int64_t)chain * p.save_nc + entry) * C * p.V + 32 * vgroup, C);
+            }
+        };
         __syncthreads();
         for (int c = 0; c < nchunks; c++) {
             if constexpr (QS) __syncthreads();  // barrier Q
-            __syncthreads();
-            if (c > 0) flush(c - 1);
+            __syncthreads();  // the state of chunk c, V~ and the output of chunk c - 1 are staged
+            flush_state(c);
+            if (c > 0) flush(c - 1), flush_vnew(c - 1);
         }
         __syncthreads();
-        if (nchunks > 0) flush(nchunks - 1);
+        if (nchunks > 0) flush(nchunks - 1), flush_vnew(nchunks - 1);
         return;
     }
     if (is_loader) {
@@ -722,7 +764,17 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
             if constexpr (SAVE) {
                 // the state this chunk starts from, for the backward pass (one wave-uniform base plus one per-lane
                 // byte offset, as in the whole-slice scan)
-                if (p.save_state != nullptr && c % p.save_every == 0 && c / p.save_every < p.save_nc) {
+                if constexpr (LSAVE) {
+                    // into this chunk's staging buffer (read by the store wave after this chunk's barrier, written again two
+                    // chunks on, after the next chunk's barrier)
+                    if (p.save_state != nullptr && save_entry(c) >= 0) {
+                        uint8_t* const base = sstage[c & 1] + (8 * g) * SROW + (16 * half + j16) * 4;
+#pragma unroll
+                        for (int t = 0; t < KT; t++)
+#pragma unroll
+                            for (int r = 0; r < 4; r++) *reinterpret_cast<float*>(base + (32 * (t / 2) + 4 * (t % 2) + r) * SROW) = S[t][r];
+                    }
+                } else if (p.save_state != nullptr && c % p.save_every == 0 && c / p.save_every < p.save_nc) {
                     const int entry = p.save_reverse ? p.save_nc - 1 - c / p.save_every : c / p.save_every;
                     char* base = reinterpret_cast<char*>(p.save_state + ((int64_t)chain * p.save_nc + entry) * K * p.V);
                     const uint32_t lane_off = (uint32_t)((8 * g) * p.V + c0 + j16) * 4u;
@@ -827,7 +879,16 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
             });
             if constexpr (SAVE) {
                 // V~ of this chunk: tile tt, register r holds token 16 tt + 4 g + r of this lane's column
-                if (p.save_vnew != nullptr && c % p.save_every == 0 && c / p.save_every < p.save_nc) {
+                if constexpr (LSAVE) {
+                    // after this chunk's barrier: the store wave takes it after the next one (or the last)
+                    if (p.save_vnew != nullptr && save_entry(c) >= 0) {
+                        uint8_t* const base = vstage[c & 1] + (4 * g) * SROW + (16 * half + j16) * 4;
+#pragma unroll
+                        for (int tt = 0; tt < 4; tt++)
+#pragma unroll
+                            for (int r = 0; r < 4; r++) *reinterpret_cast<float*>(base + (16 * tt + r) * SROW) = vt[tt][r];
+                    }
+                } else if (p.save_vnew != nullptr && c % p.save_every == 0 && c / p.save_every < p.save_nc) {
                     const int entry = p.save_reverse ? p.save_nc - 1 - c / p.save_every : c / p.save_every;
                     char* base = reinterpret_cast<char*>(p.save_vnew + ((int64_t)chain * p.save_nc + entry) * C * p.V);
                     const uint32_t lane_off = (uint32_t)((4 * g) * p.V + c0 + j16) * 4u;
