@@ -284,6 +284,16 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
             }
         }
 
+        // dS1 of this half is asked for now and stays in registers while the products with S0 run: its trip through
+        // memory is then behind them instead of in front of the barrier below (the workgroup has a CU to itself by its
+        // LDS, so there is no other wave to fill the wait)
+        f32x4 ds1_rows[16];
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int idx = t + BWD_THREADS * i, row = idx / 32, c4 = idx % 32;
+            ds1_rows[i] = *reinterpret_cast<const f32x4*>(ds1 + row * V + v0 + 4 * c4);
+        }
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int tt = 0; tt < 2; tt++) {
             dQeT[tt] = mma_nt(sST + 32 * wave * LDR, LDR, sDO + 32 * tt * LDR, LDR, VW, dQeT[tt], l32, lh);
@@ -301,7 +311,7 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
 #pragma unroll
             for (int i = 0; i < 16; i++) {
                 const int idx = t + BWD_THREADS * i, row = idx / 32, c4 = idx % 32;
-                const f32x4 x = *reinterpret_cast<const f32x4*>(ds1 + row * V + v0 + 4 * c4);
+                const f32x4 x = ds1_rows[i];
                 const bf16x4 sv = *reinterpret_cast<const bf16x4*>(sST + row * LDR + 4 * c4);
                 dot += x.x * (float)sv.x + x.y * (float)sv.y + x.z * (float)sv.z + x.w * (float)sv.w;
                 put4(sST + row * LDR + 4 * c4, x);
