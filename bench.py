@@ -18,6 +18,7 @@ inputs already resident in HBM.  Prints ONE JSON line:
   epilogue     rmsnorm(o * silu(gate)) behind the operator, same batch, against the HBM peak
   cpu_baseline the naive token-by-token torch restatement of the operator (oracle/), timed on
                this host's cores on a bounded prefix of the same workload
+  backward     one backward of the operator at the headline shape (and, under `other`, at the shipped head shape)
   forward_other the same forward with prepare and scan as two kernels (the headline configuration runs them as one
                launch by default), on configurations 2 (packed sequences) and 4 (long context, V=256; both ways), and
                on the head shape of the reference's shipped configurations (B=8, T=4096, H=2, K=256, V=512)
@@ -535,6 +536,15 @@ def main():
     backward = None if args.no_decode else bench_backward(w, inp, args.steps, args.warmup)
     if backward is not None:
         backward["layer_kernels"] = bench_layer_backward_kernels(w, args.steps, args.warmup)
+        if not args.no_other_configs:
+            # the same leg at the head shape of the reference's shipped configurations (K = 256, V = 512)
+            import torch
+
+            from lm_engine_amd.workloads import make_inputs
+
+            shipped = replace(get_workload(1, B=8, H=2, K=256, V=512), name="shipped_head_shape_k256_v512_bf16")
+            backward["other"] = [bench_backward(shipped, make_inputs(shipped, device="cuda"), args.steps, args.warmup)]
+            torch.cuda.empty_cache()
     other = None
     if not args.no_other_configs:
         # the forward on the other chunked configurations, and with prepare and scan in one launch where that qualifies
