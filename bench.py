@@ -7,8 +7,8 @@ A "step" is one chunked forward (``chunk_gated_delta_rule``) over one batch of s
 the benchmark configuration (default: configuration 1, B=4, T=4096, H=16, K=V=128, bf16, chunk 64),
 inputs already resident in HBM.  Prints ONE JSON line:
 
-  value        tokens/s of the whole step (B*T / wall time per step, all kernels, workspace
-               allocation through the caching allocator included)
+  value        tokens/s of the whole step (B*T / wall time per step, all kernels and the allocation of the
+               outputs included; the operator keeps its workspace between steps)
   roofline     the dominant kernel of the step against the bf16 dense MFMA peak: algorithmic
                FLOPs of the contractions that kernel performs / its HIP-event duration
   decode       the decode step (configuration 3: 256 sequences x 32 heads, fp32 state 512 MiB
