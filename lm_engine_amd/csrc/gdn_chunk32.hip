@@ -1206,6 +1206,10 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     // (Configuration 2, 11 sequences of 202 .. 6350 tokens, H = 16: 246 us with four slices per workgroup, 193 us with two.)
     if (p.cu_seqlens != nullptr && !save && nw > 1 && chains * (vtiles / (nw / 2)) <= 2 * (int64_t)num_cus) nw /= 2;
     if (save && nw == 2) nw = 1;  // the saving variant exists for 1 and 4 slices per workgroup
+    // The saving scan of a packed batch (the backward's forward sweep): started longest first as well, its half-slice
+    // variant, whose saves go through LDS, finishes a ragged batch sooner than four slices per workgroup storing from
+    // their compute waves, while there are at most four workgroups per CU (configuration 2: 352 us against 575 us).
+    if (save && p.cu_seqlens != nullptr && !p.records_given && K <= 128 && chains * vtiles <= 4 * (int64_t)num_cus) nw = 1;
     if constexpr (K > 128) nw = 1;  // K = 256 has the half-slice scan only, also as the saving variant and on given records
     if (p.records_given == 2) nw = 1;  // records given in the half-slice scan's fragment order
     // a slice with a CU to itself is scanned by two waves of 16 columns each; the records are laid out for them
