@@ -659,83 +659,109 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_bwd_prepare_kernel(const Bw
 
     // ---- rows of q, k, v, dO: 16-byte pieces, 16 lanes per row ----
     const int p8 = t % 16;
+    if (valid == 0) {
+        // A chunk slot past the end of its sequence (batches laid out with the chunk count of their longest sequence):
+        // what the code below would arrive at from rows of zeros - zero rows of the mirror problem, T = I, the constant
+        // inverse norms - written directly; only the records are then formed as for any other chunk.
+        const float r0 = p.l2norm ? rsqrtf(L2NORM_EPS) : 1.f;
 #pragma unroll
-    for (int it = 0; it < 4; it++) {
-        const int row = t / 16 + 16 * it;
-        const bool live = row < valid;
-        bf16x8 qr = *reinterpret_cast<const bf16x8*>(row_of(p.q, p.q_stride_b, p.q_stride_t, p.q_stride_h, row) + 8 * p8);
-        bf16x8 kr = *reinterpret_cast<const bf16x8*>(row_of(p.k, p.k_stride_b, p.k_stride_t, p.k_stride_h, row) + 8 * p8);
-        if (!live) qr = zero8, kr = zero8;
-        float ssq = 0.f, ssk = 0.f;
+        for (int it = 0; it < 4; it++) {
+            const int row = t / 16 + 16 * it;
+            if (p8 == 0) {
+                s_rq[row] = r0, s_rk[row] = r0;
+                p.rq[chunk * C + row] = r0, p.rk[chunk * C + row] = r0;
+            }
+            const int64_t tokA = ((int64_t)n * TM + mir0 + (C - 1 - row)) * p.H + h, tokB = tokA + (int64_t)C * p.H;
+            *reinterpret_cast<bf16x8*>(p.k_m + tokA * K + 8 * p8) = zero8;
+            *reinterpret_cast<bf16x8*>(p.k_m + tokB * K + 8 * p8) = zero8;
 #pragma unroll
-        for (int e = 0; e < 8; e++) ssq += (float)qr[e] * (float)qr[e], ssk += (float)kr[e] * (float)kr[e];
-#pragma unroll
-        for (int off = 8; off >= 1; off >>= 1) ssq += __shfl_xor(ssq, off, WAVE), ssk += __shfl_xor(ssk, off, WAVE);
-        const float rq = p.l2norm ? rsqrtf(ssq + L2NORM_EPS) : 1.f, rk = p.l2norm ? rsqrtf(ssk + L2NORM_EPS) : 1.f;
-        if (p8 == 0) {
-            s_rq[row] = rq, s_rk[row] = rk;
-            p.rq[chunk * C + row] = rq, p.rk[chunk * C + row] = rk;
-        }
-        bf16x8 qb, kb;
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-            qb[e] = (bf16_t)((float)qr[e] * rq * p.scale);
-            kb[e] = (bf16_t)((float)kr[e] * rk);
-        }
-        *reinterpret_cast<bf16x8*>(sQ + row * LDR + 8 * p8) = qb;
-        *reinterpret_cast<bf16x8*>(sK + row * LDR + 8 * p8) = kb;
-        // mirror rows: token `row` of this chunk is token 63 - row of chunks A and B
-        const int64_t tokA = ((int64_t)n * TM + mir0 + (C - 1 - row)) * p.H + h, tokB = tokA + (int64_t)C * p.H;
-        *reinterpret_cast<bf16x8*>(p.k_m + tokA * K + 8 * p8) = kr;
-        *reinterpret_cast<bf16x8*>(p.k_m + tokB * K + 8 * p8) = qr;
-#pragma unroll
-        for (int hv = 0; hv < V / 128; hv++) {
-            bf16x8 dr = *reinterpret_cast<const bf16x8*>(row_of(p.dout, p.d_stride_b, p.d_stride_t, p.d_stride_h, row) + 128 * hv + 8 * p8);
-            if (!live) dr = zero8;
-#pragma unroll
-            for (int e = 0; e < 8; e++) sDOT[(128 * hv + 8 * p8 + e) * LDS64 + row] = dr[e];
-            *reinterpret_cast<bf16x8*>(p.v_m + tokB * V + 128 * hv + 8 * p8) = dr;
-        }
-    }
-    __syncthreads();
-
-    f32x16 zero;
-#pragma unroll
-    for (int r = 0; r < 16; r++) zero[r] = 0.f;
-
-    // ---- A = stril(beta_i E . K K^T) and P^T = tril(E . Q K^T)^T: wave -> tile (ti, tj) ----
-    {
-        const int ti = wave / 2, tj = wave % 2;
-        const f32x16 KK = mma_nt(sK + 32 * ti * LDR, LDR, sK + 32 * tj * LDR, LDR, K, zero, l32, lh);
-        const f32x16 QK = mma_nt(sQ + 32 * ti * LDR, LDR, sK + 32 * tj * LDR, LDR, K, zero, l32, lh);
-        const int j = 32 * tj + l32;
-        const float gj = s_gam[j];
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int i = 32 * ti + 8 * (r / 4) + 4 * lh + r % 4;
-            const float E = i >= j ? __expf(s_gam[i] - gj) : 0.f;
-            sA[i * LDA + j] = i > j ? s_beta[i] * E * KK[r] : 0.f;
-            sPT[j * LDS64 + i] = (bf16_t)(E * QK[r]);
-        }
-    }
-    __syncthreads();
-
-    // ---- P^T dO -> rows of v_m for chunk A: rows j = 32 tj + .., columns v = 32 tv + l32, tv = wave, wave + 4, .. ----
-#pragma unroll
-    for (int tv = wave; tv < V / 32; tv += BWD_THREADS / WAVE)
-#pragma unroll
-        for (int tj = 0; tj < 2; tj++) {
-            const f32x16 u = mma_nt(sPT + 32 * tj * LDS64, LDS64, sDOT + 32 * tv * LDS64, LDS64, C, zero, l32, lh);
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int j = 32 * tj + 8 * (r / 4) + 4 * lh + r % 4;
-                p.v_m[(((int64_t)n * TM + mir0 + (C - 1 - j)) * p.H + h) * V + 32 * tv + l32] = (bf16_t)u[r];
+            for (int hv = 0; hv < V / 128; hv++) {
+                *reinterpret_cast<bf16x8*>(p.v_m + tokA * V + 128 * hv + 8 * p8) = zero8;
+                *reinterpret_cast<bf16x8*>(p.v_m + tokB * V + 128 * hv + 8 * p8) = zero8;
             }
         }
+        for (int i = t; i < C * C; i += BWD_THREADS) sA[(i / C) * LDA + i % C] = (i / C == i % C) ? 1.f : 0.f;
+        __syncthreads();
+    } else {
+#pragma unroll
+        for (int it = 0; it < 4; it++) {
+            const int row = t / 16 + 16 * it;
+            const bool live = row < valid;
+            bf16x8 qr = *reinterpret_cast<const bf16x8*>(row_of(p.q, p.q_stride_b, p.q_stride_t, p.q_stride_h, row) + 8 * p8);
+            bf16x8 kr = *reinterpret_cast<const bf16x8*>(row_of(p.k, p.k_stride_b, p.k_stride_t, p.k_stride_h, row) + 8 * p8);
+            if (!live) qr = zero8, kr = zero8;
+            float ssq = 0.f, ssk = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) ssq += (float)qr[e] * (float)qr[e], ssk += (float)kr[e] * (float)kr[e];
+#pragma unroll
+            for (int off = 8; off >= 1; off >>= 1) ssq += __shfl_xor(ssq, off, WAVE), ssk += __shfl_xor(ssk, off, WAVE);
+            const float rq = p.l2norm ? rsqrtf(ssq + L2NORM_EPS) : 1.f, rk = p.l2norm ? rsqrtf(ssk + L2NORM_EPS) : 1.f;
+            if (p8 == 0) {
+                s_rq[row] = rq, s_rk[row] = rk;
+                p.rq[chunk * C + row] = rq, p.rk[chunk * C + row] = rk;
+            }
+            bf16x8 qb, kb;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                qb[e] = (bf16_t)((float)qr[e] * rq * p.scale);
+                kb[e] = (bf16_t)((float)kr[e] * rk);
+            }
+            *reinterpret_cast<bf16x8*>(sQ + row * LDR + 8 * p8) = qb;
+            *reinterpret_cast<bf16x8*>(sK + row * LDR + 8 * p8) = kb;
+            // mirror rows: token `row` of this chunk is token 63 - row of chunks A and B
+            const int64_t tokA = ((int64_t)n * TM + mir0 + (C - 1 - row)) * p.H + h, tokB = tokA + (int64_t)C * p.H;
+            *reinterpret_cast<bf16x8*>(p.k_m + tokA * K + 8 * p8) = kr;
+            *reinterpret_cast<bf16x8*>(p.k_m + tokB * K + 8 * p8) = qr;
+#pragma unroll
+            for (int hv = 0; hv < V / 128; hv++) {
+                bf16x8 dr = *reinterpret_cast<const bf16x8*>(row_of(p.dout, p.d_stride_b, p.d_stride_t, p.d_stride_h, row) + 128 * hv + 8 * p8);
+                if (!live) dr = zero8;
+#pragma unroll
+                for (int e = 0; e < 8; e++) sDOT[(128 * hv + 8 * p8 + e) * LDS64 + row] = dr[e];
+                *reinterpret_cast<bf16x8*>(p.v_m + tokB * V + 128 * hv + 8 * p8) = dr;
+            }
+        }
+        __syncthreads();
 
-    // ---- T = (I + A)^-1 in place of A (the rows of q and k in LDS are dead: their place is the scratch) ----
-    static_assert(INVERSE_SCRATCH_FLOATS * 4 <= C * LDR * 2, "the scratch of the inverse fits the rows of q");
-    invert_unit_lower_64<LDA>(sA, reinterpret_cast<float*>(sQ), wave, lane);
+        f32x16 zero;
+#pragma unroll
+        for (int r = 0; r < 16; r++) zero[r] = 0.f;
+
+        // ---- A = stril(beta_i E . K K^T) and P^T = tril(E . Q K^T)^T: wave -> tile (ti, tj) ----
+        {
+            const int ti = wave / 2, tj = wave % 2;
+            const f32x16 KK = mma_nt(sK + 32 * ti * LDR, LDR, sK + 32 * tj * LDR, LDR, K, zero, l32, lh);
+            const f32x16 QK = mma_nt(sQ + 32 * ti * LDR, LDR, sK + 32 * tj * LDR, LDR, K, zero, l32, lh);
+            const int j = 32 * tj + l32;
+            const float gj = s_gam[j];
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int i = 32 * ti + 8 * (r / 4) + 4 * lh + r % 4;
+                const float E = i >= j ? __expf(s_gam[i] - gj) : 0.f;
+                sA[i * LDA + j] = i > j ? s_beta[i] * E * KK[r] : 0.f;
+                sPT[j * LDS64 + i] = (bf16_t)(E * QK[r]);
+            }
+        }
+        __syncthreads();
+
+        // ---- P^T dO -> rows of v_m for chunk A: rows j = 32 tj + .., columns v = 32 tv + l32, tv = wave, wave + 4, .. ----
+#pragma unroll
+        for (int tv = wave; tv < V / 32; tv += BWD_THREADS / WAVE)
+#pragma unroll
+            for (int tj = 0; tj < 2; tj++) {
+                const f32x16 u = mma_nt(sPT + 32 * tj * LDS64, LDS64, sDOT + 32 * tv * LDS64, LDS64, C, zero, l32, lh);
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int j = 32 * tj + 8 * (r / 4) + 4 * lh + r % 4;
+                    p.v_m[(((int64_t)n * TM + mir0 + (C - 1 - j)) * p.H + h) * V + 32 * tv + l32] = (bf16_t)u[r];
+                }
+            }
+
+        // ---- T = (I + A)^-1 in place of A (the rows of q and k in LDS are dead: their place is the scratch) ----
+        static_assert(INVERSE_SCRATCH_FLOATS * 4 <= C * LDR * 2, "the scratch of the inverse fits the rows of q");
+        invert_unit_lower_64<LDA>(sA, reinterpret_cast<float*>(sQ), wave, lane);
+
+    }
 
     // ---- the two records ----
     uint8_t* recA = p.rec + ((int64_t)h * ((int64_t)p.N * 2 * p.NC) + (int64_t)n * 2 * p.NC + 2 * (p.NC - 1 - ci)) * p.rec_bytes;
