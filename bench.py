@@ -506,7 +506,7 @@ def bench_backward(w, inp, steps, warmup):
         "ms_per_backward": round(ms, 3),
         "tokens_per_s": round(w.B * w.T / (ms * 1e-3), 1),
         "composition": ("5 kernel launches: backward prepare, forward prepare + saving scan, saving scan over the "
-                        "mirror problem, chunk-local gradients" if w.K == 128 and w.V in (128, 256) else
+                        "mirror problem, chunk-local gradients" if w.K == 128 and w.V in (128, 256, 512) else
                         "2 saving scans + rocBLAS batched GEMMs + elementwise torch ops"),
     }
 

@@ -187,7 +187,7 @@ int gdn_chunk_fwd_saving(const gdn_args *args, const gdn_chunk_saves *saves, voi
  * qs = scale * q (* rq), kn = k (* rk).  Outputs: dq, dk [chunks][64][K], the gradients with respect to q and
  * k themselves (through the scale and the normalisation), dbeta [chunks][64], and dgamma [chunks][64], the
  * gradient with respect to gamma (dg is its reverse prefix sum inside the chunk).
- * K = 128 with V = 128 or 256 only (GDN_ERR_UNSUPPORTED otherwise).  Counterpart upstream: the chunk-local kernels of fla's
+ * K = 128 with V = 128, 256 or 512 only (GDN_ERR_UNSUPPORTED otherwise).  Counterpart upstream: the chunk-local kernels of fla's
  * backward of chunk_gated_delta_rule, reached from gated_deltanet/module.py:197-209 under autograd.
  */
 typedef struct gdn_chunk_local_args {
@@ -228,7 +228,7 @@ int gdn_chunk_bwd_local(const gdn_chunk_local_args *args, void *stream);
  * Training support, third part: everything the backward needs per chunk before its two sweeps (batches of
  * whole chunks: T a multiple of 64, one sequence per row; other batches through seq_start / seq_len below;
  * bf16 q, k, dout as [N, T, H, D] with element
- * strides; K = 128 and V = 128 or 256, GDN_ERR_UNSUPPORTED otherwise).  One workgroup per (sequence, head, chunk) writes
+ * strides; K = 128 and V = 128, 256 or 512, GDN_ERR_UNSUPPORTED otherwise).  One workgroup per (sequence, head, chunk) writes
  *   - gamma, beta_packed, rq, rk: fp32 [N H T/64][64], operands of gdn_chunk_bwd_local;
  *   - the reverse sweep as a forward scan over 2 T tokens per sequence ("mirror" problem: tokens in reverse
  *     order, chunk c becomes chunks 2 r and 2 r + 1, r = T/64 - 1 - c): k_mirror [N, 2 T, H, K] and

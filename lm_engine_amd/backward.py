@@ -6,7 +6,7 @@ the gradients of ``(o, final_state)`` with respect to ``(q, k, v, g, beta, initi
 
 Three ways through, same formulas:
 
-* bf16, K = 128, V = 128 or 256 (whole rows, packed or left-padded batches): five kernel launches
+* bf16, K = 128, V = 128, 256 or 512 (whole rows, packed or left-padded batches): five kernel launches
   (``_backward_on_kernels``) - ``gdn_chunk_bwd_prepare``, ``gdn_chunk_fwd_saving`` for the forward sweep and
   again over the mirror problem for the reverse sweep, ``gdn_chunk_bwd_local``;
 * other bf16 shapes: the two sweeps over the chunks of a chain on the scan kernel
@@ -337,7 +337,7 @@ def _chunk_local_grads(qs, kn, vc, doc, Y, Vn, S0, dS1, gam, bc):
 
 
 def _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, l2norm, cu_seqlens, left_padded):
-    """The whole backward on five kernel launches (bf16, K = 128, V = 128 or 256): ``gdn_chunk_bwd_prepare``
+    """The whole backward on five kernel launches (bf16, K = 128, V = 128, 256 or 512): ``gdn_chunk_bwd_prepare``
     (mirror problem and per-chunk scalars), the saving forward sweep, the saving scan over the mirror problem,
     ``gdn_chunk_bwd_local`` writing the gradients in the caller's layout.  Packed and left-padded batches are laid
     out with the chunk count of their longest sequence."""

@@ -21,7 +21,7 @@
 // Every matrix product is an "A B^T" of two row-major bf16 matrices staged in LDS (the transposes of Q and K
 // are staged next to them), on 32x32x16 MFMA with fp32 accumulation.  The 64 x K results are kept transposed
 // ([key dim][token]) so that a lane owns one token: the per-token scales are per-lane scalars and the sums
-// over the key dim stay inside a lane.  Built for K = 128 and V = 128 or 256 (the value dim is staged 128 columns
+// over the key dim stay inside a lane.  Built for K = 128 and V = 128, 256 or 512 (the value dim is staged 128 columns
 // at a time; 157 KiB of LDS: one workgroup per CU).
 #include <hip/hip_runtime.h>
 
@@ -32,7 +32,7 @@ namespace gdn {
 
 namespace {
 
-constexpr int BWD_K = 128;  // the kernels of this file are built for K = 128 and V = 128 or 256
+constexpr int BWD_K = 128;  // the kernels of this file are built for K = 128 and V = 128, 256 or 512
 constexpr int BWD_THREADS = 256;
 constexpr int LDR = 136;  // bf16 per LDS row of a [.][128] matrix: 16 bytes of padding
 constexpr int LDS64 = 72;  // bf16 per LDS row of a [.][64] matrix
@@ -823,15 +823,16 @@ int launch_chunk_bwd_local(const gdn_chunk_local_args& a, hipStream_t stream) {
     p.v_stride_b = a.v_stride_b, p.v_stride_t = a.v_stride_t, p.v_stride_h = a.v_stride_h;
     p.d_stride_b = a.dout_stride_b, p.d_stride_t = a.dout_stride_t, p.d_stride_h = a.dout_stride_h;
     p.seq_start = a.seq_start, p.seq_len = a.seq_len, p.T_rows = a.seq_start != nullptr ? a.T_rows : a.NC * C;
-    if (a.V == 256) hipLaunchKernelGGL(chunk_local_grads_kernel<256>, dim3((unsigned)a.chunks), dim3(BWD_THREADS), 0, stream, p);
+    if (a.V == 512) hipLaunchKernelGGL(chunk_local_grads_kernel<512>, dim3((unsigned)a.chunks), dim3(BWD_THREADS), 0, stream, p);
+    else if (a.V == 256) hipLaunchKernelGGL(chunk_local_grads_kernel<256>, dim3((unsigned)a.chunks), dim3(BWD_THREADS), 0, stream, p);
     else hipLaunchKernelGGL(chunk_local_grads_kernel<128>, dim3((unsigned)a.chunks), dim3(BWD_THREADS), 0, stream, p);
     return (int)hipGetLastError();
 }
 
-bool chunk_bwd_local_supported(const gdn_chunk_local_args& a) { return a.K == BWD_K && (a.V == 128 || a.V == 256); }
+bool chunk_bwd_local_supported(const gdn_chunk_local_args& a) { return a.K == BWD_K && (a.V == 128 || a.V == 256 || a.V == 512); }
 
 bool chunk_bwd_prepare_supported(const gdn_chunk_bwd_prepare_args& a) {
-    if (a.K != BWD_K || (a.V != 128 && a.V != 256) || a.T <= 0) return false;
+    if (a.K != BWD_K || (a.V != 128 && a.V != 256 && a.V != 512) || a.T <= 0) return false;
     return a.seq_start != nullptr ? (a.seq_len != nullptr && a.NC > 0) : a.T % C == 0;
 }
 
@@ -860,7 +861,8 @@ int launch_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args& a, hipStream_t st
     p.rec = static_cast<uint8_t*>(a.records);
     p.rec_bytes = r.bytes, p.off_p = r.off_p, p.off_qs = r.off_qs, p.off_ks = r.off_ks, p.off_cs = r.off_cs, p.off_eg = r.off_eg;
     const int64_t chunks = (int64_t)a.N * a.H * p.NC;
-    if (a.V == 256) hipLaunchKernelGGL(chunk_bwd_prepare_kernel<256>, dim3((unsigned)chunks), dim3(BWD_THREADS), 0, stream, p);
+    if (a.V == 512) hipLaunchKernelGGL(chunk_bwd_prepare_kernel<512>, dim3((unsigned)chunks), dim3(BWD_THREADS), 0, stream, p);
+    else if (a.V == 256) hipLaunchKernelGGL(chunk_bwd_prepare_kernel<256>, dim3((unsigned)chunks), dim3(BWD_THREADS), 0, stream, p);
     else hipLaunchKernelGGL(chunk_bwd_prepare_kernel<128>, dim3((unsigned)chunks), dim3(BWD_THREADS), 0, stream, p);
     return (int)hipGetLastError();
 }

@@ -324,7 +324,7 @@ def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_ch
     return o, ht
 
 
-CHUNK_LOCAL_KV = ((128, 128), (128, 256))  # head dims gdn_chunk_bwd_local and gdn_chunk_bwd_prepare are built for
+CHUNK_LOCAL_KV = ((128, 128), (128, 256), (128, 512))  # head dims gdn_chunk_bwd_local and gdn_chunk_bwd_prepare are built for
 
 
 def chunk_local_grads(qs, kn, v, dout, y, v_new, states, dstates, gamma, beta, scale, rq=None, rk=None):

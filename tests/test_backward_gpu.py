@@ -123,7 +123,7 @@ def test_chunk_bf16_k256_packed():
     _run_case(lm_engine_amd.chunk_gated_delta_rule, inp, torch.bfloat16, cu=cu)
 
 
-@pytest.mark.parametrize("V", [128, 256])
+@pytest.mark.parametrize("V", [128, 256, 512])
 def test_chunk_bf16_whole_chunks_all_on_kernels(V):
     # whole chunks, K = 128: prepare, both sweeps and the chunk-local gradients are kernel launches
     inp = random_inputs(B=2, T=192, H=3, K=128, V=V, dtype=torch.bfloat16, seed=30 + V, normalize=False)
@@ -197,7 +197,7 @@ def test_saved_chunk_states_are_the_states_of_the_prefixes(K, V):
         assert_parity(states[:, :, c], want, torch.bfloat16, f"state at the start of chunk {c}")
 
 
-@pytest.mark.parametrize("V", [128, 256])
+@pytest.mark.parametrize("V", [128, 256, 512])
 def test_chunk_local_kernel_matches_the_batched_gemm_version(V):
     """``gdn_chunk_bwd_local`` against the same stage written with torch operations, on random packed inputs."""
     from lm_engine_amd import ops
