@@ -304,3 +304,26 @@ def test_recurrent_bf16_short_sequences():
     # T <= 64: the layer calls the recurrent operator; its backward runs the chunk kernels on one ragged chunk
     inp = random_inputs(B=2, T=40, H=2, K=128, V=128, dtype=torch.bfloat16, seed=14, normalize=False)
     _run_case(lm_engine_amd.fused_recurrent_gated_delta_rule, inp, torch.bfloat16)
+
+
+def test_given_records_in_both_fragment_orders_give_the_same_sweep():
+    """``gdn_chunk_fwd_saving`` on given records: the records of one mirror problem written in the lane order of the
+    32x32x16 MFMA (``records_given = 1``, whole-slice waves) and of the 16x16x32 MFMA (``records_given = 2``,
+    half-slice waves) give the same output, saved states and final state up to the rounding of two different kernels."""
+    from lm_engine_amd import ops
+
+    B, T, H, K, V = 2, 256, 2, 128, 128
+    inp = random_inputs(B=B, T=T, H=H, K=K, V=V, dtype=torch.bfloat16, seed=91, normalize=False)
+    q, k, g, beta = (inp[n].cuda() for n in ("q", "k", "g", "beta"))
+    do = torch.randn(B, T, H, V, generator=torch.Generator().manual_seed(92)).to(torch.bfloat16).cuda()
+    NC = T // 64
+    results = []
+    for half_slices in (False, True):
+        prep = ops.chunk_bwd_prepare(q, k, do, g, beta, K**-0.5, True, V, None, half_slice_records=half_slices)
+        dS1 = torch.zeros(B * H, NC, K, V, device="cuda")
+        o_m, dS = ops.chunk_scan_given_records(prep["k_mirror"], prep["v_mirror"], prep["records"], None, dS1, NC,
+                                               save_every=2, save_reverse=True, half_slice_records=half_slices)  # fmt: skip
+        torch.cuda.synchronize()
+        results.append((o_m.float().cpu(), dS1.cpu(), dS.cpu()))
+    for name, a, b in zip(("output", "saved states", "final state"), *results):
+        assert rel_l2(a, b) <= 5e-3, f"{name}: rel-L2 {rel_l2(a, b):.3e}"
