@@ -1,10 +1,10 @@
-// Chunked forward of the gated delta rule, K <= 128: kernels built on v_mfma_f32_32x32x16_bf16
-// (the only bf16 MFMA shape that reaches the full matrix-core rate on gfx950; 16x16x32 measured
-// ~0.8x of it).
+// Chunked forward of the gated delta rule (K = 64, 128, 256): the kernels.  Whole-slice waves work on
+// v_mfma_f32_32x32x16_bf16 (K <= 128), half-slice waves on v_mfma_f32_16x16x32_bf16 (K <= 128 when a slice has a
+// CU to itself, and K = 256 always).
 //
-// Two kernels as in gdn_chunk.hip (prepare: what does not depend on the state, written as MFMA
-// operand fragments to a workspace record per (head, chunk); scan: the serial pass over the chunks
-// of a sequence with the state held in MFMA accumulators), but with the WY form's T pulled out:
+// Two kernels (prepare: what does not depend on the state, written as MFMA operand fragments to a workspace
+// record per (head, chunk); scan: the serial pass over the chunks of a sequence with the state held in MFMA
+// accumulators; gdn_chunk.hip holds the host side), with the WY form's T pulled out:
 //     V~ = U - W S0 = T diag(beta) (V - diag(cs) K S0),      cs = e^{gamma} / |k|
 // so the record holds T diag(beta) and P only, prepare never touches V, and the scan works from the
 // caller's q, k and v.  Further:

@@ -35,7 +35,7 @@ struct ChunkParams {
     float scale;
     uint32_t rec_bytes, off_qs, off_ks, off_cs, off_p, off_eg;
     int scan_groups;  // workgroups per (sequence, head) in the scan kernel
-    // training support (K <= 128): when set, the scan also writes the fp32 state every
+    // training support: when set, the scan also writes the fp32 state every
     // chunk starts from, [N * H][save_nc][K][V], and V~ of every chunk, [N * H][save_nc][64][V]
     float* save_state;
     float* save_vnew;

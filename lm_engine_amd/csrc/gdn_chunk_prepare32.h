@@ -1,6 +1,6 @@
-// The prepare step of the chunked forward on v_mfma_f32_32x32x16_bf16 (K <= 128): everything about a chunk that does
-// not depend on the state, written as one record per (head, chunk slot).  A device function, so that it can run as
-// a kernel of its own (gdn_chunk32.hip) and as the producer half of the fused forward (gdn_chunk_pair.hip).
+// The prepare step of the chunked forward on v_mfma_f32_32x32x16_bf16 (K = 64, 128, 256): everything about a chunk
+// that does not depend on the state, written as one record per (head, chunk slot).  A device function, so that it can
+// run as a kernel of its own (gdn_chunk32.hip) and as the producer half of the one-launch forward (gdn_chunk_fused.hip).
 #pragma once
 
 #include "gdn_chunk32_common.h"

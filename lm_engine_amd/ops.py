@@ -411,7 +411,7 @@ def chunk_local_grads_final(q, k, v, dout, prep, y_mirror, v_new, states, dstate
     return out["dq_out"], out["dk_out"], out["dv_out"], out["dg_out"], out["dbeta_out"]
 
 
-RECORD_BYTES = 13312  # chunk record of the 32x32x16 kernels (K <= 128)
+RECORD_BYTES = 13312  # a chunk record: 12 operand fragments, 3 x 64 row scales, e^{gamma_C}
 
 
 def chunk_bwd_prepare(q, k, dout, g, beta, scale, l2norm, V, sequences=None, half_slice_records=False):
