@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define GDN_ABI_VERSION 1
+#define GDN_ABI_VERSION 2
 
 typedef enum gdn_dtype { GDN_BF16 = 0, GDN_F32 = 1 } gdn_dtype;
 
@@ -35,7 +35,8 @@ typedef enum gdn_status {
     GDN_ERR_UNSUPPORTED = -3, /* head dims / dtype / chunk size this build has no kernel for */
     GDN_ERR_ALIGN = -4,       /* pointer or stride not aligned as the kernels require */
     GDN_ERR_WORKSPACE = -5,   /* workspace missing or smaller than gdn_workspace_bytes() */
-    GDN_ERR_VARLEN = -6       /* cu_seqlens given with B != 1 */
+    GDN_ERR_VARLEN = -6,      /* cu_seqlens given with B != 1 */
+    GDN_ERR_TIMEOUT = -7      /* gdn_chunk_fwd_status: the one-launch forward gave up waiting for a record; outputs invalid */
 } gdn_status;
 
 enum {
@@ -54,6 +55,9 @@ enum {
                                    nothing else, by calls of one shape on one stream, keeps the promise by itself. */
     GDN_FLAG_RECORDS_16X16 = 32, /* gdn_chunk_bwd_prepare: write the operand fragments of the mirror problem's records in
                                    the lane order of the 16x16x32 MFMA, for gdn_chunk_fwd_saving with records_given = 2 */
+    GDN_FLAG_DEBUG_NO_PRODUCERS = 64, /* test aid for the one-launch forward: its prepare workgroups return at once, so that
+                                   the scan's bounded wait runs out (with a small args->spin_limit) and the error path can be
+                                   exercised while every kernel still ends normally; outputs are invalid */
 };
 
 /*
@@ -98,7 +102,11 @@ typedef struct gdn_args {
     int32_t beta_dtype; /* gdn_dtype of beta */
     int32_t flags;      /* GDN_FLAG_* */
     float scale;        /* multiplies q (after optional normalisation) */
-    int32_t reserved;
+    int32_t spin_limit; /* one-launch forward: polls of a record's ready flag before the scan gives up (0 = default, 2^22:
+                           seconds); see gdn_chunk_fwd_status */
+    int32_t *error_word; /* optional, may be NULL: an int32 the GPU can write (device memory, or pinned host memory, which a
+                           caller can read without synchronising); the one-launch forward stores 1 there when it gives up
+                           waiting.  Never cleared by the library. */
 } gdn_args;
 
 /* Version of this header the library was built from; a binding checks it equals GDN_ABI_VERSION. */
@@ -115,11 +123,36 @@ const char *gdn_strerror(int status);
 uint64_t gdn_workspace_bytes(const gdn_args *args);
 
 /*
+ * The leading bytes of the workspace that GDN_FLAG_READY_FLAGS_CLEAR promises to be zero (chunk offsets, the
+ * error latch and the ready flags); the records behind them need no initialisation.  0 for unsupported shapes.
+ */
+uint64_t gdn_workspace_header_bytes(const gdn_args *args);
+
+/*
  * Chunked forward over full sequences (bf16 q/k/v/o, fp32 state, chunk 64):
  * replaces fla.ops.gated_delta_rule.chunk_gated_delta_rule as called at
  * gated_deltanet/module.py:197-209.  `stream` is a hipStream_t.
  */
 int gdn_chunk_fwd(const gdn_args *args, void *stream);
+
+/*
+ * 1 when gdn_chunk_fwd would run these arguments as one launch (prepare and scan together) on the calling thread's
+ * current device, else 0.  Reads the shape fields, dtype, flags and whether cu_seqlens is NULL; no pointer is followed.
+ */
+int gdn_chunk_fwd_is_one_launch(const gdn_args *args);
+
+/*
+ * Error report of the one-launch forward (GDN_FLAG_FUSED_LAUNCH; no counterpart in the reference, whose Triton
+ * kernels are separate launches).  Its scan workgroups wait, with a bounded number of polls, for records that
+ * prepare workgroups of the same launch write.  A scan workgroup whose wait runs out latches an error word in
+ * the workspace header (and stores 1 to args->error_word when that is set), stops writing its outputs and runs
+ * to its end, so the launch always terminates; o and ht of that call are then invalid.  This function waits
+ * for `stream`, reads the latch of args->workspace (same shape fields as the gdn_chunk_fwd call) and returns
+ * GDN_OK or GDN_ERR_TIMEOUT; in the latter case it also zeroes the workspace header (latch and ready flags,
+ * which such a launch leaves in no defined state), so the workspace can be used again with
+ * GDN_FLAG_READY_FLAGS_CLEAR.  It blocks the calling thread.
+ */
+int gdn_chunk_fwd_status(const gdn_args *args, void *stream);
 
 /*
  * gdn_chunk_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving

@@ -10,7 +10,7 @@ import ctypes
 import os
 
 
-GDN_ABI_VERSION = 1
+GDN_ABI_VERSION = 2
 
 GDN_BF16 = 0
 GDN_F32 = 1
@@ -21,6 +21,9 @@ GDN_FLAG_LEFT_PADDED = 4
 GDN_FLAG_FUSED_LAUNCH = 8
 GDN_FLAG_READY_FLAGS_CLEAR = 16
 GDN_FLAG_RECORDS_16X16 = 32
+GDN_FLAG_DEBUG_NO_PRODUCERS = 64
+
+GDN_ERR_TIMEOUT = -7
 
 GDN_NOALLOC_SCRATCH_BYTES = 64 << 20  # built-in workspace of gdn_chunk_fwd_noalloc
 
@@ -33,7 +36,10 @@ EXPORTED_SYMBOLS = (
     "gdn_abi_version",
     "gdn_strerror",
     "gdn_workspace_bytes",
+    "gdn_workspace_header_bytes",
     "gdn_chunk_fwd",
+    "gdn_chunk_fwd_status",
+    "gdn_chunk_fwd_is_one_launch",
     "gdn_chunk_fwd_noalloc",
     "gdn_recurrent_fwd",
     "gdn_chunk_fwd_profile",
@@ -119,7 +125,7 @@ class GdnArgs(ctypes.Structure):
             for d in ("b", "t", "h")
         ]
         + [(name, ctypes.c_int32) for name in ("B", "T", "H", "K", "V", "N", "chunk", "dtype", "beta_dtype", "flags")]
-        + [("scale", ctypes.c_float), ("reserved", ctypes.c_int32)]
+        + [("scale", ctypes.c_float), ("spin_limit", ctypes.c_int32), ("error_word", ctypes.c_void_p)]
     )
 
 
@@ -182,8 +188,14 @@ def load_library() -> ctypes.CDLL:
     lib.gdn_strerror.restype = ctypes.c_char_p
     lib.gdn_workspace_bytes.argtypes = [ctypes.POINTER(GdnArgs)]
     lib.gdn_workspace_bytes.restype = ctypes.c_uint64
+    lib.gdn_workspace_header_bytes.argtypes = [ctypes.POINTER(GdnArgs)]
+    lib.gdn_workspace_header_bytes.restype = ctypes.c_uint64
     lib.gdn_chunk_fwd.argtypes = [ctypes.POINTER(GdnArgs), ctypes.c_void_p]
     lib.gdn_chunk_fwd.restype = ctypes.c_int
+    lib.gdn_chunk_fwd_is_one_launch.argtypes = [ctypes.POINTER(GdnArgs)]
+    lib.gdn_chunk_fwd_is_one_launch.restype = ctypes.c_int
+    lib.gdn_chunk_fwd_status.argtypes = [ctypes.POINTER(GdnArgs), ctypes.c_void_p]
+    lib.gdn_chunk_fwd_status.restype = ctypes.c_int
     lib.gdn_chunk_fwd_noalloc.argtypes = [ctypes.POINTER(GdnArgs), ctypes.c_void_p]
     lib.gdn_chunk_fwd_noalloc.restype = ctypes.c_int
     lib.gdn_recurrent_fwd.argtypes = [ctypes.POINTER(GdnArgs), ctypes.c_void_p]

@@ -96,6 +96,8 @@ const char* gdn_strerror(int status) {
         case GDN_ERR_WORKSPACE:
             return "workspace missing or too small (gdn_chunk_fwd_noalloc: the shape needs more than its built-in scratch)";
         case GDN_ERR_VARLEN: return "cu_seqlens requires B == 1 (packed) or GDN_FLAG_LEFT_PADDED";
+        case GDN_ERR_TIMEOUT:
+            return "the one-launch chunked forward gave up waiting for a record of its prepare half; the outputs of that call are invalid";
         default: break;
     }
     if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));
@@ -106,6 +108,13 @@ uint64_t gdn_workspace_bytes(const gdn_args* a) {
     if (a == nullptr || !gdn::chunk_shape_supported(*a)) return 0;
     return gdn::chunk_workspace_bytes(*a);
 }
+
+uint64_t gdn_workspace_header_bytes(const gdn_args* a) {
+    if (a == nullptr || !gdn::chunk_shape_supported(*a)) return 0;
+    return gdn::chunk_header_bytes(*a);
+}
+
+int gdn_chunk_fwd_is_one_launch(const gdn_args* a) { return a != nullptr && gdn::chunk_runs_as_one_launch(*a) ? 1 : 0; }
 
 int gdn_recurrent_fwd(const gdn_args* a, void* stream) {
     const int rc = validate_common(a);
@@ -126,6 +135,21 @@ int gdn_chunk_fwd(const gdn_args* a, void* stream) {
     const int rc = validate_chunk(a);
     if (rc != GDN_OK) return rc;
     return gdn::launch_chunk_fwd(*a, static_cast<hipStream_t>(stream));
+}
+
+int gdn_chunk_fwd_status(const gdn_args* a, void* stream) {
+    const int rc = validate_chunk(a);
+    if (rc != GDN_OK) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (hipError_t e = hipStreamSynchronize(s); e != hipSuccess) return (int)e;
+    int32_t latch = 0;
+    uint8_t* ws = static_cast<uint8_t*>(a->workspace);
+    if (hipError_t e = hipMemcpy(&latch, ws + gdn::chunk_error_latch_offset(*a), sizeof(latch), hipMemcpyDeviceToHost); e != hipSuccess) return (int)e;
+    if (latch == 0) return GDN_OK;
+    // every kernel of the failed call has ended: nobody sets a flag any more
+    if (hipError_t e = hipMemsetAsync(ws, 0, gdn::chunk_header_bytes(*a), s); e != hipSuccess) return (int)e;
+    if (hipError_t e = hipStreamSynchronize(s); e != hipSuccess) return (int)e;
+    return GDN_ERR_TIMEOUT;
 }
 
 int gdn_chunk_fwd_noalloc(const gdn_args* a, void* stream) {

@@ -33,8 +33,9 @@ static int chunk_slots(const gdn_args& a) {
     return packed ? a.T / C + a.N : a.B * nt;
 }
 
-// chunk offsets [N + 1] and the scan order of the sequences [N] (packed batches)
-static uint64_t chunk_off_bytes(const gdn_args& a) { return ((2 * (uint64_t)a.N + 1) * 4 + 255u) & ~(uint64_t)255u; }
+// chunk offsets [N + 1] and the scan order of the sequences [N] (packed batches), then the error latch of the one-launch
+// forward: the last 32-bit word of this region
+static uint64_t chunk_off_bytes(const gdn_args& a) { return ((2 * (uint64_t)a.N + 2) * 4 + 255u) & ~(uint64_t)255u; }
 
 bool chunk_shape_supported(const gdn_args& a) {
     if (a.dtype != GDN_BF16) return false;
@@ -51,6 +52,10 @@ uint64_t chunk_record_bytes(const gdn_args& a) {
 
 // one int32 flag per record (used when prepare and scan run in one launch)
 static uint64_t chunk_flag_bytes(const gdn_args& a) { return ((uint64_t)a.H * chunk_slots(a) * 4 + 255u) & ~(uint64_t)255u; }
+
+uint64_t chunk_header_bytes(const gdn_args& a) { return chunk_off_bytes(a) + chunk_flag_bytes(a); }
+
+uint64_t chunk_error_latch_offset(const gdn_args& a) { return chunk_off_bytes(a) - 4; }
 
 uint64_t chunk_workspace_bytes(const gdn_args& a) {
     const RecordLayout r = record_layout(a.K, a.V);
@@ -131,6 +136,12 @@ static int compute_units() {
     return cached[dev];
 }
 
+bool chunk_runs_as_one_launch(const gdn_args& a) {
+    if (!(a.flags & GDN_FLAG_FUSED_LAUNCH) || !chunk_shape_supported(a)) return false;
+    if ((a.K != 64 && a.K != 128) || a.V % 64 != 0 || a.cu_seqlens != nullptr) return false;  // see chunk_fused_supported
+    return fused_launch_window((int64_t)a.N * a.H, a.V, compute_units());
+}
+
 int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events, const gdn_chunk_saves* saves) {
     const RecordLayout r = record_layout(a.K, a.V);
     ChunkParams p;
@@ -148,13 +159,17 @@ int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events, 
     p.chunk_off = static_cast<int32_t*>(a.workspace);
     p.seq_order = p.chunk_off + a.N + 1;
     p.ready = reinterpret_cast<int32_t*>(static_cast<uint8_t*>(a.workspace) + chunk_off_bytes(a));
+    p.err = reinterpret_cast<int32_t*>(static_cast<uint8_t*>(a.workspace) + chunk_error_latch_offset(a));
+    p.err_caller = a.error_word;
+    p.spin_limit = a.spin_limit > 0 ? (uint32_t)a.spin_limit : (1u << 22);
+    p.no_producers = (a.flags & GDN_FLAG_DEBUG_NO_PRODUCERS) ? 1 : 0;
     p.rec = static_cast<uint8_t*>(a.workspace) + chunk_off_bytes(a) + chunk_flag_bytes(a);
     p.save_state = nullptr, p.save_vnew = nullptr, p.save_nc = 0, p.records_given = 0, p.save_every = 1, p.save_reverse = 0;
     if (saves != nullptr) {
         p.save_state = saves->states, p.save_vnew = saves->v_new, p.save_nc = saves->chunks_per_chain;
         p.save_every = saves->save_every > 0 ? saves->save_every : 1, p.save_reverse = saves->save_reverse ? 1 : 0;
         p.records_given = saves->records_given;
-        if (p.records_given) p.chunk_off = nullptr, p.seq_order = nullptr, p.ready = nullptr, p.rec = static_cast<uint8_t*>(a.workspace);
+        if (p.records_given) p.chunk_off = nullptr, p.seq_order = nullptr, p.ready = nullptr, p.err = nullptr, p.rec = static_cast<uint8_t*>(a.workspace);
     }
     p.q_stride_b = a.q_stride_b, p.q_stride_t = a.q_stride_t, p.q_stride_h = a.q_stride_h;
     p.k_stride_b = a.k_stride_b, p.k_stride_t = a.k_stride_t, p.k_stride_h = a.k_stride_h;

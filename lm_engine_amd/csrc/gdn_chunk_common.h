@@ -46,8 +46,20 @@ struct ChunkParams {
     int32_t* ready;     // [H][TC] one flag per record, for the launch that runs prepare and scan together
     int fused;          // that launch was asked for (GDN_FLAG_FUSED_LAUNCH)
     int ready_clear;    // the caller vouches that the ready flags are zero (GDN_FLAG_READY_FLAGS_CLEAR)
+    int32_t* err;         // error latch in the workspace header: set when a scan workgroup of that launch gave up waiting
+    int32_t* err_caller;  // the caller's own error word (gdn_args::error_word) or NULL
+    uint32_t spin_limit;  // polls of a ready flag before giving up
+    int no_producers;     // GDN_FLAG_DEBUG_NO_PRODUCERS
     int rec16;          // the fragments of T diag(beta) and P are laid out for v_mfma_f32_16x16x32_bf16 (the half-slice scan)
 };
+
+// The shapes the one-launch forward is used for: its scan workgroups (one per 64 columns of every chain, the chains rounded
+// up to a multiple of 8) fill between 3/8 and 1/2 of the compute units.  With fewer chains the two-kernel path's scan, one
+// slice per CU, is the faster one and prepare is short; with more, too few CUs are left for the producers.
+inline bool fused_launch_window(int64_t chains, int V, int num_cus) {
+    const int64_t scan_wgs = (chains + 7) / 8 * 8 * (V / 64);
+    return scan_wgs <= (int64_t)num_cus / 2 && scan_wgs >= (int64_t)num_cus * 3 / 8;
+}
 
 struct RecordLayout {
     uint32_t off_p, off_qs, off_ks, off_cs, off_eg, bytes;

@@ -106,6 +106,8 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
     uint8_t (*const xbuf)[XBYTES] = reinterpret_cast<uint8_t (*)[XBYTES]>(lds + 2 * STAGE_BYTES);
     uint8_t (*const ostage)[OBYTES] = reinterpret_cast<uint8_t (*)[OBYTES]>(lds + 2 * STAGE_BYTES + NS * XBYTES);
     int (*const flags)[2] = reinterpret_cast<int (*)[2]>(lds + 2 * STAGE_BYTES + NS * (XBYTES + OBYTES));
+    // set by a loader whose wait for a record ran out: from then on this workgroup writes no output
+    volatile int* const wg_failed = reinterpret_cast<volatile int*>(lds + 2 * STAGE_BYTES + NS * (XBYTES + OBYTES) + 48);
 
     const int lane = threadIdx.x % WAVE;
     const int wave = threadIdx.x / WAVE;
@@ -135,6 +137,7 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
     const uint8_t* rec = p.rec + ((int64_t)h * p.TC + slot_begin) * p.rec_bytes;
 
     if (threadIdx.x < NS * 2) flags[threadIdx.x / 2][threadIdx.x % 2] = 0;
+    if (threadIdx.x == WAVE - 1) *wg_failed = 0;
 
     // output staging: the four 16-byte pieces of a row XOR-swizzled with (row / 4) % 4 (conflict-free on both sides)
     auto ostage_at = [&](int sl, int parity, int row, int piece) -> uint8_t* {
@@ -157,6 +160,7 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
         bf16_t* const og = p.o + b * p.o_stride_b + (seq_t0 + row0) * p.o_stride_t + (int64_t)h * p.o_stride_h +
                            32 * (vgroup * NS) + 8 * piece;
         auto flush = [&](int c) {
+            if (WAIT && *wg_failed != 0) return;
             const int valid = (int)min((int64_t)C, seq_len - (int64_t)c * C);
 #pragma unroll
             for (int sl = 0; sl < NS; sl++) {
@@ -244,12 +248,14 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
             }
             if constexpr (reload) load_scalars(sc, c2);
         };
+        bool failed = false;  // this wave's wait ran out (the four loaders poll the same flags, each for itself)
         // output of chunk c: this loader writes tokens 16 lw .. 16 lw + 15 of every slice, 64 bytes per row
         const int o_row = 16 * lw + lane / 4, o_piece = lane % 4;
         bf16_t* const og = p.o + b * p.o_stride_b + (seq_t0 + o_row) * p.o_stride_t + (int64_t)h * p.o_stride_h +
                            32 * (vgroup * NS) + 8 * o_piece;
         auto flush = [&](int c) {
             if constexpr (STORE_WAVE) return;
+            if (WAIT && failed) return;
             const int valid = (int)min((int64_t)C, seq_len - (int64_t)c * C);
             bf16x8 rows[NS];
 #pragma unroll
@@ -271,8 +277,22 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
                     const int32_t got = c + lane < nchunks ? __hip_atomic_load(flag + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 1;
                     const uint64_t pending = __ballot(got == 0);
                     const int n = pending == 0 ? 64 : __builtin_ctzll(pending);
-                    if (n > 0 || spin >= (1u << 22)) {  // bounded: a launch without its prepare half must still end
-                        ready_upto = c + (n > 0 ? n : 1);
+                    if (n > 0) {
+                        ready_upto = c + n;
+                        break;
+                    }
+                    if (spin >= p.spin_limit) {
+                        // Bounded, so that a launch whose prepare half is missing or stuck still ends.  The record is NOT
+                        // there: latch the error where the host finds it (gdn_chunk_fwd_status, gdn_args::error_word),
+                        // stop this workgroup's output, and stop polling (the remaining chunks run on whatever the
+                        // workspace holds; every address stays inside it).
+                        if (lane == 0) {
+                            __hip_atomic_store(p.err, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            if (p.err_caller != nullptr) __hip_atomic_store(p.err_caller, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                            *wg_failed = 1;
+                        }
+                        failed = true;
+                        ready_upto = nchunks;
                         break;
                     }
                     __builtin_amdgcn_s_sleep(32);
@@ -596,7 +616,7 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
         if (nchunks > 0) write_out((nchunks - 1) & 1);
         __syncthreads();  // the loaders write the last output tile
 
-        if (p.ht != nullptr) {
+        if (p.ht != nullptr && !(WAIT && *wg_failed != 0)) {
 #pragma unroll
             for (int t = 0; t < KDH; t++)
 #pragma unroll
@@ -627,6 +647,7 @@ __global__ __launch_bounds__(PAIR_THREADS) void chunk_fused_kernel(const ChunkPa
         scan_pair_body<K, NS, true>(p, lds, (int)blockIdx.x - prep_wgs);  // prep_wgs is a multiple of 8: same XCD numbering
         return;
     }
+    if (p.no_producers) return;  // GDN_FLAG_DEBUG_NO_PRODUCERS: the scan's waits run out
     // producer: items of XCD x are (chunk c, chain) for the chains x * per_xcd .. the scan puts on that XCD, chunk-major
     const int xcd = blockIdx.x % 8, rank = blockIdx.x / 8, per = prep_wgs / 8;
     const int chains = p.N * p.H, per_xcd = (chains + 7) / 8;
@@ -661,12 +682,10 @@ static int launch_fused_k(ChunkParams& p, hipStream_t stream, int num_cus) {
     p.scan_groups = p.V / 64;
     const int64_t scan_wgs = chains8 * p.scan_groups;
     const int prep_wgs = (int)((num_cus - scan_wgs) / 8 * 8);
-    // Worth it only when the scan fills about half of the CUs: with fewer chains the two-kernel path's scan, one slice per
-    // CU, is the faster one and prepare is short; with more, too few CUs are left for the producers.
-    if (scan_wgs > (int64_t)num_cus / 2 || scan_wgs < (int64_t)num_cus * 3 / 8) return GDN_ERR_UNSUPPORTED;
+    if (!fused_launch_window((int64_t)p.N * p.H, p.V, num_cus)) return GDN_ERR_UNSUPPORTED;
     if (!p.ready_clear) {  // the scan waits for flags the producers set: they must start at zero (and end there: scan_pair_body)
-        const int64_t nflags = (int64_t)p.H * p.TC;
-        hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((nflags + 255) / 256 < 64 ? (nflags + 255) / 256 : 64)), dim3(256), 0, stream, p.ready, nflags);
+        const int64_t nflags = (int64_t)p.H * p.TC + 1;  // with the error latch, the word in front of them
+        hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((nflags + 255) / 256 < 64 ? (nflags + 255) / 256 : 64)), dim3(256), 0, stream, p.ready - 1, nflags);
         if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
     }
     hipLaunchKernelGGL((chunk_fused_kernel<K, 2>), dim3((unsigned)(prep_wgs + scan_wgs)), dim3(PAIR_THREADS), 0, stream, p, prep_wgs);
@@ -674,7 +693,7 @@ static int launch_fused_k(ChunkParams& p, hipStream_t stream, int num_cus) {
 }
 
 bool chunk_fused_supported(const ChunkParams& p, int K) {
-    return (K == 64 || K == 128) && p.V % 64 == 0 && p.cu_seqlens == nullptr && p.pad_lens == nullptr && p.ready != nullptr &&
+    return (K == 64 || K == 128) && p.V % 64 == 0 && p.cu_seqlens == nullptr && p.pad_lens == nullptr && p.ready != nullptr && p.err == p.ready - 1 &&
            !p.records_given && p.save_state == nullptr && p.save_vnew == nullptr;
 }
 

@@ -14,7 +14,10 @@ int launch_recurrent(const gdn_args& a, hipStream_t stream);
 int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events = nullptr, const gdn_chunk_saves* saves = nullptr);
 uint64_t chunk_workspace_bytes(const gdn_args& a);
 uint64_t chunk_record_bytes(const gdn_args& a);  // the records alone, [H][chunk slots]
+uint64_t chunk_header_bytes(const gdn_args& a);  // what precedes the records: chunk offsets, error latch, ready flags
+uint64_t chunk_error_latch_offset(const gdn_args& a);  // byte offset of the error latch (an int32) in the workspace
 bool chunk_shape_supported(const gdn_args& a);
+bool chunk_runs_as_one_launch(const gdn_args& a);  // gdn_chunk_fwd would run prepare and scan as one launch (shape fields, flags, cu_seqlens)
 int launch_chunk_bwd_local(const gdn_chunk_local_args& a, hipStream_t stream);  // gdn_chunk_bwd.hip
 bool chunk_bwd_local_supported(const gdn_chunk_local_args& a);
 int launch_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args& a, hipStream_t stream);

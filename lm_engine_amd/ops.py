@@ -25,6 +25,7 @@ call raises.  Both are differentiable (``backward.py``).
 from __future__ import annotations
 
 import ctypes
+import threading
 from collections import OrderedDict
 
 import torch
@@ -128,30 +129,93 @@ def _fill_args(q, k, v, g, beta, h0, ht, o, cu_seqlens, scale, l2norm, inplace, 
     return a
 
 
-# Workspaces of the chunked forward, kept between calls: one per (device, stream, shape), zero-filled when it is made.
-# The library then need not clear the ready flags of its one-launch mode before every call (it leaves them clear
-# itself, GDN_FLAG_READY_FLAGS_CLEAR), and a step no longer asks the allocator for tens of megabytes.  Calls on one
-# stream run in order, so they can share a workspace; another stream gets its own.  The least recently used entries
-# go when there are more than _WORKSPACE_LIMIT; release_workspaces() drops them all.
+# Workspaces of the one-launch chunked forward, kept between calls: one per (device, stream, shape), its header
+# (chunk offsets, error latch, ready flags) zero-filled when it is made.  The library then need not clear the ready flags
+# before every call (it leaves them clear itself, GDN_FLAG_READY_FLAGS_CLEAR), and a step of that shape no longer asks
+# the allocator for tens of megabytes.  Only shapes that run as one launch keep a workspace: every other call (packed
+# or left-padded batches, K = 256, shapes outside the window) reads no flag and takes a fresh torch.empty workspace
+# from the caching allocator, whatever T it comes with.  Calls on one stream run in order, so they can share a
+# workspace; another stream gets its own.  The least recently used entries go when there are more than
+# _WORKSPACE_LIMIT of them or they hold more than _WORKSPACE_BYTES_LIMIT together; release_workspaces() drops them
+# all.  The dict is guarded by a lock: forward passes on several Python threads (one stream each) may interleave.
 _WORKSPACES: "OrderedDict[tuple, torch.Tensor]" = OrderedDict()
 _WORKSPACE_LIMIT = 8
+_WORKSPACE_BYTES_LIMIT = 1 << 30
+_WORKSPACES_LOCK = threading.Lock()
+
+# One pinned int32 per device that the one-launch forward sets when a scan workgroup gave up waiting for a record
+# (gdn_args::error_word).  The host reads it without synchronising, before every chunked forward on that device: a
+# failure of an earlier call surfaces at the next one, the way asynchronous device errors do.
+_ERROR_WORDS: dict[int, torch.Tensor] = {}
 
 
 def release_workspaces() -> None:
     """Frees the workspaces that ``chunk_gated_delta_rule`` keeps between calls."""
-    _WORKSPACES.clear()
+    with _WORKSPACES_LOCK:
+        _WORKSPACES.clear()
 
 
-def _kept_workspace(device, stream_handle, dims, packed, nbytes):
-    key = (device.index, stream_handle, dims, packed, nbytes)
-    workspace = _WORKSPACES.get(key)
-    if workspace is None:
-        workspace = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+def _error_word(device) -> torch.Tensor:
+    word = _ERROR_WORDS.get(device.index)
+    if word is None:
+        word = torch.zeros(1, dtype=torch.int32).pin_memory()
+        _ERROR_WORDS[device.index] = word
+    return word
+
+
+def _raise_if_forward_failed(device) -> torch.Tensor:
+    """The error word of ``device``; raises when an earlier one-launch forward on it reported a time-out (the kept
+    workspaces of that device are dropped: their ready flags are in no defined state)."""
+    word = _error_word(device)
+    if int(word[0]) != 0:
+        word.zero_()
+        with _WORKSPACES_LOCK:
+            for key in [k for k in _WORKSPACES if k[0] == device.index]:
+                del _WORKSPACES[key]
+        raise RuntimeError(
+            "an earlier chunk_gated_delta_rule call on this device gave up waiting for its prepare half "
+            "(gdn_chunk_fwd, one-launch mode): the outputs of that call are invalid"
+        )
+    return word
+
+
+def _kept_workspace(device, stream_handle, dims, nbytes, header_bytes):
+    key = (device.index, stream_handle, dims, nbytes)
+    with _WORKSPACES_LOCK:
+        workspace = _WORKSPACES.get(key)
+        if workspace is not None:
+            _WORKSPACES.move_to_end(key)
+            return key, workspace
+    workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    workspace[:header_bytes].zero_()
+    with _WORKSPACES_LOCK:
         _WORKSPACES[key] = workspace
-        while len(_WORKSPACES) > _WORKSPACE_LIMIT:
+        while len(_WORKSPACES) > _WORKSPACE_LIMIT or (
+            len(_WORKSPACES) > 1 and sum(w.numel() for w in _WORKSPACES.values()) > _WORKSPACE_BYTES_LIMIT
+        ):
             _WORKSPACES.popitem(last=False)
+    return key, workspace
+
+
+def _drop_workspace(key) -> None:
+    with _WORKSPACES_LOCK:
+        _WORKSPACES.pop(key, None)
+
+
+def _chunk_workspace(lib, args, q, dims, stream_handle):
+    """Workspace for one ``gdn_chunk_fwd`` call: fills ``args.workspace`` / ``workspace_bytes`` (and the flag that vouches
+    for clear ready flags when the workspace is a kept one).  Returns ``(key, tensor)``; ``key`` is None for a
+    workspace that is not kept."""
+    nbytes = max(int(lib.gdn_workspace_bytes(ctypes.byref(args))), 256)
+    # (memory allocated under graph capture belongs to the graph: nothing of it is kept)
+    keep = bool(lib.gdn_chunk_fwd_is_one_launch(ctypes.byref(args))) and not torch.cuda.is_current_stream_capturing()
+    if keep:
+        header = int(lib.gdn_workspace_header_bytes(ctypes.byref(args)))
+        key, workspace = _kept_workspace(q.device, stream_handle, dims, nbytes, header)
+        args.flags |= _lib.GDN_FLAG_READY_FLAGS_CLEAR
     else:
-        _WORKSPACES.move_to_end(key)
+        key, workspace = None, torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+    args.workspace, args.workspace_bytes = workspace.data_ptr(), workspace.numel()
     return key, workspace
 
 
@@ -188,18 +252,12 @@ def _run(mode, q, k, v, g, beta, scale, initial_state, output_final_state, cu_se
 
     with torch.cuda.device(q.device):
         if mode == "chunk":
-            nbytes = max(int(lib.gdn_workspace_bytes(ctypes.byref(args))), 256)
-            if torch.cuda.is_current_stream_capturing():
-                # memory allocated under graph capture belongs to the graph: nothing of it is kept
-                key, workspace = None, torch.empty(nbytes, dtype=torch.uint8, device=q.device)
-            else:
-                key, workspace = _kept_workspace(q.device, stream.value, dims, cu_seqlens is not None, nbytes)
-                args.flags |= _lib.GDN_FLAG_READY_FLAGS_CLEAR
-            args.workspace, args.workspace_bytes = workspace.data_ptr(), workspace.numel()
+            args.error_word = _raise_if_forward_failed(q.device).data_ptr()
+            key, workspace = _chunk_workspace(lib, args, q, dims, stream.value)
             try:
                 _lib.check_status(lib.gdn_chunk_fwd(ctypes.byref(args), stream), "gdn_chunk_fwd")
             except Exception:
-                _WORKSPACES.pop(key, None)  # a call that failed may have left flags set
+                _drop_workspace(key)  # a call that failed may have left flags set
                 raise
         else:
             _lib.check_status(lib.gdn_recurrent_fwd(ctypes.byref(args), stream), "gdn_recurrent_fwd")
@@ -213,13 +271,12 @@ def fused_launch_applies(q, v, cu_seqlens=None) -> bool:
     rounded up to a multiple of 8) fill between 3/8 and 1/2 of the compute units."""
     if not is_kernel_allowed(Kernel.gated_delta_rule_fused_launch) or cu_seqlens is not None or q.dtype != torch.bfloat16:
         return False
-    B, _, H, K = q.shape
-    V = v.size(-1)
-    if K not in (64, 128) or V % 64 != 0:
-        return False
-    cus = torch.cuda.get_device_properties(q.device).multi_processor_count
-    scan_workgroups = (B * H + 7) // 8 * 8 * (V // 64)
-    return cus * 3 // 8 <= scan_workgroups <= cus // 2
+    B, T, H, K = q.shape
+    a = _lib.GdnArgs()  # the library decides (gdn_chunk_fwd_is_one_launch): shape fields and flags are all it reads
+    a.B, a.T, a.H, a.K, a.V, a.N = B, T, H, K, v.size(-1), B
+    a.chunk, a.dtype, a.flags = 64, _lib.GDN_BF16, _lib.GDN_FLAG_FUSED_LAUNCH
+    with torch.cuda.device(q.device):
+        return bool(_lib.load_library().gdn_chunk_fwd_is_one_launch(ctypes.byref(a)))
 
 
 def chunk_forward_kernel_times(
@@ -245,14 +302,12 @@ def chunk_forward_kernel_times(
     with torch.cuda.device(q.device):
         # the same kept workspace, and the same promise about its flags, as the operator itself
         stream = ctypes.c_void_p(torch.cuda.current_stream(q.device).cuda_stream)
-        nbytes = max(int(lib.gdn_workspace_bytes(ctypes.byref(args))), 256)
-        key, workspace = _kept_workspace(q.device, stream.value, dims, cu_seqlens is not None, nbytes)
-        args.flags |= _lib.GDN_FLAG_READY_FLAGS_CLEAR
-        args.workspace, args.workspace_bytes = workspace.data_ptr(), workspace.numel()
+        args.error_word = _raise_if_forward_failed(q.device).data_ptr()
+        key, workspace = _chunk_workspace(lib, args, q, dims, stream.value)
         try:
             _lib.check_status(lib.gdn_chunk_fwd_profile(ctypes.byref(args), stream, times), "gdn_chunk_fwd_profile")
         except Exception:
-            _WORKSPACES.pop(key, None)
+            _drop_workspace(key)
             raise
     return dict(zip(_lib.CHUNK_KERNEL_NAMES, (float(x) for x in times)))
 

@@ -181,7 +181,6 @@ def test_left_padded_batch_equals_separate_runs(K, V):
             assert torch.equal(ht[b], gpu["initial_state"][b])
             continue
         one = {name: x[b : b + 1, T - n :] for name, x in gpu.items() if name != "initial_state"}
-        fn = lm_engine_amd.chunk_gated_delta_rule if n > 64 else lm_engine_amd.fused_recurrent_gated_delta_rule
         o_b, h_b = lm_engine_amd.chunk_gated_delta_rule(**one, initial_state=gpu["initial_state"][b : b + 1], output_final_state=True)
         assert torch.equal(o[b : b + 1, T - n :], o_b), f"row {b}: padded-batch and separate outputs differ"
         assert torch.equal(ht[b : b + 1], h_b)

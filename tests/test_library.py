@@ -45,6 +45,7 @@ def test_struct_layout_matches_the_header():
         printf("%zu %zu %zu %zu %zu %zu %zu\n", sizeof(gdn_args), offsetof(gdn_args, workspace_bytes),
                offsetof(gdn_args, q_stride_b), offsetof(gdn_args, o_stride_h), offsetof(gdn_args, B),
                offsetof(gdn_args, flags), offsetof(gdn_args, scale));
+        printf("%zu %zu\n", offsetof(gdn_args, spin_limit), offsetof(gdn_args, error_word));
         printf("%zu %zu %zu %zu %zu\n", sizeof(gdn_conv_args), offsetof(gdn_conv_args, final_state),
                offsetof(gdn_conv_args, x_stride_b), offsetof(gdn_conv_args, B), offsetof(gdn_conv_args, activation));
         return 0;
@@ -58,7 +59,7 @@ def test_struct_layout_matches_the_header():
     A = _lib.GdnArgs
     Cv = _lib.GdnConvArgs
     assert values == [ctypes.sizeof(A), A.workspace_bytes.offset, A.q_stride_b.offset, A.o_stride_h.offset,
-                      A.B.offset, A.flags.offset, A.scale.offset,
+                      A.B.offset, A.flags.offset, A.scale.offset, A.spin_limit.offset, A.error_word.offset,
                       ctypes.sizeof(Cv), Cv.final_state.offset, Cv.x_stride_b.offset, Cv.B.offset,
                       Cv.activation.offset]  # fmt: skip
 
