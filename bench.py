@@ -485,6 +485,7 @@ def bench_backward(w, inp, steps, warmup):
     import torch
 
     from lm_engine_amd.backward import gated_delta_rule_backward
+    from lm_engine_amd.ops import backward_kernels_apply
 
     gen = torch.Generator("cpu").manual_seed(555)
     do = torch.randn(inp["v"].shape, generator=gen).to(inp["v"].dtype).cuda()
@@ -506,7 +507,7 @@ def bench_backward(w, inp, steps, warmup):
         "ms_per_backward": round(ms, 3),
         "tokens_per_s": round(w.B * w.T / (ms * 1e-3), 1),
         "composition": ("5 kernel launches: backward prepare, forward prepare + saving scan, saving scan over the "
-                        "mirror problem, chunk-local gradients" if w.K == 128 and w.V in (128, 256, 512) else
+                        "mirror problem, chunk-local gradients" if backward_kernels_apply(w.K, w.V) else
                         "2 saving scans + rocBLAS batched GEMMs + elementwise torch ops"),
     }
 

@@ -209,51 +209,46 @@ int gdn_chunk_fwd_saving(const gdn_args *args, const gdn_chunk_saves *saves, voi
 /*
  * Training support, second part: the chunk-local gradients, one workgroup per (sequence, head, chunk), once
  * the two sweeps over the chunks (gdn_chunk_fwd_saving, forward and mirrored) have delivered per chunk the
- * state it starts from, the gradient of the state it ends with, V~ and Y = T^T dV~.  All arrays fp32,
- * contiguous, chunk-major ("packed": sequences padded with zeros to whole chunks):
- *     qs, kn        [chunks][64][K]   q normalised and scaled, k normalised
- *     v, dout, y, v_new  [chunks][64][V]
- *     states, dstates    [chunks][K][V]
- *     gamma, beta   [chunks][64]      prefix sum of g inside the chunk, beta
+ * state it starts from, the gradient of the state it ends with, V~ and Y = T^T dV~.  Chunk index
+ * = (n * H + h) * NC + c; per-chunk arrays are contiguous and chunk-major:
+ *     v_new         [chunks][64][V]   V~, in saves_dtype (what gdn_chunk_fwd_saving wrote)
+ *     states        [chunks][K][V]    the state a chunk starts from, in saves_dtype
+ *     dstates       [chunks][K][V]    the gradient of the state it ends with, fp32
+ *     gamma, beta   [chunks][64]      prefix sum of g inside the chunk, beta (fp32; from gdn_chunk_bwd_prepare)
  *     rq, rk        [chunks][64]      1 / sqrt(|q|^2 + 1e-6), likewise for k, when q and k were normalised
  *                                     (the l2norm flag of the forward); both NULL otherwise
- * qs = scale * q (* rq), kn = k (* rk).  Outputs: dq, dk [chunks][64][K], the gradients with respect to q and
- * k themselves (through the scale and the normalisation), dbeta [chunks][64], and dgamma [chunks][64], the
- * gradient with respect to gamma (dg is its reverse prefix sum inside the chunk).
- * K = 128 with V = 128, 256 or 512 only (GDN_ERR_UNSUPPORTED otherwise).  Counterpart upstream: the chunk-local kernels of fla's
- * backward of chunk_gated_delta_rule, reached from gated_deltanet/module.py:197-209 under autograd.
+ *     y_mirror      bf16 [N, 2 * NC * 64, H, V]: the output of the scan over the mirror problem of
+ *                   gdn_chunk_bwd_prepare (Y at its even chunks, tokens reversed)
+ *     q_raw, k_raw, v_raw, dout_raw   the caller's bf16 q, k, v, dO, [N, NC * 64, H, D] with element strides
+ * Outputs, in the caller's layout, contiguous: dq_out, dk_out [N, NC * 64, H, K] and dv_out [N, NC * 64, H, V]
+ * (bf16; the gradients with respect to q and k themselves, through the scale and the normalisation), dg_out and
+ * dbeta_out fp32 [N, NC * 64, H] (dg_out is the gradient with respect to g: the reverse prefix sum of the gradient
+ * with respect to gamma inside the chunk).
+ * K = 64, 128 or 256 and V a multiple of 64 (GDN_ERR_UNSUPPORTED otherwise).  Counterpart upstream: the chunk-local
+ * kernels of fla's backward of chunk_gated_delta_rule, reached from gated_deltanet/module.py:197-209 under autograd.
  */
 typedef struct gdn_chunk_local_args {
-    const float *qs, *kn, *v, *dout, *y, *v_new, *states, *dstates, *gamma, *beta, *rq, *rk;
-    float *dq, *dk, *dbeta, *dgamma;
+    const void *v_new, *states;
+    const float *dstates, *gamma, *beta, *rq, *rk;
+    int32_t saves_dtype; /* gdn_dtype of v_new and states */
+    float scale;
     int64_t chunks;
     int32_t K, V;
-    float scale;
-    int32_t reserved;
-    /*
-     * "Final" mode, for batches of whole chunks (chunk index = (n * H + h) * NC + c), when y_mirror != NULL:
-     * Y is read from the output of the scan over the mirror problem of gdn_chunk_bwd_prepare
-     * (bf16 [N, 2 * NC * 64, H, V]) instead of `y`, and the gradients are written in the caller's layout instead
-     * of dq, dk, dbeta, dgamma: dq_out, dk_out [N, NC * 64, H, K] and dv_out [N, NC * 64, H, V] = beta Y (bf16,
-     * contiguous), dg_out and dbeta_out fp32 [N, NC * 64, H] (dg_out is the gradient with respect to g).
-     */
     const void *y_mirror;
     void *dq_out, *dk_out, *dv_out;
     float *dg_out, *dbeta_out;
     int32_t H, NC;
-    /* final mode reads the caller's bf16 q, k, v, dout ([N, NC * 64, H, D], element strides) instead of qs, kn, v,
-     * dout, which may then be NULL; rq and rk (or NULL), gamma, beta stay packed fp32 */
     const void *q_raw, *k_raw, *v_raw, *dout_raw;
     int64_t q_stride_b, q_stride_t, q_stride_h;
     int64_t k_stride_b, k_stride_t, k_stride_h;
     int64_t v_stride_b, v_stride_t, v_stride_h;
     int64_t dout_stride_b, dout_stride_t, dout_stride_h;
-    /* final mode for packed or left-padded batches: sequence n starts at token seq_start[n] (a flat index over the
+    /* packed or left-padded batches: sequence n starts at token seq_start[n] (a flat index over the
      * rows of the caller's tensors, T_rows tokens per row) and has seq_len[n] tokens; its chunks c * 64 >= seq_len[n]
      * are skipped, tokens past its end are not written.  NULL: sequence n is row n, NC * 64 tokens. */
     const int32_t *seq_start, *seq_len;
     int32_t T_rows;
-    int32_t reserved2;
+    int32_t reserved;
 } gdn_chunk_local_args;
 int gdn_chunk_bwd_local(const gdn_chunk_local_args *args, void *stream);
 
@@ -261,7 +256,7 @@ int gdn_chunk_bwd_local(const gdn_chunk_local_args *args, void *stream);
  * Training support, third part: everything the backward needs per chunk before its two sweeps (batches of
  * whole chunks: T a multiple of 64, one sequence per row; other batches through seq_start / seq_len below;
  * bf16 q, k, dout as [N, T, H, D] with element
- * strides; K = 128 and V = 128, 256 or 512, GDN_ERR_UNSUPPORTED otherwise).  One workgroup per (sequence, head, chunk) writes
+ * strides; K = 64, 128 or 256 and V a multiple of 64, GDN_ERR_UNSUPPORTED otherwise).  One workgroup per (sequence, head, chunk) writes
  *   - gamma, beta_packed, rq, rk: fp32 [N H T/64][64], operands of gdn_chunk_bwd_local;
  *   - the reverse sweep as a forward scan over 2 T tokens per sequence ("mirror" problem: tokens in reverse
  *     order, chunk c becomes chunks 2 r and 2 r + 1, r = T/64 - 1 - c): k_mirror [N, 2 T, H, K] and

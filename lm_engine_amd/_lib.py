@@ -69,17 +69,16 @@ class GdnChunkSaves(ctypes.Structure):
 
 
 class GdnChunkLocalArgs(ctypes.Structure):
-    _fields_ = [(name, ctypes.c_void_p) for name in (
-        "qs", "kn", "v", "dout", "y", "v_new", "states", "dstates", "gamma", "beta", "rq", "rk",
-        "dq", "dk", "dbeta", "dgamma",
-    )] + [("chunks", ctypes.c_int64), ("K", ctypes.c_int32), ("V", ctypes.c_int32), ("scale", ctypes.c_float),
-          ("reserved", ctypes.c_int32)] + [(name, ctypes.c_void_p) for name in (
-        "y_mirror", "dq_out", "dk_out", "dv_out", "dg_out", "dbeta_out",
-    )] + [("H", ctypes.c_int32), ("NC", ctypes.c_int32)] + [(name, ctypes.c_void_p) for name in (
-        "q_raw", "k_raw", "v_raw", "dout_raw",
-    )] + [(f"{x}_stride_{d}", ctypes.c_int64) for x in ("q", "k", "v", "dout") for d in ("b", "t", "h")] + [
-        ("seq_start", ctypes.c_void_p), ("seq_len", ctypes.c_void_p), ("T_rows", ctypes.c_int32), ("reserved2", ctypes.c_int32),
-    ]  # fmt: skip
+    _fields_ = (
+        [(name, ctypes.c_void_p) for name in ("v_new", "states", "dstates", "gamma", "beta", "rq", "rk")]
+        + [("saves_dtype", ctypes.c_int32), ("scale", ctypes.c_float), ("chunks", ctypes.c_int64), ("K", ctypes.c_int32),
+           ("V", ctypes.c_int32)]
+        + [(name, ctypes.c_void_p) for name in ("y_mirror", "dq_out", "dk_out", "dv_out", "dg_out", "dbeta_out")]
+        + [("H", ctypes.c_int32), ("NC", ctypes.c_int32)]
+        + [(name, ctypes.c_void_p) for name in ("q_raw", "k_raw", "v_raw", "dout_raw")]
+        + [(f"{x}_stride_{d}", ctypes.c_int64) for x in ("q", "k", "v", "dout") for d in ("b", "t", "h")]
+        + [("seq_start", ctypes.c_void_p), ("seq_len", ctypes.c_void_p), ("T_rows", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+    )  # fmt: skip
 
 
 class GdnChunkBwdPrepareArgs(ctypes.Structure):

@@ -286,10 +286,10 @@ def _sweeps_on_scan_kernel(q, k, v, do, g, beta, scale, initial_state, cu_seqlen
     return S0, Vn, dS1, Y, dS.reshape(Bt, K, V)
 
 
-def _chunk_local_kv():
+def _kernels_apply(K, V):
     from . import ops  # late: ops imports this module
 
-    return ops.CHUNK_LOCAL_KV
+    return ops.backward_kernels_apply(K, V)
 
 
 def _chunk_local_grads(qs, kn, vc, doc, Y, Vn, S0, dS1, gam, bc):
@@ -355,7 +355,7 @@ def _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, l2norm
         sequences = (as_i32(starts), as_i32(lens), NC)
     Bt = N * H
     q, k, v, do = (x if x.stride(-1) == 1 else x.contiguous() for x in (q, k, v, do.to(torch.bfloat16)))
-    half_slices = ops.half_slice_records_pay(Bt, V, dev)
+    half_slices = K > 128 or ops.half_slice_records_pay(Bt, V, dev)  # K = 256 scans on half-slice waves only
     prep = ops.chunk_bwd_prepare(q, k, do, g, beta, scale, l2norm, V, sequences, half_slice_records=half_slices)
     S0 = torch.empty(Bt, NC, K, V, device=dev)
     Vn = torch.empty(Bt, NC, CHUNK, V, device=dev)
@@ -364,7 +364,7 @@ def _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, l2norm
     dht32 = None if dht is None else dht.to(torch.float32).contiguous()
     o_m, dS = ops.chunk_scan_given_records(prep["k_mirror"], prep["v_mirror"], prep["records"], dht32, dS1, NC,
                                            save_every=2, save_reverse=True, half_slice_records=half_slices)  # fmt: skip
-    dq, dk, dv, dg, dbeta = ops.chunk_local_grads_final(q, k, v, do, prep, o_m, Vn, S0, dS1, scale, l2norm, sequences)
+    dq, dk, dv, dg, dbeta = ops.chunk_local_grads(q, k, v, do, prep, o_m, Vn, S0, dS1, scale, l2norm, sequences)
     return (
         dq,
         dk,
@@ -389,7 +389,7 @@ def gated_delta_rule_backward(
     V = v.size(-1)
     dev = q.device
     scale = K**-0.5 if scale is None else scale
-    if q.is_cuda and q.dtype == torch.bfloat16 and (K, V) in _chunk_local_kv():
+    if q.is_cuda and q.dtype == torch.bfloat16 and _kernels_apply(K, V):
         return _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, use_qk_l2norm_in_kernel,
                                     cu_seqlens, left_padded)  # fmt: skip
     pk = _Packing(B, T, H, cu_seqlens, left_padded, dev)
@@ -445,18 +445,12 @@ def gated_delta_rule_backward(
         )  # fmt: skip
     dh0 = dS.reshape(N, H, K, V) if initial_state is not None else None
 
-    if on_kernel and (K, V) in _chunk_local_kv():
-        from . import ops
-
-        norms = dict(rq=rq[..., 0], rk=rk[..., 0]) if use_qk_l2norm_in_kernel else {}
-        dqc, dkc, dbc, dgam = ops.chunk_local_grads(qs, kn, vc, doc, Y, Vn, S0, dS1, gam, bc, scale, **norms)
+    dqs, dkn, dbc, dgam = _chunk_local_grads(qs, kn, vc, doc, Y, Vn, S0, dS1, gam, bc)
+    dqn = dqs * scale
+    if use_qk_l2norm_in_kernel:
+        dqc, dkc = _l2norm_grad(qn, rq, dqn), _l2norm_grad(kn, rk, dkn)
     else:
-        dqs, dkn, dbc, dgam = _chunk_local_grads(qs, kn, vc, doc, Y, Vn, S0, dS1, gam, bc)
-        dqn = dqs * scale
-        if use_qk_l2norm_in_kernel:
-            dqc, dkc = _l2norm_grad(qn, rq, dqn), _l2norm_grad(kn, rk, dkn)
-        else:
-            dqc, dkc = dqn, dkn
+        dqc, dkc = dqn, dkn
     dvc = Y * bc[..., None]
     dgc = dgam.flip(-1).cumsum(-1).flip(-1)
     return (

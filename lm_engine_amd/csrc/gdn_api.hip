@@ -190,29 +190,18 @@ int gdn_chunk_fwd_saving(const gdn_args* a, const gdn_chunk_saves* saves, void* 
 
 int gdn_chunk_bwd_local(const gdn_chunk_local_args* a, void* stream) {
     if (a == nullptr) return GDN_ERR_NULL;
-    const bool final_mode = a->y_mirror != nullptr;
-    const void* common[] = {a->v_new, a->states, a->dstates, a->gamma, a->beta};
-    const void* packed[] = {a->qs, a->kn, a->v, a->dout, a->y, a->dq, a->dk, a->dbeta, a->dgamma};
-    const void* final_[] = {a->y_mirror, a->dq_out, a->dk_out, a->dv_out, a->dg_out, a->dbeta_out,
-                            a->q_raw, a->k_raw, a->v_raw, a->dout_raw};
-    for (const void* x : common)
+    const void* needed[] = {a->v_new, a->states, a->dstates, a->gamma, a->beta, a->y_mirror, a->dq_out, a->dk_out,
+                            a->dv_out, a->dg_out, a->dbeta_out, a->q_raw, a->k_raw, a->v_raw, a->dout_raw};
+    for (const void* x : needed)
         if (x == nullptr) return GDN_ERR_NULL;
         else if (!aligned(x, 16)) return GDN_ERR_ALIGN;
-    if (final_mode) {
-        for (const void* x : final_)
-            if (x == nullptr) return GDN_ERR_NULL;
-            else if (!aligned(x, 16)) return GDN_ERR_ALIGN;
-        if (a->H <= 0 || a->NC <= 0 || a->chunks % ((int64_t)a->H * a->NC) != 0) return GDN_ERR_SHAPE;
-        if (a->seq_start != nullptr && (a->seq_len == nullptr || a->T_rows <= 0)) return GDN_ERR_SHAPE;
-        const int64_t raw_strides[] = {a->q_stride_b, a->q_stride_t, a->q_stride_h, a->k_stride_b, a->k_stride_t, a->k_stride_h,
-                                       a->v_stride_b, a->v_stride_t, a->v_stride_h, a->dout_stride_b, a->dout_stride_t, a->dout_stride_h};
-        for (int64_t st : raw_strides)
-            if (st < 0 || st % 8 != 0) return GDN_ERR_ALIGN;
-    } else {
-        for (const void* x : packed)
-            if (x == nullptr) return GDN_ERR_NULL;
-            else if (!aligned(x, 16)) return GDN_ERR_ALIGN;
-    }
+    if (a->saves_dtype != GDN_BF16 && a->saves_dtype != GDN_F32) return GDN_ERR_UNSUPPORTED;
+    if (a->H <= 0 || a->NC <= 0 || a->chunks % ((int64_t)a->H * a->NC) != 0) return GDN_ERR_SHAPE;
+    if (a->seq_start != nullptr && (a->seq_len == nullptr || a->T_rows <= 0)) return GDN_ERR_SHAPE;
+    const int64_t raw_strides[] = {a->q_stride_b, a->q_stride_t, a->q_stride_h, a->k_stride_b, a->k_stride_t, a->k_stride_h,
+                                   a->v_stride_b, a->v_stride_t, a->v_stride_h, a->dout_stride_b, a->dout_stride_t, a->dout_stride_h};
+    for (int64_t st : raw_strides)
+        if (st < 0 || st % 8 != 0) return GDN_ERR_ALIGN;
     if ((a->rq == nullptr) != (a->rk == nullptr)) return GDN_ERR_NULL;
     if (a->rq != nullptr && (!aligned(a->rq, 4) || !aligned(a->rk, 4))) return GDN_ERR_ALIGN;
     if (!(a->scale > 0.f)) return GDN_ERR_SHAPE;

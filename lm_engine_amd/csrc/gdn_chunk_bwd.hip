@@ -18,12 +18,22 @@
 //                + e_i <dQe_i, Q_i> - tail_i <dKd_i, K_i> - beta_i e_i <Z_i, K_i>
 //     dgamma_C += exp(gamma_C) <dS1, S0> + sum_i tail_i <dKd_i, K_i>
 //
-// Every matrix product is an "A B^T" of two row-major bf16 matrices staged in LDS (the transposes of Q and K
-// are staged next to them), on 32x32x16 MFMA with fp32 accumulation.  The 64 x K results are kept transposed
-// ([key dim][token]) so that a lane owns one token: the per-token scales are per-lane scalars and the sums
-// over the key dim stay inside a lane.  Built for K = 128 and V = 128, 256 or 512 (the value dim is staged 128 columns
-// at a time; 157 KiB of LDS: one workgroup per CU).
+// Every matrix product is an "A B^T" of two row-major bf16 matrices staged in LDS, on 32x32x16 MFMA with fp32
+// accumulation.  The 64 x K results are kept transposed ([key dim][token]) so that a lane owns one token: the
+// per-token scales are per-lane scalars and the sums over the key dim stay inside a lane.
+//
+// Three phases share one LDS buffer of 64.5 KiB at most, so that two workgroups fit a CU and one's loads run beside
+// the other's products (K <= 128; K = 256 holds its 64 x K results for both key halves in registers and takes a CU
+// to itself by its register count):
+//   1. over the value dim in slabs of 64 columns: dO, Y, V~ and the slab of S0, then of dS1, staged; the products
+//      with the states and the two 64 x 64 products that contract over the value dim accumulate;
+//   2. the rows of q and k (128 keys at a time) for Q K^T and K K^T, then the 64 x 64 stage: G, G^T and Hm + Hm^T
+//      are left in LDS;
+//   3. per 128 keys: the transposes of q and k staged, the per-token sums over the key dim, dQ^T and dK^T.
+// K = 64, 128, 256; V a multiple of 64.
 #include <hip/hip_runtime.h>
+
+#include <type_traits>
 
 #include "gdn_chunk_common.h"
 #include "gdn_launch.h"
@@ -32,34 +42,23 @@ namespace gdn {
 
 namespace {
 
-constexpr int BWD_K = 128;  // the kernels of this file are built for K = 128 and V = 128, 256 or 512
 constexpr int BWD_THREADS = 256;
-constexpr int LDR = 136;  // bf16 per LDS row of a [.][128] matrix: 16 bytes of padding
-constexpr int LDS64 = 72;  // bf16 per LDS row of a [.][64] matrix
+constexpr int LDS64 = 72;  // bf16 per LDS row of a [.][64] matrix: 16 bytes of padding
 
 struct ChunkLocalParams {
-    const float* qs;
-    const float* kn;
-    const float* v;
-    const float* dout;
-    const float* y;
-    const float* vnew;
-    const float* s0;
-    const float* ds1;
+    const void* vnew;   // V~ [chunk][64][V], fp32 or bf16 (saves_bf16)
+    const void* s0;     // S0 [chunk][K][V], fp32 or bf16 (saves_bf16)
+    const float* ds1;   // dS1 [chunk][K][V]
+    int saves_bf16;
     const float* gam;
     const float* beta;
     const float* rq;  // 1 / |q|, 1 / |k| per token when q and k were normalised, else NULL
     const float* rk;
     float scale;
-    float* dq;
-    float* dk;
-    float* dbeta;
-    float* dgam;
-    // "final" mode (whole-chunk batches; chunk = (n H + h) NC + c): Y is read from the output of the scan over
-    // the mirror problem, and the gradients go out in the caller's layout, [N, NC 64, H, .] bf16 for q, k, v and
-    // fp32 [N, NC 64, H] for g (reverse prefix sum of dgamma done here) and beta
-    const bf16_t* y_mirror;  // [N][2 NC 64][H][V], NULL = packed mode
-    // final mode reads the caller's q, k, v, dO (bf16, element strides) instead of the packed qs, kn, v, dout
+    // chunk = (n H + h) NC + c.  Y is read from the output of the scan over the mirror problem; q, k, v, dO are the
+    // caller's tensors (bf16, element strides); the gradients go out in the caller's layout, [N, NC 64, H, .] bf16
+    // for q, k, v and fp32 [N, NC 64, H] for g (reverse prefix sum of dgamma done here) and beta
+    const bf16_t* y_mirror;  // [N][2 NC 64][H][V]
     const bf16_t* q_raw;
     const bf16_t* k_raw;
     const bf16_t* v_raw;
@@ -73,7 +72,7 @@ struct ChunkLocalParams {
     bf16_t* dv_out;
     float* dg_out;
     float* dbeta_out;
-    int H, NC;
+    int H, NC, V;
     // sequences that are not whole rows of whole chunks (packed or left-padded batches): first token (flat index
     // over the rows of the caller's tensors) and length of every sequence; NULL = sequence n is row n
     const int32_t* seq_start;
@@ -98,61 +97,78 @@ __device__ __forceinline__ float half_sum(float x) {
     return x;
 }
 
-template <int V>
-__global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const ChunkLocalParams p) {
-    constexpr int K = BWD_K, VW = 128;  // VW: columns of the value dim staged at a time
-    __shared__ __attribute__((aligned(16))) bf16_t sQ[C * LDR];
-    __shared__ __attribute__((aligned(16))) bf16_t sK[C * LDR];
-    __shared__ __attribute__((aligned(16))) bf16_t sQT[K * LDS64];
-    __shared__ __attribute__((aligned(16))) bf16_t sKT[K * LDS64];
-    __shared__ __attribute__((aligned(16))) bf16_t sDO[C * LDR];
-    __shared__ __attribute__((aligned(16))) bf16_t sVN[C * LDR];
-    __shared__ __attribute__((aligned(16))) bf16_t sY[C * LDR];
-    __shared__ __attribute__((aligned(16))) bf16_t sST[K * LDR];  // S0, then dS1, then G | G^T | Hm + Hm^T
-    __shared__ float s_gam[C], s_beta[C], s_e[C], s_tail[C], s_dgam[C], s_dbeta[C], s_dotq[C], s_dotk[C], s_red[4];
-    bf16_t* const sG = sST;
-    bf16_t* const sGT = sST + C * LDS64;
-    bf16_t* const sH = sST + 2 * C * LDS64;
+__device__ __forceinline__ void put4(bf16_t* dst, f32x4 x) {
+    bf16x4 r;
+    r.x = (bf16_t)x.x, r.y = (bf16_t)x.y, r.z = (bf16_t)x.z, r.w = (bf16_t)x.w;
+    *reinterpret_cast<bf16x4*>(dst) = r;
+}
+
+constexpr int cmax(int a, int b) { return a > b ? a : b; }
+
+template <int K>
+__global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_grads_kernel(const ChunkLocalParams p) {
+    const int V = p.V;
+    constexpr int VW = 64;                     // columns of the value dim staged at a time
+    constexpr int KW = K < 128 ? K : 128;      // keys staged at a time in phases 2 and 3
+    constexpr int KH = K / KW;                 // key halves: 1 or 2
+    constexpr int LDK = KW + 8;                // bf16 per LDS row of a [.][KW] matrix
+    constexpr int NKT = KW / 32;               // key tiles per half: 2 or 4
+    // wave -> 32-key tile of every half and token tiles: with four key tiles a wave has one of them and both token
+    // tiles, with two (K = 64) a quarter each
+    constexpr int NTW = NKT == 4 ? 2 : 1;
+    static_assert(K == 64 || K == 128 || K == 256, "head dims");
+    constexpr int SLAB = C * LDS64 * 2;        // bytes of a staged [64][64] matrix
+    constexpr int PHASE1 = 3 * SLAB + K * LDS64 * 2;        // dO | Y | V~ | states
+    constexpr int PHASE2 = 3 * SLAB + 2 * C * LDK * 2;      // G | G^T | Hm + Hm^T | q | k
+    constexpr int PHASE3 = 3 * SLAB + 2 * KW * LDS64 * 2;   // G | G^T | Hm + Hm^T | q^T | k^T
+    constexpr int LDS_BYTES = cmax(PHASE1, cmax(PHASE2, PHASE3));
+    __shared__ __attribute__((aligned(16))) uint8_t lds[LDS_BYTES];
+    __shared__ float s_gam[C], s_beta[C], s_e[C], s_tail[C], s_dgam[C], s_dbeta[C], s_dotq[C], s_dotk[C], s_fq[C], s_fk[C], s_red[4];
+    bf16_t* const sDO = reinterpret_cast<bf16_t*>(lds);
+    bf16_t* const sY = sDO + C * LDS64;
+    bf16_t* const sVN = sY + C * LDS64;
+    bf16_t* const sST = sVN + C * LDS64;  // [K][LDS64]: S0, then dS1
+    bf16_t* const sG = reinterpret_cast<bf16_t*>(lds);
+    bf16_t* const sGT = sG + C * LDS64;
+    bf16_t* const sH = sGT + C * LDS64;
+    bf16_t* const sQ = sH + C * LDS64;    // phase 2: [64][LDK]
+    bf16_t* const sK = sQ + C * LDK;
+    bf16_t* const sQT = sH + C * LDS64;   // phase 3: [KW][LDS64]
+    bf16_t* const sKT = sQT + KW * LDS64;
 
     const int t = threadIdx.x;
     const int lane = t % WAVE, wave = t / WAVE;
     const int l32 = lane % 32, lh = lane / 32;
+    const int ktl = NKT == 4 ? wave : wave % 2;              // this wave's key tile within a half
+    auto tt_of = [&](int m) { return NTW == 2 ? m : wave / 2; };  // its token tiles
     const int64_t chunk = blockIdx.x;
-    const float* qs = p.qs + chunk * C * K;  // packed mode only
-    const float* kn = p.kn + chunk * C * K;
-    const float* vv = p.v + chunk * C * V;
-    const float* dout = p.dout + chunk * C * V;
-    const bool final_mode = p.y_mirror != nullptr;
-    const int ci = final_mode ? (int)(chunk % p.NC) : 0;
-    const int chain = final_mode ? (int)(chunk / p.NC) : 0;
-    const int n = final_mode ? chain / p.H : 0, h = final_mode ? chain % p.H : 0;
+    const int ci = (int)(chunk % p.NC);
+    const int chain = (int)(chunk / p.NC);
+    const int n = chain / p.H, h = chain % p.H;
     // first token of the chunk as a flat index over the rows of the caller's tensors, and its number of tokens
     int valid = C;
-    int64_t tok0 = 0;
-    if (final_mode) {
-        if (p.seq_start != nullptr) {
-            valid = min(max(p.seq_len[n] - ci * C, 0), C);
-            tok0 = (int64_t)p.seq_start[n] + (int64_t)ci * C;
-        } else {
-            tok0 = (int64_t)n * p.T_rows + (int64_t)ci * C;
-        }
-        if (valid == 0) return;  // a chunk past the end of its sequence (whole workgroup)
+    int64_t tok0;
+    if (p.seq_start != nullptr) {
+        valid = min(max(p.seq_len[n] - ci * C, 0), C);
+        tok0 = (int64_t)p.seq_start[n] + (int64_t)ci * C;
+    } else {
+        tok0 = (int64_t)n * p.T_rows + (int64_t)ci * C;
     }
+    if (valid == 0) return;  // a chunk past the end of its sequence (whole workgroup)
     const int64_t mirA = ((int64_t)n * p.NC + (p.NC - 1 - ci)) * 2 * C;  // first token of mirror chunk A
-    // row `row` of the chunk in one of the caller's tensors; rows past the end read token 0 and are zeroed
+    // row `row` of the chunk in one of the caller's tensors (a chunk lies within one row of the batch); rows past the
+    // end of the sequence read its last token and are zeroed
+    const int64_t row_b = tok0 / p.T_rows, row_t = tok0 % p.T_rows;
     auto row_of = [&](const bf16_t* base, int64_t sb, int64_t st, int64_t sh, int row) -> const bf16_t* {
-        const int64_t f = row < valid ? tok0 + row : 0;
-        return base + (f / p.T_rows) * sb + (f % p.T_rows) * st + (int64_t)h * sh;
+        return base + row_b * sb + (row_t + min(row, valid - 1)) * st + (int64_t)h * sh;
     };
     bf16x8 zero8;
 #pragma unroll
     for (int e = 0; e < 8; e++) zero8[e] = (bf16_t)0.f;
-    const float* yy = final_mode ? nullptr : p.y + chunk * C * V;
-    const float* vnew = p.vnew + chunk * C * V;
-    const float* s0 = p.s0 + chunk * K * V;
-    const float* ds1 = p.ds1 + chunk * K * V;
+    f32x16 zero;
+#pragma unroll
+    for (int r = 0; r < 16; r++) zero[r] = 0.f;
 
-    // ---- stage everything but the states ----
     if (t < C) {
         const float g = p.gam[chunk * C + t];
         s_gam[t] = g;
@@ -163,68 +179,35 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
         s_dbeta[t] = 0.f;
         s_dotq[t] = 0.f;
         s_dotk[t] = 0.f;
+        s_fq[t] = (p.rq != nullptr ? p.rq[chunk * C + t] : 1.f) * p.scale;  // q and k rows are scaled on their way into LDS
+        s_fk[t] = p.rk != nullptr ? p.rk[chunk * C + t] : 1.f;
     }
     if (t < 4) s_red[t] = 0.f;
-    auto put4 = [](bf16_t* dst, f32x4 x) {
-        bf16x4 r;
-        r.x = (bf16_t)x.x, r.y = (bf16_t)x.y, r.z = (bf16_t)x.z, r.w = (bf16_t)x.w;
-        *reinterpret_cast<bf16x4*>(dst) = r;
-    };
-    // ---- q, k and their transposes (final mode: with the first half of v, dO, Y below, one batch of loads) ----
-    if (!final_mode) {
-#pragma unroll
-        for (int i = 0; i < 8; i++) {  // [64][128] fp32: 2048 groups of 4, row = 8 i + t / 32
-            const int idx = t + BWD_THREADS * i, row = idx / 32, c4 = idx % 32;
-            const f32x4 a = *reinterpret_cast<const f32x4*>(qs + row * K + 4 * c4);
-            const f32x4 b = *reinterpret_cast<const f32x4*>(kn + row * K + 4 * c4);
-            put4(sQ + row * LDR + 4 * c4, a);
-            put4(sK + row * LDR + 4 * c4, b);
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                sQT[(4 * c4 + e) * LDS64 + row] = (bf16_t)a[e];
-                sKT[(4 * c4 + e) * LDS64 + row] = (bf16_t)b[e];
-            }
-        }
-    }
 
-    f32x16 zero;
+    // ---------------- phase 1: everything that contracts over the value dim, 64 columns at a time ----------------
+    // products with the states, transposed: rows = keys 32 (ktl + NKT kh) .., columns = tokens 32 tt + l32; and the
+    // 64 x 64 products dO V~^T and Y V~^T (wave -> tile (wave / 2, wave % 2))
+    f32x16 dQeT[KH][NTW], ZT[KH][NTW], dKdT[KH][NTW], DP = zero, DA = zero;
 #pragma unroll
-    for (int r = 0; r < 16; r++) zero[r] = 0.f;
-
-    // Everything that contracts over the value dim runs over V in halves of 128 columns (VW), accumulating:
-    // the products with the states, transposed (rows = key dims 32 wave .., columns = tokens 32 tt + l32), and
-    // the 64 x 64 products dO V~^T and Y V~^T (wave -> tile (wave / 2, wave % 2)).
-    f32x16 dQeT[2] = {zero, zero}, ZT[2] = {zero, zero}, dKdT[2] = {zero, zero}, DP = zero, DA = zero;
+    for (int kh = 0; kh < KH; kh++)
 #pragma unroll
+        for (int m = 0; m < NTW; m++) dQeT[kh][m] = zero, ZT[kh][m] = zero, dKdT[kh][m] = zero;
+    const char* const s0b = static_cast<const char*>(p.s0) + chunk * K * (int64_t)V * (p.saves_bf16 ? 2 : 4);
+    const char* const vnb = static_cast<const char*>(p.vnew) + chunk * C * (int64_t)V * (p.saves_bf16 ? 2 : 4);
+    const float* const ds1 = p.ds1 + chunk * K * (int64_t)V;
+    constexpr int SROWS = K / 16;  // 16-byte fp32 pieces of a state slab per thread: K rows x 16 pieces
+    float dot = 0.f;
+#pragma unroll 1
     for (int hv = 0; hv < V / VW; hv++) {
         const int v0 = VW * hv;
-        float yv[8];  // <Y_i, V_i> pieces, reduced after the barrier (s_dbeta is cleared before the first one)
-#pragma unroll
-        for (int i = 0; i < 8; i++) yv[i] = 0.f;
-        if (final_mode) {
+        float yv[2];  // <Y_i, V_i> pieces, reduced after the barrier (s_dbeta is cleared before the first one)
+        {
             // v, dO and Y (token `row` is token 63 - row of mirror chunk A); dV = beta Y goes out right away
-            const int p8 = t % 16;
+            const int p8 = t % 8;
 #pragma unroll
-            for (int it = 0; it < 4; it++) {
-                const int row = t / 16 + 16 * it;
+            for (int it = 0; it < 2; it++) {
+                const int row = t / 8 + 32 * it;
                 const bool live = row < valid;
-                if (hv == 0) {
-                    bf16x8 qr = *reinterpret_cast<const bf16x8*>(row_of(p.q_raw, p.q_stride_b, p.q_stride_t, p.q_stride_h, row) + 8 * p8);
-                    bf16x8 kr = *reinterpret_cast<const bf16x8*>(row_of(p.k_raw, p.k_stride_b, p.k_stride_t, p.k_stride_h, row) + 8 * p8);
-                    if (!live) qr = zero8, kr = zero8;
-                    const float fq = (p.rq != nullptr ? p.rq[chunk * C + row] : 1.f) * p.scale;
-                    const float fk = p.rk != nullptr ? p.rk[chunk * C + row] : 1.f;
-                    bf16x8 qb, kb;
-#pragma unroll
-                    for (int e = 0; e < 8; e++) {
-                        qb[e] = (bf16_t)((float)qr[e] * fq);
-                        kb[e] = (bf16_t)((float)kr[e] * fk);
-                        sQT[(8 * p8 + e) * LDS64 + row] = qb[e];
-                        sKT[(8 * p8 + e) * LDS64 + row] = kb[e];
-                    }
-                    *reinterpret_cast<bf16x8*>(sQ + row * LDR + 8 * p8) = qb;
-                    *reinterpret_cast<bf16x8*>(sK + row * LDR + 8 * p8) = kb;
-                }
                 bf16x8 vr = *reinterpret_cast<const bf16x8*>(row_of(p.v_raw, p.v_stride_b, p.v_stride_t, p.v_stride_h, row) + v0 + 8 * p8);
                 bf16x8 dr = *reinterpret_cast<const bf16x8*>(row_of(p.d_raw, p.d_stride_b, p.d_stride_t, p.d_stride_h, row) + v0 + 8 * p8);
                 if (!live) vr = zero8, dr = zero8;
@@ -237,102 +220,131 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
                     dv[e] = (bf16_t)((float)yr[e] * b);
                     acc += (float)yr[e] * (float)vr[e];
                 }
-                *reinterpret_cast<bf16x8*>(sDO + row * LDR + 8 * p8) = dr;
-                *reinterpret_cast<bf16x8*>(sY + row * LDR + 8 * p8) = yr;
+                *reinterpret_cast<bf16x8*>(sDO + row * LDS64 + 8 * p8) = dr;
+                *reinterpret_cast<bf16x8*>(sY + row * LDS64 + 8 * p8) = yr;
                 if (live) *reinterpret_cast<bf16x8*>(p.dv_out + ((tok0 + row) * p.H + h) * V + v0 + 8 * p8) = dv;
                 yv[it] = acc;
             }
+            if (p.saves_bf16) {
+                const bf16_t* vnew = reinterpret_cast<const bf16_t*>(vnb);
 #pragma unroll
-            for (int i = 0; i < 8; i++) {  // rows of V~ past the end of the sequence hold whatever the scan left
-                const int idx = t + BWD_THREADS * i, row = idx / 32, c4 = idx % 32;
-                const f32x4 x = *reinterpret_cast<const f32x4*>(vnew + row * V + v0 + 4 * c4);
-                put4(sVN + row * LDR + 4 * c4, row < valid ? x : f32x4{0.f, 0.f, 0.f, 0.f});
+                for (int it = 0; it < 2; it++) {  // rows of V~ past the end of the sequence hold whatever the scan left
+                    const int row = t / 8 + 32 * it;
+                    const bf16x8 x = *reinterpret_cast<const bf16x8*>(vnew + row * V + v0 + 8 * p8);
+                    *reinterpret_cast<bf16x8*>(sVN + row * LDS64 + 8 * p8) = row < valid ? x : zero8;
+                }
+                const bf16_t* s0 = reinterpret_cast<const bf16_t*>(s0b);
+#pragma unroll
+                for (int i = 0; i < K / 32; i++) {  // S0[:, v0 .. v0 + 63]: row = 32 i + t / 8
+                    const int row = t / 8 + 32 * i;
+                    *reinterpret_cast<bf16x8*>(sST + row * LDS64 + 8 * p8) = *reinterpret_cast<const bf16x8*>(s0 + row * V + v0 + 8 * p8);
+                }
+            } else {
+                const float* vnew = reinterpret_cast<const float*>(vnb);
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int idx = t + BWD_THREADS * i, row = idx / 16, c4 = idx % 16;
+                    const f32x4 x = *reinterpret_cast<const f32x4*>(vnew + row * V + v0 + 4 * c4);
+                    put4(sVN + row * LDS64 + 4 * c4, row < valid ? x : f32x4{0.f, 0.f, 0.f, 0.f});
+                }
+                const float* s0 = reinterpret_cast<const float*>(s0b);
+#pragma unroll
+                for (int i = 0; i < SROWS; i++) {  // S0[:, v0 .. v0 + 63] fp32: row = 16 i + t / 16
+                    const int idx = t + BWD_THREADS * i, row = idx / 16, c4 = idx % 16;
+                    put4(sST + row * LDS64 + 4 * c4, *reinterpret_cast<const f32x4*>(s0 + row * V + v0 + 4 * c4));
+                }
             }
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const int idx = t + BWD_THREADS * i, row = idx / 32, c4 = idx % 32;
-                const f32x4 d = *reinterpret_cast<const f32x4*>(dout + row * V + v0 + 4 * c4);
-                const f32x4 n4 = *reinterpret_cast<const f32x4*>(vnew + row * V + v0 + 4 * c4);
-                const f32x4 y = *reinterpret_cast<const f32x4*>(yy + row * V + v0 + 4 * c4);
-                const f32x4 x = *reinterpret_cast<const f32x4*>(vv + row * V + v0 + 4 * c4);
-                put4(sDO + row * LDR + 4 * c4, d);
-                put4(sVN + row * LDR + 4 * c4, n4);
-                put4(sY + row * LDR + 4 * c4, y);
-                yv[i] = y.x * x.x + y.y * x.y + y.z * x.z + y.w * x.w;
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < 16; i++) {  // S0[:, v0 .. v0 + 127] fp32: row = 8 i + t / 32
-            const int idx = t + BWD_THREADS * i, row = idx / 32, c4 = idx % 32;
-            put4(sST + row * LDR + 4 * c4, *reinterpret_cast<const f32x4*>(s0 + row * V + v0 + 4 * c4));
         }
         __syncthreads();
-        if (final_mode) {
 #pragma unroll
-            for (int it = 0; it < 4; it++) {  // 16 lanes hold one row
-                float x = yv[it];
+        for (int it = 0; it < 2; it++) {  // 8 lanes hold one row
+            float x = yv[it];
 #pragma unroll
-                for (int off = 8; off >= 1; off >>= 1) x += __shfl_xor(x, off, WAVE);
-                if (t % 16 == 0) atomicAdd(&s_dbeta[t / 16 + 16 * it], x);
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; i++) {  // the 32 lanes of a wave half hold one row
-                const float x = half_sum(yv[i]);
-                if (l32 == 0) atomicAdd(&s_dbeta[8 * i + t / 32], x);
-            }
+            for (int off = 4; off >= 1; off >>= 1) x += __shfl_xor(x, off, WAVE);
+            if (t % 8 == 0) atomicAdd(&s_dbeta[t / 8 + 32 * it], x);
         }
 
-        // dS1 of this half is asked for now and stays in registers while the products with S0 run: its trip through
-        // memory is then behind them instead of in front of the barrier below (the workgroup has a CU to itself by its
-        // LDS, so there is no other wave to fill the wait)
-        f32x4 ds1_rows[16];
+        // K = 256 (a CU to itself, registers to spare): dS1 of this slab is asked for now and stays in registers while the
+        // products with S0 run, so that its trip through memory is behind them instead of in front of the barrier below.
+        // With two workgroups per CU the other one's products fill that wait, and the registers are needed.
+        constexpr bool PREFETCH = K > 128;
+        f32x4 ds1_rows[SROWS];
+        if constexpr (PREFETCH) {
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int idx = t + BWD_THREADS * i, row = idx / 32, c4 = idx % 32;
-            ds1_rows[i] = *reinterpret_cast<const f32x4*>(ds1 + row * V + v0 + 4 * c4);
+            for (int i = 0; i < SROWS; i++) {
+                const int idx = t + BWD_THREADS * i, row = idx / 16, c4 = idx % 16;
+                ds1_rows[i] = *reinterpret_cast<const f32x4*>(ds1 + row * V + v0 + 4 * c4);
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int tt = 0; tt < 2; tt++) {
-            dQeT[tt] = mma_nt(sST + 32 * wave * LDR, LDR, sDO + 32 * tt * LDR, LDR, VW, dQeT[tt], l32, lh);
-            ZT[tt] = mma_nt(sST + 32 * wave * LDR, LDR, sY + 32 * tt * LDR, LDR, VW, ZT[tt], l32, lh);
-        }
-        if constexpr (V > VW) {  // with a single half they wait until the 64 x 64 stage below (dO, V~, Y stay staged)
-            DP = mma_nt(sDO + 32 * (wave / 2) * LDR, LDR, sVN + 32 * (wave % 2) * LDR, LDR, VW, DP, l32, lh);
-            DA = mma_nt(sY + 32 * (wave / 2) * LDR, LDR, sVN + 32 * (wave % 2) * LDR, LDR, VW, DA, l32, lh);
+        for (int kh = 0; kh < KH; kh++)
+#pragma unroll
+            for (int m = 0; m < NTW; m++) {
+                const bf16_t* srows = sST + 32 * (ktl + NKT * kh) * LDS64;
+                dQeT[kh][m] = mma_nt(srows, LDS64, sDO + 32 * tt_of(m) * LDS64, LDS64, VW, dQeT[kh][m], l32, lh);
+                ZT[kh][m] = mma_nt(srows, LDS64, sY + 32 * tt_of(m) * LDS64, LDS64, VW, ZT[kh][m], l32, lh);
+            }
+        DP = mma_nt(sDO + 32 * (wave / 2) * LDS64, LDS64, sVN + 32 * (wave % 2) * LDS64, LDS64, VW, DP, l32, lh);
+        DA = mma_nt(sY + 32 * (wave / 2) * LDS64, LDS64, sVN + 32 * (wave % 2) * LDS64, LDS64, VW, DA, l32, lh);
+        if constexpr (!PREFETCH) {
+#pragma unroll
+            for (int i = 0; i < SROWS; i++) {
+                const int idx = t + BWD_THREADS * i, row = idx / 16, c4 = idx % 16;
+                ds1_rows[i] = *reinterpret_cast<const f32x4*>(ds1 + row * V + v0 + 4 * c4);
+            }
         }
         __syncthreads();  // S0 has been read by every wave
 
-        // dS1 takes the place of S0; <dS1, S0> on the way
-        {
-            float dot = 0.f;
+        // dS1 takes the place of S0; <dS1, S0> on the way (S0 as the bf16 the products used)
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const int idx = t + BWD_THREADS * i, row = idx / 32, c4 = idx % 32;
-                const f32x4 x = ds1_rows[i];
-                const bf16x4 sv = *reinterpret_cast<const bf16x4*>(sST + row * LDR + 4 * c4);
-                dot += x.x * (float)sv.x + x.y * (float)sv.y + x.z * (float)sv.z + x.w * (float)sv.w;
-                put4(sST + row * LDR + 4 * c4, x);
-            }
-            dot = wave_sum(dot);
-            if (lane == 0) atomicAdd(&s_red[0], dot);
+        for (int i = 0; i < SROWS; i++) {
+            const int idx = t + BWD_THREADS * i, row = idx / 16, c4 = idx % 16;
+            const f32x4 x = ds1_rows[i];
+            const bf16x4 sv = *reinterpret_cast<const bf16x4*>(sST + row * LDS64 + 4 * c4);
+            dot += x.x * (float)sv.x + x.y * (float)sv.y + x.z * (float)sv.z + x.w * (float)sv.w;
+            put4(sST + row * LDS64 + 4 * c4, x);
         }
         __syncthreads();
 #pragma unroll
-        for (int tt = 0; tt < 2; tt++) dKdT[tt] = mma_nt(sST + 32 * wave * LDR, LDR, sVN + 32 * tt * LDR, LDR, VW, dKdT[tt], l32, lh);
-        __syncthreads();  // the staged half is free
+        for (int kh = 0; kh < KH; kh++)
+#pragma unroll
+            for (int m = 0; m < NTW; m++)
+                dKdT[kh][m] = mma_nt(sST + 32 * (ktl + NKT * kh) * LDS64, LDS64, sVN + 32 * tt_of(m) * LDS64, LDS64, VW, dKdT[kh][m], l32, lh);
+        __syncthreads();  // the staged slab is free
     }
+    dot = wave_sum(dot);
+    if (lane == 0) atomicAdd(&s_red[0], dot);
 
-    // ---- the 64 x 64 products: wave -> tile (ti, tj); rows i = 32 ti + 8 (r/4) + 4 h + r%4, column j = 32 tj + l32 ----
+    // ---------------- phase 2: Q K^T, K K^T and the 64 x 64 stage ----------------
+    // wave -> tile (ti, tj); rows i = 32 ti + 8 (r/4) + 4 h + r%4, column j = 32 tj + l32
     {
         const int ti = wave / 2, tj = wave % 2;
-        const f32x16 QK = mma_nt(sQ + 32 * ti * LDR, LDR, sK + 32 * tj * LDR, LDR, K, zero, l32, lh);
-        const f32x16 KK = mma_nt(sK + 32 * ti * LDR, LDR, sK + 32 * tj * LDR, LDR, K, zero, l32, lh);
-        if constexpr (V == VW) {
-            DP = mma_nt(sDO + 32 * ti * LDR, LDR, sVN + 32 * tj * LDR, LDR, VW, zero, l32, lh);
-            DA = mma_nt(sY + 32 * ti * LDR, LDR, sVN + 32 * tj * LDR, LDR, VW, zero, l32, lh);
+        f32x16 QK = zero, KK = zero;
+        constexpr int CPR = KW / 8, RPP = BWD_THREADS / CPR;  // 16-byte pieces per staged row, rows per pass
+#pragma unroll
+        for (int kh = 0; kh < KH; kh++) {
+            if (kh > 0) __syncthreads();  // the products of the previous half have read q and k
+            const int p8 = t % CPR;
+#pragma unroll
+            for (int it = 0; it < C / RPP; it++) {
+                const int row = t / CPR + RPP * it;
+                bf16x8 qr = *reinterpret_cast<const bf16x8*>(row_of(p.q_raw, p.q_stride_b, p.q_stride_t, p.q_stride_h, row) + KW * kh + 8 * p8);
+                bf16x8 kr = *reinterpret_cast<const bf16x8*>(row_of(p.k_raw, p.k_stride_b, p.k_stride_t, p.k_stride_h, row) + KW * kh + 8 * p8);
+                if (row >= valid) qr = zero8, kr = zero8;
+                const float fq = s_fq[row], fk = s_fk[row];
+                bf16x8 qb, kb;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    qb[e] = (bf16_t)((float)qr[e] * fq);
+                    kb[e] = (bf16_t)((float)kr[e] * fk);
+                }
+                *reinterpret_cast<bf16x8*>(sQ + row * LDK + 8 * p8) = qb;
+                *reinterpret_cast<bf16x8*>(sK + row * LDK + 8 * p8) = kb;
+            }
+            __syncthreads();
+            QK = mma_nt(sQ + 32 * ti * LDK, LDK, sK + 32 * tj * LDK, LDK, KW, QK, l32, lh);
+            KK = mma_nt(sK + 32 * ti * LDK, LDK, sK + 32 * tj * LDK, LDK, KW, KK, l32, lh);
         }
         const int j = 32 * tj + l32;
         const float gj = s_gam[j];
@@ -367,46 +379,71 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
         }
         atomicAdd(&s_dgam[j], -colsum);
     }
-    __syncthreads();
 
-    // ---- per-token sums over the key dim, then dQ^T and dK^T ----
+    // ---------------- phase 3: per-token sums over the key dim, dQ^T and dK^T, 128 keys at a time ----------------
+    // (dQ^T and dK^T are built in the registers of dQe^T and dKd^T)
     float nkd = 0.f;
-    f32x16 accq[2], acck[2];
+    auto& accq = dQeT;
+    auto& acck = dKdT;
+    bf16x8 qv[KH][NTW][2], kv[KH][NTW][2];  // this lane's entries of q and k, kept for the backward of the normalisation
 #pragma unroll
-    for (int tt = 0; tt < 2; tt++) {
-        const int i = 32 * tt + l32;
-        const float ei = s_e[i], tl = s_tail[i], bi = s_beta[i];
-        float s_qe = 0.f, s_kd = 0.f, s_zk = 0.f;
+    for (int kh = 0; kh < KH; kh++) {
+        __syncthreads();  // G, G^T, Hm + Hm^T are complete; q and k of phase 2 (or the previous half's transposes) are dead
+        {
+            constexpr int CPR = KW / 8, RPP = BWD_THREADS / CPR;
+            const int p8 = t % CPR;
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int d = 32 * wave + 8 * (r / 4) + 4 * lh + r % 4;
-            const float qv = (float)sQT[d * LDS64 + i], kv = (float)sKT[d * LDS64 + i];
-            s_qe += dQeT[tt][r] * qv;
-            s_kd += dKdT[tt][r] * kv;
-            s_zk += ZT[tt][r] * kv;
+            for (int it = 0; it < C / RPP; it++) {
+                const int row = t / CPR + RPP * it;
+                bf16x8 qr = *reinterpret_cast<const bf16x8*>(row_of(p.q_raw, p.q_stride_b, p.q_stride_t, p.q_stride_h, row) + KW * kh + 8 * p8);
+                bf16x8 kr = *reinterpret_cast<const bf16x8*>(row_of(p.k_raw, p.k_stride_b, p.k_stride_t, p.k_stride_h, row) + KW * kh + 8 * p8);
+                if (row >= valid) qr = zero8, kr = zero8;
+                const float fq = s_fq[row], fk = s_fk[row];
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    sQT[(8 * p8 + e) * LDS64 + row] = (bf16_t)((float)qr[e] * fq);
+                    sKT[(8 * p8 + e) * LDS64 + row] = (bf16_t)((float)kr[e] * fk);
+                }
+            }
         }
-        atomicAdd(&s_dgam[i], ei * s_qe - tl * s_kd - bi * ei * s_zk);
-        atomicAdd(&s_dbeta[i], -ei * s_zk);
-        nkd += tl * s_kd;
-
+        __syncthreads();
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            accq[tt][r] = dQeT[tt][r] * ei;
-            acck[tt][r] = dKdT[tt][r] * tl - ZT[tt][r] * (bi * ei);
-        }
-        accq[tt] = mma_nt(sKT + 32 * wave * LDS64, LDS64, sG + 32 * tt * LDS64, LDS64, C, accq[tt], l32, lh);
-        acck[tt] = mma_nt(sQT + 32 * wave * LDS64, LDS64, sGT + 32 * tt * LDS64, LDS64, C, acck[tt], l32, lh);
-        acck[tt] = mma_nt(sKT + 32 * wave * LDS64, LDS64, sH + 32 * tt * LDS64, LDS64, C, acck[tt], l32, lh);
-        if (p.rq != nullptr) {  // <dQs_i, Qs_i> and <dK_i, K_i> for the backward of the normalisation
-            float dq_q = 0.f, dk_k = 0.f;
+        for (int m = 0; m < NTW; m++) {
+            const int tt = tt_of(m);
+            const int i = 32 * tt + l32;
+            const float ei = s_e[i], tl = s_tail[i], bi = s_beta[i];
+            float s_qe = 0.f, s_kd = 0.f, s_zk = 0.f;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const int d = 32 * wave + 8 * (r / 4) + 4 * lh + r % 4;
-                dq_q += accq[tt][r] * (float)sQT[d * LDS64 + i];
-                dk_k += acck[tt][r] * (float)sKT[d * LDS64 + i];
+                const int d = 32 * ktl + 8 * (r / 4) + 4 * lh + r % 4;
+                const bf16_t qe = sQT[d * LDS64 + i], ke = sKT[d * LDS64 + i];
+                qv[kh][m][r / 8][r % 8] = qe, kv[kh][m][r / 8][r % 8] = ke;
+                s_qe += dQeT[kh][m][r] * (float)qe;
+                s_kd += dKdT[kh][m][r] * (float)ke;
+                s_zk += ZT[kh][m][r] * (float)ke;
             }
-            atomicAdd(&s_dotq[i], dq_q);
-            atomicAdd(&s_dotk[i], dk_k);
+            atomicAdd(&s_dgam[i], ei * s_qe - tl * s_kd - bi * ei * s_zk);
+            atomicAdd(&s_dbeta[i], -ei * s_zk);
+            nkd += tl * s_kd;
+
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                accq[kh][m][r] *= ei;
+                acck[kh][m][r] = acck[kh][m][r] * tl - ZT[kh][m][r] * (bi * ei);
+            }
+            accq[kh][m] = mma_nt(sKT + 32 * ktl * LDS64, LDS64, sG + 32 * tt * LDS64, LDS64, C, accq[kh][m], l32, lh);
+            acck[kh][m] = mma_nt(sQT + 32 * ktl * LDS64, LDS64, sGT + 32 * tt * LDS64, LDS64, C, acck[kh][m], l32, lh);
+            acck[kh][m] = mma_nt(sKT + 32 * ktl * LDS64, LDS64, sH + 32 * tt * LDS64, LDS64, C, acck[kh][m], l32, lh);
+            if (p.rq != nullptr) {  // <dQs_i, Qs_i> and <dK_i, K_i> for the backward of the normalisation
+                float dq_q = 0.f, dk_k = 0.f;
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    dq_q += accq[kh][m][r] * (float)qv[kh][m][r / 8][r % 8];
+                    dk_k += acck[kh][m][r] * (float)kv[kh][m][r / 8][r % 8];
+                }
+                atomicAdd(&s_dotq[i], dq_q);
+                atomicAdd(&s_dotk[i], dk_k);
+            }
         }
     }
     nkd = wave_sum(nkd);
@@ -416,50 +453,42 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
     // With x = y / r the normalised row (y: input, r = |y|^-1 incl. epsilon): dy = r (dx - x <x, dx>); the scale of
     // q moves through: Qs = scale Qn, so dQn = scale dQs and Qn <Qn, dQn> = Qs <Qs, dQs> / scale.
 #pragma unroll
-    for (int tt = 0; tt < 2; tt++) {
-        const int i = 32 * tt + l32;
-        const int64_t at = final_mode ? ((tok0 + i) * p.H + h) * K + 32 * wave + 4 * lh : (chunk * C + i) * K + 32 * wave + 4 * lh;
-        const bool norm = p.rq != nullptr;
-        const float rq = norm ? p.rq[chunk * C + i] : 1.f, rk = norm ? p.rk[chunk * C + i] : 1.f;
-        const float cq = norm ? s_dotq[i] / p.scale : 0.f, ck = norm ? s_dotk[i] : 0.f;
+    for (int kh = 0; kh < KH; kh++)
 #pragma unroll
-        for (int r4 = 0; r4 < 4; r4++) {
-            f32x4 oq, ok;
+        for (int m = 0; m < NTW; m++) {
+            const int i = 32 * tt_of(m) + l32;
+            const int64_t at = ((tok0 + i) * p.H + h) * K + KW * kh + 32 * ktl + 4 * lh;
+            const bool norm = p.rq != nullptr;
+            const float rq = norm ? p.rq[chunk * C + i] : 1.f, rk = norm ? p.rk[chunk * C + i] : 1.f;
+            const float cq = norm ? s_dotq[i] / p.scale : 0.f, ck = norm ? s_dotk[i] : 0.f;
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const int r = 4 * r4 + e, d = 32 * wave + 8 * r4 + 4 * lh + e;
-                oq[e] = rq * (accq[tt][r] * p.scale - cq * (float)sQT[d * LDS64 + i]);
-                ok[e] = rk * (acck[tt][r] - ck * (float)sKT[d * LDS64 + i]);
-            }
-            if (final_mode) {
+            for (int r4 = 0; r4 < 4; r4++) {
+                f32x4 oq, ok;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int r = 4 * r4 + e;
+                    oq[e] = rq * (accq[kh][m][r] * p.scale - cq * (float)qv[kh][m][r / 8][r % 8]);
+                    ok[e] = rk * (acck[kh][m][r] - ck * (float)kv[kh][m][r / 8][r % 8]);
+                }
                 if (i < valid) {
                     store4<bf16_t>(p.dq_out + at + 8 * r4, oq);
                     store4<bf16_t>(p.dk_out + at + 8 * r4, ok);
                 }
-            } else {
-                *reinterpret_cast<f32x4*>(p.dq + at + 8 * r4) = oq;
-                *reinterpret_cast<f32x4*>(p.dk + at + 8 * r4) = ok;
             }
         }
-    }
 
     if (t < C) {  // wave 0
         float dg = s_dgam[t];
         if (t == C - 1) dg += s_e[C - 1] * s_red[0] + s_red[1];
-        if (final_mode) {
-            // dg_t = sum of dgamma over the tokens t .. 63 of the chunk
+        // dg_t = sum of dgamma over the tokens t .. 63 of the chunk
 #pragma unroll
-            for (int off = 1; off < WAVE; off <<= 1) {
-                const float y = __shfl_down(dg, off, WAVE);
-                if (t + off < C) dg += y;
-            }
-            if (t < valid) {
-                p.dg_out[(tok0 + t) * p.H + h] = dg;
-                p.dbeta_out[(tok0 + t) * p.H + h] = s_dbeta[t];
-            }
-        } else {
-            p.dgam[chunk * C + t] = dg;
-            p.dbeta[chunk * C + t] = s_dbeta[t];
+        for (int off = 1; off < WAVE; off <<= 1) {
+            const float y = __shfl_down(dg, off, WAVE);
+            if (t + off < C) dg += y;
+        }
+        if (t < valid) {
+            p.dg_out[(tok0 + t) * p.H + h] = dg;
+            p.dbeta_out[(tok0 + t) * p.H + h] = s_dbeta[t];
         }
     }
 }
@@ -476,7 +505,8 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_local_grads_kernel(const Ch
 //             -beta e / |k| for the state update, e^{gamma_C} decay
 //         B:  v := dO, k := q, T' := I, P := 0, row scale e scale / |q| for the state update, no decay
 //     i.e. the rows of k_m and v_m and both records, in the layout chunk_prepare32_kernel writes.
-// T = (I + A)^-1 is formed by forward substitution in one wave (a lane owns a column, 2016 multiply-adds).
+// K = 64, 128, 256; V a multiple of 64 up to 512.  The rows of q and k are only needed for K K^T and Q K^T; slabs of
+// dO^T and the scratch of the inverse then take their place in LDS (K <= 128: two workgroups per CU).
 // ------------------------------------------------------------------------------------------
 constexpr int LDA = 68;  // floats per LDS row of A / T
 
@@ -490,7 +520,7 @@ struct BwdPrepareParams {
     int64_t q_stride_b, q_stride_t, q_stride_h;
     int64_t k_stride_b, k_stride_t, k_stride_h;
     int64_t d_stride_b, d_stride_t, d_stride_h;
-    int N, H, NC;
+    int N, H, NC, V;
     int l2norm;
     int rec16;  // fragments of the records in the lane order of the 16x16x32 MFMA (GDN_FLAG_RECORDS_16X16)
     float scale;
@@ -606,15 +636,21 @@ __device__ __forceinline__ void invert_unit_lower_64(float* sA, float* scratch, 
     __syncthreads();  // T is complete
 }
 
-template <int V>
-__global__ __launch_bounds__(BWD_THREADS) void chunk_bwd_prepare_kernel(const BwdPrepareParams p) {
-    constexpr int K = BWD_K;
-    __shared__ __attribute__((aligned(16))) bf16_t sQ[C * LDR];
-    __shared__ __attribute__((aligned(16))) bf16_t sK[C * LDR];
-    __shared__ __attribute__((aligned(16))) bf16_t sDOT[V * LDS64];  // dO^T
-    __shared__ __attribute__((aligned(16))) bf16_t sPT[C * LDS64];   // P^T
-    __shared__ __attribute__((aligned(16))) float sA[C * LDA];       // A, then T in its place
+template <int K>
+__global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_bwd_prepare_kernel(const BwdPrepareParams p) {
+    const int V = p.V;
+    constexpr int LDK = K + 8;                 // bf16 per LDS row of q / k
+    constexpr int CPR = K / 8;                 // 16-byte pieces per row of q / k
+    constexpr int RPP = BWD_THREADS / CPR;     // rows per pass of their copy
+    // dO is staged transposed, 128 (or a last 64) columns at a time, over the rows of q and k once they are dead
+    static_assert(128 * LDS64 * 2 <= 2 * C * LDK * 2, "a slab of dO^T fits the rows of q and k");
+    __shared__ __attribute__((aligned(16))) bf16_t sQK[2 * C * LDK];   // rows of q, of k; then slabs of dO^T; then the scratch of the inverse
+    __shared__ __attribute__((aligned(16))) bf16_t sPT[C * LDS64];     // P^T
+    __shared__ __attribute__((aligned(16))) float sA[C * LDA];         // A, then T in its place
     __shared__ float s_gam[C], s_beta[C], s_e[C], s_tail[C], s_rq[C], s_rk[C];
+    bf16_t* const sQ = sQK;
+    bf16_t* const sK = sQK + C * LDK;
+    bf16_t* const sDOT = sQK;  // [VS][LDS64]
 
     const int t = threadIdx.x;
     const int lane = t % WAVE, wave = t / WAVE;
@@ -632,14 +668,17 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_bwd_prepare_kernel(const Bw
         valid = min(max(p.seq_len[n] - ci * C, 0), C);
         tok0 = (int64_t)p.seq_start[n] + (int64_t)ci * C;
     }
+    // (a chunk lies within one row of the batch; rows past the end of the sequence read its last token and are zeroed)
+    const int64_t row_b = tok0 / p.T_rows, row_t = tok0 % p.T_rows;
     auto row_of = [&](const bf16_t* base, int64_t sb, int64_t st, int64_t sh, int row) -> const bf16_t* {
-        const int64_t f = row < valid ? tok0 + row : 0;
-        return base + (f / p.T_rows) * sb + (f % p.T_rows) * st + (int64_t)h * sh;
+        return base + row_b * sb + (row_t + max(min(row, valid - 1), 0)) * st + (int64_t)h * sh;
     };
     bf16x8 zero8;
 #pragma unroll
     for (int e = 0; e < 8; e++) zero8[e] = (bf16_t)0.f;
     const int64_t mir0 = (int64_t)(p.NC - 1 - ci) * 2 * C;  // first token of chunk A in the mirror problem
+    // token `row` of this chunk is token 63 - row of the mirror chunks A and B
+    auto tok_a = [&](int row) -> int64_t { return ((int64_t)n * TM + mir0 + (C - 1 - row)) * p.H + h; };
 
     // ---- gamma (prefix sum of g inside the chunk) and beta: wave 0 ----
     if (wave == 0) {
@@ -657,68 +696,60 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_bwd_prepare_kernel(const Bw
         p.bc[chunk * C + lane] = b;
     }
 
-    // ---- rows of q, k, v, dO: 16-byte pieces, 16 lanes per row ----
-    const int p8 = t % 16;
     if (valid == 0) {
         // A chunk slot past the end of its sequence (batches laid out with the chunk count of their longest sequence):
         // what the code below would arrive at from rows of zeros - zero rows of the mirror problem, T = I, the constant
         // inverse norms - written directly; only the records are then formed as for any other chunk.
         const float r0 = p.l2norm ? rsqrtf(L2NORM_EPS) : 1.f;
-#pragma unroll
-        for (int it = 0; it < 4; it++) {
-            const int row = t / 16 + 16 * it;
-            if (p8 == 0) {
-                s_rq[row] = r0, s_rk[row] = r0;
-                p.rq[chunk * C + row] = r0, p.rk[chunk * C + row] = r0;
-            }
-            const int64_t tokA = ((int64_t)n * TM + mir0 + (C - 1 - row)) * p.H + h, tokB = tokA + (int64_t)C * p.H;
-            *reinterpret_cast<bf16x8*>(p.k_m + tokA * K + 8 * p8) = zero8;
-            *reinterpret_cast<bf16x8*>(p.k_m + tokB * K + 8 * p8) = zero8;
-#pragma unroll
-            for (int hv = 0; hv < V / 128; hv++) {
-                *reinterpret_cast<bf16x8*>(p.v_m + tokA * V + 128 * hv + 8 * p8) = zero8;
-                *reinterpret_cast<bf16x8*>(p.v_m + tokB * V + 128 * hv + 8 * p8) = zero8;
-            }
+        if (t < C) {
+            s_rq[t] = r0, s_rk[t] = r0;
+            p.rq[chunk * C + t] = r0, p.rk[chunk * C + t] = r0;
+        }
+        for (int i = t; i < C * (K / 8); i += BWD_THREADS) {
+            const int row = i / (K / 8), p8 = i % (K / 8);
+            *reinterpret_cast<bf16x8*>(p.k_m + tok_a(row) * K + 8 * p8) = zero8;
+            *reinterpret_cast<bf16x8*>(p.k_m + (tok_a(row) + (int64_t)C * p.H) * K + 8 * p8) = zero8;
+        }
+        for (int i = t; i < C * (V / 8); i += BWD_THREADS) {
+            const int row = i / (V / 8), p8 = i % (V / 8);
+            *reinterpret_cast<bf16x8*>(p.v_m + tok_a(row) * V + 8 * p8) = zero8;
+            *reinterpret_cast<bf16x8*>(p.v_m + (tok_a(row) + (int64_t)C * p.H) * V + 8 * p8) = zero8;
         }
         for (int i = t; i < C * C; i += BWD_THREADS) sA[(i / C) * LDA + i % C] = (i / C == i % C) ? 1.f : 0.f;
         __syncthreads();
     } else {
+        // ---- rows of q and k: 16-byte pieces, CPR lanes per row ----
+        {
+            const int p8 = t % CPR;
 #pragma unroll
-        for (int it = 0; it < 4; it++) {
-            const int row = t / 16 + 16 * it;
-            const bool live = row < valid;
-            bf16x8 qr = *reinterpret_cast<const bf16x8*>(row_of(p.q, p.q_stride_b, p.q_stride_t, p.q_stride_h, row) + 8 * p8);
-            bf16x8 kr = *reinterpret_cast<const bf16x8*>(row_of(p.k, p.k_stride_b, p.k_stride_t, p.k_stride_h, row) + 8 * p8);
-            if (!live) qr = zero8, kr = zero8;
-            float ssq = 0.f, ssk = 0.f;
+            for (int it = 0; it < C / RPP; it++) {
+                const int row = t / CPR + RPP * it;
+                const bool live = row < valid;
+                bf16x8 qr = *reinterpret_cast<const bf16x8*>(row_of(p.q, p.q_stride_b, p.q_stride_t, p.q_stride_h, row) + 8 * p8);
+                bf16x8 kr = *reinterpret_cast<const bf16x8*>(row_of(p.k, p.k_stride_b, p.k_stride_t, p.k_stride_h, row) + 8 * p8);
+                if (!live) qr = zero8, kr = zero8;
+                float ssq = 0.f, ssk = 0.f;
 #pragma unroll
-            for (int e = 0; e < 8; e++) ssq += (float)qr[e] * (float)qr[e], ssk += (float)kr[e] * (float)kr[e];
+                for (int e = 0; e < 8; e++) ssq += (float)qr[e] * (float)qr[e], ssk += (float)kr[e] * (float)kr[e];
 #pragma unroll
-            for (int off = 8; off >= 1; off >>= 1) ssq += __shfl_xor(ssq, off, WAVE), ssk += __shfl_xor(ssk, off, WAVE);
-            const float rq = p.l2norm ? rsqrtf(ssq + L2NORM_EPS) : 1.f, rk = p.l2norm ? rsqrtf(ssk + L2NORM_EPS) : 1.f;
-            if (p8 == 0) {
-                s_rq[row] = rq, s_rk[row] = rk;
-                p.rq[chunk * C + row] = rq, p.rk[chunk * C + row] = rk;
-            }
-            bf16x8 qb, kb;
+                for (int off = CPR / 2; off >= 1; off >>= 1) ssq += __shfl_xor(ssq, off, WAVE), ssk += __shfl_xor(ssk, off, WAVE);
+                const float rq = p.l2norm ? rsqrtf(ssq + L2NORM_EPS) : 1.f, rk = p.l2norm ? rsqrtf(ssk + L2NORM_EPS) : 1.f;
+                if (p8 == 0) {
+                    s_rq[row] = rq, s_rk[row] = rk;
+                    p.rq[chunk * C + row] = rq, p.rk[chunk * C + row] = rk;
+                }
+                bf16x8 qb, kb;
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
-                qb[e] = (bf16_t)((float)qr[e] * rq * p.scale);
-                kb[e] = (bf16_t)((float)kr[e] * rk);
-            }
-            *reinterpret_cast<bf16x8*>(sQ + row * LDR + 8 * p8) = qb;
-            *reinterpret_cast<bf16x8*>(sK + row * LDR + 8 * p8) = kb;
-            // mirror rows: token `row` of this chunk is token 63 - row of chunks A and B
-            const int64_t tokA = ((int64_t)n * TM + mir0 + (C - 1 - row)) * p.H + h, tokB = tokA + (int64_t)C * p.H;
-            *reinterpret_cast<bf16x8*>(p.k_m + tokA * K + 8 * p8) = kr;
-            *reinterpret_cast<bf16x8*>(p.k_m + tokB * K + 8 * p8) = qr;
-#pragma unroll
-            for (int hv = 0; hv < V / 128; hv++) {
-                bf16x8 dr = *reinterpret_cast<const bf16x8*>(row_of(p.dout, p.d_stride_b, p.d_stride_t, p.d_stride_h, row) + 128 * hv + 8 * p8);
-                if (!live) dr = zero8;
-#pragma unroll
-                for (int e = 0; e < 8; e++) sDOT[(128 * hv + 8 * p8 + e) * LDS64 + row] = dr[e];
-                *reinterpret_cast<bf16x8*>(p.v_m + tokB * V + 128 * hv + 8 * p8) = dr;
+                for (int e = 0; e < 8; e++) {
+                    qb[e] = (bf16_t)((float)qr[e] * rq * p.scale);
+                    kb[e] = (bf16_t)((float)kr[e] * rk);
+                }
+                *reinterpret_cast<bf16x8*>(sQ + row * LDK + 8 * p8) = qb;
+                *reinterpret_cast<bf16x8*>(sK + row * LDK + 8 * p8) = kb;
+                // mirror rows: k of chunk A is k, k of chunk B is q
+                const int64_t tokA = tok_a(row), tokB = tokA + (int64_t)C * p.H;
+                *reinterpret_cast<bf16x8*>(p.k_m + tokA * K + 8 * p8) = kr;
+                *reinterpret_cast<bf16x8*>(p.k_m + tokB * K + 8 * p8) = qr;
             }
         }
         __syncthreads();
@@ -730,8 +761,8 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_bwd_prepare_kernel(const Bw
         // ---- A = stril(beta_i E . K K^T) and P^T = tril(E . Q K^T)^T: wave -> tile (ti, tj) ----
         {
             const int ti = wave / 2, tj = wave % 2;
-            const f32x16 KK = mma_nt(sK + 32 * ti * LDR, LDR, sK + 32 * tj * LDR, LDR, K, zero, l32, lh);
-            const f32x16 QK = mma_nt(sQ + 32 * ti * LDR, LDR, sK + 32 * tj * LDR, LDR, K, zero, l32, lh);
+            const f32x16 KK = mma_nt(sK + 32 * ti * LDK, LDK, sK + 32 * tj * LDK, LDK, K, zero, l32, lh);
+            const f32x16 QK = mma_nt(sQ + 32 * ti * LDK, LDK, sK + 32 * tj * LDK, LDK, K, zero, l32, lh);
             const int j = 32 * tj + l32;
             const float gj = s_gam[j];
 #pragma unroll
@@ -742,25 +773,45 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_bwd_prepare_kernel(const Bw
                 sPT[j * LDS64 + i] = (bf16_t)(E * QK[r]);
             }
         }
-        __syncthreads();
+        __syncthreads();  // the rows of q and k are dead
 
-        // ---- P^T dO -> rows of v_m for chunk A: rows j = 32 tj + .., columns v = 32 tv + l32, tv = wave, wave + 4, .. ----
+        // ---- P^T dO -> rows of v_m for chunk A, a slab of columns at a time; dO itself -> rows of v_m for chunk B ----
+        auto slab = [&](int v0, auto vsc) {
+            constexpr int VS = decltype(vsc)::value;
+            constexpr int VPR = VS / 8, VRPP = BWD_THREADS / VPR;  // pieces per row of the slab, rows per pass
+            const int p8 = t % VPR;
 #pragma unroll
-        for (int tv = wave; tv < V / 32; tv += BWD_THREADS / WAVE)
+            for (int it = 0; it < C / VRPP; it++) {
+                const int row = t / VPR + VRPP * it;
+                bf16x8 dr = *reinterpret_cast<const bf16x8*>(row_of(p.dout, p.d_stride_b, p.d_stride_t, p.d_stride_h, row) + v0 + 8 * p8);
+                if (row >= valid) dr = zero8;
 #pragma unroll
-            for (int tj = 0; tj < 2; tj++) {
-                const f32x16 u = mma_nt(sPT + 32 * tj * LDS64, LDS64, sDOT + 32 * tv * LDS64, LDS64, C, zero, l32, lh);
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int j = 32 * tj + 8 * (r / 4) + 4 * lh + r % 4;
-                    p.v_m[(((int64_t)n * TM + mir0 + (C - 1 - j)) * p.H + h) * V + 32 * tv + l32] = (bf16_t)u[r];
-                }
+                for (int e = 0; e < 8; e++) sDOT[(8 * p8 + e) * LDS64 + row] = dr[e];
+                *reinterpret_cast<bf16x8*>(p.v_m + (tok_a(row) + (int64_t)C * p.H) * V + v0 + 8 * p8) = dr;
             }
+            __syncthreads();
+            // rows j = 32 tj + .., columns v = v0 + 32 tv + l32, tv = wave, wave + 4, ..
+#pragma unroll
+            for (int tv = wave; tv < VS / 32; tv += BWD_THREADS / WAVE)
+#pragma unroll
+                for (int tj = 0; tj < 2; tj++) {
+                    const f32x16 u = mma_nt(sPT + 32 * tj * LDS64, LDS64, sDOT + 32 * tv * LDS64, LDS64, C, zero, l32, lh);
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int j = 32 * tj + 8 * (r / 4) + 4 * lh + r % 4;
+                        p.v_m[tok_a(j) * V + v0 + 32 * tv + l32] = (bf16_t)u[r];
+                    }
+                }
+            __syncthreads();  // the slab is free (also for the scratch of the inverse)
+        };
+        int v0 = 0;
+#pragma unroll 1
+        for (; v0 + 128 <= V; v0 += 128) slab(v0, std::integral_constant<int, 128>{});
+        if (v0 < V) slab(v0, std::integral_constant<int, 64>{});
 
-        // ---- T = (I + A)^-1 in place of A (the rows of q and k in LDS are dead: their place is the scratch) ----
-        static_assert(INVERSE_SCRATCH_FLOATS * 4 <= C * LDR * 2, "the scratch of the inverse fits the rows of q");
-        invert_unit_lower_64<LDA>(sA, reinterpret_cast<float*>(sQ), wave, lane);
-
+        // ---- T = (I + A)^-1 in place of A (its scratch over the dead rows of q) ----
+        static_assert(INVERSE_SCRATCH_FLOATS * 4 <= 2 * C * LDK * 2, "the scratch of the inverse fits the rows of q and k");
+        invert_unit_lower_64<LDA>(sA, reinterpret_cast<float*>(sQK), wave, lane);
     }
 
     // ---- the two records ----
@@ -806,16 +857,17 @@ __global__ __launch_bounds__(BWD_THREADS) void chunk_bwd_prepare_kernel(const Bw
 
 }  // namespace
 
+static bool bwd_shape_built(int K, int V) { return (K == 64 || K == 128 || K == 256) && V > 0 && V % 64 == 0; }
+
 int launch_chunk_bwd_local(const gdn_chunk_local_args& a, hipStream_t stream) {
     ChunkLocalParams p;
-    p.qs = a.qs, p.kn = a.kn, p.v = a.v, p.dout = a.dout, p.y = a.y, p.vnew = a.v_new;
-    p.s0 = a.states, p.ds1 = a.dstates, p.gam = a.gamma, p.beta = a.beta;
+    p.vnew = a.v_new, p.s0 = a.states, p.ds1 = a.dstates, p.saves_bf16 = a.saves_dtype == GDN_BF16 ? 1 : 0;
+    p.gam = a.gamma, p.beta = a.beta;
     p.rq = a.rq, p.rk = a.rk, p.scale = a.scale;
-    p.dq = a.dq, p.dk = a.dk, p.dbeta = a.dbeta, p.dgam = a.dgamma;
     p.y_mirror = static_cast<const bf16_t*>(a.y_mirror);
     p.dq_out = static_cast<bf16_t*>(a.dq_out), p.dk_out = static_cast<bf16_t*>(a.dk_out), p.dv_out = static_cast<bf16_t*>(a.dv_out);
     p.dg_out = a.dg_out, p.dbeta_out = a.dbeta_out;
-    p.H = a.H, p.NC = a.NC;
+    p.H = a.H, p.NC = a.NC, p.V = a.V;
     p.q_raw = static_cast<const bf16_t*>(a.q_raw), p.k_raw = static_cast<const bf16_t*>(a.k_raw);
     p.v_raw = static_cast<const bf16_t*>(a.v_raw), p.d_raw = static_cast<const bf16_t*>(a.dout_raw);
     p.q_stride_b = a.q_stride_b, p.q_stride_t = a.q_stride_t, p.q_stride_h = a.q_stride_h;
@@ -823,16 +875,17 @@ int launch_chunk_bwd_local(const gdn_chunk_local_args& a, hipStream_t stream) {
     p.v_stride_b = a.v_stride_b, p.v_stride_t = a.v_stride_t, p.v_stride_h = a.v_stride_h;
     p.d_stride_b = a.dout_stride_b, p.d_stride_t = a.dout_stride_t, p.d_stride_h = a.dout_stride_h;
     p.seq_start = a.seq_start, p.seq_len = a.seq_len, p.T_rows = a.seq_start != nullptr ? a.T_rows : a.NC * C;
-    if (a.V == 512) hipLaunchKernelGGL(chunk_local_grads_kernel<512>, dim3((unsigned)a.chunks), dim3(BWD_THREADS), 0, stream, p);
-    else if (a.V == 256) hipLaunchKernelGGL(chunk_local_grads_kernel<256>, dim3((unsigned)a.chunks), dim3(BWD_THREADS), 0, stream, p);
-    else hipLaunchKernelGGL(chunk_local_grads_kernel<128>, dim3((unsigned)a.chunks), dim3(BWD_THREADS), 0, stream, p);
+    const dim3 grid((unsigned)a.chunks), block(BWD_THREADS);
+    if (a.K == 64) hipLaunchKernelGGL(chunk_local_grads_kernel<64>, grid, block, 0, stream, p);
+    else if (a.K == 128) hipLaunchKernelGGL(chunk_local_grads_kernel<128>, grid, block, 0, stream, p);
+    else hipLaunchKernelGGL(chunk_local_grads_kernel<256>, grid, block, 0, stream, p);
     return (int)hipGetLastError();
 }
 
-bool chunk_bwd_local_supported(const gdn_chunk_local_args& a) { return a.K == BWD_K && (a.V == 128 || a.V == 256 || a.V == 512); }
+bool chunk_bwd_local_supported(const gdn_chunk_local_args& a) { return bwd_shape_built(a.K, a.V); }
 
 bool chunk_bwd_prepare_supported(const gdn_chunk_bwd_prepare_args& a) {
-    if (a.K != BWD_K || (a.V != 128 && a.V != 256 && a.V != 512) || a.T <= 0) return false;
+    if (!bwd_shape_built(a.K, a.V) || a.T <= 0) return false;
     return a.seq_start != nullptr ? (a.seq_len != nullptr && a.NC > 0) : a.T % C == 0;
 }
 
@@ -850,7 +903,7 @@ int launch_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args& a, hipStream_t st
     p.q_stride_b = a.q_stride_b, p.q_stride_t = a.q_stride_t, p.q_stride_h = a.q_stride_h;
     p.k_stride_b = a.k_stride_b, p.k_stride_t = a.k_stride_t, p.k_stride_h = a.k_stride_h;
     p.d_stride_b = a.dout_stride_b, p.d_stride_t = a.dout_stride_t, p.d_stride_h = a.dout_stride_h;
-    p.N = a.N, p.H = a.H, p.NC = a.seq_start != nullptr ? a.NC : a.T / C;
+    p.N = a.N, p.H = a.H, p.V = a.V, p.NC = a.seq_start != nullptr ? a.NC : a.T / C;
     p.seq_start = a.seq_start, p.seq_len = a.seq_len, p.T_rows = a.T;
     p.l2norm = (a.flags & GDN_FLAG_L2NORM) ? 1 : 0;
     p.rec16 = (a.flags & GDN_FLAG_RECORDS_16X16) ? 1 : 0;
@@ -861,9 +914,10 @@ int launch_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args& a, hipStream_t st
     p.rec = static_cast<uint8_t*>(a.records);
     p.rec_bytes = r.bytes, p.off_p = r.off_p, p.off_qs = r.off_qs, p.off_ks = r.off_ks, p.off_cs = r.off_cs, p.off_eg = r.off_eg;
     const int64_t chunks = (int64_t)a.N * a.H * p.NC;
-    if (a.V == 512) hipLaunchKernelGGL(chunk_bwd_prepare_kernel<512>, dim3((unsigned)chunks), dim3(BWD_THREADS), 0, stream, p);
-    else if (a.V == 256) hipLaunchKernelGGL(chunk_bwd_prepare_kernel<256>, dim3((unsigned)chunks), dim3(BWD_THREADS), 0, stream, p);
-    else hipLaunchKernelGGL(chunk_bwd_prepare_kernel<128>, dim3((unsigned)chunks), dim3(BWD_THREADS), 0, stream, p);
+    const dim3 grid((unsigned)chunks), block(BWD_THREADS);
+    if (a.K == 64) hipLaunchKernelGGL(chunk_bwd_prepare_kernel<64>, grid, block, 0, stream, p);
+    else if (a.K == 128) hipLaunchKernelGGL(chunk_bwd_prepare_kernel<128>, grid, block, 0, stream, p);
+    else hipLaunchKernelGGL(chunk_bwd_prepare_kernel<256>, grid, block, 0, stream, p);
     return (int)hipGetLastError();
 }
 

@@ -379,47 +379,16 @@ def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_ch
     return o, ht
 
 
-CHUNK_LOCAL_KV = ((128, 128), (128, 256), (128, 512))  # head dims gdn_chunk_bwd_local and gdn_chunk_bwd_prepare are built for
+def backward_kernels_apply(K: int, V: int) -> bool:
+    """Head dims ``gdn_chunk_bwd_prepare`` and ``gdn_chunk_bwd_local`` are built for."""
+    return K in _SUPPORTED_K and V % 64 == 0
 
 
-def chunk_local_grads(qs, kn, v, dout, y, v_new, states, dstates, gamma, beta, scale, rq=None, rk=None):
-    """``gdn_chunk_bwd_local`` on packed fp32 tensors (``[Bt, NC, 64, K or V]``, states ``[Bt, NC, K, V]``,
-    gamma, beta and the inverse norms rq, rk ``[Bt, NC, 64]``; ``qs = scale * q * rq``, ``kn = k * rk``, without
-    rq and rk q and k were not normalised).  Returns ``dq, dk`` (like qs), ``dbeta, dgamma`` (like gamma)."""
-    _require_hip_path()
-    lib = _lib.load_library()
-    Bt, NC, C, K = qs.shape
-    V = v.size(-1)
-    shapes = {"qs": (Bt, NC, C, K), "kn": (Bt, NC, C, K), "v": (Bt, NC, C, V), "dout": (Bt, NC, C, V),
-              "y": (Bt, NC, C, V), "v_new": (Bt, NC, C, V), "states": (Bt, NC, K, V), "dstates": (Bt, NC, K, V),
-              "gamma": (Bt, NC, C), "beta": (Bt, NC, C), "rq": (Bt, NC, C), "rk": (Bt, NC, C)}  # fmt: skip
-    tensors = dict(qs=qs, kn=kn, v=v, dout=dout, y=y, v_new=v_new, states=states, dstates=dstates, gamma=gamma, beta=beta)
-    if (rq is None) != (rk is None):
-        raise ValueError("rq and rk come together")
-    if rq is not None:
-        tensors.update(rq=rq, rk=rk)
-    for name, x in tensors.items():
-        if tuple(x.shape) != shapes[name] or x.dtype != torch.float32 or not x.is_cuda:
-            raise ValueError(f"{name} must be a device fp32 tensor of shape {shapes[name]}, got {tuple(x.shape)} {x.dtype}")
-        tensors[name] = x.contiguous()
-    if C != 64 or (K, V) not in CHUNK_LOCAL_KV:
-        raise ValueError(f"chunk-local gradients are built for chunk 64 and K, V = {CHUNK_LOCAL_KV}")
-    out = dict(dq=torch.empty_like(tensors["qs"]), dk=torch.empty_like(tensors["kn"]),
-               dbeta=torch.empty_like(tensors["gamma"]), dgamma=torch.empty_like(tensors["gamma"]))  # fmt: skip
-    a = _lib.GdnChunkLocalArgs()
-    for name, x in {**tensors, **out}.items():
-        setattr(a, name, x.data_ptr())
-    a.chunks, a.K, a.V, a.scale = Bt * NC, K, V, float(scale)
-    with torch.cuda.device(qs.device):
-        stream = ctypes.c_void_p(torch.cuda.current_stream(qs.device).cuda_stream)
-        _lib.check_status(lib.gdn_chunk_bwd_local(ctypes.byref(a), stream), "gdn_chunk_bwd_local")
-    return out["dq"], out["dk"], out["dbeta"], out["dgamma"]
-
-
-def chunk_local_grads_final(q, k, v, dout, prep, y_mirror, v_new, states, dstates, scale, l2norm, sequences=None):
-    """``gdn_chunk_bwd_local`` in its final mode: q, k, v, dout are the caller's bf16 ``[B, T, H, D]`` tensors (last
-    dim contiguous), ``prep`` what ``chunk_bwd_prepare`` returned (same ``sequences``), ``y_mirror`` the output of
-    the scan over its mirror problem.  Returns ``dq, dk, dv`` bf16 ``[B, T, H, D]`` and ``dg, dbeta`` fp32
+def chunk_local_grads(q, k, v, dout, prep, y_mirror, v_new, states, dstates, scale, l2norm, sequences=None):
+    """``gdn_chunk_bwd_local``: q, k, v, dout are the caller's bf16 ``[B, T, H, D]`` tensors (last dim contiguous),
+    ``prep`` what ``chunk_bwd_prepare`` returned (same ``sequences``), ``y_mirror`` the output of the scan over its
+    mirror problem, ``v_new`` and ``states`` what the saving forward sweep wrote (both fp32 or both bf16), ``dstates``
+    the states the mirror scan saved (fp32).  Returns ``dq, dk, dv`` bf16 ``[B, T, H, D]`` and ``dg, dbeta`` fp32
     ``[B, T, H]`` (zero where no sequence lives)."""
     _require_hip_path()
     lib = _lib.load_library()
@@ -431,9 +400,14 @@ def chunk_local_grads_final(q, k, v, dout, prep, y_mirror, v_new, states, dstate
     if (sequences is None and (N != B or NC * C != T)) or tuple(y_mirror.shape) != (N, 2 * NC * C, H, V) \
             or y_mirror.dtype != torch.bfloat16 or not y_mirror.is_contiguous():  # fmt: skip
         raise ValueError("y_mirror must be the contiguous bf16 [N, 2 NC 64, H, V] output of the scan over the mirror problem")
-    for name, x, shape in (("v_new", v_new, (Bt, NC, C, V)), ("states", states, (Bt, NC, K, V)), ("dstates", dstates, (Bt, NC, K, V))):
-        if tuple(x.shape) != shape or x.dtype != torch.float32 or not x.is_contiguous():
-            raise ValueError(f"{name} must be contiguous fp32 {shape}")
+    if not backward_kernels_apply(K, V):
+        raise ValueError(f"chunk-local gradients are built for K in {_SUPPORTED_K} and V a multiple of 64, got {K}, {V}")
+    if states.dtype != v_new.dtype or states.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("v_new and states must both be fp32 or both be bf16")
+    for name, x, shape, dtype in (("v_new", v_new, (Bt, NC, C, V), states.dtype), ("states", states, (Bt, NC, K, V), states.dtype),
+                                  ("dstates", dstates, (Bt, NC, K, V), torch.float32)):  # fmt: skip
+        if tuple(x.shape) != shape or x.dtype != dtype or not x.is_contiguous():
+            raise ValueError(f"{name} must be contiguous {dtype} {shape}")
     alloc = torch.empty if sequences is None else torch.zeros  # tokens outside every sequence are not written
     out = dict(
         dq_out=alloc(B, T, H, K, dtype=torch.bfloat16, device=dev),
@@ -447,6 +421,7 @@ def chunk_local_grads_final(q, k, v, dout, prep, y_mirror, v_new, states, dstate
     if l2norm:
         a.rq, a.rk = prep["rq"].data_ptr(), prep["rk"].data_ptr()
     a.v_new, a.states, a.dstates = v_new.data_ptr(), states.data_ptr(), dstates.data_ptr()
+    a.saves_dtype = _dtype_code(states.dtype, "states")
     a.y_mirror = y_mirror.data_ptr()
     for name, x in (("q", q), ("k", k), ("v", v), ("dout", dout)):
         if x.dtype != torch.bfloat16 or x.stride(-1) != 1:
@@ -480,8 +455,8 @@ def chunk_bwd_prepare(q, k, dout, g, beta, scale, l2norm, V, sequences=None, hal
     _require_hip_path()
     lib = _lib.load_library()
     B, T, H, K = q.shape
-    if (K, V) not in CHUNK_LOCAL_KV or q.dtype != torch.bfloat16:
-        raise ValueError(f"built for bf16 and K, V in {CHUNK_LOCAL_KV}")
+    if not backward_kernels_apply(K, V) or q.dtype != torch.bfloat16:
+        raise ValueError(f"built for bf16, K in {_SUPPORTED_K} and V a multiple of 64, got {q.dtype}, {K}, {V}")
     if sequences is None:
         if T % 64 != 0:
             raise ValueError("without `sequences` T must be a multiple of 64")
