@@ -195,16 +195,29 @@ int gdn_recurrent_fwd(const gdn_args *args, void *stream);
  * 16x16x32 MFMA (any K, required for K = 256); the scan then runs one slice per workgroup on two half-slice
  * waves, which is the faster kernel as long as N * H * V / 32 does not exceed the number of compute units.
  * The backward pass of this package runs its reverse sweep over the chunks that way.
+ * states_dtype, v_new_dtype: GDN_F32, or GDN_BF16 (the pointer is then a bf16 array of the same shape).  bf16 saves
+ * need the variant of the scan that stages its saves through LDS, which gdn_chunk_fwd_saving_is_staged reports for
+ * the same arguments (K <= 128 and one column slice per workgroup); GDN_ERR_UNSUPPORTED otherwise.
+ * no_output != 0: the caller does not need args->o (a sweep that is run for its saves); where a variant of the scan
+ * without the products that only serve the output exists (staged saves, K = 128) it runs and args->o, which must
+ * still be a valid buffer, is left unwritten; elsewhere the flag changes nothing.
  */
 typedef struct gdn_chunk_saves {
-    float *states;
-    float *v_new;
+    void *states;
+    void *v_new;
     int32_t chunks_per_chain;
     int32_t records_given;
     int32_t save_every;
     int32_t save_reverse;
+    int32_t states_dtype; /* gdn_dtype of states */
+    int32_t v_new_dtype;  /* gdn_dtype of v_new */
+    int32_t no_output;
+    int32_t reserved;
 } gdn_chunk_saves;
 int gdn_chunk_fwd_saving(const gdn_args *args, const gdn_chunk_saves *saves, void *stream);
+/* 1 when gdn_chunk_fwd_saving would run these arguments (shape fields, flags, cu_seqlens NULL or not, saves->records_given)
+ * on the scan that stages its saves through LDS, on the calling thread's current device; else 0. */
+int gdn_chunk_fwd_saving_is_staged(const gdn_args *args, const gdn_chunk_saves *saves);
 
 /*
  * Training support, second part: the chunk-local gradients, one workgroup per (sequence, head, chunk), once
@@ -218,7 +231,9 @@ int gdn_chunk_fwd_saving(const gdn_args *args, const gdn_chunk_saves *saves, voi
  *     rq, rk        [chunks][64]      1 / sqrt(|q|^2 + 1e-6), likewise for k, when q and k were normalised
  *                                     (the l2norm flag of the forward); both NULL otherwise
  *     y_mirror      bf16 [N, 2 * NC * 64, H, V]: the output of the scan over the mirror problem of
- *                   gdn_chunk_bwd_prepare (Y at its even chunks, tokens reversed)
+ *                   gdn_chunk_bwd_prepare (Y at its even chunks, tokens reversed); or NULL and
+ *     y_chunks      bf16 [chunks][64][V]: the V~ that scan saved at its even chunks (save_every = 2, save_reverse,
+ *                   bf16 saves, no output): Y of chunk (n, h, c) with its tokens in reverse order
  *     q_raw, k_raw, v_raw, dout_raw   the caller's bf16 q, k, v, dO, [N, NC * 64, H, D] with element strides
  * Outputs, in the caller's layout, contiguous: dq_out, dk_out [N, NC * 64, H, K] and dv_out [N, NC * 64, H, V]
  * (bf16; the gradients with respect to q and k themselves, through the scale and the normalisation), dg_out and
@@ -234,7 +249,7 @@ typedef struct gdn_chunk_local_args {
     float scale;
     int64_t chunks;
     int32_t K, V;
-    const void *y_mirror;
+    const void *y_mirror, *y_chunks;
     void *dq_out, *dk_out, *dv_out;
     float *dg_out, *dbeta_out;
     int32_t H, NC;

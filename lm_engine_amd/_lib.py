@@ -44,6 +44,7 @@ EXPORTED_SYMBOLS = (
     "gdn_recurrent_fwd",
     "gdn_chunk_fwd_profile",
     "gdn_chunk_fwd_saving",
+    "gdn_chunk_fwd_saving_is_staged",
     "gdn_chunk_bwd_local",
     "gdn_chunk_bwd_prepare",
     "gdn_causal_conv1d_fwd",
@@ -65,6 +66,10 @@ class GdnChunkSaves(ctypes.Structure):
         ("records_given", ctypes.c_int32),
         ("save_every", ctypes.c_int32),
         ("save_reverse", ctypes.c_int32),
+        ("states_dtype", ctypes.c_int32),
+        ("v_new_dtype", ctypes.c_int32),
+        ("no_output", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
     ]
 
 
@@ -73,7 +78,7 @@ class GdnChunkLocalArgs(ctypes.Structure):
         [(name, ctypes.c_void_p) for name in ("v_new", "states", "dstates", "gamma", "beta", "rq", "rk")]
         + [("saves_dtype", ctypes.c_int32), ("scale", ctypes.c_float), ("chunks", ctypes.c_int64), ("K", ctypes.c_int32),
            ("V", ctypes.c_int32)]
-        + [(name, ctypes.c_void_p) for name in ("y_mirror", "dq_out", "dk_out", "dv_out", "dg_out", "dbeta_out")]
+        + [(name, ctypes.c_void_p) for name in ("y_mirror", "y_chunks", "dq_out", "dk_out", "dv_out", "dg_out", "dbeta_out")]
         + [("H", ctypes.c_int32), ("NC", ctypes.c_int32)]
         + [(name, ctypes.c_void_p) for name in ("q_raw", "k_raw", "v_raw", "dout_raw")]
         + [(f"{x}_stride_{d}", ctypes.c_int64) for x in ("q", "k", "v", "dout") for d in ("b", "t", "h")]
@@ -203,6 +208,8 @@ def load_library() -> ctypes.CDLL:
     lib.gdn_chunk_fwd_profile.restype = ctypes.c_int
     lib.gdn_chunk_fwd_saving.argtypes = [ctypes.POINTER(GdnArgs), ctypes.POINTER(GdnChunkSaves), ctypes.c_void_p]
     lib.gdn_chunk_fwd_saving.restype = ctypes.c_int
+    lib.gdn_chunk_fwd_saving_is_staged.argtypes = [ctypes.POINTER(GdnArgs), ctypes.POINTER(GdnChunkSaves)]
+    lib.gdn_chunk_fwd_saving_is_staged.restype = ctypes.c_int
     lib.gdn_chunk_bwd_local.argtypes = [ctypes.POINTER(GdnChunkLocalArgs), ctypes.c_void_p]
     lib.gdn_chunk_bwd_local.restype = ctypes.c_int
     lib.gdn_chunk_bwd_prepare.argtypes = [ctypes.POINTER(GdnChunkBwdPrepareArgs), ctypes.c_void_p]

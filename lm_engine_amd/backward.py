@@ -357,14 +357,23 @@ def _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, l2norm
     q, k, v, do = (x if x.stride(-1) == 1 else x.contiguous() for x in (q, k, v, do.to(torch.bfloat16)))
     half_slices = K > 128 or ops.half_slice_records_pay(Bt, V, dev)  # K = 256 scans on half-slice waves only
     prep = ops.chunk_bwd_prepare(q, k, do, g, beta, scale, l2norm, V, sequences, half_slice_records=half_slices)
-    S0 = torch.empty(Bt, NC, K, V, device=dev)
-    Vn = torch.empty(Bt, NC, CHUNK, V, device=dev)
-    ops.chunk_forward_saving(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2norm, left_padded, S0, Vn, NC)
+    # Where the saving scan stages its saves through LDS, the sweeps write S0, V~ and Y as bf16 (what the chunk-local
+    # products round them to anyway) and form no output; elsewhere fp32 saves and Y from the mirror scan's output.
+    staged = ops.saving_scan_is_staged(N, T, H, K, V, cu_seqlens, left_padded, 0, dev)
+    saves = dict(dtype=torch.bfloat16 if staged else torch.float32, device=dev)
+    S0 = torch.empty(Bt, NC, K, V, **saves)
+    Vn = torch.empty(Bt, NC, CHUNK, V, **saves)
+    ops.chunk_forward_saving(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2norm, left_padded, S0, Vn, NC,
+                             no_output=staged)  # fmt: skip
     dS1 = torch.empty(Bt, NC, K, V, device=dev)
     dht32 = None if dht is None else dht.to(torch.float32).contiguous()
+    staged_m = ops.saving_scan_is_staged(N, 2 * NC * CHUNK, H, K, V, None, False, 2 if half_slices else 1, dev)
+    Y = torch.empty(Bt, NC, CHUNK, V, dtype=torch.bfloat16, device=dev) if staged_m else None
     o_m, dS = ops.chunk_scan_given_records(prep["k_mirror"], prep["v_mirror"], prep["records"], dht32, dS1, NC,
-                                           save_every=2, save_reverse=True, half_slice_records=half_slices)  # fmt: skip
-    dq, dk, dv, dg, dbeta = ops.chunk_local_grads(q, k, v, do, prep, o_m, Vn, S0, dS1, scale, l2norm, sequences)
+                                           save_every=2, save_reverse=True, half_slice_records=half_slices,
+                                           v_new=Y, no_output=staged_m)  # fmt: skip
+    dq, dk, dv, dg, dbeta = ops.chunk_local_grads(q, k, v, do, prep, Y if staged_m else o_m, Vn, S0, dS1, scale, l2norm,
+                                                  sequences)  # fmt: skip
     return (
         dq,
         dk,

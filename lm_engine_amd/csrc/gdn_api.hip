@@ -185,13 +185,21 @@ int gdn_chunk_fwd_saving(const gdn_args* a, const gdn_chunk_saves* saves, void* 
         need = gdn::chunk_record_bytes(*a);
     }
     if (a->workspace == nullptr || a->workspace_bytes < need || !aligned(a->workspace, 256)) return GDN_ERR_WORKSPACE;
+    if ((saves->states_dtype != GDN_F32 && saves->states_dtype != GDN_BF16) || (saves->v_new_dtype != GDN_F32 && saves->v_new_dtype != GDN_BF16))
+        return GDN_ERR_UNSUPPORTED;
+    if ((saves->states_dtype == GDN_BF16 || saves->v_new_dtype == GDN_BF16) && !gdn::chunk_saving_scan_is_staged(*a, *saves))
+        return GDN_ERR_UNSUPPORTED;
     return gdn::launch_chunk_fwd(*a, static_cast<hipStream_t>(stream), nullptr, saves);
+}
+
+int gdn_chunk_fwd_saving_is_staged(const gdn_args* a, const gdn_chunk_saves* saves) {
+    return a != nullptr && saves != nullptr && gdn::chunk_saving_scan_is_staged(*a, *saves) ? 1 : 0;
 }
 
 int gdn_chunk_bwd_local(const gdn_chunk_local_args* a, void* stream) {
     if (a == nullptr) return GDN_ERR_NULL;
-    const void* needed[] = {a->v_new, a->states, a->dstates, a->gamma, a->beta, a->y_mirror, a->dq_out, a->dk_out,
-                            a->dv_out, a->dg_out, a->dbeta_out, a->q_raw, a->k_raw, a->v_raw, a->dout_raw};
+    const void* needed[] = {a->v_new, a->states, a->dstates, a->gamma, a->beta, a->y_mirror != nullptr ? a->y_mirror : a->y_chunks,
+                            a->dq_out, a->dk_out, a->dv_out, a->dg_out, a->dbeta_out, a->q_raw, a->k_raw, a->v_raw, a->dout_raw};
     for (const void* x : needed)
         if (x == nullptr) return GDN_ERR_NULL;
         else if (!aligned(x, 16)) return GDN_ERR_ALIGN;

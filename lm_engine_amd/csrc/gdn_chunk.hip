@@ -136,6 +136,12 @@ static int compute_units() {
     return cached[dev];
 }
 
+bool chunk_saving_scan_is_staged(const gdn_args& a, const gdn_chunk_saves& saves) {
+    if (!chunk_shape_supported(a)) return false;
+    const bool packed = a.cu_seqlens != nullptr && !(a.flags & GDN_FLAG_LEFT_PADDED);
+    return plan_scan(a.K, (int64_t)a.N * a.H, a.V, packed, true, saves.records_given, compute_units()).staged_saves;
+}
+
 bool chunk_runs_as_one_launch(const gdn_args& a) {
     if (!(a.flags & GDN_FLAG_FUSED_LAUNCH) || !chunk_shape_supported(a)) return false;
     if ((a.K != 64 && a.K != 128) || a.V % 64 != 0 || a.cu_seqlens != nullptr) return false;  // see chunk_fused_supported
@@ -165,8 +171,11 @@ int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events, 
     p.no_producers = (a.flags & GDN_FLAG_DEBUG_NO_PRODUCERS) ? 1 : 0;
     p.rec = static_cast<uint8_t*>(a.workspace) + chunk_off_bytes(a) + chunk_flag_bytes(a);
     p.save_state = nullptr, p.save_vnew = nullptr, p.save_nc = 0, p.records_given = 0, p.save_every = 1, p.save_reverse = 0;
+    p.save_state_bf16 = 0, p.save_vnew_bf16 = 0, p.no_output = 0;
     if (saves != nullptr) {
-        p.save_state = saves->states, p.save_vnew = saves->v_new, p.save_nc = saves->chunks_per_chain;
+        p.save_state = static_cast<float*>(saves->states), p.save_vnew = static_cast<float*>(saves->v_new), p.save_nc = saves->chunks_per_chain;
+        p.save_state_bf16 = saves->states_dtype == GDN_BF16 ? 1 : 0, p.save_vnew_bf16 = saves->v_new_dtype == GDN_BF16 ? 1 : 0;
+        p.no_output = saves->no_output ? 1 : 0;
         p.save_every = saves->save_every > 0 ? saves->save_every : 1, p.save_reverse = saves->save_reverse ? 1 : 0;
         p.records_given = saves->records_given;
         if (p.records_given) p.chunk_off = nullptr, p.seq_order = nullptr, p.ready = nullptr, p.err = nullptr, p.rec = static_cast<uint8_t*>(a.workspace);

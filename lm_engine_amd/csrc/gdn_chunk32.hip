@@ -223,10 +223,12 @@ struct ScanSchedule : ScanScheduleRules<K> {
 // The pieces are half as large as in the whole-slice schedule; placement is the same earliest-deadline walk.  With
 // MFMAs this short an op can be over in 16 cycles, so results are taken DIST ops after their MFMA and LDS data
 // LA ops (operand fragments) or AHEAD ops (scales, rows of v) after the read was issued.
-template <int K>
+// NOOUT: a scan that only carries the state and V~ (the sweeps of the backward pass): the two groups that form the output
+// and the pieces that serve them are left out.
+template <int K, bool NOOUT = false>
 struct Scan16Rules {
     static constexpr int KS = K / 32, KT = K / 16;
-    static constexpr int NSF = 4 * KS, NQF = 4 * KS, NTF = 6, NKF = 2 * KT, NPF = 6;
+    static constexpr int NSF = 4 * KS, NQF = NOOUT ? 0 : 4 * KS, NTF = 6, NKF = 2 * KT, NPF = NOOUT ? 0 : 6;
     static constexpr int NOPS = NSF + NQF + NTF + NKF + NPF;
     static constexpr int LA = 10;
     static constexpr int OP_Q = NSF, OP_T = OP_Q + NQF, OP_K = OP_T + NTF, OP_P = OP_K + NKF, OP_BAR = NOPS - LA;
@@ -252,7 +254,7 @@ struct Scan16Rules {
 
     // pieces: X of a token tile | X of a slab as operand | previous output tile to LDS | q row scale of a tile |
     // decay of a state tile | scaled V~ of a token tile (half an operand) | plain V~ of a slab | new state slab
-    static constexpr int N_XC = 4, N_XB = 2, N_OUT = 4, N_AS = 4, N_DEC = KT, N_VS = 4, N_VB = 2, N_SB = KS;
+    static constexpr int N_XC = 4, N_XB = 2, N_OUT = NOOUT ? 0 : 4, N_AS = NOOUT ? 0 : 4, N_DEC = KT, N_VS = 4, N_VB = NOOUT ? 0 : 2, N_SB = KS;
     static constexpr int P_XC = 0, P_XB = P_XC + N_XC, P_OUT = P_XB + N_XB, P_AS = P_OUT + N_OUT, P_DEC = P_AS + N_AS,
                          P_VS = P_DEC + N_DEC, P_VB = P_VS + N_VS, P_SB = P_VB + N_VB, NPIECES = P_SB + N_SB;
     struct Window {
@@ -282,8 +284,13 @@ struct Scan16Rules {
             const int s = pc - P_VB;
             return {OP_T + t_last(2 * s + 1) + DIST, OP_P + s_first(s)};
         }
+        // The new state slab, from the tiles 2 s and 2 s + 1 that the last group finishes; without the output groups
+        // behind it the last slabs no longer fit this chunk: they are packed at the start of the next one, before the
+        // first MFMA that takes them (op 2 s of K S0; the loop is entered with all slabs packed, so chunk 0 packs them twice)
         const int s = pc - P_SB;
-        return {OP_K + KT + 2 * s + 1 + DIST, NOPS};
+        const int first = OP_K + KT + 2 * s + 1 + DIST;
+        if (NOOUT && first >= NOPS) return {first - NOPS, 2 * s};
+        return {first, NOPS};
     }
     struct Table {
         int op[NPIECES];
@@ -324,9 +331,9 @@ struct Scan16Rules {
     }
 };
 
-template <int K>
-struct Scan16Schedule : Scan16Rules<K> {
-    static constexpr typename Scan16Rules<K>::Table TABLE = Scan16Rules<K>::make();
+template <int K, bool NOOUT = false>
+struct Scan16Schedule : Scan16Rules<K, NOOUT> {
+    static constexpr typename Scan16Rules<K, NOOUT>::Table TABLE = Scan16Rules<K, NOOUT>::make();
     static_assert(TABLE.ok, "no placement of the side work satisfies the windows");
     static constexpr int op_of(int pc) { return TABLE.op[pc]; }
 };
@@ -338,9 +345,13 @@ struct Scan16Schedule : Scan16Rules<K> {
 // A wave has the same number of MFMAs and operand reads as a whole-slice wave but half the accumulators, so half the
 // vector work on them (decay, X, the bf16 copies), and the two halves need nothing from each other.  The records must
 // hold the fragments of T diag(beta) and P in the layout of that instruction (ChunkParams::rec16).
-template <int K, int NW, bool NT = false, bool SAVE = false, bool HALF = false>
+//
+// NOOUT (with SAVE and HALF, K <= 128): the scan writes no output and skips the products that form it; what it saves (the
+// state every chunk starts from, V~) is all it is run for.  The loaders still stage the whole record and the rows of q.
+template <int K, int NW, bool NT = false, bool SAVE = false, bool HALF = false, bool NOOUT = false>
 __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kernel(const ChunkParams p) {
     static_assert(!HALF || NW == 1, "the half-slice scan has one slice per workgroup");
+    static_assert(!NOOUT || (SAVE && HALF && K == 128), "the scan without output is the saving half-slice scan at K = 128");
     // K = 256: two stage halves with the rows of q and k do not fit the LDS.  The rows of q, which a chunk needs for
     // one group of MFMAs only, then get a single buffer and a second workgroup barrier per chunk ("barrier Q"), passed
     // by a compute wave once it holds the last fragment of q: the loaders write the next chunk's rows of q between
@@ -471,6 +482,18 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
                         __builtin_nontemporal_store(rows[i], reinterpret_cast<bf16x8*>(og + ((int64_t)c * C + 16 * i) * p.o_stride_t + 32 * w));
             }
         };
+        // LSAVE, bf16 saves: rows of 32 bf16 columns (64 bytes), 4 lanes per row, 16 rows per instruction
+        auto flush_rows16 = [&](const uint8_t* staged, bf16_t* dst, int rows) {  // dst: row 0, column 0 of this slice
+            const int r0 = lane / 4, piece = lane % 4;
+            for (int r = 0; r < rows; r += 64) {
+                bf16x8 x[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) x[i] = *reinterpret_cast<const bf16x8*>(staged + (r + 16 * i + r0) * (SROW / 2) + 16 * piece);
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    __builtin_nontemporal_store(x[i], reinterpret_cast<bf16x8*>(dst + (int64_t)(r + 16 * i + r0) * p.V + 8 * piece));
+            }
+        };
         // LSAVE: rows of 32 fp32 columns, 8 lanes per row, 8 rows per instruction
         auto flush_rows = [&](const uint8_t* staged, float* dst, int rows) {  // dst: row 0, column 0 of this slice
             const int r0 = lane / 8, piece = lane % 8;
@@ -486,15 +509,21 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
         auto flush_state = [&](int c) {  // the state chunk c starts from
             if constexpr (LSAVE) {
                 const int entry = save_entry(c);
-                if (p.save_state != nullptr && entry >= 0)
-                    flush_rows(sstage[c & 1], p.save_state + ((int64_t)chain * p.save_nc + entry) * K * p.V + 32 * vgroup, K);
+                if (p.save_state != nullptr && entry >= 0) {
+                    const int64_t at = ((int64_t)chain * p.save_nc + entry) * K * p.V + 32 * vgroup;
+                    if (p.save_state_bf16) flush_rows16(sstage[c & 1], reinterpret_cast<bf16_t*>(p.save_state) + at, K);
+                    else flush_rows(sstage[c & 1], p.save_state + at, K);
+                }
             }
         };
         auto flush_vnew = [&](int c) {  // V~ of chunk c
             if constexpr (LSAVE) {
                 const int entry = save_entry(c);
-                if (p.save_vnew != nullptr && entry >= 0)
-                    flush_rows(vstage[c & 1], p.save_vnew + ((int64_t)chain * p.save_nc + entry) * C * p.V + 32 * vgroup, C);
+                if (p.save_vnew != nullptr && entry >= 0) {
+                    const int64_t at = ((int64_t)chain * p.save_nc + entry) * C * p.V + 32 * vgroup;
+                    if (p.save_vnew_bf16) flush_rows16(vstage[c & 1], reinterpret_cast<bf16_t*>(p.save_vnew) + at, C);
+                    else flush_rows(vstage[c & 1], p.save_vnew + at, C);
+                }
             }
         };
         __syncthreads();
@@ -502,10 +531,16 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
             if constexpr (QS) __syncthreads();  // barrier Q
             __syncthreads();  // the state of chunk c, V~ and the output of chunk c - 1 are staged
             flush_state(c);
-            if (c > 0) flush(c - 1), flush_vnew(c - 1);
+            if (c > 0) {
+                if constexpr (!NOOUT) flush(c - 1);
+                flush_vnew(c - 1);
+            }
         }
         __syncthreads();
-        if (nchunks > 0) flush(nchunks - 1), flush_vnew(nchunks - 1);
+        if (nchunks > 0) {
+            if constexpr (!NOOUT) flush(nchunks - 1);
+            flush_vnew(nchunks - 1);
+        }
         return;
     }
     if (is_loader) {
@@ -688,7 +723,7 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
         //     over the tokens 32 s + 4 g + 0..3 and 32 s + 16 + 4 g + 0..3: the reduction order of every fragment of
         //     T diag(beta), P and k^T that multiplies them.
         //   O^T tile it, register r: column c0 + 4 g + r of token 16 it + j.
-        typedef Scan16Schedule<K> SCH;
+        typedef Scan16Schedule<K, NOOUT> SCH;
         constexpr int NOPS = SCH::NOPS, OP_Q = SCH::OP_Q, OP_T = SCH::OP_T, OP_K = SCH::OP_K, OP_P = SCH::OP_P, OP_BAR = SCH::OP_BAR;
         constexpr int LA = SCH::LA, KS = SCH::KS, KT = SCH::KT;
         const int j16 = lane % 16, g = lane / 16;
@@ -752,8 +787,10 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
 
         __syncthreads();  // stage[0] holds chunk 0
         egc = lds_eg(stage[0]);
+        if constexpr (!NOOUT) {
 #pragma unroll
-        for (int it = 0; it < 4; it++) qsc[it] = lds_qs(stage[0], it);
+            for (int it = 0; it < 4; it++) qsc[it] = lds_qs(stage[0], it);
+        }
         static_for<0, LA>([&](auto i) { fnext[decltype(i)::value] = lds_frag(stage[0], i); });
 #pragma unroll
         for (int sl = 0; sl < KS; sl++) sb[sl] = pack4x2(S[2 * sl], S[2 * sl + 1]);
@@ -768,11 +805,19 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
                     // into this chunk's staging buffer (read by the store wave after this chunk's barrier, written again two
                     // chunks on, after the next chunk's barrier)
                     if (p.save_state != nullptr && save_entry(c) >= 0) {
-                        uint8_t* const base = sstage[c & 1] + (8 * g) * SROW + (16 * half + j16) * 4;
+                        if (p.save_state_bf16) {
+                            uint8_t* const base = sstage[c & 1] + (8 * g) * (SROW / 2) + (16 * half + j16) * 2;
 #pragma unroll
-                        for (int t = 0; t < KT; t++)
+                            for (int t = 0; t < KT; t++)
 #pragma unroll
-                            for (int r = 0; r < 4; r++) *reinterpret_cast<float*>(base + (32 * (t / 2) + 4 * (t % 2) + r) * SROW) = S[t][r];
+                                for (int r = 0; r < 4; r++) *reinterpret_cast<bf16_t*>(base + (32 * (t / 2) + 4 * (t % 2) + r) * (SROW / 2)) = (bf16_t)S[t][r];
+                        } else {
+                            uint8_t* const base = sstage[c & 1] + (8 * g) * SROW + (16 * half + j16) * 4;
+#pragma unroll
+                            for (int t = 0; t < KT; t++)
+#pragma unroll
+                                for (int r = 0; r < 4; r++) *reinterpret_cast<float*>(base + (32 * (t / 2) + 4 * (t % 2) + r) * SROW) = S[t][r];
+                        }
                     }
                 } else if (p.save_state != nullptr && c % p.save_every == 0 && c / p.save_every < p.save_nc) {
                     const int entry = p.save_reverse ? p.save_nc - 1 - c / p.save_every : c / p.save_every;
@@ -831,8 +876,10 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
                 if constexpr (op == OP_BAR) {
                     __syncthreads();  // this wave is done with chunk c's half; chunk c + 1 is in the other one
                     egc = lds_eg(stn);
+                    if constexpr (!NOOUT) {
 #pragma unroll
-                    for (int it = 0; it < 4; it++) qsc[it] = lds_qs(stn, it);
+                        for (int it = 0; it < 4; it++) qsc[it] = lds_qs(stn, it);
+                    }
                 }
                 if constexpr (QS && op == OP_T) {
                     // Barrier Q.  The MFMA before this point took the last fragment of q, and LDS reads return in order:
@@ -882,11 +929,19 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
                 if constexpr (LSAVE) {
                     // after this chunk's barrier: the store wave takes it after the next one (or the last)
                     if (p.save_vnew != nullptr && save_entry(c) >= 0) {
-                        uint8_t* const base = vstage[c & 1] + (4 * g) * SROW + (16 * half + j16) * 4;
+                        if (p.save_vnew_bf16) {
+                            uint8_t* const base = vstage[c & 1] + (4 * g) * (SROW / 2) + (16 * half + j16) * 2;
 #pragma unroll
-                        for (int tt = 0; tt < 4; tt++)
+                            for (int tt = 0; tt < 4; tt++)
 #pragma unroll
-                            for (int r = 0; r < 4; r++) *reinterpret_cast<float*>(base + (16 * tt + r) * SROW) = vt[tt][r];
+                                for (int r = 0; r < 4; r++) *reinterpret_cast<bf16_t*>(base + (16 * tt + r) * (SROW / 2)) = (bf16_t)vt[tt][r];
+                        } else {
+                            uint8_t* const base = vstage[c & 1] + (4 * g) * SROW + (16 * half + j16) * 4;
+#pragma unroll
+                            for (int tt = 0; tt < 4; tt++)
+#pragma unroll
+                                for (int r = 0; r < 4; r++) *reinterpret_cast<float*>(base + (16 * tt + r) * SROW) = vt[tt][r];
+                        }
                     }
                 } else if (p.save_vnew != nullptr && c % p.save_every == 0 && c / p.save_every < p.save_nc) {
                     const int entry = p.save_reverse ? p.save_nc - 1 - c / p.save_every : c / p.save_every;
@@ -901,9 +956,11 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
                 }
             }
         }
-        if (nchunks > 0) {
+        if constexpr (!NOOUT) {
+            if (nchunks > 0) {
 #pragma unroll
-            for (int it = 0; it < 4; it++) out_tile(acco[it], (nchunks - 1) & 1, it);
+                for (int it = 0; it < 4; it++) out_tile(acco[it], (nchunks - 1) & 1, it);
+            }
         }
         __syncthreads();  // the store wave writes the last output tile
         if (p.ht != nullptr) {
@@ -1179,6 +1236,35 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
 // ------------------------------------------------------------------------------------------
 int launch_chunk_fused(ChunkParams& p, int K, hipStream_t stream, int num_cus);  // gdn_chunk_fused.hip
 
+// Which scan kernel a launch gets: compute waves (32-column slices) per workgroup, and whether a slice is split over
+// two half-slice waves.
+ScanPlan plan_scan(int K, int64_t chains, int V, bool packed, bool save, int records_given, int num_cus) {
+    // Slices per scan workgroup: one while that gives no more workgroups than CUs, so that every slice has a CU's load
+    // bandwidth to itself; otherwise 2 or 4 slices of a chain share the records through one workgroup's LDS (they must
+    // divide the V / 32 tiles).
+    const int vtiles = V / 32;
+    int nw = 1;
+    while (nw < 4 && vtiles % (2 * nw) == 0 && chains * (vtiles / nw) > (int64_t)num_cus) nw *= 2;
+    // Packed batches are ragged as a rule, and their chains start longest first (chunk_offsets_kernel): the launch then
+    // takes as long as the longest chain, which runs faster the fewer slices share its workgroup, while the workgroups
+    // that do not fit at first fill in behind the short chains.  So up to two workgroups per CU are accepted there.
+    // (Configuration 2, 11 sequences of 202 .. 6350 tokens, H = 16: 246 us with four slices per workgroup, 193 us with two.)
+    if (packed && !save && nw > 1 && chains * (vtiles / (nw / 2)) <= 2 * (int64_t)num_cus) nw /= 2;
+    if (save && nw == 2) nw = 1;  // the saving variant exists for 1 and 4 slices per workgroup
+    // The saving scan of a packed batch (the backward's forward sweep): started longest first as well, its half-slice
+    // variant, whose saves go through LDS, finishes a ragged batch sooner than four slices per workgroup storing from
+    // their compute waves, while there are at most four workgroups per CU (configuration 2: 352 us against 575 us).
+    if (save && packed && !records_given && K <= 128 && chains * vtiles <= 4 * (int64_t)num_cus) nw = 1;
+    if (K > 128) nw = 1;  // K = 256 has the half-slice scan only, also as the saving variant and on given records
+    if (records_given == 2) nw = 1;  // records given in the half-slice scan's fragment order
+    ScanPlan plan;
+    plan.nw = nw;
+    // a slice with a CU to itself is scanned by two waves of 16 columns each; the records are laid out for them
+    plan.half = K > 128 || records_given == 2 || (nw == 1 && !records_given);
+    plan.staged_saves = save && plan.half && K <= 128;
+    return plan;
+}
+
 template <int K>
 static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int num_cus) {
     const int64_t items = (int64_t)((p.TC + 7) / 8) * 8 * p.H;  // a multiple of 8, see the kernel
@@ -1191,29 +1277,14 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
         const int rc = launch_chunk_fused(p, K, stream, num_cus);
         if (rc != GDN_ERR_UNSUPPORTED) return rc;
     }
-    // Compute waves (32-column slices) per scan workgroup: one while that gives no more workgroups than CUs, so
-    // that every slice has a CU's load bandwidth to itself; otherwise 2 or 4 slices of a chain share the
-    // records through one workgroup's LDS (they must divide the V / 32 tiles).
     const int64_t chains = (int64_t)p.N * p.H;
     const int64_t chains8 = (chains + 7) / 8 * 8;
     const int vtiles = p.V / 32;
-    int nw = 1;
-    while (nw < 4 && vtiles % (2 * nw) == 0 && chains * (vtiles / nw) > (int64_t)num_cus) nw *= 2;
     const bool save = p.save_state != nullptr || p.save_vnew != nullptr;
-    // Packed batches are ragged as a rule, and their chains start longest first (chunk_offsets_kernel): the launch then
-    // takes as long as the longest chain, which runs faster the fewer slices share its workgroup, while the workgroups
-    // that do not fit at first fill in behind the short chains.  So up to two workgroups per CU are accepted there.
-    // (Configuration 2, 11 sequences of 202 .. 6350 tokens, H = 16: 246 us with four slices per workgroup, 193 us with two.)
-    if (p.cu_seqlens != nullptr && !save && nw > 1 && chains * (vtiles / (nw / 2)) <= 2 * (int64_t)num_cus) nw /= 2;
-    if (save && nw == 2) nw = 1;  // the saving variant exists for 1 and 4 slices per workgroup
-    // The saving scan of a packed batch (the backward's forward sweep): started longest first as well, its half-slice
-    // variant, whose saves go through LDS, finishes a ragged batch sooner than four slices per workgroup storing from
-    // their compute waves, while there are at most four workgroups per CU (configuration 2: 352 us against 575 us).
-    if (save && p.cu_seqlens != nullptr && !p.records_given && K <= 128 && chains * vtiles <= 4 * (int64_t)num_cus) nw = 1;
-    if constexpr (K > 128) nw = 1;  // K = 256 has the half-slice scan only, also as the saving variant and on given records
-    if (p.records_given == 2) nw = 1;  // records given in the half-slice scan's fragment order
-    // a slice with a CU to itself is scanned by two waves of 16 columns each; the records are laid out for them
-    const bool half = K > 128 || p.records_given == 2 || (nw == 1 && !p.records_given);
+    const ScanPlan plan = plan_scan(K, chains, p.V, p.cu_seqlens != nullptr, save, p.records_given, num_cus);
+    const int nw = plan.nw;
+    const bool half = plan.half;
+    if ((p.save_state_bf16 || p.save_vnew_bf16) && !plan.staged_saves) return GDN_ERR_UNSUPPORTED;  // (the C entry asks plan_scan first)
     p.rec16 = half ? 1 : 0;
     if (!p.records_given) {
         hipLaunchKernelGGL((chunk_prepare32_kernel<K>), dim3(grid_prep), dim3(PREP_THREADS), 0, stream, p);
@@ -1229,6 +1300,7 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     } else {
     if (save) {
         if (nw == 4) hipLaunchKernelGGL((chunk_scan32_kernel<K, 4, false, true>), grid, dim3(scan_waves(4) * WAVE), 0, stream, p);
+        else if (half && p.no_output && K == 128) hipLaunchKernelGGL((chunk_scan32_kernel<128, 1, false, true, true, true>), grid, dim3(scan_waves(1, true) * WAVE), 0, stream, p);
         else if (half) hipLaunchKernelGGL((chunk_scan32_kernel<K, 1, false, true, true>), grid, dim3(scan_waves(1, true) * WAVE), 0, stream, p);
         else hipLaunchKernelGGL((chunk_scan32_kernel<K, 1, false, true>), grid, dim3(scan_waves(1) * WAVE), 0, stream, p);
         return (int)hipGetLastError();

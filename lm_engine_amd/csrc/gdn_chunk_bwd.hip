@@ -58,7 +58,8 @@ struct ChunkLocalParams {
     // chunk = (n H + h) NC + c.  Y is read from the output of the scan over the mirror problem; q, k, v, dO are the
     // caller's tensors (bf16, element strides); the gradients go out in the caller's layout, [N, NC 64, H, .] bf16
     // for q, k, v and fp32 [N, NC 64, H] for g (reverse prefix sum of dgamma done here) and beta
-    const bf16_t* y_mirror;  // [N][2 NC 64][H][V]
+    const bf16_t* y_mirror;  // [N][2 NC 64][H][V], or NULL and
+    const bf16_t* y_chunks;  // [chunk][64][V]: Y of the chunk, tokens reversed
     const bf16_t* q_raw;
     const bf16_t* k_raw;
     const bf16_t* v_raw;
@@ -211,7 +212,9 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
                 bf16x8 vr = *reinterpret_cast<const bf16x8*>(row_of(p.v_raw, p.v_stride_b, p.v_stride_t, p.v_stride_h, row) + v0 + 8 * p8);
                 bf16x8 dr = *reinterpret_cast<const bf16x8*>(row_of(p.d_raw, p.d_stride_b, p.d_stride_t, p.d_stride_h, row) + v0 + 8 * p8);
                 if (!live) vr = zero8, dr = zero8;
-                const bf16x8 yr = *reinterpret_cast<const bf16x8*>(p.y_mirror + ((mirA + (C - 1 - row)) * p.H + h) * V + v0 + 8 * p8);
+                const bf16_t* const yrow = p.y_mirror != nullptr ? p.y_mirror + ((mirA + (C - 1 - row)) * p.H + h) * V
+                                                                 : p.y_chunks + (chunk * C + (C - 1 - row)) * V;
+                const bf16x8 yr = *reinterpret_cast<const bf16x8*>(yrow + v0 + 8 * p8);
                 const float b = p.beta[chunk * C + row];
                 bf16x8 dv;
                 float acc = 0.f;
@@ -864,7 +867,7 @@ int launch_chunk_bwd_local(const gdn_chunk_local_args& a, hipStream_t stream) {
     p.vnew = a.v_new, p.s0 = a.states, p.ds1 = a.dstates, p.saves_bf16 = a.saves_dtype == GDN_BF16 ? 1 : 0;
     p.gam = a.gamma, p.beta = a.beta;
     p.rq = a.rq, p.rk = a.rk, p.scale = a.scale;
-    p.y_mirror = static_cast<const bf16_t*>(a.y_mirror);
+    p.y_mirror = static_cast<const bf16_t*>(a.y_mirror), p.y_chunks = static_cast<const bf16_t*>(a.y_chunks);
     p.dq_out = static_cast<bf16_t*>(a.dq_out), p.dk_out = static_cast<bf16_t*>(a.dk_out), p.dv_out = static_cast<bf16_t*>(a.dv_out);
     p.dg_out = a.dg_out, p.dbeta_out = a.dbeta_out;
     p.H = a.H, p.NC = a.NC, p.V = a.V;

@@ -42,6 +42,8 @@ struct ChunkParams {
     int save_nc;
     int save_every;    // only chunks c with c % save_every == 0 are saved, as entry c / save_every ...
     int save_reverse;  // ... or, when set, as entry save_nc - 1 - c / save_every
+    int save_state_bf16, save_vnew_bf16;  // that array is bf16 (the pointer then points at bf16 data); staged saves only
+    int no_output;     // the scan writes no output (a sweep of the backward pass); staged saves only
     int records_given;  // the records are already in place: prepare is not run
     int32_t* ready;     // [H][TC] one flag per record, for the launch that runs prepare and scan together
     int fused;          // that launch was asked for (GDN_FLAG_FUSED_LAUNCH)
@@ -60,6 +62,14 @@ inline bool fused_launch_window(int64_t chains, int V, int num_cus) {
     const int64_t scan_wgs = (chains + 7) / 8 * 8 * (V / 64);
     return scan_wgs <= (int64_t)num_cus / 2 && scan_wgs >= (int64_t)num_cus * 3 / 8;
 }
+
+// Kernel choice of the scan (plan_scan, gdn_chunk32.hip)
+struct ScanPlan {
+    int nw;             // 32-column slices per workgroup
+    bool half;          // a slice is scanned by two waves of 16 columns (records in the 16x16x32 fragment order)
+    bool staged_saves;  // a saving scan whose saves go through LDS and the store wave: bf16 saves and the scan without output exist there
+};
+ScanPlan plan_scan(int K, int64_t chains, int V, bool packed, bool save, int records_given, int num_cus);
 
 struct RecordLayout {
     uint32_t off_p, off_qs, off_ks, off_cs, off_eg, bytes;

@@ -17,6 +17,7 @@ uint64_t chunk_record_bytes(const gdn_args& a);  // the records alone, [H][chunk
 uint64_t chunk_header_bytes(const gdn_args& a);  // what precedes the records: chunk offsets, error latch, ready flags
 uint64_t chunk_error_latch_offset(const gdn_args& a);  // byte offset of the error latch (an int32) in the workspace
 bool chunk_shape_supported(const gdn_args& a);
+bool chunk_saving_scan_is_staged(const gdn_args& a, const gdn_chunk_saves& saves);  // bf16 saves / no output available
 bool chunk_runs_as_one_launch(const gdn_args& a);  // gdn_chunk_fwd would run prepare and scan as one launch (shape fields, flags, cu_seqlens)
 int launch_chunk_bwd_local(const gdn_chunk_local_args& a, hipStream_t stream);  // gdn_chunk_bwd.hip
 bool chunk_bwd_local_supported(const gdn_chunk_local_args& a);

@@ -312,11 +312,33 @@ def chunk_forward_kernel_times(
     return dict(zip(_lib.CHUNK_KERNEL_NAMES, (float(x) for x in times)))
 
 
+def _save_dtype_code(x, shape, what):
+    if x.dtype not in (torch.float32, torch.bfloat16) or not x.is_contiguous() or tuple(x.shape) != shape:
+        raise ValueError(f"{what} must be a contiguous fp32 or bf16 tensor of shape {shape}")
+    return _dtype_code(x.dtype, what)
+
+
+def saving_scan_is_staged(N, T, H, K, V, cu_seqlens=None, left_padded=False, records_given=0, device=None) -> bool:
+    """Whether ``gdn_chunk_fwd_saving`` runs this batch (``N`` sequences; ``T`` tokens per row, or packed tokens with
+    ``cu_seqlens``) on the scan that stages its saves through LDS: only that one writes bf16 saves and has the mode
+    without output (``gdn_chunk_fwd_saving_is_staged``)."""
+    a = _lib.GdnArgs()
+    packed = cu_seqlens is not None and not left_padded
+    a.B, a.T, a.H, a.K, a.V, a.N = (1 if packed else N), T, H, K, V, N
+    a.chunk, a.dtype = 64, _lib.GDN_BF16
+    a.flags = _lib.GDN_FLAG_LEFT_PADDED if left_padded else 0
+    a.cu_seqlens = None if cu_seqlens is None else cu_seqlens.data_ptr()
+    saves = _lib.GdnChunkSaves(None, None, 1, records_given, 1, 0, _lib.GDN_F32, _lib.GDN_F32, 0, 0)
+    with torch.cuda.device(device):
+        return bool(_lib.load_library().gdn_chunk_fwd_saving_is_staged(ctypes.byref(a), ctypes.byref(saves)))
+
+
 def chunk_forward_saving(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2norm, left_padded, states, v_new,
-                         chunks_per_chain):  # fmt: skip
+                         chunks_per_chain, no_output=False):  # fmt: skip
     """The chunked forward once more, for the backward pass: through ``gdn_chunk_fwd_saving`` it writes the
     state every chunk starts from into ``states`` ``[N * H, chunks_per_chain, K, V]`` and V~ into ``v_new``
-    ``[N * H, chunks_per_chain, 64, V]`` (both fp32, contiguous).  The output itself is discarded."""
+    ``[N * H, chunks_per_chain, 64, V]`` (contiguous; fp32, or bf16 where ``saving_scan_is_staged``).  The output
+    itself is discarded (``no_output``: the library skips forming it where it has a scan without output)."""
     _require_hip_path()
     lib = _lib.load_library()
     dims = _check_inputs(q, k, v, g, beta, initial_state, cu_seqlens, left_padded)
@@ -327,12 +349,12 @@ def chunk_forward_saving(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2n
         beta = beta.contiguous() if beta.dtype in (torch.bfloat16, torch.float32) else beta.float().contiguous()
     cu_seqlens = None if cu_seqlens is None else cu_seqlens.to(torch.int32).contiguous()
     h0 = None if initial_state is None else initial_state.contiguous()
-    for x, rows in ((states, K), (v_new, 64)):
-        if x.dtype != torch.float32 or not x.is_contiguous() or tuple(x.shape) != (N * H, chunks_per_chain, rows, V):
-            raise ValueError(f"save array must be contiguous fp32 {(N * H, chunks_per_chain, rows, V)}")
+    states_code = _save_dtype_code(states, (N * H, chunks_per_chain, K, V), "states")
+    v_new_code = _save_dtype_code(v_new, (N * H, chunks_per_chain, 64, V), "v_new")
     o = torch.empty(B, T, H, V, dtype=v.dtype, device=v.device)
     args = _fill_args(q, k, v, g, beta, h0, None, o, cu_seqlens, scale, l2norm, False, dims, left_padded)
-    saves = _lib.GdnChunkSaves(states.data_ptr(), v_new.data_ptr(), chunks_per_chain, 0, 1, 0)
+    saves = _lib.GdnChunkSaves(states.data_ptr(), v_new.data_ptr(), chunks_per_chain, 0, 1, 0, states_code, v_new_code,
+                               1 if no_output else 0, 0)  # fmt: skip
     with torch.cuda.device(q.device):
         nbytes = lib.gdn_workspace_bytes(ctypes.byref(args))
         workspace = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=q.device)
@@ -350,33 +372,36 @@ def half_slice_records_pay(chains: int, V: int, device) -> bool:
 
 
 def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_chain, save_every=1, save_reverse=False,
-                             half_slice_records=False):
+                             half_slice_records=False, v_new=None, no_output=False):
     """The scan kernel alone over a fixed-length batch whose chunk records the caller has written
     (``records`` uint8 ``[H, B * T / 64, record bytes]``, T a multiple of 64); it reads the rows of ``k`` (also
     in the place of q: such records carry zero row scales for q) and of ``v``.  Returns ``(o, final_state)``
     and writes the state that chunk ``c`` starts from, for every ``c`` divisible by ``save_every``, into entry
     ``c / save_every`` of ``states`` ``[B * H, chunks_per_chain, K, V]`` (counted from the end with
-    ``save_reverse``).  ``half_slice_records``: the fragments of the records are in the lane order of the
-    16x16x32 MFMA (K = 256 needs that) instead of the 32x32x16 one."""
+    ``save_reverse``), and V~ of those chunks into ``v_new`` ``[B * H, chunks_per_chain, 64, V]`` when that is given.
+    ``half_slice_records``: the fragments of the records are in the lane order of the 16x16x32 MFMA (K = 256 needs
+    that) instead of the 32x32x16 one.  bf16 save arrays where ``saving_scan_is_staged``; ``no_output``: the caller
+    does not need ``o`` (None is returned; the library skips forming it where it has a scan without output)."""
     _require_hip_path()
     lib = _lib.load_library()
     dims = _check_inputs(k, k, v, None, None, initial_state, None)
     B, T, H, K, V, N = dims
     if T % 64 != 0 or not records.is_contiguous() or records.dtype != torch.uint8 or tuple(records.shape[:2]) != (H, B * T // 64):
         raise ValueError("records must be contiguous uint8 [H, B * T / 64, record bytes] with T a multiple of 64")
-    if states.dtype != torch.float32 or not states.is_contiguous() or tuple(states.shape) != (B * H, chunks_per_chain, K, V):
-        raise ValueError(f"states must be contiguous fp32 {(B * H, chunks_per_chain, K, V)}")
+    states_code = _save_dtype_code(states, (B * H, chunks_per_chain, K, V), "states")
+    v_new_code = _lib.GDN_F32 if v_new is None else _save_dtype_code(v_new, (B * H, chunks_per_chain, 64, V), "v_new")
     o = torch.empty(B, T, H, V, dtype=v.dtype, device=v.device)
     ht = torch.empty(N, H, K, V, dtype=torch.float32, device=v.device)
     args = _fill_args(k, k, v, None, None, initial_state, ht, o, None, 1.0, False, False, dims)
     args.workspace, args.workspace_bytes = records.data_ptr(), records.numel()
-    saves = _lib.GdnChunkSaves(states.data_ptr(), None, chunks_per_chain, 2 if half_slice_records else 1, save_every,
-                               1 if save_reverse else 0)  # fmt: skip
+    saves = _lib.GdnChunkSaves(states.data_ptr(), None if v_new is None else v_new.data_ptr(), chunks_per_chain,
+                               2 if half_slice_records else 1, save_every, 1 if save_reverse else 0, states_code,
+                               v_new_code, 1 if no_output else 0, 0)  # fmt: skip
     with torch.cuda.device(k.device):
         stream = ctypes.c_void_p(torch.cuda.current_stream(k.device).cuda_stream)
         _lib.check_status(lib.gdn_chunk_fwd_saving(ctypes.byref(args), ctypes.byref(saves), stream),
                           "gdn_chunk_fwd_saving")  # fmt: skip
-    return o, ht
+    return (None if no_output else o), ht
 
 
 def backward_kernels_apply(K: int, V: int) -> bool:
@@ -387,8 +412,9 @@ def backward_kernels_apply(K: int, V: int) -> bool:
 def chunk_local_grads(q, k, v, dout, prep, y_mirror, v_new, states, dstates, scale, l2norm, sequences=None):
     """``gdn_chunk_bwd_local``: q, k, v, dout are the caller's bf16 ``[B, T, H, D]`` tensors (last dim contiguous),
     ``prep`` what ``chunk_bwd_prepare`` returned (same ``sequences``), ``y_mirror`` the output of the scan over its
-    mirror problem, ``v_new`` and ``states`` what the saving forward sweep wrote (both fp32 or both bf16), ``dstates``
-    the states the mirror scan saved (fp32).  Returns ``dq, dk, dv`` bf16 ``[B, T, H, D]`` and ``dg, dbeta`` fp32
+    mirror problem (bf16 ``[N, 2 NC 64, H, V]``) or, as a 4-D tensor, the V~ that scan saved at its even chunks (bf16
+    ``[N H, NC, 64, V]``), ``v_new`` and ``states`` what the saving forward sweep wrote (both fp32 or both bf16),
+    ``dstates`` the states the mirror scan saved (fp32).  Returns ``dq, dk, dv`` bf16 ``[B, T, H, D]`` and ``dg, dbeta`` fp32
     ``[B, T, H]`` (zero where no sequence lives)."""
     _require_hip_path()
     lib = _lib.load_library()
@@ -397,9 +423,11 @@ def chunk_local_grads(q, k, v, dout, prep, y_mirror, v_new, states, dstates, sca
     Bt, NC, C = prep["gamma"].shape
     N = Bt // H
     dev = y_mirror.device
-    if (sequences is None and (N != B or NC * C != T)) or tuple(y_mirror.shape) != (N, 2 * NC * C, H, V) \
+    y_chunked = tuple(y_mirror.shape) == (Bt, NC, C, V)
+    if (sequences is None and (N != B or NC * C != T)) or (not y_chunked and tuple(y_mirror.shape) != (N, 2 * NC * C, H, V)) \
             or y_mirror.dtype != torch.bfloat16 or not y_mirror.is_contiguous():  # fmt: skip
-        raise ValueError("y_mirror must be the contiguous bf16 [N, 2 NC 64, H, V] output of the scan over the mirror problem")
+        raise ValueError("y_mirror must be the contiguous bf16 [N, 2 NC 64, H, V] output of the scan over the mirror "
+                         "problem or the [N H, NC, 64, V] V~ it saved")
     if not backward_kernels_apply(K, V):
         raise ValueError(f"chunk-local gradients are built for K in {_SUPPORTED_K} and V a multiple of 64, got {K}, {V}")
     if states.dtype != v_new.dtype or states.dtype not in (torch.float32, torch.bfloat16):
@@ -422,7 +450,10 @@ def chunk_local_grads(q, k, v, dout, prep, y_mirror, v_new, states, dstates, sca
         a.rq, a.rk = prep["rq"].data_ptr(), prep["rk"].data_ptr()
     a.v_new, a.states, a.dstates = v_new.data_ptr(), states.data_ptr(), dstates.data_ptr()
     a.saves_dtype = _dtype_code(states.dtype, "states")
-    a.y_mirror = y_mirror.data_ptr()
+    if y_chunked:
+        a.y_chunks = y_mirror.data_ptr()
+    else:
+        a.y_mirror = y_mirror.data_ptr()
     for name, x in (("q", q), ("k", k), ("v", v), ("dout", dout)):
         if x.dtype != torch.bfloat16 or x.stride(-1) != 1:
             raise ValueError(f"{name} must be bf16 with a contiguous last dim")
