@@ -301,6 +301,12 @@ typedef struct gdn_chunk_bwd_prepare_args {
     const int32_t *seq_start, *seq_len;
     int32_t NC;
     int32_t reserved;
+    /* optional (whole-chunk batches only: seq_start NULL): the records of the forward pass itself, [H][N * T/64] as
+     * gdn_chunk_fwd's prepare step writes them (fragment order as chosen by GDN_FLAG_RECORDS_16X16), for a forward
+     * sweep through gdn_chunk_fwd_saving with records_given (q, k, v are then the caller's own tensors);
+     * records_fwd_bytes >= H * N * T/64 * 13312 */
+    void *records_fwd;
+    uint64_t records_fwd_bytes;
 } gdn_chunk_bwd_prepare_args;
 int gdn_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args *args, void *stream);
 

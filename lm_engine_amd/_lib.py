@@ -94,7 +94,8 @@ class GdnChunkBwdPrepareArgs(ctypes.Structure):
         + [("scale", ctypes.c_float)]
         + [(name, ctypes.c_void_p) for name in ("gamma", "beta_packed", "rq", "rk", "k_mirror", "v_mirror", "records")]
         + [("records_bytes", ctypes.c_uint64), ("seq_start", ctypes.c_void_p), ("seq_len", ctypes.c_void_p),
-           ("NC", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+           ("NC", ctypes.c_int32), ("reserved", ctypes.c_int32), ("records_fwd", ctypes.c_void_p),
+           ("records_fwd_bytes", ctypes.c_uint64)]
     )  # fmt: skip
 
 

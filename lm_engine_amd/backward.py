@@ -356,15 +356,23 @@ def _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, l2norm
     Bt = N * H
     q, k, v, do = (x if x.stride(-1) == 1 else x.contiguous() for x in (q, k, v, do.to(torch.bfloat16)))
     half_slices = K > 128 or ops.half_slice_records_pay(Bt, V, dev)  # K = 256 scans on half-slice waves only
-    prep = ops.chunk_bwd_prepare(q, k, do, g, beta, scale, l2norm, V, sequences, half_slice_records=half_slices)
+    # a batch of whole chunks gets the forward sweep's records from the same kernel: no prepare launch of its own
+    prep = ops.chunk_bwd_prepare(q, k, do, g, beta, scale, l2norm, V, sequences, half_slice_records=half_slices,
+                                 forward_records=sequences is None)  # fmt: skip
     # Where the saving scan stages its saves through LDS, the sweeps write S0, V~ and Y as bf16 (what the chunk-local
     # products round them to anyway) and form no output; elsewhere fp32 saves and Y from the mirror scan's output.
-    staged = ops.saving_scan_is_staged(N, T, H, K, V, cu_seqlens, left_padded, 0, dev)
+    given = 0 if sequences is not None else 2 if half_slices else 1
+    staged = ops.saving_scan_is_staged(N, T, H, K, V, cu_seqlens, left_padded, given, dev)
     saves = dict(dtype=torch.bfloat16 if staged else torch.float32, device=dev)
     S0 = torch.empty(Bt, NC, K, V, **saves)
     Vn = torch.empty(Bt, NC, CHUNK, V, **saves)
-    ops.chunk_forward_saving(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2norm, left_padded, S0, Vn, NC,
-                             no_output=staged)  # fmt: skip
+    if sequences is None:
+        h0 = None if initial_state is None else initial_state.to(torch.float32).contiguous()
+        ops.chunk_scan_given_records(k, v, prep["records_fwd"], h0, S0, NC, half_slice_records=half_slices, v_new=Vn,
+                                     no_output=True, q=q)  # fmt: skip
+    else:
+        ops.chunk_forward_saving(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2norm, left_padded, S0, Vn, NC,
+                                 no_output=True)  # fmt: skip
     dS1 = torch.empty(Bt, NC, K, V, device=dev)
     dht32 = None if dht is None else dht.to(torch.float32).contiguous()
     staged_m = ops.saving_scan_is_staged(N, 2 * NC * CHUNK, H, K, V, None, False, 2 if half_slices else 1, dev)

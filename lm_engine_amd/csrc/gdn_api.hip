@@ -235,6 +235,10 @@ int gdn_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args* a, void* stream) {
         if (s < 0 || s % 8 != 0) return GDN_ERR_ALIGN;
     if ((int64_t)a->N * a->H * (a->seq_start != nullptr ? a->NC : a->T / 64) > 0x7fffffff) return GDN_ERR_UNSUPPORTED;
     if (!aligned(a->records, 256) || a->records_bytes < gdn::chunk_bwd_record_bytes(*a)) return GDN_ERR_WORKSPACE;
+    if (a->records_fwd != nullptr) {
+        if (a->seq_start != nullptr) return GDN_ERR_VARLEN;  // the forward's records are laid out for whole-chunk batches
+        if (!aligned(a->records_fwd, 256) || a->records_fwd_bytes < gdn::chunk_bwd_record_bytes(*a) / 2) return GDN_ERR_WORKSPACE;
+    }
     return gdn::launch_chunk_bwd_prepare(*a, static_cast<hipStream_t>(stream));
 }
 

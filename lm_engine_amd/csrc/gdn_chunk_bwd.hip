@@ -537,6 +537,7 @@ struct BwdPrepareParams {
     bf16_t* k_m;
     bf16_t* v_m;
     uint8_t* rec;
+    uint8_t* rec_fwd;  // the forward sweep's own records, [H][N NC] (whole-chunk batches), or NULL
     uint32_t rec_bytes, off_p, off_qs, off_ks, off_cs, off_eg;
 };
 
@@ -843,6 +844,33 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_bwd_pre
         reinterpret_cast<bf16x8*>(recB)[fl] = id;
         reinterpret_cast<bf16x8*>(recB + p.off_p)[fl] = zz;
     }
+    if (p.rec_fwd != nullptr) {
+        // The record the forward's prepare step would write for this chunk (T diag(beta), P, the three row scales,
+        // e^{gamma_C}), so that the forward sweep of the backward pass needs no prepare launch of its own.
+        uint8_t* const recF = p.rec_fwd + ((int64_t)h * ((int64_t)p.N * p.NC) + (int64_t)n * p.NC + ci) * p.rec_bytes;
+        for (int fl = t; fl < 6 * WAVE; fl += BWD_THREADS) {
+            const int f = fl / WAVE, L = fl % WAVE;
+            const int row = p.rec16 ? 16 * (f < 2 ? f : 2 + (f - 2) / 2) + L % 16 : 32 * (f < 2 ? 0 : 1) + L % 32;
+            const int col0 = p.rec16 ? 32 * (f < 2 ? 0 : f % 2) + 4 * (L / 16) : 16 * (f < 2 ? f : f - 2) + 4 * (L / 32);
+            const int second = p.rec16 ? 12 : 4;
+            bf16x8 tb, pm;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const int col = col0 + (e < 4 ? e : e + second);
+                tb[e] = (bf16_t)(row >= col ? sA[row * LDA + col] * s_beta[col] : 0.f);
+                pm[e] = (valid > 0 && row >= col) ? sPT[col * LDS64 + row] : (bf16_t)0.f;
+            }
+            reinterpret_cast<bf16x8*>(recF)[fl] = tb;
+            reinterpret_cast<bf16x8*>(recF + p.off_p)[fl] = pm;
+        }
+        if (t < C) {
+            const bool live = t < valid;
+            reinterpret_cast<float*>(recF + p.off_qs)[t] = s_e[t] * s_rq[t] * p.scale;
+            reinterpret_cast<float*>(recF + p.off_ks)[t] = live ? s_tail[t] * s_rk[t] : 0.f;
+            reinterpret_cast<float*>(recF + p.off_cs)[t] = live ? s_e[t] * s_rk[t] : 0.f;
+            if (t == 0) *reinterpret_cast<float*>(recF + p.off_eg) = s_e[C - 1];
+        }
+    }
     if (t < C) {
         const int src = C - 1 - t;
         reinterpret_cast<float*>(recA + p.off_qs)[t] = 0.f;
@@ -915,6 +943,7 @@ int launch_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args& a, hipStream_t st
     p.rq = a.rq, p.rk = a.rk;
     p.k_m = static_cast<bf16_t*>(a.k_mirror), p.v_m = static_cast<bf16_t*>(a.v_mirror);
     p.rec = static_cast<uint8_t*>(a.records);
+    p.rec_fwd = a.seq_start == nullptr ? static_cast<uint8_t*>(a.records_fwd) : nullptr;
     p.rec_bytes = r.bytes, p.off_p = r.off_p, p.off_qs = r.off_qs, p.off_ks = r.off_ks, p.off_cs = r.off_cs, p.off_eg = r.off_eg;
     const int64_t chunks = (int64_t)a.N * a.H * p.NC;
     const dim3 grid((unsigned)chunks), block(BWD_THREADS);

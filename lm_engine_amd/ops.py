@@ -372,10 +372,10 @@ def half_slice_records_pay(chains: int, V: int, device) -> bool:
 
 
 def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_chain, save_every=1, save_reverse=False,
-                             half_slice_records=False, v_new=None, no_output=False):
+                             half_slice_records=False, v_new=None, no_output=False, q=None):
     """The scan kernel alone over a fixed-length batch whose chunk records the caller has written
-    (``records`` uint8 ``[H, B * T / 64, record bytes]``, T a multiple of 64); it reads the rows of ``k`` (also
-    in the place of q: such records carry zero row scales for q) and of ``v``.  Returns ``(o, final_state)``
+    (``records`` uint8 ``[H, B * T / 64, record bytes]``, T a multiple of 64); it reads the rows of ``q``, ``k`` and
+    ``v`` (without ``q``, ``k`` stands in its place: the records of a mirror problem carry zero row scales for q).  Returns ``(o, final_state)``
     and writes the state that chunk ``c`` starts from, for every ``c`` divisible by ``save_every``, into entry
     ``c / save_every`` of ``states`` ``[B * H, chunks_per_chain, K, V]`` (counted from the end with
     ``save_reverse``), and V~ of those chunks into ``v_new`` ``[B * H, chunks_per_chain, 64, V]`` when that is given.
@@ -384,15 +384,17 @@ def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_ch
     does not need ``o`` (None is returned; the library skips forming it where it has a scan without output)."""
     _require_hip_path()
     lib = _lib.load_library()
-    dims = _check_inputs(k, k, v, None, None, initial_state, None)
+    q = k if q is None else q
+    dims = _check_inputs(q, k, v, None, None, initial_state, None)
     B, T, H, K, V, N = dims
+    q, k, v = _last_dim_contiguous(q), _last_dim_contiguous(k), _last_dim_contiguous(v)
     if T % 64 != 0 or not records.is_contiguous() or records.dtype != torch.uint8 or tuple(records.shape[:2]) != (H, B * T // 64):
         raise ValueError("records must be contiguous uint8 [H, B * T / 64, record bytes] with T a multiple of 64")
     states_code = _save_dtype_code(states, (B * H, chunks_per_chain, K, V), "states")
     v_new_code = _lib.GDN_F32 if v_new is None else _save_dtype_code(v_new, (B * H, chunks_per_chain, 64, V), "v_new")
     o = torch.empty(B, T, H, V, dtype=v.dtype, device=v.device)
     ht = torch.empty(N, H, K, V, dtype=torch.float32, device=v.device)
-    args = _fill_args(k, k, v, None, None, initial_state, ht, o, None, 1.0, False, False, dims)
+    args = _fill_args(q, k, v, None, None, initial_state, ht, o, None, 1.0, False, False, dims)
     args.workspace, args.workspace_bytes = records.data_ptr(), records.numel()
     saves = _lib.GdnChunkSaves(states.data_ptr(), None if v_new is None else v_new.data_ptr(), chunks_per_chain,
                                2 if half_slice_records else 1, save_every, 1 if save_reverse else 0, states_code,
@@ -475,14 +477,17 @@ def chunk_local_grads(q, k, v, dout, prep, y_mirror, v_new, states, dstates, sca
 RECORD_BYTES = 13312  # a chunk record: 12 operand fragments, 3 x 64 row scales, e^{gamma_C}
 
 
-def chunk_bwd_prepare(q, k, dout, g, beta, scale, l2norm, V, sequences=None, half_slice_records=False):
+def chunk_bwd_prepare(q, k, dout, g, beta, scale, l2norm, V, sequences=None, half_slice_records=False,
+                      forward_records=False):
     """``gdn_chunk_bwd_prepare``.  ``q, k, dout`` are the caller's bf16 ``[B, T, H, D]`` tensors; without
     ``sequences`` every row is one sequence of whole chunks, else ``sequences = (seq_start, seq_len, NC)``: int32
     device tensors ``[N]`` (first token as a flat index over the rows, length) and the chunks per sequence to lay
     the results out with.  Returns a dict: ``gamma, beta, rq, rk`` (fp32 ``[N H, NC, 64]``: prefix sums of g inside
     the chunks, beta, inverse norms of the rows of q and k) and the mirror problem ``k_mirror, v_mirror``
     ``[N, 2 NC 64, H, D]`` bf16, ``records`` uint8 ``[H, N * 2 NC, RECORD_BYTES]`` (their fragments in the lane order
-    of the 16x16x32 MFMA with ``half_slice_records``, see ``chunk_scan_given_records``)."""
+    of the 16x16x32 MFMA with ``half_slice_records``, see ``chunk_scan_given_records``).  ``forward_records``
+    (whole-chunk batches only): also ``records_fwd`` ``[H, N * NC, RECORD_BYTES]``, the records of the forward pass
+    itself in the same fragment order, for a forward sweep without a prepare launch of its own."""
     _require_hip_path()
     lib = _lib.load_library()
     B, T, H, K = q.shape
@@ -522,6 +527,11 @@ def chunk_bwd_prepare(q, k, dout, g, beta, scale, l2norm, V, sequences=None, hal
     a.gamma, a.beta_packed, a.rq, a.rk = (out[n].data_ptr() for n in ("gamma", "beta", "rq", "rk"))
     a.k_mirror, a.v_mirror, a.records = (out[n].data_ptr() for n in ("k_mirror", "v_mirror", "records"))
     a.records_bytes = out["records"].numel()
+    if forward_records:
+        if sequences is not None:
+            raise ValueError("forward records are written for whole-chunk batches only")
+        out["records_fwd"] = torch.empty(H, N * NC, RECORD_BYTES, dtype=torch.uint8, device=dev)
+        a.records_fwd, a.records_fwd_bytes = out["records_fwd"].data_ptr(), out["records_fwd"].numel()
     if sequences is not None:
         a.seq_start, a.seq_len, a.NC = seq_start.data_ptr(), seq_len.data_ptr(), NC
     with torch.cuda.device(dev):
