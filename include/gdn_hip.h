@@ -197,9 +197,10 @@ int gdn_recurrent_fwd(const gdn_args *args, void *stream);
  * The backward pass of this package runs its reverse sweep over the chunks that way.
  * states_dtype, v_new_dtype: GDN_F32, or GDN_BF16 (the pointer is then a bf16 array of the same shape).  bf16 saves
  * need the variant of the scan that stages its saves through LDS, which gdn_chunk_fwd_saving_is_staged reports for
- * the same arguments (K <= 128 and one column slice per workgroup); GDN_ERR_UNSUPPORTED otherwise.
+ * the same arguments and saves (one column slice per workgroup, and K <= 128; or K = 256 with no_output, bf16 or no
+ * v_new, and states that are bf16 or asked for with save_every >= 2); GDN_ERR_UNSUPPORTED otherwise.
  * no_output != 0: the caller does not need args->o (a sweep that is run for its saves); where a variant of the scan
- * without the products that only serve the output exists (staged saves, K = 128) it runs and args->o, which must
+ * without the products that only serve the output exists (staged saves, K >= 128) it runs and args->o, which must
  * still be a valid buffer, is left unwritten; elsewhere the flag changes nothing.
  */
 typedef struct gdn_chunk_saves {
@@ -215,8 +216,9 @@ typedef struct gdn_chunk_saves {
     int32_t reserved;
 } gdn_chunk_saves;
 int gdn_chunk_fwd_saving(const gdn_args *args, const gdn_chunk_saves *saves, void *stream);
-/* 1 when gdn_chunk_fwd_saving would run these arguments (shape fields, flags, cu_seqlens NULL or not, saves->records_given)
- * on the scan that stages its saves through LDS, on the calling thread's current device; else 0. */
+/* 1 when gdn_chunk_fwd_saving would run these arguments (shape fields, flags, cu_seqlens NULL or not; every field of
+ * saves, its two pointers only as NULL or not) on the scan that stages its saves through LDS, on the calling thread's
+ * current device; else 0. */
 int gdn_chunk_fwd_saving_is_staged(const gdn_args *args, const gdn_chunk_saves *saves);
 
 /*

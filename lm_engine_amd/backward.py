@@ -375,7 +375,8 @@ def _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, l2norm
                                  no_output=True)  # fmt: skip
     dS1 = torch.empty(Bt, NC, K, V, device=dev)
     dht32 = None if dht is None else dht.to(torch.float32).contiguous()
-    staged_m = ops.saving_scan_is_staged(N, 2 * NC * CHUNK, H, K, V, None, False, 2 if half_slices else 1, dev)
+    staged_m = ops.saving_scan_is_staged(N, 2 * NC * CHUNK, H, K, V, None, False, 2 if half_slices else 1, dev,
+                                         states_dtype=torch.float32, save_every=2)  # fmt: skip
     Y = torch.empty(Bt, NC, CHUNK, V, dtype=torch.bfloat16, device=dev) if staged_m else None
     o_m, dS = ops.chunk_scan_given_records(prep["k_mirror"], prep["v_mirror"], prep["records"], dht32, dS1, NC,
                                            save_every=2, save_reverse=True, half_slice_records=half_slices,

@@ -139,7 +139,11 @@ static int compute_units() {
 bool chunk_saving_scan_is_staged(const gdn_args& a, const gdn_chunk_saves& saves) {
     if (!chunk_shape_supported(a)) return false;
     const bool packed = a.cu_seqlens != nullptr && !(a.flags & GDN_FLAG_LEFT_PADDED);
-    return plan_scan(a.K, (int64_t)a.N * a.H, a.V, packed, true, saves.records_given, compute_units()).staged_saves;
+    SaveRequest req;
+    req.no_output = saves.no_output != 0, req.has_state = saves.states != nullptr, req.has_vnew = saves.v_new != nullptr;
+    req.state_bf16 = saves.states_dtype == GDN_BF16, req.vnew_bf16 = saves.v_new_dtype == GDN_BF16;
+    req.save_every = saves.save_every > 0 ? saves.save_every : 1;
+    return plan_scan(a.K, (int64_t)a.N * a.H, a.V, packed, true, saves.records_given, compute_units(), req).staged_saves;
 }
 
 bool chunk_runs_as_one_launch(const gdn_args& a) {

@@ -351,13 +351,16 @@ struct Scan16Schedule : Scan16Rules<K, NOOUT> {
 template <int K, int NW, bool NT = false, bool SAVE = false, bool HALF = false, bool NOOUT = false>
 __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kernel(const ChunkParams p) {
     static_assert(!HALF || NW == 1, "the half-slice scan has one slice per workgroup");
-    static_assert(!NOOUT || (SAVE && HALF && K == 128), "the scan without output is the saving half-slice scan at K = 128");
+    static_assert(!NOOUT || (SAVE && HALF && K >= 128), "the scan without output is the saving half-slice scan at K = 128 or 256");
     // K = 256: two stage halves with the rows of q and k do not fit the LDS.  The rows of q, which a chunk needs for
     // one group of MFMAs only, then get a single buffer and a second workgroup barrier per chunk ("barrier Q"), passed
     // by a compute wave once it holds the last fragment of q: the loaders write the next chunk's rows of q between
     // that barrier and the one at the end of the chunk.
-    constexpr bool QS = K > 128;
-    static_assert(!QS || HALF, "K = 256 runs as half slices");
+    // Without output (NOOUT) no row of q is staged at all: K = 256 then fits two stage halves, needs no barrier Q, and has
+    // room for the staging of the saves.
+    constexpr bool HASQ = !NOOUT;
+    constexpr bool QS = K > 128 && HASQ;
+    static_assert(K <= 128 || HALF, "K = 256 runs as half slices");
     constexpr int NL = SCAN_LOADERS;
     // a separate wave writes the output (see below); with four compute waves the LDS has no room for its staging
     constexpr bool OS = NW < 4;
@@ -375,7 +378,7 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
     constexpr int Q_UNITS = C * 2 * K / FRAG_BYTES;  // 1 KiB pieces of the q rows: 512 / K whole rows each; as many for k
     constexpr int V_OFF = SHARED_BYTES;
     constexpr int Q_OFF = V_OFF + C * VLD;                 // not part of the stage halves when QS
-    constexpr int K_OFF = QS ? Q_OFF : Q_OFF + C * QLD;
+    constexpr int K_OFF = (QS || !HASQ) ? Q_OFF : Q_OFF + C * QLD;
     constexpr int QS_OFF = K_OFF + C * QLD;
     constexpr int KS_OFF = QS_OFF + C * 4;
     constexpr int CS_OFF = KS_OFF + C * 4;
@@ -383,24 +386,34 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
     constexpr int STAGE_BYTES = EG_OFF + 16;
     constexpr int NF = SHARED_FRAGS / NL;  // fragment slots per loader wave
     constexpr int NV = V_UNITS / NL;       // v row slots per loader wave
-    constexpr int NQ = 2 * Q_UNITS / NL;   // q / k row slots per loader wave
+    constexpr int NQ = (HASQ ? 2 : 1) * Q_UNITS / NL;   // q / k row slots per loader wave
     constexpr int NLOAD = NF + NV + NQ;    // 1 KiB moves per loader wave and chunk
     static_assert(SHARED_FRAGS % NL == 0 && V_UNITS % NL == 0 && (2 * Q_UNITS) % NL == 0, "the pieces must divide over the loader waves");
-    static_assert(2 * STAGE_BYTES + (QS ? C * QLD : 0) + (OS ? NW * 2 * C * 64 : 16) <= 160 * 1024, "stage exceeds LDS");
+    constexpr int OSTAGE_BYTES = (OS && !NOOUT) ? NW * 2 * C * 64 : 16;
+    static_assert(2 * STAGE_BYTES + (QS ? C * QLD : 0) + OSTAGE_BYTES <= 160 * 1024, "stage exceeds LDS");
 
     __shared__ __attribute__((aligned(16))) uint8_t stage[2][STAGE_BYTES];
     __shared__ __attribute__((aligned(16))) uint8_t qstage[QS ? C * QLD : 16];  // the single buffer of q rows (QS)
-    __shared__ __attribute__((aligned(16))) uint8_t ostage[OS ? NW * 2 * C * 64 : 16];
+    __shared__ __attribute__((aligned(16))) uint8_t ostage[OSTAGE_BYTES];
     // LSAVE (the saving half-slice scan, K <= 128): the compute waves leave the state a chunk starts from and V~ in LDS, as
     // rows of the slice's 32 fp32 columns, and the store wave writes them out in whole 128-byte lines.  Stores from the
     // compute waves themselves are 64-byte halves of those lines from two waves, and a store that waits for room in the
     // memory queue stalls the wave that feeds the matrix pipe.  Two buffers each, by chunk parity.  (K = 256 has no LDS
     // left for them and stores from its compute waves.)
-    constexpr bool LSAVE = SAVE && HALF && !QS;
-    constexpr int SROW = 32 * 4;  // bytes per staged row
-    __shared__ __attribute__((aligned(16))) uint8_t sstage[LSAVE ? 2 : 1][LSAVE ? K * SROW : 16];
-    __shared__ __attribute__((aligned(16))) uint8_t vstage[LSAVE ? 2 : 1][LSAVE ? C * SROW : 16];
-    static_assert(!LSAVE || 2 * STAGE_BYTES + NW * 2 * C * 64 + 2 * (K + C) * SROW <= 160 * 1024, "the staging of the saves exceeds LDS");
+    // K = 256 (NOOUT only) has half of that room: its states are staged in one buffer when they are fp32 - the launcher
+    // asks for them at every second chunk at most then, so the store wave is done with a state before the next one is
+    // staged - and in two when they are bf16; its V~ is bf16.
+    constexpr bool LSAVE = SAVE && HALF && (K <= 128 || NOOUT);
+    constexpr bool LSAVE_NARROW = LSAVE && K > 128;
+    constexpr int SROW = 32 * 4;  // bytes per staged row of fp32
+    constexpr int SSTAGE_HALF = LSAVE ? (LSAVE_NARROW ? K * SROW / 2 : K * SROW) : 8;
+    constexpr int VSTAGE_HALF = LSAVE ? (LSAVE_NARROW ? C * SROW / 2 : C * SROW) : 8;
+    __shared__ __attribute__((aligned(16))) uint8_t sstage_raw[2 * SSTAGE_HALF];
+    __shared__ __attribute__((aligned(16))) uint8_t vstage_raw[2 * VSTAGE_HALF];
+    static_assert(!LSAVE || 2 * STAGE_BYTES + OSTAGE_BYTES + 2 * SSTAGE_HALF + 2 * VSTAGE_HALF <= 160 * 1024, "the staging of the saves exceeds LDS");
+    // staging buffer of the state chunk c starts from / of its V~ (narrow fp32 states: a single buffer, see above)
+    auto sstage_of = [&](int c) -> uint8_t* { return sstage_raw + ((LSAVE_NARROW && !p.save_state_bf16) ? 0 : (c & 1) * SSTAGE_HALF); };
+    auto vstage_of = [&](int c) -> uint8_t* { return vstage_raw + (c & 1) * VSTAGE_HALF; };
     // entry of the save arrays that chunk c goes to, or -1
     auto save_entry = [&](int c) -> int {
         if (c % p.save_every != 0 || c / p.save_every >= p.save_nc) return -1;
@@ -511,8 +524,8 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
                 const int entry = save_entry(c);
                 if (p.save_state != nullptr && entry >= 0) {
                     const int64_t at = ((int64_t)chain * p.save_nc + entry) * K * p.V + 32 * vgroup;
-                    if (p.save_state_bf16) flush_rows16(sstage[c & 1], reinterpret_cast<bf16_t*>(p.save_state) + at, K);
-                    else flush_rows(sstage[c & 1], p.save_state + at, K);
+                    if (p.save_state_bf16) flush_rows16(sstage_of(c), reinterpret_cast<bf16_t*>(p.save_state) + at, K);
+                    else flush_rows(sstage_of(c), p.save_state + at, K);
                 }
             }
         };
@@ -521,8 +534,8 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
                 const int entry = save_entry(c);
                 if (p.save_vnew != nullptr && entry >= 0) {
                     const int64_t at = ((int64_t)chain * p.save_nc + entry) * C * p.V + 32 * vgroup;
-                    if (p.save_vnew_bf16) flush_rows16(vstage[c & 1], reinterpret_cast<bf16_t*>(p.save_vnew) + at, C);
-                    else flush_rows(vstage[c & 1], p.save_vnew + at, C);
+                    if (p.save_vnew_bf16) flush_rows16(vstage_of(c), reinterpret_cast<bf16_t*>(p.save_vnew) + at, C);
+                    else flush_rows(vstage_of(c), p.save_vnew + at, C);
                 }
             }
         };
@@ -608,10 +621,10 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
                 const int tok = min(c * C + vunit_of(i - NF) * V_ROWS + v_row, (int)seq_len - 1);
                 return reinterpret_cast<const uint8_t*>(vg + (int64_t)tok * p.v_stride_t);
             }
-            // units 0 .. Q_UNITS - 1 are rows of q, the rest rows of k (wave-uniform choice)
+            // units 0 .. Q_UNITS - 1 are rows of q, the rest rows of k (wave-uniform choice); without q all are rows of k
             const int u = qunit_of(i - NF - NV);
-            const bool is_k = u >= Q_UNITS;
-            const int tok = min(c * C + (is_k ? u - Q_UNITS : u) * Q_ROWS + q_row, (int)seq_len - 1);
+            const bool is_k = !HASQ || u >= Q_UNITS;
+            const int tok = min(c * C + ((is_k && HASQ) ? u - Q_UNITS : u) * Q_ROWS + q_row, (int)seq_len - 1);
             return reinterpret_cast<const uint8_t*>((is_k ? kg : qg) + (int64_t)tok * (is_k ? p.k_stride_t : p.q_stride_t));
         };
         auto dst_of = [&](uint8_t* st, int i) -> uint8_t* {
@@ -806,13 +819,13 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
                     // chunks on, after the next chunk's barrier)
                     if (p.save_state != nullptr && save_entry(c) >= 0) {
                         if (p.save_state_bf16) {
-                            uint8_t* const base = sstage[c & 1] + (8 * g) * (SROW / 2) + (16 * half + j16) * 2;
+                            uint8_t* const base = sstage_of(c) + (8 * g) * (SROW / 2) + (16 * half + j16) * 2;
 #pragma unroll
                             for (int t = 0; t < KT; t++)
 #pragma unroll
                                 for (int r = 0; r < 4; r++) *reinterpret_cast<bf16_t*>(base + (32 * (t / 2) + 4 * (t % 2) + r) * (SROW / 2)) = (bf16_t)S[t][r];
                         } else {
-                            uint8_t* const base = sstage[c & 1] + (8 * g) * SROW + (16 * half + j16) * 4;
+                            uint8_t* const base = sstage_of(c) + (8 * g) * SROW + (16 * half + j16) * 4;
 #pragma unroll
                             for (int t = 0; t < KT; t++)
 #pragma unroll
@@ -930,13 +943,13 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
                     // after this chunk's barrier: the store wave takes it after the next one (or the last)
                     if (p.save_vnew != nullptr && save_entry(c) >= 0) {
                         if (p.save_vnew_bf16) {
-                            uint8_t* const base = vstage[c & 1] + (4 * g) * (SROW / 2) + (16 * half + j16) * 2;
+                            uint8_t* const base = vstage_of(c) + (4 * g) * (SROW / 2) + (16 * half + j16) * 2;
 #pragma unroll
                             for (int tt = 0; tt < 4; tt++)
 #pragma unroll
                                 for (int r = 0; r < 4; r++) *reinterpret_cast<bf16_t*>(base + (16 * tt + r) * (SROW / 2)) = (bf16_t)vt[tt][r];
                         } else {
-                            uint8_t* const base = vstage[c & 1] + (4 * g) * SROW + (16 * half + j16) * 4;
+                            uint8_t* const base = vstage_of(c) + (4 * g) * SROW + (16 * half + j16) * 4;
 #pragma unroll
                             for (int tt = 0; tt < 4; tt++)
 #pragma unroll
@@ -1238,7 +1251,7 @@ int launch_chunk_fused(ChunkParams& p, int K, hipStream_t stream, int num_cus); 
 
 // Which scan kernel a launch gets: compute waves (32-column slices) per workgroup, and whether a slice is split over
 // two half-slice waves.
-ScanPlan plan_scan(int K, int64_t chains, int V, bool packed, bool save, int records_given, int num_cus) {
+ScanPlan plan_scan(int K, int64_t chains, int V, bool packed, bool save, int records_given, int num_cus, const SaveRequest& req) {
     // Slices per scan workgroup: one while that gives no more workgroups than CUs, so that every slice has a CU's load
     // bandwidth to itself; otherwise 2 or 4 slices of a chain share the records through one workgroup's LDS (they must
     // divide the V / 32 tiles).
@@ -1261,7 +1274,11 @@ ScanPlan plan_scan(int K, int64_t chains, int V, bool packed, bool save, int rec
     plan.nw = nw;
     // a slice with a CU to itself is scanned by two waves of 16 columns each; the records are laid out for them
     plan.half = K > 128 || records_given == 2 || (nw == 1 && !records_given);
-    plan.staged_saves = save && plan.half && K <= 128;
+    // Saves go through LDS and the store wave in the half-slice scan: always at K <= 128; at K = 256 only in the scan
+    // without output (no rows of q in LDS), with bf16 V~, and fp32 states at every second chunk at most (one buffer).
+    plan.staged_saves = save && plan.half &&
+                        (K <= 128 || (req.no_output && (!req.has_vnew || req.vnew_bf16) && (!req.has_state || req.state_bf16 || req.save_every >= 2)));
+    plan.no_output = plan.staged_saves && req.no_output && K >= 128;
     return plan;
 }
 
@@ -1281,7 +1298,10 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     const int64_t chains8 = (chains + 7) / 8 * 8;
     const int vtiles = p.V / 32;
     const bool save = p.save_state != nullptr || p.save_vnew != nullptr;
-    const ScanPlan plan = plan_scan(K, chains, p.V, p.cu_seqlens != nullptr, save, p.records_given, num_cus);
+    SaveRequest req;
+    req.no_output = p.no_output != 0, req.has_state = p.save_state != nullptr, req.has_vnew = p.save_vnew != nullptr;
+    req.state_bf16 = p.save_state_bf16 != 0, req.vnew_bf16 = p.save_vnew_bf16 != 0, req.save_every = p.save_every;
+    const ScanPlan plan = plan_scan(K, chains, p.V, p.cu_seqlens != nullptr, save, p.records_given, num_cus, req);
     const int nw = plan.nw;
     const bool half = plan.half;
     if ((p.save_state_bf16 || p.save_vnew_bf16) && !plan.staged_saves) return GDN_ERR_UNSUPPORTED;  // (the C entry asks plan_scan first)
@@ -1294,13 +1314,14 @@ static int launch32(ChunkParams& p, hipStream_t stream, hipEvent_t* events, int 
     p.scan_groups = vtiles / nw;
     const dim3 grid((unsigned)(chains8 * p.scan_groups));
     if constexpr (K > 128) {
-        if (save) hipLaunchKernelGGL((chunk_scan32_kernel<K, 1, false, true, true>), grid, dim3(scan_waves(1, true) * WAVE), 0, stream, p);
+        if (save && plan.no_output) hipLaunchKernelGGL((chunk_scan32_kernel<K, 1, false, true, true, true>), grid, dim3(scan_waves(1, true) * WAVE), 0, stream, p);
+        else if (save) hipLaunchKernelGGL((chunk_scan32_kernel<K, 1, false, true, true>), grid, dim3(scan_waves(1, true) * WAVE), 0, stream, p);
         else hipLaunchKernelGGL((chunk_scan32_kernel<K, 1, false, false, true>), grid, dim3(scan_waves(1, true) * WAVE), 0, stream, p);
         return (int)hipGetLastError();
     } else {
     if (save) {
         if (nw == 4) hipLaunchKernelGGL((chunk_scan32_kernel<K, 4, false, true>), grid, dim3(scan_waves(4) * WAVE), 0, stream, p);
-        else if (half && p.no_output && K == 128) hipLaunchKernelGGL((chunk_scan32_kernel<128, 1, false, true, true, true>), grid, dim3(scan_waves(1, true) * WAVE), 0, stream, p);
+        else if (half && plan.no_output && K == 128) hipLaunchKernelGGL((chunk_scan32_kernel<128, 1, false, true, true, true>), grid, dim3(scan_waves(1, true) * WAVE), 0, stream, p);
         else if (half) hipLaunchKernelGGL((chunk_scan32_kernel<K, 1, false, true, true>), grid, dim3(scan_waves(1, true) * WAVE), 0, stream, p);
         else hipLaunchKernelGGL((chunk_scan32_kernel<K, 1, false, true>), grid, dim3(scan_waves(1) * WAVE), 0, stream, p);
         return (int)hipGetLastError();

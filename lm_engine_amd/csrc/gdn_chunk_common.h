@@ -67,9 +67,15 @@ inline bool fused_launch_window(int64_t chains, int V, int num_cus) {
 struct ScanPlan {
     int nw;             // 32-column slices per workgroup
     bool half;          // a slice is scanned by two waves of 16 columns (records in the 16x16x32 fragment order)
-    bool staged_saves;  // a saving scan whose saves go through LDS and the store wave: bf16 saves and the scan without output exist there
+    bool staged_saves;  // a saving scan whose saves go through LDS and the store wave: only there bf16 saves exist
+    bool no_output;     // the scan without output runs
 };
-ScanPlan plan_scan(int K, int64_t chains, int V, bool packed, bool save, int records_given, int num_cus);
+// what a saving launch asks for (gdn_chunk_saves)
+struct SaveRequest {
+    bool no_output = false, has_state = true, has_vnew = true, state_bf16 = false, vnew_bf16 = false;
+    int save_every = 1;
+};
+ScanPlan plan_scan(int K, int64_t chains, int V, bool packed, bool save, int records_given, int num_cus, const SaveRequest& req);
 
 struct RecordLayout {
     uint32_t off_p, off_qs, off_ks, off_cs, off_eg, bytes;

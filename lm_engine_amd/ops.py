@@ -318,17 +318,20 @@ def _save_dtype_code(x, shape, what):
     return _dtype_code(x.dtype, what)
 
 
-def saving_scan_is_staged(N, T, H, K, V, cu_seqlens=None, left_padded=False, records_given=0, device=None) -> bool:
+def saving_scan_is_staged(N, T, H, K, V, cu_seqlens=None, left_padded=False, records_given=0, device=None,
+                          states_dtype=torch.bfloat16, v_new_dtype=torch.bfloat16, save_every=1, no_output=True) -> bool:
     """Whether ``gdn_chunk_fwd_saving`` runs this batch (``N`` sequences; ``T`` tokens per row, or packed tokens with
-    ``cu_seqlens``) on the scan that stages its saves through LDS: only that one writes bf16 saves and has the mode
-    without output (``gdn_chunk_fwd_saving_is_staged``)."""
+    ``cu_seqlens``) and these saves (dtype None: not asked for) on the scan that stages its saves through LDS: only
+    that one writes bf16 saves (``gdn_chunk_fwd_saving_is_staged``)."""
     a = _lib.GdnArgs()
     packed = cu_seqlens is not None and not left_padded
     a.B, a.T, a.H, a.K, a.V, a.N = (1 if packed else N), T, H, K, V, N
     a.chunk, a.dtype = 64, _lib.GDN_BF16
     a.flags = _lib.GDN_FLAG_LEFT_PADDED if left_padded else 0
     a.cu_seqlens = None if cu_seqlens is None else cu_seqlens.data_ptr()
-    saves = _lib.GdnChunkSaves(None, None, 1, records_given, 1, 0, _lib.GDN_F32, _lib.GDN_F32, 0, 0)
+    code = lambda dtype: _lib.GDN_BF16 if dtype == torch.bfloat16 else _lib.GDN_F32  # noqa: E731
+    saves = _lib.GdnChunkSaves(None if states_dtype is None else 1, None if v_new_dtype is None else 1, 1, records_given,
+                               save_every, 0, code(states_dtype), code(v_new_dtype), 1 if no_output else 0, 0)  # fmt: skip
     with torch.cuda.device(device):
         return bool(_lib.load_library().gdn_chunk_fwd_saving_is_staged(ctypes.byref(a), ctypes.byref(saves)))
 
