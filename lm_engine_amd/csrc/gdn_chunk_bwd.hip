@@ -756,6 +756,18 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_bwd_pre
                 *reinterpret_cast<bf16x8*>(p.k_m + tokB * K + 8 * p8) = qr;
             }
         }
+        // the first slab of dO is asked for now: its trip through memory runs beside the products below
+        bf16x8 dpre[4];
+        const bool wide = V >= 128;
+        {
+            const int vpr = wide ? 16 : 8, vrpp = BWD_THREADS / vpr;
+#pragma unroll
+            for (int it = 0; it < 4; it++) {
+                const int row = t / vpr + vrpp * it;
+                dpre[it] = zero8;
+                if (row < C) dpre[it] = *reinterpret_cast<const bf16x8*>(row_of(p.dout, p.d_stride_b, p.d_stride_t, p.d_stride_h, row) + 8 * (t % vpr));
+            }
+        }
         __syncthreads();
 
         f32x16 zero;
@@ -787,7 +799,9 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_bwd_pre
 #pragma unroll
             for (int it = 0; it < C / VRPP; it++) {
                 const int row = t / VPR + VRPP * it;
-                bf16x8 dr = *reinterpret_cast<const bf16x8*>(row_of(p.dout, p.d_stride_b, p.d_stride_t, p.d_stride_h, row) + v0 + 8 * p8);
+                bf16x8 dr;
+                if (v0 == 0) dr = dpre[it];  // (uniform)
+                else dr = *reinterpret_cast<const bf16x8*>(row_of(p.dout, p.d_stride_b, p.d_stride_t, p.d_stride_h, row) + v0 + 8 * p8);
                 if (row >= valid) dr = zero8;
 #pragma unroll
                 for (int e = 0; e < 8; e++) sDOT[(8 * p8 + e) * LDS64 + row] = dr[e];
@@ -795,6 +809,10 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_bwd_pre
             }
             __syncthreads();
             // rows j = 32 tj + .., columns v = v0 + 32 tv + l32, tv = wave, wave + 4, ..
+            // K >= 128: the rows of q and k leave room behind the slab for the 64 x VS result, which then goes out as whole
+            // rows (16 bytes per lane) instead of 2-byte pieces that fill half a line per store
+            constexpr bool STAGED = 2 * C * LDK * 2 >= 128 * LDS64 * 2 + C * 128 * 2;
+            bf16_t* const sU = sQK + 128 * LDS64;  // [64][VS]
 #pragma unroll
             for (int tv = wave; tv < VS / 32; tv += BWD_THREADS / WAVE)
 #pragma unroll
@@ -803,9 +821,18 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_bwd_pre
 #pragma unroll
                     for (int r = 0; r < 16; r++) {
                         const int j = 32 * tj + 8 * (r / 4) + 4 * lh + r % 4;
-                        p.v_m[tok_a(j) * V + v0 + 32 * tv + l32] = (bf16_t)u[r];
+                        if constexpr (STAGED) sU[j * VS + 32 * tv + l32] = (bf16_t)u[r];
+                        else p.v_m[tok_a(j) * V + v0 + 32 * tv + l32] = (bf16_t)u[r];
                     }
                 }
+            if constexpr (STAGED) {
+                __syncthreads();
+#pragma unroll
+                for (int it = 0; it < C / VRPP; it++) {
+                    const int j = t / VPR + VRPP * it;
+                    *reinterpret_cast<bf16x8*>(p.v_m + tok_a(j) * V + v0 + 8 * p8) = *reinterpret_cast<const bf16x8*>(sU + j * VS + 8 * p8);
+                }
+            }
             __syncthreads();  // the slab is free (also for the scratch of the inverse)
         };
         int v0 = 0;
