@@ -58,9 +58,14 @@ struct ChunkParams {
 // The shapes the one-launch forward is used for: its scan workgroups (one per 64 columns of every chain, the chains rounded
 // up to a multiple of 8) fill between 3/8 and 1/2 of the compute units.  With fewer chains the two-kernel path's scan, one
 // slice per CU, is the faster one and prepare is short; with more, too few CUs are left for the producers.
+// And the chains number at least 5/32 of the CUs (40 of 256).  Per chunk of a chain the one-launch scan (a pair of waves
+// per slice, two slices per CU) is ~0.4 us slower than the half-slice scan of the two-kernel path, and what it saves is
+// the prepare kernel, ~0.0115 us per chunk and chain: both grow with the sequence length, so the sign of the difference
+// depends on the number of chains alone.  Measured at steady clocks: 64 chains (B = 4, H = 16, V = 128) 0.111 ms in one
+// launch against 0.114 ms; 32 chains (H = 32, V = 256, T = 65536) 1.645 ms against 1.565 ms.
 inline bool fused_launch_window(int64_t chains, int V, int num_cus) {
     const int64_t scan_wgs = (chains + 7) / 8 * 8 * (V / 64);
-    return scan_wgs <= (int64_t)num_cus / 2 && scan_wgs >= (int64_t)num_cus * 3 / 8;
+    return scan_wgs <= (int64_t)num_cus / 2 && scan_wgs >= (int64_t)num_cus * 3 / 8 && chains * 32 >= (int64_t)num_cus * 5;
 }
 
 // Kernel choice of the scan (plan_scan, gdn_chunk32.hip)

@@ -70,9 +70,9 @@ def test_sequence_lengths_with_tail_chunks(T):
     _check(random_inputs(B=4, T=T, H=16, K=128, V=128, dtype=BF16, seed=150 + T), f"T={T}")
 
 
-@pytest.mark.parametrize("K, V, B", [(64, 64, 8), (64, 128, 4), (128, 64, 8), (128, 256, 2)])
-def test_head_dims(K, V, B):
-    _check(random_inputs(B=B, T=200, H=14, K=K, V=V, dtype=BF16, seed=160 + K + V), f"K={K} V={V}")
+@pytest.mark.parametrize("K, V, B, H", [(64, 64, 8, 14), (64, 128, 4, 14), (128, 64, 8, 14), (128, 192, 4, 10)])
+def test_head_dims(K, V, B, H):
+    _check(random_inputs(B=B, T=200, H=H, K=K, V=V, dtype=BF16, seed=160 + K + V), f"K={K} V={V}")
 
 
 def test_options_l2norm_scale_no_state_ungated():
@@ -97,10 +97,11 @@ def test_config1_full_size():
     _check(make_inputs(get_workload(1)), "cfg1 full size")
 
 
-def test_config4_long_context_and_the_split_property():
-    # H=32, K=128, V=256, random initial state, T=8192 (128 chunks per chain; the full length is checked on the default path)
-    inp = make_inputs(get_workload(4, T=8192))
-    o, ht = _check(inp, "cfg4 at T=8192")
+def test_long_context_and_the_split_property():
+    # configuration 4's distributions (slow decay, random initial state) at T = 8192 (128 chunks per chain) on 64 chains
+    # of V = 128: configuration 4 itself (32 chains of V = 256) runs as two kernels, see test_chunk_gpu.py
+    inp = make_inputs(get_workload(4, B=2, T=8192, V=128))
+    o, ht = _check(inp, "configuration 4's inputs, B=2 V=128 T=8192")
     gpu = _to_gpu(inp)
     cut = 64 * 45
     with enable_kernels(FUSED):
@@ -124,14 +125,15 @@ def test_close_to_the_two_kernel_path_and_fallback_is_unchanged():
         o_fused, h_fused = lm_engine_amd.chunk_gated_delta_rule(**inp, output_final_state=True)
     assert rel_l2(o_fused.float(), o_split.float()) < 5e-3 and rel_l2(h_fused, h_split) < 1e-3
     # shapes that do not qualify take the two-kernel path whatever the flag says: packed sequences, V not a multiple of 64,
-    # more scan workgroups than half of the CUs, fewer than three eighths
+    # more scan workgroups than half of the CUs, fewer than three eighths, too few chains (configuration 4's 32)
     packed = _to_gpu(random_inputs(B=1, T=300, H=2, K=128, V=128, dtype=BF16, seed=181, N=3))
     cu = torch.tensor([0, 70, 71, 300], dtype=torch.int32, device="cuda")
     odd_v = _to_gpu(random_inputs(B=1, T=130, H=2, K=128, V=96, dtype=BF16, seed=182))
     many = _to_gpu(random_inputs(B=20, T=130, H=16, K=128, V=128, dtype=BF16, seed=183))
     few = _to_gpu(random_inputs(B=1, T=300, H=16, K=128, V=128, dtype=BF16, seed=184))
-    assert not any(_qualifies(case) for case in (odd_v, many, few))
-    for case, extra in ((packed, dict(cu_seqlens=cu)), (odd_v, {}), (many, {}), (few, {})):
+    wide = _to_gpu(random_inputs(B=1, T=300, H=32, K=128, V=256, dtype=BF16, seed=185))
+    assert not any(_qualifies(case) for case in (odd_v, many, few, wide))
+    for case, extra in ((packed, dict(cu_seqlens=cu)), (odd_v, {}), (many, {}), (few, {}), (wide, {})):
         with two_kernels():
             a = lm_engine_amd.chunk_gated_delta_rule(**case, output_final_state=True, **extra)
         with enable_kernels(FUSED):
