@@ -95,6 +95,10 @@ def parse_args():
     ap.add_argument("--two-kernels", action="store_true",
                     help="run the headline step and everything after it with prepare and scan as two kernels "
                          "(Kernel.gated_delta_rule_fused_launch off) also where the library would use one launch")
+    ap.add_argument("--cycle-budget", action="store_true",
+                    help="instead of the benchmark: run the headline forward (as two kernels) on the measurement build of the "
+                         "library (python -m lm_engine_amd.build --cycle-budget) and print the shader-clock cycles a compute "
+                         "wave of the half-slice scan spends in each group of MFMAs of its chunk loop")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, the known-size kernel the HBM counters are scaled by")
     return ap.parse_args()
@@ -449,6 +453,51 @@ def cpu_baseline(w, inp_gpu, target_seconds):
     }
 
 
+def cycle_budget(w):
+    """The chunk loop of the half-slice scan, group by group, in shader-clock cycles per chunk: the forward of workload
+    ``w`` as two kernels on ``libgdn_hip_cycles.so``, whose scan reads the clock between its groups of MFMAs (wave 0 of
+    every 16th workgroup reports).  The instrumented loop is a few hundred cycles per chunk slower than the real one
+    (each reading waits for the wave's LDS reads in flight); the kernel's event time in the same build is printed with
+    it, next to the uninstrumented figure of the bench line."""
+    import ctypes
+
+    import torch
+
+    import lm_engine_amd
+    from lm_engine_amd import _lib
+    from lm_engine_amd.build import CYCLE_BUDGET_LIBRARY_PATH
+    from lm_engine_amd.ops import chunk_forward_kernel_times
+    from lm_engine_amd.workloads import make_inputs
+
+    if not os.path.exists(CYCLE_BUDGET_LIBRARY_PATH):
+        raise SystemExit(f"{CYCLE_BUDGET_LIBRARY_PATH} is missing: python -m lm_engine_amd.build --cycle-budget")
+    _lib.LIBRARY_PATH = CYCLE_BUDGET_LIBRARY_PATH  # before the first load
+    lib = _lib.load_library()
+    lib.gdn_cycle_budget_read.argtypes = [ctypes.POINTER(ctypes.c_uint64), ctypes.c_int]
+    lib.gdn_cycle_budget_read.restype = ctypes.c_int
+    inp = make_inputs(w, device="cuda")
+    names = ("k_s0", "s0t_qt", "t_x", "kt_vnew", "vnewt_pt", "between_chunks")
+    with launch_mode(True):
+        call = lambda: lm_engine_amd.chunk_gated_delta_rule(**inp, output_final_state=True)  # noqa: E731
+        device_warmup(call)
+        times = [chunk_forward_kernel_times(**inp, output_final_state=True) for _ in range(10)]
+        call()
+        slots = 16
+        out = (ctypes.c_uint64 * (slots * 8))()
+        _lib.check_status(lib.gdn_cycle_budget_read(out, slots), "gdn_cycle_budget_read")
+    rows = [[out[8 * i + j] for j in range(7)] for i in range(slots)]
+    rows = [r for r in rows if r[6] > 0]
+    per_chunk = {n: round(sum(r[j] / r[6] for r in rows) / len(rows), 1) for j, n in enumerate(names)}
+    scan_ms = sum(t["chunk_scan"] for t in times) / len(times)
+    chunks = rows[0][6]
+    return {
+        "workload": w.name, "kernel": "chunk_scan32_kernel, half-slice compute wave 0", "sampled_workgroups": len(rows),
+        "chunks_per_chain": int(chunks), "cycles_per_chunk": per_chunk, "cycles_per_chunk_total": round(sum(per_chunk.values()), 1),
+        "scan_kernel_ms_instrumented": round(scan_ms, 4),
+        "implied_shader_clock_ghz": round(sum(per_chunk.values()) * chunks / (scan_ms * 1e6), 3),
+    }  # fmt: skip
+
+
 def calibrate_copy():
     """A plain device-to-device copy of 1 GiB: the kernel of known traffic (1 GiB read, 1 GiB written)
     against which FETCH_SIZE / WRITE_SIZE readings of the other kernels are scaled."""
@@ -560,6 +609,9 @@ def main():
         sys.exit(2)
     torch.cuda.set_device(0)
 
+    if args.cycle_budget:
+        print(json.dumps({"cycle_budget": cycle_budget(get_workload(args.workload))}))
+        return
     w = get_workload(args.workload)
     result, inp = bench_chunk(w, args.steps, args.warmup, args.two_kernels)
     decode = None if args.no_decode else bench_decode(args.steps, args.warmup)

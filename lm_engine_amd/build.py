@@ -46,14 +46,28 @@ def _hipcc() -> str:
     return hipcc
 
 
-def build_library(verbose: bool = False, extra_flags: tuple[str, ...] = ()) -> str:
-    """Compiles every source and links the shared library; always rebuilds."""
+CYCLE_BUDGET_LIBRARY_PATH = os.path.join(PACKAGE_DIR, "libgdn_hip_cycles.so")
+CYCLE_BUDGET_SOURCES = ("gdn_api.hip", "gdn_chunk.hip", "gdn_chunk32.hip")  # the sources that read GDN_CYCLE_BUDGET
+
+
+def build_library(verbose: bool = False, extra_flags: tuple[str, ...] = (), cycle_budget: bool = False) -> str:
+    """Compiles every source and links the shared library; always rebuilds.
+
+    ``cycle_budget``: the measurement build instead, ``libgdn_hip_cycles.so`` - the same library with the shader clock
+    read between the groups of MFMAs of the half-slice scan's chunk loop (``-DGDN_CYCLE_BUDGET``; only the sources that
+    read the macro are compiled again, the rest is linked from the objects of the library proper, which must exist).
+    ``bench.py --cycle-budget`` loads it; nothing else does."""
     hipcc = _hipcc()
     build_dir = os.path.join(CSRC_DIR, "build")
     os.makedirs(build_dir, exist_ok=True)
+    sources, library_path, object_dir = SOURCES, LIBRARY_PATH, build_dir
+    if cycle_budget:
+        sources, library_path, object_dir = CYCLE_BUDGET_SOURCES, CYCLE_BUDGET_LIBRARY_PATH, os.path.join(build_dir, "cycles")
+        os.makedirs(object_dir, exist_ok=True)
+        extra_flags = (*extra_flags, "-DGDN_CYCLE_BUDGET")
 
     def compile_one(src: str) -> str:
-        obj = os.path.join(build_dir, src.replace(".hip", ".o"))
+        obj = os.path.join(object_dir, src.replace(".hip", ".o"))
         cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, f"-I{INCLUDE_DIR}", f"-I{CSRC_DIR}", "-c",
                os.path.join(CSRC_DIR, src), "-o", obj]  # fmt: skip
         proc = subprocess.run(cmd, capture_output=True, text=True)
@@ -63,17 +77,19 @@ def build_library(verbose: bool = False, extra_flags: tuple[str, ...] = ()) -> s
             print(proc.stderr, file=sys.stderr)
         return obj
 
-    with ThreadPoolExecutor(max_workers=len(SOURCES)) as pool:
-        objects = list(pool.map(compile_one, SOURCES))
+    with ThreadPoolExecutor(max_workers=len(sources)) as pool:
+        objects = list(pool.map(compile_one, sources))
+    if cycle_budget:
+        objects += [os.path.join(build_dir, src.replace(".hip", ".o")) for src in SOURCES if src not in CYCLE_BUDGET_SOURCES]
 
-    tmp = LIBRARY_PATH + ".tmp"
+    tmp = library_path + ".tmp"
     proc = subprocess.run([hipcc, "-shared", "-fPIC", "--offload-arch=gfx950", "-fno-gpu-rdc", *objects, "-o", tmp],
                           capture_output=True, text=True)  # fmt: skip
     if proc.returncode != 0:
         raise RuntimeError(f"link failed:\n{proc.stdout}\n{proc.stderr}")
-    os.replace(tmp, LIBRARY_PATH)
-    return LIBRARY_PATH
+    os.replace(tmp, library_path)
+    return library_path
 
 
 if __name__ == "__main__":
-    print(build_library(verbose=True))
+    print(build_library(verbose=True, cycle_budget="--cycle-budget" in sys.argv[1:]))

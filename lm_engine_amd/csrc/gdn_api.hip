@@ -17,6 +17,12 @@
 // address): noalloc_scratch() below asks the runtime for the address once per device and hands that out.
 static __device__ __align__(256) unsigned char scratch[GDN_NOALLOC_SCRATCH_BYTES];
 
+#ifdef GDN_CYCLE_BUDGET
+namespace gdn {
+int cycle_budget_read(uint64_t* host, int slots);  // gdn_chunk.hip, measurement build only
+}
+#endif
+
 namespace {
 
 constexpr int MAX_DEVICES = 64;
@@ -257,6 +263,13 @@ int gdn_causal_conv1d_bwd(const gdn_conv_bwd_args* a, void* stream) {
     if ((int64_t)a->B * ((a->S + a->tokens_per_block - 1) / a->tokens_per_block) > 65535) return GDN_ERR_UNSUPPORTED;  // one grid row per block
     return gdn::launch_conv_bwd(*a, static_cast<hipStream_t>(stream));
 }
+
+#ifdef GDN_CYCLE_BUDGET
+// Measurement build only (not declared in gdn_hip.h, not part of libgdn_hip.so): after a chunked forward that ran the
+// half-slice scan, the cycles wave 0 of every 16th scan workgroup spent in each group of its chunk loop, summed over its
+// chunks: out[slot * 8 + 0..5] = K S0 | S0^T q^T | T' X | k^T V~ | V~^T P^T | between chunks, out[slot * 8 + 6] = chunks.
+int gdn_cycle_budget_read(uint64_t* out, int slots) { return gdn::cycle_budget_read(out, slots); }
+#endif
 
 int gdn_chunk_fwd_profile(const gdn_args* a, void* stream, float* kernel_ms) {
     if (kernel_ms == nullptr) return GDN_ERR_NULL;

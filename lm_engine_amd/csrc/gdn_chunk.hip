@@ -152,9 +152,30 @@ bool chunk_runs_as_one_launch(const gdn_args& a) {
     return fused_launch_window((int64_t)a.N * a.H, a.V, compute_units());
 }
 
+#ifdef GDN_CYCLE_BUDGET
+// Measurement build only: a device buffer the sampled waves of the half-slice scan report into (allocated on first use;
+// this build is not the library proper and is free to), and its read-out.
+static uint64_t* cycle_buffer() {
+    static uint64_t* buf = nullptr;
+    if (buf == nullptr && hipMalloc(&buf, GDN_CYCLE_BUDGET_SLOTS * 8 * sizeof(uint64_t)) != hipSuccess) buf = nullptr;
+    return buf;
+}
+int cycle_budget_read(uint64_t* host, int slots) {
+    uint64_t* buf = cycle_buffer();
+    if (buf == nullptr || slots > GDN_CYCLE_BUDGET_SLOTS) return GDN_ERR_WORKSPACE;
+    if (hipError_t e = hipDeviceSynchronize(); e != hipSuccess) return (int)e;
+    return (int)hipMemcpy(host, buf, (size_t)slots * 8 * sizeof(uint64_t), hipMemcpyDeviceToHost);
+}
+#endif
+
 int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events, const gdn_chunk_saves* saves) {
     const RecordLayout r = record_layout(a.K, a.V);
     ChunkParams p;
+    p.cycle_out = nullptr;
+#ifdef GDN_CYCLE_BUDGET
+    p.cycle_out = cycle_buffer();
+    if (p.cycle_out != nullptr) (void)hipMemsetAsync(p.cycle_out, 0, GDN_CYCLE_BUDGET_SLOTS * 8 * sizeof(uint64_t), stream);
+#endif
     p.q = static_cast<const bf16_t*>(a.q);
     p.k = static_cast<const bf16_t*>(a.k);
     p.v = static_cast<const bf16_t*>(a.v);

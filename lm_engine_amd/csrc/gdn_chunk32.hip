@@ -808,6 +808,21 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
 #pragma unroll
         for (int sl = 0; sl < KS; sl++) sb[sl] = pack4x2(S[2 * sl], S[2 * sl + 1]);
 
+#ifdef GDN_CYCLE_BUDGET
+        // Measurement build (python -m lm_engine_amd.build --cycle-budget): the shader clock is read where one group of
+        // MFMAs of the chunk ends and the next begins, and the cycles of each group, side work included, are added up
+        // over the chunks: [K S0 | O^T = S0^T q^T | V~ = T' X | S += k^T V~ | O^T += V~^T P^T | from the last MFMA of a chunk
+        // to the first of the next].  Every reading waits for the wave's LDS reads in flight, which costs the measured
+        // loop a few hundred cycles per chunk.
+        uint64_t cyc[6] = {0, 0, 0, 0, 0, 0};
+        uint64_t cyc_t0 = __builtin_readcyclecounter();
+        auto cyc_tick = [&](int group) {
+            const uint64_t t1 = __builtin_readcyclecounter();
+            cyc[group] += t1 - cyc_t0;
+            cyc_t0 = t1;
+            __builtin_amdgcn_sched_barrier(0);
+        };
+#endif
         for (int c = 0; c < nchunks; c++) {
             const uint8_t* st = stage[c & 1];
             const uint8_t* stn = stage[(c + 1) & 1];
@@ -885,6 +900,13 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
 
             static_for<0, NOPS>([&](auto opc) {
                 constexpr int op = decltype(opc)::value;
+#ifdef GDN_CYCLE_BUDGET
+                if constexpr (op == 0) cyc_tick(5);
+                else if constexpr (op == OP_Q && !NOOUT) cyc_tick(0);
+                else if constexpr (op == OP_T) cyc_tick(NOOUT ? 0 : 1);
+                else if constexpr (op == OP_K) cyc_tick(2);
+                else if constexpr (op == OP_P && !NOOUT) cyc_tick(3);
+#endif
                 if constexpr (op + LA < NOPS) fr[op + LA] = lds_frag(st, std::integral_constant<int, (op + LA < NOPS ? op + LA : 0)>{});
                 if constexpr (op == OP_BAR) {
                     __syncthreads();  // this wave is done with chunk c's half; chunk c + 1 is in the other one
@@ -937,6 +959,9 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
                 }
                 __builtin_amdgcn_sched_barrier(0);
             });
+#ifdef GDN_CYCLE_BUDGET
+            cyc_tick(NOOUT ? 3 : 4);
+#endif
             if constexpr (SAVE) {
                 // V~ of this chunk: tile tt, register r holds token 16 tt + 4 g + r of this lane's column
                 if constexpr (LSAVE) {
@@ -969,6 +994,15 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
                 }
             }
         }
+#ifdef GDN_CYCLE_BUDGET
+        // wave 0 of every 16th workgroup reports: [workgroup / 16][6 groups | chunks]
+        if (p.cycle_out != nullptr && wave == 0 && lane == 0 && blockIdx.x % 16 == 0 && blockIdx.x / 16 < GDN_CYCLE_BUDGET_SLOTS) {
+            uint64_t* out = p.cycle_out + (blockIdx.x / 16) * 8;
+#pragma unroll
+            for (int i = 0; i < 6; i++) out[i] = cyc[i];
+            out[6] = (uint64_t)nchunks;
+        }
+#endif
         if constexpr (!NOOUT) {
             if (nchunks > 0) {
 #pragma unroll

@@ -6,6 +6,7 @@
 namespace gdn {
 
 constexpr int C = 64;  // chunk length
+constexpr int GDN_CYCLE_BUDGET_SLOTS = 64;  // sampled workgroups of the measurement build
 constexpr int PREP_THREADS = 256;
 constexpr int FRAG_BYTES = WAVE * 16;  // one MFMA operand fragment: 8 bf16 per lane
 
@@ -52,6 +53,7 @@ struct ChunkParams {
     int32_t* err_caller;  // the caller's own error word (gdn_args::error_word) or NULL
     uint32_t spin_limit;  // polls of a ready flag before giving up
     int no_producers;     // GDN_FLAG_DEBUG_NO_PRODUCERS
+    uint64_t* cycle_out;  // measurement build (GDN_CYCLE_BUDGET) only: where sampled waves of the half-slice scan report; else NULL
     int rec16;          // the fragments of T diag(beta) and P are laid out for v_mfma_f32_16x16x32_bf16 (the half-slice scan)
 };
 
