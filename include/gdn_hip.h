@@ -415,6 +415,29 @@ typedef struct gdn_gate_args {
 int gdn_gates_fwd(const gdn_gate_args *args, void *stream);
 
 /*
+ * Backward of gdn_gates_fwd (autograd through SoftplusDecayGate.forward, softplus_decay_gate/module.py:69-96, and
+ * `beta = b.sigmoid()`, gated_deltanet/module.py:179-181, when the layer trains): given dg (fp32) and dbeta (dtype),
+ * both [tokens, H] contiguous, it writes da and db ([tokens, H] contiguous, dtype) and the partial sums of the
+ * gradients of A_log and dt_bias left by each of its `partial_blocks` workgroups (1 .. 65535; a few per compute
+ * unit), dA_log_partial and ddt_bias_partial, fp32 [partial_blocks][H], which the caller adds up over the first dim.
+ */
+typedef struct gdn_gate_bwd_args {
+    const void *a, *b;
+    const float *A_log, *dt_bias;
+    const float *dg;
+    const void *dbeta;
+    void *da, *db;
+    float *dA_log_partial, *ddt_bias_partial;
+    int64_t a_stride, b_stride;
+    int64_t tokens;
+    int32_t H;
+    int32_t dtype; /* gdn_dtype of a, b, dbeta, da, db */
+    float beta_scale;
+    int32_t partial_blocks;
+} gdn_gate_bwd_args;
+int gdn_gates_bwd(const gdn_gate_bwd_args *args, void *stream);
+
+/*
  * What the layer does to the operator's output before the output projection, one pass:
  *   y = rmsnorm(o * silu(gate)) * weight   over the V columns of every (token, head)
  * gated_deltanet/module.py:238-242 (`o = o * silu(g)`, `o = self.o_norm(o)`), RMSNorm of

@@ -50,6 +50,7 @@ EXPORTED_SYMBOLS = (
     "gdn_causal_conv1d_fwd",
     "gdn_causal_conv1d_bwd",
     "gdn_gates_fwd",
+    "gdn_gates_bwd",
     "gdn_gated_rmsnorm_fwd",
     "gdn_gated_rmsnorm_bwd",
 )
@@ -154,6 +155,17 @@ class GdnGateArgs(ctypes.Structure):
     )
 
 
+class GdnGateBwdArgs(ctypes.Structure):
+    """Mirror of ``struct gdn_gate_bwd_args``."""
+
+    _fields_ = (
+        [(name, ctypes.c_void_p) for name in ("a", "b", "A_log", "dt_bias", "dg", "dbeta", "da", "db", "dA_log_partial",
+                                              "ddt_bias_partial")]
+        + [(name, ctypes.c_int64) for name in ("a_stride", "b_stride", "tokens")]
+        + [("H", ctypes.c_int32), ("dtype", ctypes.c_int32), ("beta_scale", ctypes.c_float), ("partial_blocks", ctypes.c_int32)]
+    )  # fmt: skip
+
+
 class GdnNormArgs(ctypes.Structure):
     """Mirror of ``struct gdn_norm_args``."""
 
@@ -223,6 +235,8 @@ def load_library() -> ctypes.CDLL:
     lib.gdn_causal_conv1d_bwd.restype = ctypes.c_int
     lib.gdn_gates_fwd.argtypes = [ctypes.POINTER(GdnGateArgs), ctypes.c_void_p]
     lib.gdn_gates_fwd.restype = ctypes.c_int
+    lib.gdn_gates_bwd.argtypes = [ctypes.POINTER(GdnGateBwdArgs), ctypes.c_void_p]
+    lib.gdn_gates_bwd.restype = ctypes.c_int
     lib.gdn_gated_rmsnorm_fwd.argtypes = [ctypes.POINTER(GdnNormArgs), ctypes.c_void_p]
     lib.gdn_gated_rmsnorm_fwd.restype = ctypes.c_int
 

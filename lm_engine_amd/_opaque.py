@@ -201,8 +201,12 @@ def _(a, b, A_log, dt_bias, allow_neg_eigval):
     "(Tensor, Tensor, Tensor, Tensor)",
 )
 def delta_rule_gates_backward(a, b, A_log, dt_bias, dg, dbeta, allow_neg_eigval):
-    # g = -exp(A_log) softplus(a + dt_bias), beta = s sigmoid(b): the derivatives in closed form, fp32 arithmetic
-    # (eager mode lets autograd differentiate the same formula; an operator cannot run autograd inside itself)
+    # g = -exp(A_log) softplus(a + dt_bias), beta = s sigmoid(b)
+    if a.is_cuda and a.dtype in (torch.bfloat16, torch.float32):
+        from . import layer_ops
+
+        return layer_ops._delta_rule_gates_backward(a, b, A_log, dt_bias, dg, dbeta, allow_neg_eigval)
+    # elsewhere: the derivatives in closed form, fp32 arithmetic (an operator cannot run autograd inside itself)
     dg = dg.float()
     rate = -torch.exp(A_log.float())
     z = a.float() + dt_bias.float()
@@ -305,6 +309,15 @@ def gated_delta_rule(mode, q, k, v, g, beta, scale, initial_state, output_final_
 
 
 def depthwise_causal_convolution(x, weight, bias, input_state, attention_mask, output_state, activation):
+    from . import conv
+
+    # Decided while the graph is traced: where a gradient is needed and the backward kernel does not apply (fp32 x,
+    # channels not a multiple of 8, no fused activation, too many token blocks), the convolution goes in as its formula
+    # in torch operations, which the compiler can differentiate - what eager mode does for such inputs - instead of an
+    # operator whose backward would only fail when it is reached.
+    needs_grad = torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (x, weight, bias, input_state))
+    if needs_grad and not conv._backward_kernel_applies(x, weight, activation or None):
+        return conv.convolution_formula(x, weight, bias, input_state, attention_mask, output_state, activation or None)
     y, state = torch.ops.lm_engine_amd.causal_conv1d_forward(x, weight, bias, input_state, attention_mask, output_state,
                                                              activation or "")  # fmt: skip
     return y, (state if output_state else None)

@@ -41,6 +41,60 @@ __global__ __launch_bounds__(256) void gates_kernel(const GateParams p) {
     reinterpret_cast<T*>(p.beta)[idx] = (T)((float)s * p.beta_scale);
 }
 
+// Backward of the gates: with z = a + dt_bias, rate = -exp(A_log), s = sigmoid(b)
+//     da = d_dt_bias terms = dg rate sigmoid(z)       dA_log = sum dg rate softplus(z)       db = dbeta scale s (1 - s)
+// A thread walks the flat (token, head) index with a stride that is a multiple of H, so it stays on one head and keeps
+// that head's two sums in registers; a workgroup leaves them, added up per head in a fixed order, in row blockIdx.x of
+// the two partial arrays, which the caller adds up over the rows.
+struct GateBwdParams {
+    const void* a;
+    const void* b;
+    const float* A_log;
+    const float* dt_bias;
+    const float* dg;
+    const void* dbeta;
+    void* da;
+    void* db;
+    float* dA_part;   // [gridDim.x][H]
+    float* ddt_part;  // [gridDim.x][H]
+    int64_t a_stride, b_stride;
+    int64_t tokens;
+    int H;
+    float beta_scale;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void gates_bwd_kernel(const GateBwdParams p) {
+    __shared__ float s_A[256], s_dt[256];
+    const int64_t n = p.tokens * p.H;
+    const int64_t stride = ((int64_t)gridDim.x * 256 + p.H - 1) / p.H * p.H;  // a multiple of H
+    const int64_t first = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int h = (int)(first % p.H);
+    const float rate = -expf(p.A_log[h]), bias = p.dt_bias[h];
+    float acc_A = 0.f, acc_dt = 0.f;
+    for (int64_t idx = first; idx < n; idx += stride) {
+        const int64_t t = idx / p.H;
+        const float z = (float)reinterpret_cast<const T*>(p.a)[t * p.a_stride + h] + bias;
+        const float b = (float)reinterpret_cast<const T*>(p.b)[t * p.b_stride + h];
+        const float dg = p.dg[idx];
+        const float dz = dg * rate * (1.f / (1.f + expf(-z)));
+        const float s = 1.f / (1.f + expf(-b));
+        reinterpret_cast<T*>(p.da)[idx] = (T)dz;
+        reinterpret_cast<T*>(p.db)[idx] = (T)((float)reinterpret_cast<const T*>(p.dbeta)[idx] * p.beta_scale * s * (1.f - s));
+        acc_A += dg * rate * softplus(z);
+        acc_dt += dz;
+    }
+    s_A[threadIdx.x] = acc_A, s_dt[threadIdx.x] = acc_dt;
+    __syncthreads();
+    for (int hh = threadIdx.x; hh < p.H; hh += 256) {  // thread i of this workgroup sits on head (blockIdx.x * 256 + i) % H
+        float sum_A = 0.f, sum_dt = 0.f;
+        int i = (int)((hh - (int64_t)blockIdx.x * 256 % p.H + p.H) % p.H);
+        for (; i < 256; i += p.H) sum_A += s_A[i], sum_dt += s_dt[i];
+        p.dA_part[(int64_t)blockIdx.x * p.H + hh] = sum_A;
+        p.ddt_part[(int64_t)blockIdx.x * p.H + hh] = sum_dt;
+    }
+}
+
 // 8 consecutive elements <-> fp32, with 16-byte accesses
 __device__ __forceinline__ void load8(const bf16_t* p, float (&x)[8]) {
     const bf16x8 v = *reinterpret_cast<const bf16x8*>(p);
@@ -242,6 +296,23 @@ extern "C" int gdn_gates_fwd(const gdn_gate_args* a, void* stream) {
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (a->dtype == GDN_BF16) hipLaunchKernelGGL((gdn::gates_kernel<gdn::bf16_t>), dim3((unsigned)blocks), dim3(256), 0, st, p);
     else hipLaunchKernelGGL((gdn::gates_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, st, p);
+    return (int)hipGetLastError();
+}
+
+extern "C" int gdn_gates_bwd(const gdn_gate_bwd_args* a, void* stream) {
+    if (a == nullptr || !a->a || !a->b || !a->A_log || !a->dt_bias || !a->dg || !a->dbeta || !a->da || !a->db || !a->dA_log_partial ||
+        !a->ddt_bias_partial)
+        return GDN_ERR_NULL;
+    if (a->tokens <= 0 || a->H <= 0 || a->partial_blocks <= 0 || a->partial_blocks > 65535) return GDN_ERR_SHAPE;
+    if (a->a_stride < a->H || a->b_stride < a->H) return GDN_ERR_SHAPE;
+    if (a->dtype != GDN_BF16 && a->dtype != GDN_F32) return GDN_ERR_UNSUPPORTED;
+    gdn::GateBwdParams p;
+    p.a = a->a, p.b = a->b, p.A_log = a->A_log, p.dt_bias = a->dt_bias, p.dg = a->dg, p.dbeta = a->dbeta;
+    p.da = a->da, p.db = a->db, p.dA_part = a->dA_log_partial, p.ddt_part = a->ddt_bias_partial;
+    p.a_stride = a->a_stride, p.b_stride = a->b_stride, p.tokens = a->tokens, p.H = a->H, p.beta_scale = a->beta_scale;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (a->dtype == GDN_BF16) hipLaunchKernelGGL((gdn::gates_bwd_kernel<gdn::bf16_t>), dim3((unsigned)a->partial_blocks), dim3(256), 0, st, p);
+    else hipLaunchKernelGGL((gdn::gates_bwd_kernel<float>), dim3((unsigned)a->partial_blocks), dim3(256), 0, st, p);
     return (int)hipGetLastError();
 }
 

@@ -70,7 +70,59 @@ def delta_rule_gates(
         return gates_formula(a, b, A_log, dt_bias, allow_neg_eigval)
 
     kernel = lambda a, b, A_log, dt_bias: _delta_rule_gates(a, b, A_log, dt_bias, allow_neg_eigval)  # noqa: E731
+    needs_grad = torch.is_grad_enabled() and any(t.requires_grad for t in (a, b, A_log, dt_bias))
+    if needs_grad and a.is_cuda and a.dtype in (torch.bfloat16, torch.float32):
+        return _GatesOnKernels.apply(a, b, A_log, dt_bias, allow_neg_eigval)
     return kernel_with_formula_backward(kernel, formula, a, b, A_log, dt_bias)
+
+
+class _GatesOnKernels(torch.autograd.Function):
+    """Forward and backward on the HIP kernels."""
+
+    @staticmethod
+    def forward(ctx, a, b, A_log, dt_bias, allow_neg_eigval):
+        ctx.save_for_backward(a, b, A_log, dt_bias)
+        ctx.allow_neg_eigval = allow_neg_eigval
+        return _delta_rule_gates(a, b, A_log, dt_bias, allow_neg_eigval)
+
+    @staticmethod
+    def backward(ctx, dg, dbeta):
+        a, b, A_log, dt_bias = ctx.saved_tensors
+        return (*_delta_rule_gates_backward(a, b, A_log, dt_bias, dg, dbeta, ctx.allow_neg_eigval), None)
+
+
+def _delta_rule_gates_backward(a, b, A_log, dt_bias, dg, dbeta, allow_neg_eigval):
+    """``gdn_gates_bwd``: gradients with respect to a, b (contiguous, their dtype), A_log and dt_bias."""
+    _require(a, "a")
+    H = a.size(-1)
+    a2, a_stride = _token_rows(a, H, "a")
+    b2, b_stride = _token_rows(b, H, "b")
+    tokens = a2.size(0)
+    dev = a.device
+    dg = (torch.zeros(a.shape, dtype=torch.float32, device=dev) if dg is None else dg.to(torch.float32)).contiguous()
+    dbeta = (torch.zeros(a.shape, dtype=a.dtype, device=dev) if dbeta is None else dbeta.to(a.dtype)).contiguous()
+    da = torch.empty(a.shape, dtype=a.dtype, device=dev)
+    db = torch.empty(a.shape, dtype=a.dtype, device=dev)
+    if tokens == 0:
+        return da, db, torch.zeros_like(A_log), torch.zeros_like(dt_bias)
+    blocks = min(1024, max(1, (tokens * H + 255) // 256))
+    parts = torch.empty(2, blocks, H, dtype=torch.float32, device=dev)
+    A32 = A_log.to(device=dev, dtype=torch.float32).contiguous()
+    dt32 = dt_bias.to(device=dev, dtype=torch.float32).contiguous()
+    args = _lib.GdnGateBwdArgs()
+    args.a, args.b, args.A_log, args.dt_bias = a2.data_ptr(), b2.data_ptr(), A32.data_ptr(), dt32.data_ptr()
+    args.dg, args.dbeta, args.da, args.db = dg.data_ptr(), dbeta.data_ptr(), da.data_ptr(), db.data_ptr()
+    args.dA_log_partial, args.ddt_bias_partial = parts[0].data_ptr(), parts[1].data_ptr()
+    args.a_stride, args.b_stride, args.tokens, args.H = a_stride, b_stride, tokens, H
+    args.dtype = _dtype_code(a.dtype, "a, b")
+    args.beta_scale = 2.0 if allow_neg_eigval else 1.0
+    args.partial_blocks = blocks
+    lib = _lib.load_library()
+    with torch.cuda.device(dev):
+        stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+        _lib.check_status(lib.gdn_gates_bwd(ctypes.byref(args), stream), "gdn_gates_bwd")
+    # two results that share no storage (an operator's outputs must not alias each other)
+    return da, db, parts[0].sum(dim=0).to(A_log.dtype), parts[1].sum(dim=0).to(dt_bias.dtype)
 
 
 def _delta_rule_gates(a, b, A_log, dt_bias, allow_neg_eigval):

@@ -119,3 +119,24 @@ def test_whole_layer_is_one_graph_forward_and_backward(S):
     for name in eager_in:
         assert comp_in[name].grad is not None, name
         _same_gradient(comp_in[name].grad, eager_in[name].grad, name)
+
+
+def test_compiled_convolution_without_a_backward_kernel_differentiates_its_formula():
+    """fp32 inputs and a convolution without activation have no backward kernel: under capture they go in as torch
+    operations (decided at trace time), so forward + backward compile and agree with eager mode."""
+    gen = torch.Generator().manual_seed(77)
+    for dtype, activation in ((torch.float32, "silu"), (BF16, None)):
+        x = torch.randn(2, 70, 64, generator=gen).to(dtype).cuda()
+        w = (0.3 * torch.randn(64, 1, 4, generator=gen)).to(dtype).cuda()
+
+        def run(fn):
+            xs, ws = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+            y, _ = fn(xs, ws)
+            (y.float() * torch.arange(y.numel(), device="cuda").view_as(y).float().cos()).sum().backward()
+            return y, xs.grad, ws.grad
+
+        f = lambda xs, ws: lm_engine_amd.depthwise_causal_convolution(xs, ws, None, None, None, False, activation)  # noqa: E731
+        eager = run(f)
+        compiled = run(torch.compile(f, backend="aot_eager", fullgraph=True))
+        for name, a, b in zip(("y", "dx", "dw"), compiled, eager):
+            assert torch.allclose(a.float(), b.float(), rtol=2e-2, atol=2e-2), f"{dtype} {activation} {name}"

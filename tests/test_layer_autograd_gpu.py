@@ -36,15 +36,46 @@ def _compare(got, want, tol, names):
         assert err <= tol, f"{name}: rel-L2 {err:.3e} > {tol}"
 
 
-def test_gates_gradients():
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 6e-3)])
+@pytest.mark.parametrize("shape,H", [((3, 50), 8), ((2, 1031), 12), ((777,), 40)])
+def test_gates_gradients(dtype, tol, shape, H):
+    """The gates' backward kernel (da, db per token, dA_log and ddt_bias reduced over tokens) against autograd
+    through the fp64 oracle, on the values the kernel reads (bf16 inputs are rounded first); a and b are column
+    slices of one wider projection, as the layer hands them over."""
     gen = torch.Generator().manual_seed(1)
-    H = 8
-    a, b = torch.randn(3, 50, H, generator=gen), torch.randn(3, 50, H, generator=gen)
+    proj = torch.randn(*shape, 2 * H + 3, generator=gen).to(dtype)
     A_log, dt_bias = torch.randn(H, generator=gen), torch.randn(H, generator=gen)
-    cg, cb = torch.randn(3, 50, H, generator=gen), torch.randn(3, 50, H, generator=gen)
-    want = _grads(lambda *t: delta_rule_gates_ref(*t, True), [x.to(F64) for x in (a, b, A_log, dt_bias)], [cg.to(F64), cb.to(F64)])
-    got = _grads(lambda *t: lm_engine_amd.delta_rule_gates(*t, True), [x.cuda() for x in (a, b, A_log, dt_bias)], [cg.cuda(), cb.cuda()])
-    _compare(got, want, 1e-5, ("da", "db", "dA_log", "ddt_bias"))
+    cg, cb = torch.randn(*shape, H, generator=gen), torch.randn(*shape, H, generator=gen).to(dtype)
+    cut = lambda p: (p[..., :H], p[..., H + 3 :])  # noqa: E731
+
+    def ref(p, A, d):
+        return delta_rule_gates_ref(*cut(p), A, d, True)
+
+    def ours(p, A, d):
+        return lm_engine_amd.delta_rule_gates(*cut(p), A, d, True)
+
+    want = _grads(ref, [x.to(F64) for x in (proj, A_log, dt_bias)], [cg.to(F64), cb.to(F64)])
+    got = _grads(ours, [x.cuda() for x in (proj, A_log, dt_bias)], [cg.cuda(), cb.cuda()])
+    keep = torch.ones(2 * H + 3, dtype=torch.bool)
+    keep[H : H + 3] = False
+    assert torch.count_nonzero(got[0][..., ~keep]) == 0
+    _compare([got[0][..., keep], *got[1:]], [want[0][..., keep], *want[1:]], tol, ("da|db", "dA_log", "ddt_bias"))
+
+
+def test_gates_gradient_of_one_output_only():
+    gen = torch.Generator().manual_seed(4)
+    H = 16
+    a, b = torch.randn(5, 33, H, generator=gen), torch.randn(5, 33, H, generator=gen)
+    A_log, dt_bias = torch.randn(H, generator=gen), torch.randn(H, generator=gen)
+    c = torch.randn(5, 33, H, generator=gen)
+    for which in (0, 1):
+        want = _grads_allow_unused(lambda *t: (delta_rule_gates_ref(*t, False)[which],), [x.to(F64) for x in (a, b, A_log, dt_bias)], [c.to(F64)])
+        got = _grads_allow_unused(lambda *t: (lm_engine_amd.delta_rule_gates(*t, False)[which],), [x.cuda() for x in (a, b, A_log, dt_bias)], [c.cuda()])
+        for name, x, y in zip(("da", "db", "dA_log", "ddt_bias"), got, want):
+            if y is None:
+                assert x is None or torch.count_nonzero(x) == 0, name
+            else:
+                assert rel_l2(x, y) <= 1e-5, name
 
 
 @pytest.mark.parametrize("gated", [False, True])
