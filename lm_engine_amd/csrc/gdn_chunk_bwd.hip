@@ -35,7 +35,7 @@
 
 #include <type_traits>
 
-#include "gdn_chunk_common.h"
+#include "gdn_chunk32_common.h"
 #include "gdn_launch.h"
 
 namespace gdn {
@@ -91,11 +91,35 @@ __device__ __forceinline__ f32x16 mma_nt(const bf16_t* A, int lda, const bf16_t*
     return acc;
 }
 
-// sum over the 32 lanes of a wave half, result in all of them
-__device__ __forceinline__ float half_sum(float x) {
+// acc[r] += sum_t M[t][col0 + 8 (r/4) + 4 h + r%4] B[l32][t] over t < kd: the A operand is the transpose of 32 columns of
+// the row-major matrix M, read through the transposing LDS load (4 tokens x 16 columns per instruction)
+__device__ __forceinline__ f32x16 mma_tn(const bf16_t* M, int ldm, int col0, const bf16_t* B, int ldb, int kd, f32x16 acc, int l32, int lh) {
+    const int l16 = l32 % 16, g16 = l32 / 16;
+    for (int kk = 0; kk < kd; kk += 16) {
+        const bf16x4 lo = lds_read_tr4x16<false>(M, ldm, kk + 8 * lh, col0 + 16 * g16, l16);
+        const bf16x4 hi = lds_read_tr4x16<false>(M, ldm, kk + 8 * lh + 4, col0 + 16 * g16, l16);
+        bf16x8 a;
 #pragma unroll
-    for (int off = 16; off >= 1; off >>= 1) x += __shfl_xor(x, off, WAVE);
-    return x;
+        for (int e = 0; e < 4; e++) a[e] = lo[e], a[4 + e] = hi[e];
+        const bf16x8 b = *reinterpret_cast<const bf16x8*>(B + l32 * ldb + kk + 8 * lh);
+        acc = mfma32_bf16(a, b, acc);
+    }
+    return acc;
+}
+
+// Sixteen sums over the 32 lanes of a wave half at once: on return every lane holds the sum of x[l32 / 2].  Each
+// exchange halves the number of values a lane carries (16 shuffles instead of 80).
+__device__ __forceinline__ float half_sums16(const float (&x)[16], int l32) {
+    float y[8], z[4], w[2];
+    const bool b4 = l32 & 16, b3 = l32 & 8, b2 = l32 & 4, b1 = l32 & 2;
+#pragma unroll
+    for (int e = 0; e < 8; e++) y[e] = (b4 ? x[8 + e] : x[e]) + __shfl_xor(b4 ? x[e] : x[8 + e], 16, WAVE);
+#pragma unroll
+    for (int e = 0; e < 4; e++) z[e] = (b3 ? y[4 + e] : y[e]) + __shfl_xor(b3 ? y[e] : y[4 + e], 8, WAVE);
+#pragma unroll
+    for (int e = 0; e < 2; e++) w[e] = (b2 ? z[2 + e] : z[e]) + __shfl_xor(b2 ? z[e] : z[2 + e], 4, WAVE);
+    float u = (b1 ? w[1] : w[0]) + __shfl_xor(b1 ? w[0] : w[1], 2, WAVE);
+    return u + __shfl_xor(u, 1, WAVE);
 }
 
 __device__ __forceinline__ void put4(bf16_t* dst, f32x4 x) {
@@ -121,7 +145,11 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
     constexpr int SLAB = C * LDS64 * 2;        // bytes of a staged [64][64] matrix
     constexpr int PHASE1 = 3 * SLAB + K * LDS64 * 2;        // dO | Y | V~ | states
     constexpr int PHASE2 = 3 * SLAB + 2 * C * LDK * 2;      // G | G^T | Hm + Hm^T | q | k
-    constexpr int PHASE3 = 3 * SLAB + 2 * KW * LDS64 * 2;   // G | G^T | Hm + Hm^T | q^T | k^T
+    // Phase 3 needs q^T and k^T as MFMA operands.  K = 256 (a CU to itself) reads them out of the row-major copies with
+    // the transposing LDS load; with two workgroups per CU (K <= 128) that variant ran slower (more registers, spills)
+    // than staging the transposes once more, 2 bytes at a time.
+    constexpr bool TR = K > 128;
+    constexpr int PHASE3 = TR ? PHASE2 : 3 * SLAB + 2 * KW * LDS64 * 2;  // G | G^T | Hm + Hm^T | q^T | k^T
     constexpr int LDS_BYTES = cmax(PHASE1, cmax(PHASE2, PHASE3));
     __shared__ __attribute__((aligned(16))) uint8_t lds[LDS_BYTES];
     __shared__ float s_gam[C], s_beta[C], s_e[C], s_tail[C], s_dgam[C], s_dbeta[C], s_dotq[C], s_dotk[C], s_fq[C], s_fk[C], s_red[4];
@@ -132,9 +160,9 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
     bf16_t* const sG = reinterpret_cast<bf16_t*>(lds);
     bf16_t* const sGT = sG + C * LDS64;
     bf16_t* const sH = sGT + C * LDS64;
-    bf16_t* const sQ = sH + C * LDS64;    // phase 2: [64][LDK]
+    bf16_t* const sQ = sH + C * LDS64;    // phase 2 (and 3 with TR): [64][LDK]
     bf16_t* const sK = sQ + C * LDK;
-    bf16_t* const sQT = sH + C * LDS64;   // phase 3: [KW][LDS64]
+    bf16_t* const sQT = sH + C * LDS64;   // phase 3 without TR: [KW][LDS64]
     bf16_t* const sKT = sQT + KW * LDS64;
 
     const int t = threadIdx.x;
@@ -319,31 +347,59 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
     dot = wave_sum(dot);
     if (lane == 0) atomicAdd(&s_red[0], dot);
 
+    // rows of q and k (keys KW kh ..), scaled, row-major into sQ and sK
+    auto stage_qk = [&](int kh) {
+        constexpr int CPR = KW / 8, RPP = BWD_THREADS / CPR;  // 16-byte pieces per staged row, rows per pass
+        int tl = t;
+        asm volatile("" : "+v"(tl));  // the row addresses are formed here, not ahead of phase 1 (where they would be spilled)
+        const int p8 = tl % CPR;
+#pragma unroll
+        for (int it = 0; it < C / RPP; it++) {
+            const int row = tl / CPR + RPP * it;
+            bf16x8 qr = *reinterpret_cast<const bf16x8*>(row_of(p.q_raw, p.q_stride_b, p.q_stride_t, p.q_stride_h, row) + KW * kh + 8 * p8);
+            bf16x8 kr = *reinterpret_cast<const bf16x8*>(row_of(p.k_raw, p.k_stride_b, p.k_stride_t, p.k_stride_h, row) + KW * kh + 8 * p8);
+            if (row >= valid) qr = zero8, kr = zero8;
+            const float fq = s_fq[row], fk = s_fk[row];
+            bf16x8 qb, kb;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                qb[e] = (bf16_t)((float)qr[e] * fq);
+                kb[e] = (bf16_t)((float)kr[e] * fk);
+            }
+            *reinterpret_cast<bf16x8*>(sQ + row * LDK + 8 * p8) = qb;
+            *reinterpret_cast<bf16x8*>(sK + row * LDK + 8 * p8) = kb;
+        }
+    };
+
     // ---------------- phase 2: Q K^T, K K^T and the 64 x 64 stage ----------------
     // wave -> tile (ti, tj); rows i = 32 ti + 8 (r/4) + 4 h + r%4, column j = 32 tj + l32
     {
         const int ti = wave / 2, tj = wave % 2;
         f32x16 QK = zero, KK = zero;
-        constexpr int CPR = KW / 8, RPP = BWD_THREADS / CPR;  // 16-byte pieces per staged row, rows per pass
 #pragma unroll
         for (int kh = 0; kh < KH; kh++) {
             if (kh > 0) __syncthreads();  // the products of the previous half have read q and k
-            const int p8 = t % CPR;
+            if constexpr (TR) {
+                stage_qk(kh);
+            } else {
+                constexpr int CPR = KW / 8, RPP = BWD_THREADS / CPR;
+                const int p8 = t % CPR;
 #pragma unroll
-            for (int it = 0; it < C / RPP; it++) {
-                const int row = t / CPR + RPP * it;
-                bf16x8 qr = *reinterpret_cast<const bf16x8*>(row_of(p.q_raw, p.q_stride_b, p.q_stride_t, p.q_stride_h, row) + KW * kh + 8 * p8);
-                bf16x8 kr = *reinterpret_cast<const bf16x8*>(row_of(p.k_raw, p.k_stride_b, p.k_stride_t, p.k_stride_h, row) + KW * kh + 8 * p8);
-                if (row >= valid) qr = zero8, kr = zero8;
-                const float fq = s_fq[row], fk = s_fk[row];
-                bf16x8 qb, kb;
+                for (int it = 0; it < C / RPP; it++) {
+                    const int row = t / CPR + RPP * it;
+                    bf16x8 qr = *reinterpret_cast<const bf16x8*>(row_of(p.q_raw, p.q_stride_b, p.q_stride_t, p.q_stride_h, row) + KW * kh + 8 * p8);
+                    bf16x8 kr = *reinterpret_cast<const bf16x8*>(row_of(p.k_raw, p.k_stride_b, p.k_stride_t, p.k_stride_h, row) + KW * kh + 8 * p8);
+                    if (row >= valid) qr = zero8, kr = zero8;
+                    const float fq = s_fq[row], fk = s_fk[row];
+                    bf16x8 qb, kb;
 #pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    qb[e] = (bf16_t)((float)qr[e] * fq);
-                    kb[e] = (bf16_t)((float)kr[e] * fk);
+                    for (int e = 0; e < 8; e++) {
+                        qb[e] = (bf16_t)((float)qr[e] * fq);
+                        kb[e] = (bf16_t)((float)kr[e] * fk);
+                    }
+                    *reinterpret_cast<bf16x8*>(sQ + row * LDK + 8 * p8) = qb;
+                    *reinterpret_cast<bf16x8*>(sK + row * LDK + 8 * p8) = kb;
                 }
-                *reinterpret_cast<bf16x8*>(sQ + row * LDK + 8 * p8) = qb;
-                *reinterpret_cast<bf16x8*>(sK + row * LDK + 8 * p8) = kb;
             }
             __syncthreads();
             QK = mma_nt(sQ + 32 * ti * LDK, LDK, sK + 32 * tj * LDK, LDK, KW, QK, l32, lh);
@@ -352,6 +408,7 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
         const int j = 32 * tj + l32;
         const float gj = s_gam[j];
         float colsum = 0.f;
+        float rowm[16], rowb[16];  // this lane's terms of the row sums for dgamma and dbeta
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int i = 32 * ti + 8 * (r / 4) + 4 * lh + r % 4;
@@ -365,12 +422,8 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
             const float Hm = dA * bi * E;
             const float m = dP * Pm + dA * Am;
             colsum += m;
-            const float rowm = half_sum(m);
-            const float rowb = half_sum(dA * E * KK[r]);
-            if (l32 == 0) {
-                atomicAdd(&s_dgam[i], rowm);
-                atomicAdd(&s_dbeta[i], rowb);
-            }
+            rowm[r] = m;
+            rowb[r] = dA * E * KK[r];
             sG[i * LDS64 + j] = (bf16_t)G;
             sGT[j * LDS64 + i] = (bf16_t)G;
             if (i > j) {
@@ -380,9 +433,17 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
                 sH[i * LDS64 + i] = (bf16_t)0.f;
             }
         }
+        {
+            const float sm = half_sums16(rowm, l32), sb = half_sums16(rowb, l32);
+            const int r = l32 / 2;
+            const int i = 32 * ti + 8 * (r / 4) + 4 * lh + r % 4;
+            if (l32 % 2 == 0) {
+                atomicAdd(&s_dgam[i], sm);
+                atomicAdd(&s_dbeta[i], sb);
+            }
+        }
         atomicAdd(&s_dgam[j], -colsum);
     }
-
     // ---------------- phase 3: per-token sums over the key dim, dQ^T and dK^T, 128 keys at a time ----------------
     // (dQ^T and dK^T are built in the registers of dQe^T and dKd^T)
     float nkd = 0.f;
@@ -390,9 +451,15 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
     auto& acck = dKdT;
     bf16x8 qv[KH][NTW][2], kv[KH][NTW][2];  // this lane's entries of q and k, kept for the backward of the normalisation
 #pragma unroll
-    for (int kh = 0; kh < KH; kh++) {
-        __syncthreads();  // G, G^T, Hm + Hm^T are complete; q and k of phase 2 (or the previous half's transposes) are dead
-        {
+    for (int kx = 0; kx < KH; kx++) {
+        const int kh = TR ? KH - 1 - kx : kx;  // TR: the half that phase 2 staged last is still there
+        __syncthreads();  // G, G^T, Hm + Hm^T are complete (or: the previous half's reads are over)
+        if constexpr (TR) {
+            if (kx > 0) {
+                stage_qk(kh);
+                __syncthreads();
+            }
+        } else {
             constexpr int CPR = KW / 8, RPP = BWD_THREADS / CPR;
             const int p8 = t % CPR;
 #pragma unroll
@@ -408,19 +475,32 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
                     sKT[(8 * p8 + e) * LDS64 + row] = (bf16_t)((float)kr[e] * fk);
                 }
             }
+            __syncthreads();
         }
-        __syncthreads();
 #pragma unroll
         for (int m = 0; m < NTW; m++) {
             const int tt = tt_of(m);
             const int i = 32 * tt + l32;
             const float ei = s_e[i], tl = s_tail[i], bi = s_beta[i];
             float s_qe = 0.f, s_kd = 0.f, s_zk = 0.f;
+            if constexpr (TR) {
+#pragma unroll
+                for (int r4 = 0; r4 < 4; r4++) {  // keys 32 ktl + 8 r4 + 4 h + 0..3 of token i
+                    const bf16x4 q4 = *reinterpret_cast<const bf16x4*>(sQ + i * LDK + 32 * ktl + 8 * r4 + 4 * lh);
+                    const bf16x4 k4 = *reinterpret_cast<const bf16x4*>(sK + i * LDK + 32 * ktl + 8 * r4 + 4 * lh);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) qv[kh][m][r4 / 2][4 * (r4 % 2) + e] = q4[e], kv[kh][m][r4 / 2][4 * (r4 % 2) + e] = k4[e];
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int d = 32 * ktl + 8 * (r / 4) + 4 * lh + r % 4;
+                    qv[kh][m][r / 8][r % 8] = sQT[d * LDS64 + i], kv[kh][m][r / 8][r % 8] = sKT[d * LDS64 + i];
+                }
+            }
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const int d = 32 * ktl + 8 * (r / 4) + 4 * lh + r % 4;
-                const bf16_t qe = sQT[d * LDS64 + i], ke = sKT[d * LDS64 + i];
-                qv[kh][m][r / 8][r % 8] = qe, kv[kh][m][r / 8][r % 8] = ke;
+                const bf16_t qe = qv[kh][m][r / 8][r % 8], ke = kv[kh][m][r / 8][r % 8];
                 s_qe += dQeT[kh][m][r] * (float)qe;
                 s_kd += dKdT[kh][m][r] * (float)ke;
                 s_zk += ZT[kh][m][r] * (float)ke;
@@ -434,9 +514,15 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
                 accq[kh][m][r] *= ei;
                 acck[kh][m][r] = acck[kh][m][r] * tl - ZT[kh][m][r] * (bi * ei);
             }
-            accq[kh][m] = mma_nt(sKT + 32 * ktl * LDS64, LDS64, sG + 32 * tt * LDS64, LDS64, C, accq[kh][m], l32, lh);
-            acck[kh][m] = mma_nt(sQT + 32 * ktl * LDS64, LDS64, sGT + 32 * tt * LDS64, LDS64, C, acck[kh][m], l32, lh);
-            acck[kh][m] = mma_nt(sKT + 32 * ktl * LDS64, LDS64, sH + 32 * tt * LDS64, LDS64, C, acck[kh][m], l32, lh);
+            if constexpr (TR) {
+                accq[kh][m] = mma_tn(sK, LDK, 32 * ktl, sG + 32 * tt * LDS64, LDS64, C, accq[kh][m], l32, lh);
+                acck[kh][m] = mma_tn(sQ, LDK, 32 * ktl, sGT + 32 * tt * LDS64, LDS64, C, acck[kh][m], l32, lh);
+                acck[kh][m] = mma_tn(sK, LDK, 32 * ktl, sH + 32 * tt * LDS64, LDS64, C, acck[kh][m], l32, lh);
+            } else {
+                accq[kh][m] = mma_nt(sKT + 32 * ktl * LDS64, LDS64, sG + 32 * tt * LDS64, LDS64, C, accq[kh][m], l32, lh);
+                acck[kh][m] = mma_nt(sQT + 32 * ktl * LDS64, LDS64, sGT + 32 * tt * LDS64, LDS64, C, acck[kh][m], l32, lh);
+                acck[kh][m] = mma_nt(sKT + 32 * ktl * LDS64, LDS64, sH + 32 * tt * LDS64, LDS64, C, acck[kh][m], l32, lh);
+            }
             if (p.rq != nullptr) {  // <dQs_i, Qs_i> and <dK_i, K_i> for the backward of the normalisation
                 float dq_q = 0.f, dk_k = 0.f;
 #pragma unroll
