@@ -365,14 +365,14 @@ typedef struct gdn_conv_args {
 int gdn_causal_conv1d_fwd(const gdn_conv_args *args, void *stream);
 
 /*
- * Backward of gdn_causal_conv1d_fwd for bf16 x (what autograd computes through
+ * Backward of gdn_causal_conv1d_fwd (what autograd computes through
  * DepthwiseCausalConvolution.forward, depthwise_causal_convolution.py:103-241, when the layer trains):
  * given dy [B, S, C] (element strides) it recomputes the pre-activation from x and writes dx [B, S, C]
- * (bf16, contiguous), dstate [B, C, kernel_size - 1] (bf16; NULL when there was no input_state) and, per
+ * (contiguous), dstate [B, C, kernel_size - 1] (NULL when there was no input_state), both in dtype, and, per
  * block of tokens_per_block (8 .. 4096) tokens of a row, the partial sums of the gradients of weight and bias:
  * dweight_partial [B * ceil(S / tokens_per_block)][C][kernel_size] and dbias_partial [same][C], fp32, which
- * the caller adds up over the first dim.  The gradient flowing into final_state is not handled (the layer
- * does not differentiate through its cache).
+ * the caller adds up over the first dim.  C even; x, dy, dx 8-byte aligned, strides even.  The gradient flowing
+ * into final_state is the caller's to add (it lands on the last kernel_size - 1 rows of dx or on dstate).
  */
 typedef struct gdn_conv_bwd_args {
     const void *x, *dy, *weight, *bias, *input_state, *mask;
@@ -384,7 +384,7 @@ typedef struct gdn_conv_bwd_args {
     int32_t w_dtype;    /* gdn_dtype of weight and bias */
     int32_t activation; /* gdn_activation */
     int32_t tokens_per_block;
-    int32_t reserved;
+    int32_t dtype;      /* gdn_dtype of x, dy, input_state, mask, dx, dstate (bf16 or fp32) */
 } gdn_conv_bwd_args;
 int gdn_causal_conv1d_bwd(const gdn_conv_bwd_args *args, void *stream);
 

@@ -106,7 +106,7 @@ class GdnConvBwdArgs(ctypes.Structure):
                                               "dweight_partial", "dbias_partial")]
         + [(name, ctypes.c_int64) for name in ("x_stride_b", "x_stride_s", "dy_stride_b", "dy_stride_s")]
         + [(name, ctypes.c_int32) for name in ("B", "S", "C", "kernel_size", "w_dtype", "activation", "tokens_per_block",
-                                               "reserved")]
+                                               "dtype")]
     )  # fmt: skip
 
 

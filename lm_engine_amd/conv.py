@@ -4,8 +4,9 @@ Functional form of the reference's ``DepthwiseCausalConvolution.forward``
 (lm_engine/modeling_utils/depthwise_causal_convolution.py:103-241): same arguments, same three
 modes (fresh prefill, one-token update, multi-token continuation), same return ``(y, final_state)``.
 It runs one HIP kernel (``gdn_causal_conv1d_fwd`` of libgdn_hip.so); there is no torch fallback.
-Under autograd the backward of bf16 inputs is one more HIP kernel (``gdn_causal_conv1d_bwd``); other inputs
-differentiate the same formula written in torch (``_autograd.py``).
+Under autograd the backward is one more HIP kernel (``gdn_causal_conv1d_bwd``, bf16 and fp32 x); shapes it does not
+take (an odd number of channels) differentiate the same formula written in torch
+(``_autograd.py``).
 
     x             [B, S, C]          bf16 or fp32, channels contiguous
     weight        [C, 1, ks] or [C, ks]   nn.Conv1d's depthwise weight, ks in 2..4
@@ -83,18 +84,18 @@ def depthwise_causal_convolution(
     return kernel_with_formula_backward(kernel, formula, x, weight, bias, input_state)
 
 
-_BWD_TOKENS_PER_BLOCK = 128  # tokens a thread of the backward kernel walks over (16: 0.31 ms, 32: 0.23, 64: 0.20, 128: 0.19, 256: 0.24 at 4 x 4096 x 6144)
+_BWD_TOKENS_PER_BLOCK = 256  # tokens a thread of the backward kernel walks over (64: 0.196 ms, 128: 0.171, 256: 0.163 at 4 x 4096 x 6144)
 
 
 def _backward_kernel_applies(x, weight, activation) -> bool:
-    if not x.is_cuda or x.dtype != torch.bfloat16 or activation not in _IN_KERNEL_ACTIVATIONS or x.dim() != 3:
+    if not x.is_cuda or x.dtype not in (torch.bfloat16, torch.float32) or activation not in _IN_KERNEL_ACTIVATIONS or x.dim() != 3:
         return False
     B, S, C = x.shape
-    return C % 8 == 0 and weight.dtype in (torch.bfloat16, torch.float32) and B * (-(-S // _BWD_TOKENS_PER_BLOCK)) <= 65535
+    return C % 2 == 0 and weight.dtype in (torch.bfloat16, torch.float32) and B * (-(-S // _BWD_TOKENS_PER_BLOCK)) <= 65535
 
 
 class _ConvolutionOnKernels(torch.autograd.Function):
-    """Forward and backward on the HIP kernels (bf16 x).  The gradient that flows into the returned state is
+    """Forward and backward on the HIP kernels (bf16 or fp32 x).  The gradient that flows into the returned state is
     not propagated: the layer's cache is not differentiated through."""
 
     @staticmethod
@@ -103,27 +104,41 @@ class _ConvolutionOnKernels(torch.autograd.Function):
                                                        activation)  # fmt: skip
         ctx.save_for_backward(x, weight, bias, input_state, attention_mask)
         ctx.activation = activation
-        if final_state is not None:
-            ctx.mark_non_differentiable(final_state)
+        ctx.set_materialize_grads(False)
         return y, final_state
 
     @staticmethod
-    def backward(ctx, dy, _dstate_out):
+    def backward(ctx, dy, dstate_out):
         x, weight, bias, input_state, attention_mask = ctx.saved_tensors
+        if dy is None:
+            dy = torch.zeros_like(x)
         dx, dweight, dbias, dstate = _convolution_backward(x, weight, bias, input_state, attention_mask, dy,
                                                            ctx.activation)  # fmt: skip
+        if dstate_out is not None:
+            # The returned state is the last ks - 1 rows of [input_state or zeros | x * mask]: its gradient goes to those
+            # rows (a few row-sized additions; the layer itself does not differentiate through its cache).
+            B, S, C = x.shape
+            ks1 = dstate_out.size(-1)
+            mask = attention_mask if attention_mask is not None and attention_mask.shape[1] > 1 and attention_mask.shape[0] > 1 else None
+            for i in range(ks1):
+                t = S + i - ks1
+                if t >= 0:
+                    row = dstate_out[:, :, i].to(dx.dtype)
+                    dx[:, t, :] += row if mask is None else row * mask[:, t, None].to(dx.dtype)
+                elif dstate is not None:
+                    dstate[:, :, S + i] += dstate_out[:, :, i].to(dstate.dtype)
         return dx, dweight, dbias, dstate, None, None, None
 
 
 def _convolution_backward(x, weight, bias, input_state, attention_mask, dy, activation):
-    """``gdn_causal_conv1d_bwd``: dx, dweight, dbias, dinput_state for bf16 x (see include/gdn_hip.h)."""
+    """``gdn_causal_conv1d_bwd``: dx, dweight, dbias, dinput_state for bf16 or fp32 x (see include/gdn_hip.h)."""
     lib = _lib.load_library()
     B, S, C = x.shape
     w2 = (weight.squeeze(1) if weight.dim() == 3 else weight).contiguous()
     ks = w2.size(1)
     if x.stride(-1) != 1:
         x = x.contiguous()
-    dy = dy.to(torch.bfloat16)
+    dy = dy.to(x.dtype)
     if dy.stride(-1) != 1:
         dy = dy.contiguous()
     b2 = None if bias is None else bias.to(w2.dtype).contiguous()
@@ -146,6 +161,7 @@ def _convolution_backward(x, weight, bias, input_state, attention_mask, dy, acti
     a.x_stride_b, a.x_stride_s, a.dy_stride_b, a.dy_stride_s = x.stride(0), x.stride(1), dy.stride(0), dy.stride(1)
     a.B, a.S, a.C, a.kernel_size, a.tokens_per_block = B, S, C, ks, _BWD_TOKENS_PER_BLOCK
     a.w_dtype = _dtype_code(w2.dtype, "weight")
+    a.dtype = _dtype_code(x.dtype, "x")
     a.activation = _IN_KERNEL_ACTIVATIONS[activation]
     with torch.cuda.device(x.device):
         stream = ctypes.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)

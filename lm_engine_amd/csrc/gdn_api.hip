@@ -252,13 +252,15 @@ int gdn_causal_conv1d_bwd(const gdn_conv_bwd_args* a, void* stream) {
     if (a == nullptr) return GDN_ERR_NULL;
     if (!a->x || !a->dy || !a->weight || !a->dx || !a->dweight_partial || !a->dbias_partial) return GDN_ERR_NULL;
     if (a->B <= 0 || a->S <= 0 || a->C <= 0) return GDN_ERR_SHAPE;
-    if (a->C % 8 != 0 || a->kernel_size < 2 || a->kernel_size > 4) return GDN_ERR_UNSUPPORTED;
+    if (a->dtype != GDN_BF16 && a->dtype != GDN_F32) return GDN_ERR_UNSUPPORTED;
+    const int vec = 2;  // channels per thread
+    if (a->C % vec != 0 || a->kernel_size < 2 || a->kernel_size > 4) return GDN_ERR_UNSUPPORTED;
     if (a->w_dtype != GDN_BF16 && a->w_dtype != GDN_F32) return GDN_ERR_UNSUPPORTED;
     if (a->activation != GDN_ACT_NONE && a->activation != GDN_ACT_SILU) return GDN_ERR_UNSUPPORTED;
-    if (!aligned(a->x, 16) || !aligned(a->dy, 16) || !aligned(a->dx, 16)) return GDN_ERR_ALIGN;
+    if (!aligned(a->x, 8) || !aligned(a->dy, 8) || !aligned(a->dx, 8)) return GDN_ERR_ALIGN;
     const int64_t strides[] = {a->x_stride_b, a->x_stride_s, a->dy_stride_b, a->dy_stride_s};
     for (int64_t s : strides)
-        if (s < 0 || s % 8 != 0) return GDN_ERR_ALIGN;
+        if (s < 0 || s % vec != 0) return GDN_ERR_ALIGN;
     if (a->tokens_per_block < 8 || a->tokens_per_block > 4096) return GDN_ERR_SHAPE;
     if ((int64_t)a->B * ((a->S + a->tokens_per_block - 1) / a->tokens_per_block) > 65535) return GDN_ERR_UNSUPPORTED;  // one grid row per block
     return gdn::launch_conv_bwd(*a, static_cast<hipStream_t>(stream));

@@ -460,15 +460,19 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
                 __syncthreads();
             }
         } else {
-            constexpr int CPR = KW / 8, RPP = BWD_THREADS / CPR;
-            const int p8 = t % CPR;
+            // a wave takes 16 bytes of all 64 rows at a time: its 2-byte writes of one key then cover 64 consecutive
+            // tokens of a transposed row (no bank conflicts; the rows themselves come out of the cache)
+            constexpr int CPR = KW / 8;
+            const int row = t % C;
+            const float fq = s_fq[row], fk = s_fk[row];
+            const bf16_t* const qrow = row_of(p.q_raw, p.q_stride_b, p.q_stride_t, p.q_stride_h, row) + KW * kh;
+            const bf16_t* const krow = row_of(p.k_raw, p.k_stride_b, p.k_stride_t, p.k_stride_h, row) + KW * kh;
 #pragma unroll
-            for (int it = 0; it < C / RPP; it++) {
-                const int row = t / CPR + RPP * it;
-                bf16x8 qr = *reinterpret_cast<const bf16x8*>(row_of(p.q_raw, p.q_stride_b, p.q_stride_t, p.q_stride_h, row) + KW * kh + 8 * p8);
-                bf16x8 kr = *reinterpret_cast<const bf16x8*>(row_of(p.k_raw, p.k_stride_b, p.k_stride_t, p.k_stride_h, row) + KW * kh + 8 * p8);
+            for (int it = 0; it < CPR / 4; it++) {
+                const int p8 = t / C + 4 * it;
+                bf16x8 qr = *reinterpret_cast<const bf16x8*>(qrow + 8 * p8);
+                bf16x8 kr = *reinterpret_cast<const bf16x8*>(krow + 8 * p8);
                 if (row >= valid) qr = zero8, kr = zero8;
-                const float fq = s_fq[row], fk = s_fk[row];
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
                     sQT[(8 * p8 + e) * LDS64 + row] = (bf16_t)((float)qr[e] * fq);

@@ -6,7 +6,7 @@
 // y[s] = act(z[s]) * mask[s].  Backward with dz[s] = dy[s] mask[s] act'(z[s]):
 //     dxx[u]  = sum_j w[j] dz[u - j]           dx[t] = mask[t] dxx[t + KS - 1]      dstate[i] = dxx[i]
 //     dw[j]   = sum_{b, s} dz[s] xx[s + j]     dbias = sum_{b, s} dz[s]
-// One pass: a thread owns 8 consecutive channels and walks a block of tokens upward, recomputing z from a
+// One pass: a thread owns 2 consecutive channels and walks a block of tokens upward, recomputing z from a
 // sliding window of xx (nothing was saved by the forward), keeping KS partial sums of dxx in flight, and
 // accumulating dw and dbias for its block in registers; the KS - 1 rows of dz past the block's end are recomputed
 // for dx only.  The per-block partial sums of dw and dbias go to a [blocks][C] array each that the caller adds up.
@@ -20,17 +20,21 @@ namespace gdn {
 namespace {
 
 constexpr int CB_THREADS = 256;
-constexpr int CB_VEC = 8;
+// Channels per thread.  The kernel is bound by its arithmetic (about 35 vector instructions per token and channel against
+// 6 bytes), so narrow accesses that put more waves on a CU beat 16-byte ones: at B = 4, S = 4096, C = 6144 bf16, kernel plus
+// the two sums of the partial results, 8 channels 189 us, 4 channels 173 us, 2 channels (8 rows in flight, 256 tokens
+// per block) 163 us.
+constexpr int CB_VEC = 2;
 
 struct ConvBwdParams {
-    const bf16_t* x;
-    const bf16_t* dy;
+    const void* x;  // x, dy, input_state, mask, dx, dstate: bf16 or fp32 (the kernel's T)
+    const void* dy;
     const void* weight;
     const void* bias;
-    const bf16_t* input_state;
-    const bf16_t* mask;
-    bf16_t* dx;
-    bf16_t* dstate;
+    const void* input_state;
+    const void* mask;
+    void* dx;
+    void* dstate;
     float* dw_part;  // [B * blocks per row][C][KS]
     float* db_part;  // [B * blocks per row][C]
     int64_t x_stride_b, x_stride_s, dy_stride_b, dy_stride_s;
@@ -43,9 +47,10 @@ __device__ __forceinline__ float load_w(const void* w, int is_bf16, int64_t i) {
     return is_bf16 ? (float)reinterpret_cast<const bf16_t*>(w)[i] : reinterpret_cast<const float*>(w)[i];
 }
 
-template <int KS, bool SILU>
+// T: element type of the activations; VEC consecutive channels per thread, one vector access per row
+template <typename T, int KS, bool SILU, int VEC, bool MASK>
 __global__ __launch_bounds__(CB_THREADS) void causal_conv1d_bwd_kernel(const ConvBwdParams p) {
-    constexpr int VEC = CB_VEC;
+    typedef T vec_t __attribute__((ext_vector_type(VEC)));
     const int c0 = (blockIdx.x * CB_THREADS + threadIdx.x) * VEC;
     if (c0 >= p.C) return;
     const int blocks_per_row = (p.S + p.tokens_per_block - 1) / p.tokens_per_block;
@@ -54,10 +59,12 @@ __global__ __launch_bounds__(CB_THREADS) void causal_conv1d_bwd_kernel(const Con
     const int s_own = min(s_begin + p.tokens_per_block, p.S);      // dz of [s_begin, s_own) belongs to this block
     const int s_end = min(s_own + KS - 1, p.S);           // dz up to here feeds dx of this block
 
-    const bf16_t* xb = p.x + (int64_t)b * p.x_stride_b + c0;
-    const bf16_t* dyb = p.dy + (int64_t)b * p.dy_stride_b + c0;
-    const bf16_t* mb = p.mask == nullptr ? nullptr : p.mask + (int64_t)b * p.S;
-    bf16_t* dxb = p.dx + ((int64_t)b * p.S) * p.C + c0;
+    const T* xb = static_cast<const T*>(p.x) + (int64_t)b * p.x_stride_b + c0;
+    const T* dyb = static_cast<const T*>(p.dy) + (int64_t)b * p.dy_stride_b + c0;
+    const T* mb = MASK ? static_cast<const T*>(p.mask) + (int64_t)b * p.S : nullptr;  // MASK is false when there is none
+    T* dxb = static_cast<T*>(p.dx) + ((int64_t)b * p.S) * p.C + c0;
+    const T* const state_in = static_cast<const T*>(p.input_state);
+    T* const state_out = static_cast<T*>(p.dstate);
 
     float w[VEC][KS], bias[VEC];
 #pragma unroll
@@ -70,14 +77,14 @@ __global__ __launch_bounds__(CB_THREADS) void causal_conv1d_bwd_kernel(const Con
     // row s of xx in x's index (s < 0: carried state or zeros)
     auto load_xx = [&](int s, float (&row)[VEC]) {
         if (s >= 0) {
-            const bf16x8 v = *reinterpret_cast<const bf16x8*>(xb + (int64_t)s * p.x_stride_s);
-            const float m = mb == nullptr ? 1.f : (float)mb[s];
+            const vec_t v = *reinterpret_cast<const vec_t*>(xb + (int64_t)s * p.x_stride_s);
+            const float m = MASK ? (float)mb[s] : 1.f;
 #pragma unroll
             for (int e = 0; e < VEC; e++) row[e] = (float)v[e] * m;
         } else {
 #pragma unroll
             for (int e = 0; e < VEC; e++)
-                row[e] = p.input_state == nullptr ? 0.f : (float)p.input_state[((int64_t)b * p.C + c0 + e) * (KS - 1) + (KS - 1) + s];
+                row[e] = state_in == nullptr ? 0.f : (float)state_in[((int64_t)b * p.C + c0 + e) * (KS - 1) + (KS - 1) + s];
         }
     };
 
@@ -96,14 +103,14 @@ __global__ __launch_bounds__(CB_THREADS) void causal_conv1d_bwd_kernel(const Con
     // The walk goes in steps of UNROLL tokens whose rows of x and dy are all requested before the first is used: a
     // thread then has 2 UNROLL loads in flight instead of two, which is what a streaming kernel with this few waves
     // per CU needs to keep the memory system busy.  (Rows past s_end are read again from row s_end - 1 and not used.)
-    constexpr int UNROLL = 4;
+    constexpr int UNROLL = 8;
     for (int s0 = s_begin; s0 < s_end; s0 += UNROLL) {
-        bf16x8 xr[UNROLL], gr[UNROLL];
+        vec_t xr[UNROLL], gr[UNROLL];
 #pragma unroll
         for (int u = 0; u < UNROLL; u++) {
             const int su = min(s0 + u, s_end - 1);
-            xr[u] = *reinterpret_cast<const bf16x8*>(xb + (int64_t)su * p.x_stride_s);
-            gr[u] = *reinterpret_cast<const bf16x8*>(dyb + (int64_t)su * p.dy_stride_s);
+            xr[u] = *reinterpret_cast<const vec_t*>(xb + (int64_t)su * p.x_stride_s);
+            gr[u] = *reinterpret_cast<const vec_t*>(dyb + (int64_t)su * p.dy_stride_s);
         }
 #pragma unroll
         for (int u = 0; u < UNROLL; u++) {
@@ -116,10 +123,10 @@ __global__ __launch_bounds__(CB_THREADS) void causal_conv1d_bwd_kernel(const Con
                 for (int j = 0; j + 1 < KS; j++) win[j][e] = win[j + 1][e], pend[j][e] = pend[j + 1][e];
                 pend[KS - 1][e] = 0.f;
             }
-            const float m = mb == nullptr ? 1.f : (float)mb[s];
+            const float m = MASK ? (float)mb[s] : 1.f;
 #pragma unroll
             for (int e = 0; e < VEC; e++) win[KS - 1][e] = (float)xr[u][e] * m;
-            const bf16x8 g = gr[u];
+            const vec_t g = gr[u];
             const bool own = s < s_own;
 #pragma unroll
             for (int e = 0; e < VEC; e++) {
@@ -142,14 +149,14 @@ __global__ __launch_bounds__(CB_THREADS) void causal_conv1d_bwd_kernel(const Con
             // x index t = s - (KS - 1) is complete now
             const int t = s - (KS - 1);
             if (t >= s_begin) {
-                const float mt = mb == nullptr ? 1.f : (float)mb[t];
-                bf16x8 out;
+                const float mt = MASK ? (float)mb[t] : 1.f;
+                vec_t out;
 #pragma unroll
-                for (int e = 0; e < VEC; e++) out[e] = (bf16_t)(pend[0][e] * mt);
-                *reinterpret_cast<bf16x8*>(dxb + (int64_t)t * p.C) = out;
-            } else if (t < 0 && p.dstate != nullptr) {  // only in the first block of a row
+                for (int e = 0; e < VEC; e++) out[e] = (T)(pend[0][e] * mt);
+                *reinterpret_cast<vec_t*>(dxb + (int64_t)t * p.C) = out;
+            } else if (t < 0 && state_out != nullptr) {  // only in the first block of a row
 #pragma unroll
-                for (int e = 0; e < VEC; e++) p.dstate[((int64_t)b * p.C + c0 + e) * (KS - 1) + (KS - 1) + t] = (bf16_t)pend[0][e];
+                for (int e = 0; e < VEC; e++) state_out[((int64_t)b * p.C + c0 + e) * (KS - 1) + (KS - 1) + t] = (T)pend[0][e];
             }
         }
     }
@@ -160,14 +167,14 @@ __global__ __launch_bounds__(CB_THREADS) void causal_conv1d_bwd_kernel(const Con
         for (int j = 1; j < KS; j++) {
             const int t = s_end - 1 - (KS - 1) + j;
             if (t >= s_begin && t < s_own) {
-                const float mt = mb == nullptr ? 1.f : (float)mb[t];
-                bf16x8 out;
+                const float mt = MASK ? (float)mb[t] : 1.f;
+                vec_t out;
 #pragma unroll
-                for (int e = 0; e < VEC; e++) out[e] = (bf16_t)(pend[j][e] * mt);
-                *reinterpret_cast<bf16x8*>(dxb + (int64_t)t * p.C) = out;
-            } else if (t < 0 && t >= -(KS - 1) && s_begin == 0 && p.dstate != nullptr) {
+                for (int e = 0; e < VEC; e++) out[e] = (T)(pend[j][e] * mt);
+                *reinterpret_cast<vec_t*>(dxb + (int64_t)t * p.C) = out;
+            } else if (t < 0 && t >= -(KS - 1) && s_begin == 0 && state_out != nullptr) {
 #pragma unroll
-                for (int e = 0; e < VEC; e++) p.dstate[((int64_t)b * p.C + c0 + e) * (KS - 1) + (KS - 1) + t] = (bf16_t)pend[j][e];
+                for (int e = 0; e < VEC; e++) state_out[((int64_t)b * p.C + c0 + e) * (KS - 1) + (KS - 1) + t] = (T)pend[j][e];
             }
         }
     }
@@ -180,35 +187,44 @@ __global__ __launch_bounds__(CB_THREADS) void causal_conv1d_bwd_kernel(const Con
     }
 }
 
-template <int KS>
+template <typename T, int KS>
 int launch_ks(const ConvBwdParams& p, bool silu, hipStream_t stream) {
+    constexpr int VEC = CB_VEC;
     const int blocks_per_row = (p.S + p.tokens_per_block - 1) / p.tokens_per_block;
-    const dim3 grid((unsigned)((p.C / CB_VEC + CB_THREADS - 1) / CB_THREADS), (unsigned)(p.B * blocks_per_row));
-    if (silu) hipLaunchKernelGGL((causal_conv1d_bwd_kernel<KS, true>), grid, dim3(CB_THREADS), 0, stream, p);
-    else hipLaunchKernelGGL((causal_conv1d_bwd_kernel<KS, false>), grid, dim3(CB_THREADS), 0, stream, p);
+    const dim3 grid((unsigned)((p.C / VEC + CB_THREADS - 1) / CB_THREADS), (unsigned)(p.B * blocks_per_row));
+    const bool mask = p.mask != nullptr;
+    if (silu && mask) hipLaunchKernelGGL((causal_conv1d_bwd_kernel<T, KS, true, VEC, true>), grid, dim3(CB_THREADS), 0, stream, p);
+    else if (silu) hipLaunchKernelGGL((causal_conv1d_bwd_kernel<T, KS, true, VEC, false>), grid, dim3(CB_THREADS), 0, stream, p);
+    else if (mask) hipLaunchKernelGGL((causal_conv1d_bwd_kernel<T, KS, false, VEC, true>), grid, dim3(CB_THREADS), 0, stream, p);
+    else hipLaunchKernelGGL((causal_conv1d_bwd_kernel<T, KS, false, VEC, false>), grid, dim3(CB_THREADS), 0, stream, p);
     return (int)hipGetLastError();
+}
+
+template <typename T>
+int launch_t(const ConvBwdParams& p, int kernel_size, bool silu, hipStream_t stream) {
+    switch (kernel_size) {
+        case 2: return launch_ks<T, 2>(p, silu, stream);
+        case 3: return launch_ks<T, 3>(p, silu, stream);
+        case 4: return launch_ks<T, 4>(p, silu, stream);
+        default: return GDN_ERR_UNSUPPORTED;
+    }
 }
 
 }  // namespace
 
 int launch_conv_bwd(const gdn_conv_bwd_args& a, hipStream_t stream) {
     ConvBwdParams p;
-    p.x = static_cast<const bf16_t*>(a.x), p.dy = static_cast<const bf16_t*>(a.dy);
+    p.x = a.x, p.dy = a.dy;
     p.weight = a.weight, p.bias = a.bias;
-    p.input_state = static_cast<const bf16_t*>(a.input_state), p.mask = static_cast<const bf16_t*>(a.mask);
-    p.dx = static_cast<bf16_t*>(a.dx), p.dstate = static_cast<bf16_t*>(a.dstate);
+    p.input_state = a.input_state, p.mask = a.mask;
+    p.dx = a.dx, p.dstate = a.dstate;
     p.dw_part = a.dweight_partial, p.db_part = a.dbias_partial;
     p.x_stride_b = a.x_stride_b, p.x_stride_s = a.x_stride_s, p.dy_stride_b = a.dy_stride_b, p.dy_stride_s = a.dy_stride_s;
     p.B = a.B, p.S = a.S, p.C = a.C;
     p.w_is_bf16 = a.w_dtype == GDN_BF16 ? 1 : 0;
     p.tokens_per_block = a.tokens_per_block;
     const bool silu = a.activation == GDN_ACT_SILU;
-    switch (a.kernel_size) {
-        case 2: return launch_ks<2>(p, silu, stream);
-        case 3: return launch_ks<3>(p, silu, stream);
-        case 4: return launch_ks<4>(p, silu, stream);
-        default: return GDN_ERR_UNSUPPORTED;
-    }
+    return a.dtype == GDN_BF16 ? launch_t<bf16_t>(p, a.kernel_size, silu, stream) : launch_t<float>(p, a.kernel_size, silu, stream);
 }
 
 }  // namespace gdn

@@ -152,16 +152,19 @@ def test_convolution_gradients_bf16_kernel(with_state, masked, silu, S, ks):
             assert rel_l2(a, b) <= 1e-2, f"{name}: rel-L2 {rel_l2(a, b):.3e}"
 
 
-@pytest.mark.parametrize("with_state, masked", [(False, False), (True, False), (False, True)])
-def test_convolution_gradients(with_state, masked):
+@pytest.mark.parametrize("S, ks", [(37, 4), (1, 4), (2, 3), (200, 2)])
+@pytest.mark.parametrize("with_state, masked", [(False, False), (True, False), (False, True), (True, True)])
+def test_convolution_gradients(with_state, masked, S, ks):
+    """fp32 x: ``gdn_causal_conv1d_bwd`` again (4 channels per 16-byte access), and the gradient that flows into the
+    returned state (rows of dx, or of dstate when the sequence is shorter than the state)."""
     gen = torch.Generator().manual_seed(3)
-    B, S, C, ks = 3, 37, 64, 4
+    B, C = 3, 68
     x, w, bias = torch.randn(B, S, C, generator=gen), 0.5 * torch.randn(C, 1, ks, generator=gen), torch.randn(C, generator=gen)
     state = torch.randn(B, C, ks - 1, generator=gen)
     mask = torch.ones(B, S)
-    if masked:
-        mask[1, :10] = 0
-        mask[2, :36] = 0
+    if masked and S > 1:
+        mask[1, : S // 3] = 0
+        mask[2, : S - 1] = 0
     cy, cs = torch.randn(B, S, C, generator=gen), torch.randn(B, C, ks - 1, generator=gen)
     m = mask if masked else None
     if with_state:
