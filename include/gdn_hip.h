@@ -228,7 +228,7 @@ int gdn_chunk_fwd_saving_is_staged(const gdn_args *args, const gdn_chunk_saves *
  * = (n * H + h) * NC + c; per-chunk arrays are contiguous and chunk-major:
  *     v_new         [chunks][64][V]   V~, in saves_dtype (what gdn_chunk_fwd_saving wrote)
  *     states        [chunks][K][V]    the state a chunk starts from, in saves_dtype
- *     dstates       [chunks][K][V]    the gradient of the state it ends with, fp32
+ *     dstates       [chunks][K][V]    the gradient of the state it ends with, in dstates_dtype (fp32 or bf16)
  *     gamma, beta   [chunks][64]      prefix sum of g inside the chunk, beta (fp32; from gdn_chunk_bwd_prepare)
  *     rq, rk        [chunks][64]      1 / sqrt(|q|^2 + 1e-6), likewise for k, when q and k were normalised
  *                                     (the l2norm flag of the forward); both NULL otherwise
@@ -245,8 +245,8 @@ int gdn_chunk_fwd_saving_is_staged(const gdn_args *args, const gdn_chunk_saves *
  * kernels of fla's backward of chunk_gated_delta_rule, reached from gated_deltanet/module.py:197-209 under autograd.
  */
 typedef struct gdn_chunk_local_args {
-    const void *v_new, *states;
-    const float *dstates, *gamma, *beta, *rq, *rk;
+    const void *v_new, *states, *dstates;
+    const float *gamma, *beta, *rq, *rk;
     int32_t saves_dtype; /* gdn_dtype of v_new and states */
     float scale;
     int64_t chunks;
@@ -265,7 +265,7 @@ typedef struct gdn_chunk_local_args {
      * are skipped, tokens past its end are not written.  NULL: sequence n is row n, NC * 64 tokens. */
     const int32_t *seq_start, *seq_len;
     int32_t T_rows;
-    int32_t reserved;
+    int32_t dstates_dtype; /* gdn_dtype of dstates */
 } gdn_chunk_local_args;
 int gdn_chunk_bwd_local(const gdn_chunk_local_args *args, void *stream);
 

@@ -210,6 +210,7 @@ int gdn_chunk_bwd_local(const gdn_chunk_local_args* a, void* stream) {
         if (x == nullptr) return GDN_ERR_NULL;
         else if (!aligned(x, 16)) return GDN_ERR_ALIGN;
     if (a->saves_dtype != GDN_BF16 && a->saves_dtype != GDN_F32) return GDN_ERR_UNSUPPORTED;
+    if (a->dstates_dtype != GDN_BF16 && a->dstates_dtype != GDN_F32) return GDN_ERR_UNSUPPORTED;
     if (a->H <= 0 || a->NC <= 0 || a->chunks % ((int64_t)a->H * a->NC) != 0) return GDN_ERR_SHAPE;
     if (a->seq_start != nullptr && (a->seq_len == nullptr || a->T_rows <= 0)) return GDN_ERR_SHAPE;
     const int64_t raw_strides[] = {a->q_stride_b, a->q_stride_t, a->q_stride_h, a->k_stride_b, a->k_stride_t, a->k_stride_h,

@@ -124,18 +124,6 @@ __global__ __launch_bounds__(256) void chunk_offsets_kernel(const int32_t* __res
 // ------------------------------------------------------------------------------------------
 int launch_chunk32(ChunkParams& p, int K, hipStream_t stream, hipEvent_t* events, int num_cus);  // gdn_chunk32.hip
 
-static int compute_units() {
-    static int cached[64] = {};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-    if (cached[dev] == 0) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-        cached[dev] = n;
-    }
-    return cached[dev];
-}
-
 bool chunk_saving_scan_is_staged(const gdn_args& a, const gdn_chunk_saves& saves) {
     if (!chunk_shape_supported(a)) return false;
     const bool packed = a.cu_seqlens != nullptr && !(a.flags & GDN_FLAG_LEFT_PADDED);

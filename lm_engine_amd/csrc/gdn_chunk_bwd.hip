@@ -48,7 +48,7 @@ constexpr int LDS64 = 72;  // bf16 per LDS row of a [.][64] matrix: 16 bytes of 
 struct ChunkLocalParams {
     const void* vnew;   // V~ [chunk][64][V], fp32 or bf16 (saves_bf16)
     const void* s0;     // S0 [chunk][K][V], fp32 or bf16 (saves_bf16)
-    const float* ds1;   // dS1 [chunk][K][V]
+    const void* ds1;    // dS1 [chunk][K][V], fp32 or bf16 (the kernel's DS1H)
     int saves_bf16;
     const float* gam;
     const float* beta;
@@ -130,7 +130,8 @@ __device__ __forceinline__ void put4(bf16_t* dst, f32x4 x) {
 
 constexpr int cmax(int a, int b) { return a > b ? a : b; }
 
-template <int K>
+// DS1H: dS1 comes as bf16 (fp32 otherwise)
+template <int K, bool DS1H>
 __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_grads_kernel(const ChunkLocalParams p) {
     const int V = p.V;
     constexpr int VW = 64;                     // columns of the value dim staged at a time
@@ -223,7 +224,8 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
         for (int m = 0; m < NTW; m++) dQeT[kh][m] = zero, ZT[kh][m] = zero, dKdT[kh][m] = zero;
     const char* const s0b = static_cast<const char*>(p.s0) + chunk * K * (int64_t)V * (p.saves_bf16 ? 2 : 4);
     const char* const vnb = static_cast<const char*>(p.vnew) + chunk * C * (int64_t)V * (p.saves_bf16 ? 2 : 4);
-    const float* const ds1 = p.ds1 + chunk * K * (int64_t)V;
+    const float* const ds1 = static_cast<const float*>(p.ds1) + chunk * K * (int64_t)V;         // when fp32
+    const bf16_t* const ds1h = static_cast<const bf16_t*>(p.ds1) + chunk * K * (int64_t)V;    // when bf16
     constexpr int SROWS = K / 16;  // 16-byte fp32 pieces of a state slab per thread: K rows x 16 pieces
     float dot = 0.f;
 #pragma unroll 1
@@ -299,13 +301,22 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
         // products with S0 run, so that its trip through memory is behind them instead of in front of the barrier below.
         // With two workgroups per CU the other one's products fill that wait, and the registers are needed.
         constexpr bool PREFETCH = K > 128;
-        f32x4 ds1_rows[SROWS];
-        if constexpr (PREFETCH) {
+        f32x4 ds1_rows[DS1H ? 1 : SROWS];     // fp32 dS1: 16 pieces of 16 bytes per row of the slab
+        bf16x8 ds1_half[DS1H ? K / 32 : 1];   // bf16 dS1: 8 pieces per row, as for S0
+        auto ask_ds1 = [&]() {
+            if constexpr (DS1H) {
 #pragma unroll
-            for (int i = 0; i < SROWS; i++) {
-                const int idx = t + BWD_THREADS * i, row = idx / 16, c4 = idx % 16;
-                ds1_rows[i] = *reinterpret_cast<const f32x4*>(ds1 + row * V + v0 + 4 * c4);
+                for (int i = 0; i < K / 32; i++) ds1_half[i] = *reinterpret_cast<const bf16x8*>(ds1h + (t / 8 + 32 * i) * V + v0 + 8 * (t % 8));
+            } else {
+#pragma unroll
+                for (int i = 0; i < SROWS; i++) {
+                    const int idx = t + BWD_THREADS * i, row = idx / 16, c4 = idx % 16;
+                    ds1_rows[i] = *reinterpret_cast<const f32x4*>(ds1 + row * V + v0 + 4 * c4);
+                }
             }
+        };
+        if constexpr (PREFETCH) {
+            ask_ds1();
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
@@ -318,23 +329,28 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
             }
         DP = mma_nt(sDO + 32 * (wave / 2) * LDS64, LDS64, sVN + 32 * (wave % 2) * LDS64, LDS64, VW, DP, l32, lh);
         DA = mma_nt(sY + 32 * (wave / 2) * LDS64, LDS64, sVN + 32 * (wave % 2) * LDS64, LDS64, VW, DA, l32, lh);
-        if constexpr (!PREFETCH) {
-#pragma unroll
-            for (int i = 0; i < SROWS; i++) {
-                const int idx = t + BWD_THREADS * i, row = idx / 16, c4 = idx % 16;
-                ds1_rows[i] = *reinterpret_cast<const f32x4*>(ds1 + row * V + v0 + 4 * c4);
-            }
-        }
+        if constexpr (!PREFETCH) ask_ds1();
         __syncthreads();  // S0 has been read by every wave
 
         // dS1 takes the place of S0; <dS1, S0> on the way (S0 as the bf16 the products used)
+        if constexpr (DS1H) {
 #pragma unroll
-        for (int i = 0; i < SROWS; i++) {
-            const int idx = t + BWD_THREADS * i, row = idx / 16, c4 = idx % 16;
-            const f32x4 x = ds1_rows[i];
-            const bf16x4 sv = *reinterpret_cast<const bf16x4*>(sST + row * LDS64 + 4 * c4);
-            dot += x.x * (float)sv.x + x.y * (float)sv.y + x.z * (float)sv.z + x.w * (float)sv.w;
-            put4(sST + row * LDS64 + 4 * c4, x);
+            for (int i = 0; i < K / 32; i++) {
+                bf16_t* const at = sST + (t / 8 + 32 * i) * LDS64 + 8 * (t % 8);
+                const bf16x8 sv = *reinterpret_cast<const bf16x8*>(at);
+#pragma unroll
+                for (int e = 0; e < 8; e++) dot += (float)ds1_half[i][e] * (float)sv[e];
+                *reinterpret_cast<bf16x8*>(at) = ds1_half[i];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < SROWS; i++) {
+                const int idx = t + BWD_THREADS * i, row = idx / 16, c4 = idx % 16;
+                const f32x4 x = ds1_rows[i];
+                const bf16x4 sv = *reinterpret_cast<const bf16x4*>(sST + row * LDS64 + 4 * c4);
+                dot += x.x * (float)sv.x + x.y * (float)sv.y + x.z * (float)sv.z + x.w * (float)sv.w;
+                put4(sST + row * LDS64 + 4 * c4, x);
+            }
         }
         __syncthreads();
 #pragma unroll
@@ -1010,6 +1026,7 @@ static bool bwd_shape_built(int K, int V) { return (K == 64 || K == 128 || K == 
 int launch_chunk_bwd_local(const gdn_chunk_local_args& a, hipStream_t stream) {
     ChunkLocalParams p;
     p.vnew = a.v_new, p.s0 = a.states, p.ds1 = a.dstates, p.saves_bf16 = a.saves_dtype == GDN_BF16 ? 1 : 0;
+    const bool h = a.dstates_dtype == GDN_BF16;
     p.gam = a.gamma, p.beta = a.beta;
     p.rq = a.rq, p.rk = a.rk, p.scale = a.scale;
     p.y_mirror = static_cast<const bf16_t*>(a.y_mirror), p.y_chunks = static_cast<const bf16_t*>(a.y_chunks);
@@ -1024,9 +1041,12 @@ int launch_chunk_bwd_local(const gdn_chunk_local_args& a, hipStream_t stream) {
     p.d_stride_b = a.dout_stride_b, p.d_stride_t = a.dout_stride_t, p.d_stride_h = a.dout_stride_h;
     p.seq_start = a.seq_start, p.seq_len = a.seq_len, p.T_rows = a.seq_start != nullptr ? a.T_rows : a.NC * C;
     const dim3 grid((unsigned)a.chunks), block(BWD_THREADS);
-    if (a.K == 64) hipLaunchKernelGGL(chunk_local_grads_kernel<64>, grid, block, 0, stream, p);
-    else if (a.K == 128) hipLaunchKernelGGL(chunk_local_grads_kernel<128>, grid, block, 0, stream, p);
-    else hipLaunchKernelGGL(chunk_local_grads_kernel<256>, grid, block, 0, stream, p);
+    if (a.K == 64 && h) hipLaunchKernelGGL((chunk_local_grads_kernel<64, true>), grid, block, 0, stream, p);
+    else if (a.K == 64) hipLaunchKernelGGL((chunk_local_grads_kernel<64, false>), grid, block, 0, stream, p);
+    else if (a.K == 128 && h) hipLaunchKernelGGL((chunk_local_grads_kernel<128, true>), grid, block, 0, stream, p);
+    else if (a.K == 128) hipLaunchKernelGGL((chunk_local_grads_kernel<128, false>), grid, block, 0, stream, p);
+    else if (h) hipLaunchKernelGGL((chunk_local_grads_kernel<256, true>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((chunk_local_grads_kernel<256, false>), grid, block, 0, stream, p);
     return (int)hipGetLastError();
 }
 

@@ -7,6 +7,19 @@
 
 namespace gdn {
 
+// compute units of the current device (looked up once per device)
+inline int compute_units() {
+    static int cached[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
 // Arguments are validated by the caller (gdn_api.hip); these only pick an instantiation and launch.
 int launch_recurrent(const gdn_args& a, hipStream_t stream);
 // `events`, when not null, holds GDN_CHUNK_KERNELS + 1 events recorded around the kernels.

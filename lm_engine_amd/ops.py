@@ -419,7 +419,7 @@ def chunk_local_grads(q, k, v, dout, prep, y_mirror, v_new, states, dstates, sca
     ``prep`` what ``chunk_bwd_prepare`` returned (same ``sequences``), ``y_mirror`` the output of the scan over its
     mirror problem (bf16 ``[N, 2 NC 64, H, V]``) or, as a 4-D tensor, the V~ that scan saved at its even chunks (bf16
     ``[N H, NC, 64, V]``), ``v_new`` and ``states`` what the saving forward sweep wrote (both fp32 or both bf16),
-    ``dstates`` the states the mirror scan saved (fp32).  Returns ``dq, dk, dv`` bf16 ``[B, T, H, D]`` and ``dg, dbeta`` fp32
+    ``dstates`` the states the mirror scan saved (fp32 or bf16).  Returns ``dq, dk, dv`` bf16 ``[B, T, H, D]`` and ``dg, dbeta`` fp32
     ``[B, T, H]`` (zero where no sequence lives)."""
     _require_hip_path()
     lib = _lib.load_library()
@@ -438,7 +438,7 @@ def chunk_local_grads(q, k, v, dout, prep, y_mirror, v_new, states, dstates, sca
     if states.dtype != v_new.dtype or states.dtype not in (torch.float32, torch.bfloat16):
         raise ValueError("v_new and states must both be fp32 or both be bf16")
     for name, x, shape, dtype in (("v_new", v_new, (Bt, NC, C, V), states.dtype), ("states", states, (Bt, NC, K, V), states.dtype),
-                                  ("dstates", dstates, (Bt, NC, K, V), torch.float32)):  # fmt: skip
+                                  ("dstates", dstates, (Bt, NC, K, V), dstates.dtype)):  # fmt: skip
         if tuple(x.shape) != shape or x.dtype != dtype or not x.is_contiguous():
             raise ValueError(f"{name} must be contiguous {dtype} {shape}")
     alloc = torch.empty if sequences is None else torch.zeros  # tokens outside every sequence are not written
@@ -455,6 +455,7 @@ def chunk_local_grads(q, k, v, dout, prep, y_mirror, v_new, states, dstates, sca
         a.rq, a.rk = prep["rq"].data_ptr(), prep["rk"].data_ptr()
     a.v_new, a.states, a.dstates = v_new.data_ptr(), states.data_ptr(), dstates.data_ptr()
     a.saves_dtype = _dtype_code(states.dtype, "states")
+    a.dstates_dtype = _dtype_code(dstates.dtype, "dstates")
     if y_chunked:
         a.y_chunks = y_mirror.data_ptr()
     else:
