@@ -104,6 +104,10 @@ typedef struct gdn_args {
     float scale;        /* multiplies q (after optional normalisation) */
     int32_t spin_limit; /* one-launch forward: polls of a record's ready flag before the scan gives up (0 = default, 2^22:
                            seconds); see gdn_chunk_fwd_status */
+    int32_t qk_heads;   /* heads of q and k when fewer than H (grouped value attention, gated_deltanet/module.py:175-177:
+                           value head h reads q and k of head h / (H / qk_heads), what repeat_interleave would copy
+                           there); must divide H.  0 = H */
+    int32_t reserved;
     int32_t *error_word; /* optional, may be NULL: an int32 the GPU can write (device memory, or pinned host memory, which a
                            caller can read without synchronising); the one-launch forward stores 1 there when it gives up
                            waiting.  Never cleared by the library. */

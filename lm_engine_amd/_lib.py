@@ -131,7 +131,7 @@ class GdnArgs(ctypes.Structure):
             for d in ("b", "t", "h")
         ]
         + [(name, ctypes.c_int32) for name in ("B", "T", "H", "K", "V", "N", "chunk", "dtype", "beta_dtype", "flags")]
-        + [("scale", ctypes.c_float), ("spin_limit", ctypes.c_int32), ("error_word", ctypes.c_void_p)]
+        + [("scale", ctypes.c_float), ("spin_limit", ctypes.c_int32), ("qk_heads", ctypes.c_int32), ("reserved", ctypes.c_int32), ("error_word", ctypes.c_void_p)]
     )
 
 

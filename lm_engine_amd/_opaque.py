@@ -41,8 +41,8 @@ def gated_delta_rule_forward(q, k, v, g, beta, initial_state, cu_seqlens, mode, 
 
 @gated_delta_rule_forward.register_fake
 def _(q, k, v, g, beta, initial_state, cu_seqlens, mode, scale, output_final_state, l2norm, left_padded):
-    B, T, H, K = q.shape
-    V = v.size(-1)
+    B, T, _, K = q.shape
+    H, V = v.size(2), v.size(-1)
     N = B if cu_seqlens is None or left_padded else cu_seqlens.numel() - 1
     o = v.new_empty(B, T, H, V)
     ht = v.new_empty((N, H, K, V), dtype=torch.float32) if output_final_state else v.new_empty(0)
@@ -106,8 +106,7 @@ def gated_delta_rule_decode_(q, k, v, g, beta, state, cu_seqlens, scale, l2norm,
 
 @gated_delta_rule_decode_.register_fake
 def _(q, k, v, g, beta, state, cu_seqlens, scale, l2norm, left_padded):
-    B, T, H, _ = q.shape
-    return v.new_empty(B, T, H, v.size(-1))
+    return v.new_empty(v.shape)
 
 
 # ---------------------------------------------------------------------------------------

@@ -405,6 +405,15 @@ def gated_delta_rule_backward(
     shape of ``o``, ``dht`` that of the final state or is None.  Returns
     ``dq, dk, dv, dg, dbeta, dh0`` in the dtypes of the corresponding inputs (fp32 for dh0); entries for
     absent inputs are None."""
+    if q.size(2) != v.size(2):
+        # Grouped value attention: the backward runs on the expanded heads (what the reference's repeat_interleave hands
+        # its operator, gated_deltanet/module.py:175-177) and adds the gradients of a group's copies up.
+        group = v.size(2) // q.size(2)
+        dq, dk, *rest = gated_delta_rule_backward(
+            q.repeat_interleave(group, dim=2), k.repeat_interleave(group, dim=2), v, g, beta, do, dht, scale, initial_state,
+            cu_seqlens, use_qk_l2norm_in_kernel, left_padded)  # fmt: skip
+        fold = lambda d: d.view(*q.shape[:2], q.size(2), group, q.size(3)).sum(dim=3, dtype=torch.float32).to(d.dtype)  # noqa: E731
+        return (fold(dq), fold(dk), *rest)
     B, T, H, K = q.shape
     V = v.size(-1)
     dev = q.device

@@ -51,6 +51,7 @@ int validate_common(const gdn_args* a) {
     if (a == nullptr) return GDN_ERR_NULL;
     if (!a->q || !a->k || !a->v || !a->o) return GDN_ERR_NULL;
     if (a->B <= 0 || a->T <= 0 || a->H <= 0 || a->K <= 0 || a->V <= 0 || a->N <= 0) return GDN_ERR_SHAPE;
+    if (a->qk_heads < 0 || (a->qk_heads > 0 && a->H % a->qk_heads != 0)) return GDN_ERR_SHAPE;
     if (a->cu_seqlens != nullptr && !(a->flags & GDN_FLAG_LEFT_PADDED)) {
         if (a->B != 1) return GDN_ERR_VARLEN;
     } else if (a->N != a->B) {

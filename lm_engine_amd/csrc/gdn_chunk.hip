@@ -198,6 +198,7 @@ int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events, 
     p.v_stride_b = a.v_stride_b, p.v_stride_t = a.v_stride_t, p.v_stride_h = a.v_stride_h;
     p.o_stride_b = a.o_stride_b, p.o_stride_t = a.o_stride_t, p.o_stride_h = a.o_stride_h;
     p.B = a.B, p.T = a.T, p.H = a.H, p.V = a.V, p.N = a.N;
+    p.qk_div = a.qk_heads > 0 ? a.H / a.qk_heads : 1;
     p.NT = (a.T + C - 1) / C;
     p.TC = chunk_slots(a);
     p.beta_dtype = a.beta_dtype;

@@ -584,8 +584,9 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
         constexpr int V_ROWS = C / V_UNITS, V_PIECES = WAVE / V_ROWS;
         const int q_row = lane / Q_PIECES, q_piece = lane % Q_PIECES;
         const int v_row = lane / V_PIECES, v_piece = lane % V_PIECES;
-        const bf16_t* const qg = p.q + b * p.q_stride_b + seq_t0 * p.q_stride_t + (int64_t)h * p.q_stride_h + q_piece * 8;
-        const bf16_t* const kg = p.k + b * p.k_stride_b + seq_t0 * p.k_stride_t + (int64_t)h * p.k_stride_h + q_piece * 8;
+        const int hqk = qk_head_of(h, p.qk_div);
+        const bf16_t* const qg = p.q + b * p.q_stride_b + seq_t0 * p.q_stride_t + (int64_t)hqk * p.q_stride_h + q_piece * 8;
+        const bf16_t* const kg = p.k + b * p.k_stride_b + seq_t0 * p.k_stride_t + (int64_t)hqk * p.k_stride_h + q_piece * 8;
         const bf16_t* const vg = p.v + b * p.v_stride_b + seq_t0 * p.v_stride_t + (int64_t)h * p.v_stride_h + 32 * (vgroup * NW) + v_piece * 8;
         // two register buffers: while one chunk is written to LDS, younger ones are in flight
         bf16x8 buf0[NLOAD], buf1[NLOAD];
@@ -596,8 +597,8 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
         Scalars sc0 = {0.f, 0.f, 0.f, 0.f}, sc1 = {0.f, 0.f, 0.f, 0.f};
         // (QS: wave-uniform 64-bit base of the chunk + 32-bit per-lane byte offset formed at the load, so that no
         // per-slot 64-bit lane addresses stay live: with 20 slots per buffer they would not fit the registers)
-        const bf16_t* const qg0 = p.q + b * p.q_stride_b + seq_t0 * p.q_stride_t + (int64_t)h * p.q_stride_h;
-        const bf16_t* const kg0 = p.k + b * p.k_stride_b + seq_t0 * p.k_stride_t + (int64_t)h * p.k_stride_h;
+        const bf16_t* const qg0 = p.q + b * p.q_stride_b + seq_t0 * p.q_stride_t + (int64_t)hqk * p.q_stride_h;
+        const bf16_t* const kg0 = p.k + b * p.k_stride_b + seq_t0 * p.k_stride_t + (int64_t)hqk * p.k_stride_h;
         const bf16_t* const vg0 = p.v + b * p.v_stride_b + seq_t0 * p.v_stride_t + (int64_t)h * p.v_stride_h + 32 * (vgroup * NW);
         auto src_of = [&](int c, int i) -> const uint8_t* {
             if (i < NF) return rec + ((int64_t)c * p.rec_bytes + (int64_t)frag_of(i) * FRAG_BYTES) + lane * 16;

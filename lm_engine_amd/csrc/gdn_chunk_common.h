@@ -10,6 +10,9 @@ constexpr int GDN_CYCLE_BUDGET_SLOTS = 64;  // sampled workgroups of the measure
 constexpr int PREP_THREADS = 256;
 constexpr int FRAG_BYTES = WAVE * 16;  // one MFMA operand fragment: 8 bf16 per lane
 
+// head of q and k that value head h reads
+__host__ __device__ inline int qk_head_of(int h, int qk_div) { return qk_div > 1 ? h / qk_div : h; }
+
 struct ChunkParams {
     const bf16_t* q;
     const bf16_t* k;
@@ -29,6 +32,7 @@ struct ChunkParams {
     int64_t v_stride_b, v_stride_t, v_stride_h;
     int64_t o_stride_b, o_stride_t, o_stride_h;
     int B, T, H, V, N;
+    int qk_div;  // value heads per head of q and k (grouped value attention): head h reads q and k of head h / qk_div
     int NT;  // chunks per sequence (fixed-length input)
     int TC;  // chunk slots per head
     int beta_dtype;

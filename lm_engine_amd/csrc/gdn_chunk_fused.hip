@@ -196,8 +196,9 @@ __device__ __forceinline__ void scan_pair_body(const ChunkParams& p, uint8_t* ld
         constexpr int V_ROWS = C / V_UNITS, V_PIECES = WAVE / V_ROWS;
         const int q_row = lane / Q_PIECES, q_piece = lane % Q_PIECES;
         const int v_row = lane / V_PIECES, v_piece = lane % V_PIECES;
-        const bf16_t* const qg = p.q + b * p.q_stride_b + seq_t0 * p.q_stride_t + (int64_t)h * p.q_stride_h + q_piece * 8;
-        const bf16_t* const kg = p.k + b * p.k_stride_b + seq_t0 * p.k_stride_t + (int64_t)h * p.k_stride_h + q_piece * 8;
+        const int hqk = qk_head_of(h, p.qk_div);
+        const bf16_t* const qg = p.q + b * p.q_stride_b + seq_t0 * p.q_stride_t + (int64_t)hqk * p.q_stride_h + q_piece * 8;
+        const bf16_t* const kg = p.k + b * p.k_stride_b + seq_t0 * p.k_stride_t + (int64_t)hqk * p.k_stride_h + q_piece * 8;
         const bf16_t* const vg = p.v + b * p.v_stride_b + seq_t0 * p.v_stride_t + (int64_t)h * p.v_stride_h + 32 * (vgroup * NS) + v_piece * 8;
         bf16x8 buf[NB][NLOAD];
         struct Scalars {

@@ -115,8 +115,9 @@ __device__ __forceinline__ void chunk_prepare32_body(const ChunkParams& p, uint8
     const uint32_t q_lane_off = kq_row0 * (uint32_t)p.q_stride_t + kq_piece * 8;
     const int lane0 = tid % WAVE;
     auto prefetch_kq = [&]() {
-        const bf16_t* kg = p.k + ncc.b * p.k_stride_b + ncc.t0 * p.k_stride_t + (int64_t)nh * p.k_stride_h;
-        const bf16_t* qg = p.q + ncc.b * p.q_stride_b + ncc.t0 * p.q_stride_t + (int64_t)nh * p.q_stride_h;
+        const int nhqk = qk_head_of(nh, p.qk_div);
+        const bf16_t* kg = p.k + ncc.b * p.k_stride_b + ncc.t0 * p.k_stride_t + (int64_t)nhqk * p.k_stride_h;
+        const bf16_t* qg = p.q + ncc.b * p.q_stride_b + ncc.t0 * p.q_stride_t + (int64_t)nhqk * p.q_stride_h;
 #pragma unroll
         for (int it = 0; it < NPASS; it++) {
             const int row = kq_row0 + it * RPP;

@@ -39,6 +39,7 @@ struct RecurrentParams {
     int64_t v_stride_b, v_stride_t, v_stride_h;
     int64_t o_stride_b, o_stride_t, o_stride_h;
     int T, H, V;
+    int qk_div;  // value heads per head of q and k
     int beta_dtype;
     int l2norm;
     float scale;
@@ -89,8 +90,9 @@ __global__ __launch_bounds__(REC_THREADS) void recurrent_kernel(const RecurrentP
         for (int i = 0; i < RPT; i++) S[i] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    const T* qp = reinterpret_cast<const T*>(p.q) + b * p.q_stride_b + h * p.q_stride_h;
-    const T* kp = reinterpret_cast<const T*>(p.k) + b * p.k_stride_b + h * p.k_stride_h;
+    const int64_t hqk = p.qk_div > 1 ? h / p.qk_div : h;
+    const T* qp = reinterpret_cast<const T*>(p.q) + b * p.q_stride_b + hqk * p.q_stride_h;
+    const T* kp = reinterpret_cast<const T*>(p.k) + b * p.k_stride_b + hqk * p.k_stride_h;
     const T* vp = reinterpret_cast<const T*>(p.v) + b * p.v_stride_b + h * p.v_stride_h + v0;
     T* op = reinterpret_cast<T*>(p.o) + b * p.o_stride_b + h * p.o_stride_h + v0;
 
@@ -220,6 +222,7 @@ int launch_recurrent(const gdn_args& a, hipStream_t stream) {
     p.v_stride_b = a.v_stride_b, p.v_stride_t = a.v_stride_t, p.v_stride_h = a.v_stride_h;
     p.o_stride_b = a.o_stride_b, p.o_stride_t = a.o_stride_t, p.o_stride_h = a.o_stride_h;
     p.T = a.T, p.H = a.H, p.V = a.V;
+    p.qk_div = a.qk_heads > 0 ? a.H / a.qk_heads : 1;
     p.beta_dtype = a.beta_dtype;
     p.l2norm = (a.flags & GDN_FLAG_L2NORM) ? 1 : 0;
     p.scale = a.scale;

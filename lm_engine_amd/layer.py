@@ -3,7 +3,7 @@
 Follows lm_engine/modeling_utils/sequence_mixer_blocks/gated_deltanet/module.py:168-242 step by step:
 
     qkv, conv_state = conv1d(qkv, conv_state)            :168-170  -> depthwise_causal_convolution
-    q, k, v = split / view / GVA repeat                   :172-177  (views; repeat_interleave copies, as upstream)
+    q, k, v = split / view                                :172-177  (views; GVA heads are shared inside the operator)
     beta, g = sigmoid(b) [* 2], decay_gate(a)             :179-183  -> delta_rule_gates
     o, h = chunk or fused_recurrent (T <= 64)             :193-222  -> gated_delta_rule kernels
     o = o_norm(o * silu(gate))                            :238-241  -> gated_rmsnorm
@@ -65,9 +65,8 @@ def gated_deltanet_mixing(
     q = q.view(B, S, num_k_heads, k_head_dim)
     k = k.view(B, S, num_k_heads, k_head_dim)
     v = v.view(B, S, num_v_heads, v_head_dim)
-    if num_v_heads > num_k_heads:
-        q = q.repeat_interleave(repeats=num_v_heads // num_k_heads, dim=-2)
-        k = k.repeat_interleave(repeats=num_v_heads // num_k_heads, dim=-2)
+    # grouped value attention (num_v_heads > num_k_heads): the operator reads head h / (num_v_heads / num_k_heads) of q
+    # and k for value head h, so the reference's repeat_interleave copies (module.py:175-177) are not made
 
     g, beta = delta_rule_gates(a, b, A_log, dt_bias, allow_neg_eigval)
 

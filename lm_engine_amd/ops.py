@@ -63,12 +63,14 @@ def _last_dim_contiguous(x: torch.Tensor) -> torch.Tensor:
 def _check_inputs(q, k, v, g, beta, initial_state, cu_seqlens, left_padded=False):
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
         raise ValueError("q, k, v must be [B, T, H, D] tensors")
-    B, T, H, K = q.shape
-    V = v.size(-1)
+    B, T, HQK, K = q.shape
+    H, V = v.size(2), v.size(-1)
     if k.shape != q.shape:
         raise ValueError(f"k {tuple(k.shape)} must have the shape of q {tuple(q.shape)}")
-    if v.shape[:3] != q.shape[:3]:
-        raise ValueError(f"v {tuple(v.shape)} must share [B, T, H] with q {tuple(q.shape)}")
+    if v.shape[:2] != q.shape[:2]:
+        raise ValueError(f"v {tuple(v.shape)} must share [B, T] with q {tuple(q.shape)}")
+    if H % HQK != 0:  # grouped value attention: H / HQK consecutive value heads share a head of q and k
+        raise ValueError(f"the heads of v ({H}) must be a multiple of the heads of q and k ({HQK})")
     if not q.is_cuda:
         raise ValueError("the gated delta rule runs on the GPU only; inputs must be device tensors")
     for name, x in (("k", k), ("v", v), ("g", g), ("beta", beta), ("initial_state", initial_state),
@@ -119,6 +121,7 @@ def _fill_args(q, k, v, g, beta, h0, ht, o, cu_seqlens, scale, l2norm, inplace, 
         setattr(a, f"{name}_stride_t", x.stride(1))
         setattr(a, f"{name}_stride_h", x.stride(2))
     a.B, a.T, a.H, a.K, a.V, a.N = B, T, H, K, V, N
+    a.qk_heads = 0 if q.size(2) == H else q.size(2)
     a.chunk = 64
     a.dtype = _dtype_code(q.dtype, "q, k, v")
     a.beta_dtype = _lib.GDN_F32 if beta is None else _dtype_code(beta.dtype, "beta")
@@ -271,9 +274,9 @@ def fused_launch_applies(q, v, cu_seqlens=None) -> bool:
     rounded up to a multiple of 8) fill between 3/8 and 1/2 of the compute units."""
     if not is_kernel_allowed(Kernel.gated_delta_rule_fused_launch) or cu_seqlens is not None or q.dtype != torch.bfloat16:
         return False
-    B, T, H, K = q.shape
+    B, T, _, K = q.shape
     a = _lib.GdnArgs()  # the library decides (gdn_chunk_fwd_is_one_launch): shape fields and flags are all it reads
-    a.B, a.T, a.H, a.K, a.V, a.N = B, T, H, K, v.size(-1), B
+    a.B, a.T, a.H, a.K, a.V, a.N = B, T, v.size(2), K, v.size(-1), B
     a.chunk, a.dtype, a.flags = 64, _lib.GDN_BF16, _lib.GDN_FLAG_FUSED_LAUNCH
     with torch.cuda.device(q.device):
         return bool(_lib.load_library().gdn_chunk_fwd_is_one_launch(ctypes.byref(a)))
