@@ -153,7 +153,7 @@ __global__ __launch_bounds__(CB_THREADS) void causal_conv1d_bwd_kernel(const Con
                 vec_t out;
 #pragma unroll
                 for (int e = 0; e < VEC; e++) out[e] = (T)(pend[0][e] * mt);
-                *reinterpret_cast<vec_t*>(dxb + (int64_t)t * p.C) = out;
+                __builtin_nontemporal_store(out, reinterpret_cast<vec_t*>(dxb + (int64_t)t * p.C));  // (nobody reads dx back soon)
             } else if (t < 0 && state_out != nullptr) {  // only in the first block of a row
 #pragma unroll
                 for (int e = 0; e < VEC; e++) state_out[((int64_t)b * p.C + c0 + e) * (KS - 1) + (KS - 1) + t] = (T)pend[0][e];
@@ -171,7 +171,7 @@ __global__ __launch_bounds__(CB_THREADS) void causal_conv1d_bwd_kernel(const Con
                 vec_t out;
 #pragma unroll
                 for (int e = 0; e < VEC; e++) out[e] = (T)(pend[j][e] * mt);
-                *reinterpret_cast<vec_t*>(dxb + (int64_t)t * p.C) = out;
+                __builtin_nontemporal_store(out, reinterpret_cast<vec_t*>(dxb + (int64_t)t * p.C));  // (nobody reads dx back soon)
             } else if (t < 0 && t >= -(KS - 1) && s_begin == 0 && state_out != nullptr) {
 #pragma unroll
                 for (int e = 0; e < VEC; e++) state_out[((int64_t)b * p.C + c0 + e) * (KS - 1) + (KS - 1) + t] = (T)pend[j][e];

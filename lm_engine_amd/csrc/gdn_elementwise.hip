@@ -117,6 +117,18 @@ __device__ __forceinline__ void store8(float* p, const float (&x)[8]) {
     *reinterpret_cast<f32x4*>(p + 4) = f32x4{x[4], x[5], x[6], x[7]};
 }
 
+// the same with non-temporal stores (streams that nobody reads again soon)
+__device__ __forceinline__ void store8_stream(bf16_t* p, const float (&x)[8]) {
+    bf16x8 v;
+#pragma unroll
+    for (int e = 0; e < 8; e++) v[e] = (bf16_t)x[e];
+    __builtin_nontemporal_store(v, reinterpret_cast<bf16x8*>(p));
+}
+__device__ __forceinline__ void store8_stream(float* p, const float (&x)[8]) {
+    __builtin_nontemporal_store(f32x4{x[0], x[1], x[2], x[3]}, reinterpret_cast<f32x4*>(p));
+    __builtin_nontemporal_store(f32x4{x[4], x[5], x[6], x[7]}, reinterpret_cast<f32x4*>(p + 4));
+}
+
 struct NormParams {
     const void* o;
     const void* gate;
@@ -248,8 +260,10 @@ __global__ __launch_bounds__(256) void gated_rmsnorm_bwd_kernel(const NormBwdPar
                     d_o[e] = dx;
                 }
             }
-            store8(reinterpret_cast<T*>(p.d_o) + row * p.V + c, d_o);
-            if (p.gate != nullptr) store8(reinterpret_cast<T*>(p.d_gate) + row * p.V + c, d_g);
+            // non-temporal: nobody reads the gradients back soon, and they would push o, gate and dy out of the cache
+            // (76 -> 68 us at 4 x 4096 x 16 x 128; non-temporal loads on top of that lose it again)
+            store8_stream(reinterpret_cast<T*>(p.d_o) + row * p.V + c, d_o);
+            if (p.gate != nullptr) store8_stream(reinterpret_cast<T*>(p.d_gate) + row * p.V + c, d_g);
         }
     }
 #pragma unroll
