@@ -586,8 +586,10 @@ def bench_backward(w, inp, steps, warmup):
         "steps": steps,
         "ms_per_backward": round(ms, 3),
         "tokens_per_s": round(w.B * w.T / (ms * 1e-3), 1),
-        "composition": ("5 kernel launches: backward prepare, forward prepare + saving scan, saving scan over the "
-                        "mirror problem, chunk-local gradients" if backward_kernels_apply(w.K, w.V) else
+        "composition": ("4 kernel launches: backward prepare (also writes the forward sweep's records), saving scan "
+                        "on those records (forward sweep), saving scan over the mirror problem (reverse sweep), "
+                        "chunk-local gradients; chunk states, V~ and Y pass between them as bf16"
+                        if backward_kernels_apply(w.K, w.V) else
                         "2 saving scans + rocBLAS batched GEMMs + elementwise torch ops"),
     }
 
