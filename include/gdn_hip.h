@@ -206,6 +206,14 @@ int gdn_recurrent_fwd(const gdn_args *args, void *stream);
  * no_output != 0: the caller does not need args->o (a sweep that is run for its saves); where a variant of the scan
  * without the products that only serve the output exists (staged saves, K >= 128) it runs and args->o, which must
  * still be a valid buffer, is left unwritten; elsewhere the flag changes nothing.
+ * mirror_reads != 0 (records_given and no_output set, the scan without output: staged saves, K >= 128; else
+ * GDN_ERR_UNSUPPORTED): the sequence of T tokens that the scan walks is a sequence of T / 2 tokens read backwards with
+ * every chunk taken twice - the reverse sweep of the backward pass over gdn_chunk_bwd_prepare's mirror problem without
+ * its reversed copies.  Row i of chunk 2 r is token 64 (T/128 - 1 - r) + 63 - i of args->k and args->v, row i of chunk
+ * 2 r + 1 that token of k_odd and v_odd; all four are [N, T / 2, H, .] bf16 with element strides (args' for k and v).
+ * T / 64 must be even.  The twelve operand fragments of every odd chunk are read from the record of chunk 1 of the chain
+ * (in the mirror problem they are the same for all odd chunks: T' = I, P = 0); an odd chunk's own record supplies its
+ * row scales and e^{gamma_C} only.
  */
 typedef struct gdn_chunk_saves {
     void *states;
@@ -217,7 +225,10 @@ typedef struct gdn_chunk_saves {
     int32_t states_dtype; /* gdn_dtype of states */
     int32_t v_new_dtype;  /* gdn_dtype of v_new */
     int32_t no_output;
-    int32_t reserved;
+    int32_t mirror_reads;
+    const void *k_odd, *v_odd;
+    int64_t k_odd_stride_b, k_odd_stride_t, k_odd_stride_h;
+    int64_t v_odd_stride_b, v_odd_stride_t, v_odd_stride_h;
 } gdn_chunk_saves;
 int gdn_chunk_fwd_saving(const gdn_args *args, const gdn_chunk_saves *saves, void *stream);
 /* 1 when gdn_chunk_fwd_saving would run these arguments (shape fields, flags, cu_seqlens NULL or not; every field of
@@ -283,6 +294,10 @@ int gdn_chunk_bwd_local(const gdn_chunk_local_args *args, void *stream);
  *     order, chunk c becomes chunks 2 r and 2 r + 1, r = T/64 - 1 - c): k_mirror [N, 2 T, H, K] and
  *     v_mirror [N, 2 T, H, V] (bf16, contiguous) and the chunk records [H][N * 2 T/64], records_bytes >=
  *     H * N * 2 T/64 * 13312, for gdn_chunk_fwd_saving with records_given (k_mirror also in the place of q).
+ *     With k_mirror == NULL (batches of whole chunks only) no reversed copies are written: v_mirror is then
+ *     [N, T, H, V] and receives P^T dO, the rows of v of the even chunks, in the caller's token order, for a scan with
+ *     gdn_chunk_saves.mirror_reads (k = the caller's k, v = this array, k_odd = the caller's q, v_odd = dout); of the
+ *     odd chunks' records only chunk 1 of every chain then carries its operand fragments, the others their scales.
  *     The scan's output at the even chunks is Y = T^T dV~ (reversed), the states it saves there are the
  *     gradients of the chunks' final states, its final state is the gradient of the initial state.
  * flags: GDN_FLAG_L2NORM only.  g (fp32 [N, T, H]) and beta ([N, T, H], beta_dtype) may be NULL (0 and 1).

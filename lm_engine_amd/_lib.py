@@ -70,7 +70,15 @@ class GdnChunkSaves(ctypes.Structure):
         ("states_dtype", ctypes.c_int32),
         ("v_new_dtype", ctypes.c_int32),
         ("no_output", ctypes.c_int32),
-        ("reserved", ctypes.c_int32),
+        ("mirror_reads", ctypes.c_int32),
+        ("k_odd", ctypes.c_void_p),
+        ("v_odd", ctypes.c_void_p),
+        ("k_odd_stride_b", ctypes.c_int64),
+        ("k_odd_stride_t", ctypes.c_int64),
+        ("k_odd_stride_h", ctypes.c_int64),
+        ("v_odd_stride_b", ctypes.c_int64),
+        ("v_odd_stride_t", ctypes.c_int64),
+        ("v_odd_stride_h", ctypes.c_int64),
     ]
 
 

@@ -337,10 +337,12 @@ def _chunk_local_grads(qs, kn, vc, doc, Y, Vn, S0, dS1, gam, bc):
 
 
 def _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, l2norm, cu_seqlens, left_padded):
-    """The whole backward on five kernel launches (bf16, K = 128, V = 128, 256 or 512): ``gdn_chunk_bwd_prepare``
-    (mirror problem and per-chunk scalars), the saving forward sweep, the saving scan over the mirror problem,
-    ``gdn_chunk_bwd_local`` writing the gradients in the caller's layout.  Packed and left-padded batches are laid
-    out with the chunk count of their longest sequence."""
+    """The whole backward on four kernel launches (bf16; K = 64, 128 or 256; V a multiple of 64): ``gdn_chunk_bwd_prepare``
+    (per-chunk scalars, the mirror problem, and for whole-chunk batches the forward sweep's records), the saving
+    forward sweep, the saving scan over the mirror problem (reverse sweep), ``gdn_chunk_bwd_local`` writing the
+    gradients in the caller's layout.  Chunk states, V~ and Y pass between them as bf16 where the saving scan stages
+    its saves through LDS.  Packed and left-padded batches are laid out with the chunk count of their longest
+    sequence and run one more launch (their forward sweep prepares its own records)."""
     from . import ops  # late: ops imports this module
 
     B, T, H, K = q.shape
@@ -356,9 +358,16 @@ def _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, l2norm
     Bt = N * H
     q, k, v, do = (x if x.stride(-1) == 1 else x.contiguous() for x in (q, k, v, do.to(torch.bfloat16)))
     half_slices = K > 128 or ops.half_slice_records_pay(Bt, V, dev)  # K = 256 scans on half-slice waves only
+    # Where the mirror scan stages its saves through LDS, Y and the gradients of the chunks' final states leave as bf16
+    # (the chunk-local products round them to that anyway; their part in dg, <dS1, S0>, moved by less than its third
+    # digit in every test), and where it is the scan without output it reads the caller's q, k and dO backwards itself
+    # instead of reversed copies of them (whole-chunk batches).
+    staged_m = ops.saving_scan_is_staged(N, 2 * NC * CHUNK, H, K, V, None, False, 2 if half_slices else 1, dev,
+                                         states_dtype=torch.bfloat16, save_every=2)  # fmt: skip
+    mirror_reads = staged_m and K >= 128 and sequences is None
     # a batch of whole chunks gets the forward sweep's records from the same kernel: no prepare launch of its own
     prep = ops.chunk_bwd_prepare(q, k, do, g, beta, scale, l2norm, V, sequences, half_slice_records=half_slices,
-                                 forward_records=sequences is None)  # fmt: skip
+                                 forward_records=sequences is None, reversed_copies=not mirror_reads)  # fmt: skip
     # Where the saving scan stages its saves through LDS, the sweeps write S0, V~ and Y as bf16 (what the chunk-local
     # products round them to anyway) and form no output; elsewhere fp32 saves and Y from the mirror scan's output.
     given = 0 if sequences is not None else 2 if half_slices else 1
@@ -374,15 +383,12 @@ def _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, l2norm
         ops.chunk_forward_saving(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2norm, left_padded, S0, Vn, NC,
                                  no_output=True)  # fmt: skip
     dht32 = None if dht is None else dht.to(torch.float32).contiguous()
-    # Likewise the mirror scan: the gradients of the chunks' final states leave as bf16 (the chunk-local products round
-    # them to that anyway; their part in dg, <dS1, S0>, moved by less than its third digit in every test)
-    staged_m = ops.saving_scan_is_staged(N, 2 * NC * CHUNK, H, K, V, None, False, 2 if half_slices else 1, dev,
-                                         states_dtype=torch.bfloat16, save_every=2)  # fmt: skip
     dS1 = torch.empty(Bt, NC, K, V, device=dev, dtype=torch.bfloat16 if staged_m else torch.float32)
     Y = torch.empty(Bt, NC, CHUNK, V, dtype=torch.bfloat16, device=dev) if staged_m else None
-    o_m, dS = ops.chunk_scan_given_records(prep["k_mirror"], prep["v_mirror"], prep["records"], dht32, dS1, NC,
-                                           save_every=2, save_reverse=True, half_slice_records=half_slices,
-                                           v_new=Y, no_output=staged_m)  # fmt: skip
+    o_m, dS = ops.chunk_scan_given_records(k if mirror_reads else prep["k_mirror"], prep["v_mirror"], prep["records"],
+                                           dht32, dS1, NC, save_every=2, save_reverse=True,
+                                           half_slice_records=half_slices, v_new=Y, no_output=staged_m,
+                                           mirror_odd=(q, do) if mirror_reads else None)  # fmt: skip
     dq, dk, dv, dg, dbeta = ops.chunk_local_grads(q, k, v, do, prep, Y if staged_m else o_m, Vn, S0, dS1, scale, l2norm,
                                                   sequences)  # fmt: skip
     return (

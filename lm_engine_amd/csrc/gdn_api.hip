@@ -196,6 +196,18 @@ int gdn_chunk_fwd_saving(const gdn_args* a, const gdn_chunk_saves* saves, void* 
         return GDN_ERR_UNSUPPORTED;
     if ((saves->states_dtype == GDN_BF16 || saves->v_new_dtype == GDN_BF16) && !gdn::chunk_saving_scan_is_staged(*a, *saves))
         return GDN_ERR_UNSUPPORTED;
+    if (saves->mirror_reads) {
+        // only the scan without output reads that way
+        if (!saves->records_given || !saves->no_output || a->K < 128 || !gdn::chunk_saving_scan_is_staged(*a, *saves)) return GDN_ERR_UNSUPPORTED;
+        if (saves->k_odd == nullptr || saves->v_odd == nullptr) return GDN_ERR_NULL;
+        if (!aligned(saves->k_odd, 16) || !aligned(saves->v_odd, 16)) return GDN_ERR_ALIGN;
+        if (a->T % 128 != 0) return GDN_ERR_SHAPE;
+        const int64_t odd_strides[] = {saves->k_odd_stride_b, saves->k_odd_stride_t, saves->k_odd_stride_h,
+                                       saves->v_odd_stride_b, saves->v_odd_stride_t, saves->v_odd_stride_h};
+        for (int64_t s : odd_strides)
+            if (s < 0 || s % 8 != 0) return GDN_ERR_ALIGN;
+        if (saves->k_odd_stride_t > (1 << 24) || saves->v_odd_stride_t > (1 << 24)) return GDN_ERR_UNSUPPORTED;
+    }
     return gdn::launch_chunk_fwd(*a, static_cast<hipStream_t>(stream), nullptr, saves);
 }
 
@@ -228,11 +240,13 @@ int gdn_chunk_bwd_local(const gdn_chunk_local_args* a, void* stream) {
 
 int gdn_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args* a, void* stream) {
     if (a == nullptr) return GDN_ERR_NULL;
-    const void* ptrs[] = {a->q, a->k, a->dout, a->gamma, a->beta_packed, a->rq, a->rk, a->k_mirror, a->v_mirror, a->records};
+    const void* ptrs[] = {a->q, a->k, a->dout, a->gamma, a->beta_packed, a->rq, a->rk, a->v_mirror, a->records};
     for (const void* x : ptrs) {
         if (x == nullptr) return GDN_ERR_NULL;
         if (!aligned(x, 16)) return GDN_ERR_ALIGN;
     }
+    if (a->k_mirror == nullptr && a->seq_start != nullptr) return GDN_ERR_VARLEN;  // no reversed copies: whole-chunk batches only
+    if (a->k_mirror != nullptr && !aligned(a->k_mirror, 16)) return GDN_ERR_ALIGN;
     if (a->N <= 0 || a->T <= 0 || a->H <= 0 || a->N > 65535 || a->H > 65535) return GDN_ERR_SHAPE;
     if (!gdn::chunk_bwd_prepare_supported(*a)) return GDN_ERR_UNSUPPORTED;
     if (a->beta && a->beta_dtype != GDN_BF16 && a->beta_dtype != GDN_F32) return GDN_ERR_UNSUPPORTED;

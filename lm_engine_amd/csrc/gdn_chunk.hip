@@ -185,6 +185,13 @@ int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events, 
     p.rec = static_cast<uint8_t*>(a.workspace) + chunk_off_bytes(a) + chunk_flag_bytes(a);
     p.save_state = nullptr, p.save_vnew = nullptr, p.save_nc = 0, p.records_given = 0, p.save_every = 1, p.save_reverse = 0;
     p.save_state_bf16 = 0, p.save_vnew_bf16 = 0, p.no_output = 0;
+    p.mirror = 0, p.k2 = nullptr, p.v2 = nullptr;
+    p.k2_stride_b = p.k2_stride_t = p.k2_stride_h = p.v2_stride_b = p.v2_stride_t = p.v2_stride_h = 0;
+    if (saves != nullptr && saves->mirror_reads) {
+        p.mirror = 1, p.k2 = static_cast<const bf16_t*>(saves->k_odd), p.v2 = static_cast<const bf16_t*>(saves->v_odd);
+        p.k2_stride_b = saves->k_odd_stride_b, p.k2_stride_t = saves->k_odd_stride_t, p.k2_stride_h = saves->k_odd_stride_h;
+        p.v2_stride_b = saves->v_odd_stride_b, p.v2_stride_t = saves->v_odd_stride_t, p.v2_stride_h = saves->v_odd_stride_h;
+    }
     if (saves != nullptr) {
         p.save_state = static_cast<float*>(saves->states), p.save_vnew = static_cast<float*>(saves->v_new), p.save_nc = saves->chunks_per_chain;
         p.save_state_bf16 = saves->states_dtype == GDN_BF16 ? 1 : 0, p.save_vnew_bf16 = saves->v_new_dtype == GDN_BF16 ? 1 : 0;

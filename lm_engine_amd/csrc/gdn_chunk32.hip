@@ -600,8 +600,17 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
         const bf16_t* const qg0 = p.q + b * p.q_stride_b + seq_t0 * p.q_stride_t + (int64_t)hqk * p.q_stride_h;
         const bf16_t* const kg0 = p.k + b * p.k_stride_b + seq_t0 * p.k_stride_t + (int64_t)hqk * p.k_stride_h;
         const bf16_t* const vg0 = p.v + b * p.v_stride_b + seq_t0 * p.v_stride_t + (int64_t)h * p.v_stride_h + 32 * (vgroup * NW);
+        // mirror reads (scan without output only): the odd chunks' tensors, and the token a row stands for
+        const bool mirror = NOOUT && p.mirror != 0;
+        const bf16_t* const kg2 = mirror ? p.k2 + b * p.k2_stride_b + (int64_t)h * p.k2_stride_h + q_piece * 8 : kg;
+        const bf16_t* const vg2 = mirror ? p.v2 + b * p.v2_stride_b + (int64_t)h * p.v2_stride_h + 32 * (vgroup * NW) + v_piece * 8 : vg;
         auto src_of = [&](int c, int i) -> const uint8_t* {
-            if (i < NF) return rec + ((int64_t)c * p.rec_bytes + (int64_t)frag_of(i) * FRAG_BYTES) + lane * 16;
+            // (mirror reads: selects, not branches - a branch in these loops makes the compiler wait for the loads in flight)
+            const bool odd = mirror && (c & 1);
+            // the operand fragments of the odd chunks of a mirror problem (T' = I, P = 0) are the same for every chunk:
+            // only chunk 1 of a chain carries them, the row scales come from the chunk's own record (load_scalars)
+            if (i < NF) return rec + ((int64_t)(odd ? 1 : c) * p.rec_bytes + (int64_t)frag_of(i) * FRAG_BYTES) + lane * 16;
+            const int row0_tok = ((nchunks >> 1) - 1 - (c >> 1)) * C + C - 1;  // mirror reads: the token of row 0
             if constexpr (QS) {
                 const int last = (int)min((int64_t)C, seq_len - (int64_t)c * C) - 1;  // wave-uniform
                 if (i < NF + NV) {
@@ -619,14 +628,16 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
             }
             // a row past the end of the sequence (tail chunk) is read from the last token instead: never used
             if (i < NF + NV) {
-                const int tok = min(c * C + vunit_of(i - NF) * V_ROWS + v_row, (int)seq_len - 1);
-                return reinterpret_cast<const uint8_t*>(vg + (int64_t)tok * p.v_stride_t);
+                const int row = vunit_of(i - NF) * V_ROWS + v_row;
+                const int tok = mirror ? row0_tok - row : min(c * C + row, (int)seq_len - 1);
+                return reinterpret_cast<const uint8_t*>((odd ? vg2 : vg) + (int64_t)tok * (odd ? p.v2_stride_t : p.v_stride_t));
             }
             // units 0 .. Q_UNITS - 1 are rows of q, the rest rows of k (wave-uniform choice); without q all are rows of k
             const int u = qunit_of(i - NF - NV);
             const bool is_k = !HASQ || u >= Q_UNITS;
-            const int tok = min(c * C + ((is_k && HASQ) ? u - Q_UNITS : u) * Q_ROWS + q_row, (int)seq_len - 1);
-            return reinterpret_cast<const uint8_t*>((is_k ? kg : qg) + (int64_t)tok * (is_k ? p.k_stride_t : p.q_stride_t));
+            const int row = ((is_k && HASQ) ? u - Q_UNITS : u) * Q_ROWS + q_row;
+            const int tok = mirror ? row0_tok - row : min(c * C + row, (int)seq_len - 1);
+            return reinterpret_cast<const uint8_t*>((is_k ? (odd ? kg2 : kg) : qg) + (int64_t)tok * (is_k ? (odd ? p.k2_stride_t : p.k_stride_t) : p.q_stride_t));
         };
         auto dst_of = [&](uint8_t* st, int i) -> uint8_t* {
             if (i < NF) return st + frag_of(i) * FRAG_BYTES + lane * 16;

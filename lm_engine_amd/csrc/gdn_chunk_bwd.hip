@@ -789,18 +789,41 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_bwd_pre
     const int64_t mir0 = (int64_t)(p.NC - 1 - ci) * 2 * C;  // first token of chunk A in the mirror problem
     // token `row` of this chunk is token 63 - row of the mirror chunks A and B
     auto tok_a = [&](int row) -> int64_t { return ((int64_t)n * TM + mir0 + (C - 1 - row)) * p.H + h; };
+    // without reversed copies (k_m NULL) P^T dO goes out in the caller's token order, [N, NC 64, H, V], and nothing else
+    const bool copies = p.k_m != nullptr;
+    auto tok_u = [&](int row) -> int64_t { return copies ? tok_a(row) : (((int64_t)n * p.NC + ci) * C + row) * p.H + h; };
+
+    // Everything the chunk reads first is asked for at once - the rows of q and k, the first slab of dO, g and beta - so
+    // that wave 0's prefix sum below runs while the rows are on their way, not in front of them.
+    bf16x8 qn[C / RPP], kn[C / RPP], dpre[4];
+    if (valid > 0) {
+        const int p8 = t % CPR;
+#pragma unroll
+        for (int it = 0; it < C / RPP; it++) {
+            const int row = t / CPR + RPP * it;
+            qn[it] = *reinterpret_cast<const bf16x8*>(row_of(p.q, p.q_stride_b, p.q_stride_t, p.q_stride_h, row) + 8 * p8);
+            kn[it] = *reinterpret_cast<const bf16x8*>(row_of(p.k, p.k_stride_b, p.k_stride_t, p.k_stride_h, row) + 8 * p8);
+        }
+        const int vpr = V >= 128 ? 16 : 8, vrpp = BWD_THREADS / vpr;
+#pragma unroll
+        for (int it = 0; it < 4; it++) {
+            const int row = t / vpr + vrpp * it;
+            dpre[it] = zero8;
+            if (row < C) dpre[it] = *reinterpret_cast<const bf16x8*>(row_of(p.dout, p.d_stride_b, p.d_stride_t, p.d_stride_h, row) + 8 * (t % vpr));
+        }
+    }
 
     // ---- gamma (prefix sum of g inside the chunk) and beta: wave 0 ----
     if (wave == 0) {
         const int64_t at = (lane < valid ? tok0 + lane : 0) * p.H + h;
         float x = (p.g == nullptr || lane >= valid) ? 0.f : p.g[at];
+        const float b = lane < valid ? load_beta(p.beta, p.beta_dtype, at) : 0.f;
 #pragma unroll
         for (int off = 1; off < WAVE; off <<= 1) {
             const float y = __shfl_up(x, off, WAVE);
             if (lane >= off) x += y;
         }
         const float gl = __shfl(x, WAVE - 1, WAVE);
-        const float b = lane < valid ? load_beta(p.beta, p.beta_dtype, at) : 0.f;
         s_gam[lane] = x, s_beta[lane] = b, s_e[lane] = __expf(x), s_tail[lane] = __expf(gl - x);
         p.gam[chunk * C + lane] = x;
         p.bc[chunk * C + lane] = b;
@@ -835,8 +858,7 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_bwd_pre
             for (int it = 0; it < C / RPP; it++) {
                 const int row = t / CPR + RPP * it;
                 const bool live = row < valid;
-                bf16x8 qr = *reinterpret_cast<const bf16x8*>(row_of(p.q, p.q_stride_b, p.q_stride_t, p.q_stride_h, row) + 8 * p8);
-                bf16x8 kr = *reinterpret_cast<const bf16x8*>(row_of(p.k, p.k_stride_b, p.k_stride_t, p.k_stride_h, row) + 8 * p8);
+                bf16x8 qr = qn[it], kr = kn[it];
                 if (!live) qr = zero8, kr = zero8;
                 float ssq = 0.f, ssk = 0.f;
 #pragma unroll
@@ -857,21 +879,11 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_bwd_pre
                 *reinterpret_cast<bf16x8*>(sQ + row * LDK + 8 * p8) = qb;
                 *reinterpret_cast<bf16x8*>(sK + row * LDK + 8 * p8) = kb;
                 // mirror rows: k of chunk A is k, k of chunk B is q
-                const int64_t tokA = tok_a(row), tokB = tokA + (int64_t)C * p.H;
-                *reinterpret_cast<bf16x8*>(p.k_m + tokA * K + 8 * p8) = kr;
-                *reinterpret_cast<bf16x8*>(p.k_m + tokB * K + 8 * p8) = qr;
-            }
-        }
-        // the first slab of dO is asked for now: its trip through memory runs beside the products below
-        bf16x8 dpre[4];
-        const bool wide = V >= 128;
-        {
-            const int vpr = wide ? 16 : 8, vrpp = BWD_THREADS / vpr;
-#pragma unroll
-            for (int it = 0; it < 4; it++) {
-                const int row = t / vpr + vrpp * it;
-                dpre[it] = zero8;
-                if (row < C) dpre[it] = *reinterpret_cast<const bf16x8*>(row_of(p.dout, p.d_stride_b, p.d_stride_t, p.d_stride_h, row) + 8 * (t % vpr));
+                if (copies) {
+                    const int64_t tokA = tok_a(row), tokB = tokA + (int64_t)C * p.H;
+                    *reinterpret_cast<bf16x8*>(p.k_m + tokA * K + 8 * p8) = kr;
+                    *reinterpret_cast<bf16x8*>(p.k_m + tokB * K + 8 * p8) = qr;
+                }
             }
         }
         __syncthreads();
@@ -911,7 +923,7 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_bwd_pre
                 if (row >= valid) dr = zero8;
 #pragma unroll
                 for (int e = 0; e < 8; e++) sDOT[(8 * p8 + e) * LDS64 + row] = dr[e];
-                *reinterpret_cast<bf16x8*>(p.v_m + (tok_a(row) + (int64_t)C * p.H) * V + v0 + 8 * p8) = dr;
+                if (copies) *reinterpret_cast<bf16x8*>(p.v_m + (tok_a(row) + (int64_t)C * p.H) * V + v0 + 8 * p8) = dr;
             }
             __syncthreads();
             // rows j = 32 tj + .., columns v = v0 + 32 tv + l32, tv = wave, wave + 4, ..
@@ -928,7 +940,7 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_bwd_pre
                     for (int r = 0; r < 16; r++) {
                         const int j = 32 * tj + 8 * (r / 4) + 4 * lh + r % 4;
                         if constexpr (STAGED) sU[j * VS + 32 * tv + l32] = (bf16_t)u[r];
-                        else p.v_m[tok_a(j) * V + v0 + 32 * tv + l32] = (bf16_t)u[r];
+                        else p.v_m[tok_u(j) * V + v0 + 32 * tv + l32] = (bf16_t)u[r];
                     }
                 }
             if constexpr (STAGED) {
@@ -936,7 +948,7 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_bwd_pre
 #pragma unroll
                 for (int it = 0; it < C / VRPP; it++) {
                     const int j = t / VPR + VRPP * it;
-                    *reinterpret_cast<bf16x8*>(p.v_m + tok_a(j) * V + v0 + 8 * p8) = *reinterpret_cast<const bf16x8*>(sU + j * VS + 8 * p8);
+                    *reinterpret_cast<bf16x8*>(p.v_m + tok_u(j) * V + v0 + 8 * p8) = *reinterpret_cast<const bf16x8*>(sU + j * VS + 8 * p8);
                 }
             }
             __syncthreads();  // the slab is free (also for the scratch of the inverse)
@@ -974,8 +986,12 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_bwd_pre
         }
         reinterpret_cast<bf16x8*>(recA)[fl] = tm;
         reinterpret_cast<bf16x8*>(recA + p.off_p)[fl] = id;
-        reinterpret_cast<bf16x8*>(recB)[fl] = id;
-        reinterpret_cast<bf16x8*>(recB + p.off_p)[fl] = zz;
+        // (the fragments of a B chunk are the same for every chunk: a scan with mirror reads takes them from chunk 1 of the
+        // chain, which is this sequence's last chunk, and only the row scales from the chunk's own record)
+        if (copies || ci == p.NC - 1) {
+            reinterpret_cast<bf16x8*>(recB)[fl] = id;
+            reinterpret_cast<bf16x8*>(recB + p.off_p)[fl] = zz;
+        }
     }
     if (p.rec_fwd != nullptr) {
         // The record the forward's prepare step would write for this chunk (T diag(beta), P, the three row scales,

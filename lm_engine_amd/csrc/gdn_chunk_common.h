@@ -33,6 +33,14 @@ struct ChunkParams {
     int64_t o_stride_b, o_stride_t, o_stride_h;
     int B, T, H, V, N;
     int qk_div;  // value heads per head of q and k (grouped value attention): head h reads q and k of head h / qk_div
+    // Mirror reads (the reverse sweep of the backward pass on the scan without output): the sequence the scan walks is
+    // the caller's sequence backwards, every chunk twice - chunk 2 r takes its rows of k from k and of v from v, chunk
+    // 2 r + 1 from k2 and v2, both as tokens 64 (NT / 2 - 1 - r) + 63 - row of those tensors ([N, T / 2, H, .]).
+    int mirror;
+    const bf16_t* k2;
+    const bf16_t* v2;
+    int64_t k2_stride_b, k2_stride_t, k2_stride_h;
+    int64_t v2_stride_b, v2_stride_t, v2_stride_h;
     int NT;  // chunks per sequence (fixed-length input)
     int TC;  // chunk slots per head
     int beta_dtype;

@@ -378,7 +378,7 @@ def half_slice_records_pay(chains: int, V: int, device) -> bool:
 
 
 def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_chain, save_every=1, save_reverse=False,
-                             half_slice_records=False, v_new=None, no_output=False, q=None):
+                             half_slice_records=False, v_new=None, no_output=False, q=None, mirror_odd=None):
     """The scan kernel alone over a fixed-length batch whose chunk records the caller has written
     (``records`` uint8 ``[H, B * T / 64, record bytes]``, T a multiple of 64); it reads the rows of ``q``, ``k`` and
     ``v`` (without ``q``, ``k`` stands in its place: the records of a mirror problem carry zero row scales for q).  Returns ``(o, final_state)``
@@ -387,13 +387,23 @@ def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_ch
     ``save_reverse``), and V~ of those chunks into ``v_new`` ``[B * H, chunks_per_chain, 64, V]`` when that is given.
     ``half_slice_records``: the fragments of the records are in the lane order of the 16x16x32 MFMA (K = 256 needs
     that) instead of the 32x32x16 one.  bf16 save arrays where ``saving_scan_is_staged``; ``no_output``: the caller
-    does not need ``o`` (None is returned; the library skips forming it where it has a scan without output)."""
+    does not need ``o`` (None is returned; the library skips forming it where it has a scan without output).
+    ``mirror_odd = (k_odd, v_odd)`` (with ``no_output``, where the scan without output exists): ``k``, ``v`` and these two
+    are ``[B, T / 2, H, .]`` tensors that the scan reads backwards, every chunk twice - the even chunks' rows from ``k``
+    and ``v``, the odd chunks' from ``k_odd`` and ``v_odd`` (``gdn_chunk_saves.mirror_reads``): the mirror problem of
+    ``chunk_bwd_prepare(..., reversed_copies=False)``."""
     _require_hip_path()
     lib = _lib.load_library()
     q = k if q is None else q
     dims = _check_inputs(q, k, v, None, None, initial_state, None)
     B, T, H, K, V, N = dims
     q, k, v = _last_dim_contiguous(q), _last_dim_contiguous(k), _last_dim_contiguous(v)
+    if mirror_odd is not None:
+        k_odd, v_odd = (_last_dim_contiguous(x) for x in mirror_odd)
+        if not no_output or k_odd.shape != k.shape or v_odd.shape != v.shape or k_odd.dtype != k.dtype or v_odd.dtype != v.dtype:
+            raise ValueError("mirror_odd needs no_output and tensors of the shapes and dtype of k and v")
+        T = 2 * T  # the sequence the scan walks
+        dims = (B, T, H, K, V, N)
     if T % 64 != 0 or not records.is_contiguous() or records.dtype != torch.uint8 or tuple(records.shape[:2]) != (H, B * T // 64):
         raise ValueError("records must be contiguous uint8 [H, B * T / 64, record bytes] with T a multiple of 64")
     states_code = _save_dtype_code(states, (B * H, chunks_per_chain, K, V), "states")
@@ -405,6 +415,10 @@ def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_ch
     saves = _lib.GdnChunkSaves(states.data_ptr(), None if v_new is None else v_new.data_ptr(), chunks_per_chain,
                                2 if half_slice_records else 1, save_every, 1 if save_reverse else 0, states_code,
                                v_new_code, 1 if no_output else 0, 0)  # fmt: skip
+    if mirror_odd is not None:
+        saves.mirror_reads, saves.k_odd, saves.v_odd = 1, k_odd.data_ptr(), v_odd.data_ptr()
+        saves.k_odd_stride_b, saves.k_odd_stride_t, saves.k_odd_stride_h = k_odd.stride(0), k_odd.stride(1), k_odd.stride(2)
+        saves.v_odd_stride_b, saves.v_odd_stride_t, saves.v_odd_stride_h = v_odd.stride(0), v_odd.stride(1), v_odd.stride(2)
     with torch.cuda.device(k.device):
         stream = ctypes.c_void_p(torch.cuda.current_stream(k.device).cuda_stream)
         _lib.check_status(lib.gdn_chunk_fwd_saving(ctypes.byref(args), ctypes.byref(saves), stream),
@@ -485,7 +499,7 @@ RECORD_BYTES = 13312  # a chunk record: 12 operand fragments, 3 x 64 row scales,
 
 
 def chunk_bwd_prepare(q, k, dout, g, beta, scale, l2norm, V, sequences=None, half_slice_records=False,
-                      forward_records=False):
+                      forward_records=False, reversed_copies=True):
     """``gdn_chunk_bwd_prepare``.  ``q, k, dout`` are the caller's bf16 ``[B, T, H, D]`` tensors; without
     ``sequences`` every row is one sequence of whole chunks, else ``sequences = (seq_start, seq_len, NC)``: int32
     device tensors ``[N]`` (first token as a flat index over the rows, length) and the chunks per sequence to lay
@@ -494,10 +508,14 @@ def chunk_bwd_prepare(q, k, dout, g, beta, scale, l2norm, V, sequences=None, hal
     ``[N, 2 NC 64, H, D]`` bf16, ``records`` uint8 ``[H, N * 2 NC, RECORD_BYTES]`` (their fragments in the lane order
     of the 16x16x32 MFMA with ``half_slice_records``, see ``chunk_scan_given_records``).  ``forward_records``
     (whole-chunk batches only): also ``records_fwd`` ``[H, N * NC, RECORD_BYTES]``, the records of the forward pass
-    itself in the same fragment order, for a forward sweep without a prepare launch of its own."""
+    itself in the same fragment order, for a forward sweep without a prepare launch of its own.  Without
+    ``reversed_copies`` (whole-chunk batches only) ``k_mirror`` is None and ``v_mirror`` is ``[N, T, H, V]``: P^T dO in
+    the caller's token order, for a scan with ``mirror_odd`` that reads the caller's q, k and dout backwards itself."""
     _require_hip_path()
     lib = _lib.load_library()
     B, T, H, K = q.shape
+    if not reversed_copies and sequences is not None:
+        raise ValueError("a batch that is not whole rows of whole chunks needs the reversed copies")
     if not backward_kernels_apply(K, V) or q.dtype != torch.bfloat16:
         raise ValueError(f"built for bf16, K in {_SUPPORTED_K} and V a multiple of 64, got {q.dtype}, {K}, {V}")
     if sequences is None:
@@ -515,8 +533,8 @@ def chunk_bwd_prepare(q, k, dout, g, beta, scale, l2norm, V, sequences=None, hal
     out = dict(
         gamma=torch.empty(Bt, NC, 64, **f32), beta=torch.empty(Bt, NC, 64, **f32),
         rq=torch.empty(Bt, NC, 64, **f32), rk=torch.empty(Bt, NC, 64, **f32),
-        k_mirror=torch.empty(N, 2 * NC * 64, H, K, dtype=torch.bfloat16, device=dev),
-        v_mirror=torch.empty(N, 2 * NC * 64, H, V, dtype=torch.bfloat16, device=dev),
+        k_mirror=torch.empty(N, 2 * NC * 64, H, K, dtype=torch.bfloat16, device=dev) if reversed_copies else None,
+        v_mirror=torch.empty(N, (2 if reversed_copies else 1) * NC * 64, H, V, dtype=torch.bfloat16, device=dev),
         records=torch.empty(H, N * 2 * NC, RECORD_BYTES, dtype=torch.uint8, device=dev),
     )  # fmt: skip
     a = _lib.GdnChunkBwdPrepareArgs()
@@ -532,7 +550,8 @@ def chunk_bwd_prepare(q, k, dout, g, beta, scale, l2norm, V, sequences=None, hal
     a.flags = (_lib.GDN_FLAG_L2NORM if l2norm else 0) | (_lib.GDN_FLAG_RECORDS_16X16 if half_slice_records else 0)
     a.scale = float(scale)
     a.gamma, a.beta_packed, a.rq, a.rk = (out[n].data_ptr() for n in ("gamma", "beta", "rq", "rk"))
-    a.k_mirror, a.v_mirror, a.records = (out[n].data_ptr() for n in ("k_mirror", "v_mirror", "records"))
+    a.k_mirror = out["k_mirror"].data_ptr() if reversed_copies else None
+    a.v_mirror, a.records = out["v_mirror"].data_ptr(), out["records"].data_ptr()
     a.records_bytes = out["records"].numel()
     if forward_records:
         if sequences is not None:

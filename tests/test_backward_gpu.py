@@ -374,3 +374,34 @@ def test_given_records_in_both_fragment_orders_give_the_same_sweep():
         results.append((o_m.float().cpu(), dS1.cpu(), dS.cpu()))
     for name, a, b in zip(("output", "saved states", "final state"), *results):
         assert rel_l2(a, b) <= 5e-3, f"{name}: rel-L2 {rel_l2(a, b):.3e}"
+
+
+@pytest.mark.parametrize("K, V, B, T, H", [(128, 128, 2, 256, 2), (256, 512, 1, 192, 2), (128, 256, 3, 128, 4)])
+def test_mirror_reads_equal_the_scan_over_reversed_copies(K, V, B, T, H):
+    """The reverse sweep with ``gdn_chunk_saves.mirror_reads`` - the scan reads the caller's q, k, dO backwards and
+    P^T dO in the caller's order, the odd chunks' operand fragments from chunk 1's record - against the same scan over
+    the reversed copies that ``gdn_chunk_bwd_prepare`` otherwise writes: same kernel, same arithmetic, bit for bit."""
+    from lm_engine_amd import ops
+
+    inp = random_inputs(B=B, T=T, H=H, K=K, V=V, dtype=torch.bfloat16, seed=93, normalize=False)
+    q, k, g, beta = (inp[n].cuda() for n in ("q", "k", "g", "beta"))
+    gen = torch.Generator().manual_seed(94)
+    do = torch.randn(B, T, H, V, generator=gen).to(torch.bfloat16).cuda()
+    dht = torch.randn(B, H, K, V, generator=gen).cuda()
+    NC = T // 64
+    staged = ops.saving_scan_is_staged(B, 2 * T, H, K, V, None, False, 2, q.device, states_dtype=torch.bfloat16, save_every=2)
+    assert staged, "this shape should run the scan without output"
+    results = []
+    for copies in (True, False):
+        prep = ops.chunk_bwd_prepare(q, k, do, g, beta, K**-0.5, True, V, None, half_slice_records=True, reversed_copies=copies)
+        assert (prep["k_mirror"] is None) == (not copies)
+        dS1 = torch.zeros(B * H, NC, K, V, dtype=torch.bfloat16, device="cuda")
+        Y = torch.zeros(B * H, NC, 64, V, dtype=torch.bfloat16, device="cuda")
+        _, dS = ops.chunk_scan_given_records(prep["k_mirror"] if copies else k, prep["v_mirror"], prep["records"], dht, dS1, NC,
+                                             save_every=2, save_reverse=True, half_slice_records=True, v_new=Y, no_output=True,
+                                             mirror_odd=None if copies else (q, do))  # fmt: skip
+        torch.cuda.synchronize()
+        results.append((dS1.cpu(), Y.cpu(), dS.cpu()))
+    for name, a, b in zip(("saved states", "saved Y", "final state"), *results):
+        assert a.abs().max() > 0, name
+        assert torch.equal(a, b), f"{name}: rel-L2 {rel_l2(a.float(), b.float()):.3e}"
