@@ -211,6 +211,10 @@ int gdn_recurrent_fwd(const gdn_args *args, void *stream);
  * every chunk taken twice - the reverse sweep of the backward pass over gdn_chunk_bwd_prepare's mirror problem without
  * its reversed copies.  Row i of chunk 2 r is token 64 (T/128 - 1 - r) + 63 - i of args->k and args->v, row i of chunk
  * 2 r + 1 that token of k_odd and v_odd; all four are [N, T / 2, H, .] bf16 with element strides (args' for k and v).
+ * sliced != 0 (bf16 saves through the staging variant only; GDN_ERR_UNSUPPORTED otherwise): states and v_new are laid
+ * out by 32-column slice, [N * H][chunks_per_chain][V / 32][K or 64][32]: what one scan workgroup saves of a chunk is
+ * then one contiguous block (whole 128-byte lines from one CU instead of 64-byte halves of lines from several), which
+ * gdn_chunk_bwd_local reads with saves_sliced.
  * T / 64 must be even.  The twelve operand fragments of every odd chunk are read from the record of chunk 1 of the chain
  * (in the mirror problem they are the same for all odd chunks: T' = I, P = 0); an odd chunk's own record supplies its
  * row scales and e^{gamma_C} only.
@@ -226,6 +230,8 @@ typedef struct gdn_chunk_saves {
     int32_t v_new_dtype;  /* gdn_dtype of v_new */
     int32_t no_output;
     int32_t mirror_reads;
+    int32_t sliced;
+    int32_t reserved;
     const void *k_odd, *v_odd;
     int64_t k_odd_stride_b, k_odd_stride_t, k_odd_stride_h;
     int64_t v_odd_stride_b, v_odd_stride_t, v_odd_stride_h;
@@ -281,6 +287,9 @@ typedef struct gdn_chunk_local_args {
     const int32_t *seq_start, *seq_len;
     int32_t T_rows;
     int32_t dstates_dtype; /* gdn_dtype of dstates */
+    int32_t saves_sliced;  /* v_new, states, dstates and y_chunks are laid out by 32-column slice, [chunks][V / 32][rows][32]
+                              (gdn_chunk_saves.sliced); all of them bf16 then */
+    int32_t reserved;
 } gdn_chunk_local_args;
 int gdn_chunk_bwd_local(const gdn_chunk_local_args *args, void *stream);
 

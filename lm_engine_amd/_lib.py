@@ -71,6 +71,8 @@ class GdnChunkSaves(ctypes.Structure):
         ("v_new_dtype", ctypes.c_int32),
         ("no_output", ctypes.c_int32),
         ("mirror_reads", ctypes.c_int32),
+        ("sliced", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
         ("k_odd", ctypes.c_void_p),
         ("v_odd", ctypes.c_void_p),
         ("k_odd_stride_b", ctypes.c_int64),
@@ -91,7 +93,8 @@ class GdnChunkLocalArgs(ctypes.Structure):
         + [("H", ctypes.c_int32), ("NC", ctypes.c_int32)]
         + [(name, ctypes.c_void_p) for name in ("q_raw", "k_raw", "v_raw", "dout_raw")]
         + [(f"{x}_stride_{d}", ctypes.c_int64) for x in ("q", "k", "v", "dout") for d in ("b", "t", "h")]
-        + [("seq_start", ctypes.c_void_p), ("seq_len", ctypes.c_void_p), ("T_rows", ctypes.c_int32), ("dstates_dtype", ctypes.c_int32)]
+        + [("seq_start", ctypes.c_void_p), ("seq_len", ctypes.c_void_p), ("T_rows", ctypes.c_int32), ("dstates_dtype", ctypes.c_int32),
+           ("saves_sliced", ctypes.c_int32), ("reserved", ctypes.c_int32)]
     )  # fmt: skip
 
 

@@ -372,25 +372,27 @@ def _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, l2norm
     # products round them to anyway) and form no output; elsewhere fp32 saves and Y from the mirror scan's output.
     given = 0 if sequences is not None else 2 if half_slices else 1
     staged = ops.saving_scan_is_staged(N, T, H, K, V, cu_seqlens, left_padded, given, dev)
+    # where both sweeps stage their saves, what a scan workgroup saves of a chunk lies in one piece (by 32-column slice)
+    sliced = staged and staged_m
     saves = dict(dtype=torch.bfloat16 if staged else torch.float32, device=dev)
     S0 = torch.empty(Bt, NC, K, V, **saves)
     Vn = torch.empty(Bt, NC, CHUNK, V, **saves)
     if sequences is None:
         h0 = None if initial_state is None else initial_state.to(torch.float32).contiguous()
         ops.chunk_scan_given_records(k, v, prep["records_fwd"], h0, S0, NC, half_slice_records=half_slices, v_new=Vn,
-                                     no_output=True, q=q)  # fmt: skip
+                                     no_output=True, q=q, sliced=sliced)  # fmt: skip
     else:
         ops.chunk_forward_saving(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2norm, left_padded, S0, Vn, NC,
-                                 no_output=True)  # fmt: skip
+                                 no_output=True, sliced=sliced)  # fmt: skip
     dht32 = None if dht is None else dht.to(torch.float32).contiguous()
     dS1 = torch.empty(Bt, NC, K, V, device=dev, dtype=torch.bfloat16 if staged_m else torch.float32)
     Y = torch.empty(Bt, NC, CHUNK, V, dtype=torch.bfloat16, device=dev) if staged_m else None
     o_m, dS = ops.chunk_scan_given_records(k if mirror_reads else prep["k_mirror"], prep["v_mirror"], prep["records"],
                                            dht32, dS1, NC, save_every=2, save_reverse=True,
                                            half_slice_records=half_slices, v_new=Y, no_output=staged_m,
-                                           mirror_odd=(q, do) if mirror_reads else None)  # fmt: skip
+                                           mirror_odd=(q, do) if mirror_reads else None, sliced=sliced)  # fmt: skip
     dq, dk, dv, dg, dbeta = ops.chunk_local_grads(q, k, v, do, prep, Y if staged_m else o_m, Vn, S0, dS1, scale, l2norm,
-                                                  sequences)  # fmt: skip
+                                                  sequences, sliced=sliced)  # fmt: skip
     return (
         dq,
         dk,

@@ -196,6 +196,10 @@ int gdn_chunk_fwd_saving(const gdn_args* a, const gdn_chunk_saves* saves, void* 
         return GDN_ERR_UNSUPPORTED;
     if ((saves->states_dtype == GDN_BF16 || saves->v_new_dtype == GDN_BF16) && !gdn::chunk_saving_scan_is_staged(*a, *saves))
         return GDN_ERR_UNSUPPORTED;
+    if (saves->sliced) {  // bf16 saves through the staging variant only
+        if ((saves->states && saves->states_dtype != GDN_BF16) || (saves->v_new && saves->v_new_dtype != GDN_BF16)) return GDN_ERR_UNSUPPORTED;
+        if (!gdn::chunk_saving_scan_is_staged(*a, *saves)) return GDN_ERR_UNSUPPORTED;
+    }
     if (saves->mirror_reads) {
         // only the scan without output reads that way
         if (!saves->records_given || !saves->no_output || a->K < 128 || !gdn::chunk_saving_scan_is_staged(*a, *saves)) return GDN_ERR_UNSUPPORTED;
@@ -224,6 +228,7 @@ int gdn_chunk_bwd_local(const gdn_chunk_local_args* a, void* stream) {
         else if (!aligned(x, 16)) return GDN_ERR_ALIGN;
     if (a->saves_dtype != GDN_BF16 && a->saves_dtype != GDN_F32) return GDN_ERR_UNSUPPORTED;
     if (a->dstates_dtype != GDN_BF16 && a->dstates_dtype != GDN_F32) return GDN_ERR_UNSUPPORTED;
+    if (a->saves_sliced && (a->saves_dtype != GDN_BF16 || a->dstates_dtype != GDN_BF16 || a->y_chunks == nullptr)) return GDN_ERR_UNSUPPORTED;
     if (a->H <= 0 || a->NC <= 0 || a->chunks % ((int64_t)a->H * a->NC) != 0) return GDN_ERR_SHAPE;
     if (a->seq_start != nullptr && (a->seq_len == nullptr || a->T_rows <= 0)) return GDN_ERR_SHAPE;
     const int64_t raw_strides[] = {a->q_stride_b, a->q_stride_t, a->q_stride_h, a->k_stride_b, a->k_stride_t, a->k_stride_h,

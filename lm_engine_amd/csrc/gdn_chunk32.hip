@@ -406,8 +406,14 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
     constexpr bool LSAVE = SAVE && HALF && (K <= 128 || NOOUT);
     constexpr bool LSAVE_NARROW = LSAVE && K > 128;
     constexpr int SROW = 32 * 4;  // bytes per staged row of fp32
-    constexpr int SSTAGE_HALF = LSAVE ? (LSAVE_NARROW ? K * SROW / 2 : K * SROW) : 8;
-    constexpr int VSTAGE_HALF = LSAVE ? (LSAVE_NARROW ? C * SROW / 2 : C * SROW) : 8;
+    // bf16 saves are staged TRANSPOSED, [32 columns][K + 8 keys] (V~: [32 columns][64 + 8 tokens]): a compute-wave lane holds
+    // four consecutive keys (tokens) of one column, so it stages them with one 8-byte write instead of four 2-byte ones
+    // (48 LDS writes per chunk became 12: the staging was 1,660 of the 4,030 cycles of a saving chunk step), and the
+    // store wave turns them back into rows with the transposing LDS load on its way out.
+    constexpr int SCOL = (K + 8) * 2, VCOL = (C + 8) * 2;  // bytes per staged column
+    constexpr int SSTAGE_HALF = LSAVE ? (LSAVE_NARROW ? 32 * SCOL : K * SROW) : 8;
+    constexpr int VSTAGE_HALF = LSAVE ? (LSAVE_NARROW ? 32 * VCOL : C * SROW) : 8;
+    static_assert(32 * SCOL <= K * SROW && 32 * VCOL <= C * SROW, "the transposed bf16 staging fits the fp32 one");
     __shared__ __attribute__((aligned(16))) uint8_t sstage_raw[2 * SSTAGE_HALF];
     __shared__ __attribute__((aligned(16))) uint8_t vstage_raw[2 * VSTAGE_HALF];
     static_assert(!LSAVE || 2 * STAGE_BYTES + OSTAGE_BYTES + 2 * SSTAGE_HALF + 2 * VSTAGE_HALF <= 160 * 1024, "the staging of the saves exceeds LDS");
@@ -495,16 +501,31 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
                         __builtin_nontemporal_store(rows[i], reinterpret_cast<bf16x8*>(og + ((int64_t)c * C + 16 * i) * p.o_stride_t + 32 * w));
             }
         };
-        // LSAVE, bf16 saves: rows of 32 bf16 columns (64 bytes), 4 lanes per row, 16 rows per instruction
-        auto flush_rows16 = [&](const uint8_t* staged, bf16_t* dst, int rows) {  // dst: row 0, column 0 of this slice
-            const int r0 = lane / 4, piece = lane % 4;
+        // LSAVE, bf16 saves: staged as [32 columns][ld rows]; out as rows of 32 columns (64 bytes): lane group `piece`
+        // (16 lanes) takes columns 8 piece .. + 7 of 16 consecutive rows through two transposing loads (4 columns x 16 rows
+        // each), so an instruction writes 16 rows of 64 bytes, 4 lanes per row
+        // (save_sliced: groups of 8 rows, and within a group slice by slice - 8 rows x 64 bytes of a slice are 512
+        // contiguous bytes: element (row, column) at ((row / 8) (V / 32) + column / 32) 256 + (row % 8) 32 + column % 32)
+        const int nslices = p.V / 32;
+        auto flush_rows16 = [&](const uint8_t* staged, int ld, bf16_t* dst, int rows) {  // dst: row 0, column 0 of this slice
+            const int l16 = lane % 16, piece = lane / 16;
+            const bf16_t* const m = reinterpret_cast<const bf16_t*>(staged);
             for (int r = 0; r < rows; r += 64) {
                 bf16x8 x[4];
 #pragma unroll
-                for (int i = 0; i < 4; i++) x[i] = *reinterpret_cast<const bf16x8*>(staged + (r + 16 * i + r0) * (SROW / 2) + 16 * piece);
+                for (int i = 0; i < 4; i++) {
+                    const bf16x4 lo = lds_read_tr4x16<false>(m, ld, 8 * piece, r + 16 * i, l16);
+                    const bf16x4 hi = lds_read_tr4x16<false>(m, ld, 8 * piece + 4, r + 16 * i, l16);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) x[i][e] = lo[e], x[i][4 + e] = hi[e];
+                }
 #pragma unroll
                 for (int i = 0; i < 4; i++)
-                    __builtin_nontemporal_store(x[i], reinterpret_cast<bf16x8*>(dst + (int64_t)(r + 16 * i + r0) * p.V + 8 * piece));
+                {
+                    const int row = r + 16 * i + l16;
+                    bf16_t* const at = p.save_sliced ? dst + ((int64_t)(row / 8) * nslices) * 256 + (row % 8) * 32 + 8 * piece : dst + (int64_t)row * p.V + 8 * piece;
+                    __builtin_nontemporal_store(x[i], reinterpret_cast<bf16x8*>(at));
+                }
             }
         };
         // LSAVE: rows of 32 fp32 columns, 8 lanes per row, 8 rows per instruction
@@ -523,8 +544,8 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
             if constexpr (LSAVE) {
                 const int entry = save_entry(c);
                 if (p.save_state != nullptr && entry >= 0) {
-                    const int64_t at = ((int64_t)chain * p.save_nc + entry) * K * p.V + 32 * vgroup;
-                    if (p.save_state_bf16) flush_rows16(sstage_of(c), reinterpret_cast<bf16_t*>(p.save_state) + at, K);
+                    const int64_t at = ((int64_t)chain * p.save_nc + entry) * K * p.V + (p.save_sliced ? 256 * vgroup : 32 * vgroup);
+                    if (p.save_state_bf16) flush_rows16(sstage_of(c), SCOL / 2, reinterpret_cast<bf16_t*>(p.save_state) + at, K);
                     else flush_rows(sstage_of(c), p.save_state + at, K);
                 }
             }
@@ -533,22 +554,35 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
             if constexpr (LSAVE) {
                 const int entry = save_entry(c);
                 if (p.save_vnew != nullptr && entry >= 0) {
-                    const int64_t at = ((int64_t)chain * p.save_nc + entry) * C * p.V + 32 * vgroup;
-                    if (p.save_vnew_bf16) flush_rows16(vstage_of(c), reinterpret_cast<bf16_t*>(p.save_vnew) + at, C);
+                    const int64_t at = ((int64_t)chain * p.save_nc + entry) * C * p.V + (p.save_sliced ? 256 * vgroup : 32 * vgroup);
+                    if (p.save_vnew_bf16) flush_rows16(vstage_of(c), VCOL / 2, reinterpret_cast<bf16_t*>(p.save_vnew) + at, C);
                     else flush_rows(vstage_of(c), p.save_vnew + at, C);
                 }
             }
         };
         __syncthreads();
+#ifdef GDN_CYCLE_BUDGET
+        uint64_t store_wait = 0;  // cycles this wave spends at the chunks' barriers (slot 7 of the report)
+#endif
         for (int c = 0; c < nchunks; c++) {
             if constexpr (QS) __syncthreads();  // barrier Q
+#ifdef GDN_CYCLE_BUDGET
+            const uint64_t w0 = __builtin_readcyclecounter();
+#endif
             __syncthreads();  // the state of chunk c, V~ and the output of chunk c - 1 are staged
+#ifdef GDN_CYCLE_BUDGET
+            store_wait += __builtin_readcyclecounter() - w0;
+#endif
             flush_state(c);
             if (c > 0) {
                 if constexpr (!NOOUT) flush(c - 1);
                 flush_vnew(c - 1);
             }
         }
+#ifdef GDN_CYCLE_BUDGET
+        if (p.cycle_out != nullptr && lane == 0 && blockIdx.x % 16 == 0 && blockIdx.x / 16 < GDN_CYCLE_BUDGET_SLOTS)
+            p.cycle_out[(blockIdx.x / 16) * 8 + 7] = store_wait;
+#endif
         __syncthreads();
         if (nchunks > 0) {
             if constexpr (!NOOUT) flush(nchunks - 1);
@@ -846,11 +880,14 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
                     // chunks on, after the next chunk's barrier)
                     if (p.save_state != nullptr && save_entry(c) >= 0) {
                         if (p.save_state_bf16) {
-                            uint8_t* const base = sstage_of(c) + (8 * g) * (SROW / 2) + (16 * half + j16) * 2;
+                            // column 16 half + j16, keys 32 (t / 2) + 4 (t % 2) + 8 g + 0..3 of tile t: one 8-byte write
+                            uint8_t* const base = sstage_of(c) + (16 * half + j16) * SCOL + (8 * g) * 2;
 #pragma unroll
-                            for (int t = 0; t < KT; t++)
-#pragma unroll
-                                for (int r = 0; r < 4; r++) *reinterpret_cast<bf16_t*>(base + (32 * (t / 2) + 4 * (t % 2) + r) * (SROW / 2)) = (bf16_t)S[t][r];
+                            for (int t = 0; t < KT; t++) {
+                                bf16x4 x;
+                                x.x = (bf16_t)S[t][0], x.y = (bf16_t)S[t][1], x.z = (bf16_t)S[t][2], x.w = (bf16_t)S[t][3];
+                                *reinterpret_cast<bf16x4*>(base + (32 * (t / 2) + 4 * (t % 2)) * 2) = x;
+                            }
                         } else {
                             uint8_t* const base = sstage_of(c) + (8 * g) * SROW + (16 * half + j16) * 4;
 #pragma unroll
@@ -921,7 +958,13 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
 #endif
                 if constexpr (op + LA < NOPS) fr[op + LA] = lds_frag(st, std::integral_constant<int, (op + LA < NOPS ? op + LA : 0)>{});
                 if constexpr (op == OP_BAR) {
+#ifdef GDN_CYCLE_BUDGET
+                    if constexpr (NOOUT) cyc_tick(3);  // (the scan without output has groups 1 and 4 to spare: 4 = the wait at the barrier)
+#endif
                     __syncthreads();  // this wave is done with chunk c's half; chunk c + 1 is in the other one
+#ifdef GDN_CYCLE_BUDGET
+                    if constexpr (NOOUT) cyc_tick(4);
+#endif
                     egc = lds_eg(stn);
                     if constexpr (!NOOUT) {
 #pragma unroll
@@ -980,11 +1023,14 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
                     // after this chunk's barrier: the store wave takes it after the next one (or the last)
                     if (p.save_vnew != nullptr && save_entry(c) >= 0) {
                         if (p.save_vnew_bf16) {
-                            uint8_t* const base = vstage_of(c) + (4 * g) * (SROW / 2) + (16 * half + j16) * 2;
+                            // column 16 half + j16, tokens 16 tt + 4 g + 0..3: one 8-byte write per tile
+                            uint8_t* const base = vstage_of(c) + (16 * half + j16) * VCOL + (4 * g) * 2;
 #pragma unroll
-                            for (int tt = 0; tt < 4; tt++)
-#pragma unroll
-                                for (int r = 0; r < 4; r++) *reinterpret_cast<bf16_t*>(base + (16 * tt + r) * (SROW / 2)) = (bf16_t)vt[tt][r];
+                            for (int tt = 0; tt < 4; tt++) {
+                                bf16x4 x;
+                                x.x = (bf16_t)vt[tt][0], x.y = (bf16_t)vt[tt][1], x.z = (bf16_t)vt[tt][2], x.w = (bf16_t)vt[tt][3];
+                                *reinterpret_cast<bf16x4*>(base + (16 * tt) * 2) = x;
+                            }
                         } else {
                             uint8_t* const base = vstage_of(c) + (4 * g) * SROW + (16 * half + j16) * 4;
 #pragma unroll
@@ -1005,6 +1051,9 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
                             *reinterpret_cast<float*>(base + (size_t)((16 * tt + r) * row_bytes) + lane_off) = vt[tt][r];
                 }
             }
+#ifdef GDN_CYCLE_BUDGET
+            if constexpr (NOOUT) cyc_tick(1);  // 1 = staging V~ for the store wave (5 then holds the state's staging)
+#endif
         }
 #ifdef GDN_CYCLE_BUDGET
         // wave 0 of every 16th workgroup reports: [workgroup / 16][6 groups | chunks]

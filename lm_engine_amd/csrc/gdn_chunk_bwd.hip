@@ -130,8 +130,11 @@ __device__ __forceinline__ void put4(bf16_t* dst, f32x4 x) {
 
 constexpr int cmax(int a, int b) { return a > b ? a : b; }
 
-// DS1H: dS1 comes as bf16 (fp32 otherwise)
-template <int K, bool DS1H>
+// element (row, column c) of a [rows][V] array laid out by groups of 8 rows and, within a group, by 32-column slice
+__device__ __forceinline__ int sliced_at(int row, int c, int V) { return ((row / 8) * (V / 32) + c / 32) * 256 + (row % 8) * 32 + c % 32; }
+
+// DS1H: dS1 comes as bf16 (fp32 otherwise); SL: V~, S0, dS1 and Y lie in the sliced layout of the staging scans (all bf16)
+template <int K, bool DS1H, bool SL>
 __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_grads_kernel(const ChunkLocalParams p) {
     const int V = p.V;
     constexpr int VW = 64;                     // columns of the value dim staged at a time
@@ -242,9 +245,11 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
                 bf16x8 vr = *reinterpret_cast<const bf16x8*>(row_of(p.v_raw, p.v_stride_b, p.v_stride_t, p.v_stride_h, row) + v0 + 8 * p8);
                 bf16x8 dr = *reinterpret_cast<const bf16x8*>(row_of(p.d_raw, p.d_stride_b, p.d_stride_t, p.d_stride_h, row) + v0 + 8 * p8);
                 if (!live) vr = zero8, dr = zero8;
-                const bf16_t* const yrow = p.y_mirror != nullptr ? p.y_mirror + ((mirA + (C - 1 - row)) * p.H + h) * V
-                                                                 : p.y_chunks + (chunk * C + (C - 1 - row)) * V;
-                const bf16x8 yr = *reinterpret_cast<const bf16x8*>(yrow + v0 + 8 * p8);
+                const bf16_t* yrow;
+                if constexpr (SL) yrow = p.y_chunks + chunk * C * V + sliced_at(C - 1 - row, v0 + 8 * p8, V);
+                else yrow = p.y_mirror != nullptr ? p.y_mirror + ((mirA + (C - 1 - row)) * p.H + h) * V + v0 + 8 * p8
+                                                  : p.y_chunks + (chunk * C + (C - 1 - row)) * V + v0 + 8 * p8;
+                const bf16x8 yr = *reinterpret_cast<const bf16x8*>(yrow);
                 const float b = p.beta[chunk * C + row];
                 bf16x8 dv;
                 float acc = 0.f;
@@ -263,14 +268,16 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
 #pragma unroll
                 for (int it = 0; it < 2; it++) {  // rows of V~ past the end of the sequence hold whatever the scan left
                     const int row = t / 8 + 32 * it;
-                    const bf16x8 x = *reinterpret_cast<const bf16x8*>(vnew + row * V + v0 + 8 * p8);
+                    const bf16x8 x = *reinterpret_cast<const bf16x8*>(SL ? vnew + sliced_at(row, v0 + 8 * p8, V)
+                                                                                : vnew + row * V + v0 + 8 * p8);
                     *reinterpret_cast<bf16x8*>(sVN + row * LDS64 + 8 * p8) = row < valid ? x : zero8;
                 }
                 const bf16_t* s0 = reinterpret_cast<const bf16_t*>(s0b);
 #pragma unroll
                 for (int i = 0; i < K / 32; i++) {  // S0[:, v0 .. v0 + 63]: row = 32 i + t / 8
                     const int row = t / 8 + 32 * i;
-                    *reinterpret_cast<bf16x8*>(sST + row * LDS64 + 8 * p8) = *reinterpret_cast<const bf16x8*>(s0 + row * V + v0 + 8 * p8);
+                    *reinterpret_cast<bf16x8*>(sST + row * LDS64 + 8 * p8) =
+                        *reinterpret_cast<const bf16x8*>(SL ? s0 + sliced_at(row, v0 + 8 * p8, V) : s0 + row * V + v0 + 8 * p8);
                 }
             } else {
                 const float* vnew = reinterpret_cast<const float*>(vnb);
@@ -306,7 +313,10 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
         auto ask_ds1 = [&]() {
             if constexpr (DS1H) {
 #pragma unroll
-                for (int i = 0; i < K / 32; i++) ds1_half[i] = *reinterpret_cast<const bf16x8*>(ds1h + (t / 8 + 32 * i) * V + v0 + 8 * (t % 8));
+                for (int i = 0; i < K / 32; i++) {
+                    const int row = t / 8 + 32 * i, c8 = 8 * (t % 8);
+                    ds1_half[i] = *reinterpret_cast<const bf16x8*>(SL ? ds1h + sliced_at(row, v0 + c8, V) : ds1h + row * V + v0 + c8);
+                }
             } else {
 #pragma unroll
                 for (int i = 0; i < SROWS; i++) {
@@ -1043,6 +1053,7 @@ int launch_chunk_bwd_local(const gdn_chunk_local_args& a, hipStream_t stream) {
     ChunkLocalParams p;
     p.vnew = a.v_new, p.s0 = a.states, p.ds1 = a.dstates, p.saves_bf16 = a.saves_dtype == GDN_BF16 ? 1 : 0;
     const bool h = a.dstates_dtype == GDN_BF16;
+    const bool sl = a.saves_sliced != 0;
     p.gam = a.gamma, p.beta = a.beta;
     p.rq = a.rq, p.rk = a.rk, p.scale = a.scale;
     p.y_mirror = static_cast<const bf16_t*>(a.y_mirror), p.y_chunks = static_cast<const bf16_t*>(a.y_chunks);
@@ -1057,12 +1068,15 @@ int launch_chunk_bwd_local(const gdn_chunk_local_args& a, hipStream_t stream) {
     p.d_stride_b = a.dout_stride_b, p.d_stride_t = a.dout_stride_t, p.d_stride_h = a.dout_stride_h;
     p.seq_start = a.seq_start, p.seq_len = a.seq_len, p.T_rows = a.seq_start != nullptr ? a.T_rows : a.NC * C;
     const dim3 grid((unsigned)a.chunks), block(BWD_THREADS);
-    if (a.K == 64 && h) hipLaunchKernelGGL((chunk_local_grads_kernel<64, true>), grid, block, 0, stream, p);
-    else if (a.K == 64) hipLaunchKernelGGL((chunk_local_grads_kernel<64, false>), grid, block, 0, stream, p);
-    else if (a.K == 128 && h) hipLaunchKernelGGL((chunk_local_grads_kernel<128, true>), grid, block, 0, stream, p);
-    else if (a.K == 128) hipLaunchKernelGGL((chunk_local_grads_kernel<128, false>), grid, block, 0, stream, p);
-    else if (h) hipLaunchKernelGGL((chunk_local_grads_kernel<256, true>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((chunk_local_grads_kernel<256, false>), grid, block, 0, stream, p);
+    auto launch = [&](auto kc) {
+        constexpr int KK = decltype(kc)::value;
+        if (sl) hipLaunchKernelGGL((chunk_local_grads_kernel<KK, true, true>), grid, block, 0, stream, p);
+        else if (h) hipLaunchKernelGGL((chunk_local_grads_kernel<KK, true, false>), grid, block, 0, stream, p);
+        else hipLaunchKernelGGL((chunk_local_grads_kernel<KK, false, false>), grid, block, 0, stream, p);
+    };
+    if (a.K == 64) launch(std::integral_constant<int, 64>{});
+    else if (a.K == 128) launch(std::integral_constant<int, 128>{});
+    else launch(std::integral_constant<int, 256>{});
     return (int)hipGetLastError();
 }
 

@@ -340,7 +340,7 @@ def saving_scan_is_staged(N, T, H, K, V, cu_seqlens=None, left_padded=False, rec
 
 
 def chunk_forward_saving(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2norm, left_padded, states, v_new,
-                         chunks_per_chain, no_output=False):  # fmt: skip
+                         chunks_per_chain, no_output=False, sliced=False):  # fmt: skip
     """The chunked forward once more, for the backward pass: through ``gdn_chunk_fwd_saving`` it writes the
     state every chunk starts from into ``states`` ``[N * H, chunks_per_chain, K, V]`` and V~ into ``v_new``
     ``[N * H, chunks_per_chain, 64, V]`` (contiguous; fp32, or bf16 where ``saving_scan_is_staged``).  The output
@@ -360,7 +360,7 @@ def chunk_forward_saving(q, k, v, g, beta, scale, initial_state, cu_seqlens, l2n
     o = torch.empty(B, T, H, V, dtype=v.dtype, device=v.device)
     args = _fill_args(q, k, v, g, beta, h0, None, o, cu_seqlens, scale, l2norm, False, dims, left_padded)
     saves = _lib.GdnChunkSaves(states.data_ptr(), v_new.data_ptr(), chunks_per_chain, 0, 1, 0, states_code, v_new_code,
-                               1 if no_output else 0, 0)  # fmt: skip
+                               1 if no_output else 0, 0, 1 if sliced else 0)  # fmt: skip
     with torch.cuda.device(q.device):
         nbytes = lib.gdn_workspace_bytes(ctypes.byref(args))
         workspace = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=q.device)
@@ -378,7 +378,7 @@ def half_slice_records_pay(chains: int, V: int, device) -> bool:
 
 
 def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_chain, save_every=1, save_reverse=False,
-                             half_slice_records=False, v_new=None, no_output=False, q=None, mirror_odd=None):
+                             half_slice_records=False, v_new=None, no_output=False, q=None, mirror_odd=None, sliced=False):
     """The scan kernel alone over a fixed-length batch whose chunk records the caller has written
     (``records`` uint8 ``[H, B * T / 64, record bytes]``, T a multiple of 64); it reads the rows of ``q``, ``k`` and
     ``v`` (without ``q``, ``k`` stands in its place: the records of a mirror problem carry zero row scales for q).  Returns ``(o, final_state)``
@@ -391,7 +391,9 @@ def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_ch
     ``mirror_odd = (k_odd, v_odd)`` (with ``no_output``, where the scan without output exists): ``k``, ``v`` and these two
     are ``[B, T / 2, H, .]`` tensors that the scan reads backwards, every chunk twice - the even chunks' rows from ``k``
     and ``v``, the odd chunks' from ``k_odd`` and ``v_odd`` (``gdn_chunk_saves.mirror_reads``): the mirror problem of
-    ``chunk_bwd_prepare(..., reversed_copies=False)``."""
+    ``chunk_bwd_prepare(..., reversed_copies=False)``.  ``sliced`` (bf16 saves where ``saving_scan_is_staged``): the
+    save arrays are laid out by 32-column slice, ``[B H, chunks_per_chain, V / 32, K or 64, 32]`` in the memory of the
+    arrays given (``gdn_chunk_saves.sliced``), for ``chunk_local_grads(..., sliced=True)``."""
     _require_hip_path()
     lib = _lib.load_library()
     q = k if q is None else q
@@ -415,6 +417,7 @@ def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_ch
     saves = _lib.GdnChunkSaves(states.data_ptr(), None if v_new is None else v_new.data_ptr(), chunks_per_chain,
                                2 if half_slice_records else 1, save_every, 1 if save_reverse else 0, states_code,
                                v_new_code, 1 if no_output else 0, 0)  # fmt: skip
+    saves.sliced = 1 if sliced else 0
     if mirror_odd is not None:
         saves.mirror_reads, saves.k_odd, saves.v_odd = 1, k_odd.data_ptr(), v_odd.data_ptr()
         saves.k_odd_stride_b, saves.k_odd_stride_t, saves.k_odd_stride_h = k_odd.stride(0), k_odd.stride(1), k_odd.stride(2)
@@ -431,7 +434,7 @@ def backward_kernels_apply(K: int, V: int) -> bool:
     return K in _SUPPORTED_K and V % 64 == 0
 
 
-def chunk_local_grads(q, k, v, dout, prep, y_mirror, v_new, states, dstates, scale, l2norm, sequences=None):
+def chunk_local_grads(q, k, v, dout, prep, y_mirror, v_new, states, dstates, scale, l2norm, sequences=None, sliced=False):
     """``gdn_chunk_bwd_local``: q, k, v, dout are the caller's bf16 ``[B, T, H, D]`` tensors (last dim contiguous),
     ``prep`` what ``chunk_bwd_prepare`` returned (same ``sequences``), ``y_mirror`` the output of the scan over its
     mirror problem (bf16 ``[N, 2 NC 64, H, V]``) or, as a 4-D tensor, the V~ that scan saved at its even chunks (bf16
@@ -473,6 +476,7 @@ def chunk_local_grads(q, k, v, dout, prep, y_mirror, v_new, states, dstates, sca
     a.v_new, a.states, a.dstates = v_new.data_ptr(), states.data_ptr(), dstates.data_ptr()
     a.saves_dtype = _dtype_code(states.dtype, "states")
     a.dstates_dtype = _dtype_code(dstates.dtype, "dstates")
+    a.saves_sliced = 1 if sliced else 0  # (the sweeps wrote v_new, states, dstates and the chunked Y by 32-column slice)
     if y_chunked:
         a.y_chunks = y_mirror.data_ptr()
     else:
