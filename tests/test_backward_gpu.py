@@ -405,3 +405,35 @@ def test_mirror_reads_equal_the_scan_over_reversed_copies(K, V, B, T, H):
     for name, a, b in zip(("saved states", "saved Y", "final state"), *results):
         assert a.abs().max() > 0, name
         assert torch.equal(a, b), f"{name}: rel-L2 {rel_l2(a.float(), b.float()):.3e}"
+
+
+def _unslice(x, rows):
+    """[chains, entries, rows, V] array written with ``gdn_chunk_saves.sliced`` -> its [.., rows, V] meaning: memory is
+    [rows / 8][V / 32][8][32] per entry."""
+    ch, nc, r, V = x.shape
+    assert r == rows
+    return x.reshape(ch, nc, rows // 8, V // 32, 8, 32).permute(0, 1, 2, 4, 3, 5).reshape(ch, nc, rows, V)
+
+
+@pytest.mark.parametrize("K, V, no_output", [(128, 128, False), (128, 256, True), (256, 512, True), (64, 64, False)])
+def test_sliced_saves_hold_the_same_values(K, V, no_output):
+    """bf16 saves in the sliced layout (groups of 8 rows, 32-column slice by slice: whole lines per scan workgroup) against
+    the same saves in rows of V columns: the same values, bit for bit, once the layout is undone."""
+    from lm_engine_amd import ops
+
+    B, T, H = 2, 256, 2
+    inp = random_inputs(B=B, T=T, H=H, K=K, V=V, dtype=torch.bfloat16, seed=17)
+    dev = {n: (None if x is None else x.cuda()) for n, x in inp.items()}
+    NC = T // 64
+    assert ops.saving_scan_is_staged(B, T, H, K, V, None, False, 0, "cuda", no_output=no_output)
+    out = []
+    for sliced in (False, True):
+        states = torch.zeros(B * H, NC, K, V, dtype=torch.bfloat16, device="cuda")
+        v_new = torch.zeros(B * H, NC, 64, V, dtype=torch.bfloat16, device="cuda")
+        ops.chunk_forward_saving(dev["q"], dev["k"], dev["v"], dev["g"], dev["beta"], None, dev["initial_state"], None,
+                                 True, False, states, v_new, NC, no_output=no_output, sliced=sliced)  # fmt: skip
+        torch.cuda.synchronize()
+        out.append((states.cpu(), v_new.cpu()))
+    assert out[0][0].abs().max() > 0 and out[0][1].abs().max() > 0
+    assert torch.equal(out[0][0], _unslice(out[1][0], K)), "states"
+    assert torch.equal(out[0][1], _unslice(out[1][1], 64)), "V~"
