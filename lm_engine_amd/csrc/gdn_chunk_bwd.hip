@@ -107,6 +107,22 @@ __device__ __forceinline__ f32x16 mma_tn(const bf16_t* M, int ldm, int col0, con
     return acc;
 }
 
+// acc[r] += sum_t A[8 (r/4) + 4 h + r%4][t] M[t][col0 + l32] over t < kd: the B operand is the transpose of 32 columns of the
+// row-major matrix M (same transposing loads as mma_tn, on the other operand)
+__device__ __forceinline__ f32x16 mma_nn(const bf16_t* A, int lda, const bf16_t* M, int ldm, int col0, int kd, f32x16 acc, int l32, int lh) {
+    const int l16 = l32 % 16, g16 = l32 / 16;
+    for (int kk = 0; kk < kd; kk += 16) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(A + l32 * lda + kk + 8 * lh);
+        const bf16x4 lo = lds_read_tr4x16<false>(M, ldm, kk + 8 * lh, col0 + 16 * g16, l16);
+        const bf16x4 hi = lds_read_tr4x16<false>(M, ldm, kk + 8 * lh + 4, col0 + 16 * g16, l16);
+        bf16x8 b;
+#pragma unroll
+        for (int e = 0; e < 4; e++) b[e] = lo[e], b[4 + e] = hi[e];
+        acc = mfma32_bf16(a, b, acc);
+    }
+    return acc;
+}
+
 // Sixteen sums over the 32 lanes of a wave half at once: on return every lane holds the sum of x[l32 / 2].  Each
 // exchange halves the number of values a lane carries (16 shuffles instead of 80).
 __device__ __forceinline__ float half_sums16(const float (&x)[16], int l32) {
@@ -757,20 +773,22 @@ __device__ __forceinline__ void invert_unit_lower_64(float* sA, float* scratch, 
 }
 
 template <int K>
-__global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_bwd_prepare_kernel(const BwdPrepareParams p) {
+__global__ __launch_bounds__(BWD_THREADS, (K <= 64 ? 3 : K <= 128 ? 2 : 1)) void chunk_bwd_prepare_kernel(const BwdPrepareParams p) {
     const int V = p.V;
     constexpr int LDK = K + 8;                 // bf16 per LDS row of q / k
     constexpr int CPR = K / 8;                 // 16-byte pieces per row of q / k
     constexpr int RPP = BWD_THREADS / CPR;     // rows per pass of their copy
-    // dO is staged transposed, 128 (or a last 64) columns at a time, over the rows of q and k once they are dead
-    static_assert(128 * LDS64 * 2 <= 2 * C * LDK * 2, "a slab of dO^T fits the rows of q and k");
-    __shared__ __attribute__((aligned(16))) bf16_t sQK[2 * C * LDK];   // rows of q, of k; then slabs of dO^T; then the scratch of the inverse
+    // dO is staged as it lies (rows of tokens), 128 (or a last 64) columns at a time, over the rows of q and k once they
+    // are dead; P^T dO takes it as the B operand through the transposing LDS load (staging it transposed took 32 2-byte
+    // writes per thread and slab with 16-way bank conflicts: a third of the kernel's cycles at V = 512)
+    static_assert(128 * LDS64 * 2 <= 2 * C * LDK * 2, "a slab of dO fits the rows of q and k");
+    __shared__ __attribute__((aligned(16))) bf16_t sQK[2 * C * LDK];   // rows of q, of k; then slabs of dO; then the scratch of the inverse
     __shared__ __attribute__((aligned(16))) bf16_t sPT[C * LDS64];     // P^T
     __shared__ __attribute__((aligned(16))) float sA[C * LDA];         // A, then T in its place
     __shared__ float s_gam[C], s_beta[C], s_e[C], s_tail[C], s_rq[C], s_rk[C];
     bf16_t* const sQ = sQK;
     bf16_t* const sK = sQK + C * LDK;
-    bf16_t* const sDOT = sQK;  // [VS][LDS64]
+    bf16_t* const sDO = sQK;  // [64][VS + 8]
 
     const int t = threadIdx.x;
     const int lane = t % WAVE, wave = t / WAVE;
@@ -931,8 +949,7 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_bwd_pre
                 if (v0 == 0) dr = dpre[it];  // (uniform)
                 else dr = *reinterpret_cast<const bf16x8*>(row_of(p.dout, p.d_stride_b, p.d_stride_t, p.d_stride_h, row) + v0 + 8 * p8);
                 if (row >= valid) dr = zero8;
-#pragma unroll
-                for (int e = 0; e < 8; e++) sDOT[(8 * p8 + e) * LDS64 + row] = dr[e];
+                *reinterpret_cast<bf16x8*>(sDO + row * (VS + 8) + 8 * p8) = dr;
                 if (copies) *reinterpret_cast<bf16x8*>(p.v_m + (tok_a(row) + (int64_t)C * p.H) * V + v0 + 8 * p8) = dr;
             }
             __syncthreads();
@@ -945,7 +962,7 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_bwd_pre
             for (int tv = wave; tv < VS / 32; tv += BWD_THREADS / WAVE)
 #pragma unroll
                 for (int tj = 0; tj < 2; tj++) {
-                    const f32x16 u = mma_nt(sPT + 32 * tj * LDS64, LDS64, sDOT + 32 * tv * LDS64, LDS64, C, zero, l32, lh);
+                    const f32x16 u = mma_nn(sPT + 32 * tj * LDS64, LDS64, sDO, VS + 8, 32 * tv, C, zero, l32, lh);
 #pragma unroll
                     for (int r = 0; r < 16; r++) {
                         const int j = 32 * tj + 8 * (r / 4) + 4 * lh + r % 4;
