@@ -773,7 +773,7 @@ __device__ __forceinline__ void invert_unit_lower_64(float* sA, float* scratch, 
 }
 
 template <int K>
-__global__ __launch_bounds__(BWD_THREADS, (K <= 64 ? 3 : K <= 128 ? 2 : 1)) void chunk_bwd_prepare_kernel(const BwdPrepareParams p) {
+__global__ __launch_bounds__(BWD_THREADS, (K <= 64 ? 3 : 2)) void chunk_bwd_prepare_kernel(const BwdPrepareParams p) {
     const int V = p.V;
     constexpr int LDK = K + 8;                 // bf16 per LDS row of q / k
     constexpr int CPR = K / 8;                 // 16-byte pieces per row of q / k
@@ -781,13 +781,18 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 64 ? 3 : K <= 128 ? 2 : 1)) void
     // dO is staged as it lies (rows of tokens), 128 (or a last 64) columns at a time, over the rows of q and k once they
     // are dead; P^T dO takes it as the B operand through the transposing LDS load (staging it transposed took 32 2-byte
     // writes per thread and slab with 16-way bank conflicts: a third of the kernel's cycles at V = 512)
-    static_assert(128 * LDS64 * 2 <= 2 * C * LDK * 2, "a slab of dO fits the rows of q and k");
-    __shared__ __attribute__((aligned(16))) bf16_t sQK[2 * C * LDK];   // rows of q, of k; then slabs of dO; then the scratch of the inverse
+    // K = 256: the rows of q are staged one half of the key dim at a time (Q K^T adds up over the halves, the second
+    // half waits in registers), which brings the workgroup from 96 KB of LDS to 79 KB: two per CU instead of one.
+    constexpr bool QH = K > 128;
+    constexpr int LDQ = QH ? K / 2 + 8 : LDK;  // bf16 per LDS row of (the staged half of) q
+    constexpr int QK_ELEMS = C * LDQ + C * LDK;
+    static_assert((128 + 8) * C <= QK_ELEMS, "a slab of dO fits the rows of q and k");
+    __shared__ __attribute__((aligned(16))) bf16_t sQK[QK_ELEMS];   // rows of q, of k; then slabs of dO; then the scratch of the inverse
     __shared__ __attribute__((aligned(16))) bf16_t sPT[C * LDS64];     // P^T
     __shared__ __attribute__((aligned(16))) float sA[C * LDA];         // A, then T in its place
     __shared__ float s_gam[C], s_beta[C], s_e[C], s_tail[C], s_rq[C], s_rk[C];
     bf16_t* const sQ = sQK;
-    bf16_t* const sK = sQK + C * LDK;
+    bf16_t* const sK = sQK + C * LDQ;
     bf16_t* const sDO = sQK;  // [64][VS + 8]
 
     const int t = threadIdx.x;
@@ -904,7 +909,12 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 64 ? 3 : K <= 128 ? 2 : 1)) void
                     qb[e] = (bf16_t)((float)qr[e] * rq * p.scale);
                     kb[e] = (bf16_t)((float)kr[e] * rk);
                 }
-                *reinterpret_cast<bf16x8*>(sQ + row * LDK + 8 * p8) = qb;
+                if constexpr (QH) {
+                    qn[it] = qb;  // scaled; the pieces of the second half are written after the first half's products
+                    if (p8 < CPR / 2) *reinterpret_cast<bf16x8*>(sQ + row * LDQ + 8 * p8) = qb;
+                } else {
+                    *reinterpret_cast<bf16x8*>(sQ + row * LDQ + 8 * p8) = qb;
+                }
                 *reinterpret_cast<bf16x8*>(sK + row * LDK + 8 * p8) = kb;
                 // mirror rows: k of chunk A is k, k of chunk B is q
                 if (copies) {
@@ -924,7 +934,17 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 64 ? 3 : K <= 128 ? 2 : 1)) void
         {
             const int ti = wave / 2, tj = wave % 2;
             const f32x16 KK = mma_nt(sK + 32 * ti * LDK, LDK, sK + 32 * tj * LDK, LDK, K, zero, l32, lh);
-            const f32x16 QK = mma_nt(sQ + 32 * ti * LDK, LDK, sK + 32 * tj * LDK, LDK, K, zero, l32, lh);
+            f32x16 QK = mma_nt(sQ + 32 * ti * LDQ, LDQ, sK + 32 * tj * LDK, LDK, QH ? K / 2 : K, zero, l32, lh);
+            if constexpr (QH) {
+                __syncthreads();  // the first half of q has been read
+                const int p8 = t % CPR;
+                if (p8 >= CPR / 2) {
+#pragma unroll
+                    for (int it = 0; it < C / RPP; it++) *reinterpret_cast<bf16x8*>(sQ + (t / CPR + RPP * it) * LDQ + 8 * (p8 - CPR / 2)) = qn[it];
+                }
+                __syncthreads();
+                QK = mma_nt(sQ + 32 * ti * LDQ, LDQ, sK + 32 * tj * LDK + K / 2, LDK, K / 2, QK, l32, lh);
+            }
             const int j = 32 * tj + l32;
             const float gj = s_gam[j];
 #pragma unroll
@@ -956,7 +976,7 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 64 ? 3 : K <= 128 ? 2 : 1)) void
             // rows j = 32 tj + .., columns v = v0 + 32 tv + l32, tv = wave, wave + 4, ..
             // K >= 128: the rows of q and k leave room behind the slab for the 64 x VS result, which then goes out as whole
             // rows (16 bytes per lane) instead of 2-byte pieces that fill half a line per store
-            constexpr bool STAGED = 2 * C * LDK * 2 >= 128 * LDS64 * 2 + C * 128 * 2;
+            constexpr bool STAGED = QK_ELEMS >= 128 * LDS64 + C * 128;
             bf16_t* const sU = sQK + 128 * LDS64;  // [64][VS]
 #pragma unroll
             for (int tv = wave; tv < VS / 32; tv += BWD_THREADS / WAVE)
@@ -986,7 +1006,7 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 64 ? 3 : K <= 128 ? 2 : 1)) void
         if (v0 < V) slab(v0, std::integral_constant<int, 64>{});
 
         // ---- T = (I + A)^-1 in place of A (its scratch over the dead rows of q) ----
-        static_assert(INVERSE_SCRATCH_FLOATS * 4 <= 2 * C * LDK * 2, "the scratch of the inverse fits the rows of q and k");
+        static_assert(INVERSE_SCRATCH_FLOATS * 4 <= QK_ELEMS * 2, "the scratch of the inverse fits the rows of q and k");
         invert_unit_lower_64<LDA>(sA, reinterpret_cast<float*>(sQK), wave, lane);
     }
 
