@@ -6,10 +6,10 @@ the gradients of ``(o, final_state)`` with respect to ``(q, k, v, g, beta, initi
 
 Three ways through, same formulas:
 
-* bf16, K = 128, V = 128, 256 or 512 (whole rows, packed or left-padded batches): five kernel launches
+* bf16, K = 64, 128 or 256, V a multiple of 64 (whole rows, packed or left-padded batches): four kernel launches
   (``_backward_on_kernels``) - ``gdn_chunk_bwd_prepare``, ``gdn_chunk_fwd_saving`` for the forward sweep and
   again over the mirror problem for the reverse sweep, ``gdn_chunk_bwd_local``;
-* other bf16 shapes: the two sweeps over the chunks of a chain on the scan kernel
+* other bf16 shapes (V a multiple of 32 only): the two sweeps over the chunks of a chain on the scan kernel
   (``gdn_chunk_fwd_saving``: the forward's scan in a variant that also writes the chunk states and V~),
   everything chunk-local as batched library GEMMs (fp32, ``torch.bmm``) and elementwise torch operations on
   sequences padded to whole chunks;
