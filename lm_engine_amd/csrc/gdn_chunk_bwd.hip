@@ -247,11 +247,86 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
     const bf16_t* const ds1h = static_cast<const bf16_t*>(p.ds1) + chunk * K * (int64_t)V;    // when bf16
     constexpr int SROWS = K / 16;  // 16-byte fp32 pieces of a state slab per thread: K rows x 16 pieces
     float dot = 0.f;
+    // K = 256 on the sliced bf16 saves (a CU to itself: one wave per SIMD, 512 registers each): the rows of the next
+    // slab are asked for while the products of this one run and wait in registers, so that no trip through memory
+    // stands between a slab's barriers.
+    constexpr bool PIPE = SL && K > 128;
+    bf16x8 nx_v[PIPE ? 2 : 1], nx_d[PIPE ? 2 : 1], nx_y[PIPE ? 2 : 1], nx_vn[PIPE ? 2 : 1], nx_s0[TR ? K / 32 : 1];  // nx_s0: also q and k on their way into LDS
+    auto ask_slab = [&](int v0) {
+        const int p8 = t % 8;
+        const bf16_t* vnew = reinterpret_cast<const bf16_t*>(vnb);
+        const bf16_t* s0 = reinterpret_cast<const bf16_t*>(s0b);
+#pragma unroll
+        for (int it = 0; it < 2; it++) {
+            const int row = t / 8 + 32 * it;
+            nx_v[it] = *reinterpret_cast<const bf16x8*>(row_of(p.v_raw, p.v_stride_b, p.v_stride_t, p.v_stride_h, row) + v0 + 8 * p8);
+            nx_d[it] = *reinterpret_cast<const bf16x8*>(row_of(p.d_raw, p.d_stride_b, p.d_stride_t, p.d_stride_h, row) + v0 + 8 * p8);
+            nx_y[it] = *reinterpret_cast<const bf16x8*>(p.y_chunks + chunk * C * V + sliced_at(C - 1 - row, v0 + 8 * p8, V));
+            nx_vn[it] = *reinterpret_cast<const bf16x8*>(vnew + sliced_at(row, v0 + 8 * p8, V));
+        }
+#pragma unroll
+        for (int i = 0; i < K / 32; i++) nx_s0[i] = *reinterpret_cast<const bf16x8*>(s0 + sliced_at(t / 8 + 32 * i, v0 + 8 * p8, V));
+    };
+    // rows of q and k (keys KW kh ..) into registers, and from there, scaled, row-major into sQ and sK (TR only)
+    auto ask_qk = [&](int kh) {
+        constexpr int CPR = KW / 8, RPP = BWD_THREADS / CPR;  // 16-byte pieces per staged row, rows per pass
+        int tl = t;
+        asm volatile("" : "+v"(tl));  // the row addresses are formed here, not ahead of phase 1 (where they would be spilled)
+        const int p8 = tl % CPR;
+#pragma unroll
+        for (int it = 0; it < C / RPP; it++) {
+            const int row = tl / CPR + RPP * it;
+            nx_s0[2 * it] = *reinterpret_cast<const bf16x8*>(row_of(p.q_raw, p.q_stride_b, p.q_stride_t, p.q_stride_h, row) + KW * kh + 8 * p8);
+            nx_s0[2 * it + 1] = *reinterpret_cast<const bf16x8*>(row_of(p.k_raw, p.k_stride_b, p.k_stride_t, p.k_stride_h, row) + KW * kh + 8 * p8);
+        }
+    };
+    auto put_qk = [&]() {
+        constexpr int CPR = KW / 8, RPP = BWD_THREADS / CPR;
+        const int p8 = t % CPR;
+#pragma unroll
+        for (int it = 0; it < C / RPP; it++) {
+            const int row = t / CPR + RPP * it;
+            const bool live = row < valid;
+            const float fq = live ? s_fq[row] : 0.f, fk = live ? s_fk[row] : 0.f;
+            bf16x8 qb, kb;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                qb[e] = (bf16_t)((float)nx_s0[2 * it][e] * fq);
+                kb[e] = (bf16_t)((float)nx_s0[2 * it + 1][e] * fk);
+            }
+            *reinterpret_cast<bf16x8*>(sQ + row * LDK + 8 * p8) = qb;
+            *reinterpret_cast<bf16x8*>(sK + row * LDK + 8 * p8) = kb;
+        }
+    };
+    if constexpr (PIPE) ask_slab(0);
 #pragma unroll 1
     for (int hv = 0; hv < V / VW; hv++) {
         const int v0 = VW * hv;
         float yv[2];  // <Y_i, V_i> pieces, reduced after the barrier (s_dbeta is cleared before the first one)
-        {
+        if constexpr (PIPE) {
+            const int p8 = t % 8;
+#pragma unroll
+            for (int it = 0; it < 2; it++) {
+                const int row = t / 8 + 32 * it;
+                const bool live = row < valid;
+                const bf16x8 vr = live ? nx_v[it] : zero8, dr = live ? nx_d[it] : zero8, yr = nx_y[it];
+                const float b = p.beta[chunk * C + row];
+                bf16x8 dv;
+                float acc = 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    dv[e] = (bf16_t)((float)yr[e] * b);
+                    acc += (float)yr[e] * (float)vr[e];
+                }
+                *reinterpret_cast<bf16x8*>(sDO + row * LDS64 + 8 * p8) = dr;
+                *reinterpret_cast<bf16x8*>(sY + row * LDS64 + 8 * p8) = yr;
+                *reinterpret_cast<bf16x8*>(sVN + row * LDS64 + 8 * p8) = live ? nx_vn[it] : zero8;
+                if (live) *reinterpret_cast<bf16x8*>(p.dv_out + ((tok0 + row) * p.H + h) * V + v0 + 8 * p8) = dv;
+                yv[it] = acc;
+            }
+#pragma unroll
+            for (int i = 0; i < K / 32; i++) *reinterpret_cast<bf16x8*>(sST + (t / 8 + 32 * i) * LDS64 + 8 * p8) = nx_s0[i];
+        } else {
             // v, dO and Y (token `row` is token 63 - row of mirror chunk A); dV = beta Y goes out right away
             const int p8 = t % 8;
 #pragma unroll
@@ -342,7 +417,11 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
             }
         };
         if constexpr (PREFETCH) {
-            ask_ds1();
+            ask_ds1();  // first: it is waited for first
+            if constexpr (PIPE) {
+                if (hv + 1 < V / VW) ask_slab(v0 + VW);
+                else ask_qk(0);
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
@@ -389,30 +468,6 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
     dot = wave_sum(dot);
     if (lane == 0) atomicAdd(&s_red[0], dot);
 
-    // rows of q and k (keys KW kh ..), scaled, row-major into sQ and sK
-    auto stage_qk = [&](int kh) {
-        constexpr int CPR = KW / 8, RPP = BWD_THREADS / CPR;  // 16-byte pieces per staged row, rows per pass
-        int tl = t;
-        asm volatile("" : "+v"(tl));  // the row addresses are formed here, not ahead of phase 1 (where they would be spilled)
-        const int p8 = tl % CPR;
-#pragma unroll
-        for (int it = 0; it < C / RPP; it++) {
-            const int row = tl / CPR + RPP * it;
-            bf16x8 qr = *reinterpret_cast<const bf16x8*>(row_of(p.q_raw, p.q_stride_b, p.q_stride_t, p.q_stride_h, row) + KW * kh + 8 * p8);
-            bf16x8 kr = *reinterpret_cast<const bf16x8*>(row_of(p.k_raw, p.k_stride_b, p.k_stride_t, p.k_stride_h, row) + KW * kh + 8 * p8);
-            if (row >= valid) qr = zero8, kr = zero8;
-            const float fq = s_fq[row], fk = s_fk[row];
-            bf16x8 qb, kb;
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                qb[e] = (bf16_t)((float)qr[e] * fq);
-                kb[e] = (bf16_t)((float)kr[e] * fk);
-            }
-            *reinterpret_cast<bf16x8*>(sQ + row * LDK + 8 * p8) = qb;
-            *reinterpret_cast<bf16x8*>(sK + row * LDK + 8 * p8) = kb;
-        }
-    };
-
     // ---------------- phase 2: Q K^T, K K^T and the 64 x 64 stage ----------------
     // wave -> tile (ti, tj); rows i = 32 ti + 8 (r/4) + 4 h + r%4, column j = 32 tj + l32
     {
@@ -422,7 +477,10 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
         for (int kh = 0; kh < KH; kh++) {
             if (kh > 0) __syncthreads();  // the products of the previous half have read q and k
             if constexpr (TR) {
-                stage_qk(kh);
+                if constexpr (!PIPE) {
+                    if (kh == 0) ask_qk(0);
+                }
+                put_qk();
             } else {
                 constexpr int CPR = KW / 8, RPP = BWD_THREADS / CPR;
                 const int p8 = t % CPR;
@@ -444,6 +502,10 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
                 }
             }
             __syncthreads();
+            if constexpr (TR) {  // the rows staged next travel while these products run: the other half, then half 0 again for phase 3
+                ask_qk(kh + 1 < KH ? kh + 1 : 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
             QK = mma_nt(sQ + 32 * ti * LDK, LDK, sK + 32 * tj * LDK, LDK, KW, QK, l32, lh);
             KK = mma_nt(sK + 32 * ti * LDK, LDK, sK + 32 * tj * LDK, LDK, KW, KK, l32, lh);
         }
@@ -498,7 +560,7 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
         __syncthreads();  // G, G^T, Hm + Hm^T are complete (or: the previous half's reads are over)
         if constexpr (TR) {
             if (kx > 0) {
-                stage_qk(kh);
+                put_qk();
                 __syncthreads();
             }
         } else {
