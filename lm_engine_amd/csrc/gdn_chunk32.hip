@@ -504,9 +504,8 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
         // LSAVE, bf16 saves: staged as [32 columns][ld rows]; out as rows of 32 columns (64 bytes): lane group `piece`
         // (16 lanes) takes columns 8 piece .. + 7 of 16 consecutive rows through two transposing loads (4 columns x 16 rows
         // each), so an instruction writes 16 rows of 64 bytes, 4 lanes per row
-        // (save_sliced: groups of 8 rows, and within a group slice by slice - 8 rows x 64 bytes of a slice are 512
-        // contiguous bytes: element (row, column) at ((row / 8) (V / 32) + column / 32) 256 + (row % 8) 32 + column % 32)
-        const int nslices = p.V / 32;
+        // (save_sliced: slice by slice, a slice's rows of 64 bytes one after the other - what a workgroup saves of a chunk
+        // is one contiguous block: element (row, column) at (column / 32) rows 32 + row 32 + column % 32)
         auto flush_rows16 = [&](const uint8_t* staged, int ld, bf16_t* dst, int rows) {  // dst: row 0, column 0 of this slice
             const int l16 = lane % 16, piece = lane / 16;
             const bf16_t* const m = reinterpret_cast<const bf16_t*>(staged);
@@ -523,7 +522,7 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
                 for (int i = 0; i < 4; i++)
                 {
                     const int row = r + 16 * i + l16;
-                    bf16_t* const at = p.save_sliced ? dst + ((int64_t)(row / 8) * nslices) * 256 + (row % 8) * 32 + 8 * piece : dst + (int64_t)row * p.V + 8 * piece;
+                    bf16_t* const at = p.save_sliced ? dst + row * 32 + 8 * piece : dst + (int64_t)row * p.V + 8 * piece;
                     __builtin_nontemporal_store(x[i], reinterpret_cast<bf16x8*>(at));
                 }
             }
@@ -544,7 +543,7 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
             if constexpr (LSAVE) {
                 const int entry = save_entry(c);
                 if (p.save_state != nullptr && entry >= 0) {
-                    const int64_t at = ((int64_t)chain * p.save_nc + entry) * K * p.V + (p.save_sliced ? 256 * vgroup : 32 * vgroup);
+                    const int64_t at = ((int64_t)chain * p.save_nc + entry) * K * p.V + (p.save_sliced ? K * 32 * vgroup : 32 * vgroup);
                     if (p.save_state_bf16) flush_rows16(sstage_of(c), SCOL / 2, reinterpret_cast<bf16_t*>(p.save_state) + at, K);
                     else flush_rows(sstage_of(c), p.save_state + at, K);
                 }
@@ -554,7 +553,7 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
             if constexpr (LSAVE) {
                 const int entry = save_entry(c);
                 if (p.save_vnew != nullptr && entry >= 0) {
-                    const int64_t at = ((int64_t)chain * p.save_nc + entry) * C * p.V + (p.save_sliced ? 256 * vgroup : 32 * vgroup);
+                    const int64_t at = ((int64_t)chain * p.save_nc + entry) * C * p.V + (p.save_sliced ? C * 32 * vgroup : 32 * vgroup);
                     if (p.save_vnew_bf16) flush_rows16(vstage_of(c), VCOL / 2, reinterpret_cast<bf16_t*>(p.save_vnew) + at, C);
                     else flush_rows(vstage_of(c), p.save_vnew + at, C);
                 }

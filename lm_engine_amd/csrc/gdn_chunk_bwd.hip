@@ -147,7 +147,7 @@ __device__ __forceinline__ void put4(bf16_t* dst, f32x4 x) {
 constexpr int cmax(int a, int b) { return a > b ? a : b; }
 
 // element (row, column c) of a [rows][V] array laid out by groups of 8 rows and, within a group, by 32-column slice
-__device__ __forceinline__ int sliced_at(int row, int c, int V) { return ((row / 8) * (V / 32) + c / 32) * 256 + (row % 8) * 32 + c % 32; }
+__device__ __forceinline__ int sliced_at(int row, int c, int rows) { return (c / 32) * rows * 32 + row * 32 + c % 32; }
 
 // DS1H: dS1 comes as bf16 (fp32 otherwise); SL: V~, S0, dS1 and Y lie in the sliced layout of the staging scans (all bf16)
 template <int K, bool DS1H, bool SL>
@@ -261,11 +261,11 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
             const int row = t / 8 + 32 * it;
             nx_v[it] = *reinterpret_cast<const bf16x8*>(row_of(p.v_raw, p.v_stride_b, p.v_stride_t, p.v_stride_h, row) + v0 + 8 * p8);
             nx_d[it] = *reinterpret_cast<const bf16x8*>(row_of(p.d_raw, p.d_stride_b, p.d_stride_t, p.d_stride_h, row) + v0 + 8 * p8);
-            nx_y[it] = *reinterpret_cast<const bf16x8*>(p.y_chunks + chunk * C * V + sliced_at(C - 1 - row, v0 + 8 * p8, V));
-            nx_vn[it] = *reinterpret_cast<const bf16x8*>(vnew + sliced_at(row, v0 + 8 * p8, V));
+            nx_y[it] = *reinterpret_cast<const bf16x8*>(p.y_chunks + chunk * C * V + sliced_at(C - 1 - row, v0 + 8 * p8, C));
+            nx_vn[it] = *reinterpret_cast<const bf16x8*>(vnew + sliced_at(row, v0 + 8 * p8, C));
         }
 #pragma unroll
-        for (int i = 0; i < K / 32; i++) nx_s0[i] = *reinterpret_cast<const bf16x8*>(s0 + sliced_at(t / 8 + 32 * i, v0 + 8 * p8, V));
+        for (int i = 0; i < K / 32; i++) nx_s0[i] = *reinterpret_cast<const bf16x8*>(s0 + sliced_at(t / 8 + 32 * i, v0 + 8 * p8, K));
     };
     // rows of q and k (keys KW kh ..) into registers, and from there, scaled, row-major into sQ and sK (TR only)
     auto ask_qk = [&](int kh) {
@@ -337,7 +337,7 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
                 bf16x8 dr = *reinterpret_cast<const bf16x8*>(row_of(p.d_raw, p.d_stride_b, p.d_stride_t, p.d_stride_h, row) + v0 + 8 * p8);
                 if (!live) vr = zero8, dr = zero8;
                 const bf16_t* yrow;
-                if constexpr (SL) yrow = p.y_chunks + chunk * C * V + sliced_at(C - 1 - row, v0 + 8 * p8, V);
+                if constexpr (SL) yrow = p.y_chunks + chunk * C * V + sliced_at(C - 1 - row, v0 + 8 * p8, C);
                 else yrow = p.y_mirror != nullptr ? p.y_mirror + ((mirA + (C - 1 - row)) * p.H + h) * V + v0 + 8 * p8
                                                   : p.y_chunks + (chunk * C + (C - 1 - row)) * V + v0 + 8 * p8;
                 const bf16x8 yr = *reinterpret_cast<const bf16x8*>(yrow);
@@ -359,7 +359,7 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
 #pragma unroll
                 for (int it = 0; it < 2; it++) {  // rows of V~ past the end of the sequence hold whatever the scan left
                     const int row = t / 8 + 32 * it;
-                    const bf16x8 x = *reinterpret_cast<const bf16x8*>(SL ? vnew + sliced_at(row, v0 + 8 * p8, V)
+                    const bf16x8 x = *reinterpret_cast<const bf16x8*>(SL ? vnew + sliced_at(row, v0 + 8 * p8, C)
                                                                                 : vnew + row * V + v0 + 8 * p8);
                     *reinterpret_cast<bf16x8*>(sVN + row * LDS64 + 8 * p8) = row < valid ? x : zero8;
                 }
@@ -368,7 +368,7 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
                 for (int i = 0; i < K / 32; i++) {  // S0[:, v0 .. v0 + 63]: row = 32 i + t / 8
                     const int row = t / 8 + 32 * i;
                     *reinterpret_cast<bf16x8*>(sST + row * LDS64 + 8 * p8) =
-                        *reinterpret_cast<const bf16x8*>(SL ? s0 + sliced_at(row, v0 + 8 * p8, V) : s0 + row * V + v0 + 8 * p8);
+                        *reinterpret_cast<const bf16x8*>(SL ? s0 + sliced_at(row, v0 + 8 * p8, K) : s0 + row * V + v0 + 8 * p8);
                 }
             } else {
                 const float* vnew = reinterpret_cast<const float*>(vnb);
@@ -406,7 +406,7 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
 #pragma unroll
                 for (int i = 0; i < K / 32; i++) {
                     const int row = t / 8 + 32 * i, c8 = 8 * (t % 8);
-                    ds1_half[i] = *reinterpret_cast<const bf16x8*>(SL ? ds1h + sliced_at(row, v0 + c8, V) : ds1h + row * V + v0 + c8);
+                    ds1_half[i] = *reinterpret_cast<const bf16x8*>(SL ? ds1h + sliced_at(row, v0 + c8, K) : ds1h + row * V + v0 + c8);
                 }
             } else {
 #pragma unroll

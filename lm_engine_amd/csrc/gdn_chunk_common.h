@@ -37,7 +37,7 @@ struct ChunkParams {
     // the caller's sequence backwards, every chunk twice - chunk 2 r takes its rows of k from k and of v from v, chunk
     // 2 r + 1 from k2 and v2, both as tokens 64 (NT / 2 - 1 - r) + 63 - row of those tensors ([N, T / 2, H, .]).
     int mirror;
-    int save_sliced;  // bf16 staged saves: [entry][rows / 8][V / 32 slices][8 rows][32] instead of [entry][rows][V]
+    int save_sliced;  // bf16 staged saves: [entry][V / 32 slices][rows][32] instead of [entry][rows][V]
     const bf16_t* k2;
     const bf16_t* v2;
     int64_t k2_stride_b, k2_stride_t, k2_stride_h;

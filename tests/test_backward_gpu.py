@@ -409,15 +409,15 @@ def test_mirror_reads_equal_the_scan_over_reversed_copies(K, V, B, T, H):
 
 def _unslice(x, rows):
     """[chains, entries, rows, V] array written with ``gdn_chunk_saves.sliced`` -> its [.., rows, V] meaning: memory is
-    [rows / 8][V / 32][8][32] per entry."""
+    [V / 32][rows][32] per entry."""
     ch, nc, r, V = x.shape
     assert r == rows
-    return x.reshape(ch, nc, rows // 8, V // 32, 8, 32).permute(0, 1, 2, 4, 3, 5).reshape(ch, nc, rows, V)
+    return x.reshape(ch, nc, V // 32, rows, 32).permute(0, 1, 3, 2, 4).reshape(ch, nc, rows, V)
 
 
 @pytest.mark.parametrize("K, V, no_output", [(128, 128, False), (128, 256, True), (256, 512, True), (64, 64, False)])
 def test_sliced_saves_hold_the_same_values(K, V, no_output):
-    """bf16 saves in the sliced layout (groups of 8 rows, 32-column slice by slice: whole lines per scan workgroup) against
+    """bf16 saves in the sliced layout (32-column slice by slice: one contiguous block per scan workgroup and chunk) against
     the same saves in rows of V columns: the same values, bit for bit, once the layout is undone."""
     from lm_engine_amd import ops
 
