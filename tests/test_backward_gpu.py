@@ -265,6 +265,20 @@ def test_chunk_local_kernel_matches_the_batched_gemm_version(K, V, saves):
         got = ops.chunk_local_grads(q.cuda(), k.cuda(), v.cuda(), dout.cuda(), prep, y_mirror.cuda(), v_new.cuda(),
                                     s0.cuda(), ds1.cuda(), scale, l2norm)  # fmt: skip
         torch.cuda.synchronize()
+        if saves == bf:
+            # the same call on the sliced layout of the sweeps (all bf16, Y per chunk as the mirror scan saves it: tokens
+            # reversed): the kernel's other template variant - at K = 256 the one that keeps the next slab's loads in
+            # flight - must give the same numbers up to the rounding of dS1 to bf16
+            y_saved = y.flip(2)
+            sliced = ops.chunk_local_grads(q.cuda(), k.cuda(), v.cuda(), dout.cuda(), prep, _slice(y_saved).cuda(),
+                                           _slice(v_new).cuda(), _slice(s0).cuda(), _slice(ds1.to(bf)).cuda(), scale, l2norm,
+                                           sliced=True)  # fmt: skip
+            plain = ops.chunk_local_grads(q.cuda(), k.cuda(), v.cuda(), dout.cuda(), prep, y_saved.cuda(), v_new.cuda(),
+                                          s0.cuda(), ds1.to(bf).cuda(), scale, l2norm)  # fmt: skip
+            torch.cuda.synchronize()
+            for name, a, b in zip(("dq", "dk", "dv", "dg", "dbeta"), sliced, plain):
+                err = rel_l2(a, b)
+                assert err <= 1e-5, f"sliced saves, {name}: rel-L2 {err:.3e} against the same call on rows of V columns"
         qn, kn = pack(q) * pack(rq[..., None]), pack(k) * pack(rk[..., None])
         dqs, dkn, dbeta, dgamma = _chunk_local_grads(qn * scale, kn, pack(v), pack(dout), y.double(), v_new.double(),
                                                      s0.double(), ds1.double(), gam.double(), beta.double())  # fmt: skip
@@ -405,6 +419,13 @@ def test_mirror_reads_equal_the_scan_over_reversed_copies(K, V, B, T, H):
     for name, a, b in zip(("saved states", "saved Y", "final state"), *results):
         assert a.abs().max() > 0, name
         assert torch.equal(a, b), f"{name}: rel-L2 {rel_l2(a.float(), b.float()):.3e}"
+
+
+def _slice(x):
+    """[chains, entries, rows, V] -> the same values in the memory order of ``gdn_chunk_saves.sliced``, [V / 32][rows][32]
+    per entry (shape kept)."""
+    ch, nc, rows, V = x.shape
+    return x.reshape(ch, nc, rows, V // 32, 32).permute(0, 1, 3, 2, 4).contiguous().view(ch, nc, rows, V)
 
 
 def _unslice(x, rows):
