@@ -98,7 +98,9 @@ def parse_args():
     ap.add_argument("--cycle-budget", action="store_true",
                     help="instead of the benchmark: run the headline forward (as two kernels) on the measurement build of the "
                          "library (python -m lm_engine_amd.build --cycle-budget) and print the shader-clock cycles a compute "
-                         "wave of the half-slice scan spends in each group of MFMAs of its chunk loop")
+                         "wave of the half-slice scan spends in each group of MFMAs of its chunk loop, then one backward at the "
+                         "headline shape and one at the shipped head shape and the cycles of the chunk-local backward "
+                         "kernel's steps")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, the known-size kernel the HBM counters are scaled by")
     return ap.parse_args()
@@ -558,6 +560,42 @@ def bench_layer_backward_kernels(w, steps, warmup):
     }  # fmt: skip
 
 
+LOCAL_GROUPS = ("stage_slab", "barrier_a", "row_sums", "ask_ds1", "ask_next_slab", "products_s0", "barrier_b",
+                "stage_ds1", "barrier_c", "products_ds1", "barrier_d", "reduce_dot", "phase2", "phase3", "stores_tail")
+
+
+def cycle_budget_backward_local(w):
+    """The chunk-local backward kernel (``gdn_chunk_bwd_local``) step by step, in shader-clock cycles per chunk: one
+    backward of workload ``w`` on ``libgdn_hip_cycles.so`` (loaded by ``cycle_budget`` before this), whose kernel reads
+    the clock between its steps (wave 0 of 32 workgroups spread over the grid reports).  Phase 1 runs once per slab of 64
+    value columns: its groups are sums over the slabs of a chunk."""
+    import ctypes
+
+    import torch
+
+    from lm_engine_amd import _lib
+    from lm_engine_amd.backward import gated_delta_rule_backward
+    from lm_engine_amd.workloads import make_inputs
+
+    lib = _lib.load_library()
+    inp = make_inputs(w, device="cuda")
+    do = torch.randn(inp["v"].shape, generator=torch.Generator("cpu").manual_seed(555)).to(inp["v"].dtype).cuda()
+    call = lambda: gated_delta_rule_backward(  # noqa: E731
+        inp["q"], inp["k"], inp["v"], inp["g"], inp["beta"], do, None, scale=inp["scale"],
+        initial_state=inp["initial_state"], cu_seqlens=inp["cu_seqlens"])  # fmt: skip
+    device_warmup(call)
+    call()
+    out = (ctypes.c_uint64 * 512)()
+    _lib.check_status(lib.gdn_cycle_budget_read(out, 64), "gdn_cycle_budget_read")
+    rows = [[out[16 * i + j] for j in range(16)] for i in range(32)]
+    rows = [r for r in rows if r[15] > 0]
+    per_chunk = {n: round(sum(r[j] for r in rows) / len(rows), 1) for j, n in enumerate(LOCAL_GROUPS)}
+    return {
+        "workload": w.name, "K": w.K, "V": w.V, "kernel": "chunk_local_grads_kernel, wave 0", "sampled_workgroups": len(rows),
+        "slabs_per_chunk": int(rows[0][15]), "cycles_per_chunk": per_chunk, "cycles_per_chunk_total": round(sum(per_chunk.values()), 1),
+    }  # fmt: skip
+
+
 def bench_backward(w, inp, steps, warmup):
     """One backward pass of the chunked operator on the same workload (``lm_engine_amd.backward``), gradient
     of the output only.  Wall time per call with the device idle before and after."""
@@ -613,6 +651,9 @@ def main():
 
     if args.cycle_budget:
         print(json.dumps({"cycle_budget": cycle_budget(get_workload(args.workload))}))
+        shipped = replace(get_workload(1, B=8, H=2, K=256, V=512), name="shipped_head_shape_k256_v512_bf16")
+        print(json.dumps({"cycle_budget_backward_local": [cycle_budget_backward_local(get_workload(args.workload)),
+                                                          cycle_budget_backward_local(shipped)]}))
         return
     w = get_workload(args.workload)
     result, inp = bench_chunk(w, args.steps, args.warmup, args.two_kernels)

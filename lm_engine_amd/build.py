@@ -47,14 +47,15 @@ def _hipcc() -> str:
 
 
 CYCLE_BUDGET_LIBRARY_PATH = os.path.join(PACKAGE_DIR, "libgdn_hip_cycles.so")
-CYCLE_BUDGET_SOURCES = ("gdn_api.hip", "gdn_chunk.hip", "gdn_chunk32.hip")  # the sources that read GDN_CYCLE_BUDGET
+CYCLE_BUDGET_SOURCES = ("gdn_api.hip", "gdn_chunk.hip", "gdn_chunk32.hip", "gdn_chunk_bwd.hip")  # the sources that read GDN_CYCLE_BUDGET
 
 
 def build_library(verbose: bool = False, extra_flags: tuple[str, ...] = (), cycle_budget: bool = False) -> str:
     """Compiles every source and links the shared library; always rebuilds.
 
     ``cycle_budget``: the measurement build instead, ``libgdn_hip_cycles.so`` - the same library with the shader clock
-    read between the groups of MFMAs of the half-slice scan's chunk loop (``-DGDN_CYCLE_BUDGET``; only the sources that
+    read between the groups of MFMAs of the half-slice scan's chunk loop and between the steps of the chunk-local backward
+    kernel (``-DGDN_CYCLE_BUDGET``; only the sources that
     read the macro are compiled again, the rest is linked from the objects of the library proper, which must exist).
     ``bench.py --cycle-budget`` loads it; nothing else does."""
     hipcc = _hipcc()

@@ -141,9 +141,10 @@ bool chunk_runs_as_one_launch(const gdn_args& a) {
 }
 
 #ifdef GDN_CYCLE_BUDGET
-// Measurement build only: a device buffer the sampled waves of the half-slice scan report into (allocated on first use;
-// this build is not the library proper and is free to), and its read-out.
-static uint64_t* cycle_buffer() {
+// Measurement build only: a device buffer the sampled waves of the half-slice scan (and the sampled workgroups of the
+// chunk-local backward kernel) report into (allocated on first use; this build is not the library proper and is free
+// to), and its read-out.
+uint64_t* cycle_buffer() {
     static uint64_t* buf = nullptr;
     if (buf == nullptr && hipMalloc(&buf, GDN_CYCLE_BUDGET_SLOTS * 8 * sizeof(uint64_t)) != hipSuccess) buf = nullptr;
     return buf;

@@ -46,6 +46,9 @@ constexpr int BWD_THREADS = 256;
 constexpr int LDS64 = 72;  // bf16 per LDS row of a [.][64] matrix: 16 bytes of padding
 
 struct ChunkLocalParams {
+#ifdef GDN_CYCLE_BUDGET
+    uint64_t* cycle_out;  // measurement build only: where sampled workgroups report their cycles
+#endif
     const void* vnew;   // V~ [chunk][64][V], fp32 or bf16 (saves_bf16)
     const void* s0;     // S0 [chunk][K][V], fp32 or bf16 (saves_bf16)
     const void* ds1;    // dS1 [chunk][K][V], fp32 or bf16 (the kernel's DS1H)
@@ -232,6 +235,21 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
         s_fk[t] = p.rk != nullptr ? p.rk[chunk * C + t] : 1.f;
     }
     if (t < 4) s_red[t] = 0.f;
+#ifdef GDN_CYCLE_BUDGET
+    // Measurement build (python -m lm_engine_amd.build --cycle-budget): wave 0 reads the shader clock between the steps
+    // of the kernel and adds the cycles of each up; sampled workgroups report at the end (see LOCAL_GROUPS below).
+    uint64_t cyc[16] = {};
+    uint64_t cyc_t0 = __builtin_readcyclecounter();
+    auto ltick = [&](int g) {
+        const uint64_t t1 = __builtin_readcyclecounter();
+        cyc[g] += t1 - cyc_t0;
+        cyc_t0 = t1;
+        __builtin_amdgcn_sched_barrier(0);
+    };
+#define LTICK(g) ltick(g)
+#else
+#define LTICK(g)
+#endif
 
     // ---------------- phase 1: everything that contracts over the value dim, 64 columns at a time ----------------
     // products with the states, transposed: rows = keys 32 (ktl + NKT kh) .., columns = tokens 32 tt + l32; and the
@@ -386,7 +404,9 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
                 }
             }
         }
+        LTICK(0);
         __syncthreads();
+        LTICK(1);
 #pragma unroll
         for (int it = 0; it < 2; it++) {  // 8 lanes hold one row
             float x = yv[it];
@@ -416,13 +436,16 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
                 }
             }
         };
+        LTICK(2);
         if constexpr (PREFETCH) {
             ask_ds1();  // first: it is waited for first
+            LTICK(3);
             if constexpr (PIPE) {
                 if (hv + 1 < V / VW) ask_slab(v0 + VW);
                 else ask_qk(0);
             }
             __builtin_amdgcn_sched_barrier(0);
+            LTICK(4);
         }
 #pragma unroll
         for (int kh = 0; kh < KH; kh++)
@@ -435,7 +458,9 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
         DP = mma_nt(sDO + 32 * (wave / 2) * LDS64, LDS64, sVN + 32 * (wave % 2) * LDS64, LDS64, VW, DP, l32, lh);
         DA = mma_nt(sY + 32 * (wave / 2) * LDS64, LDS64, sVN + 32 * (wave % 2) * LDS64, LDS64, VW, DA, l32, lh);
         if constexpr (!PREFETCH) ask_ds1();
+        LTICK(5);
         __syncthreads();  // S0 has been read by every wave
+        LTICK(6);
 
         // dS1 takes the place of S0; <dS1, S0> on the way (S0 as the bf16 the products used)
         if constexpr (DS1H) {
@@ -457,17 +482,22 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
                 put4(sST + row * LDS64 + 4 * c4, x);
             }
         }
+        LTICK(7);
         __syncthreads();
+        LTICK(8);
 #pragma unroll
         for (int kh = 0; kh < KH; kh++)
 #pragma unroll
             for (int m = 0; m < NTW; m++)
                 dKdT[kh][m] = mma_nt(sST + 32 * (ktl + NKT * kh) * LDS64, LDS64, sVN + 32 * tt_of(m) * LDS64, LDS64, VW, dKdT[kh][m], l32, lh);
+        LTICK(9);
         __syncthreads();  // the staged slab is free
+        LTICK(10);
     }
     dot = wave_sum(dot);
     if (lane == 0) atomicAdd(&s_red[0], dot);
 
+    LTICK(11);
     // ---------------- phase 2: Q K^T, K K^T and the 64 x 64 stage ----------------
     // wave -> tile (ti, tj); rows i = 32 ti + 8 (r/4) + 4 h + r%4, column j = 32 tj + l32
     {
@@ -548,6 +578,19 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
         }
         atomicAdd(&s_dgam[j], -colsum);
     }
+    LTICK(12);
+    // K <= 128: the transposes of phase 3 take the place of the rows of q and k in LDS; every thread picks its pieces of
+    // the rows up here, before the barrier that ends their use
+    bf16x8 tq[TR ? 1 : KW / 32], tk[TR ? 1 : KW / 32];
+    if constexpr (!TR) {
+        static_assert(TR || KH == 1, "one staging of q and k");
+#pragma unroll
+        for (int it = 0; it < KW / 32; it++) {
+            const int row = t % C, p8 = t / C + 4 * it;
+            tq[it] = *reinterpret_cast<const bf16x8*>(sQ + row * LDK + 8 * p8);
+            tk[it] = *reinterpret_cast<const bf16x8*>(sK + row * LDK + 8 * p8);
+        }
+    }
     // ---------------- phase 3: per-token sums over the key dim, dQ^T and dK^T, 128 keys at a time ----------------
     // (dQ^T and dK^T are built in the registers of dQe^T and dKd^T)
     float nkd = 0.f;
@@ -566,21 +609,16 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
         } else {
             // a wave takes 16 bytes of all 64 rows at a time: its 2-byte writes of one key then cover 64 consecutive
             // tokens of a transposed row (no bank conflicts; the rows themselves come out of the cache)
+            // (the values are the scaled rows that phase 2 staged, taken out of LDS before the barrier above)
             constexpr int CPR = KW / 8;
             const int row = t % C;
-            const float fq = s_fq[row], fk = s_fk[row];
-            const bf16_t* const qrow = row_of(p.q_raw, p.q_stride_b, p.q_stride_t, p.q_stride_h, row) + KW * kh;
-            const bf16_t* const krow = row_of(p.k_raw, p.k_stride_b, p.k_stride_t, p.k_stride_h, row) + KW * kh;
 #pragma unroll
             for (int it = 0; it < CPR / 4; it++) {
                 const int p8 = t / C + 4 * it;
-                bf16x8 qr = *reinterpret_cast<const bf16x8*>(qrow + 8 * p8);
-                bf16x8 kr = *reinterpret_cast<const bf16x8*>(krow + 8 * p8);
-                if (row >= valid) qr = zero8, kr = zero8;
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
-                    sQT[(8 * p8 + e) * LDS64 + row] = (bf16_t)((float)qr[e] * fq);
-                    sKT[(8 * p8 + e) * LDS64 + row] = (bf16_t)((float)kr[e] * fk);
+                    sQT[(8 * p8 + e) * LDS64 + row] = tq[it][e];
+                    sKT[(8 * p8 + e) * LDS64 + row] = tk[it][e];
                 }
             }
             __syncthreads();
@@ -643,6 +681,7 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
             }
         }
     }
+    LTICK(13);
     nkd = wave_sum(nkd);
     if (lane == 0) atomicAdd(&s_red[1], nkd);
     __syncthreads();
@@ -688,6 +727,18 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
             p.dbeta_out[(tok0 + t) * p.H + h] = s_dbeta[t];
         }
     }
+#ifdef GDN_CYCLE_BUDGET
+    LTICK(14);
+    // 32 workgroups spread over the grid report: [slot][15 groups | slabs]
+    const int stride = max((int)gridDim.x / GDN_LOCAL_CYCLE_SLOTS, 1);
+    if (p.cycle_out != nullptr && t == 0 && blockIdx.x % stride == 0 && blockIdx.x / stride < GDN_LOCAL_CYCLE_SLOTS) {
+        uint64_t* out = p.cycle_out + (blockIdx.x / stride) * 16;
+#pragma unroll
+        for (int i = 0; i < 15; i++) out[i] = cyc[i];
+        out[15] = (uint64_t)(V / VW);
+    }
+#endif
+#undef LTICK
 }
 
 
@@ -1150,6 +1201,10 @@ static bool bwd_shape_built(int K, int V) { return (K == 64 || K == 128 || K == 
 
 int launch_chunk_bwd_local(const gdn_chunk_local_args& a, hipStream_t stream) {
     ChunkLocalParams p;
+#ifdef GDN_CYCLE_BUDGET
+    p.cycle_out = cycle_buffer();
+    if (p.cycle_out != nullptr) (void)hipMemsetAsync(p.cycle_out, 0, GDN_LOCAL_CYCLE_SLOTS * 16 * sizeof(uint64_t), stream);
+#endif
     p.vnew = a.v_new, p.s0 = a.states, p.ds1 = a.dstates, p.saves_bf16 = a.saves_dtype == GDN_BF16 ? 1 : 0;
     const bool h = a.dstates_dtype == GDN_BF16;
     const bool sl = a.saves_sliced != 0;

@@ -7,6 +7,7 @@ namespace gdn {
 
 constexpr int C = 64;  // chunk length
 constexpr int GDN_CYCLE_BUDGET_SLOTS = 64;  // sampled workgroups of the measurement build
+constexpr int GDN_LOCAL_CYCLE_SLOTS = 32;   // of them the chunk-local backward kernel uses two each (16 counters per workgroup)
 constexpr int PREP_THREADS = 256;
 constexpr int FRAG_BYTES = WAVE * 16;  // one MFMA operand fragment: 8 bf16 per lane
 

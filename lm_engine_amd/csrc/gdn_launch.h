@@ -38,5 +38,8 @@ int launch_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args& a, hipStream_t st
 bool chunk_bwd_prepare_supported(const gdn_chunk_bwd_prepare_args& a);
 uint64_t chunk_bwd_record_bytes(const gdn_chunk_bwd_prepare_args& a);
 int launch_conv_bwd(const gdn_conv_bwd_args& a, hipStream_t stream);  // gdn_conv1d_bwd.hip
+#ifdef GDN_CYCLE_BUDGET
+uint64_t* cycle_buffer();  // gdn_chunk.hip, measurement build only: the device buffer sampled waves report their cycles into
+#endif
 
 }  // namespace gdn
