@@ -291,6 +291,8 @@ int gdn_causal_conv1d_bwd(const gdn_conv_bwd_args* a, void* stream) {
 // Measurement build only (not declared in gdn_hip.h, not part of libgdn_hip.so): after a chunked forward that ran the
 // half-slice scan, the cycles wave 0 of every 16th scan workgroup spent in each group of its chunk loop, summed over its
 // chunks: out[slot * 8 + 0..5] = K S0 | S0^T q^T | T' X | k^T V~ | V~^T P^T | between chunks, out[slot * 8 + 6] = chunks.
+// After a gdn_chunk_bwd_local call the same buffer holds that kernel's report instead (read it with slots = 64): 32 sampled
+// workgroups, out[w * 16 + 0..14] = the cycles of the kernel's steps (bench.py's LOCAL_GROUPS), out[w * 16 + 15] = slabs per chunk.
 int gdn_cycle_budget_read(uint64_t* out, int slots) { return gdn::cycle_budget_read(out, slots); }
 #endif
 
