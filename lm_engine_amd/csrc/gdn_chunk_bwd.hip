@@ -29,7 +29,11 @@
 //      with the states and the two 64 x 64 products that contract over the value dim accumulate;
 //   2. the rows of q and k (128 keys at a time) for Q K^T and K K^T, then the 64 x 64 stage: G, G^T and Hm + Hm^T
 //      are left in LDS;
-//   3. per 128 keys: the transposes of q and k staged, the per-token sums over the key dim, dQ^T and dK^T.
+//   3. per 128 keys: the transposes of q and k (K <= 128: staged from the rows phase 2 left in LDS; K = 256: read out
+//      of those rows with the transposing LDS load), the per-token sums over the key dim, dQ^T and dK^T.
+// K = 256 on the sliced saves of the staging scans has one wave per SIMD and so 512 registers per lane: it asks for the
+// rows of the next slab, and of the next half of q and k, while the products of the current one run, and keeps them
+// in registers until their turn (PIPE below).
 // K = 64, 128, 256; V a multiple of 64.
 #include <hip/hip_runtime.h>
 
@@ -237,7 +241,7 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 128 ? 2 : 1)) void chunk_local_g
     if (t < 4) s_red[t] = 0.f;
 #ifdef GDN_CYCLE_BUDGET
     // Measurement build (python -m lm_engine_amd.build --cycle-budget): wave 0 reads the shader clock between the steps
-    // of the kernel and adds the cycles of each up; sampled workgroups report at the end (see LOCAL_GROUPS below).
+    // of the kernel and adds the cycles of each up; sampled workgroups report at the end (the steps are named in bench.py's LOCAL_GROUPS).
     uint64_t cyc[16] = {};
     uint64_t cyc_t0 = __builtin_readcyclecounter();
     auto ltick = [&](int g) {
