@@ -55,6 +55,10 @@ enum {
                                    nothing else, by calls of one shape on one stream, keeps the promise by itself. */
     GDN_FLAG_RECORDS_16X16 = 32, /* gdn_chunk_bwd_prepare: write the operand fragments of the mirror problem's records in
                                    the lane order of the 16x16x32 MFMA, for gdn_chunk_fwd_saving with records_given = 2 */
+    GDN_FLAG_SKIP_EMPTY_CHUNKS = 128, /* gdn_chunk_bwd_prepare with seq_start / seq_len: chunk slots past the end of their
+                                       * sequence (other than a sequence's first slot) get no records and no rows of the
+                                       * mirror problem - for a mirror scan that walks every row over its own length
+                                       * (gdn_chunk_fwd_saving with records_given on a left-padded batch) */
     GDN_FLAG_DEBUG_NO_PRODUCERS = 64, /* test aid for the one-launch forward: its prepare workgroups return at once, so that
                                    the scan's bounded wait runs out (with a small args->spin_limit) and the error path can be
                                    exercised while every kernel still ends normally; outputs are invalid */
@@ -215,7 +219,13 @@ int gdn_recurrent_fwd(const gdn_args *args, void *stream);
  * out by 32-column slice, [N * H][chunks_per_chain][V / 32][K or 64][32]: what one scan workgroup saves of a chunk is
  * then one contiguous block (whole 128-byte lines from one CU instead of 64-byte halves of lines from several), which
  * gdn_chunk_bwd_local reads with saves_sliced.
- * T / 64 must be even.  The twelve operand fragments of every odd chunk are read from the record of chunk 1 of the chain
+ * records_given with a left-padded batch (GDN_FLAG_LEFT_PADDED, args->cu_seqlens the prefix sums of the rows' valid lengths,
+ * which must be multiples of 64; not with mirror_reads): row n is scanned over its last tokens only, its records lie at
+ * the slots of those tokens (the last ones of the row), and with save_reverse the row's last saved chunk goes to entry 0
+ * of ITS entries whatever the row's length.  row_order (then only; NULL = as they lie): the rows in the order in which
+ * their chains are dealt out to the XCDs and started, best longest first - a ragged batch takes as long as the XCD with
+ * the most chunks.
+ * mirror_reads: T / 64 must be even.  The twelve operand fragments of every odd chunk are read from the record of chunk 1 of the chain
  * (in the mirror problem they are the same for all odd chunks: T' = I, P = 0); an odd chunk's own record supplies its
  * row scales and e^{gamma_C} only.
  */
@@ -235,6 +245,7 @@ typedef struct gdn_chunk_saves {
     const void *k_odd, *v_odd;
     int64_t k_odd_stride_b, k_odd_stride_t, k_odd_stride_h;
     int64_t v_odd_stride_b, v_odd_stride_t, v_odd_stride_h;
+    const int32_t *row_order; /* [N] or NULL */
 } gdn_chunk_saves;
 int gdn_chunk_fwd_saving(const gdn_args *args, const gdn_chunk_saves *saves, void *stream);
 /* 1 when gdn_chunk_fwd_saving would run these arguments (shape fields, flags, cu_seqlens NULL or not; every field of
@@ -309,7 +320,7 @@ int gdn_chunk_bwd_local(const gdn_chunk_local_args *args, void *stream);
  *     odd chunks' records only chunk 1 of every chain then carries its operand fragments, the others their scales.
  *     The scan's output at the even chunks is Y = T^T dV~ (reversed), the states it saves there are the
  *     gradients of the chunks' final states, its final state is the gradient of the initial state.
- * flags: GDN_FLAG_L2NORM only.  g (fp32 [N, T, H]) and beta ([N, T, H], beta_dtype) may be NULL (0 and 1).
+ * flags: GDN_FLAG_L2NORM, GDN_FLAG_RECORDS_16X16, GDN_FLAG_SKIP_EMPTY_CHUNKS.  g (fp32 [N, T, H]) and beta ([N, T, H], beta_dtype) may be NULL (0 and 1).
  */
 typedef struct gdn_chunk_bwd_prepare_args {
     const void *q, *k, *dout;

@@ -22,6 +22,7 @@ GDN_FLAG_FUSED_LAUNCH = 8
 GDN_FLAG_READY_FLAGS_CLEAR = 16
 GDN_FLAG_RECORDS_16X16 = 32
 GDN_FLAG_DEBUG_NO_PRODUCERS = 64
+GDN_FLAG_SKIP_EMPTY_CHUNKS = 128
 
 GDN_ERR_TIMEOUT = -7
 
@@ -81,6 +82,7 @@ class GdnChunkSaves(ctypes.Structure):
         ("v_odd_stride_b", ctypes.c_int64),
         ("v_odd_stride_t", ctypes.c_int64),
         ("v_odd_stride_h", ctypes.c_int64),
+        ("row_order", ctypes.c_void_p),
     ]
 
 

@@ -357,7 +357,11 @@ def _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, l2norm
         sequences = (as_i32(starts), as_i32(lens), NC)
     Bt = N * H
     q, k, v, do = (x if x.stride(-1) == 1 else x.contiguous() for x in (q, k, v, do.to(torch.bfloat16)))
-    half_slices = K > 128 or ops.half_slice_records_pay(Bt, V, dev)  # K = 256 scans on half-slice waves only
+    # The sweeps run on the half-slice scan, one 32-column slice per workgroup, whatever the number of chains: it is the
+    # variant that stages its saves through LDS (bf16, whole lines) and scans without output, which outweighs the records
+    # that four slices per workgroup would share (measured with 2 to 6 workgroups per CU: 1.35 against 2.17 ms at twice
+    # configuration 1's batch, 3.17 against 4.29 ms at B = 12, V = 256).
+    half_slices = True
     # Where the mirror scan stages its saves through LDS, Y and the gradients of the chunks' final states leave as bf16
     # (the chunk-local products round them to that anyway; their part in dg, <dS1, S0>, moved by less than its third
     # digit in every test), and where it is the scan without output it reads the caller's q, k and dO backwards itself
@@ -367,7 +371,8 @@ def _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, l2norm
     mirror_reads = staged_m and K >= 128 and sequences is None
     # a batch of whole chunks gets the forward sweep's records from the same kernel: no prepare launch of its own
     prep = ops.chunk_bwd_prepare(q, k, do, g, beta, scale, l2norm, V, sequences, half_slice_records=half_slices,
-                                 forward_records=sequences is None, reversed_copies=not mirror_reads)  # fmt: skip
+                                 forward_records=sequences is None, reversed_copies=not mirror_reads,
+                                 skip_empty_chunks=True)  # fmt: skip
     # Where the saving scan stages its saves through LDS, the sweeps write S0, V~ and Y as bf16 (what the chunk-local
     # products round them to anyway) and form no output; elsewhere fp32 saves and Y from the mirror scan's output.
     given = 0 if sequences is not None else 2 if half_slices else 1
@@ -387,10 +392,14 @@ def _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, l2norm
     dht32 = None if dht is None else dht.to(torch.float32).contiguous()
     dS1 = torch.empty(Bt, NC, K, V, device=dev, dtype=torch.bfloat16 if staged_m else torch.float32)
     Y = torch.empty(Bt, NC, CHUNK, V, dtype=torch.bfloat16, device=dev) if staged_m else None
+    # (ragged batches: a row of the mirror problem is scanned over the two chunks per chunk of ITS sequence, which lie at
+    # the row's end, not over those of the longest one)
+    mirror_lengths = None if sequences is None else [2 * CHUNK * max(1, -(-length // CHUNK)) for length in lens]
     o_m, dS = ops.chunk_scan_given_records(k if mirror_reads else prep["k_mirror"], prep["v_mirror"], prep["records"],
                                            dht32, dS1, NC, save_every=2, save_reverse=True,
                                            half_slice_records=half_slices, v_new=Y, no_output=staged_m,
-                                           mirror_odd=(q, do) if mirror_reads else None, sliced=sliced)  # fmt: skip
+                                           mirror_odd=(q, do) if mirror_reads else None, sliced=sliced,
+                                           valid_lengths=mirror_lengths)  # fmt: skip
     dq, dk, dv, dg, dbeta = ops.chunk_local_grads(q, k, v, do, prep, Y if staged_m else o_m, Vn, S0, dS1, scale, l2norm,
                                                   sequences, sliced=sliced)  # fmt: skip
     return (

@@ -188,7 +188,9 @@ int gdn_chunk_fwd_saving(const gdn_args* a, const gdn_chunk_saves* saves, void* 
     if (saves->records_given < 0 || saves->records_given > 2) return GDN_ERR_SHAPE;
     if (saves->records_given == 1 && a->K > 128) return GDN_ERR_UNSUPPORTED;  // K = 256 scans on half-slice waves only
     if (saves->records_given) {
-        if (a->cu_seqlens != nullptr) return GDN_ERR_VARLEN;  // records are given for fixed-length batches only
+        // records are given for batches of rows: fixed-length, or left-padded with whole chunks per row
+        if (a->cu_seqlens != nullptr && (!(a->flags & GDN_FLAG_LEFT_PADDED) || saves->mirror_reads)) return GDN_ERR_VARLEN;
+        if (saves->row_order != nullptr && !aligned(saves->row_order, 4)) return GDN_ERR_ALIGN;
         need = gdn::chunk_record_bytes(*a);
     }
     if (a->workspace == nullptr || a->workspace_bytes < need || !aligned(a->workspace, 256)) return GDN_ERR_WORKSPACE;

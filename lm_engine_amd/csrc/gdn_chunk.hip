@@ -187,6 +187,7 @@ int launch_chunk_fwd(const gdn_args& a, hipStream_t stream, hipEvent_t* events, 
     p.save_state = nullptr, p.save_vnew = nullptr, p.save_nc = 0, p.records_given = 0, p.save_every = 1, p.save_reverse = 0;
     p.save_state_bf16 = 0, p.save_vnew_bf16 = 0, p.no_output = 0;
     p.mirror = 0, p.k2 = nullptr, p.v2 = nullptr;
+    p.row_order = saves != nullptr && saves->records_given && left_padded ? saves->row_order : nullptr;
     p.save_sliced = saves != nullptr && saves->sliced ? 1 : 0;
     p.k2_stride_b = p.k2_stride_t = p.k2_stride_h = p.v2_stride_b = p.v2_stride_t = p.v2_stride_h = 0;
     if (saves != nullptr && saves->mirror_reads) {

@@ -420,10 +420,13 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
     // staging buffer of the state chunk c starts from / of its V~ (narrow fp32 states: a single buffer, see above)
     auto sstage_of = [&](int c) -> uint8_t* { return sstage_raw + ((LSAVE_NARROW && !p.save_state_bf16) ? 0 : (c & 1) * SSTAGE_HALF); };
     auto vstage_of = [&](int c) -> uint8_t* { return vstage_raw + (c & 1) * VSTAGE_HALF; };
-    // entry of the save arrays that chunk c goes to, or -1
+    // entry of the save arrays that chunk c goes to, or -1; with save_reverse the chain's last saved chunk goes to entry 0
+    // (save_last: the entry of its first one - save_nc - 1 unless the chain is a shorter row of a left-padded batch of
+    // given records, set below)
+    int save_last = p.save_nc - 1;
     auto save_entry = [&](int c) -> int {
         if (c % p.save_every != 0 || c / p.save_every >= p.save_nc) return -1;
-        return p.save_reverse ? p.save_nc - 1 - c / p.save_every : c / p.save_every;
+        return p.save_reverse ? save_last - c / p.save_every : c / p.save_every;
     };
 
     const int lane = threadIdx.x % WAVE;
@@ -437,7 +440,8 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
     const int vgroup = rest % p.scan_groups;
     const int per_xcd = (p.N * p.H + 7) / 8;
     int n, h;
-    if (p.cu_seqlens == nullptr) {
+    const int32_t* const order = p.cu_seqlens != nullptr ? p.seq_order : p.row_order;  // (row_order: left-padded rows of given records)
+    if (order == nullptr) {
         // XCD x takes the chains x * per_xcd .. : consecutive chains are different heads
         const int chain = xcd * per_xcd + rest / p.scan_groups;
         if (rest / p.scan_groups >= per_xcd || chain >= p.N * p.H) return;  // whole workgroup
@@ -450,7 +454,7 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
         const int i = rest / p.scan_groups;
         const int rank = 8 * i + ((xcd - i) % 8 + 8) % 8;
         if (i >= per_xcd || rank >= p.N * p.H) return;  // whole workgroup
-        n = p.seq_order[rank / p.H], h = rank % p.H;
+        n = order[rank / p.H], h = rank % p.H;
     }
     const int chain = n * p.H + h;
 
@@ -467,7 +471,11 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
         b = 0, seq_t0 = t0, seq_len = min(len, (slot_end - slot_begin) * C);
     }
     const int nchunks = slot_end - slot_begin;
-    const uint8_t* rec = p.rec + ((int64_t)h * p.TC + slot_begin) * p.rec_bytes;
+    // Given records of a left-padded batch lie at the slots of the tokens they cover, the last ones of the row; and a
+    // reverse save counts from the row's own last chunk.
+    const bool padded_given = p.records_given && p.pad_lens != nullptr;
+    if (padded_given) save_last = min(p.save_nc, (nchunks + p.save_every - 1) / p.save_every) - 1;
+    const uint8_t* rec = p.rec + ((int64_t)h * p.TC + slot_begin + (padded_given ? p.NT - nchunks : 0)) * p.rec_bytes;
 
     // output staging: [compute wave][chunk parity][64 tokens][64 bytes], the four 16-byte pieces of a row
     // XOR-swizzled with (row / 4) % 4 so that both sides access it without bank conflicts
@@ -896,7 +904,7 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
                         }
                     }
                 } else if (p.save_state != nullptr && c % p.save_every == 0 && c / p.save_every < p.save_nc) {
-                    const int entry = p.save_reverse ? p.save_nc - 1 - c / p.save_every : c / p.save_every;
+                    const int entry = p.save_reverse ? save_last - c / p.save_every : c / p.save_every;
                     char* base = reinterpret_cast<char*>(p.save_state + ((int64_t)chain * p.save_nc + entry) * K * p.V);
                     const uint32_t lane_off = (uint32_t)((8 * g) * p.V + c0 + j16) * 4u;
                     const uint32_t row_bytes = (uint32_t)p.V * 4u;
@@ -1039,7 +1047,7 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
                         }
                     }
                 } else if (p.save_vnew != nullptr && c % p.save_every == 0 && c / p.save_every < p.save_nc) {
-                    const int entry = p.save_reverse ? p.save_nc - 1 - c / p.save_every : c / p.save_every;
+                    const int entry = p.save_reverse ? save_last - c / p.save_every : c / p.save_every;
                     char* base = reinterpret_cast<char*>(p.save_vnew + ((int64_t)chain * p.save_nc + entry) * C * p.V);
                     const uint32_t lane_off = (uint32_t)((4 * g) * p.V + c0 + j16) * 4u;
                     const uint32_t row_bytes = (uint32_t)p.V * 4u;
@@ -1160,7 +1168,7 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
             // (one wave-uniform base per store plus one per-lane byte offset: 64-bit per-lane addresses for
             // all of them would not fit the register file)
             if (p.save_state != nullptr && c % p.save_every == 0 && c / p.save_every < p.save_nc) {
-                const int entry = p.save_reverse ? p.save_nc - 1 - c / p.save_every : c / p.save_every;
+                const int entry = p.save_reverse ? save_last - c / p.save_every : c / p.save_every;
                 char* base = reinterpret_cast<char*>(p.save_state + ((int64_t)chain * p.save_nc + entry) * K * p.V);
                 const uint32_t lane_off = (uint32_t)((8 * lh) * p.V + 32 * tn + slice_col(l32)) * 4u;
                 const uint32_t row_bytes = (uint32_t)p.V * 4u;
@@ -1299,7 +1307,7 @@ __global__ __launch_bounds__(scan_waves(NW, HALF) * WAVE) void chunk_scan32_kern
         if constexpr (SAVE) {
             // V~ of this chunk: tile tt, register r holds token 32 tt + 8 (r/4) + 4 h + r%4 of this lane's column
             if (p.save_vnew != nullptr && c % p.save_every == 0 && c / p.save_every < p.save_nc) {
-                const int entry = p.save_reverse ? p.save_nc - 1 - c / p.save_every : c / p.save_every;
+                const int entry = p.save_reverse ? save_last - c / p.save_every : c / p.save_every;
                 char* base = reinterpret_cast<char*>(p.save_vnew + ((int64_t)chain * p.save_nc + entry) * C * p.V);
                 const uint32_t lane_off = (uint32_t)((4 * lh) * p.V + 32 * tn + slice_col(l32)) * 4u;
                 const uint32_t row_bytes = (uint32_t)p.V * 4u;

@@ -775,6 +775,7 @@ struct BwdPrepareParams {
     int N, H, NC, V;
     int l2norm;
     int rec16;  // fragments of the records in the lane order of the 16x16x32 MFMA (GDN_FLAG_RECORDS_16X16)
+    int skip_empty;  // chunk slots past the end of a sequence get nothing (GDN_FLAG_SKIP_EMPTY_CHUNKS)
     float scale;
     float* gam;
     float* bc;
@@ -928,6 +929,9 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 64 ? 3 : 2)) void chunk_bwd_prep
         valid = min(max(p.seq_len[n] - ci * C, 0), C);
         tok0 = (int64_t)p.seq_start[n] + (int64_t)ci * C;
     }
+    // (GDN_FLAG_SKIP_EMPTY_CHUNKS: the mirror scan walks every row over its own chunks and never comes here; an empty
+    // sequence keeps its first slot, which that scan does walk)
+    if (valid == 0 && p.skip_empty && ci > 0) return;  // whole workgroup
     // (a chunk lies within one row of the batch; rows past the end of the sequence read its last token and are zeroed)
     const int64_t row_b = tok0 / p.T_rows, row_t = tok0 % p.T_rows;
     auto row_of = [&](const bf16_t* base, int64_t sb, int64_t st, int64_t sh, int row) -> const bf16_t* {
@@ -1263,6 +1267,7 @@ int launch_chunk_bwd_prepare(const gdn_chunk_bwd_prepare_args& a, hipStream_t st
     p.seq_start = a.seq_start, p.seq_len = a.seq_len, p.T_rows = a.T;
     p.l2norm = (a.flags & GDN_FLAG_L2NORM) ? 1 : 0;
     p.rec16 = (a.flags & GDN_FLAG_RECORDS_16X16) ? 1 : 0;
+    p.skip_empty = (a.flags & GDN_FLAG_SKIP_EMPTY_CHUNKS) ? 1 : 0;
     p.scale = a.scale;
     p.gam = a.gamma, p.bc = a.beta_packed;
     p.rq = a.rq, p.rk = a.rk;

@@ -57,6 +57,7 @@ struct ChunkParams {
     int save_nc;
     int save_every;    // only chunks c with c % save_every == 0 are saved, as entry c / save_every ...
     int save_reverse;  // ... or, when set, as entry save_nc - 1 - c / save_every
+    const int32_t* row_order;  // left-padded rows of given records: the order in which the rows' chains are dealt out (or NULL)
     int save_state_bf16, save_vnew_bf16;  // that array is bf16 (the pointer then points at bf16 data); staged saves only
     int no_output;     // the scan writes no output (a sweep of the backward pass); staged saves only
     int records_given;  // the records are already in place: prepare is not run

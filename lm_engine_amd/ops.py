@@ -378,7 +378,8 @@ def half_slice_records_pay(chains: int, V: int, device) -> bool:
 
 
 def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_chain, save_every=1, save_reverse=False,
-                             half_slice_records=False, v_new=None, no_output=False, q=None, mirror_odd=None, sliced=False):
+                             half_slice_records=False, v_new=None, no_output=False, q=None, mirror_odd=None, sliced=False,
+                             valid_lengths=None):
     """The scan kernel alone over a fixed-length batch whose chunk records the caller has written
     (``records`` uint8 ``[H, B * T / 64, record bytes]``, T a multiple of 64); it reads the rows of ``q``, ``k`` and
     ``v`` (without ``q``, ``k`` stands in its place: the records of a mirror problem carry zero row scales for q).  Returns ``(o, final_state)``
@@ -393,11 +394,24 @@ def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_ch
     and ``v``, the odd chunks' from ``k_odd`` and ``v_odd`` (``gdn_chunk_saves.mirror_reads``): the mirror problem of
     ``chunk_bwd_prepare(..., reversed_copies=False)``.  ``sliced`` (bf16 saves where ``saving_scan_is_staged``): the
     save arrays are laid out by 32-column slice, ``[B H, chunks_per_chain, V / 32, K or 64, 32]`` in the memory of the
-    arrays given (``gdn_chunk_saves.sliced``), for ``chunk_local_grads(..., sliced=True)``."""
+    arrays given (``gdn_chunk_saves.sliced``), for ``chunk_local_grads(..., sliced=True)``.
+    ``valid_lengths`` (``B`` host integers, multiples of 64; not with ``mirror_odd``): the rows are left-padded - row ``n`` is
+    scanned over its last ``valid_lengths[n]`` tokens only, with the records at the slots of those tokens, and a reverse
+    save counts a row's entries from its own last saved chunk (entry 0)."""
     _require_hip_path()
     lib = _lib.load_library()
     q = k if q is None else q
-    dims = _check_inputs(q, k, v, None, None, initial_state, None)
+    pad_lens = None
+    if valid_lengths is not None:
+        if mirror_odd is not None:
+            raise ValueError("valid_lengths and mirror_odd exclude each other")
+        sums = [0]
+        for length in valid_lengths:
+            sums.append(sums[-1] + int(length))
+        pad_lens = torch.tensor(sums, dtype=torch.int32, device=k.device)
+        longest_first = sorted(range(len(valid_lengths)), key=lambda n: (-int(valid_lengths[n]), n))
+        row_order = torch.tensor(longest_first, dtype=torch.int32, device=k.device)
+    dims = _check_inputs(q, k, v, None, None, initial_state, pad_lens, pad_lens is not None)
     B, T, H, K, V, N = dims
     q, k, v = _last_dim_contiguous(q), _last_dim_contiguous(k), _last_dim_contiguous(v)
     if mirror_odd is not None:
@@ -412,12 +426,14 @@ def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_ch
     v_new_code = _lib.GDN_F32 if v_new is None else _save_dtype_code(v_new, (B * H, chunks_per_chain, 64, V), "v_new")
     o = torch.empty(B, T, H, V, dtype=v.dtype, device=v.device)
     ht = torch.empty(N, H, K, V, dtype=torch.float32, device=v.device)
-    args = _fill_args(q, k, v, None, None, initial_state, ht, o, None, 1.0, False, False, dims)
+    args = _fill_args(q, k, v, None, None, initial_state, ht, o, pad_lens, 1.0, False, False, dims, pad_lens is not None)
     args.workspace, args.workspace_bytes = records.data_ptr(), records.numel()
     saves = _lib.GdnChunkSaves(states.data_ptr(), None if v_new is None else v_new.data_ptr(), chunks_per_chain,
                                2 if half_slice_records else 1, save_every, 1 if save_reverse else 0, states_code,
                                v_new_code, 1 if no_output else 0, 0)  # fmt: skip
     saves.sliced = 1 if sliced else 0
+    if pad_lens is not None:
+        saves.row_order = row_order.data_ptr()
     if mirror_odd is not None:
         saves.mirror_reads, saves.k_odd, saves.v_odd = 1, k_odd.data_ptr(), v_odd.data_ptr()
         saves.k_odd_stride_b, saves.k_odd_stride_t, saves.k_odd_stride_h = k_odd.stride(0), k_odd.stride(1), k_odd.stride(2)
@@ -503,7 +519,7 @@ RECORD_BYTES = 13312  # a chunk record: 12 operand fragments, 3 x 64 row scales,
 
 
 def chunk_bwd_prepare(q, k, dout, g, beta, scale, l2norm, V, sequences=None, half_slice_records=False,
-                      forward_records=False, reversed_copies=True):
+                      forward_records=False, reversed_copies=True, skip_empty_chunks=False):
     """``gdn_chunk_bwd_prepare``.  ``q, k, dout`` are the caller's bf16 ``[B, T, H, D]`` tensors; without
     ``sequences`` every row is one sequence of whole chunks, else ``sequences = (seq_start, seq_len, NC)``: int32
     device tensors ``[N]`` (first token as a flat index over the rows, length) and the chunks per sequence to lay
@@ -514,7 +530,9 @@ def chunk_bwd_prepare(q, k, dout, g, beta, scale, l2norm, V, sequences=None, hal
     (whole-chunk batches only): also ``records_fwd`` ``[H, N * NC, RECORD_BYTES]``, the records of the forward pass
     itself in the same fragment order, for a forward sweep without a prepare launch of its own.  Without
     ``reversed_copies`` (whole-chunk batches only) ``k_mirror`` is None and ``v_mirror`` is ``[N, T, H, V]``: P^T dO in
-    the caller's token order, for a scan with ``mirror_odd`` that reads the caller's q, k and dout backwards itself."""
+    the caller's token order, for a scan with ``mirror_odd`` that reads the caller's q, k and dout backwards itself.
+    ``skip_empty_chunks`` (with ``sequences``): chunk slots past the end of their sequence get no records and no mirror
+    rows (``GDN_FLAG_SKIP_EMPTY_CHUNKS``), for a mirror scan with ``valid_lengths``."""
     _require_hip_path()
     lib = _lib.load_library()
     B, T, H, K = q.shape
@@ -551,7 +569,8 @@ def chunk_bwd_prepare(q, k, dout, g, beta, scale, l2norm, V, sequences=None, hal
         setattr(a, f"{name}_stride_h", x.stride(2))
     a.N, a.T, a.H, a.K, a.V = N, T, H, K, V
     a.beta_dtype = _lib.GDN_F32 if beta is None else _dtype_code(beta.dtype, "beta")
-    a.flags = (_lib.GDN_FLAG_L2NORM if l2norm else 0) | (_lib.GDN_FLAG_RECORDS_16X16 if half_slice_records else 0)
+    a.flags = ((_lib.GDN_FLAG_L2NORM if l2norm else 0) | (_lib.GDN_FLAG_RECORDS_16X16 if half_slice_records else 0)
+               | (_lib.GDN_FLAG_SKIP_EMPTY_CHUNKS if skip_empty_chunks and sequences is not None else 0))
     a.scale = float(scale)
     a.gamma, a.beta_packed, a.rq, a.rk = (out[n].data_ptr() for n in ("gamma", "beta", "rq", "rk"))
     a.k_mirror = out["k_mirror"].data_ptr() if reversed_copies else None
