@@ -623,8 +623,12 @@ def bench_backward(w, inp, steps, warmup):
         "workload": w.name,
         "steps": steps,
         "ms_per_backward": round(ms, 3),
-        "tokens_per_s": round(w.B * w.T / (ms * 1e-3), 1),
-        "composition": ("4 kernel launches: backward prepare (also writes the forward sweep's records), saving scan "
+        "tokens_per_s": round(inp["q"].size(0) * inp["q"].size(1) / (ms * 1e-3), 1),
+        "composition": ("5 kernel launches: backward prepare, forward prepare + saving scan (forward sweep), saving scan "
+                        "over the mirror problem with every row scanned over its own chunks (reverse sweep), chunk-local "
+                        "gradients; chunk states, V~ and Y pass between them as bf16"
+                        if backward_kernels_apply(w.K, w.V) and inp["cu_seqlens"] is not None else
+                        "4 kernel launches: backward prepare (also writes the forward sweep's records), saving scan "
                         "on those records (forward sweep), saving scan over the mirror problem (reverse sweep), "
                         "chunk-local gradients; chunk states, V~ and Y pass between them as bf16"
                         if backward_kernels_apply(w.K, w.V) else
@@ -671,6 +675,10 @@ def main():
 
             shipped = replace(get_workload(1, B=8, H=2, K=256, V=512), name="shipped_head_shape_k256_v512_bf16")
             backward["other"] = [bench_backward(shipped, make_inputs(shipped, device="cuda"), args.steps, args.warmup)]
+            torch.cuda.empty_cache()
+            # and on the packed, ragged batch of configuration 2 (the rows of its mirror problem are scanned over their own lengths)
+            ragged = get_workload(2)
+            backward["other"].append(bench_backward(ragged, make_inputs(ragged, device="cuda"), args.steps, args.warmup))
             torch.cuda.empty_cache()
     other = None
     if not args.no_other_configs:
