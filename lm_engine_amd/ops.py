@@ -395,7 +395,7 @@ def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_ch
     ``chunk_bwd_prepare(..., reversed_copies=False)``.  ``sliced`` (bf16 saves where ``saving_scan_is_staged``): the
     save arrays are laid out by 32-column slice, ``[B H, chunks_per_chain, V / 32, K or 64, 32]`` in the memory of the
     arrays given (``gdn_chunk_saves.sliced``), for ``chunk_local_grads(..., sliced=True)``.
-    ``valid_lengths`` (``B`` host integers, multiples of 64; not with ``mirror_odd``): the rows are left-padded - row ``n`` is
+    ``valid_lengths`` (``B`` host integers, positive multiples of 64; not with ``mirror_odd``): the rows are left-padded - row ``n`` is
     scanned over its last ``valid_lengths[n]`` tokens only, with the records at the slots of those tokens, and a reverse
     save counts a row's entries from its own last saved chunk (entry 0)."""
     _require_hip_path()
@@ -405,6 +405,8 @@ def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_ch
     if valid_lengths is not None:
         if mirror_odd is not None:
             raise ValueError("valid_lengths and mirror_odd exclude each other")
+        if len(valid_lengths) != k.size(0) or any(int(n) <= 0 or int(n) % 64 != 0 or int(n) > k.size(1) for n in valid_lengths):
+            raise ValueError(f"valid_lengths must be {k.size(0)} positive multiples of 64 of at most T = {k.size(1)}")
         sums = [0]
         for length in valid_lengths:
             sums.append(sums[-1] + int(length))

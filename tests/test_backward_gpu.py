@@ -434,6 +434,54 @@ def test_mirror_reads_equal_the_scan_over_reversed_copies(K, V, B, T, H):
         assert torch.equal(a, b), f"{name}: rel-L2 {rel_l2(a.float(), b.float()):.3e}"
 
 
+@pytest.mark.parametrize("K, V, half", [(128, 128, True), (256, 128, True), (64, 64, True), (128, 128, False), (64, 128, False)])
+def test_rows_scanned_over_their_own_lengths_equal_the_fixed_length_scan(K, V, half):
+    """The mirror problem of a ragged batch, scanned as a left-padded batch of given records (every row over its own
+    chunks, records at the slots of its tokens, reverse saves counted from its own last chunk, ``row_order``) with the
+    chunk slots past a sequence's end left unwritten, against the scan of all rows over the chunks of the longest one
+    with neutral records there: the same saved states, Y and final states at the real chunks, bit for bit (a neutral
+    chunk leaves the state as it is)."""
+    from lm_engine_amd import ops
+
+    lens = [70, 300, 129, 64]
+    N, H, total = len(lens), 3, sum(lens)
+    inp = random_inputs(B=1, T=total, H=H, K=K, V=V, dtype=torch.bfloat16, seed=101, normalize=False, N=N)
+    q, k, g, beta = (inp[n].cuda() for n in ("q", "k", "g", "beta"))
+    gen = torch.Generator().manual_seed(102)
+    do = torch.randn(1, total, H, V, generator=gen).to(torch.bfloat16).cuda()
+    dht = torch.randn(N, H, K, V, generator=gen).cuda()
+    starts = [sum(lens[:n]) for n in range(N)]
+    chunks = [-(-length // 64) for length in lens]
+    NC = max(chunks)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")  # noqa: E731
+    sequences = (i32(starts), i32(lens), NC)
+    saves = torch.bfloat16 if half else torch.float32
+    results = []
+    for own_lengths in (False, True):
+        prep = ops.chunk_bwd_prepare(q, k, do, g, beta, K**-0.5, True, V, sequences, half_slice_records=half,
+                                     skip_empty_chunks=own_lengths)  # fmt: skip
+        if own_lengths:  # what the prepare kernel skipped must not matter
+            live = torch.zeros(N, NC, dtype=torch.bool)
+            for n in range(N):
+                live[n, : chunks[n]] = True
+            dead_rows = (~live).flip(1).repeat_interleave(128, dim=1).cuda()  # mirror rows: chunk c at pair NC - 1 - c
+            prep["k_mirror"][dead_rows] = float("nan")
+            prep["v_mirror"][dead_rows] = float("nan")
+        dS1 = torch.zeros(N * H, NC, K, V, dtype=saves, device="cuda")
+        Y = torch.zeros(N * H, NC, 64, V, dtype=saves, device="cuda")
+        _, dS = ops.chunk_scan_given_records(prep["k_mirror"], prep["v_mirror"], prep["records"], dht, dS1, NC, save_every=2,
+                                             save_reverse=True, half_slice_records=half, v_new=Y, no_output=half,
+                                             valid_lengths=[128 * c for c in chunks] if own_lengths else None)  # fmt: skip
+        torch.cuda.synchronize()
+        results.append((dS1.cpu().view(N, H, NC, K, V), Y.cpu().view(N, H, NC, 64, V), dS.cpu()))
+    (s_a, y_a, f_a), (s_b, y_b, f_b) = results
+    assert torch.equal(f_a, f_b), "final states"
+    for n in range(N):
+        assert s_a[n, :, : chunks[n]].abs().max() > 0
+        assert torch.equal(s_a[n, :, : chunks[n]], s_b[n, :, : chunks[n]]), f"saved states of sequence {n}"
+        assert torch.equal(y_a[n, :, : chunks[n]], y_b[n, :, : chunks[n]]), f"saved Y of sequence {n}"
+
+
 def _slice(x):
     """[chains, entries, rows, V] -> the same values in the memory order of ``gdn_chunk_saves.sliced``, [V / 32][rows][32]
     per entry (shape kept)."""
