@@ -357,6 +357,11 @@ def _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, l2norm
         sequences = (as_i32(starts), as_i32(lens), NC)
     Bt = N * H
     q, k, v, do = (x if x.stride(-1) == 1 else x.contiguous() for x in (q, k, v, do.to(torch.bfloat16)))
+    # (ragged batches: a row of the mirror problem is scanned over the two chunks per chunk of ITS sequence, which lie at
+    # the row's end, not over those of the longest one; the small tensors that say so are made here, ahead of the launches)
+    mirror_lengths = None
+    if sequences is not None:
+        mirror_lengths = ops.left_padded_rows([2 * CHUNK * max(1, -(-length // CHUNK)) for length in lens], 2 * NC * CHUNK, dev)
     # The sweeps run on the half-slice scan, one 32-column slice per workgroup, whatever the number of chains: it is the
     # variant that stages its saves through LDS (bf16, whole lines) and scans without output, which outweighs the records
     # that four slices per workgroup would share (measured with 2 to 6 workgroups per CU: 1.35 against 2.17 ms at twice
@@ -392,9 +397,6 @@ def _backward_on_kernels(q, k, v, g, beta, do, dht, scale, initial_state, l2norm
     dht32 = None if dht is None else dht.to(torch.float32).contiguous()
     dS1 = torch.empty(Bt, NC, K, V, device=dev, dtype=torch.bfloat16 if staged_m else torch.float32)
     Y = torch.empty(Bt, NC, CHUNK, V, dtype=torch.bfloat16, device=dev) if staged_m else None
-    # (ragged batches: a row of the mirror problem is scanned over the two chunks per chunk of ITS sequence, which lie at
-    # the row's end, not over those of the longest one)
-    mirror_lengths = None if sequences is None else [2 * CHUNK * max(1, -(-length // CHUNK)) for length in lens]
     o_m, dS = ops.chunk_scan_given_records(k if mirror_reads else prep["k_mirror"], prep["v_mirror"], prep["records"],
                                            dht32, dS1, NC, save_every=2, save_reverse=True,
                                            half_slice_records=half_slices, v_new=Y, no_output=staged_m,

@@ -377,6 +377,20 @@ def half_slice_records_pay(chains: int, V: int, device) -> bool:
     return chains * (V // 32) <= torch.cuda.get_device_properties(device).multi_processor_count
 
 
+def left_padded_rows(valid_lengths, T: int, device):
+    """Device tensors for ``chunk_scan_given_records(..., valid_lengths=...)`` from the rows' valid lengths (host integers,
+    positive multiples of 64, at most ``T``): the int32 prefix sums ``[B + 1]`` and the rows longest first ``[B]``.  Making
+    them is two small host-to-device copies; a caller that scans several times, or wants the copies out of the way of
+    its launches, makes them once and passes the pair."""
+    if any(int(n) <= 0 or int(n) % 64 != 0 or int(n) > T for n in valid_lengths):
+        raise ValueError(f"valid_lengths must be positive multiples of 64 of at most T = {T}")
+    sums = [0]
+    for length in valid_lengths:
+        sums.append(sums[-1] + int(length))
+    longest_first = sorted(range(len(valid_lengths)), key=lambda n: (-int(valid_lengths[n]), n))
+    return (torch.tensor(sums, dtype=torch.int32, device=device), torch.tensor(longest_first, dtype=torch.int32, device=device))
+
+
 def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_chain, save_every=1, save_reverse=False,
                              half_slice_records=False, v_new=None, no_output=False, q=None, mirror_odd=None, sliced=False,
                              valid_lengths=None):
@@ -395,7 +409,7 @@ def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_ch
     ``chunk_bwd_prepare(..., reversed_copies=False)``.  ``sliced`` (bf16 saves where ``saving_scan_is_staged``): the
     save arrays are laid out by 32-column slice, ``[B H, chunks_per_chain, V / 32, K or 64, 32]`` in the memory of the
     arrays given (``gdn_chunk_saves.sliced``), for ``chunk_local_grads(..., sliced=True)``.
-    ``valid_lengths`` (``B`` host integers, positive multiples of 64; not with ``mirror_odd``): the rows are left-padded - row ``n`` is
+    ``valid_lengths`` (``B`` host integers, positive multiples of 64, or what ``left_padded_rows`` made of them; not with ``mirror_odd``): the rows are left-padded - row ``n`` is
     scanned over its last ``valid_lengths[n]`` tokens only, with the records at the slots of those tokens, and a reverse
     save counts a row's entries from its own last saved chunk (entry 0)."""
     _require_hip_path()
@@ -405,14 +419,9 @@ def chunk_scan_given_records(k, v, records, initial_state, states, chunks_per_ch
     if valid_lengths is not None:
         if mirror_odd is not None:
             raise ValueError("valid_lengths and mirror_odd exclude each other")
-        if len(valid_lengths) != k.size(0) or any(int(n) <= 0 or int(n) % 64 != 0 or int(n) > k.size(1) for n in valid_lengths):
-            raise ValueError(f"valid_lengths must be {k.size(0)} positive multiples of 64 of at most T = {k.size(1)}")
-        sums = [0]
-        for length in valid_lengths:
-            sums.append(sums[-1] + int(length))
-        pad_lens = torch.tensor(sums, dtype=torch.int32, device=k.device)
-        longest_first = sorted(range(len(valid_lengths)), key=lambda n: (-int(valid_lengths[n]), n))
-        row_order = torch.tensor(longest_first, dtype=torch.int32, device=k.device)
+        pad_lens, row_order = valid_lengths if isinstance(valid_lengths, tuple) else left_padded_rows(valid_lengths, k.size(1), k.device)
+        if pad_lens.numel() != k.size(0) + 1 or row_order.numel() != k.size(0):
+            raise ValueError(f"valid_lengths must describe the {k.size(0)} rows of k")
     dims = _check_inputs(q, k, v, None, None, initial_state, pad_lens, pad_lens is not None)
     B, T, H, K, V, N = dims
     q, k, v = _last_dim_contiguous(q), _last_dim_contiguous(k), _last_dim_contiguous(v)
