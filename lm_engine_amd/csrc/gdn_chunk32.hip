@@ -1367,9 +1367,11 @@ ScanPlan plan_scan(int K, int64_t chains, int V, bool packed, bool save, int rec
     if (packed && !save && nw > 1 && chains * (vtiles / (nw / 2)) <= 2 * (int64_t)num_cus) nw /= 2;
     if (save && nw == 2) nw = 1;  // the saving variant exists for 1 and 4 slices per workgroup
     // The saving scan of a packed batch (the backward's forward sweep): started longest first as well, its half-slice
-    // variant, whose saves go through LDS, finishes a ragged batch sooner than four slices per workgroup storing from
-    // their compute waves, while there are at most four workgroups per CU (configuration 2: 352 us against 575 us).
-    if (save && packed && !records_given && K <= 128 && chains * vtiles <= 4 * (int64_t)num_cus) nw = 1;
+    // variant, whose saves go through LDS (and may be bf16, which the chunk-local backward kernel reads at half the
+    // traffic), finishes a ragged batch sooner than four slices per workgroup storing from their compute waves
+    // (configuration 2, 2.75 workgroups per CU: 352 us against 575 us; the whole backward of 131072 ragged tokens, 7.5
+    // workgroups per CU: 6.3 against 7.4 ms).
+    if (save && packed && !records_given && K <= 128) nw = 1;
     if (K > 128) nw = 1;  // K = 256 has the half-slice scan only, also as the saving variant and on given records
     if (records_given == 2) nw = 1;  // records given in the half-slice scan's fragment order
     ScanPlan plan;

@@ -153,16 +153,22 @@ def test_chunk_bf16_k256_packed():
     _run_case(lm_engine_amd.chunk_gated_delta_rule, inp, torch.bfloat16, cu=cu)
 
 
-@pytest.mark.parametrize("layout", ["rows", "packed"])
+@pytest.mark.parametrize("layout", ["rows", "packed", "packed_many"])
 def test_chunk_bf16_more_slices_than_compute_units(layout):
     # 6 x 16 chains x 4 slices = 384 scan workgroups for 256 CUs: the sweeps still run on the half-slice scan (bf16 saves
     # through LDS); the packed batch is ragged, so the rows of its mirror problem are scanned over their own lengths
     if layout == "rows":
         inp = random_inputs(B=6, T=192, H=16, K=128, V=128, dtype=torch.bfloat16, seed=71, normalize=False)
         _run_case(lm_engine_amd.chunk_gated_delta_rule, inp, torch.bfloat16)
-    else:
+    elif layout == "packed":
         cu = torch.tensor([0, 200, 230, 520, 584, 800, 1000], dtype=torch.int32)
         inp = random_inputs(B=1, T=1000, H=16, K=128, V=128, dtype=torch.bfloat16, seed=72, normalize=False, N=6)
+        _run_case(lm_engine_amd.chunk_gated_delta_rule, inp, torch.bfloat16, cu=cu)
+    else:
+        # 17 sequences x 16 heads x 4 slices = 1088 workgroups, more than four per CU
+        lens = [40 + 7 * n for n in range(17)]
+        cu = torch.tensor([0] + lens, dtype=torch.int32).cumsum(0).to(torch.int32)
+        inp = random_inputs(B=1, T=sum(lens), H=16, K=128, V=128, dtype=torch.bfloat16, seed=73, normalize=False, N=17)
         _run_case(lm_engine_amd.chunk_gated_delta_rule, inp, torch.bfloat16, cu=cu)
 
 
