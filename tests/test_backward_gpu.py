@@ -153,6 +153,16 @@ def test_chunk_bf16_k256_packed():
     _run_case(lm_engine_amd.chunk_gated_delta_rule, inp, torch.bfloat16, cu=cu)
 
 
+@pytest.mark.parametrize("K, V", [(128, 128), (256, 128)])
+def test_chunk_bf16_packed_with_empty_sequences(K, V):
+    # sequences of length 0 inside a packed batch: no gradient but that of their initial state (= the gradient of their
+    # final state); their rows of the mirror problem are one neutral pair of chunks, which the prepare kernel still writes
+    lens = [70, 0, 129, 0, 64]
+    cu = torch.tensor([0] + lens, dtype=torch.int32).cumsum(0).to(torch.int32)
+    inp = random_inputs(B=1, T=sum(lens), H=2, K=K, V=V, dtype=torch.bfloat16, seed=83, normalize=False, N=len(lens))
+    _run_case(lm_engine_amd.chunk_gated_delta_rule, inp, torch.bfloat16, cu=cu)
+
+
 @pytest.mark.parametrize("layout", ["rows", "packed", "packed_many"])
 def test_chunk_bf16_more_slices_than_compute_units(layout):
     # 6 x 16 chains x 4 slices = 384 scan workgroups for 256 CUs: the sweeps still run on the half-slice scan (bf16 saves
