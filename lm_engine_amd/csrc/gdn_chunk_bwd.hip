@@ -922,7 +922,8 @@ __global__ __launch_bounds__(BWD_THREADS, (K <= 64 ? 3 : 2)) void chunk_bwd_prep
     const int n = chain / p.H, h = chain % p.H;
     const int64_t TM = (int64_t)p.NC * 2 * C;  // tokens per sequence of the mirror problem
     // first token of the chunk as a flat index over the rows of the caller's tensors, and its number of tokens;
-    // a chunk past the end of its sequence (valid = 0) still gets its (neutral) records and zero rows
+    // a chunk past the end of its sequence (valid = 0) still gets its (neutral) records and zero rows, unless the caller
+    // scans without them (skip_empty below)
     int valid = C;
     int64_t tok0 = (int64_t)n * p.T_rows + (int64_t)ci * C;
     if (p.seq_start != nullptr) {
