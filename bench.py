@@ -624,7 +624,7 @@ def bench_backward(w, inp, steps, warmup):
         "steps": steps,
         "ms_per_backward": round(ms, 3),
         "tokens_per_s": round(inp["q"].size(0) * inp["q"].size(1) / (ms * 1e-3), 1),
-        "composition": ("5 kernel launches: backward prepare, forward prepare + saving scan (forward sweep), saving scan "
+        "composition": ("5 kernel launches (and the 7 us chunk-offsets helper): backward prepare, forward prepare + saving scan (forward sweep), saving scan "
                         "over the mirror problem with every row scanned over its own chunks (reverse sweep), chunk-local "
                         "gradients; chunk states, V~ and Y pass between them as bf16"
                         if backward_kernels_apply(w.K, w.V) and inp["cu_seqlens"] is not None else
